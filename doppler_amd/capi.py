@@ -1,0 +1,99 @@
+"""ctypes binding of libdopplerhip.so (the C ABI declared in include/doppler_hip.h).
+
+There is no fallback: if the shared library is missing or a call fails, a DopplerHipError is
+raised with the library's own message.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libdopplerhip.so")
+
+F32, F16 = 0, 1
+ACT_SILU, ACT_GELU = 0, 1
+KV_CONTIGUOUS, KV_RING = 0, 1
+
+
+class DopplerHipError(RuntimeError):
+    pass
+
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_I64 = ctypes.c_int64
+_F = ctypes.c_float
+_SZ = ctypes.c_size_t
+
+# name -> (restype, argtypes); every symbol include/doppler_hip.h declares
+SIGNATURES = {
+    "dh_init": (_I, [_I]),
+    "dh_shutdown": (_I, []),
+    "dh_last_error": (ctypes.c_char_p, []),
+    "dh_set_stream": (_I, [_P]),
+    "dh_get_stream": (_P, []),
+    "dh_malloc": (_I, [_SZ, ctypes.POINTER(_P)]),
+    "dh_free": (_I, [_P]),
+    "dh_upload": (_I, [_P, _SZ, _P, _SZ]),
+    "dh_download": (_I, [_P, _P, _SZ, _SZ]),
+    "dh_copy": (_I, [_P, _SZ, _P, _SZ, _SZ]),
+    "dh_fill_zero": (_I, [_P, _SZ, _SZ]),
+    "dh_sync": (_I, []),
+    "dh_event_create": (_I, [ctypes.POINTER(_P)]),
+    "dh_event_record": (_I, [_P]),
+    "dh_event_elapsed_ms": (_I, [_P, _P, ctypes.POINTER(_F)]),
+    "dh_event_destroy": (_I, [_P]),
+    "dh_q4k_dequant": (_I, [_P, _I64, _P]),
+    "dh_q4k_matmul": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
+    "dh_q4k_ffn_gate_up": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
+    "dh_f16w_matmul": (_I, [_P, _P, _P, _I, _I, _I, _F]),
+    "dh_lmhead_argmax_workspace_bytes": (_SZ, [_I]),
+    "dh_lmhead_argmax_f16": (_I, [_P, _P, _I, _I, _I64, _F, _P, _P, _I, _P]),
+    "dh_attn_decode_workspace_bytes": (_SZ, [_I, _I, _I]),
+    "dh_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _F, _I, _I, _I, _P]),
+    "dh_rmsnorm": (_I, [_P, _P, _I, _P, _I, _I, _F, _I, _P, _P, _P, _F]),
+    "dh_rope": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I]),
+    "dh_qkv_norm_rope_kvwrite": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F,
+                                      _I, _I64, _I]),
+    "dh_kv_write_f16": (_I, [_P, _P, _P, _P, _I64, _I64, _I64]),
+    "dh_residual_add": (_I, [_P, _P, _P, _I64, _F]),
+    "dh_gather_f16": (_I, [_P, _P, _P, _I, _I, _I, _I]),
+    "dh_act_gate": (_I, [_P, _P, _P, _I64, _I, _F]),
+    "dh_act_gate_rowsplit": (_I, [_P, _P, _I, _I, _I, _F]),
+    "dh_argmax_workspace_bytes": (_SZ, []),
+    "dh_argmax": (_I, [_P, _I, _I64, _F, _P, _P, _I]),
+    "dh_cast_f32_to_f16": (_I, [_P, _P, _I64]),
+    "dh_cast_f16_to_f32": (_I, [_P, _P, _I64]),
+}
+
+_lib = None
+
+
+def load():
+    """Loads the shared library (no GPU needed for loading) and types every symbol."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise DopplerHipError(
+                "libdopplerhip.so is not built (expected %s); run `python -m doppler_amd.build`" % LIB_PATH)
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise DopplerHipError(load().dh_last_error().decode("utf-8", "replace"))
+
+
+_initialised = False
+
+
+def init(device=0):
+    global _initialised
+    check(load().dh_init(device))
+    _initialised = True
+    return _lib

@@ -1,0 +1,180 @@
+// Device, memory and stream entry points of the C ABI.
+#include <cstring>
+#include <mutex>
+
+#include "dh_common.h"
+
+namespace {
+std::mutex g_mu;
+thread_local char g_err[1024] = "";
+bool g_ready = false;
+int g_device = -1;
+hipStream_t g_own_stream = nullptr;
+hipStream_t g_stream = nullptr;
+}  // namespace
+
+namespace dh {
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+hipStream_t stream() { return g_stream; }
+bool ready() { return g_ready; }
+}  // namespace dh
+
+extern "C" {
+
+const char* dh_last_error(void) { return g_err; }
+
+int dh_init(int device_ordinal) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (g_ready) {
+    if (device_ordinal != g_device)
+      return dh::fail(1, "[dh_init] already initialised on device %d", g_device);
+    return 0;
+  }
+  int count = 0;
+  DH_CHECK_HIP("dh_init", hipGetDeviceCount(&count));
+  if (device_ordinal < 0 || device_ordinal >= count)
+    return dh::fail(1, "[dh_init] device %d not present (%d visible)", device_ordinal, count);
+  DH_CHECK_HIP("dh_init", hipSetDevice(device_ordinal));
+  hipDeviceProp_t prop;
+  DH_CHECK_HIP("dh_init", hipGetDeviceProperties(&prop, device_ordinal));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return dh::fail(1, "[dh_init] this library is built for gfx950 only, device is %s",
+                    prop.gcnArchName);
+  DH_CHECK_HIP("dh_init", hipStreamCreateWithFlags(&g_own_stream, hipStreamDefault));
+  g_stream = g_own_stream;
+  g_device = device_ordinal;
+  g_ready = true;
+  return 0;
+}
+
+int dh_shutdown(void) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (!g_ready) return 0;
+  DH_CHECK_HIP("dh_shutdown", hipStreamSynchronize(g_stream));
+  if (g_own_stream) DH_CHECK_HIP("dh_shutdown", hipStreamDestroy(g_own_stream));
+  g_own_stream = nullptr;
+  g_stream = nullptr;
+  g_ready = false;
+  g_device = -1;
+  return 0;
+}
+
+int dh_set_stream(void* hip_stream) {
+  DH_REQUIRE_INIT("dh_set_stream");
+  g_stream = hip_stream ? static_cast<hipStream_t>(hip_stream) : g_own_stream;
+  return 0;
+}
+
+void* dh_get_stream(void) { return g_stream; }
+
+int dh_malloc(size_t bytes, void** d_out) {
+  DH_REQUIRE_INIT("dh_malloc");
+  if (!d_out) return dh::fail(1, "[dh_malloc] output pointer is null");
+  *d_out = nullptr;
+  if (bytes == 0) return dh::fail(1, "[dh_malloc] size must be positive");
+  DH_CHECK_HIP("dh_malloc", hipMalloc(d_out, bytes));
+  return 0;
+}
+
+int dh_free(void* d_ptr) {
+  DH_REQUIRE_INIT("dh_free");
+  if (!d_ptr) return 0;
+  DH_CHECK_HIP("dh_free", hipStreamSynchronize(g_stream));
+  DH_CHECK_HIP("dh_free", hipFree(d_ptr));
+  return 0;
+}
+
+int dh_upload(void* d_dst, size_t dst_offset, const void* host_src, size_t bytes) {
+  DH_REQUIRE_INIT("dh_upload");
+  if (bytes == 0) return 0;
+  if (!d_dst || !host_src) return dh::fail(1, "[dh_upload] null pointer");
+  // Pageable host memory: hipMemcpyAsync stages it before returning, so the caller may
+  // reuse host_src at once; ordering with earlier ops comes from the stream.
+  DH_CHECK_HIP("dh_upload", hipMemcpyAsync(static_cast<char*>(d_dst) + dst_offset, host_src, bytes,
+                                           hipMemcpyHostToDevice, g_stream));
+  DH_CHECK_HIP("dh_upload", hipStreamSynchronize(g_stream));
+  return 0;
+}
+
+int dh_download(void* host_dst, const void* d_src, size_t src_offset, size_t bytes) {
+  DH_REQUIRE_INIT("dh_download");
+  if (bytes == 0) return 0;
+  if (!host_dst || !d_src) return dh::fail(1, "[dh_download] null pointer");
+  DH_CHECK_HIP("dh_download", hipMemcpyAsync(host_dst, static_cast<const char*>(d_src) + src_offset,
+                                             bytes, hipMemcpyDeviceToHost, g_stream));
+  DH_CHECK_HIP("dh_download", hipStreamSynchronize(g_stream));
+  return 0;
+}
+
+int dh_copy(void* d_dst, size_t dst_offset, const void* d_src, size_t src_offset, size_t bytes) {
+  DH_REQUIRE_INIT("dh_copy");
+  if (bytes == 0) return 0;
+  if (!d_dst || !d_src) return dh::fail(1, "[dh_copy] null pointer");
+  DH_CHECK_HIP("dh_copy", hipMemcpyAsync(static_cast<char*>(d_dst) + dst_offset,
+                                         static_cast<const char*>(d_src) + src_offset, bytes,
+                                         hipMemcpyDeviceToDevice, g_stream));
+  return 0;
+}
+
+__global__ void dh_fill_zero_kernel(uint32_t* p, int64_t words) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < words; i += stride) p[i] = 0u;
+}
+
+int dh_fill_zero(void* d_dst, size_t offset, size_t bytes) {
+  DH_REQUIRE_INIT("dh_fill_zero");
+  if (bytes == 0) return 0;
+  if (!d_dst) return dh::fail(1, "[dh_fill_zero] null pointer");
+  if ((offset | bytes) & 3) return dh::fail(1, "[dh_fill_zero] offset and size must be multiples of 4");
+  // A fill kernel rather than hipMemsetAsync so the call can sit inside a captured graph.
+  const int64_t words = (int64_t)(bytes / 4);
+  const int grid = (int)std::min<int64_t>(dh::ceil_div(words, 256), 2048);
+  hipLaunchKernelGGL(dh_fill_zero_kernel, dim3(grid), dim3(256), 0, g_stream,
+                     reinterpret_cast<uint32_t*>(static_cast<char*>(d_dst) + offset), words);
+  DH_CHECK_LAUNCH("dh_fill_zero");
+  return 0;
+}
+
+int dh_event_create(void** ev_out) {
+  DH_REQUIRE_INIT("dh_event_create");
+  if (!ev_out) return dh::fail(1, "[dh_event_create] null pointer");
+  hipEvent_t ev;
+  DH_CHECK_HIP("dh_event_create", hipEventCreate(&ev));
+  *ev_out = ev;
+  return 0;
+}
+
+int dh_event_record(void* ev) {
+  DH_REQUIRE_INIT("dh_event_record");
+  DH_CHECK_HIP("dh_event_record", hipEventRecord(static_cast<hipEvent_t>(ev), g_stream));
+  return 0;
+}
+
+int dh_event_elapsed_ms(void* start, void* stop, float* ms_out) {
+  DH_REQUIRE_INIT("dh_event_elapsed_ms");
+  DH_CHECK_HIP("dh_event_elapsed_ms", hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+  DH_CHECK_HIP("dh_event_elapsed_ms", hipEventElapsedTime(ms_out, static_cast<hipEvent_t>(start),
+                                                          static_cast<hipEvent_t>(stop)));
+  return 0;
+}
+
+int dh_event_destroy(void* ev) {
+  DH_REQUIRE_INIT("dh_event_destroy");
+  DH_CHECK_HIP("dh_event_destroy", hipEventDestroy(static_cast<hipEvent_t>(ev)));
+  return 0;
+}
+
+int dh_sync(void) {
+  DH_REQUIRE_INIT("dh_sync");
+  DH_CHECK_HIP("dh_sync", hipStreamSynchronize(g_stream));
+  return 0;
+}
+
+}  // extern "C"

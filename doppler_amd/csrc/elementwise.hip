@@ -1,0 +1,403 @@
+// Normalisation, rotary embedding, KV-cache writes and the elementwise glue ops.
+// All of these move a few KB per token: they are launch-bound, so each is one launch with
+// 16-byte accesses where alignment allows and no intermediate buffers.
+#include <algorithm>
+
+#include "dh_common.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// Sum over a 256-thread workgroup; every thread gets the result.  `red` is 4 floats of LDS.
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  const float total = red[0] + red[1] + red[2] + red[3];
+  __syncthreads();
+  return total;
+}
+
+__device__ __forceinline__ float load_norm_weight(const void* w, int is_f16, int i, int offset) {
+  float v = 1.0f;
+  if (w) v = is_f16 ? __half2float(static_cast<const __half*>(w)[i]) : static_cast<const float*>(w)[i];
+  else return 1.0f;
+  return offset ? 1.0f + v : v;
+}
+
+// ---------------------------------------------------------------------------------------
+// RMSNorm: one workgroup per token.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const void* __restrict__ w,
+                                                      int w_f16, float* __restrict__ out, int hidden,
+                                                      float eps, int w_offset,
+                                                      const float* __restrict__ pre,
+                                                      const float* __restrict__ post,
+                                                      float* __restrict__ prenorm, float out_scale) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    float v = x[base + i];
+    if (pre) v += pre[base + i];
+    ss = fmaf(v, v, ss);
+  }
+  const float total = block_sum_256(ss, red);
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    float v = x[base + i];
+    if (pre) v += pre[base + i];
+    if (prenorm) prenorm[base + i] = v;
+    float y = v * inv * load_norm_weight(w, w_f16, i, w_offset);
+    if (post) y += post[base + i];
+    out[base + i] = y * out_scale;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// RoPE in place: one thread per rotated pair.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rope_kernel(float* __restrict__ x, const float* __restrict__ cos_t,
+                                                   const float* __restrict__ sin_t, int64_t total_pairs,
+                                                   int heads, int head_dim, int half, int partner,
+                                                   int interleaved, int start_pos) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total_pairs) return;
+  const int pair = (int)(idx % half);
+  const int64_t th = idx / half;  // token * heads + head
+  const int64_t token = th / heads;
+  const int64_t pos = start_pos + token;
+  const float c = cos_t[pos * half + pair], s = sin_t[pos * half + pair];
+  float* row = x + th * head_dim;
+  const int i0 = interleaved ? 2 * pair : pair;
+  const int i1 = interleaved ? 2 * pair + 1 : pair + partner;
+  const float x0 = row[i0], x1 = row[i1];
+  row[i0] = x0 * c - x1 * s;
+  row[i1] = x0 * s + x1 * c;
+}
+
+// ---------------------------------------------------------------------------------------
+// Fused split-QKV + per-head RMSNorm + RoPE + f16 KV write.  One wave per (token, head)
+// row for Q and K rows; the trailing workgroups narrow V.  D <= 512.
+// ---------------------------------------------------------------------------------------
+struct QkvArgs {
+  const float* qkv;
+  const float* qw;
+  const float* kw;
+  const float* cos_t;
+  const float* sin_t;
+  float* q_out;
+  __half* cache_k;
+  __half* cache_v;
+  int T, H, Hkv, D, start_pos, rotary_dim, interleaved, w_offset, use_norm;
+  float eps;
+  int64_t kv_dst;
+  int64_t qk_rows;   // T * (H + Hkv)
+  int64_t total_v;   // T * Hkv * D
+};
+
+__global__ __launch_bounds__(256) void qkv_norm_rope_kernel(const QkvArgs a) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t qk_groups = (a.qk_rows + 3) / 4;
+  if ((int64_t)blockIdx.x >= qk_groups) {
+    // V: plain narrowing copy
+    const int64_t i = ((int64_t)blockIdx.x - qk_groups) * 256 + threadIdx.x;
+    if (i < a.total_v) {
+      const int64_t v_size = (int64_t)a.Hkv * a.D;
+      const int64_t t = i / v_size, e = i - t * v_size;
+      const int64_t stride = (int64_t)(a.H + 2 * a.Hkv) * a.D;
+      a.cache_v[a.kv_dst + i] = __float2half(a.qkv[t * stride + (int64_t)(a.H + a.Hkv) * a.D + e]);
+    }
+    return;
+  }
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row >= a.qk_rows) return;
+  const int rows_per_tok = a.H + a.Hkv;
+  const int64_t t = row / rows_per_tok;
+  const int r = (int)(row - t * rows_per_tok);
+  const bool is_q = r < a.H;
+  const int head = is_q ? r : r - a.H;
+  const int64_t stride = (int64_t)(a.H + 2 * a.Hkv) * a.D;
+  const float* src = a.qkv + t * stride + (is_q ? 0 : (int64_t)a.H * a.D) + (int64_t)head * a.D;
+  const float* w = is_q ? a.qw : a.kw;
+  const int D = a.D;
+  float inv = 1.0f;
+  if (a.use_norm) {
+    float ss = 0.f;
+    for (int i = lane; i < D; i += 64) ss = fmaf(src[i], src[i], ss);
+    ss = wave_sum(ss);
+    inv = 1.0f / sqrtf(ss / (float)D + a.eps);
+  }
+  const int half = a.rotary_dim / 2;
+  const int64_t pos = a.start_pos + t;
+  float* qdst = a.q_out + (t * a.H + head) * D;
+  __half* kdst = a.cache_k + a.kv_dst + (t * a.Hkv + head) * D;
+  auto nv = [&](int i) -> float {
+    float v = src[i];
+    if (a.use_norm) v = v * inv * (a.w_offset ? 1.0f + w[i] : w[i]);
+    return v;
+  };
+  for (int p = lane; p < half; p += 64) {
+    const int i0 = a.interleaved ? 2 * p : p;
+    const int i1 = a.interleaved ? 2 * p + 1 : p + half;
+    const float c = a.cos_t[pos * half + p], s = a.sin_t[pos * half + p];
+    const float x0 = nv(i0), x1 = nv(i1);
+    const float y0 = x0 * c - x1 * s, y1 = x0 * s + x1 * c;
+    if (is_q) { qdst[i0] = y0; qdst[i1] = y1; }
+    else { kdst[i0] = __float2half(y0); kdst[i1] = __float2half(y1); }
+  }
+  for (int i = a.rotary_dim + lane; i < D; i += 64) {
+    const float v = nv(i);
+    if (is_q) qdst[i] = v; else kdst[i] = __float2half(v);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Elementwise
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void kv_write_kernel(const float* __restrict__ k, const float* __restrict__ v,
+                                                       __half* __restrict__ ck, __half* __restrict__ cv,
+                                                       int64_t src, int64_t dst, int64_t count) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  ck[dst + i] = __float2half(k[src + i]);
+  cv[dst + i] = __float2half(v[src + i]);
+}
+
+__global__ __launch_bounds__(256) void residual_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                       float* __restrict__ out, int64_t n, float scale) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = (a[i] + b[i]) * scale;
+}
+
+__global__ __launch_bounds__(256) void gather_f16_kernel(const uint32_t* __restrict__ ids,
+                                                         const __half* __restrict__ table,
+                                                         float* __restrict__ out, int64_t total, int hidden,
+                                                         uint32_t vocab, int index_offset) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / hidden;
+  const int d = (int)(i - t * hidden);
+  const uint32_t id = ids[t + index_offset];
+  out[i] = id >= vocab ? 0.0f : __half2float(table[(int64_t)id * hidden + d]);
+}
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float gelu_f(float x) {
+  const float inner = 0.7978845608f * (x + 0.044715f * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(fminf(fmaxf(inner, -15.0f), 15.0f)));
+}
+__device__ __forceinline__ float gate_mul(float g, float u, int act, float clamp_max) {
+  if (act == DH_ACT_SILU) {
+    float v = silu_f(g) * u;
+    if (clamp_max > 0.f) v = fminf(fmaxf(v, -clamp_max), clamp_max);
+    return v;
+  }
+  return gelu_f(g) * u;
+}
+
+__global__ __launch_bounds__(256) void act_gate_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                       float* __restrict__ out, int64_t n, int act,
+                                                       float clamp_max) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = gate_mul(gate[i], up[i], act, clamp_max);
+}
+
+__global__ __launch_bounds__(256) void act_gate_rowsplit_kernel(const float* __restrict__ in,
+                                                                float* __restrict__ out, int64_t total, int dim,
+                                                                int act, float clamp_max) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / dim;
+  const int d = (int)(i - t * dim);
+  const float* row = in + t * 2 * dim;
+  out[i] = gate_mul(row[d], row[dim + d], act, clamp_max);
+}
+
+__global__ __launch_bounds__(256) void cast_f32_f16_kernel(const float* __restrict__ in, __half* __restrict__ out,
+                                                           int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = __float2half(in[i]);
+}
+__global__ __launch_bounds__(256) void cast_f16_f32_kernel(const __half* __restrict__ in, float* __restrict__ out,
+                                                           int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = __half2float(in[i]);
+}
+
+unsigned grid_for(int64_t n) { return (unsigned)dh::ceil_div(n, 256); }
+
+}  // namespace
+
+extern "C" {
+
+int dh_rmsnorm(const float* d_x, const void* d_weight, int weight_dtype, float* d_out, int batch,
+               int hidden, float eps, int weight_offset, const float* d_pre_residual,
+               const float* d_post_residual, float* d_prenorm_out, float output_scale) {
+  const char* op = "dh_rmsnorm";
+  DH_REQUIRE_INIT(op);
+  if (batch <= 0 || hidden <= 0) return dh::fail(1, "[%s] batch=%d hidden=%d must be positive", op, batch, hidden);
+  if (!d_x || !d_out) return dh::fail(1, "[%s] null pointer", op);
+  if (weight_dtype != DH_F32 && weight_dtype != DH_F16)
+    return dh::fail(1, "[%s] weight dtype must be f32 or f16", op);
+  if (d_prenorm_out && !d_pre_residual)
+    return dh::fail(1, "[%s] prenorm output needs a pre-residual input", op);
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(batch), dim3(256), 0, dh::stream(), d_x, d_weight,
+                     weight_dtype == DH_F16, d_out, hidden, eps, weight_offset, d_pre_residual,
+                     d_post_residual, d_prenorm_out, output_scale);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_rope(float* d_x, const float* d_cos, const float* d_sin, int seq, int heads, int head_dim,
+            int rotary_dim, int pair_span_dim, int interleaved, int start_pos) {
+  const char* op = "dh_rope";
+  DH_REQUIRE_INIT(op);
+  if (seq <= 0 || heads <= 0) return dh::fail(1, "[%s] seq=%d heads=%d must be positive", op, seq, heads);
+  if (head_dim <= 0 || head_dim % 2) return dh::fail(1, "RoPE headDim must be even, got %d", head_dim);
+  if (rotary_dim % 2) return dh::fail(1, "RoPE rotaryDim must be even, got %d", rotary_dim);
+  if (rotary_dim <= 0 || rotary_dim > head_dim)
+    return dh::fail(1, "RoPE rotaryDim must be in (0, headDim]; got %d for headDim %d", rotary_dim, head_dim);
+  if (pair_span_dim % 2) return dh::fail(1, "RoPE pairSpanDim must be even, got %d", pair_span_dim);
+  if (pair_span_dim < rotary_dim || pair_span_dim > head_dim)
+    return dh::fail(1, "RoPE pairSpanDim must be in [rotaryDim, headDim]; got %d for rotaryDim %d and headDim %d",
+                    pair_span_dim, rotary_dim, head_dim);
+  if (start_pos < 0) return dh::fail(1, "[%s] startPos must be non-negative", op);
+  if (!d_x || !d_cos || !d_sin) return dh::fail(1, "[%s] null pointer", op);
+  const int half = rotary_dim / 2;
+  const int64_t pairs = (int64_t)seq * heads * half;
+  hipLaunchKernelGGL(rope_kernel, dim3(grid_for(pairs)), dim3(256), 0, dh::stream(), d_x, d_cos, d_sin,
+                     pairs, heads, head_dim, half, pair_span_dim / 2, interleaved, start_pos);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_qkv_norm_rope_kvwrite(const float* d_qkv, const float* d_q_weight, const float* d_k_weight,
+                             const float* d_cos, const float* d_sin, float* d_q_out, void* d_cache_k,
+                             void* d_cache_v, int T, int H, int Hkv, int D, int start_pos,
+                             int rotary_dim, int interleaved, float eps, int weight_offset,
+                             int64_t kv_dst_offset, int use_norm) {
+  const char* op = "dh_qkv_norm_rope_kvwrite";
+  DH_REQUIRE_INIT(op);
+  if (T <= 0 || H <= 0 || Hkv <= 0 || D <= 0)
+    return dh::fail(1, "[%s] numTokens/numHeads/numKVHeads/headDim must be positive integers", op);
+  if (D % 2 || rotary_dim % 2 || rotary_dim <= 0 || rotary_dim > D)
+    return dh::fail(1, "[%s] rotaryDim %d must be even and in (0, headDim=%d]", op, rotary_dim, D);
+  if (start_pos < 0 || kv_dst_offset < 0) return dh::fail(1, "[%s] startPos and dstOffset must be non-negative", op);
+  if (!d_qkv || !d_cos || !d_sin || !d_q_out || !d_cache_k || !d_cache_v)
+    return dh::fail(1, "[%s] null pointer", op);
+  if (use_norm && (!d_q_weight || !d_k_weight)) return dh::fail(1, "[%s] q/k norm weights are required", op);
+  QkvArgs a{};
+  a.qkv = d_qkv; a.qw = d_q_weight; a.kw = d_k_weight; a.cos_t = d_cos; a.sin_t = d_sin;
+  a.q_out = d_q_out; a.cache_k = static_cast<__half*>(d_cache_k); a.cache_v = static_cast<__half*>(d_cache_v);
+  a.T = T; a.H = H; a.Hkv = Hkv; a.D = D; a.start_pos = start_pos; a.rotary_dim = rotary_dim;
+  a.interleaved = interleaved; a.w_offset = weight_offset; a.use_norm = use_norm; a.eps = eps;
+  a.kv_dst = kv_dst_offset;
+  a.qk_rows = (int64_t)T * (H + Hkv);
+  a.total_v = (int64_t)T * Hkv * D;
+  const int64_t groups = dh::ceil_div(a.qk_rows, 4) + dh::ceil_div(a.total_v, 256);
+  hipLaunchKernelGGL(qkv_norm_rope_kernel, dim3((unsigned)groups), dim3(256), 0, dh::stream(), a);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_kv_write_f16(const float* d_k, const float* d_v, void* d_cache_k, void* d_cache_v,
+                    int64_t src_offset, int64_t dst_offset, int64_t count) {
+  const char* op = "dh_kv_write_f16";
+  DH_REQUIRE_INIT(op);
+  if (src_offset < 0 || dst_offset < 0 || count < 0)
+    return dh::fail(1, "[%s] srcOffset, dstOffset and elementCount must be non-negative integers", op);
+  if (count == 0) return 0;
+  if (!d_k || !d_v || !d_cache_k || !d_cache_v) return dh::fail(1, "[%s] null pointer", op);
+  hipLaunchKernelGGL(kv_write_kernel, dim3(grid_for(count)), dim3(256), 0, dh::stream(), d_k, d_v,
+                     static_cast<__half*>(d_cache_k), static_cast<__half*>(d_cache_v), src_offset,
+                     dst_offset, count);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_residual_add(const float* d_a, const float* d_b, float* d_out, int64_t n, float scale) {
+  const char* op = "dh_residual_add";
+  DH_REQUIRE_INIT(op);
+  if (n < 0) return dh::fail(1, "[%s] size must be non-negative", op);
+  if (n == 0) return 0;
+  if (!d_a || !d_b || !d_out) return dh::fail(1, "[%s] null pointer", op);
+  if (!(scale == scale) || scale > 3.0e38f || scale < -3.0e38f)
+    return dh::fail(1, "[Residual] outputScale must be finite");
+  hipLaunchKernelGGL(residual_kernel, dim3(grid_for(n)), dim3(256), 0, dh::stream(), d_a, d_b, d_out, n, scale);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_gather_f16(const uint32_t* d_ids, const void* d_table, float* d_out, int T, int hidden, int vocab,
+                  int index_offset) {
+  const char* op = "dh_gather_f16";
+  DH_REQUIRE_INIT(op);
+  if (T <= 0 || hidden <= 0 || vocab <= 0 || index_offset < 0)
+    return dh::fail(1, "[%s] numTokens/hiddenSize/vocabSize must be positive", op);
+  if (!d_ids || !d_table || !d_out) return dh::fail(1, "[%s] null pointer", op);
+  const int64_t total = (int64_t)T * hidden;
+  hipLaunchKernelGGL(gather_f16_kernel, dim3(grid_for(total)), dim3(256), 0, dh::stream(), d_ids,
+                     static_cast<const __half*>(d_table), d_out, total, hidden, (uint32_t)vocab, index_offset);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_act_gate(const float* d_gate, const float* d_up, float* d_out, int64_t n, int activation,
+                float swiglu_limit) {
+  const char* op = "dh_act_gate";
+  DH_REQUIRE_INIT(op);
+  if (n < 0) return dh::fail(1, "[%s] size must be non-negative", op);
+  if (activation != DH_ACT_SILU && activation != DH_ACT_GELU) return dh::fail(1, "[%s] unknown activation %d", op, activation);
+  if (n == 0) return 0;
+  if (!d_gate || !d_up || !d_out) return dh::fail(1, "[%s] null pointer", op);
+  hipLaunchKernelGGL(act_gate_kernel, dim3(grid_for(n)), dim3(256), 0, dh::stream(), d_gate, d_up, d_out, n,
+                     activation, swiglu_limit);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_act_gate_rowsplit(const float* d_in, float* d_out, int T, int dim, int activation, float swiglu_limit) {
+  const char* op = "dh_act_gate_rowsplit";
+  DH_REQUIRE_INIT(op);
+  if (T <= 0 || dim <= 0) return dh::fail(1, "[%s] numTokens=%d dim=%d must be positive", op, T, dim);
+  if (activation != DH_ACT_SILU && activation != DH_ACT_GELU) return dh::fail(1, "[%s] unknown activation %d", op, activation);
+  if (!d_in || !d_out) return dh::fail(1, "[%s] null pointer", op);
+  const int64_t total = (int64_t)T * dim;
+  hipLaunchKernelGGL(act_gate_rowsplit_kernel, dim3(grid_for(total)), dim3(256), 0, dh::stream(), d_in, d_out,
+                     total, dim, activation, swiglu_limit);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_cast_f32_to_f16(const float* d_in, void* d_out, int64_t n) {
+  const char* op = "dh_cast_f32_to_f16";
+  DH_REQUIRE_INIT(op);
+  if (n < 0) return dh::fail(1, "[%s] size must be non-negative", op);
+  if (n == 0) return 0;
+  if (!d_in || !d_out) return dh::fail(1, "[%s] null pointer", op);
+  hipLaunchKernelGGL(cast_f32_f16_kernel, dim3(grid_for(n)), dim3(256), 0, dh::stream(), d_in,
+                     static_cast<__half*>(d_out), n);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_cast_f16_to_f32(const void* d_in, float* d_out, int64_t n) {
+  const char* op = "dh_cast_f16_to_f32";
+  DH_REQUIRE_INIT(op);
+  if (n < 0) return dh::fail(1, "[%s] size must be non-negative", op);
+  if (n == 0) return 0;
+  if (!d_in || !d_out) return dh::fail(1, "[%s] null pointer", op);
+  hipLaunchKernelGGL(cast_f16_f32_kernel, dim3(grid_for(n)), dim3(256), 0, dh::stream(),
+                     static_cast<const __half*>(d_in), d_out, n);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,267 @@
+// Dense f16-weight GEMV (the tied LM head), optionally fused with greedy argmax, and the
+// stand-alone two-phase argmax over f32 logits.
+//
+// The LM head reads vocab*hidden*2 bytes per token (1.24 GB at 151936 x 4096): pure HBM
+// streaming.  One wave per output row, 16 bytes (8 halves) per lane per step so a wave
+// consumes 1 KB of the row per load instruction; activations sit in LDS as f32 and are
+// read with conflict-free 16-byte accesses.  Argmax candidates (value, index) are reduced
+// per wave, per workgroup, then across workgroups by a one-workgroup kernel; ties always go
+// to the lower index, the rule of the reference's candidate_beats().
+#include <algorithm>
+#include <cfloat>
+
+#include "dh_common.h"
+
+namespace {
+
+constexpr int kMaxParts = 2048;
+
+struct Cand {
+  float v;
+  uint32_t i;
+};
+
+__device__ __forceinline__ bool beats(float cv, uint32_t ci, float bv, uint32_t bi) {
+  if (cv > bv) return true;
+  if (cv < bv) return false;
+  return ci < bi;
+}
+
+__device__ __forceinline__ Cand wave_best(Cand c) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(c.v, off, 64);
+    const uint32_t oi = __shfl_xor(c.i, off, 64);
+    if (beats(ov, oi, c.v, c.i)) { c.v = ov; c.i = oi; }
+  }
+  return c;
+}
+
+// Workgroup-wide best of 256 threads; valid in thread 0.
+__device__ __forceinline__ Cand block_best_256(Cand c, float* sv, uint32_t* si) {
+  c = wave_best(c);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) { sv[wave] = c.v; si[wave] = c.i; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; w++)
+      if (beats(sv[w], si[w], c.v, c.i)) { c.v = sv[w]; c.i = si[w]; }
+  }
+  return c;
+}
+
+__device__ __forceinline__ float softcap_f(float x, float cap) {
+  return cap > 0.f ? cap * tanhf(x / cap) : x;
+}
+
+struct F16GemvArgs {
+  const float* A;      // [M][K]
+  const __half* W;     // [N][K]
+  float* C;            // [M][N] or null
+  int N, K;
+  float alpha;
+  int rows_per_wave;
+  // argmax (M == 1 only)
+  float softcap;
+  int64_t pad_id;
+  float* part_val;
+  uint32_t* part_idx;
+};
+
+template <int MT, bool ARGMAX>
+__global__ __launch_bounds__(256) void f16w_gemv_kernel(const F16GemvArgs a) {
+  extern __shared__ float xs[];   // [MT][K]
+  __shared__ float sv[4];
+  __shared__ uint32_t si[4];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  for (int i = tid; i < MT * a.K; i += 256) xs[i] = a.A[i];
+  __syncthreads();
+
+  const int kvec = a.K >> 3;
+  const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * a.rows_per_wave;
+  Cand best{-3.402823e+38f, 0xFFFFFFFFu};   // only lane 0 ever updates its candidate
+  for (int r = 0; r < a.rows_per_wave; r++) {
+    const int64_t row = row0 + r;
+    if (row >= a.N) break;   // wave-uniform
+    const uint4* wrow = reinterpret_cast<const uint4*>(a.W + row * a.K);
+    float acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; m++) acc[m] = 0.f;
+    for (int v = lane; v < kvec; v += 64) {
+      const uint4 raw = wrow[v];
+      const __half2* h2 = reinterpret_cast<const __half2*>(&raw);
+      const float2 w0 = __half22float2(h2[0]), w1 = __half22float2(h2[1]);
+      const float2 w2 = __half22float2(h2[2]), w3 = __half22float2(h2[3]);
+#pragma unroll
+      for (int m = 0; m < MT; m++) {
+        const float4 xa = *reinterpret_cast<const float4*>(xs + m * a.K + v * 8);
+        const float4 xb = *reinterpret_cast<const float4*>(xs + m * a.K + v * 8 + 4);
+        float s = acc[m];
+        s = fmaf(xa.x, w0.x, s); s = fmaf(xa.y, w0.y, s);
+        s = fmaf(xa.z, w1.x, s); s = fmaf(xa.w, w1.y, s);
+        s = fmaf(xb.x, w2.x, s); s = fmaf(xb.y, w2.y, s);
+        s = fmaf(xb.z, w3.x, s); s = fmaf(xb.w, w3.y, s);
+        acc[m] = s;
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+      float s = acc[m];
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+      acc[m] = s * a.alpha;
+    }
+    if (lane == 0) {
+      if (a.C) {
+#pragma unroll
+        for (int m = 0; m < MT; m++) a.C[(int64_t)m * a.N + row] = acc[m];
+      }
+      if (ARGMAX && row != a.pad_id) {
+        const float v = softcap_f(acc[0], a.softcap);
+        if (beats(v, (uint32_t)row, best.v, best.i)) { best.v = v; best.i = (uint32_t)row; }
+      }
+    }
+  }
+  if (ARGMAX) {
+    const Cand c = block_best_256(best, sv, si);
+    if (tid == 0) { a.part_val[blockIdx.x] = c.v; a.part_idx[blockIdx.x] = c.i; }
+  }
+}
+
+// Phase 1 of the stand-alone argmax: grid-stride scan of f32 logits.
+__global__ __launch_bounds__(256) void argmax_scan_kernel(const float* __restrict__ logits, int vocab,
+                                                          int64_t pad_id, float softcap,
+                                                          float* __restrict__ part_val,
+                                                          uint32_t* __restrict__ part_idx) {
+  __shared__ float sv[4];
+  __shared__ uint32_t si[4];
+  Cand best{-3.402823e+38f, 0xFFFFFFFFu};
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < vocab; i += (int64_t)gridDim.x * 256) {
+    if (i == pad_id) continue;
+    const float v = softcap_f(logits[i], softcap);
+    if (beats(v, (uint32_t)i, best.v, best.i)) { best.v = v; best.i = (uint32_t)i; }
+  }
+  const Cand c = block_best_256(best, sv, si);
+  if (threadIdx.x == 0) { part_val[blockIdx.x] = c.v; part_idx[blockIdx.x] = c.i; }
+}
+
+// Phase 2: one workgroup folds the per-workgroup candidates and writes the token.
+__global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ part_val,
+                                                           const uint32_t* __restrict__ part_idx, int parts,
+                                                           uint32_t* __restrict__ token_out, int out_index) {
+  __shared__ float sv[4];
+  __shared__ uint32_t si[4];
+  Cand best{-3.402823e+38f, 0xFFFFFFFFu};
+  for (int i = threadIdx.x; i < parts; i += 256)
+    if (beats(part_val[i], part_idx[i], best.v, best.i)) { best.v = part_val[i]; best.i = part_idx[i]; }
+  const Cand c = block_best_256(best, sv, si);
+  // nothing beat the neutral start (every logit <= -3.4e38, NaN, or masked): index 0, as the
+  // reference kernel's (NEG_INF, 0) start does
+  if (threadIdx.x == 0) token_out[out_index] = c.i == 0xFFFFFFFFu ? 0u : c.i;
+}
+
+template <int MT, bool ARGMAX>
+int launch_gemv(F16GemvArgs a, int* parts_out, const char* op) {
+  const size_t lds = (size_t)MT * a.K * sizeof(float);
+  auto kern = f16w_gemv_kernel<MT, ARGMAX>;
+  DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+  // ~1024 workgroups when N allows (4 per CU), never more than kMaxParts partial candidates
+  int rpw = (int)std::max<int64_t>(1, dh::ceil_div(a.N, (int64_t)4 * 1024));
+  int grid = (int)dh::ceil_div(a.N, (int64_t)4 * rpw);
+  while (grid > kMaxParts) { rpw++; grid = (int)dh::ceil_div(a.N, (int64_t)4 * rpw); }
+  a.rows_per_wave = rpw;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, dh::stream(), a);
+  DH_CHECK_LAUNCH(op);
+  if (parts_out) *parts_out = grid;
+  return 0;
+}
+
+int check_f16w_shape(const char* op, int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0) return dh::fail(1, "[%s] Dimensions must be positive: M=%d, N=%d, K=%d", op, M, N, K);
+  if (K % 8) return dh::fail(1, "[%s] K=%d must be a multiple of 8 for f16 weights", op, K);
+  if ((size_t)K * sizeof(float) > 128 * 1024) return dh::fail(1, "[%s] K=%d too large (max 32768)", op, K);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int dh_f16w_matmul(const float* d_A, const void* d_W, float* d_C, int M, int N, int K, float alpha) {
+  const char* op = "dh_f16w_matmul";
+  DH_REQUIRE_INIT(op);
+  if (int rc = check_f16w_shape(op, M, N, K)) return rc;
+  if (!d_A || !d_W || !d_C) return dh::fail(1, "[%s] null pointer", op);
+  if (reinterpret_cast<uintptr_t>(d_W) & 15) return dh::fail(1, "[%s] weight pointer must be 16-byte aligned", op);
+  int mt = std::min(M, 4);
+  while (mt > 1 && (size_t)mt * K * sizeof(float) > 128 * 1024) mt--;
+  for (int m0 = 0; m0 < M; m0 += mt) {
+    F16GemvArgs a{};
+    const int cur = std::min(mt, M - m0);
+    a.A = d_A + (int64_t)m0 * K;
+    a.W = static_cast<const __half*>(d_W);
+    a.C = d_C + (int64_t)m0 * N;
+    a.N = N; a.K = K; a.alpha = alpha;
+    int rc;
+    switch (cur) {
+      case 1: rc = launch_gemv<1, false>(a, nullptr, op); break;
+      case 2: rc = launch_gemv<2, false>(a, nullptr, op); break;
+      case 3: rc = launch_gemv<3, false>(a, nullptr, op); break;
+      default: rc = launch_gemv<4, false>(a, nullptr, op); break;
+    }
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+size_t dh_lmhead_argmax_workspace_bytes(int vocab) {
+  (void)vocab;
+  return (size_t)kMaxParts * 8;
+}
+
+int dh_lmhead_argmax_f16(const float* d_h, const void* d_E, int vocab, int hidden, int64_t pad_token_id,
+                         float logit_softcap, void* d_workspace, uint32_t* d_token_out, int output_index,
+                         float* d_logits_out) {
+  const char* op = "dh_lmhead_argmax_f16";
+  DH_REQUIRE_INIT(op);
+  if (int rc = check_f16w_shape(op, 1, vocab, hidden)) return rc;
+  if (!d_h || !d_E || !d_workspace || !d_token_out) return dh::fail(1, "[%s] null pointer", op);
+  if (output_index < 0) return dh::fail(1, "[%s] outputIndex must be non-negative", op);
+  if (reinterpret_cast<uintptr_t>(d_E) & 15) return dh::fail(1, "[%s] weight pointer must be 16-byte aligned", op);
+  F16GemvArgs a{};
+  a.A = d_h; a.W = static_cast<const __half*>(d_E); a.C = d_logits_out;
+  a.N = vocab; a.K = hidden; a.alpha = 1.0f;
+  a.softcap = logit_softcap; a.pad_id = pad_token_id;
+  a.part_val = static_cast<float*>(d_workspace);
+  a.part_idx = reinterpret_cast<uint32_t*>(static_cast<char*>(d_workspace) + (size_t)kMaxParts * 4);
+  int parts = 0;
+  if (int rc = launch_gemv<1, true>(a, &parts, op)) return rc;
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, dh::stream(), a.part_val, a.part_idx, parts,
+                     d_token_out, output_index);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+size_t dh_argmax_workspace_bytes(void) { return (size_t)kMaxParts * 8; }
+
+int dh_argmax(const float* d_logits, int vocab, int64_t pad_token_id, float logit_softcap, void* d_workspace,
+              uint32_t* d_token_out, int output_index) {
+  const char* op = "dh_argmax";
+  DH_REQUIRE_INIT(op);
+  if (vocab <= 0) return dh::fail(1, "[%s] vocabSize must be positive, got %d", op, vocab);
+  if (!d_logits || !d_workspace || !d_token_out) return dh::fail(1, "[%s] null pointer", op);
+  if (output_index < 0) return dh::fail(1, "[%s] outputIndex must be non-negative", op);
+  float* pv = static_cast<float*>(d_workspace);
+  uint32_t* pi = reinterpret_cast<uint32_t*>(static_cast<char*>(d_workspace) + (size_t)kMaxParts * 4);
+  const int parts = (int)std::min<int64_t>(256, dh::ceil_div(vocab, 256));
+  hipLaunchKernelGGL(argmax_scan_kernel, dim3(parts), dim3(256), 0, dh::stream(), d_logits, vocab, pad_token_id,
+                     logit_softcap, pv, pi);
+  DH_CHECK_LAUNCH(op);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, dh::stream(), pv, pi, parts, d_token_out,
+                     output_index);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+}  // extern "C"

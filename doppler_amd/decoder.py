@@ -1,0 +1,172 @@
+"""Single-stream greedy decoder for a Q4_K transformer, built only from the C-ABI ops.
+
+Op order per layer follows the reference's execution graph for Qwen3-class models
+(src/config/conversion/qwen3/qwen-3-embedding-0-6b-q4k-ehf16-af32.json `execution.decode`,
+driven by src/inference/pipelines/text/generator-steps.js:588-820 decodeStep):
+
+    gather -> [ input_norm -> q,k,v (one fused Q4_K GEMV over the stacked rows) ->
+                q/k RMSNorm + RoPE + f16 KV write -> decode attention -> o_proj (+residual) ->
+                post_attn_norm -> gate,up + SiLU gate (fused) -> down_proj (+residual) ] x L
+           -> final_norm -> tied f16 LM head + argmax -> 4-byte token readback
+
+All buffers are allocated once; a step enqueues ~8 launches per layer on the library's
+stream and reads back one token id, the reference's only device->host crossing per token.
+"""
+import ctypes
+import math
+
+import numpy as np
+import torch
+
+from . import capi, synth
+
+_P = ctypes.c_void_p
+
+
+def _dev_bytes(arr):
+    """Upload a numpy array into a fresh torch.uint8 CUDA buffer."""
+    arr = np.ascontiguousarray(arr)
+    t = torch.from_numpy(arr.view(np.uint8).reshape(-1)).cuda()
+    return t
+
+
+class HipDecoder:
+    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq):
+        """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
+        layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
+        input_norm, post_attn_norm, q_norm, k_norm: f32); embed_bits: uint16 [vocab, hidden]."""
+        self.cfg = dict(cfg)
+        self.L = capi.init(torch.cuda.current_device())
+        c = self.cfg
+        self.max_seq = max_seq
+        H, Hkv, D, Hd, I = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"], c["inter"]
+        self.qs, self.ks = H * D, Hkv * D
+        self.layers = []
+        for l in layers:
+            d = {}
+            # q, k, v rows stacked: one GEMV produces the fused qkv vector the K8 kernel consumes
+            d["wqkv"] = _dev_bytes(np.concatenate([l["wq"], l["wk"], l["wv"]]))
+            d["wo"] = _dev_bytes(l["wo"])
+            d["wgate"] = _dev_bytes(l["wgate"])
+            d["wup"] = _dev_bytes(l["wup"])
+            d["wdown"] = _dev_bytes(l["wdown"])
+            for n in ("input_norm", "post_attn_norm", "q_norm", "k_norm"):
+                d[n] = _dev_bytes(l[n].astype(np.float32))
+            d["cache_k"] = torch.zeros(max_seq * self.ks, dtype=torch.float16, device="cuda")
+            d["cache_v"] = torch.zeros(max_seq * self.ks, dtype=torch.float16, device="cuda")
+            self.layers.append(d)
+        self.embed = _dev_bytes(embed_bits)
+        self.final_norm = _dev_bytes(final_norm.astype(np.float32))
+        self.cos = _dev_bytes(cos[:max_seq])
+        self.sin = _dev_bytes(sin[:max_seq])
+        f32 = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
+        self.x = f32(Hd)            # residual stream
+        self.x2 = f32(Hd)
+        self.normed = f32(Hd)
+        self.qkv = f32(self.qs + 2 * self.ks)
+        self.q = f32(self.qs)
+        self.attn = f32(self.qs)
+        self.act = f32(I)
+        self.logits = f32(c["vocab"])
+        self.token = torch.zeros(4, dtype=torch.int32, device="cuda")
+        self.ids = torch.zeros(4, dtype=torch.int32, device="cuda")
+        self.attn_ws = torch.zeros(int(self.L.dh_attn_decode_workspace_bytes(H, D, max_seq)), dtype=torch.uint8,
+                                   device="cuda")
+        self.lm_ws = torch.zeros(int(self.L.dh_lmhead_argmax_workspace_bytes(c["vocab"])), dtype=torch.uint8,
+                                 device="cuda")
+        self.scale = 1.0 / math.sqrt(D)
+        self._host_token = np.zeros(1, np.uint32)
+        torch.cuda.synchronize()
+
+    def weight_bytes_per_token(self, ctx):
+        """Algorithmic HBM bytes one decode step must read: all Q4_K weights, the f16 LM head
+        and the KV cache rows up to ctx."""
+        c = self.cfg
+        q4 = 0
+        for (n, k) in ((self.qs + 2 * self.ks, c["hidden"]), (c["hidden"], self.qs), (c["inter"], c["hidden"]),
+                       (c["inter"], c["hidden"]), (c["hidden"], c["inter"])):
+            q4 += synth.q4k_nbytes(n, k)
+        return c["layers"] * q4 + c["vocab"] * c["hidden"] * 2 + c["layers"] * 2 * self.ks * 2 * ctx
+
+    def enqueue_step(self, pos, want_logits=False, from_device_token=False):
+        """Enqueue one decode step for the token id in self.ids[0] (or the previous step's
+        argmax when from_device_token) at position `pos`.  No host synchronisation."""
+        L, c = self.L, self.cfg
+        ck = capi.check
+        H, Hkv, D, Hd, I = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"], c["inter"]
+        ids = self.token if from_device_token else self.ids
+        ck(L.dh_gather_f16(ids.data_ptr(), self.embed.data_ptr(), self.x.data_ptr(), 1, Hd, c["vocab"], 0))
+        x, x2 = self.x, self.x2
+        for d in self.layers:
+            ck(L.dh_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd,
+                            c["eps"], 0, None, None, None, 1.0))
+            ck(L.dh_q4k_matmul(self.normed.data_ptr(), capi.F32, d["wqkv"].data_ptr(), self.qkv.data_ptr(), capi.F32,
+                               1, self.qs + 2 * self.ks, Hd, 1.0, None))
+            ck(L.dh_qkv_norm_rope_kvwrite(self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
+                                          self.cos.data_ptr(), self.sin.data_ptr(), self.q.data_ptr(),
+                                          d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), 1, H, Hkv, D, pos, D, 0,
+                                          c["eps"], 0, pos * self.ks, int(c.get("qk_norm", 1))))
+            ck(L.dh_attn_decode(self.q.data_ptr(), d["cache_k"].data_ptr(), d["cache_v"].data_ptr(),
+                                self.attn.data_ptr(), H, Hkv, D, pos + 1, self.scale, 1, pos, 0.0, 0, 0,
+                                capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
+            ck(L.dh_q4k_matmul(self.attn.data_ptr(), capi.F32, d["wo"].data_ptr(), x2.data_ptr(), capi.F32, 1, Hd,
+                               self.qs, 1.0, x.data_ptr()))
+            ck(L.dh_rmsnorm(x2.data_ptr(), d["post_attn_norm"].data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd,
+                            c["eps"], 0, None, None, None, 1.0))
+            ck(L.dh_q4k_ffn_gate_up(self.normed.data_ptr(), d["wgate"].data_ptr(), d["wup"].data_ptr(),
+                                    self.act.data_ptr(), 1, Hd, I, capi.ACT_SILU, 1.0, 0.0))
+            ck(L.dh_q4k_matmul(self.act.data_ptr(), capi.F32, d["wdown"].data_ptr(), x.data_ptr(), capi.F32, 1, Hd, I,
+                               1.0, x2.data_ptr()))
+        ck(L.dh_rmsnorm(x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"],
+                        0, None, None, None, 1.0))
+        ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
+                                  self.lm_ws.data_ptr(), self.token.data_ptr(), 0,
+                                  self.logits.data_ptr() if want_logits else None))
+
+    def set_token(self, token):
+        self._host_token[0] = token
+        capi.check(self.L.dh_upload(self.ids.data_ptr(), 0, self._host_token.ctypes.data, 4))
+
+    def read_token(self):
+        capi.check(self.L.dh_download(self._host_token.ctypes.data, self.token.data_ptr(), 0, 4))
+        return int(self._host_token[0])
+
+    def step(self, token, pos, want_logits=False):
+        """One full step with the reference's single device->host crossing (the token id)."""
+        self.set_token(token)
+        self.enqueue_step(pos, want_logits)
+        return self.read_token()
+
+    def read_logits(self):
+        out = np.empty(self.cfg["vocab"], np.float32)
+        capi.check(self.L.dh_download(out.ctypes.data, self.logits.data_ptr(), 0, out.nbytes))
+        return out
+
+    def read_kv(self, layer, rows):
+        n = rows * self.ks
+        k = np.empty(n, np.uint16)
+        v = np.empty(n, np.uint16)
+        d = self.layers[layer]
+        capi.check(self.L.dh_download(k.ctypes.data, d["cache_k"].data_ptr(), 0, n * 2))
+        capi.check(self.L.dh_download(v.ctypes.data, d["cache_v"].data_ptr(), 0, n * 2))
+        return k, v
+
+
+def random_model(cfg, seed=0, max_seq=None):
+    """Random-init weights of a Q4_K decoder (config-4 recipe): Q4_K linears with the synthetic
+    block distribution, norm weights N(1, 0.02), tied f16 embedding N(0, 0.02)."""
+    H, Hkv, D, Hd, I = cfg["heads"], cfg["kv_heads"], cfg["head_dim"], cfg["hidden"], cfg["inter"]
+    qs, ks = H * D, Hkv * D
+    layers = []
+    for i in range(cfg["layers"]):
+        s = seed + 100 * (i + 1)
+        layers.append(dict(
+            wq=synth.q4k_tensor(qs, Hd, s + 1), wk=synth.q4k_tensor(ks, Hd, s + 2), wv=synth.q4k_tensor(ks, Hd, s + 3),
+            wo=synth.q4k_tensor(Hd, qs, s + 4), wgate=synth.q4k_tensor(I, Hd, s + 5),
+            wup=synth.q4k_tensor(I, Hd, s + 6), wdown=synth.q4k_tensor(Hd, I, s + 7),
+            input_norm=1 + synth.normal_f32(Hd, s + 8, 0.02), post_attn_norm=1 + synth.normal_f32(Hd, s + 9, 0.02),
+            q_norm=1 + synth.normal_f32(D, s + 10, 0.02), k_norm=1 + synth.normal_f32(D, s + 11, 0.02)))
+    embed = synth.normal_f16_bits((cfg["vocab"], Hd), seed + 7, 0.02)
+    final_norm = 1 + synth.normal_f32(Hd, seed + 8, 0.02)
+    cos, sin = synth.rope_tables(D, max_seq or cfg.get("max_seq", 4096), cfg.get("theta", 1e6))
+    return layers, embed, final_norm, cos, sin

@@ -1,0 +1,424 @@
+"""Python host mirror of the reference's op API for the quantized-inference hot path.
+
+Names, argument meaning and error behaviour follow the reference's JavaScript wrappers
+(src/gpu/kernels/index.js): `runMatmul`, `runAttention`, `runRMSNorm`, `runRoPE`,
+`runKVCacheWriteF32ToF16`, `runSplitQKVRMSNormRoPEQK`, `runSiLU`, `runSiLURowSplit`, `runGeLU`,
+`runResidualAdd`, `runGather`, `runFusedFFN`, `runArgmax`, `recordLmHeadArgmaxF16`, plus the
+handle helpers `createTensor` / `createWeightBuffer` and the pool calls `acquireBuffer` /
+`uploadData` / `readBuffer`.  Options are keyword arguments with the reference's camelCase
+names.  Every op goes through the C ABI of libdopplerhip.so; torch only provides device
+memory (a buffer is a torch.uint8 CUDA tensor) -- there is no torch or CPU compute path.
+"""
+import math
+
+import numpy as np
+import torch
+
+from . import capi
+from .capi import DopplerHipError
+
+QK_K = 256
+Q4K_BLOCK_BYTES = 144
+
+
+def padToQ4KBlock(size):
+    """src/config/schema/quantization.schema.js:26-28"""
+    return (size + QK_K - 1) // QK_K * QK_K
+
+
+class Tensor:
+    """src/gpu/tensor.js:7-19 createTensor: {buffer, dtype, shape, label}."""
+    __slots__ = ("buffer", "dtype", "shape", "label")
+
+    def __init__(self, buffer, dtype, shape, label=None):
+        self.buffer, self.dtype, self.shape, self.label = buffer, dtype, tuple(shape), label
+
+
+class WeightBuffer:
+    """src/gpu/weight-buffer.js:78-115 createWeightBuffer."""
+    __slots__ = ("buffer", "dtype", "layout", "shape", "label")
+
+    def __init__(self, buffer, dtype, layout, shape, label=None):
+        self.buffer, self.dtype, self.layout, self.shape, self.label = buffer, dtype, layout, tuple(shape), label
+
+
+def createTensor(buffer, dtype, shape, label=None):
+    return Tensor(buffer, dtype, shape, label)
+
+
+def createWeightBuffer(buffer, dtype, layout, shape, label=None):
+    return WeightBuffer(buffer, dtype, layout, shape, label)
+
+
+def _lib():
+    if not torch.cuda.is_available():
+        raise DopplerHipError("no GPU visible: the HIP path cannot run (there is no CPU fallback)")
+    return capi.init(torch.cuda.current_device())
+
+
+def _dev():
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+# ------------------------------------------------------------------ buffer pool mirror
+
+def acquireBuffer(size, usage=None, label=None):
+    """src/memory/buffer-pool.js:815 acquireBuffer(size, usage, label): zero-filled device bytes."""
+    _lib()
+    return torch.zeros(int(size), dtype=torch.uint8, device=_dev())
+
+
+def releaseBuffer(buffer):
+    return None   # torch's caching allocator owns the memory
+
+
+def uploadData(buffer, data, offset=0):
+    """src/memory/buffer-pool.js:863 uploadData(buffer, data, offset)."""
+    src = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+    if offset + src.size > buffer.numel():
+        raise DopplerHipError("uploadData: %d bytes at offset %d exceed buffer of %d" % (src.size, offset, buffer.numel()))
+    capi.check(_lib().dh_upload(buffer.data_ptr(), offset, src.ctypes.data, src.size))
+    return buffer
+
+
+def readBuffer(buffer, size=None, dtype=np.uint8):
+    """src/memory/buffer-pool.js:866 readBuffer(buffer, size): waits for queued work."""
+    size = buffer.numel() * buffer.element_size() if size is None else int(size)
+    out = np.empty(size, np.uint8)
+    capi.check(_lib().dh_download(out.ctypes.data, buffer.data_ptr(), 0, size))
+    return out.view(dtype)
+
+
+def tensorFromNumpy(arr, dtype=None, label=None):
+    """Upload a numpy array as a Tensor (f32 stays f32; uint16 is taken as f16 bits)."""
+    arr = np.ascontiguousarray(arr)
+    if dtype is None:
+        dtype = "f16" if arr.dtype in (np.uint16, np.float16) else "f32"
+    buf = acquireBuffer(max(arr.nbytes, 4))
+    uploadData(buf, arr)
+    return Tensor(buf, dtype, arr.shape, label)
+
+
+def readTensor(t, count=None):
+    n = int(np.prod(t.shape)) if count is None else count
+    if t.dtype == "f16":
+        return readBuffer(t.buffer, n * 2, np.uint16)
+    return readBuffer(t.buffer, n * 4, np.float32)
+
+
+def _buf(x):
+    return x.buffer if isinstance(x, (Tensor, WeightBuffer)) else x
+
+
+def _ptr(x):
+    return None if x is None else _buf(x).data_ptr()
+
+
+def _nbytes(x):
+    b = _buf(x)
+    return b.numel() * b.element_size()
+
+
+def _out(outputBuffer, nbytes):
+    if outputBuffer is not None:
+        if _nbytes(outputBuffer) < nbytes:
+            raise DopplerHipError("output buffer too small: %d < %d" % (_nbytes(outputBuffer), nbytes))
+        return _buf(outputBuffer)
+    return acquireBuffer(nbytes)
+
+
+def _act_code(activation, op):
+    if activation == "silu":
+        return capi.ACT_SILU
+    if activation in ("gelu", "gelu_tanh", "geglu"):
+        return capi.ACT_GELU
+    raise DopplerHipError("[%s] unsupported activation %r" % (op, activation))
+
+
+# ------------------------------------------------------------------ matmul
+
+def runMatmul(A, B, M, N, K, alpha=1.0, outputBuffer=None, transposeB=True, outputDtype=None, role=None,
+              layerIdx=None, residualTensor=None, **_ignored):
+    """src/gpu/kernels/matmul.js:659 runMatmul(A, B, M, N, K, options) for q4k ('row') and f16
+    weights ([N, K] row-major, transposeB true)."""
+    op = "runMatmul"
+    for v in (M, N, K):
+        if not isinstance(v, (int, np.integer)):
+            raise DopplerHipError("[%s] Invalid dimensions: M=%s, N=%s, K=%s" % (op, M, N, K))
+    if M <= 0 or N <= 0 or K <= 0:
+        raise DopplerHipError("[%s] Dimensions must be positive: M=%s, N=%s, K=%s" % (op, M, N, K))
+    if outputDtype not in ("f16", "f32"):
+        raise DopplerHipError('[%s] options.outputDtype is required and must be "f16" or "f32", got %s.' % (op, outputDtype))
+    bdtype = B.dtype if isinstance(B, (Tensor, WeightBuffer)) else None
+    if not bdtype:
+        raise DopplerHipError("[%s] B dtype is required for matmul dispatch%s." % (op, " (role=%s)" % role if role else ""))
+    if A.dtype != "f32":
+        raise DopplerHipError("[%s] f32 activations required, got %s" % (op, A.dtype))
+    if _nbytes(A) < M * K * 4:
+        raise DopplerHipError("[%s] A buffer too small: %d < %d (M=%d, K=%d, aDtype=f32)" % (op, _nbytes(A), M * K * 4, M, K))
+    L = _lib()
+    if bdtype == "q4k":
+        need = N * ((K + QK_K - 1) // QK_K) * Q4K_BLOCK_BYTES
+        if _nbytes(B) < need:
+            raise DopplerHipError("[%s] B buffer too small: %d < %d (N=%d, K=%d, bDtype=q4k, transposeB=%s)"
+                                  % (op, _nbytes(B), need, N, K, transposeB))
+        out = _out(outputBuffer, M * N * (2 if outputDtype == "f16" else 4))
+        capi.check(L.dh_q4k_matmul(_ptr(A), capi.F32, _ptr(B), out.data_ptr(),
+                                   capi.F16 if outputDtype == "f16" else capi.F32, M, N, K, alpha,
+                                   _ptr(residualTensor)))
+        return Tensor(out, outputDtype, (M, N), "matmul_output")
+    if bdtype == "f16":
+        if transposeB not in (True, "auto"):
+            raise DopplerHipError("[%s] f16 weights must be row-major [N, K] (transposeB=true)" % op)
+        if outputDtype != "f32" or residualTensor is not None:
+            raise DopplerHipError("[%s] f16-weight matmul supports f32 output without residual only" % op)
+        if _nbytes(B) < N * K * 2:
+            raise DopplerHipError("[%s] B buffer too small: %d < %d (N=%d, K=%d, bDtype=f16, transposeB=true)"
+                                  % (op, _nbytes(B), N * K * 2, N, K))
+        out = _out(outputBuffer, M * N * 4)
+        capi.check(L.dh_f16w_matmul(_ptr(A), _ptr(B), out.data_ptr(), M, N, K, alpha))
+        return Tensor(out, "f32", (M, N), "matmul_output")
+    raise DopplerHipError("[%s] weight dtype %r is not supported by the HIP path" % (op, bdtype))
+
+
+def runDequantQ4K(W, numBlocks, outputBuffer=None):
+    """Dequantize Q4_K super-blocks to f32 (src/gpu/kernels/dequant.js dequantize, q4k -> f32)."""
+    if _nbytes(W) < numBlocks * Q4K_BLOCK_BYTES:
+        raise DopplerHipError("[runDequantQ4K] weight buffer too small")
+    out = _out(outputBuffer, numBlocks * QK_K * 4)
+    capi.check(_lib().dh_q4k_dequant(_ptr(W), numBlocks, out.data_ptr()))
+    return Tensor(out, "f32", (numBlocks * QK_K,), "dequant_output")
+
+
+def runFusedFFN(input, W_gate, W_up, hiddenSize, intermediateSize, batchSize=1, activation="silu",
+                alpha=1.0, outputBuffer=None, swigluLimit=None, **_ignored):
+    """src/gpu/kernels/fused_ffn.js:501 runFusedFFN."""
+    gd = W_gate.dtype if isinstance(W_gate, (Tensor, WeightBuffer)) else None
+    ud = W_up.dtype if isinstance(W_up, (Tensor, WeightBuffer)) else None
+    if not gd or not ud:
+        raise DopplerHipError("Fused FFN requires explicit gate/up weight dtypes")
+    if gd != ud:
+        raise DopplerHipError("Fused FFN requires matching gate/up dtypes (gate=%s, up=%s)" % (gd, ud))
+    if gd != "q4k":
+        raise DopplerHipError("Fused FFN does not support %s weights" % gd)
+    if input.dtype != "f32":
+        raise DopplerHipError("Fused FFN requires f32 activations")
+    out = _out(outputBuffer, batchSize * intermediateSize * 4)
+    capi.check(_lib().dh_q4k_ffn_gate_up(_ptr(input), _ptr(W_gate), _ptr(W_up), out.data_ptr(), batchSize,
+                                         hiddenSize, intermediateSize, _act_code(activation, "FusedFFN"),
+                                         alpha, float(swigluLimit or 0.0) if activation == "silu" else 0.0))
+    return Tensor(out, "f32", (batchSize, intermediateSize), "fused_ffn_output")
+
+
+# ------------------------------------------------------------------ attention
+
+def attentionWorkspaceBytes(numHeads, headDim, kvLen):
+    return int(capi.load().dh_attn_decode_workspace_bytes(numHeads, headDim, kvLen))
+
+
+def runAttention(Q, K, V, mask, numHeads, headDim, seqLen=1, kvLen=None, numKVHeads=None, scale=None,
+                 causal=True, startPos=0, outputBuffer=None, attnSoftcap=0, slidingWindow=0, kvStart=0,
+                 kvLayout="contiguous", workspace=None, **_ignored):
+    """src/gpu/kernels/attention.js:2007 runAttention, decode (seqLen == 1) over an f16 KV cache."""
+    kvLen = seqLen if kvLen is None else kvLen
+    numKVHeads = numHeads if numKVHeads is None else numKVHeads
+    scale = 1.0 / math.sqrt(headDim) if scale is None else scale
+    if seqLen != 1:
+        raise DopplerHipError("[Attention] only decode (seqLen=1) runs on the HIP path, got seqLen=%d" % seqLen)
+    if mask is not None:
+        raise DopplerHipError("[Attention] explicit masks are not supported on the decode path")
+    if Q.dtype != "f32" or K.dtype != "f16" or V.dtype != "f16":
+        raise DopplerHipError("[Attention] decode path needs f32 Q and f16 K/V (got %s/%s/%s)" % (Q.dtype, K.dtype, V.dtype))
+    layouts = {"contiguous": capi.KV_CONTIGUOUS, "ring": capi.KV_RING}
+    if kvLayout not in layouts:
+        raise DopplerHipError("[Attention] kvLayout %r is not supported by the HIP path" % (kvLayout,))
+    rows = slidingWindow if kvLayout == "ring" else kvStart + kvLen
+    if kvLen > 0 and min(_nbytes(K), _nbytes(V)) < rows * numKVHeads * headDim * 2:
+        raise DopplerHipError("[Attention] KV buffer smaller than kvLen=%d rows" % kvLen)
+    padded = padToQ4KBlock(numHeads * headDim)
+    out = _out(outputBuffer, seqLen * padded * 4)
+    L = _lib()
+    if workspace is None:
+        workspace = acquireBuffer(attentionWorkspaceBytes(numHeads, headDim, max(kvLen, 1)))
+    capi.check(L.dh_attn_decode(_ptr(Q), _ptr(K), _ptr(V), out.data_ptr(), numHeads, numKVHeads, headDim, kvLen,
+                                scale, int(bool(causal)), startPos, float(attnSoftcap), slidingWindow, kvStart,
+                                layouts[kvLayout], _ptr(workspace)))
+    return Tensor(out, "f32", (seqLen, numHeads, headDim), "attention_output")
+
+
+# ------------------------------------------------------------------ norm / rope / kv
+
+def runRMSNorm(input, weight, eps, batchSize=1, hiddenSize=None, residual=None, outputBuffer=None,
+               rmsNormWeightOffset=False, preResidual=None, residualSumOutput=None, outputScale=None, **_ignored):
+    """src/gpu/kernels/rmsnorm.js:146 runRMSNorm."""
+    if input.dtype != "f32":
+        raise DopplerHipError("[RMSNorm] f32 input required, got %s" % input.dtype)
+    hidden = hiddenSize if hiddenSize else input.shape[-1]
+    scale = 1.0 if outputScale is None else float(outputScale)
+    if not math.isfinite(scale):
+        raise DopplerHipError('[RMSNorm] outputScale must be finite; got "%s".' % outputScale)
+    wdt = capi.F32
+    if weight is not None:
+        wd = weight.dtype if isinstance(weight, (Tensor, WeightBuffer)) else "f32"
+        wdt = capi.F16 if wd == "f16" else capi.F32
+        if _nbytes(weight) < hidden * (2 if wdt == capi.F16 else 4):
+            raise DopplerHipError("[RMSNorm] weight buffer smaller than hiddenSize=%d" % hidden)
+    out = _out(outputBuffer, batchSize * padToQ4KBlock(hidden) * 4)
+    capi.check(_lib().dh_rmsnorm(_ptr(input), _ptr(weight), wdt, out.data_ptr(), batchSize, hidden, eps,
+                                 int(bool(rmsNormWeightOffset)), _ptr(preResidual), _ptr(residual),
+                                 _ptr(residualSumOutput) if preResidual is not None else None, scale))
+    return Tensor(out, "f32", (batchSize, hidden), "rmsnorm_output")
+
+
+def runRoPE(input, freqsCos, freqsSin, seqLen, numHeads=1, headDim=64, rotaryDim=None, pairSpanDim=None,
+            interleaved=False, startPos=0, **_ignored):
+    """src/gpu/kernels/rope.js:108 runRoPE: in place, returns a Tensor aliasing the input."""
+    rotaryDim = headDim if rotaryDim is None else rotaryDim
+    pairSpanDim = rotaryDim if pairSpanDim is None else pairSpanDim
+    if input.dtype != "f32":
+        raise DopplerHipError("[RoPE] f32 input required, got %s" % input.dtype)
+    need = (startPos + seqLen) * (rotaryDim // 2) * 4
+    if min(_nbytes(freqsCos), _nbytes(freqsSin)) < need:
+        raise DopplerHipError("[RoPE] cos/sin tables smaller than %d bytes" % need)
+    capi.check(_lib().dh_rope(_ptr(input), _ptr(freqsCos), _ptr(freqsSin), seqLen, numHeads, headDim, rotaryDim,
+                              pairSpanDim, int(bool(interleaved)), startPos))
+    return Tensor(input.buffer, input.dtype, input.shape, "rope_output")
+
+
+def runKVCacheWriteF32ToF16(keys, values, outputKeys, outputValues, srcOffset=0, dstOffset=0, elementCount=None):
+    """src/gpu/kernels/kv-cache-write.js:107 runKVCacheWriteF32ToF16."""
+    for name, v in (("srcOffset", srcOffset), ("dstOffset", dstOffset), ("elementCount", elementCount)):
+        if not isinstance(v, (int, np.integer)) or v < 0:
+            raise DopplerHipError("KV cache write %s must be a non-negative integer, got %s." % (name, v))
+    if elementCount == 0:
+        return
+    for buf, off, bpe, label in ((keys, srcOffset, 4, "keys input"), (values, srcOffset, 4, "values input"),
+                                 (outputKeys, dstOffset, 2, "keys output"), (outputValues, dstOffset, 2, "values output")):
+        if (off + elementCount) * bpe > _nbytes(buf):
+            raise DopplerHipError("KV cache write %s buffer is smaller than requested range (%d > %d bytes)."
+                                  % (label, (off + elementCount) * bpe, _nbytes(buf)))
+    capi.check(_lib().dh_kv_write_f16(_ptr(keys), _ptr(values), _ptr(outputKeys), _ptr(outputValues), srcOffset,
+                                      dstOffset, elementCount))
+
+
+def runSplitQKVRMSNormRoPEQK(qkvTensor, qWeight, kWeight, freqsCos, freqsSin, eps, numTokens=None, numHeads=None,
+                             numKVHeads=None, headDim=None, qSize=None, kSize=None, vSize=None, startPos=0,
+                             rotaryDim=None, interleaved=False, rmsNormWeightOffset=False, f16KVCacheWrite=None,
+                             **_ignored):
+    """src/gpu/kernels/split-qkv-rmsnorm-rope-qk.js:244 with f16KVCacheWrite = {keysBuffer,
+    valuesBuffer, dstOffset}: returns {Q, K: None, V: None, wroteF16KVCache: True}."""
+    rotaryDim = headDim if rotaryDim is None else rotaryDim
+    for name, v in (("numTokens", numTokens), ("numHeads", numHeads), ("numKVHeads", numKVHeads), ("headDim", headDim),
+                    ("qSize", qSize), ("kSize", kSize), ("vSize", vSize)):
+        if not isinstance(v, (int, np.integer)) or v <= 0:
+            raise DopplerHipError("split_qkv_rmsnorm_rope_qk %s must be a positive integer, got %s." % (name, v))
+    if qSize != numHeads * headDim or kSize != numKVHeads * headDim or vSize != kSize:
+        raise DopplerHipError("split_qkv_rmsnorm_rope_qk sizes do not match heads*headDim")
+    if qkvTensor.dtype != "f32":
+        raise DopplerHipError("split_qkv_rmsnorm_rope_qk requires f32 QKV input, got %s." % qkvTensor.dtype)
+    if f16KVCacheWrite is None:
+        raise DopplerHipError("split_qkv_rmsnorm_rope_qk: the HIP path writes K/V to the f16 cache (f16KVCacheWrite is required)")
+    dst = f16KVCacheWrite["dstOffset"]
+    need = (dst + numTokens * numKVHeads * headDim) * 2
+    if _nbytes(f16KVCacheWrite["keysBuffer"]) < need or _nbytes(f16KVCacheWrite["valuesBuffer"]) < need:
+        raise DopplerHipError("split_qkv_rmsnorm_rope_qk f16 KV cache is smaller than %d bytes" % need)
+    qRows = numTokens * numHeads
+    q_out = acquireBuffer(qRows * padToQ4KBlock(headDim) * 4)
+    capi.check(_lib().dh_qkv_norm_rope_kvwrite(_ptr(qkvTensor), _ptr(qWeight), _ptr(kWeight), _ptr(freqsCos),
+                                               _ptr(freqsSin), q_out.data_ptr(), _ptr(f16KVCacheWrite["keysBuffer"]),
+                                               _ptr(f16KVCacheWrite["valuesBuffer"]), numTokens, numHeads, numKVHeads,
+                                               headDim, startPos, rotaryDim, int(bool(interleaved)), eps,
+                                               int(bool(rmsNormWeightOffset)), dst, 1))
+    return dict(Q=Tensor(q_out, "f32", (qRows, headDim), "split_qkv_rmsnorm_rope_qk_q_output"), K=None, V=None,
+                wroteF16KVCache=True)
+
+
+# ------------------------------------------------------------------ elementwise
+
+def runResidualAdd(a, b, size, outputBuffer=None, outputScale=None, **_ignored):
+    """src/gpu/kernels/residual.js:210 runResidualAdd: (a + b) * outputScale."""
+    scale = 1.0 if outputScale is None else float(outputScale)
+    if not math.isfinite(scale):
+        raise DopplerHipError('[Residual] outputScale must be finite; got "%s".' % outputScale)
+    out = _out(outputBuffer, size * 4)
+    capi.check(_lib().dh_residual_add(_ptr(a), _ptr(b), out.data_ptr(), size, scale))
+    return Tensor(out, "f32", (size,), "residual_output")
+
+
+def runGather(indices, embeddings, numTokens, hiddenSize, vocabSize, outputBuffer=None, embeddingDtype=None,
+              outputDtype=None, transpose=False, indexOffset=0, **_ignored):
+    """src/gpu/kernels/gather.js:370 runGather for f16 tables -> f32 rows."""
+    if embeddingDtype is None:
+        raise DopplerHipError("[Gather] embeddingDtype is required.")
+    if outputDtype is None:
+        raise DopplerHipError("[Gather] outputDtype is required.")
+    if embeddingDtype != "f16" or outputDtype != "f32" or transpose:
+        raise DopplerHipError('[Gather] unsupported embeddingDtype="%s" / outputDtype="%s" on the HIP path.' % (embeddingDtype, outputDtype))
+    out = _out(outputBuffer, numTokens * padToQ4KBlock(hiddenSize) * 4)
+    capi.check(_lib().dh_gather_f16(_ptr(indices), _ptr(embeddings), out.data_ptr(), numTokens, hiddenSize, vocabSize,
+                                    indexOffset))
+    return Tensor(out, "f32", (numTokens, hiddenSize), "gather_output")
+
+
+def runSiLU(input, size=None, gate=None, outputBuffer=None, swigluLimit=None, **_ignored):
+    """src/gpu/kernels/silu.js:95 runSiLU with `gate`: silu(gate) * input."""
+    if gate is None:
+        raise DopplerHipError("[SiLU] the HIP path implements the gated form only (options.gate)")
+    n = size or _nbytes(input) // 4
+    out = _out(outputBuffer, n * 4)
+    capi.check(_lib().dh_act_gate(_ptr(gate), _ptr(input), out.data_ptr(), n, capi.ACT_SILU, float(swigluLimit or 0.0)))
+    return Tensor(out, "f32", (n,), "silu_output")
+
+
+def runGeLU(input, size=None, gate=None, outputBuffer=None, **_ignored):
+    """src/gpu/kernels/gelu.js:49 runGeLU with `gate`: gelu_tanh(gate) * input."""
+    if gate is None:
+        raise DopplerHipError("[GeLU] the HIP path implements the gated form only (options.gate)")
+    n = size or _nbytes(input) // 4
+    out = _out(outputBuffer, n * 4)
+    capi.check(_lib().dh_act_gate(_ptr(gate), _ptr(input), out.data_ptr(), n, capi.ACT_GELU, 0.0))
+    return Tensor(out, "f32", (n,), "gelu_output")
+
+
+def runSiLURowSplit(input, numTokens=None, dim=None, activation="silu", outputBuffer=None, swigluLimit=None):
+    """src/gpu/kernels/silu.js:230 runSiLURowSplit: [T, 2*dim] -> act(gate) * up."""
+    out = _out(outputBuffer, numTokens * dim * 4)
+    code = _act_code(activation, "SiLU row-split")
+    capi.check(_lib().dh_act_gate_rowsplit(_ptr(input), out.data_ptr(), numTokens, dim, code,
+                                           float(swigluLimit or 0.0) if activation == "silu" else 0.0))
+    return Tensor(out, "f32", (numTokens, dim), "silu_rowsplit_output")
+
+
+def runArgmax(logits, vocabSize, padTokenId=None, logitSoftcap=0.0, logitsDtype="f32", outputBuffer=None,
+              outputIndex=0, readback=True):
+    """src/gpu/kernels/sample.js:334 runArgmax: returns the token id (reads it back)."""
+    if logitsDtype != "f32":
+        raise DopplerHipError("[Argmax] logitsDtype %r is not supported on the HIP path" % (logitsDtype,))
+    L = _lib()
+    ws = acquireBuffer(int(L.dh_argmax_workspace_bytes()))
+    out = _out(outputBuffer, max(4, (outputIndex + 1) * 4))
+    capi.check(L.dh_argmax(_ptr(logits), vocabSize, -1 if padTokenId is None else padTokenId, logitSoftcap,
+                           ws.data_ptr(), out.data_ptr(), outputIndex))
+    if not readback:
+        return out
+    return int(readBuffer(out, (outputIndex + 1) * 4, np.uint32)[outputIndex])
+
+
+def recordLmHeadArgmaxF16(recorder, inputTensor, lmHead, vocabSize=None, hiddenSize=None, padTokenId=None,
+                          logitSoftcap=0.0, outputBuffer=None, outputIndex=0, logitsOutput=None):
+    """src/gpu/kernels/lm-head-argmax.js:304 recordLmHeadArgmaxF16: returns the output buffer
+    (token at outputIndex).  `recorder` is accepted for signature parity and unused: every op
+    already enqueues in order on one stream."""
+    if inputTensor.dtype != "f32":
+        raise DopplerHipError('[LmHeadArgmax] input tensor must be f32, got "%s".' % inputTensor.dtype)
+    L = _lib()
+    ws = acquireBuffer(int(L.dh_lmhead_argmax_workspace_bytes(vocabSize)))
+    out = _out(outputBuffer, max(4, (outputIndex + 1) * 4))
+    capi.check(L.dh_lmhead_argmax_f16(_ptr(inputTensor), _ptr(lmHead), vocabSize, hiddenSize,
+                                      -1 if padTokenId is None else padTokenId, logitSoftcap, ws.data_ptr(),
+                                      out.data_ptr(), outputIndex, _ptr(logitsOutput)))
+    return out
+
+
+def sync():
+    capi.check(_lib().dh_sync())

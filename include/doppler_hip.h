@@ -1,0 +1,190 @@
+/*
+ * doppler_hip.h -- C ABI of libdopplerhip.so: the MI355X (gfx950) implementation of
+ * Doppler's quantized-inference ops.
+ *
+ * Every entry point below replaces one op of the reference's kernel API
+ * (src/gpu/kernels/index.js, re-exported by src/gpu/kernel-selector.js:1-12); the
+ * reference function it stands in for is cited on each declaration.  The reference's ops
+ * are `runX(...)` / `recordX(recorder, ...)` pairs that enqueue on one GPUQueue; here
+ * every op enqueues on one HIP stream (the library's own, which orders itself against
+ * the legacy default stream, or the one given to dh_set_stream) and returns at once.  Ops never allocate: outputs are caller-provided
+ * device pointers, as when the reference's callers pass `outputBuffer`.
+ *
+ * Conventions
+ *   - all pointers named d_* are device pointers (from dh_malloc or any hipMalloc);
+ *   - return value 0 = success, non-zero = failure with a message in dh_last_error()
+ *     (the reference throws `new Error('[Op] ...')`: the Node addon turns a non-zero
+ *     code into exactly such an exception);
+ *   - shapes are validated on the host before any launch; an unsupported combination
+ *     fails closed (no silent fallback), like src/gpu/kernels/matmul-selection.js:528-539;
+ *   - dtype codes: DH_F32 / DH_F16 for activations, Q4_K weights are always the raw
+ *     llama.cpp block_q4_K rows the reference's loader uploads
+ *     (src/loader/tensors/tensor-loader.js:540-555): W[N,K] = N*ceil(K/256) blocks of
+ *     144 bytes, row n at byte n*ceil(K/256)*144.
+ */
+#ifndef DOPPLER_HIP_H
+#define DOPPLER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DH_F32 0
+#define DH_F16 1
+
+#define DH_ACT_SILU 0
+#define DH_ACT_GELU 1
+
+#define DH_KV_CONTIGUOUS 0
+#define DH_KV_RING 1
+
+/* ---- device, memory, stream (reference: src/gpu/device.js:605-700 initDevice,
+ *      src/memory/buffer-pool.js:815-869 acquireBuffer/releaseBuffer/uploadData/readBuffer,
+ *      src/gpu/command-recorder.js:499-560 submit/submitAndWait) ---- */
+int dh_init(int device_ordinal);
+int dh_shutdown(void);
+const char* dh_last_error(void);
+/* Use a caller-owned hipStream_t for all following ops (NULL: back to the library's). */
+int dh_set_stream(void* hip_stream);
+void* dh_get_stream(void);
+int dh_malloc(size_t bytes, void** d_out);
+int dh_free(void* d_ptr);
+int dh_upload(void* d_dst, size_t dst_offset, const void* host_src, size_t bytes);
+int dh_download(void* host_dst, const void* d_src, size_t src_offset, size_t bytes); /* waits */
+int dh_copy(void* d_dst, size_t dst_offset, const void* d_src, size_t src_offset, size_t bytes);
+int dh_fill_zero(void* d_dst, size_t offset, size_t bytes);
+int dh_sync(void);
+/* Timestamps on the op stream (reference: CommandRecorder timestamp-query profiling,
+ * src/gpu/command-recorder.js:116-140,728). dh_event_elapsed_ms waits for `stop`. */
+int dh_event_create(void** ev_out);
+int dh_event_record(void* ev);
+int dh_event_elapsed_ms(void* start, void* stop, float* ms_out);
+int dh_event_destroy(void* ev);
+
+/* ---- Q4_K ---- */
+
+/* Dequantize `num_blocks` super-blocks to f32 (bit-exact with
+ * tests/kernels/reference/dequant.js:253-300 dequantizeQ4_KBlockRef). */
+int dh_q4k_dequant(const void* d_W, int64_t num_blocks, float* d_out);
+
+/* C[M,N] = alpha * A[M,K] . dequant(W)[N,K]^T (+ residual[M,N]).
+ * Replaces runMatmul/recordMatmul for Q4_K weights, src/gpu/kernels/matmul.js:659-666
+ * (kernels fused_matmul_q4.wgsl:122-258, fused_matmul_q4_batched.wgsl:123-194,
+ * fused_matmul_q4_prefill_tiled_f16.wgsl:119-261).  A is f32 (a_dtype DH_F32); C is f32 or
+ * f16 (c_dtype).  K need not be a multiple of 256: the padded tail of each row's last
+ * block is ignored.  d_residual (may be NULL) is added after alpha, as the reference's
+ * `residualTensor` option does.  M = 1..8 takes the HBM-bound GEMV path, larger M the
+ * MFMA GEMM path. */
+int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int c_dtype,
+                  int M, int N, int K, float alpha, const void* d_residual);
+
+/* out[M,inter] = clamp(act(x.Wgate^T) * (x.Wup^T) * alpha).
+ * Replaces runFusedFFN/recordFusedFFN, src/gpu/kernels/fused_ffn.js:501,605
+ * (fused_ffn_q4k.wgsl:129-363).  clamp (swigluLimit) applies to DH_ACT_SILU only;
+ * 0 disables it. */
+int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup, float* d_out,
+                       int M, int hidden, int inter, int activation, float alpha,
+                       float swiglu_limit);
+
+/* ---- dense f16-weight GEMV (LM head) ----
+ * C[M,N] = alpha * A[M,K] . f32(W[N,K])^T, W row-major f16.  Replaces the f16-weight branch
+ * of runMatmul (matmul_gemv_subgroup.wgsl) used by recordLogitsGPU,
+ * src/inference/pipelines/text/logits/gpu.js:1122-1157. */
+int dh_f16w_matmul(const float* d_A, const void* d_W, float* d_C, int M, int N, int K,
+                   float alpha);
+
+/* Final-logit GEMV fused with greedy argmax: token = argmax_v softcap(h . E[v,:]).
+ * Replaces recordLmHeadArgmaxF16, src/gpu/kernels/lm-head-argmax.js:304-315
+ * (lm_head_argmax_f16.wgsl:53-147).  Ties go to the lowest index; pad_token_id < 0 = none.
+ * d_workspace needs dh_lmhead_argmax_workspace_bytes(vocab) bytes; d_logits_out may be NULL. */
+size_t dh_lmhead_argmax_workspace_bytes(int vocab);
+int dh_lmhead_argmax_f16(const float* d_h, const void* d_E, int vocab, int hidden,
+                         int64_t pad_token_id, float logit_softcap, void* d_workspace,
+                         uint32_t* d_token_out, int output_index, float* d_logits_out);
+
+/* ---- attention ----
+ * Decode attention of one query token over an f16 KV cache.  Replaces
+ * runAttention/recordAttention for seqLen == 1, src/gpu/kernels/attention.js:2007-2030
+ * (attention_decode_online_f16kv.wgsl:84-243).  Q f32 [H][D], K/V f16 [pos][Hkv][D],
+ * O f32 [H][D].  kv_layout DH_KV_RING reads row (kv_start+k) % sliding_window.
+ * d_workspace needs dh_attn_decode_workspace_bytes(H, D, kv_len) bytes (split-K partials). */
+size_t dh_attn_decode_workspace_bytes(int H, int D, int kv_len);
+int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H,
+                   int Hkv, int D, int kv_len, float scale, int causal, int start_pos,
+                   float softcap, int sliding_window, int kv_start, int kv_layout,
+                   void* d_workspace);
+
+/* ---- normalisation / rotary / KV ---- */
+
+/* y = x' * rsqrt(mean(x'^2)+eps) * (w | 1+w) [+ post_residual] * output_scale with
+ * x' = x (+ pre_residual); optional side output prenorm_out = x'.  Replaces
+ * runRMSNorm/recordRMSNorm, src/gpu/kernels/rmsnorm.js:146-297 (rmsnorm.wgsl:120-187).
+ * weight_dtype DH_F32 or DH_F16; d_weight NULL = all ones. */
+int dh_rmsnorm(const float* d_x, const void* d_weight, int weight_dtype, float* d_out,
+               int batch, int hidden, float eps, int weight_offset, const float* d_pre_residual,
+               const float* d_post_residual, float* d_prenorm_out, float output_scale);
+
+/* In-place rotary embedding on x[seq][heads][head_dim] with host-built tables
+ * cos/sin[max_seq][rotary_dim/2].  Replaces runRoPE/recordRoPE,
+ * src/gpu/kernels/rope.js:108-114 (rope.wgsl:63-106). */
+int dh_rope(float* d_x, const float* d_cos, const float* d_sin, int seq, int heads,
+            int head_dim, int rotary_dim, int pair_span_dim, int interleaved, int start_pos);
+
+/* From fused qkv[T][(H+2Hkv)*D]: per-head RMSNorm (q/k weights) -> RoPE -> Q out f32,
+ * K and V narrowed to f16 straight into the caches at element kv_dst_offset.  Replaces
+ * recordSplitQKVRMSNormRoPEQK with f16KVCacheWrite,
+ * src/gpu/kernels/split-qkv-rmsnorm-rope-qk.js:244-250
+ * (split_qkv_rmsnorm_rope_qk_f16kv_cache.wgsl:168-217).  use_norm 0 skips the RMSNorm
+ * (plain RoPE + KV write, i.e. recordRoPE x2 + recordKVCacheWriteF32ToF16). */
+int dh_qkv_norm_rope_kvwrite(const float* d_qkv, const float* d_q_weight, const float* d_k_weight,
+                             const float* d_cos, const float* d_sin, float* d_q_out,
+                             void* d_cache_k, void* d_cache_v, int T, int H, int Hkv, int D,
+                             int start_pos, int rotary_dim, int interleaved, float eps,
+                             int weight_offset, int64_t kv_dst_offset, int use_norm);
+
+/* cache[dst+i] = f16(src[src_off+i]) for K and V.  Replaces
+ * runKVCacheWriteF32ToF16, src/gpu/kernels/kv-cache-write.js:107-126
+ * (kv_cache_write_f32_to_f16.wgsl:18-32). */
+int dh_kv_write_f16(const float* d_k, const float* d_v, void* d_cache_k, void* d_cache_v,
+                    int64_t src_offset, int64_t dst_offset, int64_t count);
+
+/* ---- elementwise glue ---- */
+
+/* out = (a + b) * scale.  Replaces runResidualAdd, src/gpu/kernels/residual.js:210-216
+ * (residual.wgsl:24-31). */
+int dh_residual_add(const float* d_a, const float* d_b, float* d_out, int64_t n, float scale);
+
+/* out[t,:] = f32(E[ids[t + index_offset], :]) (zero row when the id is outside the
+ * vocabulary).  Replaces runGather for f16 tables, src/gpu/kernels/gather.js:370-391
+ * (gather_f16.wgsl:35-66). */
+int dh_gather_f16(const uint32_t* d_ids, const void* d_table, float* d_out, int T, int hidden,
+                  int vocab, int index_offset);
+
+/* out = clamp(act(gate) * up).  Replaces runSiLU with `gate` (src/gpu/kernels/silu.js:95,
+ * silu.wgsl:100-106) and runGeLU with `gate` (gelu.wgsl:60-65). */
+int dh_act_gate(const float* d_gate, const float* d_up, float* d_out, int64_t n, int activation,
+                float swiglu_limit);
+
+/* Row-split form: in[T][2*dim] -> out[T][dim].  Replaces runSiLURowSplit,
+ * src/gpu/kernels/silu.js:230-288 (silu.wgsl:83-98, gelu.wgsl:37-52). */
+int dh_act_gate_rowsplit(const float* d_in, float* d_out, int T, int dim, int activation,
+                         float swiglu_limit);
+
+/* Greedy argmax over f32 logits, ties to the lowest index, optional pad id (<0: none) and
+ * soft cap.  Replaces runArgmax/recordArgmax, src/gpu/kernels/sample.js:258-341
+ * (sample.wgsl:311-400).  d_workspace needs dh_argmax_workspace_bytes() bytes. */
+size_t dh_argmax_workspace_bytes(void);
+int dh_argmax(const float* d_logits, int vocab, int64_t pad_token_id, float logit_softcap,
+              void* d_workspace, uint32_t* d_token_out, int output_index);
+
+/* f32 <-> f16 casts.  Replaces castF32ToF16/castF16ToF32, src/gpu/kernels/cast.js:98-116. */
+int dh_cast_f32_to_f16(const float* d_in, void* d_out, int64_t n);
+int dh_cast_f16_to_f32(const void* d_in, float* d_out, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DOPPLER_HIP_H */

@@ -1,0 +1,384 @@
+"""GPU parity tests: every op goes through the C ABI (doppler_amd.ops -> libdopplerhip.so)
+and is compared with the CPU oracle on the same seeded inputs.
+
+Bars (BASELINE north star): bit-exact for Q4_K unpacking / dequantized weights, integer
+results (argmax, gather, f16 narrowing); relative L2 <= 1e-3 for f32-accumulate matmul,
+attention and logits.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from doppler_amd import ops, synth
+from doppler_amd.capi import DopplerHipError
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_F32 = 1e-3
+
+
+def rel_l2(got, want):
+    got = np.asarray(got, np.float64).reshape(-1)
+    want = np.asarray(want, np.float64).reshape(-1)
+    return float(np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30))
+
+
+def q4k_weight(N, K, seed):
+    W = synth.q4k_tensor(N, K, seed)
+    buf = ops.acquireBuffer(W.size)
+    ops.uploadData(buf, W)
+    return W, ops.createWeightBuffer(buf, "q4k", "row", (N, K), "w%d" % seed)
+
+
+# ----------------------------------------------------------------------------- dequant (bit-exact)
+
+def test_dequant_bit_exact_synthetic_cfg0():
+    N, K = synth.CFG0["N"], synth.CFG0["K"]
+    W, wb = q4k_weight(N, K, seed=1000)
+    nblk = W.size // 144
+    got = ops.readTensor(ops.runDequantQ4K(wb, nblk))
+    want = oracle.q4k_dequant_blocks(W)
+    assert got.tobytes() == want.tobytes()
+
+
+def test_dequant_bit_exact_real_scales_and_edge_d(receipt):
+    nb = 20000
+    q = synth.rng(5).integers(0, 16, size=(nb, 256), dtype=np.uint8)
+    d_bits = receipt["d_bits"][:nb].copy()
+    dmin_bits = receipt["dmin_bits"][:nb].copy()
+    # edge cases for the f16 multipliers: zero, smallest/largest subnormal, smallest normal, max finite
+    d_bits[:6] = [0, 1, 0x3FF, 0x400, 0x7BFF, 0x3C00]
+    dmin_bits[:6] = [0x7BFF, 0x400, 1, 0, 0x3FF, 0x3C00]
+    blocks = synth.q4k_pack_block_fields(d_bits, dmin_bits, receipt["scale_bits"][:nb * 8].reshape(nb, 8),
+                                         receipt["min_bits"][:nb * 8].reshape(nb, 8), q).reshape(-1)
+    buf = ops.acquireBuffer(blocks.size)
+    ops.uploadData(buf, blocks)
+    got = ops.readTensor(ops.runDequantQ4K(buf, nb))
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = oracle.q4k_dequant_blocks(blocks)
+    assert got.tobytes() == want.tobytes()
+
+
+# ----------------------------------------------------------------------------- Q4_K matmul
+
+def _matmul_case(M, N, K, seed, alpha=1.0, outputDtype="f32", residual=False):
+    W, wb = q4k_weight(N, K, seed)
+    A = synth.normal_f32((M, K), seed + 1)
+    a = ops.tensorFromNumpy(A)
+    res = synth.normal_f32((M, N), seed + 2) if residual else None
+    r = ops.tensorFromNumpy(res) if residual else None
+    out = ops.runMatmul(a, wb, M, N, K, alpha=alpha, outputDtype=outputDtype, role="test", residualTensor=r)
+    assert out.shape == (M, N) and out.dtype == outputDtype
+    got = ops.readTensor(out)
+    if outputDtype == "f16":
+        got = got.view(np.float16).astype(np.float32)
+    want = oracle.q4k_matmul(A, W, M, N, K, alpha)
+    if residual:
+        want = want + res
+    # the weight buffer must come back untouched (the reference's parity test asserts the same)
+    assert ops.readBuffer(wb.buffer, W.size).tobytes() == W.tobytes()
+    return rel_l2(got, want)
+
+
+def test_matmul_cfg0_gemv():
+    assert _matmul_case(1, synth.CFG0["N"], synth.CFG0["K"], seed=1100) <= REL_L2_F32
+
+
+@pytest.mark.parametrize("name", sorted(synth.CFG1_SHAPES))
+@pytest.mark.parametrize("M", [1, 2, 4, 8])
+def test_matmul_cfg1_block_sweep(name, M):
+    N, K = synth.CFG1_SHAPES[name]
+    assert _matmul_case(M, N, K, seed=1200 + 10 * M + len(name)) <= REL_L2_F32
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (1, 1024, 4096), (1, 12288, 4096), (1, 4096, 12288),
+                                   (3, 4096, 4096), (8, 1024, 12288)])
+def test_matmul_cfg4_shapes(M, N, K):
+    assert _matmul_case(M, N, K, seed=1300 + M) <= REL_L2_F32
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 33, 256), (5, 7, 512), (3, 64, 1152), (2, 1000, 300), (1, 1, 256),
+                                   (7, 129, 5120), (12, 96, 1152), (17, 40, 768)])
+def test_matmul_ragged_shapes(M, N, K):
+    assert _matmul_case(M, N, K, seed=1400 + M + N) <= REL_L2_F32
+
+
+def test_matmul_alpha_residual_f16_output():
+    assert _matmul_case(2, 512, 1024, seed=1500, alpha=0.125, residual=True) <= REL_L2_F32
+    assert _matmul_case(4, 512, 1024, seed=1510, alpha=2.0 ** -8, outputDtype="f16") <= 1e-3
+
+
+def test_matmul_one_hot_returns_dequantized_column():
+    N, K = 256, 1152
+    W, wb = q4k_weight(N, K, seed=1600)
+    Wd = oracle.q4k_dequant_rows(W, N, K)
+    for k in (0, 31, 32, 255, 256, 1151):
+        e = np.zeros((1, K), np.float32)
+        e[0, k] = 1.0
+        got = ops.readTensor(ops.runMatmul(ops.tensorFromNumpy(e), wb, 1, N, K, outputDtype="f32"))
+        assert np.array_equal(got, Wd[:, k]), k
+
+
+def test_matmul_padded_tail_is_ignored():
+    M, N, K = 2, 64, 640
+    W = synth.q4k_tensor(N, K, seed=1700)
+    A = synth.normal_f32((M, K), seed=1701)
+    W2 = W.reshape(N, 3, 144).copy()
+    W2[:, 2, 16 + 64:] ^= 0xFF        # k 640..767 of every row
+    outs = []
+    for w in (W, W2.reshape(-1)):
+        buf = ops.acquireBuffer(w.size)
+        ops.uploadData(buf, w)
+        outs.append(ops.readTensor(ops.runMatmul(ops.tensorFromNumpy(A), ops.createWeightBuffer(buf, "q4k", "row", (N, K)),
+                                                 M, N, K, outputDtype="f32")))
+    assert np.array_equal(outs[0], outs[1])
+
+
+def test_matmul_errors_match_reference_behaviour():
+    W, wb = q4k_weight(8, 256, seed=1800)
+    a = ops.tensorFromNumpy(np.zeros((1, 256), np.float32))
+    with pytest.raises(DopplerHipError, match="outputDtype is required"):
+        ops.runMatmul(a, wb, 1, 8, 256)
+    with pytest.raises(DopplerHipError, match="Dimensions must be positive"):
+        ops.runMatmul(a, wb, 0, 8, 256, outputDtype="f32")
+    with pytest.raises(DopplerHipError, match="B buffer too small"):
+        ops.runMatmul(a, wb, 1, 9, 256, outputDtype="f32")
+    with pytest.raises(DopplerHipError, match="A buffer too small"):
+        ops.runMatmul(a, wb, 2, 8, 256, outputDtype="f32")
+    with pytest.raises(DopplerHipError, match="B dtype is required"):
+        ops.runMatmul(a, wb.buffer, 1, 8, 256, outputDtype="f32")
+
+
+# ----------------------------------------------------------------------------- fused FFN gate/up
+
+@pytest.mark.parametrize("M,activation,limit", [(1, "silu", None), (4, "silu", 7.0), (1, "gelu", None), (3, "gelu", None)])
+def test_fused_ffn_q4k(M, activation, limit):
+    hidden, inter = 1536, 6144          # the shape of the reference's fused-ffn-q4k parity test
+    Wg, wg = q4k_weight(inter, hidden, seed=2000)
+    Wu, wu = q4k_weight(inter, hidden, seed=2001)
+    X = synth.normal_f32((M, hidden), seed=2002, scale=0.02)
+    out = ops.runFusedFFN(ops.tensorFromNumpy(X), wg, wu, hidden, inter, batchSize=M, activation=activation,
+                          alpha=0.5, swigluLimit=limit)
+    want = oracle.q4k_ffn_gate_up(X, Wg, Wu, M, hidden, inter, alpha=0.5, activation=activation, swiglu_limit=limit or 0.0)
+    assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
+
+
+# ----------------------------------------------------------------------------- LM head, argmax, gather
+
+def test_f16_weight_matmul_and_lmhead_argmax():
+    vocab, hidden = 5000, 1024
+    E = synth.normal_f16_bits((vocab, hidden), seed=3000, scale=0.02)
+    h = synth.normal_f32((1, hidden), seed=3001)
+    eb = ops.createWeightBuffer(ops.tensorFromNumpy(E).buffer, "f16", "row", (vocab, hidden))
+    ht = ops.tensorFromNumpy(h)
+    want = oracle.f16w_matmul(h, E, 1, vocab, hidden)
+    got = ops.readTensor(ops.runMatmul(ht, eb, 1, vocab, hidden, outputDtype="f32"))
+    assert rel_l2(got, want) <= REL_L2_F32
+    logits = ops.acquireBuffer(vocab * 4)
+    tok = ops.recordLmHeadArgmaxF16(None, ht, eb, vocabSize=vocab, hiddenSize=hidden, logitsOutput=logits)
+    assert int(ops.readBuffer(tok, 4, np.uint32)[0]) == oracle.argmax(want[0])
+    assert rel_l2(ops.readBuffer(logits, vocab * 4, np.float32), want) <= REL_L2_F32
+    pad = oracle.argmax(want[0])
+    tok = ops.recordLmHeadArgmaxF16(None, ht, eb, vocabSize=vocab, hiddenSize=hidden, padTokenId=pad, outputIndex=3,
+                                    outputBuffer=ops.acquireBuffer(16))
+    assert int(ops.readBuffer(tok, 16, np.uint32)[3]) == oracle.argmax(want[0], pad_id=pad)
+    # batched dense rows
+    A = synth.normal_f32((5, hidden), seed=3002)
+    got = ops.readTensor(ops.runMatmul(ops.tensorFromNumpy(A), eb, 5, vocab, hidden, outputDtype="f32"))
+    assert rel_l2(got, oracle.f16w_matmul(A, E, 5, vocab, hidden)) <= REL_L2_F32
+
+
+def test_argmax_exact_ties_pad_softcap():
+    g = synth.rng(3100)
+    for vocab in (1, 7, 256, 257, 151936):
+        x = g.integers(-50, 50, vocab).astype(np.float32)      # many exact ties
+        t = ops.tensorFromNumpy(x)
+        assert ops.runArgmax(t, vocab) == oracle.argmax(x)
+        pad = oracle.argmax(x)
+        assert ops.runArgmax(t, vocab, padTokenId=pad) == oracle.argmax(x, pad_id=pad)
+    x = synth.normal_f32(4096, seed=3101, scale=40.0)
+    assert ops.runArgmax(ops.tensorFromNumpy(x), 4096, logitSoftcap=30.0) == oracle.argmax(x, softcap=30.0)
+
+
+def test_gather_f16_exact():
+    vocab, hidden = 300, 640
+    E = synth.normal_f16_bits((vocab, hidden), seed=3200, scale=0.02)
+    ids = np.array([5, 299, 300, 0, 4000000000, 17], np.uint32)
+    out = ops.runGather(ops.tensorFromNumpy(ids).buffer, ops.tensorFromNumpy(E).buffer, 4, hidden, vocab,
+                        embeddingDtype="f16", outputDtype="f32", indexOffset=1)
+    want = oracle.gather_f16(ids[1:5], E, hidden, vocab)
+    assert np.array_equal(ops.readTensor(out).reshape(4, hidden), want)
+    with pytest.raises(DopplerHipError, match="embeddingDtype is required"):
+        ops.runGather(ops.tensorFromNumpy(ids).buffer, ops.tensorFromNumpy(E).buffer, 4, hidden, vocab)
+
+
+# ----------------------------------------------------------------------------- norm / rope / kv / elementwise
+
+@pytest.mark.parametrize("hidden", [640, 1024, 1152, 4096, 100])
+def test_rmsnorm_options(hidden):
+    B = 3
+    x = synth.normal_f32((B, hidden), seed=4000 + hidden, scale=3.0)
+    w = synth.normal_f32(hidden, seed=4001, scale=0.1)
+    r = synth.normal_f32((B, hidden), seed=4002)
+    xt, wt, rt = ops.tensorFromNumpy(x), ops.tensorFromNumpy(w), ops.tensorFromNumpy(r)
+    got = ops.readTensor(ops.runRMSNorm(xt, wt, 1e-6, batchSize=B, hiddenSize=hidden))
+    assert rel_l2(got, oracle.rmsnorm(x, w, 1e-6)) <= 1e-5
+    got = ops.readTensor(ops.runRMSNorm(xt, wt, 1e-6, batchSize=B, hiddenSize=hidden, rmsNormWeightOffset=True,
+                                        residual=rt, outputScale=0.5))
+    assert rel_l2(got, oracle.rmsnorm(x, w, 1e-6, weight_offset=True, post_residual=r, output_scale=0.5)) <= 1e-5
+    pre_out = ops.acquireBuffer(B * hidden * 4)
+    got = ops.readTensor(ops.runRMSNorm(xt, wt, 1e-6, batchSize=B, hiddenSize=hidden, preResidual=rt,
+                                        residualSumOutput=pre_out))
+    want, want_pre = oracle.rmsnorm(x, w, 1e-6, pre_residual=r, want_prenorm=True)
+    assert rel_l2(got, want) <= 1e-5
+    assert np.array_equal(ops.readBuffer(pre_out, B * hidden * 4, np.float32).reshape(B, hidden), want_pre)
+    w16 = w.astype(np.float16)
+    got = ops.readTensor(ops.runRMSNorm(xt, ops.tensorFromNumpy(w16.view(np.uint16), "f16"), 1e-6, batchSize=B, hiddenSize=hidden))
+    assert rel_l2(got, oracle.rmsnorm(x, w16.astype(np.float32), 1e-6)) <= 1e-5
+
+
+def test_rope_variants():
+    S, H, D, start = 5, 16, 128, 32000
+    cos, sin = synth.rope_tables(D, start + S, 1e6)
+    x = synth.normal_f32((S, H, D), seed=4100)
+    ct, st = ops.tensorFromNumpy(cos), ops.tensorFromNumpy(sin)
+    xt = ops.tensorFromNumpy(x)
+    out = ops.runRoPE(xt, ct, st, S, numHeads=H, headDim=D, startPos=start)
+    assert out.buffer is xt.buffer
+    assert rel_l2(ops.readTensor(out), oracle.rope_apply(x, cos, sin, S, H, D, start)) <= 1e-6
+    got = ops.readTensor(ops.runRoPE(ops.tensorFromNumpy(x), ct, st, S, numHeads=H, headDim=D, startPos=start, interleaved=True))
+    assert rel_l2(got, oracle.rope_apply(x, cos, sin, S, H, D, start, interleaved=True)) <= 1e-6
+    c32, s32 = synth.rope_tables(32, start + S, 1e4)
+    for span in (32, 128):
+        got = ops.readTensor(ops.runRoPE(ops.tensorFromNumpy(x), ops.tensorFromNumpy(c32), ops.tensorFromNumpy(s32), S,
+                                         numHeads=H, headDim=D, rotaryDim=32, pairSpanDim=span, startPos=start))
+        assert rel_l2(got, oracle.rope_apply(x, c32, s32, S, H, D, start, rotary_dim=32, pair_span_dim=span)) <= 1e-6
+    with pytest.raises(DopplerHipError, match="rotaryDim must be even"):
+        ops.runRoPE(xt, ct, st, S, numHeads=H, headDim=D, rotaryDim=31)
+
+
+def test_kv_cache_write_bit_exact():
+    n = 8 * 128 * 3
+    k = synth.normal_f32(n + 64, seed=4200)
+    v = synth.normal_f32(n + 64, seed=4201)
+    k[64:70] = [65504.0, 65520.0, 1e-8, 2.0 ** -24, 1.0 + 2.0 ** -11, -(1.0 + 3 * 2.0 ** -11)]   # overflow, underflow, ties
+    ck, cv = ops.acquireBuffer(4096 * 2 * 2), ops.acquireBuffer(4096 * 2 * 2)
+    ops.runKVCacheWriteF32ToF16(ops.tensorFromNumpy(k).buffer, ops.tensorFromNumpy(v).buffer, ck, cv,
+                                srcOffset=64, dstOffset=1024, elementCount=n)
+    wk, wv = np.zeros(8192, np.uint16), np.zeros(8192, np.uint16)
+    oracle.kv_write_f16(k, v, wk, wv, 64, 1024, n)
+    assert np.array_equal(ops.readBuffer(ck, dtype=np.uint16), wk)
+    assert np.array_equal(ops.readBuffer(cv, dtype=np.uint16), wv)
+    with pytest.raises(DopplerHipError, match="smaller than requested range"):
+        ops.runKVCacheWriteF32ToF16(ops.tensorFromNumpy(k).buffer, ops.tensorFromNumpy(v).buffer, ck, cv,
+                                    srcOffset=0, dstOffset=8000, elementCount=n)
+
+
+@pytest.mark.parametrize("T,H,Hkv,D", [(1, 32, 8, 128), (3, 16, 8, 128), (2, 4, 2, 64)])
+def test_split_qkv_rmsnorm_rope_kvwrite(T, H, Hkv, D):
+    start, max_seq = 37, 64
+    cos, sin = synth.rope_tables(D, max_seq, 1e6)
+    qkv = synth.normal_f32((T, (H + 2 * Hkv) * D), seed=4300)
+    qw = 1 + synth.normal_f32(D, seed=4301, scale=0.1)
+    kw = 1 + synth.normal_f32(D, seed=4302, scale=0.1)
+    ck, cv = ops.acquireBuffer(max_seq * Hkv * D * 2), ops.acquireBuffer(max_seq * Hkv * D * 2)
+    res = ops.runSplitQKVRMSNormRoPEQK(ops.tensorFromNumpy(qkv), ops.tensorFromNumpy(qw), ops.tensorFromNumpy(kw),
+                                       ops.tensorFromNumpy(cos), ops.tensorFromNumpy(sin), 1e-6, numTokens=T,
+                                       numHeads=H, numKVHeads=Hkv, headDim=D, qSize=H * D, kSize=Hkv * D, vSize=Hkv * D,
+                                       startPos=start,
+                                       f16KVCacheWrite=dict(keysBuffer=ck, valuesBuffer=cv, dstOffset=start * Hkv * D))
+    assert res["wroteF16KVCache"] and res["K"] is None
+    wk = np.zeros((max_seq, Hkv, D), np.uint16)
+    wv = np.zeros((max_seq, Hkv, D), np.uint16)
+    want_q = oracle.qkv_norm_rope_kvwrite(qkv, qw, kw, cos, sin, T, H, Hkv, D, start, wk, wv, start * Hkv * D)
+    assert rel_l2(ops.readTensor(res["Q"]), want_q) <= 1e-5
+    got_k = ops.readBuffer(ck, dtype=np.uint16).reshape(max_seq, Hkv, D)
+    # V is a pure narrowing: exact.  K goes through fp32 norm+rotation before rounding: values may
+    # differ from the f64 oracle by one f16 ulp at rounding boundaries.
+    assert np.array_equal(ops.readBuffer(cv, dtype=np.uint16).reshape(max_seq, Hkv, D), wv)
+    assert not got_k[:start].any() and not got_k[start + T:].any()
+    gk, ek = got_k.view(np.float16).astype(np.float64), wk.view(np.float16).astype(np.float64)
+    assert rel_l2(gk, ek) <= 5e-4
+    assert np.mean(got_k != wk) < 0.02
+
+
+def test_residual_and_gated_activations():
+    n = 12288
+    a, b = synth.normal_f32(n, seed=4400, scale=4.0), synth.normal_f32(n, seed=4401)
+    at, bt = ops.tensorFromNumpy(a), ops.tensorFromNumpy(b)
+    assert np.array_equal(ops.readTensor(ops.runResidualAdd(at, bt, n)), oracle.residual_add(a, b))
+    assert rel_l2(ops.readTensor(ops.runResidualAdd(at, bt, n, outputScale=0.25)), oracle.residual_add(a, b, 0.25)) <= 1e-7
+    assert rel_l2(ops.readTensor(ops.runSiLU(bt, size=n, gate=at)), oracle.act_gate(a, b, "silu")) <= 1e-5
+    assert rel_l2(ops.readTensor(ops.runSiLU(bt, size=n, gate=at, swigluLimit=0.5)), oracle.act_gate(a, b, "silu", 0.5)) <= 1e-5
+    assert rel_l2(ops.readTensor(ops.runGeLU(bt, size=n, gate=at)), oracle.act_gate(a, b, "gelu")) <= 1e-5
+    x = synth.normal_f32((4, 2 * 768), seed=4402, scale=3.0)
+    for act in ("silu", "gelu"):
+        got = ops.readTensor(ops.runSiLURowSplit(ops.tensorFromNumpy(x), numTokens=4, dim=768, activation=act))
+        assert rel_l2(got, oracle.act_gate_rowsplit(x, 4, 768, act)) <= 1e-5
+
+
+# ----------------------------------------------------------------------------- decode attention
+
+def _attn_inputs(H, Hkv, D, ctx, seed, theta=1e6):
+    """Config-3 recipe: N(0,1)/sqrt(D) values, RoPE applied to Q at ctx-1 and to K row p at p,
+    then K, V and Q rounded to f16 (Q widened back to f32)."""
+    cos, sin = synth.rope_tables(D, ctx, theta)
+    q = synth.normal_f32((1, H, D), seed, D ** -0.5)
+    k = synth.normal_f32((ctx, Hkv, D), seed + 1, D ** -0.5)
+    v = synth.normal_f32((ctx, Hkv, D), seed + 2, D ** -0.5)
+    q = oracle.rope_apply(q, cos, sin, 1, H, D, start_pos=ctx - 1)
+    k = oracle.rope_apply(k, cos, sin, ctx, Hkv, D, start_pos=0)
+    qf = q.astype(np.float16).astype(np.float32).reshape(H, D)
+    return qf, k.astype(np.float16).view(np.uint16), v.astype(np.float16).view(np.uint16)
+
+
+@pytest.mark.parametrize("ctx", [1, 63, 512, 4096, 32768])
+def test_attention_decode_cfg3(ctx):
+    H, Hkv, D = synth.CFG3["H"], synth.CFG3["Hkv"], synth.CFG3["D"]
+    q, kb, vb = _attn_inputs(H, Hkv, D, ctx, seed=5000 + ctx)
+    out = ops.runAttention(ops.tensorFromNumpy(q), ops.tensorFromNumpy(kb), ops.tensorFromNumpy(vb), None, H, D,
+                           seqLen=1, kvLen=ctx, numKVHeads=Hkv, causal=True, startPos=ctx - 1)
+    assert out.shape == (1, H, D)
+    want = oracle.attention_decode_f16kv(q, kb, vb, H, Hkv, D, ctx)
+    assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
+
+
+@pytest.mark.parametrize("H,Hkv,D", [(32, 8, 128), (8, 8, 128), (8, 1, 64), (6, 2, 64)])
+def test_attention_decode_head_geometries(H, Hkv, D):
+    ctx = 777
+    q, kb, vb = _attn_inputs(H, Hkv, D, ctx, seed=5100 + H)
+    out = ops.runAttention(ops.tensorFromNumpy(q), ops.tensorFromNumpy(kb), ops.tensorFromNumpy(vb), None, H, D,
+                           kvLen=ctx, numKVHeads=Hkv, startPos=ctx - 1)
+    assert rel_l2(ops.readTensor(out), oracle.attention_decode_f16kv(q, kb, vb, H, Hkv, D, ctx)) <= REL_L2_F32
+
+
+def test_attention_decode_options():
+    H, Hkv, D, ctx = 16, 8, 128, 1500
+    q, kb, vb = _attn_inputs(H, Hkv, D, ctx, seed=5200)
+    qt, kt, vt = ops.tensorFromNumpy(q * 20), ops.tensorFromNumpy(kb), ops.tensorFromNumpy(vb)
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, kvLen=ctx, numKVHeads=Hkv, startPos=ctx - 1,
+                                          scale=0.3, attnSoftcap=4.0))
+    assert rel_l2(got, oracle.attention_decode_f16kv(q * 20, kb, vb, H, Hkv, D, ctx, scale=0.3, softcap=4.0)) <= REL_L2_F32
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, kvLen=ctx, numKVHeads=Hkv, startPos=ctx - 1,
+                                          slidingWindow=200))
+    assert rel_l2(got, oracle.attention_decode_f16kv(q * 20, kb, vb, H, Hkv, D, ctx, sliding_window=200)) <= REL_L2_F32
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, kvLen=ctx, numKVHeads=Hkv, startPos=700))
+    assert rel_l2(got, oracle.attention_decode_f16kv(q * 20, kb, vb, H, Hkv, D, ctx, start_pos=700)) <= REL_L2_F32
+    # ring layout, window 256
+    win = 256
+    ring_k = np.zeros((win, Hkv, D), np.uint16)
+    ring_v = np.zeros((win, Hkv, D), np.uint16)
+    kk, vv = kb.reshape(ctx, Hkv, D), vb.reshape(ctx, Hkv, D)
+    for pos in range(ctx):
+        ring_k[pos % win], ring_v[pos % win] = kk[pos], vv[pos]
+    got = ops.readTensor(ops.runAttention(qt, ops.tensorFromNumpy(ring_k), ops.tensorFromNumpy(ring_v), None, H, D,
+                                          kvLen=win, numKVHeads=Hkv, startPos=ctx - 1, slidingWindow=win,
+                                          kvStart=ctx - win, kvLayout="ring"))
+    want = oracle.attention_decode_f16kv(q * 20, ring_k, ring_v, H, Hkv, D, win, sliding_window=win, kv_start=ctx - win,
+                                         kv_layout=1, start_pos=ctx - 1)
+    assert rel_l2(got, want) <= REL_L2_F32
+    # nothing visible -> zeros
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, kvLen=0, numKVHeads=Hkv, startPos=0))
+    assert not got.any()
+    with pytest.raises(DopplerHipError, match="kvLayout"):
+        ops.runAttention(qt, kt, vt, None, H, D, kvLen=ctx, numKVHeads=Hkv, kvLayout="paged")
