@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-inference hot path on one MI355X.
+
+A "step" is one greedy decode token of BASELINE config 4: a random-init 9B-class Q4_K decoder
+(36 layers, hidden 4096, FFN 12288, 32 query / 8 KV heads of 128, tied f16 LM head over a
+151,936-token vocabulary), KV cache prefilled to 2048 positions, every op on the HIP path
+through the C ABI, one 4-byte token readback per step.  Prints ONE JSON line with
+  value     decode tokens/s over exactly --steps steps (weights, KV and activations resident
+            in HBM; the only host traffic is the token id),
+  roofline  the dominant kernel (the fused gate/up Q4_K GEMV, 56.7 MB of weights per launch)
+            timed with HIP events on the op stream, against the 8 TB/s HBM peak,
+  cpu_baseline  the CPU oracle's decode step timed on this host's cores on a bounded sample.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def gate_up_kernel_bandwidth(dec, reps):
+    """Average duration of the fused gate/up GEMV launch, measured with HIP events on the
+    stream the kernel runs on.  Launches cycle through the layers' weights (36 x 56.6 MB,
+    far beyond the 256 MB infinity cache) so every launch streams from HBM."""
+    from doppler_amd import capi
+    L, c = dec.L, dec.cfg
+    Hd, I = c["hidden"], c["inter"]
+    ev = [ctypes.c_void_p() for _ in range(2)]
+    for e in ev:
+        capi.check(L.dh_event_create(ctypes.byref(e)))
+    total_ms, n = 0.0, 0
+    for r in range(reps):
+        for d in dec.layers:
+            capi.check(L.dh_event_record(ev[0]))
+            capi.check(L.dh_q4k_ffn_gate_up(dec.normed.data_ptr(), d["wgate"].data_ptr(), d["wup"].data_ptr(),
+                                            dec.act.data_ptr(), 1, Hd, I, capi.ACT_SILU, 1.0, 0.0))
+            capi.check(L.dh_event_record(ev[1]))
+            ms = ctypes.c_float()
+            capi.check(L.dh_event_elapsed_ms(ev[0], ev[1], ctypes.byref(ms)))
+            if r > 0:                      # first sweep warms code and TLBs
+                total_ms += ms.value
+                n += 1
+    for e in ev:
+        capi.check(L.dh_event_destroy(e))
+    return total_ms / max(n, 1)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="debug only: fewer layers (result is not the metric)")
+    ap.add_argument("--prefill", type=int, default=None, help="debug only: shorter prefill")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (single-stream decode has nothing to shard in this tier); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from doppler_amd import decoder, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+
+    c = dict(synth.CFG4)
+    prefill, _ = c.pop("prefill"), c.pop("steps")
+    if args.layers:
+        c["layers"] = args.layers
+    if args.prefill is not None:
+        prefill = args.prefill
+    max_seq = prefill + args.warmup + args.steps + 1
+    cfg = dict(c, max_seq=max_seq)
+
+    t0 = time.time()
+    layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=4, max_seq=max_seq)
+    log("[bench] synthetic weights generated in %.1f s" % (time.time() - t0))
+    t0 = time.time()
+    dec = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, max_seq)
+    log("[bench] uploaded in %.1f s" % (time.time() - t0))
+
+    # ---- KV prefill: the prompt goes through the decode path one token at a time (untimed)
+    ids = synth.rng(40).integers(0, cfg["vocab"], max(prefill, 1))
+    t0 = time.time()
+    tok = int(ids[0])
+    for pos in range(prefill):
+        tok = dec.step(int(ids[pos]), pos)
+    torch.cuda.synchronize()
+    log("[bench] prefill of %d positions in %.1f s" % (prefill, time.time() - t0))
+
+    pos = prefill
+    for _ in range(args.warmup):
+        tok = dec.step(tok, pos)
+        pos += 1
+    torch.cuda.synchronize()
+    capi_sync = dec.L.dh_sync
+    capi_sync()
+    t0 = time.perf_counter()
+    tokens = []
+    for _ in range(args.steps):
+        tok = dec.step(tok, pos)
+        tokens.append(tok)
+        pos += 1
+    capi_sync()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    tok_s = args.steps / elapsed
+    ctx_mid = prefill + args.warmup + args.steps // 2
+    step_bytes = dec.weight_bytes_per_token(ctx_mid)
+    log("[bench] %d steps in %.3f s -> %.1f tok/s (%.0f GB/s of algorithmic traffic)" %
+        (args.steps, elapsed, tok_s, step_bytes * tok_s / 1e9))
+
+    # ---- roofline of the dominant kernel
+    Hd, I = cfg["hidden"], cfg["inter"]
+    launch_bytes = 2 * synth.q4k_nbytes(I, Hd) + Hd * 4 + I * 4
+    avg_ms = gate_up_kernel_bandwidth(dec, reps=4)
+    achieved = launch_bytes / (avg_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": "q4k fused gate/up GEMV [2x12288x4096]", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "bytes_per_launch": launch_bytes, "avg_launch_us": round(avg_ms * 1e3, 2), "traffic": None}
+
+    # ---- CPU baseline: the oracle's decode step (a restatement of the reference's JS per-op
+    #      references) on this host, same weights, same KV
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle
+        ol = []
+        for i, l in enumerate(layers):
+            d = dict(l)
+            k, v = dec.read_kv(i, prefill)
+            d["cache_k"] = np.zeros((max_seq, cfg["kv_heads"], cfg["head_dim"]), np.uint16)
+            d["cache_v"] = np.zeros_like(d["cache_k"])
+            d["cache_k"].reshape(-1)[:k.size] = k
+            d["cache_v"].reshape(-1)[:v.size] = v
+            ol.append(d)
+        ocl = oracle.DecoderOracle(cfg, ol, embed, final_norm, cos, sin)
+        n_cpu, t_cpu, ctok = 0, 0.0, int(ids[-1])
+        t0 = time.perf_counter()
+        while n_cpu < 3 or (t_cpu < 12.0 and n_cpu < 64):
+            ctok = ocl.step(ctok, prefill + n_cpu)
+            n_cpu += 1
+            t_cpu = time.perf_counter() - t0
+        threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        cpu = {"value": round(n_cpu / t_cpu, 4), "unit": "tokens/s", "cores": threads, "kind": "port",
+               "sample": "%d full decode steps of the same model from the same prefilled KV cache "
+                         "(C restatement of the reference's JS per-op references, f64 accumulate, OpenMP)" % n_cpu}
+
+    out = {
+        "metric": "decode tokens/sec at 9B-class Q4_K, 1 GPU (Q4_K GEMV HBM GB/s in roofline)",
+        "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32 (Q4_K weights, f16 KV/LM head)", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[4]: 36-layer 9B-class Q4_K decoder, hidden 4096, FFN 12288, "
+                               "32/8 heads x128, vocab 151936, KV prefilled to %d, greedy, batch 1" % prefill,
+                   "layers": cfg["layers"], "context": prefill, "algorithmic_bytes_per_step": step_bytes,
+                   "hbm_frac_whole_step": round(step_bytes * tok_s / 1e9 / HBM_PEAK_GBPS, 4)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "tokens_head": tokens[:4],
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -166,7 +166,8 @@ def random_model(cfg, seed=0, max_seq=None):
             wup=synth.q4k_tensor(I, Hd, s + 6), wdown=synth.q4k_tensor(Hd, I, s + 7),
             input_norm=1 + synth.normal_f32(Hd, s + 8, 0.02), post_attn_norm=1 + synth.normal_f32(Hd, s + 9, 0.02),
             q_norm=1 + synth.normal_f32(D, s + 10, 0.02), k_norm=1 + synth.normal_f32(D, s + 11, 0.02)))
-    embed = synth.normal_f16_bits((cfg["vocab"], Hd), seed + 7, 0.02)
+    big = cfg["vocab"] * Hd >= 50_000_000
+    embed = (synth.normal_f16_bits_large if big else synth.normal_f16_bits)((cfg["vocab"], Hd), seed + 7, 0.02)
     final_norm = 1 + synth.normal_f32(Hd, seed + 8, 0.02)
     cos, sin = synth.rope_tables(D, max_seq or cfg.get("max_seq", 4096), cfg.get("theta", 1e6))
     return layers, embed, final_norm, cos, sin

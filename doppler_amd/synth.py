@@ -64,6 +64,19 @@ def normal_f16_bits(shape, seed, scale=1.0):
     return normal_f32(shape, seed, scale).astype(np.float16).view(np.uint16)
 
 
+def normal_f16_bits_large(shape, seed, scale=1.0):
+    """Same distribution as normal_f16_bits for tensors of 10^8+ elements (the 9B-class tied
+    embedding): torch's CPU generator and vectorised f32->f16 (round-to-nearest-even) are an
+    order of magnitude faster than numpy here.  Different PRNG, so different bytes than
+    normal_f16_bits for the same seed; both parity sides always share one host array."""
+    import torch
+    g = torch.Generator().manual_seed(int(seed))
+    n = int(np.prod(shape))
+    x = torch.randn(n, generator=g, dtype=torch.float32)
+    x.mul_(float(scale))
+    return x.to(torch.float16).numpy().view(np.uint16).reshape(shape)
+
+
 def rope_tables(rotary_dim, max_seq, theta, rope_scale=1.0):
     """cos/sin tables [max_seq, rotary_dim/2] f32: frequency rounded to f32, angle and
     cos/sin in f64 (the recipe of the reference's init-rope.js:21-26,120-133)."""

@@ -37,6 +37,7 @@ def lib():
             build()
         _lib = ctypes.CDLL(_LIB_PATH)
         _declare(_lib)
+        _lib.dor_init_tables()
     return _lib
 
 
@@ -68,6 +69,7 @@ def _declare(L):
     L.dor_f32_to_f16_rne_array.argtypes = [_P, _P, _I64]
     L.dor_q4k_unpack_scale_bits.argtypes = [_P, _P, _P]
     L.dor_q4k_dequant_blocks.argtypes = [_P, _I64, _P]
+    L.dor_q4k_dequant_blocks_fast.argtypes = [_P, _I64, _P]
     L.dor_q4k_decoded_scales.argtypes = [_P, _I64, _P, _P]
     L.dor_q4k_dequant_rows.argtypes = [_P, _I64, _I64, _P]
     L.dor_q4k_matmul.argtypes = [_P, _P, _I64, _I64, _I64, _F, _P]
@@ -142,6 +144,15 @@ def q4k_dequant_blocks(packed):
     nb = packed.size // Q4K_BLOCK_BYTES
     out = np.empty(nb * QK_K, np.float32)
     lib().dor_q4k_dequant_blocks(_ptr(packed), nb, _ptr(out))
+    return out
+
+
+def q4k_dequant_blocks_fast(packed):
+    """f32-arithmetic twin used inside the matmul loops; must equal q4k_dequant_blocks bit for bit."""
+    packed = _c(packed, np.uint8).reshape(-1)
+    nb = packed.size // Q4K_BLOCK_BYTES
+    out = np.empty(nb * QK_K, np.float32)
+    lib().dor_q4k_dequant_blocks_fast(_ptr(packed), nb, _ptr(out))
     return out
 
 

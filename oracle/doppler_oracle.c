@@ -136,6 +136,21 @@ uint16_t dor_f32_to_f16_trunc(float value) {
   return (uint16_t)((sign << 15) | ((uint32_t)exp << 10) | (frac >> 13));
 }
 
+/* Table of all 65,536 widenings, filled from dor_f16_to_f32 by dor_init_tables(); the bulk
+ * loops (LM head, attention over the KV cache) read it instead of calling ldexp per element. */
+static float g_f16_lut[65536];
+static int g_f16_lut_ready = 0;
+
+void dor_init_tables(void) {
+  if (g_f16_lut_ready) return;
+  for (int i = 0; i < 65536; i++) g_f16_lut[i] = dor_f16_to_f32((uint16_t)i);
+  g_f16_lut_ready = 1;
+}
+
+static inline float f16_widen(uint16_t bits) {
+  return g_f16_lut_ready ? g_f16_lut[bits] : dor_f16_to_f32(bits);
+}
+
 void dor_f16_to_f32_array(const uint16_t* in, float* out, int64_t n) {
   for (int64_t i = 0; i < n; i++) out[i] = dor_f16_to_f32(in[i]);
 }
@@ -197,6 +212,31 @@ void dor_q4k_dequant_block(const uint8_t* block, float out[QK_K]) {
   }
 }
 
+/* Same values as dor_q4k_dequant_block, computed in f32: scale*q is exact in f32 (at most
+ * 21 significant bits) so `scale*q - min` rounds once, to the same f32 the double expression
+ * rounds to.  Compiled without FMA contraction; tests assert bit equality with the double
+ * version.  Used by the matmul loops, where the per-element double arithmetic dominated. */
+static void q4k_dequant_block_fast(const uint8_t* block, float* out) {
+  float scales[8], mins[8];
+  dor_q4k_block_scales(block, scales, mins);
+  for (int chunk = 0; chunk < 4; chunk++) {
+    const uint8_t* q = block + 16 + chunk * 32;
+    float* o = out + chunk * 64;
+    const float s0 = scales[chunk * 2], s1 = scales[chunk * 2 + 1];
+    const float m0 = mins[chunk * 2], m1 = mins[chunk * 2 + 1];
+    for (int i = 0; i < 32; i++) {
+      o[i] = s0 * (float)(q[i] & 0x0f) - m0;
+      o[32 + i] = s1 * (float)(q[i] >> 4) - m1;
+    }
+  }
+}
+
+void dor_q4k_dequant_blocks_fast(const uint8_t* packed, int64_t num_blocks, float* out) {
+#pragma omp parallel for schedule(static)
+  for (int64_t b = 0; b < num_blocks; b++)
+    q4k_dequant_block_fast(packed + b * Q4K_BLOCK_BYTES, out + b * QK_K);
+}
+
 void dor_q4k_dequant_blocks(const uint8_t* packed, int64_t num_blocks, float* out) {
 #pragma omp parallel for schedule(static)
   for (int64_t b = 0; b < num_blocks; b++)
@@ -240,16 +280,42 @@ void dor_q4k_dequant_rows(const uint8_t* packed, int64_t N, int64_t K, float* ou
 void dor_q4k_matmul(const float* A, const uint8_t* W, int64_t M, int64_t N, int64_t K,
                     float alpha, float* C) {
   const int64_t nb = (K + QK_K - 1) / QK_K;
-#pragma omp parallel for schedule(static)
-  for (int64_t n = 0; n < N; n++) {
-    float* wrow = (float*)malloc((size_t)nb * QK_K * sizeof(float));
-    for (int64_t b = 0; b < nb; b++)
-      dor_q4k_dequant_block(W + (n * nb + b) * Q4K_BLOCK_BYTES, wrow + b * QK_K);
-    for (int64_t m = 0; m < M; m++) {
-      double sum = 0.0;
-      const float* a = A + m * K;
-      for (int64_t k = 0; k < K; k++) sum += (double)a[k] * (double)wrow[k];
-      C[m * N + n] = (float)(sum * (double)alpha);
+  const int64_t kp = nb * QK_K;
+  /* Four rows at a time: four independent accumulators keep the adder busy; each row's own
+   * sum still runs over k in ascending order, one f64 add per element. */
+#pragma omp parallel
+  {
+    float* wrow = (float*)malloc((size_t)4 * kp * sizeof(float));
+#pragma omp for schedule(static)
+    for (int64_t n0 = 0; n0 < N; n0 += 4) {
+      const int64_t rows = (N - n0) < 4 ? (N - n0) : 4;
+      for (int64_t r = 0; r < rows; r++)
+        for (int64_t b = 0; b < nb; b++)
+          q4k_dequant_block_fast(W + ((n0 + r) * nb + b) * Q4K_BLOCK_BYTES, wrow + r * kp + b * QK_K);
+      for (int64_t m = 0; m < M; m++) {
+        const float* a = A + m * K;
+        if (rows == 4) {
+          double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+          const float *w0 = wrow, *w1 = wrow + kp, *w2 = wrow + 2 * kp, *w3 = wrow + 3 * kp;
+          for (int64_t k = 0; k < K; k++) {
+            const double av = (double)a[k];
+            s0 += av * (double)w0[k];
+            s1 += av * (double)w1[k];
+            s2 += av * (double)w2[k];
+            s3 += av * (double)w3[k];
+          }
+          C[m * N + n0] = (float)(s0 * (double)alpha);
+          C[m * N + n0 + 1] = (float)(s1 * (double)alpha);
+          C[m * N + n0 + 2] = (float)(s2 * (double)alpha);
+          C[m * N + n0 + 3] = (float)(s3 * (double)alpha);
+        } else {
+          for (int64_t r = 0; r < rows; r++) {
+            double sum = 0.0;
+            for (int64_t k = 0; k < K; k++) sum += (double)a[k] * (double)wrow[r * kp + k];
+            C[m * N + n0 + r] = (float)(sum * (double)alpha);
+          }
+        }
+      }
     }
     free(wrow);
   }
@@ -266,7 +332,7 @@ void dor_f16w_matmul(const float* A, const uint16_t* W, int64_t M, int64_t N, in
       double sum = 0.0;
       const float* a = A + m * K;
       const uint16_t* w = W + n * K;
-      for (int64_t k = 0; k < K; k++) sum += (double)a[k] * (double)dor_f16_to_f32(w[k]);
+      for (int64_t k = 0; k < K; k++) sum += (double)a[k] * (double)f16_widen(w[k]);
       C[m * N + n] = (float)(sum * (double)alpha);
     }
   }
@@ -530,7 +596,7 @@ void dor_attention_decode_f16kv(const float* Q, const uint16_t* K, const uint16_
       double s = 0.0;
       const float* qv = Q + h * D;
       const uint16_t* kv = K + (row * Hkv + kvh) * D;
-      for (int64_t d = 0; d < D; d++) s += (double)qv[d] * (double)dor_f16_to_f32(kv[d]);
+      for (int64_t d = 0; d < D; d++) s += (double)qv[d] * (double)f16_widen(kv[d]);
       s = (double)(float)(s * scale);
       if (softcap > 0.0f) s = (double)(float)(tanh(s / (double)softcap) * (double)softcap);
       scores[k] = (float)s;
@@ -549,7 +615,7 @@ void dor_attention_decode_f16kv(const float* Q, const uint16_t* K, const uint16_
       for (int64_t d = 0; d < D; d++) {
         double val = 0.0;
         for (int64_t k = 0; k < kv_len; k++)
-          val += (double)scores[k] * (double)dor_f16_to_f32(V[(rows[k] * Hkv + kvh) * D + d]);
+          val += (double)scores[k] * (double)f16_widen(V[(rows[k] * Hkv + kvh) * D + d]);
         out[h * D + d] = (float)val;
       }
     }
@@ -629,7 +695,7 @@ void dor_gather_f16(const uint32_t* ids, const uint16_t* table, int64_t T, int64
   for (int64_t t = 0; t < T; t++) {
     for (int64_t i = 0; i < hidden; i++)
       out[t * hidden + i] =
-          ids[t] >= (uint32_t)vocab ? 0.0f : dor_f16_to_f32(table[(int64_t)ids[t] * hidden + i]);
+          ids[t] >= (uint32_t)vocab ? 0.0f : f16_widen(table[(int64_t)ids[t] * hidden + i]);
   }
 }
 

@@ -111,6 +111,20 @@ def test_receipt_dequant_matches_fields(receipt):
     assert np.array_equal(w, want.astype(np.float32))
 
 
+def test_fast_f32_dequant_equals_double_dequant(receipt):
+    blocks, _ = _receipt_blocks(receipt, seed=9)
+    sub = blocks[:30000].reshape(-1)
+    assert oracle.q4k_dequant_blocks_fast(sub).tobytes() == oracle.q4k_dequant_blocks(sub).tobytes()
+    g = np.random.default_rng(10)
+    n = 20000
+    rnd = synth.q4k_pack_block_fields(g.integers(0, 0x7C00, n, dtype=np.uint16), g.integers(0, 0x7C00, n, dtype=np.uint16),
+                                      g.integers(0, 64, (n, 8), dtype=np.uint8), g.integers(0, 64, (n, 8), dtype=np.uint8),
+                                      g.integers(0, 16, (n, 256), dtype=np.uint8)).reshape(-1)
+    with np.errstate(over="ignore", invalid="ignore"):
+        a, b = oracle.q4k_dequant_blocks_fast(rnd), oracle.q4k_dequant_blocks(rnd)
+    assert a.tobytes() == b.tobytes()
+
+
 # ----------------------------------------------------------------------------- Q4_K: closed forms
 
 def test_dequant_is_single_correct_rounding_of_exact_value():
