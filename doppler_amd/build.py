@@ -54,8 +54,9 @@ def build_addon():
     inc = "/usr/include/node"
     if not os.path.exists(os.path.join(inc, "node_api.h")):
         raise RuntimeError("node_api.h not found under /usr/include/node")
-    _run(["gcc", "-O2", "-fPIC", "-shared", "-std=c11", "-Wall", "-I", inc,
-          "-I", os.path.join(HERE, "..", "include"), "-o", ADDON, src, "-ldl"])
+    _run(["gcc", "-O2", "-fPIC", "-shared", "-std=c11", "-Wall", "-DNAPI_VERSION=6",
+          "-DNODE_GYP_MODULE_NAME=doppler_hip", "-I", inc, "-I", os.path.join(HERE, "..", "include"),
+          "-o", ADDON, src, "-L", LIB_DIR, "-ldopplerhip", "-Wl,-rpath,$ORIGIN/../lib"])
     return ADDON
 
 
