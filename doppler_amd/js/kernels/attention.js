@@ -1,0 +1,64 @@
+// runAttention / recordAttention for decode (seqLen 1) over an f16 KV cache:
+// reference src/gpu/kernels/attention.js:1047-1310,2007-2030.
+import { getNative, KV_LAYOUT } from '../native.js';
+import { createTensor } from '../tensor.js';
+import { acquireBuffer, releaseBuffer } from '../buffer-pool.js';
+import { padToQ4KBlock, noteDispatch } from './constants.js';
+
+async function executeAttention(recorder, Q, K, V, mask, numHeads, headDim, options = {}) {
+  const {
+    seqLen = 1,
+    kvLen = seqLen,
+    numKVHeads = numHeads,
+    scale = 1.0 / Math.sqrt(headDim),
+    causal = true,
+    startPos = 0,
+    outputBuffer = null,
+    attnSoftcap = 0,
+    slidingWindow = 0,
+    kvStart = 0,
+    kvLayout = 'contiguous',
+  } = options;
+  if (seqLen !== 1) {
+    throw new Error(`[Attention] the HIP path serves decode (seqLen=1) only, got seqLen=${seqLen}.`);
+  }
+  if (mask) {
+    throw new Error('[Attention] explicit masks are not supported on the decode path.');
+  }
+  if (!(kvLayout in KV_LAYOUT)) {
+    throw new Error(`[Attention] kvLayout "${kvLayout}" is not supported by the HIP path (contiguous, ring).`);
+  }
+  if (Q.dtype !== 'f32' || K.dtype !== 'f16' || V.dtype !== 'f16') {
+    throw new Error(`[Attention] decode needs f32 Q and f16 K/V, got ${Q.dtype}/${K.dtype}/${V.dtype}.`);
+  }
+  const rows = kvLayout === 'ring' ? slidingWindow : kvStart + kvLen;
+  const kvBytes = rows * numKVHeads * headDim * 2;
+  if (kvLen > 0 && (K.buffer.size < kvBytes || V.buffer.size < kvBytes)) {
+    throw new Error(`[Attention] KV buffers are smaller than kvLen=${kvLen} rows (${kvBytes} bytes).`);
+  }
+  const native = getNative();
+  const outputSize = seqLen * padToQ4KBlock(numHeads * headDim) * 4;
+  const output = outputBuffer || acquireBuffer(outputSize, undefined, 'attention_output');
+  const owned = outputBuffer ? null : output;
+  const workspace = acquireBuffer(native.attnDecodeWorkspaceBytes(numHeads, headDim, Math.max(kvLen, 1)), undefined,
+    'attention_splitk_workspace');
+  try {
+    native.attnDecode(Q.buffer.ptr, K.buffer.ptr, V.buffer.ptr, output.ptr, numHeads, numKVHeads, headDim, kvLen,
+      scale, causal ? 1 : 0, startPos, attnSoftcap, slidingWindow, kvStart, KV_LAYOUT[kvLayout], workspace.ptr);
+  } catch (error) {
+    if (owned) releaseBuffer(owned);
+    releaseBuffer(workspace);
+    throw error;
+  }
+  if (recorder) recorder.trackTemporaryBuffer(workspace); else releaseBuffer(workspace);
+  noteDispatch(recorder, 'attention');
+  return createTensor(output, 'f32', [seqLen, numHeads, headDim], 'attention_output');
+}
+
+export async function runAttention(Q, K, V, mask, numHeads, headDim, options = {}) {
+  return executeAttention(null, Q, K, V, mask, numHeads, headDim, options);
+}
+
+export async function recordAttention(recorder, Q, K, V, mask, numHeads, headDim, options = {}) {
+  return executeAttention(recorder, Q, K, V, mask, numHeads, headDim, options);
+}

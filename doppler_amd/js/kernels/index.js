@@ -1,0 +1,17 @@
+// Op API of the HIP path: the subset of the reference's src/gpu/kernels/index.js that the
+// text pipeline's quantized decode path calls (src/inference/pipelines/text/ops.js:3-30,
+// attention/interpreter.js:6-23).  Same names, argument order and option names.
+export { runMatmul, recordMatmul, runDequantQ4K } from './matmul.js';
+export { runFusedFFN, recordFusedFFN } from './fused_ffn.js';
+export { runAttention, recordAttention } from './attention.js';
+export { runRMSNorm, recordRMSNorm } from './rmsnorm.js';
+export { runRoPE, recordRoPE } from './rope.js';
+export { runKVCacheWriteF32ToF16, recordKVCacheWriteF32ToF16 } from './kv-cache-write.js';
+export { runSplitQKVRMSNormRoPEQK, recordSplitQKVRMSNormRoPEQK } from './split-qkv-rmsnorm-rope-qk.js';
+export { runSiLU, recordSiLU, runSiLURowSplit, recordSiLURowSplit } from './silu.js';
+export { runGeLU, recordGeLU } from './gelu.js';
+export { runResidualAdd, recordResidualAdd } from './residual.js';
+export { runGather, recordGather } from './gather.js';
+export { runArgmax, recordArgmax } from './sample.js';
+export { recordLmHeadArgmax, recordLmHeadArgmaxF16 } from './lm-head-argmax.js';
+export { castF32ToF16, castF16ToF32, recordCastF32ToF16, recordCastF16ToF32 } from './cast.js';

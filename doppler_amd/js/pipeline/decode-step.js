@@ -1,0 +1,96 @@
+// Greedy decode loop over the HIP op API: the shape of the reference's decodeStep
+// (src/inference/pipelines/text/generator-steps.js:588-820) for a Qwen3-class Q4_K model.
+// One CommandRecorder per token, every op recorded in execution-graph order
+// (src/config/conversion/qwen3/qwen-3-embedding-0-6b-q4k-ehf16-af32.json `execution.decode`),
+// one 4-byte readback per token.
+import {
+  createTensor, createWeightBuffer, acquireBuffer, releaseBuffer, uploadData, readBufferSlice,
+  createCommandRecorder, recordGather, recordRMSNorm, recordMatmul, recordSplitQKVRMSNormRoPEQK,
+  recordAttention, recordFusedFFN, recordLmHeadArgmaxF16,
+} from '../kernel-selector.js';
+
+function upload(bytes, label) {
+  const buf = acquireBuffer(bytes.byteLength, undefined, label);
+  uploadData(buf, bytes);
+  return buf;
+}
+
+export class HipTextDecoder {
+  // config: {layers, hidden, inter, heads, kvHeads, headDim, vocab, eps, maxSeq}
+  // weights: {layers: [{wqkv, wo, wgate, wup, wdown (Uint8Array Q4_K), inputNorm, postAttnNorm,
+  //           qNorm, kNorm (Float32Array)}], embed (Uint16Array f16 bits), finalNorm, cos, sin}
+  constructor(config, weights) {
+    this.config = config;
+    const c = config;
+    this.qSize = c.heads * c.headDim;
+    this.kSize = c.kvHeads * c.headDim;
+    this.layers = weights.layers.map((l, i) => ({
+      wqkv: createWeightBuffer(upload(l.wqkv, `L${i}.qkv`), 'q4k', 'row', [this.qSize + 2 * this.kSize, c.hidden], `L${i}.qkv`),
+      wo: createWeightBuffer(upload(l.wo, `L${i}.o`), 'q4k', 'row', [c.hidden, this.qSize], `L${i}.o`),
+      wgate: createWeightBuffer(upload(l.wgate, `L${i}.gate`), 'q4k', 'row', [c.inter, c.hidden], `L${i}.gate`),
+      wup: createWeightBuffer(upload(l.wup, `L${i}.up`), 'q4k', 'row', [c.inter, c.hidden], `L${i}.up`),
+      wdown: createWeightBuffer(upload(l.wdown, `L${i}.down`), 'q4k', 'row', [c.hidden, c.inter], `L${i}.down`),
+      inputNorm: createTensor(upload(l.inputNorm), 'f32', [c.hidden], 'input_norm'),
+      postAttnNorm: createTensor(upload(l.postAttnNorm), 'f32', [c.hidden], 'post_attn_norm'),
+      qNorm: createTensor(upload(l.qNorm), 'f32', [c.headDim], 'q_norm'),
+      kNorm: createTensor(upload(l.kNorm), 'f32', [c.headDim], 'k_norm'),
+      cacheK: createTensor(acquireBuffer(c.maxSeq * this.kSize * 2, undefined, 'kv_k'), 'f16', [c.maxSeq, c.kvHeads, c.headDim], 'kv_k'),
+      cacheV: createTensor(acquireBuffer(c.maxSeq * this.kSize * 2, undefined, 'kv_v'), 'f16', [c.maxSeq, c.kvHeads, c.headDim], 'kv_v'),
+    }));
+    this.embed = createWeightBuffer(upload(weights.embed, 'embed'), 'f16', 'row', [c.vocab, c.hidden], 'embed');
+    this.finalNorm = createTensor(upload(weights.finalNorm), 'f32', [c.hidden], 'final_norm');
+    this.cos = createTensor(upload(weights.cos), 'f32', [c.maxSeq, c.headDim / 2], 'rope_cos');
+    this.sin = createTensor(upload(weights.sin), 'f32', [c.maxSeq, c.headDim / 2], 'rope_sin');
+    this.ids = acquireBuffer(16, undefined, 'token_ids');
+    this.tokenOut = acquireBuffer(16, undefined, 'sampled_token');
+  }
+
+  // Returns the greedy token for `token` at position `pos` (KV rows 0..pos-1 present).
+  async decodeStep(token, pos, options = {}) {
+    const c = this.config;
+    const recorder = createCommandRecorder('decode');
+    const temps = [];
+    const temp = (t) => { temps.push(t.buffer); return t; };
+    uploadData(this.ids, new Uint32Array([token]));
+    let x = temp(await recordGather(recorder, this.ids, this.embed, 1, c.hidden, c.vocab,
+      { embeddingDtype: 'f16', outputDtype: 'f32' }));
+    for (let li = 0; li < this.layers.length; li++) {
+      const l = this.layers[li];
+      const normed = temp(await recordRMSNorm(recorder, x, l.inputNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden }));
+      const qkv = temp(await recordMatmul(recorder, normed, l.wqkv, 1, this.qSize + 2 * this.kSize, c.hidden,
+        { outputDtype: 'f32', role: 'qkv_proj', layerIdx: li }));
+      const split = await recordSplitQKVRMSNormRoPEQK(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps, {
+        numTokens: 1, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim,
+        qSize: this.qSize, kSize: this.kSize, vSize: this.kSize, startPos: pos,
+        f16KVCacheWrite: { keysBuffer: l.cacheK.buffer, valuesBuffer: l.cacheV.buffer, dstOffset: pos * this.kSize },
+      });
+      temp(split.Q);
+      const attn = temp(await recordAttention(recorder, split.Q, l.cacheK, l.cacheV, null, c.heads, c.headDim, {
+        seqLen: 1, kvLen: pos + 1, numKVHeads: c.kvHeads, causal: true, startPos: pos, layerIdx: li,
+      }));
+      const attnFlat = createTensor(attn.buffer, 'f32', [1, this.qSize], 'attn_flat');
+      const x2 = temp(await recordMatmul(recorder, attnFlat, l.wo, 1, c.hidden, this.qSize,
+        { outputDtype: 'f32', role: 'o_proj', layerIdx: li, residualTensor: x }));
+      const normed2 = temp(await recordRMSNorm(recorder, x2, l.postAttnNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden }));
+      const act = temp(await recordFusedFFN(recorder, normed2, l.wgate, l.wup, c.hidden, c.inter,
+        { batchSize: 1, activation: 'silu' }));
+      x = temp(await recordMatmul(recorder, act, l.wdown, 1, c.hidden, c.inter,
+        { outputDtype: 'f32', role: 'down_proj', layerIdx: li, residualTensor: x2 }));
+    }
+    const finalNormed = temp(await recordRMSNorm(recorder, x, this.finalNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden }));
+    await recordLmHeadArgmaxF16(recorder, finalNormed, this.embed, {
+      vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: this.tokenOut, outputIndex: 0,
+      logitsOutput: options.logitsOutput || null,
+    });
+    for (const b of temps) recorder.trackTemporaryBuffer(b);
+    recorder.submit();
+    const bytes = await readBufferSlice(this.tokenOut, 0, 4);   // the only device->host crossing
+    return new Uint32Array(bytes)[0];
+  }
+
+  destroy() {
+    for (const l of this.layers) {
+      for (const key of Object.keys(l)) releaseBuffer(l[key].buffer);
+    }
+  }
+}

@@ -1,0 +1,166 @@
+// Runs op cases prepared by tests/test_gpu_js.py through the JavaScript host API
+// (doppler_amd/js/kernel-selector.js -> Node-API addon -> libdopplerhip.so) and writes each
+// result next to its inputs.  Usage: node tests/js/run_cases.mjs <case-dir>
+import fs from 'fs';
+import path from 'path';
+import * as dh from '../../doppler_amd/js/kernel-selector.js';
+import { HipTextDecoder } from '../../doppler_amd/js/pipeline/decode-step.js';
+
+const dir = process.argv[2];
+const manifest = JSON.parse(fs.readFileSync(path.join(dir, 'manifest.json'), 'utf8'));
+
+function load(name) {
+  const b = fs.readFileSync(path.join(dir, name));
+  return new Uint8Array(b.buffer, b.byteOffset, b.byteLength).slice();
+}
+function dev(name, label) {
+  const bytes = load(name);
+  const buf = dh.acquireBuffer(Math.max(bytes.byteLength, 4), undefined, label || name);
+  dh.uploadData(buf, bytes);
+  return buf;
+}
+function tensor(name, dtype, shape) {
+  return dh.createTensor(dev(name), dtype, shape, name);
+}
+async function save(name, buffer, bytes) {
+  const ab = await dh.readBuffer(buffer, bytes);
+  fs.writeFileSync(path.join(dir, name), Buffer.from(ab));
+}
+async function expectThrow(results, label, pattern, fn) {
+  try {
+    await fn();
+    results.errors.push({ label, ok: false, message: 'did not throw' });
+  } catch (e) {
+    results.errors.push({ label, ok: new RegExp(pattern).test(e.message), message: e.message });
+  }
+}
+
+async function main() {
+  const results = { cases: [], errors: [] };
+  dh.initDevice(0);
+
+  for (const c of manifest.cases) {
+    const out = `${c.name}.out.bin`;
+    if (c.op === 'dequant') {
+      const t = await dh.runDequantQ4K(dh.createWeightBuffer(dev(c.W), 'q4k', 'row', [c.blocks, 256]), c.blocks);
+      await save(out, t.buffer, c.blocks * 256 * 4);
+    } else if (c.op === 'matmul') {
+      const W = dh.createWeightBuffer(dev(c.W), c.wdtype, 'row', [c.N, c.K], c.name);
+      const A = tensor(c.A, 'f32', [c.M, c.K]);
+      const opts = { outputDtype: c.outputDtype, alpha: c.alpha, role: 'test' };
+      if (c.residual) opts.residualTensor = tensor(c.residual, 'f32', [c.M, c.N]);
+      const rec = c.record ? dh.createCommandRecorder('t') : null;
+      const t = rec ? await dh.recordMatmul(rec, A, W, c.M, c.N, c.K, opts) : await dh.runMatmul(A, W, c.M, c.N, c.K, opts);
+      if (rec) await rec.submitAndWait();
+      await save(out, t.buffer, c.M * c.N * (c.outputDtype === 'f16' ? 2 : 4));
+    } else if (c.op === 'fused_ffn') {
+      const Wg = dh.createWeightBuffer(dev(c.Wg), 'q4k', 'row', [c.inter, c.hidden]);
+      const Wu = dh.createWeightBuffer(dev(c.Wu), 'q4k', 'row', [c.inter, c.hidden]);
+      const t = await dh.runFusedFFN(tensor(c.X, 'f32', [c.M, c.hidden]), Wg, Wu, c.hidden, c.inter,
+        { batchSize: c.M, activation: c.activation, alpha: c.alpha, swigluLimit: c.swigluLimit });
+      await save(out, t.buffer, c.M * c.inter * 4);
+    } else if (c.op === 'rmsnorm') {
+      const opts = { batchSize: c.batch, hiddenSize: c.hidden, rmsNormWeightOffset: c.weightOffset };
+      if (c.residual) opts.residual = tensor(c.residual, 'f32', [c.batch, c.hidden]);
+      if (c.outputScale) opts.outputScale = c.outputScale;
+      const t = await dh.runRMSNorm(tensor(c.x, 'f32', [c.batch, c.hidden]), tensor(c.w, 'f32', [c.hidden]), c.eps, opts);
+      await save(out, t.buffer, c.batch * c.hidden * 4);
+    } else if (c.op === 'rope') {
+      const x = tensor(c.x, 'f32', [c.seq, c.heads, c.headDim]);
+      const t = await dh.runRoPE(x, tensor(c.cos, 'f32', [1]), tensor(c.sin, 'f32', [1]), c.seq,
+        { numHeads: c.heads, headDim: c.headDim, startPos: c.startPos, interleaved: c.interleaved });
+      if (t.buffer !== x.buffer) throw new Error('runRoPE must alias its input');
+      await save(out, t.buffer, c.seq * c.heads * c.headDim * 4);
+    } else if (c.op === 'split_qkv') {
+      const ck = dh.acquireBuffer(c.maxSeq * c.kvHeads * c.headDim * 2);
+      const cv = dh.acquireBuffer(c.maxSeq * c.kvHeads * c.headDim * 2);
+      const r = await dh.runSplitQKVRMSNormRoPEQK(tensor(c.qkv, 'f32', [c.T, (c.heads + 2 * c.kvHeads) * c.headDim]),
+        tensor(c.qw, 'f32', [c.headDim]), tensor(c.kw, 'f32', [c.headDim]), tensor(c.cos, 'f32', [1]), tensor(c.sin, 'f32', [1]),
+        c.eps, { numTokens: c.T, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim, qSize: c.heads * c.headDim,
+          kSize: c.kvHeads * c.headDim, vSize: c.kvHeads * c.headDim, startPos: c.startPos,
+          f16KVCacheWrite: { keysBuffer: ck, valuesBuffer: cv, dstOffset: c.startPos * c.kvHeads * c.headDim } });
+      await save(out, r.Q.buffer, c.T * c.heads * c.headDim * 4);
+      await save(`${c.name}.k.bin`, ck, c.maxSeq * c.kvHeads * c.headDim * 2);
+      await save(`${c.name}.v.bin`, cv, c.maxSeq * c.kvHeads * c.headDim * 2);
+    } else if (c.op === 'kv_write') {
+      const ck = dh.acquireBuffer(c.cacheElems * 2);
+      const cv = dh.acquireBuffer(c.cacheElems * 2);
+      await dh.runKVCacheWriteF32ToF16(dev(c.k), dev(c.v), ck, cv, { srcOffset: c.srcOffset, dstOffset: c.dstOffset, elementCount: c.count });
+      await save(out, ck, c.cacheElems * 2);
+      await save(`${c.name}.v.bin`, cv, c.cacheElems * 2);
+    } else if (c.op === 'attention') {
+      const t = await dh.runAttention(tensor(c.Q, 'f32', [c.heads, c.headDim]), tensor(c.K, 'f16', [c.kvLen, c.kvHeads, c.headDim]),
+        tensor(c.V, 'f16', [c.kvLen, c.kvHeads, c.headDim]), null, c.heads, c.headDim,
+        { seqLen: 1, kvLen: c.kvLen, numKVHeads: c.kvHeads, causal: true, startPos: c.kvLen - 1 });
+      await save(out, t.buffer, c.heads * c.headDim * 4);
+    } else if (c.op === 'residual') {
+      const t = await dh.runResidualAdd(tensor(c.a, 'f32', [c.n]), tensor(c.b, 'f32', [c.n]), c.n, { outputScale: c.outputScale });
+      await save(out, t.buffer, c.n * 4);
+    } else if (c.op === 'silu_rowsplit') {
+      const t = await dh.runSiLURowSplit(tensor(c.x, 'f32', [c.T, 2 * c.dim]), { numTokens: c.T, dim: c.dim, activation: c.activation });
+      await save(out, t.buffer, c.T * c.dim * 4);
+    } else if (c.op === 'gated') {
+      const fn = c.activation === 'silu' ? dh.runSiLU : dh.runGeLU;
+      const t = await fn(tensor(c.up, 'f32', [c.n]), { size: c.n, gate: tensor(c.gate, 'f32', [c.n]) });
+      await save(out, t.buffer, c.n * 4);
+    } else if (c.op === 'gather') {
+      const t = await dh.runGather(dev(c.ids), dev(c.table), c.T, c.hidden, c.vocab, { embeddingDtype: 'f16', outputDtype: 'f32' });
+      await save(out, t.buffer, c.T * c.hidden * 4);
+    } else if (c.op === 'argmax') {
+      const tok = await dh.runArgmax(dev(c.logits), c.vocab, { padTokenId: c.padTokenId });
+      fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array([tok]).buffer));
+    } else if (c.op === 'lm_head') {
+      const rec = dh.createCommandRecorder('lm');
+      const E = dh.createWeightBuffer(dev(c.E), 'f16', 'row', [c.vocab, c.hidden]);
+      const buf = await dh.recordLmHeadArgmaxF16(rec, tensor(c.h, 'f32', [1, c.hidden]), E, { vocabSize: c.vocab, hiddenSize: c.hidden });
+      await rec.submitAndWait();
+      await save(out, buf, 4);
+    } else if (c.op === 'decoder') {
+      const cfg = c.config;
+      const weights = {
+        layers: c.layers.map((l) => ({
+          wqkv: load(l.wqkv), wo: load(l.wo), wgate: load(l.wgate), wup: load(l.wup), wdown: load(l.wdown),
+          inputNorm: load(l.inputNorm), postAttnNorm: load(l.postAttnNorm), qNorm: load(l.qNorm), kNorm: load(l.kNorm),
+        })),
+        embed: load(c.embed), finalNorm: load(c.finalNorm), cos: load(c.cos), sin: load(c.sin),
+      };
+      const dec = new HipTextDecoder(cfg, weights);
+      const tokens = [];
+      let tok = c.prompt[0];
+      for (let pos = 0; pos < c.prompt.length + c.steps; pos++) {
+        const inp = pos < c.prompt.length ? c.prompt[pos] : tok;
+        tok = await dec.decodeStep(inp, pos);
+        tokens.push(tok);
+      }
+      fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
+    } else {
+      throw new Error(`unknown case op ${c.op}`);
+    }
+    results.cases.push(c.name);
+  }
+
+  // error behaviour (reference: synchronous validation -> thrown Error with an [Op] prefix)
+  {
+    const W = dh.createWeightBuffer(dh.acquireBuffer(8 * 144), 'q4k', 'row', [8, 256], 'w');
+    const A = dh.createTensor(dh.acquireBuffer(1024), 'f32', [1, 256], 'a');
+    await expectThrow(results, 'outputDtype', 'outputDtype is required', () => dh.runMatmul(A, W, 1, 8, 256, {}));
+    await expectThrow(results, 'dims', 'Dimensions must be positive', () => dh.runMatmul(A, W, 0, 8, 256, { outputDtype: 'f32' }));
+    await expectThrow(results, 'bsmall', 'B buffer too small', () => dh.runMatmul(A, W, 1, 9, 256, { outputDtype: 'f32' }));
+    await expectThrow(results, 'asmall', 'A buffer too small', () => dh.runMatmul(A, W, 2, 8, 256, { outputDtype: 'f32' }));
+    await expectThrow(results, 'bdtype', 'B dtype is required', () => dh.runMatmul(A, W.buffer, 1, 8, 256, { outputDtype: 'f32' }));
+    await expectThrow(results, 'offsets', '256-byte aligned', () => dh.runMatmul(A, W, 1, 8, 256, { outputDtype: 'f32', aOffset: 4 }));
+    await expectThrow(results, 'rope', 'rotaryDim must be even', () => dh.runRoPE(A, A, A, 1, { numHeads: 1, headDim: 64, rotaryDim: 31 }));
+    await expectThrow(results, 'gather', 'embeddingDtype is required', () => dh.runGather(A.buffer, A.buffer, 1, 8, 8, {}));
+    await expectThrow(results, 'kvwrite', 'smaller than requested range', () => dh.runKVCacheWriteF32ToF16(A.buffer, A.buffer, A.buffer, A.buffer, { elementCount: 100000 }));
+    await expectThrow(results, 'attn', 'kvLayout', () => dh.runAttention(A, A, A, null, 2, 64, { kvLayout: 'paged' }));
+    await expectThrow(results, 'ffn', 'matching gate/up dtypes', () => dh.runFusedFFN(A, W, dh.createWeightBuffer(W.buffer, 'f16', 'row', [8, 256]), 256, 8, {}));
+  }
+
+  fs.writeFileSync(path.join(dir, 'results.json'), JSON.stringify(results));
+  console.log(`ran ${results.cases.length} cases`);
+}
+
+main().catch((e) => {
+  console.error(e && e.stack ? e.stack : e);
+  process.exit(1);
+});

@@ -1,0 +1,206 @@
+"""The JavaScript host path: doppler_amd/js (op API with the reference's signatures) ->
+Node-API addon -> libdopplerhip.so.  pytest writes seeded inputs and the oracle's expected
+outputs to a scratch directory, one node process (tests/js/run_cases.mjs) runs every case,
+and the results are compared here with the same bars as the Python-host tests."""
+import json
+import os
+import shutil
+import subprocess
+
+import numpy as np
+import pytest
+
+import oracle
+from doppler_amd import decoder, synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+NODE = shutil.which("node")
+ADDON = os.path.join(ROOT, "doppler_amd", "js", "doppler_hip.node")
+
+
+def rel_l2(a, b):
+    a, b = np.asarray(a, np.float64).reshape(-1), np.asarray(b, np.float64).reshape(-1)
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def test_addon_is_built_and_exports_the_op_api():
+    """CPU-side: the addon loads in node and the JS entry module exposes every op name the
+    reference's pipeline imports for this path."""
+    if NODE is None:
+        pytest.skip("node not installed")
+    assert os.path.exists(ADDON), "run python -m doppler_amd.build"
+    code = ("import('%s/doppler_amd/js/kernel-selector.js').then(m => console.log(JSON.stringify(Object.keys(m))))"
+            % ROOT)
+    out = subprocess.run([NODE, "-e", code], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert out.returncode == 0, out.stderr
+    names = set(json.loads(out.stdout))
+    for n in ("runMatmul", "recordMatmul", "runAttention", "recordAttention", "runRMSNorm", "recordRMSNorm", "runRoPE",
+              "recordRoPE", "runKVCacheWriteF32ToF16", "recordKVCacheWriteF32ToF16", "runSplitQKVRMSNormRoPEQK",
+              "recordSplitQKVRMSNormRoPEQK", "runSiLU", "recordSiLU", "runSiLURowSplit", "recordSiLURowSplit", "runGeLU",
+              "recordGeLU", "runResidualAdd", "recordResidualAdd", "runGather", "recordGather", "runFusedFFN",
+              "recordFusedFFN", "runArgmax", "recordArgmax", "recordLmHeadArgmax", "recordLmHeadArgmaxF16",
+              "createTensor", "createWeightBuffer", "acquireBuffer", "releaseBuffer", "uploadData", "readBuffer",
+              "createCommandRecorder", "CommandRecorder"):
+        assert n in names, n
+
+
+@pytest.mark.gpu
+@pytest.mark.timeout(600)
+def test_js_host_path_parity(tmp_path):
+    if NODE is None:
+        pytest.skip("node not installed")
+    d = str(tmp_path)
+    cases, checks = [], []
+
+    def put(name, arr):
+        np.ascontiguousarray(arr).tofile(os.path.join(d, name))
+        return name
+
+    def get(name, dtype):
+        return np.fromfile(os.path.join(d, name), dtype)
+
+    # dequant, bit exact
+    W = synth.q4k_tensor(64, 768, 9000)
+    cases.append(dict(name="dequant", op="dequant", W=put("dq.W", W), blocks=W.size // 144))
+    checks.append(lambda: get("dequant.out.bin", np.float32).tobytes() == oracle.q4k_dequant_blocks(W).tobytes())
+
+    # Q4_K matmul: config 0 GEMV, a config-1 shape at M=4 through recordMatmul, residual + f16 out
+    def mm(name, M, N, K, seed, **kw):
+        Wm = synth.q4k_tensor(N, K, seed)
+        A = synth.normal_f32((M, K), seed + 1)
+        c = dict(name=name, op="matmul", wdtype="q4k", W=put(name + ".W", Wm), A=put(name + ".A", A), M=M, N=N, K=K,
+                 outputDtype=kw.get("outputDtype", "f32"), alpha=kw.get("alpha", 1.0), record=kw.get("record", False))
+        want = oracle.q4k_matmul(A, Wm, M, N, K, c["alpha"])
+        if kw.get("residual"):
+            R = synth.normal_f32((M, N), seed + 2)
+            c["residual"] = put(name + ".R", R)
+            want = want + R
+        cases.append(c)
+        dt = np.float16 if c["outputDtype"] == "f16" else np.float32
+        checks.append(lambda: rel_l2(get(name + ".out.bin", dt).astype(np.float32), want) <= 1e-3)
+
+    mm("mm_cfg0", 1, 2048, 640, 9100)
+    mm("mm_cfg1", 4, 3072, 1024, 9110, record=True)
+    mm("mm_res", 2, 512, 1024, 9120, alpha=0.5, residual=True)
+    mm("mm_f16", 1, 512, 1024, 9130, outputDtype="f16", alpha=2.0 ** -8)
+
+    # f16 weights
+    E = synth.normal_f16_bits((3000, 512), 9200, 0.02)
+    h = synth.normal_f32((1, 512), 9201)
+    cases.append(dict(name="mm_f16w", op="matmul", wdtype="f16", W=put("e.W", E), A=put("e.A", h), M=1, N=3000, K=512,
+                      outputDtype="f32", alpha=1.0, record=False))
+    logits = oracle.f16w_matmul(h, E, 1, 3000, 512)
+    checks.append(lambda: rel_l2(get("mm_f16w.out.bin", np.float32), logits) <= 1e-3)
+    cases.append(dict(name="lm_head", op="lm_head", E="e.W", h="e.A", vocab=3000, hidden=512))
+    checks.append(lambda: int(get("lm_head.out.bin", np.uint32)[0]) == oracle.argmax(logits[0]))
+
+    # fused FFN
+    Wg, Wu = synth.q4k_tensor(1024, 768, 9300), synth.q4k_tensor(1024, 768, 9301)
+    X = synth.normal_f32((2, 768), 9302, 0.02)
+    cases.append(dict(name="ffn", op="fused_ffn", Wg=put("ffn.Wg", Wg), Wu=put("ffn.Wu", Wu), X=put("ffn.X", X), M=2,
+                      hidden=768, inter=1024, activation="silu", alpha=1.0, swigluLimit=5.0))
+    ffn_want = oracle.q4k_ffn_gate_up(X, Wg, Wu, 2, 768, 1024, activation="silu", swiglu_limit=5.0)
+    checks.append(lambda: rel_l2(get("ffn.out.bin", np.float32), ffn_want) <= 1e-3)
+
+    # rmsnorm, rope, split qkv, kv write
+    x = synth.normal_f32((3, 1152), 9400, 3.0)
+    w = synth.normal_f32(1152, 9401, 0.1)
+    r = synth.normal_f32((3, 1152), 9402)
+    cases.append(dict(name="rms", op="rmsnorm", x=put("rms.x", x), w=put("rms.w", w), residual=put("rms.r", r), batch=3,
+                      hidden=1152, eps=1e-6, weightOffset=True, outputScale=0.5))
+    rms_want = oracle.rmsnorm(x, w, 1e-6, weight_offset=True, post_residual=r, output_scale=0.5)
+    checks.append(lambda: rel_l2(get("rms.out.bin", np.float32), rms_want) <= 1e-5)
+
+    cos, sin = synth.rope_tables(128, 64, 1e6)
+    xr = synth.normal_f32((2, 16, 128), 9500)
+    cases.append(dict(name="rope", op="rope", x=put("rope.x", xr), cos=put("cos", cos), sin=put("sin", sin), seq=2,
+                      heads=16, headDim=128, startPos=40, interleaved=False))
+    rope_want = oracle.rope_apply(xr, cos, sin, 2, 16, 128, 40)
+    checks.append(lambda: rel_l2(get("rope.out.bin", np.float32), rope_want) <= 1e-6)
+
+    T, H, Hkv, D, start, max_seq = 2, 16, 8, 128, 37, 64
+    qkv = synth.normal_f32((T, (H + 2 * Hkv) * D), 9600)
+    qw, kw = 1 + synth.normal_f32(D, 9601, 0.1), 1 + synth.normal_f32(D, 9602, 0.1)
+    cases.append(dict(name="split", op="split_qkv", qkv=put("split.qkv", qkv), qw=put("split.qw", qw), kw=put("split.kw", kw),
+                      cos="cos", sin="sin", eps=1e-6, T=T, heads=H, kvHeads=Hkv, headDim=D, startPos=start, maxSeq=max_seq))
+    wk, wv = np.zeros((max_seq, Hkv, D), np.uint16), np.zeros((max_seq, Hkv, D), np.uint16)
+    want_q = oracle.qkv_norm_rope_kvwrite(qkv, qw, kw, cos, sin, T, H, Hkv, D, start, wk, wv, start * Hkv * D)
+    checks.append(lambda: rel_l2(get("split.out.bin", np.float32), want_q) <= 1e-5)
+    checks.append(lambda: np.array_equal(get("split.v.bin", np.uint16), wv.reshape(-1)))
+    checks.append(lambda: rel_l2(get("split.k.bin", np.float16).astype(np.float32), wk.reshape(-1).view(np.float16).astype(np.float32)) <= 5e-4)
+
+    kk, vv = synth.normal_f32(2048, 9700), synth.normal_f32(2048, 9701)
+    cases.append(dict(name="kvw", op="kv_write", k=put("kvw.k", kk), v=put("kvw.v", vv), cacheElems=4096, srcOffset=64,
+                      dstOffset=1024, count=1500))
+    ek, ev = np.zeros(4096, np.uint16), np.zeros(4096, np.uint16)
+    oracle.kv_write_f16(kk, vv, ek, ev, 64, 1024, 1500)
+    checks.append(lambda: np.array_equal(get("kvw.out.bin", np.uint16), ek) and np.array_equal(get("kvw.v.bin", np.uint16), ev))
+
+    # attention, config 3 at ctx 512
+    ctx = 512
+    c3, s3 = synth.rope_tables(128, ctx, 1e6)
+    q = oracle.rope_apply(synth.normal_f32((1, 16, 128), 9800, 128 ** -0.5), c3, s3, 1, 16, 128, ctx - 1)
+    q = q.astype(np.float16).astype(np.float32).reshape(16, 128)
+    kb = oracle.rope_apply(synth.normal_f32((ctx, 8, 128), 9801, 128 ** -0.5), c3, s3, ctx, 8, 128, 0).astype(np.float16).view(np.uint16)
+    vb = synth.normal_f16_bits((ctx, 8, 128), 9802, 128 ** -0.5)
+    cases.append(dict(name="attn", op="attention", Q=put("attn.q", q), K=put("attn.k", kb), V=put("attn.v", vb), heads=16,
+                      kvHeads=8, headDim=128, kvLen=ctx))
+    attn_want = oracle.attention_decode_f16kv(q, kb, vb, 16, 8, 128, ctx)
+    checks.append(lambda: rel_l2(get("attn.out.bin", np.float32), attn_want) <= 1e-3)
+
+    # elementwise, gather, argmax
+    a, b = synth.normal_f32(5000, 9900, 4.0), synth.normal_f32(5000, 9901)
+    cases.append(dict(name="res", op="residual", a=put("ew.a", a), b=put("ew.b", b), n=5000, outputScale=0.25))
+    checks.append(lambda: rel_l2(get("res.out.bin", np.float32), oracle.residual_add(a, b, 0.25)) <= 1e-7)
+    for act in ("silu", "gelu"):
+        cases.append(dict(name="gated_" + act, op="gated", gate="ew.a", up="ew.b", n=5000, activation=act))
+        checks.append(lambda act=act: rel_l2(get("gated_%s.out.bin" % act, np.float32), oracle.act_gate(a, b, act)) <= 1e-5)
+    xs = synth.normal_f32((4, 2 * 640), 9902, 3.0)
+    cases.append(dict(name="rowsplit", op="silu_rowsplit", x=put("rs.x", xs), T=4, dim=640, activation="gelu"))
+    checks.append(lambda: rel_l2(get("rowsplit.out.bin", np.float32), oracle.act_gate_rowsplit(xs, 4, 640, "gelu")) <= 1e-5)
+    ids = np.array([5, 299, 300, 0], np.uint32)
+    tab = synth.normal_f16_bits((300, 640), 9903, 0.02)
+    cases.append(dict(name="gather", op="gather", ids=put("g.ids", ids), table=put("g.tab", tab), T=4, hidden=640, vocab=300))
+    checks.append(lambda: np.array_equal(get("gather.out.bin", np.float32).reshape(4, 640), oracle.gather_f16(ids, tab, 640, 300)))
+    lg = synth.rng(9904).integers(-50, 50, 151936).astype(np.float32)
+    pad = oracle.argmax(lg)
+    cases.append(dict(name="argmax", op="argmax", logits=put("am.l", lg), vocab=151936, padTokenId=pad))
+    checks.append(lambda: int(get("argmax.out.bin", np.uint32)[0]) == oracle.argmax(lg, pad_id=pad))
+
+    # whole decode loop in JavaScript on a small model
+    cfg = dict(layers=2, hidden=512, inter=1024, heads=8, kv_heads=4, head_dim=64, vocab=700, eps=1e-6, qk_norm=1,
+               max_seq=24, theta=1e6)
+    layers, embed, final_norm, mc, ms = decoder.random_model(cfg, seed=77, max_seq=24)
+    jl = []
+    for i, l in enumerate(layers):
+        jl.append(dict(wqkv=put("L%d.qkv" % i, np.concatenate([l["wq"], l["wk"], l["wv"]])), wo=put("L%d.o" % i, l["wo"]),
+                       wgate=put("L%d.g" % i, l["wgate"]), wup=put("L%d.u" % i, l["wup"]), wdown=put("L%d.d" % i, l["wdown"]),
+                       inputNorm=put("L%d.in" % i, l["input_norm"]), postAttnNorm=put("L%d.pn" % i, l["post_attn_norm"]),
+                       qNorm=put("L%d.qn" % i, l["q_norm"]), kNorm=put("L%d.kn" % i, l["k_norm"])))
+    prompt = [int(t) for t in synth.rng(78).integers(0, 700, 6)]
+    cases.append(dict(name="decoder", op="decoder", layers=jl, embed=put("m.embed", embed), finalNorm=put("m.fn", final_norm),
+                      cos=put("m.cos", mc), sin=put("m.sin", ms), prompt=prompt, steps=10,
+                      config=dict(layers=2, hidden=512, inter=1024, heads=8, kvHeads=4, headDim=64, vocab=700, eps=1e-6, maxSeq=24)))
+    ol = []
+    for l in layers:
+        dd = dict(l)
+        dd["cache_k"] = np.zeros((24, 4, 64), np.uint16)
+        dd["cache_v"] = np.zeros((24, 4, 64), np.uint16)
+        ol.append(dd)
+    cpu = oracle.DecoderOracle(cfg, ol, embed, final_norm, mc, ms)
+    want_tokens, tok = [], None
+    for pos in range(len(prompt) + 10):
+        tok = cpu.step(prompt[pos] if pos < len(prompt) else tok, pos)
+        want_tokens.append(tok)
+    checks.append(lambda: [int(t) for t in get("decoder.out.bin", np.uint32)] == want_tokens)
+
+    json.dump(dict(cases=cases), open(os.path.join(d, "manifest.json"), "w"))
+    p = subprocess.run([NODE, os.path.join(ROOT, "tests", "js", "run_cases.mjs"), d], stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True, timeout=500)
+    assert p.returncode == 0, p.stdout
+    res = json.load(open(os.path.join(d, "results.json")))
+    assert res["cases"] == [c["name"] for c in cases]
+    for i, chk in enumerate(checks):
+        assert chk(), "check %d failed" % i
+    bad = [e for e in res["errors"] if not e["ok"]]
+    assert not bad and len(res["errors"]) >= 11, bad
