@@ -207,20 +207,37 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
 }
 
 // One workgroup per query head: out[d] = sum_s e^{m_s - M} o_s[d] / sum_s e^{m_s - M} l_s.
+// The per-split factors are computed once, in parallel over splits, and kept in LDS; the
+// D threads then walk the splits with independent (prefetchable) loads.
 template <int D>
 __global__ __launch_bounds__(D) void attn_decode_merge_kernel(const float* __restrict__ ws,
                                                               float* __restrict__ O, int nsplit) {
+  __shared__ float f_s[1024];
+  __shared__ float red[4];
   const int h = blockIdx.x, d = threadIdx.x;
   const float* base = ws + (int64_t)h * nsplit * (D + 2);
   float M = -FLT_MAX;
-  for (int s = 0; s < nsplit; s++) M = fmaxf(M, base[s * (D + 2) + D]);
-  float num = 0.f, den = 0.f;
-  for (int s = 0; s < nsplit; s++) {
-    const float* w = base + s * (D + 2);
-    const float f = __expf(w[D] - M);
-    num = fmaf(f, w[d], num);
-    den = fmaf(f, w[D + 1], den);
+  for (int s = d; s < nsplit; s += D) M = fmaxf(M, base[s * (D + 2) + D]);
+  M = wave_max(M);
+  if ((d & 63) == 0) red[d >> 6] = M;
+  __syncthreads();
+  M = red[0];
+  for (int w = 1; w < D / 64; w++) M = fmaxf(M, red[w]);
+  __syncthreads();
+  float den = 0.f;
+  for (int s = d; s < nsplit; s += D) {
+    const float f = __expf(base[s * (D + 2) + D] - M);
+    f_s[s] = f;
+    den = fmaf(f, base[s * (D + 2) + D + 1], den);
   }
+  den = wave_sum(den);
+  if ((d & 63) == 0) red[d >> 6] = den;
+  __syncthreads();
+  den = 0.f;
+  for (int w = 0; w < D / 64; w++) den += red[w];
+  float num = 0.f;
+#pragma unroll 8
+  for (int s = 0; s < nsplit; s++) num = fmaf(f_s[s], base[s * (D + 2) + d], num);
   O[(int64_t)h * D + d] = den > 0.f ? num / den : 0.f;
 }
 

@@ -60,6 +60,60 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
   }
 }
 
+// Fast path: hidden a multiple of 4 and at most 256*4*VPT.  Each thread keeps its slice of
+// the row in registers (all 16-byte loads are issued before the first use, so the row costs
+// one memory round trip instead of one per element) and the second pass re-reads nothing.
+template <int VPT>
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const float* __restrict__ x, const void* __restrict__ w,
+                                                          int w_f16, float* __restrict__ out, int hidden,
+                                                          float eps, int w_offset,
+                                                          const float* __restrict__ pre,
+                                                          const float* __restrict__ post,
+                                                          float* __restrict__ prenorm, float out_scale) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * hidden;
+  const int nvec = hidden >> 2;
+  float4 v[VPT];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; j++) {
+    const int iv = threadIdx.x + j * 256;
+    v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (iv < nvec) {
+      v[j] = reinterpret_cast<const float4*>(x + base)[iv];
+      if (pre) {
+        const float4 p = reinterpret_cast<const float4*>(pre + base)[iv];
+        v[j].x += p.x; v[j].y += p.y; v[j].z += p.z; v[j].w += p.w;
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VPT; j++) {
+    ss = fmaf(v[j].x, v[j].x, ss); ss = fmaf(v[j].y, v[j].y, ss);
+    ss = fmaf(v[j].z, v[j].z, ss); ss = fmaf(v[j].w, v[j].w, ss);
+  }
+  const float total = block_sum_256(ss, red);
+  const float inv = 1.0f / sqrtf(total / (float)hidden + eps);
+#pragma unroll
+  for (int j = 0; j < VPT; j++) {
+    const int iv = threadIdx.x + j * 256;
+    if (iv < nvec) {
+      if (prenorm) reinterpret_cast<float4*>(prenorm + base)[iv] = v[j];
+      float4 y;
+      y.x = v[j].x * inv * load_norm_weight(w, w_f16, 4 * iv, w_offset);
+      y.y = v[j].y * inv * load_norm_weight(w, w_f16, 4 * iv + 1, w_offset);
+      y.z = v[j].z * inv * load_norm_weight(w, w_f16, 4 * iv + 2, w_offset);
+      y.w = v[j].w * inv * load_norm_weight(w, w_f16, 4 * iv + 3, w_offset);
+      if (post) {
+        const float4 p = reinterpret_cast<const float4*>(post + base)[iv];
+        y.x += p.x; y.y += p.y; y.z += p.z; y.w += p.w;
+      }
+      y.x *= out_scale; y.y *= out_scale; y.z *= out_scale; y.w *= out_scale;
+      reinterpret_cast<float4*>(out + base)[iv] = y;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------------
 // RoPE in place: one thread per rotated pair.
 // ---------------------------------------------------------------------------------------
@@ -248,9 +302,22 @@ int dh_rmsnorm(const float* d_x, const void* d_weight, int weight_dtype, float* 
     return dh::fail(1, "[%s] weight dtype must be f32 or f16", op);
   if (d_prenorm_out && !d_pre_residual)
     return dh::fail(1, "[%s] prenorm output needs a pre-residual input", op);
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3(batch), dim3(256), 0, dh::stream(), d_x, d_weight,
-                     weight_dtype == DH_F16, d_out, hidden, eps, weight_offset, d_pre_residual,
-                     d_post_residual, d_prenorm_out, output_scale);
+  const uintptr_t align = reinterpret_cast<uintptr_t>(d_x) | reinterpret_cast<uintptr_t>(d_out) |
+                          reinterpret_cast<uintptr_t>(d_pre_residual) | reinterpret_cast<uintptr_t>(d_post_residual) |
+                          reinterpret_cast<uintptr_t>(d_prenorm_out);
+  const bool vec_ok = hidden % 4 == 0 && (align & 15) == 0;
+#define DH_RMS_ARGS d_x, d_weight, weight_dtype == DH_F16, d_out, hidden, eps, weight_offset, d_pre_residual, \
+                    d_post_residual, d_prenorm_out, output_scale
+  if (vec_ok && hidden <= 1024) {
+    hipLaunchKernelGGL(rmsnorm_vec_kernel<1>, dim3(batch), dim3(256), 0, dh::stream(), DH_RMS_ARGS);
+  } else if (vec_ok && hidden <= 4096) {
+    hipLaunchKernelGGL(rmsnorm_vec_kernel<4>, dim3(batch), dim3(256), 0, dh::stream(), DH_RMS_ARGS);
+  } else if (vec_ok && hidden <= 8192) {
+    hipLaunchKernelGGL(rmsnorm_vec_kernel<8>, dim3(batch), dim3(256), 0, dh::stream(), DH_RMS_ARGS);
+  } else {
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(batch), dim3(256), 0, dh::stream(), DH_RMS_ARGS);
+  }
+#undef DH_RMS_ARGS
   DH_CHECK_LAUNCH(op);
   return 0;
 }

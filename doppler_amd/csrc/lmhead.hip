@@ -164,8 +164,12 @@ template <int MT, bool ARGMAX>
 int launch_gemv(F16GemvArgs a, int* parts_out, const char* op) {
   const size_t lds = (size_t)MT * a.K * sizeof(float);
   auto kern = f16w_gemv_kernel<MT, ARGMAX>;
-  DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+  static bool attr_set = false;   // once per instantiation: the call costs microseconds
+  if (!attr_set) {
+    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+    attr_set = true;
+  }
   // ~1024 workgroups when N allows (4 per CU), never more than kMaxParts partial candidates
   int rpw = (int)std::max<int64_t>(1, dh::ceil_div(a.N, (int64_t)4 * 1024));
   int grid = (int)dh::ceil_div(a.N, (int64_t)4 * rpw);
