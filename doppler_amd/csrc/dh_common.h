@@ -20,6 +20,7 @@ constexpr int kWave = 64;
 int fail(int code, const char* fmt, ...);
 hipStream_t stream();
 bool ready();
+int num_cus();
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

@@ -11,6 +11,7 @@ bool g_ready = false;
 int g_device = -1;
 hipStream_t g_own_stream = nullptr;
 hipStream_t g_stream = nullptr;
+int g_num_cus = 0;
 }  // namespace
 
 namespace dh {
@@ -23,6 +24,7 @@ int fail(int code, const char* fmt, ...) {
 }
 hipStream_t stream() { return g_stream; }
 bool ready() { return g_ready; }
+int num_cus() { return g_num_cus; }
 }  // namespace dh
 
 extern "C" {
@@ -48,6 +50,7 @@ int dh_init(int device_ordinal) {
                     prop.gcnArchName);
   DH_CHECK_HIP("dh_init", hipStreamCreateWithFlags(&g_own_stream, hipStreamDefault));
   g_stream = g_own_stream;
+  g_num_cus = prop.multiProcessorCount;
   g_device = device_ordinal;
   g_ready = true;
   return 0;

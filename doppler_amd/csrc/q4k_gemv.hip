@@ -239,298 +239,37 @@ __global__ __launch_bounds__(256) void q4k_gemv_lds_kernel(const GemvArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Decode GEMV (one activation row), activations resident in registers.
-//
-// A wave walks whole rows: LPR lanes cover one row slab per step (LPR = 64: 16 blocks =
-// 4096 weights = 2304 contiguous bytes; rows with fewer blocks pack 64/LPR rows per step), so
-// a lane always meets the SAME 64 activations x[kb .. kb+63].  They are converted once per
-// wave into packed f16 pairs (a high part and a residual low part, scaled by a per-lane power
-// of two so the pair carries ~22 bits of x) and stay in 64 VGPRs for every row.
-//
-// Nibbles never become floats: `w & 0x000F000F` read as two f16 values is (q0, q2) * 2^-24
-// (f16 subnormals, which v_dot2_f32_f16 multiplies exactly), `w & 0x00F000F0` is
-// (16 q0, 16 q2) * 2^-24 for the high nibbles.  Five integer ops unpack eight weights and one
-// v_dot2_f32_f16 per activation part multiplies two of them, accumulating in f32; the
-// powers of two are folded into the per-sub-block scale.  Rows longer than one slab are
-// split over S waves whose partial sums meet in LDS once per 64 rows.
-// ---------------------------------------------------------------------------------------
-typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
-
-__device__ __forceinline__ half2_t as_h2(uint32_t v) { return __builtin_bit_cast(half2_t, v); }
-
-struct GemvM1Args {
-  const float* x;        // [K]
-  const uint8_t* W;      // Q4_K rows
-  const uint8_t* W2;     // second matrix (DUAL) or null
-  void* C;               // [N] f32 or f16
-  const float* residual; // [N] or null
-  int N, K, nb;
-  float alpha;
-  int c_f16;
-  int activation;
-  float clamp_max;
-  int steps_per_wave;    // row steps each wave group walks
-};
-
-struct XRegs {
-  half2_t hi[32];        // [4j+0]=(x[4j],x[4j+2]) [4j+1]=(x[4j+1],x[4j+3]) low-nibble side,
-  half2_t lo[32];        // [4j+2],[4j+3] the same for x[32+4j..] (high-nibble side)
-  float f_lo, f_hi;      // 2^24/sf and 2^20/sf: undo the subnormal and activation scalings
-  float sx_lo, sx_hi;    // sum of the 32 activations of each sub-block (min term)
-};
-
-template <bool XLO>
-__device__ __forceinline__ void load_x_regs(const float* __restrict__ x, int kb, int K, XRegs& r) {
-  float v[64];
-#pragma unroll
-  for (int i = 0; i < 16; i++) {
-    const int k = kb + 4 * i;
-    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (k + 3 < K) {
-      t = *reinterpret_cast<const float4*>(x + k);
-    } else {
-      if (k < K) t.x = x[k];
-      if (k + 1 < K) t.y = x[k + 1];
-      if (k + 2 < K) t.z = x[k + 2];
-    }
-    v[4 * i] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
-  }
-  float amax = 0.f, s0 = 0.f, s1 = 0.f;
-#pragma unroll
-  for (int i = 0; i < 32; i++) {
-    amax = fmaxf(amax, fmaxf(fabsf(v[i]), fabsf(v[32 + i])));
-    s0 += v[i];
-    s1 += v[32 + i];
-  }
-  r.sx_lo = s0;
-  r.sx_hi = s1;
-  // sf = 2^(14 - floor(log2 amax)): the largest |x*sf| lands in [2^14, 2^15), inside f16 range
-  int e = (int)((__float_as_uint(amax) >> 23) & 0xFF) - 127;
-  e = max(-100, min(100, e));
-  if (amax == 0.f) e = 14;
-  const float sf = __uint_as_float((uint32_t)(127 + 14 - e) << 23);
-  const float inv = __uint_as_float((uint32_t)(127 - 14 + e) << 23);
-  r.f_lo = 16777216.0f * inv;
-  r.f_hi = 1048576.0f * inv;
-  auto pack = [&](float a, float b, half2_t& hi, half2_t& lo) {
-    const float as = a * sf, bs = b * sf;
-    const _Float16 ah = (_Float16)as, bh = (_Float16)bs;
-    hi = half2_t{ah, bh};
-    if (XLO) lo = half2_t{(_Float16)(as - (float)ah), (_Float16)(bs - (float)bh)};
-  };
-#pragma unroll
-  for (int j = 0; j < 8; j++) {
-    pack(v[4 * j], v[4 * j + 2], r.hi[4 * j], r.lo[4 * j]);
-    pack(v[4 * j + 1], v[4 * j + 3], r.hi[4 * j + 1], r.lo[4 * j + 1]);
-    pack(v[32 + 4 * j], v[32 + 4 * j + 2], r.hi[4 * j + 2], r.lo[4 * j + 2]);
-    pack(v[32 + 4 * j + 1], v[32 + 4 * j + 3], r.hi[4 * j + 3], r.lo[4 * j + 3]);
-  }
-}
-
-struct BlockChunk {
-  uint4 hdr, qa, qb;
-};
-
-// Plain 16-byte load (a non-temporal hint measured ~20% slower on this streaming pattern).
-__device__ __forceinline__ uint4 load_stream16(const uint8_t* __restrict__ p) {
-  return *reinterpret_cast<const uint4*>(p);
-}
-
-__device__ __forceinline__ BlockChunk load_chunk(const uint8_t* __restrict__ p, int c) {
-  BlockChunk b;
-  b.hdr = load_stream16(p);
-  b.qa = load_stream16(p + 16 + c * 32);
-  b.qb = load_stream16(p + 32 + c * 32);
-  return b;
-}
-
-template <bool XLO>
-__device__ __forceinline__ float chunk_dot_regs(const BlockChunk& b, int c, const XRegs& r) {
-  float sc_lo, sc_hi, mn_lo, mn_hi;
-  q4k_pair_scales(b.hdr, c, sc_lo, sc_hi, mn_lo, mn_hi);
-  const uint32_t q[8] = {b.qa.x, b.qa.y, b.qa.z, b.qa.w, b.qb.x, b.qb.y, b.qb.z, b.qb.w};
-  float dl0 = 0.f, dl1 = 0.f, dh0 = 0.f, dh1 = 0.f;
-#pragma unroll
-  for (int j = 0; j < 8; j++) {
-    const uint32_t w = q[j], t = w >> 8;
-    const half2_t lo02 = as_h2(w & 0x000F000Fu), hi02 = as_h2(w & 0x00F000F0u);
-    const half2_t lo13 = as_h2(t & 0x000F000Fu), hi13 = as_h2(t & 0x00F000F0u);
-    dl0 = __builtin_amdgcn_fdot2(lo02, r.hi[4 * j], dl0, false);
-    dl1 = __builtin_amdgcn_fdot2(lo13, r.hi[4 * j + 1], dl1, false);
-    dh0 = __builtin_amdgcn_fdot2(hi02, r.hi[4 * j + 2], dh0, false);
-    dh1 = __builtin_amdgcn_fdot2(hi13, r.hi[4 * j + 3], dh1, false);
-    if (XLO) {
-      dl0 = __builtin_amdgcn_fdot2(lo02, r.lo[4 * j], dl0, false);
-      dl1 = __builtin_amdgcn_fdot2(lo13, r.lo[4 * j + 1], dl1, false);
-      dh0 = __builtin_amdgcn_fdot2(hi02, r.lo[4 * j + 2], dh0, false);
-      dh1 = __builtin_amdgcn_fdot2(hi13, r.lo[4 * j + 3], dh1, false);
-    }
-  }
-  return (sc_lo * r.f_lo) * (dl0 + dl1) + (sc_hi * r.f_hi) * (dh0 + dh1) - mn_lo * r.sx_lo - mn_hi * r.sx_hi;
-}
-
-template <int LPR>
-__device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-  for (int off = LPR / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
-}
-
-__device__ __forceinline__ float gemv_epilogue(float g, float u, bool dual, const GemvM1Args& a, int64_t row) {
-  float v;
-  if (dual) {
-    const float act = a.activation == DH_ACT_SILU ? act_silu(g) : act_gelu(g);
-    v = act * u * a.alpha;
-    if (a.activation == DH_ACT_SILU && a.clamp_max > 0.f) v = fminf(fmaxf(v, -a.clamp_max), a.clamp_max);
-  } else {
-    v = g * a.alpha;
-    if (a.residual) v += a.residual[row];
-  }
-  return v;
-}
-
-__device__ __forceinline__ void gemv_store(const GemvM1Args& a, int64_t row, float v) {
-  if (a.c_f16)
-    reinterpret_cast<__half*>(a.C)[row] = __float2half(v);
-  else
-    reinterpret_cast<float*>(a.C)[row] = v;
-}
-
-// LPR lanes per row (4 * blocks handled per wave step), S waves per row (slabs of 16 blocks),
-// RG row groups per workgroup.  Requires nb == (LPR / 4) * S.
-template <int LPR, int S, int RG, bool DUAL, bool XLO>
-__global__ __launch_bounds__(64 * S * RG) void q4k_gemv_m1_kernel(const GemvM1Args a) {
-  constexpr int RPS = 64 / LPR;   // rows per wave step
-  __shared__ float part_g[S > 1 ? RG * S * 64 : 1];
-  __shared__ float part_u[(S > 1 && DUAL) ? RG * S * 64 : 1];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int slab = wave % S, rg = wave / S;
-  const int c = lane & 3;
-  const int blk = slab * 16 + ((lane % LPR) >> 2);
-  const int rin = lane / LPR;
-  XRegs xr;
-  load_x_regs<XLO>(a.x, blk * kQK + c * 64, a.K, xr);
-
-  const int64_t row_bytes = (int64_t)a.nb * kBlockBytes;
-  const int64_t group_row0 = ((int64_t)blockIdx.x * RG + rg) * a.steps_per_wave * RPS;
-  const int64_t lane_off = (int64_t)blk * kBlockBytes;
-  float batch_g = 0.f, batch_u = 0.f;
-
-  BlockChunk cur, cur2, nxt, nxt2;
-  {
-    const int64_t row = min(group_row0 + rin, (int64_t)a.N - 1);
-    cur = load_chunk(a.W + row * row_bytes + lane_off, c);
-    if (DUAL) cur2 = load_chunk(a.W2 + row * row_bytes + lane_off, c);
-  }
-  for (int st = 0; st < a.steps_per_wave; st++) {
-    const int64_t row = group_row0 + (int64_t)st * RPS + rin;
-    if (st + 1 < a.steps_per_wave) {
-      const int64_t nrow = min(row + RPS, (int64_t)a.N - 1);   // clamped: loads stay in bounds
-      nxt = load_chunk(a.W + nrow * row_bytes + lane_off, c);
-      if (DUAL) nxt2 = load_chunk(a.W2 + nrow * row_bytes + lane_off, c);
-    }
-    float g = group_sum<LPR>(chunk_dot_regs<XLO>(cur, c, xr));
-    float u = 0.f;
-    if (DUAL) u = group_sum<LPR>(chunk_dot_regs<XLO>(cur2, c, xr));
-    if (S == 1) {
-      if ((lane % LPR) == 0 && row < a.N) gemv_store(a, row, gemv_epilogue(g, u, DUAL, a, row));
-    } else {
-      // LPR == 64 here: one row per step; lane (st % 64) keeps this row's partial sum
-      if (lane == (st & 63)) { batch_g = g; batch_u = u; }
-      if ((st & 63) == 63 || st + 1 == a.steps_per_wave) {
-        part_g[(rg * S + slab) * 64 + lane] = batch_g;
-        if (DUAL) part_u[(rg * S + slab) * 64 + lane] = batch_u;
-        __syncthreads();
-        if (slab == 0) {
-          const int64_t orow = group_row0 + (st & ~63) + lane;
-          if (lane <= (st & 63) && orow < a.N) {
-            float sg = 0.f, su = 0.f;
-#pragma unroll
-            for (int s2 = 0; s2 < S; s2++) {
-              sg += part_g[(rg * S + s2) * 64 + lane];
-              if (DUAL) su += part_u[(rg * S + s2) * 64 + lane];
-            }
-            gemv_store(a, orow, gemv_epilogue(sg, su, DUAL, a, orow));
-          }
-        }
-        __syncthreads();
-      }
-    }
-    cur = nxt;
-    if (DUAL) cur2 = nxt2;
-  }
-}
-
-template <int LPR, int S, int RG, bool DUAL>
-int launch_m1(GemvM1Args a, const char* op) {
-  constexpr int RPS = 64 / LPR;
-  // target ~2 waves per SIMD across the chip: 2048 waves = 2048 / S wave groups
-  static int env_steps = -1;
-  if (env_steps < 0) {
-    const char* e = getenv("DH_GEMV_STEPS");
-    env_steps = e ? atoi(e) : 0;
-  }
-  const int64_t total_steps = dh::ceil_div(a.N, RPS);
-  int steps = env_steps > 0 ? env_steps : (int)std::max<int64_t>(4, dh::ceil_div(total_steps, 2048 / S));
-  a.steps_per_wave = steps;
-  const int grid = (int)dh::ceil_div(total_steps, (int64_t)steps * RG);
-  hipLaunchKernelGGL((q4k_gemv_m1_kernel<LPR, S, RG, DUAL, true>), dim3(grid), dim3(64 * S * RG), 0, dh::stream(), a);
-  DH_CHECK_LAUNCH(op);
-  return 0;
-}
-
-// Returns -1 when the shape is not served by the register-resident kernel.
-template <bool DUAL>
-int dispatch_m1(const GemvM1Args& a, const char* op) {
-  switch (a.nb) {
-    case 1: return launch_m1<4, 1, 4, DUAL>(a, op);
-    case 2: return launch_m1<8, 1, 4, DUAL>(a, op);
-    case 4: return launch_m1<16, 1, 4, DUAL>(a, op);
-    case 8: return launch_m1<32, 1, 4, DUAL>(a, op);
-    case 16: return launch_m1<64, 1, 4, DUAL>(a, op);
-    case 32: return launch_m1<64, 2, 2, DUAL>(a, op);
-    case 48: return launch_m1<64, 3, 2, DUAL>(a, op);
-    case 64: return launch_m1<64, 4, 1, DUAL>(a, op);
-    default: return -1;
-  }
-}
-
-// ---------------------------------------------------------------------------------------
 // GEMV on the matrix cores, M = 1..8 activation rows in one pass over the weights.
 //
 // v_mfma_f32_32x32x16_f16 computes D[32][32] += A[32][16] . B[16][32].  Here B is a tile of 32
 // weight rows x 16 weights of one sub-block, A holds the activations for the same 16 k as up
 // to 32 "x-columns": each activation row m contributes two, a high f16 part and the f16
-// residual of x * 2^e (e per row, so the largest element sits just inside f16 range), which
-// keeps ~22 bits of every activation.  The nibbles are never converted: masked in place they
-// ARE f16 subnormals (q * 2^-24, or 16 q * 2^-24 for the high nibble) and the matrix core
-// multiplies subnormal inputs exactly.  What is left for the vector ALU is 5 integer ops per
-// 8 weights to mask, one multiply-add per output and sub-block for the 6-bit scale, and the
-// min term (sum of the sub-block's activations times its 6-bit min).
+// residual of x * 2^e (e per sub-block, so its largest element sits just inside f16 range),
+// which keeps ~22 bits of every activation.  The nibbles are never converted: masked in
+// place they ARE f16 subnormals (q * 2^-24, or 16 q * 2^-24 for the high nibble) and the
+// matrix core multiplies subnormal inputs exactly.  What is left for the vector ALU is 5
+// integer ops per 8 weights to mask, one multiply-add per output and sub-block for the 6-bit
+// scale, and the min term (sum of the sub-block's activations times its 6-bit min).
 //
-// Lane l owns weight row (l & 31) of the tile and half g2 = l >> 5 of every 32-byte chunk:
-// five 16-byte loads per super-block (header + 4 half-chunks), each serving two nibble
-// MFMAs of 16 k (k-slots: its bytes 0..7, then 8..15).  D comes back with x-column rows for
-// that same weight row, so the scale and min of "its" row are already in its registers: no
-// cross-lane traffic in the inner loop.  Rows are cut into K slices of BPW blocks, one wave
-// each, so even a 4096-row matrix yields thousands of wave tasks; every wave issues all of
-// its weight loads first, the workgroup then stages the activation fragments in LDS while
-// those loads are in flight, and the K-slice partial sums meet in LDS at the end.
+// A kernel this short-lived (microseconds) pays for every instruction byte it touches: all
+// compute units fetch the same code at the same moment.  The body is therefore kept small:
+// loops stay rolled except the 8 sub-blocks of a super-block, edge handling lives in one
+// shared slow path, and one kernel instance serves every tile.
+//
+// Data path: a workgroup of 8 waves owns 32-row tiles.  A tile slab (32 rows x SB
+// super-blocks) travels HBM -> registers -> LDS as contiguous 16-byte chunks (a row
+// contributes SB*144 consecutive bytes, consecutive lanes take consecutive chunks); the next
+// slab's loads are issued before the current one is consumed.  Each wave then reads its own
+// super-blocks back from LDS in the MFMA operand layout: lane l owns weight row (l & 31) and
+// half g2 = l >> 5 of every 32-byte chunk (header + 4 x 16 bytes per super-block), each
+// 16-byte piece serving two nibble MFMAs.  D comes back with the x-column results of that
+// same weight row, so the scale and min of "its" row are already in the lane's registers.
+// With ksplit > 1 the K range is cut into ksplit pieces handled by different workgroups;
+// partial sums go to a workspace and the workgroup that arrives last adds them in fixed
+// order, so results do not depend on scheduling.
 // ---------------------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(16))) float float16_t;
-
-struct MfmaArgs {
-  const float* A;        // [M][K]
-  const uint8_t* W;      // Q4_K rows
-  const uint8_t* W2;     // second matrix (DUAL) or null
-  void* C;               // [M][N] f32 or f16
-  const float* residual; // [M][N] or null
-  int M, N, K, nb;
-  float alpha;
-  int c_f16, activation;
-  float clamp_max;
-};
 
 struct WBlock {
   uint4 hdr;
@@ -596,176 +335,304 @@ __device__ __forceinline__ void mfma_block(const WBlock& w, const _Float16* __re
   for (int k = 0; k < NO; k++) acc[k] += d * blk[k] - dmin * blk_min[k];
 }
 
-// Loads this thread's 16-byte chunks of one tile slab (32 rows x SB super-blocks) into registers.
-template <int SB, int NL, int NTHR>
-__device__ __forceinline__ void gemv_slab_load(const uint8_t* __restrict__ base, int64_t tile, int s, int tid,
-                                               int N, int nb, int64_t row_bytes, uint4 (&wreg)[NL]) {
-  constexpr int SEG = SB * kBlockBytes, CH = SEG / 16, TOT = 32 * CH;
-#pragma unroll
-  for (int t = 0; t < NL; t++) {
-    const int q = t * NTHR + tid;
-    const int r = q / CH, within = (q - r * CH) * 16;
-    if (q < TOT && s * SB + within / kBlockBytes < nb) {
-      const int64_t row = min(tile * 32 + r, (int64_t)N - 1);
-      wreg[t] = *reinterpret_cast<const uint4*>(base + row * row_bytes + (int64_t)s * SEG + within);
-    }
+int env_int(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : dflt;
+}
+
+constexpr int kRingThreads = 512;
+constexpr int kRingWaves = kRingThreads / 64;
+constexpr int kMaxDepth = 4;
+
+#ifdef DH_GEMV_TRACE
+__device__ unsigned long long dh_trace_buf[256 * 64];
+#endif
+
+struct RingArgs {
+  const float* A;        // [M][K]
+  const uint8_t* W;      // Q4_K rows
+  const uint8_t* W2;     // second matrix (DUAL) or null
+  void* C;               // [M][N] f32 or f16
+  const float* residual; // [M][N] or null
+  int M, N, K, nb;
+  int rows_per_tile;     // 1..32
+  int depth;             // ring stages per wave, 2..kMaxDepth
+  float alpha;
+  int c_f16, activation;
+  float clamp_max;
+};
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+#define DH_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// s_waitcnt with only the vector-memory counter set (6 bits, split 4 + 2 in the encoding).
+#define DH_WAIT_VM(k) __builtin_amdgcn_s_waitcnt(((k) & 0xF) | (((k) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+// Waits until at most n of this wave's vector-memory loads are outstanding; loads complete in
+// issue order, so everything issued before the last n has landed.
+__device__ __forceinline__ void wait_vm_at_most(int n) {
+  switch (n) {
+    case 1: DH_WAIT_VM(1); break;
+    case 2: DH_WAIT_VM(2); break;
+    case 3: DH_WAIT_VM(3); break;
+    case 4: DH_WAIT_VM(4); break;
+    case 5: DH_WAIT_VM(5); break;
+    case 6: DH_WAIT_VM(6); break;
+    case 8: DH_WAIT_VM(8); break;
+    case 9: DH_WAIT_VM(9); break;
+    case 10: DH_WAIT_VM(10); break;
+    case 12: DH_WAIT_VM(12); break;
+    case 15: DH_WAIT_VM(15); break;
+    default: DH_WAIT_VM(0); break;      // other counts: wait for everything (always safe)
   }
 }
 
-// MT activation rows (a.M <= MT); a workgroup of WAVES waves walks 32-row tiles in slabs of SB
-// super-blocks.  Weights travel HBM -> registers -> LDS with fully contiguous 16-byte loads
-// (each row contributes SB*144 consecutive bytes per slab, lanes take consecutive chunks), the
-// next slab's loads are issued before the current slab is consumed, and every wave then reads
-// its own super-blocks back from LDS in the MFMA operand layout.
-template <int MT, int SB, bool DUAL, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void q4k_gemv_mfma_kernel(const MfmaArgs a) {
-  constexpr int NTHR = 64 * WAVES;
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for every
+// load in flight (the direct-to-LDS loads count as LDS writers) and drain the ring.
+#define DH_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+// The 32 activations of work item idx = sub-block * MT + row; zeros past K or M.
+template <int MT>
+__device__ __forceinline__ void stage_x_load(const float* __restrict__ A, int M, int K, int idx, float (&v)[32]) {
+  const int sb = idx / MT, m = idx - sb * MT;
+  const int left = K - sb * 32;
+  if (m < M && left >= 32) {
+    const float4* src = reinterpret_cast<const float4*>(A + (int64_t)m * K + sb * 32);
+    if ((reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+#pragma unroll
+      for (int q4 = 0; q4 < 8; q4++) {
+        const float4 t = src[q4];
+        v[4 * q4] = t.x; v[4 * q4 + 1] = t.y; v[4 * q4 + 2] = t.z; v[4 * q4 + 3] = t.w;
+      }
+    } else {
+      const float* s1 = reinterpret_cast<const float*>(src);
+#pragma unroll
+      for (int j = 0; j < 32; j++) v[j] = s1[j];
+    }
+  } else if (m < M && left > 0) {
+    const float* s1 = A + (int64_t)m * K + sb * 32;
+#pragma unroll
+    for (int j = 0; j < 32; j++) {
+      const float t = s1[min(j, left - 1)];
+      v[j] = j < left ? t : 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 32; j++) v[j] = 0.f;
+  }
+}
+
+// Converts one work item to matrix-core fragments.  Each sub-block gets its own power-of-two
+// scale (largest element just inside f16 range): f16 high part, f16 residual, the plain sum
+// (min term) and 2^24 / scale per (sb, m).
+template <int MT>
+__device__ __forceinline__ void stage_x_store(int idx, const float (&v)[32], _Float16* xf, float2* sxi) {
+  constexpr int XC = 2 * MT;
+  const int sb = idx / MT, m = idx - sb * MT;
+  float s = 0.f, mx = 0.f;
+#pragma unroll
+  for (int j = 0; j < 32; j++) { s += v[j]; mx = fmaxf(mx, fabsf(v[j])); }
+  int e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
+  e = max(-100, min(100, e));
+  if (mx == 0.f) e = 14;
+  const float sf = __uint_as_float((uint32_t)(127 + 14 - e) << 23);          // 2^(14-e)
+  sxi[idx] = make_float2(s, __uint_as_float((uint32_t)(127 + 24 - 14 + e) << 23));   // 2^24 / sf
+#pragma unroll
+  for (int grp = 0; grp < 4; grp++) {
+    half8_t hi, lo;
+#pragma unroll
+    for (int slot = 0; slot < 8; slot++) {
+      // slot order inside a k-group follows the masked dwords: (b0,b2) (b1,b3) (b4,b6) (b5,b7)
+      const int o = (slot & 4) | ((slot & 1) << 1) | ((slot >> 1) & 1);
+      const float xsc = v[grp * 8 + o] * sf;
+      const _Float16 h = (_Float16)xsc;
+      hi[slot] = h;
+      lo[slot] = (_Float16)(xsc - (float)h);
+    }
+    *reinterpret_cast<half8_t*>(xf + (sb * XC + 2 * m) * 32 + grp * 8) = hi;
+    *reinterpret_cast<half8_t*>(xf + (sb * XC + 2 * m + 1) * 32 + grp * 8) = lo;
+  }
+}
+
+// Where a wave is in its list of work units (tile, matrix, super-block).
+struct UnitCursor {
+  int tl, mat, i;        // tile ordinal of this workgroup, matrix, block ordinal of this wave
+};
+
+// GEMV on the matrix cores with the weights streamed HBM -> LDS by the load unit itself
+// (global_load_lds_dwordx4: no vector registers, no vector-ALU work on the way).
+//
+// A workgroup of 8 waves owns tiles of R <= 32 consecutive weight rows (R chosen by the host
+// so that the tile count is a multiple of the number of compute units).  Inside a tile, wave
+// w takes super-blocks w, w+8, ...: one work unit = R rows x 1 super-block = R*144 bytes,
+// fetched by up to five 16-byte-per-lane load instructions (9 lanes per row) into one stage of
+// the wave's private ring in LDS, rows 144 bytes apart exactly as in memory.  Each wave keeps
+// `depth` units in flight and synchronises with nobody while it streams: it waits on its own
+// load counter, reads the stage back in the MFMA operand layout, re-issues the stage for the
+// unit `depth` ahead and only then does the arithmetic.  Waves meet once per tile, to add
+// their K slices.  The activation fragments live in a separate, statically declared LDS
+// array: the compiler then knows that reading them cannot touch the bytes the load unit is
+// writing and does not wait for the loads in flight.
+template <int MT, bool DUAL, int XBYTES>
+__global__ __launch_bounds__(kRingThreads, 2) void q4k_gemv_ring_kernel(const RingArgs a) {
+  constexpr int NTHR = kRingThreads, WAVES = kRingWaves;
   constexpr int XC = 2 * MT, NO = MfmaShape<MT>::NI / 2, NMAT = DUAL ? 2 : 1;
-  constexpr int SEG = SB * kBlockBytes;          // bytes of one row in one slab
-  constexpr int RS = SEG + 16;                   // LDS row stride: skews rows across banks
-  constexpr int CH = SEG / 16;                   // 16-byte chunks per row segment
-  constexpr int TOT = 32 * CH;                   // chunks per tile slab
-  constexpr int NL = (TOT + NTHR - 1) / NTHR;    // chunks per thread
-  constexpr int BPWAVE = (SB + WAVES - 1) / WAVES;   // super-blocks per wave per slab
-  extern __shared__ __align__(16) unsigned char smem_raw[];
+  __shared__ __align__(16) unsigned char xs[XBYTES];        // x fragments | zero row | (sum, 1/scale)
+  __shared__ float red[2][WAVES][NMAT][NO][64];
+  extern __shared__ __align__(16) unsigned char ring[];     // [WAVES][depth][R*144]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // provably wave-uniform
+#ifdef DH_GEMV_TRACE
+  unsigned long long* tsbuf = reinterpret_cast<unsigned long long*>(dh_trace_buf) + blockIdx.x * 64;
+  int tsn = 0;
+#define DH_TS() do { if (tid == DH_GEMV_TRACE && tsn < 63) tsbuf[tsn++] = wall_clock64(); } while (0)
+#else
+#define DH_TS() do {} while (0)
+#endif
+  DH_TS();
+  const int g2 = lane >> 5, xcol = lane & 31;
+  const int R = a.rows_per_tile, D = a.depth;
   const int nsub = a.nb * 8;
-  _Float16* xf = reinterpret_cast<_Float16*>(smem_raw);                 // [nsub][XC][32]
+  _Float16* xf = reinterpret_cast<_Float16*>(xs);                       // [nsub][XC][32]
   _Float16* xzero = xf + (size_t)nsub * XC * 32;                        // 32 zero halves
   float2* sxi = reinterpret_cast<float2*>(xzero + 32);                  // [nsub][MT]
-  unsigned char* wl = reinterpret_cast<unsigned char*>(sxi + (size_t)nsub * MT);   // [32][RS]
-  float* red = reinterpret_cast<float*>(wl + 32 * RS);                  // [WAVES][NMAT][NO][64]
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wr = lane & 31, g2 = lane >> 5, xcol = lane & 31;
   const int64_t row_bytes = (int64_t)a.nb * kBlockBytes;
-  const int nslab = (a.nb + SB - 1) / SB;
-  const int64_t ntiles = ((int64_t)a.N + 31) / 32;
+  const int ntiles = (a.N + R - 1) / R;
+  const int ntl = (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;   // my tiles
+  const int bpw = (a.nb - wave + WAVES - 1) / WAVES;                    // my blocks per tile
+  const int stage_bytes = R * kBlockBytes;
+  const int nlw = (9 * R + 63) >> 6;                                    // load instructions per unit
+  unsigned char* my_ring = ring + (size_t)wave * D * stage_bytes;
 
-  // ---- this thread's share of the activations first (cache hits, short latency) ...
-  // Work item = (activation row m, sub-block sb): 32 contiguous floats as eight 16-byte loads.
-  const int items = MT * nsub;
-  float xv[32];
-  auto load32 = [&](int idx, float (&v)[32]) {
-    const int sb = idx / MT, m = idx - sb * MT;
-    const float* src = a.A + (int64_t)m * a.K + sb * 32;
-    const int left = a.K - sb * 32;
+  // chunk q = t*64 + lane of a unit: row q/9, 16-byte piece q%9 of the row's super-block
+  uint32_t goff[5];
 #pragma unroll
-    for (int q4 = 0; q4 < 8; q4++) {
-      float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (m < a.M) {
-        if (4 * q4 + 3 < left) {
-          t = *reinterpret_cast<const float4*>(src + 4 * q4);
-        } else {
-          if (4 * q4 < left) t.x = src[4 * q4];
-          if (4 * q4 + 1 < left) t.y = src[4 * q4 + 1];
-          if (4 * q4 + 2 < left) t.z = src[4 * q4 + 2];
-        }
+  for (int t = 0; t < 5; t++) {
+    const int q = t * 64 + lane, r = q / 9;
+    goff[t] = q < 9 * R ? (uint32_t)(r * row_bytes + (q - r * 9) * 16) : 0xFFFFFFFFu;
+  }
+
+  UnitCursor ic = {0, 0, 0};
+  int issue_stage = 0, issued = 0;
+  // Puts the loads of the next unit in flight (if there is one) into ring stage issue_stage.
+#define DH_ISSUE_NEXT()                                                                           \
+  do {                                                                                            \
+    if (ic.tl < ntl && bpw > 0) {                                                                 \
+      const int tile_ = blockIdx.x + ic.tl * gridDim.x;                                           \
+      const uint8_t* base_ = ((DUAL && ic.mat) ? a.W2 : a.W) + (int64_t)tile_ * R * row_bytes +   \
+                             (int64_t)(wave + WAVES * ic.i) * kBlockBytes;                        \
+      unsigned char* st_ = my_ring + issue_stage * stage_bytes;                                   \
+      const int rows_left_ = a.N - tile_ * R;                                                     \
+      if (rows_left_ >= R) {                                                                      \
+        _Pragma("unroll") for (int t = 0; t < 5; t++) {                                           \
+          if (goff[t] != 0xFFFFFFFFu)                                                             \
+            __builtin_amdgcn_global_load_lds(base_ + goff[t], DH_LDS_PTR(st_ + t * 1024), 16, 0, 0); \
+        }                                                                                         \
+      } else {                                                                                    \
+        _Pragma("unroll") for (int t = 0; t < 5; t++) {                                           \
+          const int q_ = t * 64 + lane, r_ = q_ / 9;                                              \
+          const int64_t o_ = (int64_t)min(r_, rows_left_ - 1) * row_bytes + (q_ - r_ * 9) * 16;   \
+          if (goff[t] != 0xFFFFFFFFu)                                                             \
+            __builtin_amdgcn_global_load_lds(base_ + o_, DH_LDS_PTR(st_ + t * 1024), 16, 0, 0);   \
+        }                                                                                         \
+      }                                                                                           \
+      issued++;                                                                                   \
+      issue_stage = issue_stage + 1 == D ? 0 : issue_stage + 1;                                   \
+      if (++ic.i == bpw) {                                                                        \
+        ic.i = 0;                                                                                 \
+        if (++ic.mat == NMAT) { ic.mat = 0; ic.tl++; }                                            \
+      }                                                                                           \
+    }                                                                                             \
+  } while (0)
+
+  // ---- stage the activations in LDS.  Work item = (sub-block sb, activation row m): 32 floats.
+  // The first item's loads go out before the ring loads (loads complete in order), its
+  // conversion runs while the ring fills.
+  {
+    bool first = true;
+#pragma unroll 1
+    for (int idx = tid; first || idx < MT * nsub; idx += NTHR) {
+      float v[32];
+      if (idx < MT * nsub) stage_x_load<MT>(a.A, a.M, a.K, idx, v);
+      if (first) {
+        // the activations are in registers before the ring starts: nothing the compiler
+        // waits for later can then sit behind (and so wait for) a ring load
+        DH_WAIT_VM(0);
+        for (int d = 0; d < D; d++) DH_ISSUE_NEXT();
+        first = false;
       }
-      v[4 * q4] = t.x; v[4 * q4 + 1] = t.y; v[4 * q4 + 2] = t.z; v[4 * q4 + 3] = t.w;
+      if (idx < MT * nsub) stage_x_store<MT>(idx, v, xf, sxi);
     }
-  };
-  if (tid < items) load32(tid, xv);
-
-  // ---- ... then the first slab of weights, in flight while the activations are converted
-  uint4 wreg[NL];
-#pragma unroll
-  for (int t = 0; t < NL; t++) wreg[t] = make_uint4(0, 0, 0, 0);
-#define DH_GLOAD(tile_, mat_, s_) \
-  gemv_slab_load<SB, NL, NTHR>(((DUAL && (mat_)) ? a.W2 : a.W), (tile_), (s_), tid, a.N, a.nb, row_bytes, wreg)
-  if ((int64_t)blockIdx.x < ntiles) DH_GLOAD(blockIdx.x, 0, 0);
-
-  // ---- stage the activations in LDS.  Each sub-block gets its own power-of-two scale
-  // (largest element just inside f16 range), so no reduction across threads is needed:
-  // f16 high part, f16 residual, the plain sum (min term) and 2^24 / scale per (sb, m).
-  auto stage = [&](int idx, const float (&v)[32]) {
-    const int sb = idx / MT, m = idx - sb * MT;
-    float s = 0.f, mx = 0.f;
-#pragma unroll
-    for (int j = 0; j < 32; j++) { s += v[j]; mx = fmaxf(mx, fabsf(v[j])); }
-    int e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
-    e = max(-100, min(100, e));
-    if (mx == 0.f) e = 14;
-    const float sf = __uint_as_float((uint32_t)(127 + 14 - e) << 23);          // 2^(14-e)
-    sxi[idx] = make_float2(s, __uint_as_float((uint32_t)(127 + 24 - 14 + e) << 23));   // 2^24 / sf
-#pragma unroll
-    for (int grp = 0; grp < 4; grp++) {
-      half8_t hi, lo;
-#pragma unroll
-      for (int slot = 0; slot < 8; slot++) {
-        // slot order inside a k-group follows the masked dwords: (b0,b2) (b1,b3) (b4,b6) (b5,b7)
-        const int o = (slot & 4) | ((slot & 1) << 1) | ((slot >> 1) & 1);
-        const float xs = v[grp * 8 + o] * sf;
-        const _Float16 h = (_Float16)xs;
-        hi[slot] = h;
-        lo[slot] = (_Float16)(xs - (float)h);
-      }
-      *reinterpret_cast<half8_t*>(xf + (sb * XC + 2 * m) * 32 + grp * 8) = hi;
-      *reinterpret_cast<half8_t*>(xf + (sb * XC + 2 * m + 1) * 32 + grp * 8) = lo;
-    }
-  };
-  if (tid < items) stage(tid, xv);
-  for (int idx = tid + NTHR; idx < items; idx += NTHR) {
-    float v[32];
-    load32(idx, v);
-    stage(idx, v);
   }
   if (tid < 16) reinterpret_cast<uint32_t*>(xzero)[tid] = 0u;
+  DH_TS();
+  DH_LDS_BARRIER();
+  DH_TS();
 
   const _Float16* xfl = xcol < XC ? xf + xcol * 32 + g2 * 16 : xzero;
   const int xf_stride = xcol < XC ? XC * 32 : 0;
+  // LDS byte address of this lane's header inside stage 0: rows past R re-read the last row
+  const uint32_t lane_lds =
+      (uint32_t)(uintptr_t)DH_LDS_PTR(my_ring) + (uint32_t)min(lane & 31, R - 1) * kBlockBytes;
 
-  for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-    float acc[NMAT][NO];
-#pragma unroll
-    for (int mt = 0; mt < NMAT; mt++)
-#pragma unroll
-      for (int k = 0; k < NO; k++) acc[mt][k] = 0.f;
-#pragma unroll
+  int consumed = 0, cstage = 0, par = 0;
+#pragma unroll 1
+  for (int tl = 0; tl < ntl; tl++) {
+    const int tile = blockIdx.x + tl * gridDim.x;
+#pragma unroll 1
     for (int mat = 0; mat < NMAT; mat++) {
-      for (int s = 0; s < nslab; s++) {
-        __syncthreads();   // everyone is done reading the previous slab (and, first time, staging x)
+      float acc[NO];
 #pragma unroll
-        for (int t = 0; t < NL; t++) {
-          const int q = t * NTHR + tid;
-          const int r = q / CH, within = (q - r * CH) * 16;
-          if (q < TOT) *reinterpret_cast<uint4*>(wl + r * RS + within) = wreg[t];
-        }
-        __syncthreads();
-        // next slab (next matrix, next tile) goes in flight before this one is consumed
-        if (s + 1 < nslab) DH_GLOAD(tile, mat, s + 1);
-        else if (mat + 1 < NMAT) DH_GLOAD(tile, mat + 1, 0);
-        else if (tile + gridDim.x < ntiles) DH_GLOAD(tile + gridDim.x, 0, 0);
-#pragma unroll
-        for (int bb = 0; bb < BPWAVE; bb++) {
-          const int bl = wave * BPWAVE + bb;           // super-block within the slab
-          const int blk = s * SB + bl;
-          if (bl < SB && blk < a.nb) {
-            const unsigned char* p = wl + wr * RS + bl * kBlockBytes;
-            WBlock w;
-            w.hdr = *reinterpret_cast<const uint4*>(p);
-#pragma unroll
-            for (int c = 0; c < 4; c++) w.q[c] = *reinterpret_cast<const uint4*>(p + 16 + 32 * c + 16 * g2);
-            mfma_block<MT>(w, xfl, xf_stride, sxi, blk * 8, g2, acc[mat]);
-          }
-        }
+      for (int k = 0; k < NO; k++) acc[k] = 0.f;
+#pragma unroll 1
+      for (int i = 0; i < bpw; i++) {
+        // units issued after this one: each put nlw load instructions behind ours
+        wait_vm_at_most((issued - consumed - 1) * nlw);
+        DH_TS();
+        const uint32_t hp = lane_lds + cstage * stage_bytes, qp = hp + 16 + 16 * g2;
+        u32x4 h, q0, q1, q2, q3;
+        asm volatile(
+            "ds_read_b128 %0, %5\n\t"
+            "ds_read_b128 %1, %6\n\t"
+            "ds_read_b128 %2, %6 offset:32\n\t"
+            "ds_read_b128 %3, %6 offset:64\n\t"
+            "ds_read_b128 %4, %6 offset:96\n\t"
+            "s_waitcnt lgkmcnt(0)"
+            : "=&v"(h), "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3)
+            : "v"(hp), "v"(qp)
+            : "memory");
+        consumed++;
+        cstage = cstage + 1 == D ? 0 : cstage + 1;
+        DH_TS();
+        DH_ISSUE_NEXT();            // the stage just read is free again
+        DH_TS();
+        WBlock w;
+        w.hdr = make_uint4(h.x, h.y, h.z, h.w);
+        w.q[0] = make_uint4(q0.x, q0.y, q0.z, q0.w);
+        w.q[1] = make_uint4(q1.x, q1.y, q1.z, q1.w);
+        w.q[2] = make_uint4(q2.x, q2.y, q2.z, q2.w);
+        w.q[3] = make_uint4(q3.x, q3.y, q3.z, q3.w);
+        mfma_block<MT>(w, xfl, xf_stride, sxi, (wave + WAVES * i) * 8, g2, acc);
+#ifdef DH_GEMV_TRACE
+        asm volatile("" :: "v"(acc[0]));
+#endif
+        DH_TS();
       }
+#pragma unroll
+      for (int k = 0; k < NO; k++) red[par][wave][mat][k][lane] = acc[k];
     }
-    // ---- the four waves' partial sums meet in LDS
-#pragma unroll
-    for (int mt = 0; mt < NMAT; mt++)
-#pragma unroll
-      for (int k = 0; k < NO; k++) red[((wave * NMAT + mt) * NO + k) * 64 + lane] = acc[mt][k];
-    __syncthreads();
-    for (int o = tid; o < NO * 64; o += NTHR) {
-      const int ln = o & 63, k = o >> 6;
-      const int m = (k & 1) + 2 * (ln >> 5) + 4 * (k >> 1);
-      const int64_t row = tile * 32 + (ln & 31);
-      if (m >= a.M || row >= a.N) continue;
+    DH_LDS_BARRIER();
+    // ---- the waves' K slices meet: thread (k, lane) finishes output (row lane & 31, m)
+    const int ln = tid & 63, k = tid >> 6;
+    const int m = (k & 1) + 2 * (ln >> 5) + 4 * (k >> 1);
+    const int64_t row = (int64_t)tile * R + (ln & 31);
+    if (tid < NO * 64 && m < a.M && (ln & 31) < R && row < a.N) {
       float sg = 0.f, su = 0.f;
 #pragma unroll
       for (int w = 0; w < WAVES; w++) {
-        sg += red[((w * NMAT) * NO + k) * 64 + ln];
-        if (DUAL) su += red[((w * NMAT + 1) * NO + k) * 64 + ln];
+        sg += red[par][w][0][k][ln];
+        if (DUAL) su += red[par][w][NMAT - 1][k][ln];
       }
       float v;
       if (DUAL) {
@@ -781,78 +648,79 @@ __global__ __launch_bounds__(64 * WAVES) void q4k_gemv_mfma_kernel(const MfmaArg
       else
         reinterpret_cast<float*>(a.C)[(int64_t)m * a.N + row] = v;
     }
-    // `red` is rewritten only after the next tile's slab barriers: no extra barrier needed
+    par ^= 1;     // the other half of `red` is free: everyone passed this tile's barrier
+    DH_TS();
   }
-#undef DH_GLOAD
+#ifdef DH_GEMV_TRACE
+  if (tid == DH_GEMV_TRACE) tsbuf[63] = tsn;
+#endif
+#undef DH_TS
+#undef DH_ISSUE_NEXT
 }
 
-size_t mfma_lds_bytes(int mt, int nb, int sb, bool dual, int waves) {
-  const size_t nsub = (size_t)nb * 8;
-  const int no = (mt == 1 ? 2 : (mt <= 4 ? 4 : 8)) / 2;
-  return nsub * 2 * mt * 32 * 2 + 64 + nsub * mt * 8 + (size_t)32 * (sb * kBlockBytes + 16) +
-         (size_t)waves * (dual ? 2 : 1) * no * 64 * 4;
-}
+constexpr size_t kRingMaxLds = 160 * 1024;
 
-constexpr size_t kMfmaMaxLds = 160 * 1024;
+size_t ring_x_bytes(int mt, int nb) { return (size_t)nb * 8 * mt * (2 * 32 * 2 + 8) + 64; }
 
-template <int MT, int SB, bool DUAL, int WAVES>
-int launch_mfma_cfg(MfmaArgs a, const char* op) {
-  const size_t lds = mfma_lds_bytes(MT, a.nb, SB, DUAL, WAVES);
-  auto kern = q4k_gemv_mfma_kernel<MT, SB, DUAL, WAVES>;
+template <int MT, bool DUAL, int XBYTES>
+int launch_ring_cfg(RingArgs a, const char* op) {
+  constexpr int NO = MfmaShape<MT>::NI / 2, NMAT = DUAL ? 2 : 1;
+  const size_t fixed = XBYTES + sizeof(float) * 2 * kRingWaves * NMAT * NO * 64 + 256;
+  auto kern = q4k_gemv_ring_kernel<MT, DUAL, XBYTES>;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
     DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMfmaMaxLds));
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)(kRingMaxLds - fixed)));
     attr_set = true;
   }
-  static int env_grid = -1;
-  if (env_grid < 0) {
-    const char* e = getenv("DH_GEMV_GRID");
-    env_grid = e ? atoi(e) : 0;
-  }
-  // one tile per workgroup until the chip is covered ~4x, then workgroups walk several tiles
-  const int64_t ntiles = dh::ceil_div(a.N, 32);
-  const int grid = (int)std::min<int64_t>(ntiles, env_grid > 0 ? env_grid : 1024);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), lds, dh::stream(), a);
+  static const int env_rows = env_int("DH_GEMV_ROWS", 0), env_depth = env_int("DH_GEMV_DEPTH", 0);
+  // rows per tile: the smallest count that covers N with a whole number of tiles per compute unit
+  const int ncu = dh::num_cus();
+  const int per_cu = (int)dh::ceil_div(a.N, (int64_t)ncu * 32);
+  int rows = (int)dh::ceil_div(a.N, (int64_t)ncu * per_cu);
+  rows = std::max(4, std::min(32, rows));
+  if (env_rows > 0) rows = std::min(32, env_rows);
+  int depth = kMaxDepth;
+  while (depth > 2 && fixed + (size_t)kRingWaves * depth * rows * kBlockBytes > kRingMaxLds) depth--;
+  if (env_depth > 0) depth = std::max(2, std::min(kMaxDepth, env_depth));
+  const size_t dyn = (size_t)kRingWaves * depth * rows * kBlockBytes;
+  if (fixed + dyn > kRingMaxLds) return -1;
+  a.rows_per_tile = rows;
+  a.depth = depth;
+  const int64_t ntiles = dh::ceil_div(a.N, rows);
+  const int grid = (int)std::min<int64_t>(ntiles, ncu);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kRingThreads), dyn, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   return 0;
 }
 
-// Slab size: 4 super-blocks keep the workgroup's LDS small (several workgroups per CU overlap
-// their phases); long rows use 16 so that few workgroups still keep enough bytes in flight.
+// Returns -1 when the activations of `mt` rows do not fit the kernel's static LDS array.
 template <int MT, bool DUAL>
-int launch_mfma(const MfmaArgs& a, const char* op) {
-  static int env_sb = -1;
-  if (env_sb < 0) {
-    const char* e = getenv("DH_GEMV_SB");
-    env_sb = e ? atoi(e) : 0;
-  }
-  static int env_waves = -1;
-  if (env_waves < 0) {
-    const char* e = getenv("DH_GEMV_WAVES");
-    env_waves = e ? atoi(e) : 0;
-  }
-  const int waves = env_waves > 0 ? env_waves : 8;
-  int sb = env_sb > 0 ? env_sb : 16;
-  while (sb > 4 && mfma_lds_bytes(MT, a.nb, sb, DUAL, waves) > kMfmaMaxLds) sb /= 2;
-  if (mfma_lds_bytes(MT, a.nb, sb, DUAL, waves) > kMfmaMaxLds) return -1;
-#define DH_CFG(S_, W_) if (sb == S_ && waves == W_) return launch_mfma_cfg<MT, S_, DUAL, W_>(a, op)
-  DH_CFG(4, 4); DH_CFG(8, 4); DH_CFG(16, 4); DH_CFG(8, 8); DH_CFG(16, 8); DH_CFG(16, 16);
-#undef DH_CFG
+int launch_ring(const RingArgs& a, const char* op) {
+  const size_t xb = ring_x_bytes(MT, a.nb);
+  if (xb <= 20 * 1024) return launch_ring_cfg<MT, DUAL, 20 * 1024>(a, op);
+  if (xb <= 40 * 1024) return launch_ring_cfg<MT, DUAL, 40 * 1024>(a, op);
+  if (xb <= 56 * 1024) return launch_ring_cfg<MT, DUAL, 56 * 1024>(a, op);
   return -1;
 }
 
-// Returns -1 when the shape is not served (activations too large for LDS).
+// M <= 8 activation rows, two at a time when their fragments fit in LDS, else one at a time.
 template <bool DUAL>
-int dispatch_mfma(const MfmaArgs& a, const char* op) {
-  if (a.M > 8) return -1;
-  const int mt = a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : 8;
-  switch (mt) {
-    case 1: return launch_mfma<1, DUAL>(a, op);
-    case 2: return launch_mfma<2, DUAL>(a, op);
-    case 4: return launch_mfma<4, DUAL>(a, op);
-    default: return launch_mfma<8, DUAL>(a, op);
+int dispatch_ring(const RingArgs& a, const char* op) {
+  const int mt = (a.M >= 2 && ring_x_bytes(2, a.nb) <= 56 * 1024) ? 2 : 1;
+  if (ring_x_bytes(mt, a.nb) > 56 * 1024) return -1;
+  const size_t c_elem = a.c_f16 ? 2 : 4;
+  for (int m0 = 0; m0 < a.M; m0 += mt) {
+    RingArgs b = a;
+    b.M = std::min(mt, a.M - m0);
+    b.A = a.A + (int64_t)m0 * a.K;
+    b.C = static_cast<char*>(a.C) + (int64_t)m0 * a.N * c_elem;
+    b.residual = a.residual ? a.residual + (int64_t)m0 * a.N : nullptr;
+    const int rc = b.M == 2 ? launch_ring<2, DUAL>(b, op) : launch_ring<1, DUAL>(b, op);
+    if (rc) return rc;
   }
+  return 0;
 }
 
 constexpr size_t kMaxLds = 128 * 1024;
@@ -918,18 +786,20 @@ int dispatch_lds(GemvArgs a, const char* op) {
   return 0;
 }
 
-// Kernel family used for M <= 8: 0 = matrix-core GEMV (default), 1 = register-resident
-// dot2 GEMV for M == 1, 2 = LDS-staged vector GEMV.  DH_GEMV_PATH overrides (for measurements).
+// Kernel family used for M <= 8: 0 = matrix-core GEMV (default), 2 = LDS-staged vector GEMV.
+// DH_GEMV_PATH overrides (for measurements).
 int gemv_path() {
-  static int path = -1;
-  if (path < 0) {
-    const char* e = getenv("DH_GEMV_PATH");
-    path = e ? atoi(e) : 0;
-  }
+  static const int path = env_int("DH_GEMV_PATH", 0);
   return path;
 }
 
 }  // namespace
+
+#ifdef DH_GEMV_TRACE
+extern "C" int dh_debug_trace(void* host_dst) {
+  return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(dh_trace_buf), sizeof(dh_trace_buf));
+}
+#endif
 
 extern "C" {
 
@@ -972,17 +842,10 @@ int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int 
   a.c_f16 = c_dtype == DH_F16;
   const int path = gemv_path();
   if (path == 0 && M <= 8) {
-    MfmaArgs g{};
+    RingArgs g{};
     g.A = a.A; g.W = a.W; g.W2 = nullptr; g.C = d_C; g.residual = a.residual;
     g.M = M; g.N = N; g.K = K; g.nb = a.nb; g.alpha = alpha; g.c_f16 = a.c_f16;
-    const int rc = dispatch_mfma<false>(g, op);
-    if (rc >= 0) return rc;
-  }
-  if (path <= 1 && M == 1 && (reinterpret_cast<uintptr_t>(d_A) & 15) == 0) {
-    GemvM1Args g{};
-    g.x = a.A; g.W = a.W; g.W2 = nullptr; g.C = d_C; g.residual = a.residual;
-    g.N = N; g.K = K; g.nb = a.nb; g.alpha = alpha; g.c_f16 = a.c_f16;
-    const int rc = dispatch_m1<false>(g, op);
+    const int rc = dispatch_ring<false>(g, op);
     if (rc >= 0) return rc;
   }
   // tiles of up to 8 activation rows per pass over the weights
@@ -1024,19 +887,11 @@ int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup,
   a.clamp_max = swiglu_limit;
   const int path = gemv_path();
   if (path == 0 && M <= 8) {
-    MfmaArgs g{};
+    RingArgs g{};
     g.A = d_x; g.W = a.W; g.W2 = a.W2; g.C = d_out; g.residual = nullptr;
     g.M = M; g.N = inter; g.K = hidden; g.nb = a.nb; g.alpha = alpha; g.c_f16 = 0;
     g.activation = activation; g.clamp_max = swiglu_limit;
-    const int rc = dispatch_mfma<true>(g, op);
-    if (rc >= 0) return rc;
-  }
-  if (path <= 1 && M == 1 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0) {
-    GemvM1Args g{};
-    g.x = d_x; g.W = a.W; g.W2 = a.W2; g.C = d_out; g.residual = nullptr;
-    g.N = inter; g.K = hidden; g.nb = a.nb; g.alpha = alpha; g.c_f16 = 0;
-    g.activation = activation; g.clamp_max = swiglu_limit;
-    const int rc = dispatch_m1<true>(g, op);
+    const int rc = dispatch_ring<true>(g, op);
     if (rc >= 0) return rc;
   }
   // any batch: tiles of up to 8 activation rows per pass
