@@ -34,25 +34,31 @@ def log(*a):
 def gate_up_kernel_bandwidth(dec, reps):
     """Average duration of the fused gate/up GEMV launch, measured with HIP events on the
     stream the kernel runs on.  Launches cycle through the layers' weights (36 x 56.6 MB,
-    far beyond the 256 MB infinity cache) so every launch streams from HBM."""
+    far beyond the 256 MB infinity cache) so every launch streams from HBM; the launches of
+    one sweep are enqueued back to back between two events, so the figure is the kernel's
+    duration plus the dispatch gap between consecutive kernels."""
     from doppler_amd import capi
     L, c = dec.L, dec.cfg
     Hd, I = c["hidden"], c["inter"]
     ev = [ctypes.c_void_p() for _ in range(2)]
     for e in ev:
         capi.check(L.dh_event_create(ctypes.byref(e)))
-    total_ms, n = 0.0, 0
-    for r in range(reps):
+
+    def sweep():
         for d in dec.layers:
-            capi.check(L.dh_event_record(ev[0]))
             capi.check(L.dh_q4k_ffn_gate_up(dec.normed.data_ptr(), d["wgate"].data_ptr(), d["wup"].data_ptr(),
                                             dec.act.data_ptr(), 1, Hd, I, capi.ACT_SILU, 1.0, 0.0))
-            capi.check(L.dh_event_record(ev[1]))
-            ms = ctypes.c_float()
-            capi.check(L.dh_event_elapsed_ms(ev[0], ev[1], ctypes.byref(ms)))
-            if r > 0:                      # first sweep warms code and TLBs
-                total_ms += ms.value
-                n += 1
+    sweep()                                # warms code and TLBs
+    capi.check(L.dh_sync())
+    total_ms, n = 0.0, 0
+    for r in range(reps):
+        capi.check(L.dh_event_record(ev[0]))
+        sweep()
+        capi.check(L.dh_event_record(ev[1]))
+        ms = ctypes.c_float()
+        capi.check(L.dh_event_elapsed_ms(ev[0], ev[1], ctypes.byref(ms)))
+        total_ms += ms.value
+        n += len(dec.layers)
     for e in ev:
         capi.check(L.dh_event_destroy(e))
     return total_ms / max(n, 1)
