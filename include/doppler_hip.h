@@ -7,8 +7,9 @@
  * reference function it stands in for is cited on each declaration.  The reference's ops
  * are `runX(...)` / `recordX(recorder, ...)` pairs that enqueue on one GPUQueue; here
  * every op enqueues on one HIP stream (the library's own, which orders itself against
- * the legacy default stream, or the one given to dh_set_stream) and returns at once.  Ops never allocate: outputs are caller-provided
- * device pointers, as when the reference's callers pass `outputBuffer`.
+ * the legacy default stream, or the one given to dh_set_stream) and returns at once.
+ * Ops never allocate: outputs are caller-provided device pointers, as when the
+ * reference's callers pass `outputBuffer`.
  *
  * Conventions
  *   - all pointers named d_* are device pointers (from dh_malloc or any hipMalloc);
