@@ -44,7 +44,9 @@ SIGNATURES = {
     "dh_event_destroy": (_I, [_P]),
     "dh_q4k_dequant": (_I, [_P, _I64, _P]),
     "dh_q4k_matmul": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
+    "dh_q4k_matmul_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
     "dh_q4k_ffn_gate_up": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
+    "dh_q4k_ffn_gate_up_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
     "dh_f16w_matmul": (_I, [_P, _P, _P, _I, _I, _I, _F]),
     "dh_lmhead_argmax_workspace_bytes": (_SZ, [_I]),
     "dh_lmhead_argmax_f16": (_I, [_P, _P, _I, _I, _I64, _F, _P, _P, _I, _P]),

@@ -340,8 +340,6 @@ int env_int(const char* name, int dflt) {
   return e ? atoi(e) : dflt;
 }
 
-constexpr int kRingThreads = 512;
-constexpr int kRingWaves = kRingThreads / 64;
 constexpr int kMaxDepth = 4;
 
 #ifdef DH_GEMV_TRACE
@@ -360,6 +358,10 @@ struct RingArgs {
   float alpha;
   int c_f16, activation;
   float clamp_max;
+  // RMSNorm prologue: A is normalised per row before the product (norm_weight null = off)
+  const float* norm_weight;   // [K]
+  float norm_eps;
+  int norm_weight_offset;     // 1: scale by (1 + w)
 };
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -391,67 +393,84 @@ __device__ __forceinline__ void wait_vm_at_most(int n) {
 // load in flight (the direct-to-LDS loads count as LDS writers) and drain the ring.
 #define DH_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
-// The 32 activations of work item idx = sub-block * MT + row; zeros past K or M.
+// Activation staging.  Work item = (sub-block sb, activation row m) = 32 floats, shared by four
+// consecutive lanes: lane grp = idx & 3 of the quad owns elements [8*grp, 8*grp+8), i.e. one
+// k-group of the matrix-core fragment.  Zeros past K or M.
 template <int MT>
-__device__ __forceinline__ void stage_x_load(const float* __restrict__ A, int M, int K, int idx, float (&v)[32]) {
-  const int sb = idx / MT, m = idx - sb * MT;
-  const int left = K - sb * 32;
-  if (m < M && left >= 32) {
-    const float4* src = reinterpret_cast<const float4*>(A + (int64_t)m * K + sb * 32);
-    if ((reinterpret_cast<uintptr_t>(src) & 15) == 0) {
-#pragma unroll
-      for (int q4 = 0; q4 < 8; q4++) {
-        const float4 t = src[q4];
-        v[4 * q4] = t.x; v[4 * q4 + 1] = t.y; v[4 * q4 + 2] = t.z; v[4 * q4 + 3] = t.w;
-      }
-    } else {
-      const float* s1 = reinterpret_cast<const float*>(src);
-#pragma unroll
-      for (int j = 0; j < 32; j++) v[j] = s1[j];
-    }
+__device__ __forceinline__ void stage_x_load(const float* __restrict__ A, int M, int K, int idx, float (&v)[8]) {
+  const int item = idx >> 2, grp = idx & 3;
+  const int sb = item / MT, m = item - sb * MT;
+  const int k0 = sb * 32 + grp * 8, left = K - k0;
+  const float* src = A + (int64_t)m * K + k0;
+  if (m < M && left >= 8 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+    const float4 t0 = reinterpret_cast<const float4*>(src)[0], t1 = reinterpret_cast<const float4*>(src)[1];
+    v[0] = t0.x; v[1] = t0.y; v[2] = t0.z; v[3] = t0.w;
+    v[4] = t1.x; v[5] = t1.y; v[6] = t1.z; v[7] = t1.w;
   } else if (m < M && left > 0) {
-    const float* s1 = A + (int64_t)m * K + sb * 32;
 #pragma unroll
-    for (int j = 0; j < 32; j++) {
-      const float t = s1[min(j, left - 1)];
+    for (int j = 0; j < 8; j++) {
+      const float t = src[min(j, left - 1)];
       v[j] = j < left ? t : 0.f;
     }
   } else {
 #pragma unroll
-    for (int j = 0; j < 32; j++) v[j] = 0.f;
+    for (int j = 0; j < 8; j++) v[j] = 0.f;
   }
 }
 
-// Converts one work item to matrix-core fragments.  Each sub-block gets its own power-of-two
-// scale (largest element just inside f16 range): f16 high part, f16 residual, the plain sum
-// (min term) and 2^24 / scale per (sb, m).
+// RMSNorm weights for the eight k of quarter item idx (1 + w when `offset`); 0 past K.
 template <int MT>
-__device__ __forceinline__ void stage_x_store(int idx, const float (&v)[32], _Float16* xf, float2* sxi) {
+__device__ __forceinline__ void stage_norm_weight_load(const float* __restrict__ w, int K, int offset, int idx,
+                                                       float (&wn)[8]) {
+  const int item = idx >> 2, grp = idx & 3;
+  const int k0 = (item / MT) * 32 + grp * 8, left = K - k0;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const float t = left > 0 ? w[k0 + min(j, left - 1)] : 0.f;
+    wn[j] = j < left ? (offset ? 1.0f + t : t) : 0.f;
+  }
+}
+
+// Sum / max across the four lanes of a quad (DPP quad_perm, no LDS traffic).
+__device__ __forceinline__ float quad_xor_f32(float x, int pattern /* 1 or 2 */) {
+  const int b = __float_as_int(x);
+  const int r = pattern == 1 ? __builtin_amdgcn_update_dpp(b, b, 0xB1, 0xF, 0xF, false)    // [1,0,3,2]
+                             : __builtin_amdgcn_update_dpp(b, b, 0x4E, 0xF, 0xF, false);   // [2,3,0,1]
+  return __int_as_float(r);
+}
+
+// Converts one quarter work item to matrix-core fragments.  Each sub-block gets its own
+// power-of-two scale (largest element just inside f16 range): f16 high part, f16 residual,
+// the plain sum (min term) and 2^24 / scale per (sb, m).  All four lanes of the quad must call.
+template <int MT>
+__device__ __forceinline__ void stage_x_store(int idx, const float (&v)[8], _Float16* xf, float2* sxi) {
   constexpr int XC = 2 * MT;
-  const int sb = idx / MT, m = idx - sb * MT;
+  const int item = idx >> 2, grp = idx & 3;
+  const int sb = item / MT, m = item - sb * MT;
   float s = 0.f, mx = 0.f;
 #pragma unroll
-  for (int j = 0; j < 32; j++) { s += v[j]; mx = fmaxf(mx, fabsf(v[j])); }
+  for (int j = 0; j < 8; j++) { s += v[j]; mx = fmaxf(mx, fabsf(v[j])); }
+  s += quad_xor_f32(s, 1);
+  mx = fmaxf(mx, quad_xor_f32(mx, 1));
+  s += quad_xor_f32(s, 2);
+  mx = fmaxf(mx, quad_xor_f32(mx, 2));
   int e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
   e = max(-100, min(100, e));
   if (mx == 0.f) e = 14;
   const float sf = __uint_as_float((uint32_t)(127 + 14 - e) << 23);          // 2^(14-e)
-  sxi[idx] = make_float2(s, __uint_as_float((uint32_t)(127 + 24 - 14 + e) << 23));   // 2^24 / sf
+  if (grp == 0) sxi[item] = make_float2(s, __uint_as_float((uint32_t)(127 + 24 - 14 + e) << 23));   // 2^24 / sf
+  half8_t hi, lo;
 #pragma unroll
-  for (int grp = 0; grp < 4; grp++) {
-    half8_t hi, lo;
-#pragma unroll
-    for (int slot = 0; slot < 8; slot++) {
-      // slot order inside a k-group follows the masked dwords: (b0,b2) (b1,b3) (b4,b6) (b5,b7)
-      const int o = (slot & 4) | ((slot & 1) << 1) | ((slot >> 1) & 1);
-      const float xsc = v[grp * 8 + o] * sf;
-      const _Float16 h = (_Float16)xsc;
-      hi[slot] = h;
-      lo[slot] = (_Float16)(xsc - (float)h);
-    }
-    *reinterpret_cast<half8_t*>(xf + (sb * XC + 2 * m) * 32 + grp * 8) = hi;
-    *reinterpret_cast<half8_t*>(xf + (sb * XC + 2 * m + 1) * 32 + grp * 8) = lo;
+  for (int slot = 0; slot < 8; slot++) {
+    // slot order inside a k-group follows the masked dwords: (b0,b2) (b1,b3) (b4,b6) (b5,b7)
+    const int o = (slot & 4) | ((slot & 1) << 1) | ((slot >> 1) & 1);
+    const float xsc = v[o] * sf;
+    const _Float16 h = (_Float16)xsc;
+    hi[slot] = h;
+    lo[slot] = (_Float16)(xsc - (float)h);
   }
+  *reinterpret_cast<half8_t*>(xf + (sb * XC + 2 * m) * 32 + grp * 8) = hi;
+  *reinterpret_cast<half8_t*>(xf + (sb * XC + 2 * m + 1) * 32 + grp * 8) = lo;
 }
 
 // Where a wave is in its list of work units (tile, matrix, super-block).
@@ -462,9 +481,9 @@ struct UnitCursor {
 // GEMV on the matrix cores with the weights streamed HBM -> LDS by the load unit itself
 // (global_load_lds_dwordx4: no vector registers, no vector-ALU work on the way).
 //
-// A workgroup of 8 waves owns tiles of R <= 32 consecutive weight rows (R chosen by the host
+// A workgroup of WAVES (8 or 16) waves owns tiles of R <= 32 consecutive weight rows (R chosen by the host
 // so that the tile count is a multiple of the number of compute units).  Inside a tile, wave
-// w takes super-blocks w, w+8, ...: one work unit = R rows x 1 super-block = R*144 bytes,
+// w takes super-blocks w, w+WAVES, ...: one work unit = R rows x 1 super-block = R*144 bytes,
 // fetched by up to five 16-byte-per-lane load instructions (9 lanes per row) into one stage of
 // the wave's private ring in LDS, rows 144 bytes apart exactly as in memory.  Each wave keeps
 // `depth` units in flight and synchronises with nobody while it streams: it waits on its own
@@ -473,12 +492,13 @@ struct UnitCursor {
 // their K slices.  The activation fragments live in a separate, statically declared LDS
 // array: the compiler then knows that reading them cannot touch the bytes the load unit is
 // writing and does not wait for the loads in flight.
-template <int MT, bool DUAL, int XBYTES>
-__global__ __launch_bounds__(kRingThreads, 2) void q4k_gemv_ring_kernel(const RingArgs a) {
-  constexpr int NTHR = kRingThreads, WAVES = kRingWaves;
+template <int MT, bool DUAL, int XBYTES, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(const RingArgs a) {
+  constexpr int NTHR = 64 * WAVES;
   constexpr int XC = 2 * MT, NO = MfmaShape<MT>::NI / 2, NMAT = DUAL ? 2 : 1;
   __shared__ __align__(16) unsigned char xs[XBYTES];        // x fragments | zero row | (sum, 1/scale)
   __shared__ float red[2][WAVES][NMAT][NO][64];
+  __shared__ float norm_ss[WAVES][MT];
   extern __shared__ __align__(16) unsigned char ring[];     // [WAVES][depth][R*144]
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -550,19 +570,66 @@ __global__ __launch_bounds__(kRingThreads, 2) void q4k_gemv_ring_kernel(const Ri
   // The first item's loads go out before the ring loads (loads complete in order), its
   // conversion runs while the ring fills.
   {
-    bool first = true;
-#pragma unroll 1
-    for (int idx = tid; first || idx < MT * nsub; idx += NTHR) {
-      float v[32];
-      if (idx < MT * nsub) stage_x_load<MT>(a.A, a.M, a.K, idx, v);
-      if (first) {
-        // the activations are in registers before the ring starts: nothing the compiler
-        // waits for later can then sit behind (and so wait for) a ring load
-        DH_WAIT_VM(0);
-        for (int d = 0; d < D; d++) DH_ISSUE_NEXT();
-        first = false;
+    // Everything this thread needs from memory for its first quarter item is loaded before the
+    // ring starts: loads complete in order, so a wait for a later load would also wait for the
+    // ring loads in front of it.
+    const int total = 4 * MT * nsub;
+    const bool norm = a.norm_weight != nullptr;
+    float v0[8], wn0[8];
+    if (tid < total) stage_x_load<MT>(a.A, a.M, a.K, tid, v0);
+    float ss = 0.f;
+    if (norm) {
+      if (tid < total) {
+        stage_norm_weight_load<MT>(a.norm_weight, a.K, a.norm_weight_offset, tid, wn0);
+#pragma unroll
+        for (int j = 0; j < 8; j++) ss = fmaf(v0[j], v0[j], ss);
       }
-      if (idx < MT * nsub) stage_x_store<MT>(idx, v, xf, sxi);
+#pragma unroll 1
+      for (int idx = tid + NTHR; idx < total; idx += NTHR) {   // rows longer than one pass
+        float t[8];
+        stage_x_load<MT>(a.A, a.M, a.K, idx, t);
+#pragma unroll
+        for (int j = 0; j < 8; j++) ss = fmaf(t[j], t[j], ss);
+      }
+    }
+    DH_TS();
+    DH_WAIT_VM(0);
+    DH_TS();
+    for (int d = 0; d < D; d++) DH_ISSUE_NEXT();
+    DH_TS();
+    float inv = 1.f;
+    if (norm) {
+      // sum of squares of activation row m = (tid >> 2) % MT: lanes of a quad share a row,
+      // lane bit 2 selects the row when MT == 2
+      ss += quad_xor_f32(ss, 1);
+      ss += quad_xor_f32(ss, 2);
+      if (MT == 1) ss += __shfl_xor(ss, 4);
+      ss += __shfl_xor(ss, 8);
+      ss += __shfl_xor(ss, 16);
+      ss += __shfl_xor(ss, 32);
+      const int my_m = (tid >> 2) % MT;
+      if ((lane & ~4) == 0 && (lane >> 2) < MT) norm_ss[wave][lane >> 2] = ss;
+      DH_LDS_BARRIER();
+      float tot = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; w++) tot += norm_ss[w][my_m];
+      inv = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
+    }
+#pragma unroll 1
+    for (int idx = tid; idx < total; idx += NTHR) {
+      float t[8], wn[8];
+      if (idx == tid) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) { t[j] = v0[j]; wn[j] = wn0[j]; }
+      } else {
+        stage_x_load<MT>(a.A, a.M, a.K, idx, t);
+        if (norm) stage_norm_weight_load<MT>(a.norm_weight, a.K, a.norm_weight_offset, idx, wn);
+      }
+      if (norm) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) t[j] = t[j] * inv * wn[j];
+      }
+      stage_x_store<MT>(idx, t, xf, sxi);
     }
   }
   if (tid < 16) reinterpret_cast<uint32_t*>(xzero)[tid] = 0u;
@@ -662,11 +729,11 @@ constexpr size_t kRingMaxLds = 160 * 1024;
 
 size_t ring_x_bytes(int mt, int nb) { return (size_t)nb * 8 * mt * (2 * 32 * 2 + 8) + 64; }
 
-template <int MT, bool DUAL, int XBYTES>
+template <int MT, bool DUAL, int XBYTES, int WAVES>
 int launch_ring_cfg(RingArgs a, const char* op) {
   constexpr int NO = MfmaShape<MT>::NI / 2, NMAT = DUAL ? 2 : 1;
-  const size_t fixed = XBYTES + sizeof(float) * 2 * kRingWaves * NMAT * NO * 64 + 256;
-  auto kern = q4k_gemv_ring_kernel<MT, DUAL, XBYTES>;
+  const size_t fixed = XBYTES + sizeof(float) * 2 * WAVES * NMAT * NO * 64 + 256;
+  auto kern = q4k_gemv_ring_kernel<MT, DUAL, XBYTES, WAVES>;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
     DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -682,15 +749,15 @@ int launch_ring_cfg(RingArgs a, const char* op) {
   rows = std::max(4, std::min(32, rows));
   if (env_rows > 0) rows = std::min(32, env_rows);
   int depth = kMaxDepth;
-  while (depth > 2 && fixed + (size_t)kRingWaves * depth * rows * kBlockBytes > kRingMaxLds) depth--;
+  while (depth > 2 && fixed + (size_t)WAVES * depth * rows * kBlockBytes > kRingMaxLds) depth--;
   if (env_depth > 0) depth = std::max(2, std::min(kMaxDepth, env_depth));
-  const size_t dyn = (size_t)kRingWaves * depth * rows * kBlockBytes;
+  const size_t dyn = (size_t)WAVES * depth * rows * kBlockBytes;
   if (fixed + dyn > kRingMaxLds) return -1;
   a.rows_per_tile = rows;
   a.depth = depth;
   const int64_t ntiles = dh::ceil_div(a.N, rows);
   const int grid = (int)std::min<int64_t>(ntiles, ncu);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kRingThreads), dyn, dh::stream(), a);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), dyn, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   return 0;
 }
@@ -699,9 +766,18 @@ int launch_ring_cfg(RingArgs a, const char* op) {
 template <int MT, bool DUAL>
 int launch_ring(const RingArgs& a, const char* op) {
   const size_t xb = ring_x_bytes(MT, a.nb);
-  if (xb <= 20 * 1024) return launch_ring_cfg<MT, DUAL, 20 * 1024>(a, op);
-  if (xb <= 40 * 1024) return launch_ring_cfg<MT, DUAL, 40 * 1024>(a, op);
-  if (xb <= 56 * 1024) return launch_ring_cfg<MT, DUAL, 56 * 1024>(a, op);
+  static const int env_waves = env_int("DH_GEMV_WAVES", 16);
+  // 16 waves per workgroup hide more latency; their rings need twice the LDS
+  if (env_waves == 16) {
+    int rc = -1;
+    if (xb <= 20 * 1024) rc = launch_ring_cfg<MT, DUAL, 20 * 1024, 16>(a, op);
+    else if (xb <= 40 * 1024) rc = launch_ring_cfg<MT, DUAL, 40 * 1024, 16>(a, op);
+    else if (xb <= 56 * 1024) rc = launch_ring_cfg<MT, DUAL, 56 * 1024, 16>(a, op);
+    if (rc >= 0) return rc;
+  }
+  if (xb <= 20 * 1024) return launch_ring_cfg<MT, DUAL, 20 * 1024, 8>(a, op);
+  if (xb <= 40 * 1024) return launch_ring_cfg<MT, DUAL, 40 * 1024, 8>(a, op);
+  if (xb <= 56 * 1024) return launch_ring_cfg<MT, DUAL, 56 * 1024, 8>(a, op);
   return -1;
 }
 
@@ -818,9 +894,10 @@ int dh_q4k_dequant(const void* d_W, int64_t num_blocks, float* d_out) {
   return 0;
 }
 
-int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int c_dtype, int M,
-                  int N, int K, float alpha, const void* d_residual) {
-  const char* op = "dh_q4k_matmul";
+// Shared body of dh_q4k_matmul and dh_q4k_matmul_rmsnorm.
+static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const float* d_norm_weight,
+                           float eps, int weight_offset, bool normed, const void* d_W, void* d_C,
+                           int c_dtype, int M, int N, int K, float alpha, const void* d_residual) {
   DH_REQUIRE_INIT(op);
   if (M <= 0 || N <= 0 || K <= 0)
     return dh::fail(1, "[%s] Dimensions must be positive: M=%d, N=%d, K=%d", op, M, N, K);
@@ -830,6 +907,7 @@ int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int 
     return dh::fail(1, "[%s] output dtype must be f32 or f16 (c_dtype=%d)", op, c_dtype);
   if (reinterpret_cast<uintptr_t>(d_W) & 15)
     return dh::fail(1, "[%s] weight pointer must be 16-byte aligned", op);
+  if (normed && !d_norm_weight) return dh::fail(1, "[%s] norm weight pointer is null", op);
   GemvArgs a{};
   a.A = static_cast<const float*>(d_A);
   a.W = static_cast<const uint8_t*>(d_W);
@@ -841,13 +919,18 @@ int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int 
   a.alpha = alpha;
   a.c_f16 = c_dtype == DH_F16;
   const int path = gemv_path();
-  if (path == 0 && M <= 8) {
+  if ((path == 0 || normed) && M <= 8) {
     RingArgs g{};
     g.A = a.A; g.W = a.W; g.W2 = nullptr; g.C = d_C; g.residual = a.residual;
     g.M = M; g.N = N; g.K = K; g.nb = a.nb; g.alpha = alpha; g.c_f16 = a.c_f16;
+    g.norm_weight = normed ? d_norm_weight : nullptr;
+    g.norm_eps = eps; g.norm_weight_offset = weight_offset;
     const int rc = dispatch_ring<false>(g, op);
     if (rc >= 0) return rc;
   }
+  if (normed)
+    return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 and K <= 14336 only (M=%d, K=%d); "
+                    "run dh_rmsnorm and dh_q4k_matmul instead", op, M, K);
   // tiles of up to 8 activation rows per pass over the weights
   const size_t c_elem = a.c_f16 ? 2 : 4;
   for (int m0 = 0; m0 < M; m0 += 8) {
@@ -862,9 +945,24 @@ int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int 
   return 0;
 }
 
-int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup, float* d_out, int M,
-                       int hidden, int inter, int activation, float alpha, float swiglu_limit) {
-  const char* op = "dh_q4k_ffn_gate_up";
+int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int c_dtype, int M,
+                  int N, int K, float alpha, const void* d_residual) {
+  return q4k_matmul_impl("dh_q4k_matmul", d_A, a_dtype, nullptr, 0.f, 0, false, d_W, d_C, c_dtype, M, N, K,
+                         alpha, d_residual);
+}
+
+int dh_q4k_matmul_rmsnorm(const float* d_A, const float* d_norm_weight, float eps, int weight_offset,
+                          const void* d_W, void* d_C, int c_dtype, int M, int N, int K, float alpha,
+                          const void* d_residual) {
+  return q4k_matmul_impl("dh_q4k_matmul_rmsnorm", d_A, DH_F32, d_norm_weight, eps, weight_offset, true, d_W,
+                         d_C, c_dtype, M, N, K, alpha, d_residual);
+}
+
+// Shared body of dh_q4k_ffn_gate_up and dh_q4k_ffn_gate_up_rmsnorm.
+static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_weight, float eps,
+                        int weight_offset, bool normed, const void* d_Wgate, const void* d_Wup,
+                        float* d_out, int M, int hidden, int inter, int activation, float alpha,
+                        float swiglu_limit) {
   DH_REQUIRE_INIT(op);
   if (M <= 0 || hidden <= 0 || inter <= 0)
     return dh::fail(1, "[%s] Dimensions must be positive: M=%d, hidden=%d, inter=%d", op, M, hidden, inter);
@@ -873,6 +971,7 @@ int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup,
     return dh::fail(1, "[%s] unknown activation %d", op, activation);
   if ((reinterpret_cast<uintptr_t>(d_Wgate) | reinterpret_cast<uintptr_t>(d_Wup)) & 15)
     return dh::fail(1, "[%s] weight pointers must be 16-byte aligned", op);
+  if (normed && !d_norm_weight) return dh::fail(1, "[%s] norm weight pointer is null", op);
   GemvArgs a{};
   a.A = d_x;
   a.W = static_cast<const uint8_t*>(d_Wgate);
@@ -886,14 +985,19 @@ int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup,
   a.activation = activation;
   a.clamp_max = swiglu_limit;
   const int path = gemv_path();
-  if (path == 0 && M <= 8) {
+  if ((path == 0 || normed) && M <= 8) {
     RingArgs g{};
     g.A = d_x; g.W = a.W; g.W2 = a.W2; g.C = d_out; g.residual = nullptr;
     g.M = M; g.N = inter; g.K = hidden; g.nb = a.nb; g.alpha = alpha; g.c_f16 = 0;
     g.activation = activation; g.clamp_max = swiglu_limit;
+    g.norm_weight = normed ? d_norm_weight : nullptr;
+    g.norm_eps = eps; g.norm_weight_offset = weight_offset;
     const int rc = dispatch_ring<true>(g, op);
     if (rc >= 0) return rc;
   }
+  if (normed)
+    return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 and hidden <= 14336 only (M=%d, hidden=%d); "
+                    "run dh_rmsnorm and dh_q4k_ffn_gate_up instead", op, M, hidden);
   // any batch: tiles of up to 8 activation rows per pass
   for (int m0 = 0; m0 < M; m0 += 8) {
     GemvArgs b = a;
@@ -904,6 +1008,19 @@ int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup,
     if (rc) return rc;
   }
   return 0;
+}
+
+int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup, float* d_out, int M,
+                       int hidden, int inter, int activation, float alpha, float swiglu_limit) {
+  return q4k_ffn_impl("dh_q4k_ffn_gate_up", d_x, nullptr, 0.f, 0, false, d_Wgate, d_Wup, d_out, M, hidden,
+                      inter, activation, alpha, swiglu_limit);
+}
+
+int dh_q4k_ffn_gate_up_rmsnorm(const float* d_x, const float* d_norm_weight, float eps, int weight_offset,
+                               const void* d_Wgate, const void* d_Wup, float* d_out, int M, int hidden,
+                               int inter, int activation, float alpha, float swiglu_limit) {
+  return q4k_ffn_impl("dh_q4k_ffn_gate_up_rmsnorm", d_x, d_norm_weight, eps, weight_offset, true, d_Wgate,
+                      d_Wup, d_out, M, hidden, inter, activation, alpha, swiglu_limit);
 }
 
 }  // extern "C"

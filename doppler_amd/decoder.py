@@ -31,11 +31,13 @@ def _dev_bytes(arr):
 
 
 class HipDecoder:
-    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq):
+    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True):
         """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
         layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
         input_norm, post_attn_norm, q_norm, k_norm: f32); embed_bits: uint16 [vocab, hidden]."""
         self.cfg = dict(cfg)
+        # RMSNorm runs inside the q/k/v and gate/up GEMVs (their prologue) unless told otherwise
+        self.fuse_norm = fuse_norm
         self.L = capi.init(torch.cuda.current_device())
         c = self.cfg
         self.max_seq = max_seq
@@ -98,10 +100,15 @@ class HipDecoder:
         ck(L.dh_gather_f16(ids.data_ptr(), self.embed.data_ptr(), self.x.data_ptr(), 1, Hd, c["vocab"], 0))
         x, x2 = self.x, self.x2
         for d in self.layers:
-            ck(L.dh_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd,
-                            c["eps"], 0, None, None, None, 1.0))
-            ck(L.dh_q4k_matmul(self.normed.data_ptr(), capi.F32, d["wqkv"].data_ptr(), self.qkv.data_ptr(), capi.F32,
-                               1, self.qs + 2 * self.ks, Hd, 1.0, None))
+            if self.fuse_norm:
+                ck(L.dh_q4k_matmul_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), c["eps"], 0,
+                                           d["wqkv"].data_ptr(), self.qkv.data_ptr(), capi.F32, 1,
+                                           self.qs + 2 * self.ks, Hd, 1.0, None))
+            else:
+                ck(L.dh_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd,
+                                c["eps"], 0, None, None, None, 1.0))
+                ck(L.dh_q4k_matmul(self.normed.data_ptr(), capi.F32, d["wqkv"].data_ptr(), self.qkv.data_ptr(),
+                                   capi.F32, 1, self.qs + 2 * self.ks, Hd, 1.0, None))
             ck(L.dh_qkv_norm_rope_kvwrite(self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
                                           self.cos.data_ptr(), self.sin.data_ptr(), self.q.data_ptr(),
                                           d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), 1, H, Hkv, D, pos, D, 0,
@@ -111,10 +118,15 @@ class HipDecoder:
                                 capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
             ck(L.dh_q4k_matmul(self.attn.data_ptr(), capi.F32, d["wo"].data_ptr(), x2.data_ptr(), capi.F32, 1, Hd,
                                self.qs, 1.0, x.data_ptr()))
-            ck(L.dh_rmsnorm(x2.data_ptr(), d["post_attn_norm"].data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd,
-                            c["eps"], 0, None, None, None, 1.0))
-            ck(L.dh_q4k_ffn_gate_up(self.normed.data_ptr(), d["wgate"].data_ptr(), d["wup"].data_ptr(),
-                                    self.act.data_ptr(), 1, Hd, I, capi.ACT_SILU, 1.0, 0.0))
+            if self.fuse_norm:
+                ck(L.dh_q4k_ffn_gate_up_rmsnorm(x2.data_ptr(), d["post_attn_norm"].data_ptr(), c["eps"], 0,
+                                                d["wgate"].data_ptr(), d["wup"].data_ptr(), self.act.data_ptr(),
+                                                1, Hd, I, capi.ACT_SILU, 1.0, 0.0))
+            else:
+                ck(L.dh_rmsnorm(x2.data_ptr(), d["post_attn_norm"].data_ptr(), capi.F32, self.normed.data_ptr(), 1,
+                                Hd, c["eps"], 0, None, None, None, 1.0))
+                ck(L.dh_q4k_ffn_gate_up(self.normed.data_ptr(), d["wgate"].data_ptr(), d["wup"].data_ptr(),
+                                        self.act.data_ptr(), 1, Hd, I, capi.ACT_SILU, 1.0, 0.0))
             ck(L.dh_q4k_matmul(self.act.data_ptr(), capi.F32, d["wdown"].data_ptr(), x.data_ptr(), capi.F32, 1, Hd, I,
                                1.0, x2.data_ptr()))
         ck(L.dh_rmsnorm(x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"],

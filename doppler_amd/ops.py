@@ -138,9 +138,12 @@ def _act_code(activation, op):
 # ------------------------------------------------------------------ matmul
 
 def runMatmul(A, B, M, N, K, alpha=1.0, outputBuffer=None, transposeB=True, outputDtype=None, role=None,
-              layerIdx=None, residualTensor=None, **_ignored):
+              layerIdx=None, residualTensor=None, normWeight=None, rmsNormEps=None, rmsNormOffset=False,
+              useFusedRmsnormWideTile=False, **_ignored):
     """src/gpu/kernels/matmul.js:659 runMatmul(A, B, M, N, K, options) for q4k ('row') and f16
-    weights ([N, K] row-major, transposeB true)."""
+    weights ([N, K] row-major, transposeB true).  With `normWeight` and
+    `useFusedRmsnormWideTile` the RMSNorm of A runs inside the matmul
+    (src/gpu/kernels/matmul-selection.js:609-620)."""
     op = "runMatmul"
     for v in (M, N, K):
         if not isinstance(v, (int, np.integer)):
@@ -163,9 +166,18 @@ def runMatmul(A, B, M, N, K, alpha=1.0, outputBuffer=None, transposeB=True, outp
             raise DopplerHipError("[%s] B buffer too small: %d < %d (N=%d, K=%d, bDtype=q4k, transposeB=%s)"
                                   % (op, _nbytes(B), need, N, K, transposeB))
         out = _out(outputBuffer, M * N * (2 if outputDtype == "f16" else 4))
-        capi.check(L.dh_q4k_matmul(_ptr(A), capi.F32, _ptr(B), out.data_ptr(),
-                                   capi.F16 if outputDtype == "f16" else capi.F32, M, N, K, alpha,
-                                   _ptr(residualTensor)))
+        cdt = capi.F16 if outputDtype == "f16" else capi.F32
+        if normWeight is not None and useFusedRmsnormWideTile:
+            if rmsNormEps is None:
+                raise DopplerHipError("[%s] rmsNormEps is required with normWeight" % op)
+            if getattr(normWeight, "dtype", "f32") != "f32":
+                raise DopplerHipError("[%s] fused RMSNorm requires an f32 norm weight" % op)
+            capi.check(L.dh_q4k_matmul_rmsnorm(_ptr(A), _ptr(normWeight), float(rmsNormEps),
+                                               1 if rmsNormOffset else 0, _ptr(B), out.data_ptr(), cdt,
+                                               M, N, K, alpha, _ptr(residualTensor)))
+        else:
+            capi.check(L.dh_q4k_matmul(_ptr(A), capi.F32, _ptr(B), out.data_ptr(), cdt, M, N, K, alpha,
+                                       _ptr(residualTensor)))
         return Tensor(out, outputDtype, (M, N), "matmul_output")
     if bdtype == "f16":
         if transposeB not in (True, "auto"):
@@ -208,6 +220,28 @@ def runFusedFFN(input, W_gate, W_up, hiddenSize, intermediateSize, batchSize=1, 
                                          hiddenSize, intermediateSize, _act_code(activation, "FusedFFN"),
                                          alpha, float(swigluLimit or 0.0) if activation == "silu" else 0.0))
     return Tensor(out, "f32", (batchSize, intermediateSize), "fused_ffn_output")
+
+
+def runFusedNormedFFN(input, normWeight, eps, W_gate, W_up, hiddenSize, intermediateSize, batchSize=1,
+                      activation="silu", alpha=1.0, outputBuffer=None, swigluLimit=None,
+                      rmsNormWeightOffset=False, **_ignored):
+    """Gate/up projection + gated activation over RMSNorm(input) in one launch.  Stands in for
+    src/gpu/kernels/fused_ffn.js:770 runFusedFFNFromRMSNormStats; the inverse RMS that the
+    reference takes as a buffer from its rmsnorm-stats pass is computed in the kernel prologue."""
+    gd = W_gate.dtype if isinstance(W_gate, (Tensor, WeightBuffer)) else None
+    ud = W_up.dtype if isinstance(W_up, (Tensor, WeightBuffer)) else None
+    if gd != "q4k" or ud != "q4k":
+        raise DopplerHipError("Fused normed FFN requires Q4_K gate/up weights; got gate=%s, up=%s." % (gd, ud))
+    if input.dtype != "f32":
+        raise DopplerHipError("Fused normed FFN requires f32 prenorm input; got %s." % input.dtype)
+    if normWeight is None:
+        raise DopplerHipError("Fused normed FFN requires a norm weight buffer.")
+    out = _out(outputBuffer, batchSize * intermediateSize * 4)
+    capi.check(_lib().dh_q4k_ffn_gate_up_rmsnorm(
+        _ptr(input), _ptr(normWeight), float(eps), 1 if rmsNormWeightOffset else 0, _ptr(W_gate), _ptr(W_up),
+        out.data_ptr(), batchSize, hiddenSize, intermediateSize, _act_code(activation, "FusedNormedFFN"), alpha,
+        float(swigluLimit or 0.0) if activation == "silu" else 0.0))
+    return Tensor(out, "f32", (batchSize, intermediateSize), "fused_normed_ffn_output")
 
 
 # ------------------------------------------------------------------ attention

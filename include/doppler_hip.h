@@ -82,6 +82,17 @@ int dh_q4k_dequant(const void* d_W, int64_t num_blocks, float* d_out);
 int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int c_dtype,
                   int M, int N, int K, float alpha, const void* d_residual);
 
+/* dh_q4k_matmul with an RMSNorm prologue: A is replaced by
+ * A * rsqrt(mean(A^2 over K) + eps) * (w | 1 + w) row by row before the product, so the
+ * standalone norm dispatch in front of the q/k/v and gate/up projections disappears.
+ * Replaces runMatmul with `normWeight` + `useFusedRmsnormWideTile`,
+ * src/gpu/kernels/matmul-selection.js:609-620 (fused_rmsnorm_q4_widetile.wgsl:4-24,189-215).
+ * d_norm_weight is f32 [K].  Served for M <= 8; other shapes fail with a message (run
+ * dh_rmsnorm + dh_q4k_matmul). */
+int dh_q4k_matmul_rmsnorm(const float* d_A, const float* d_norm_weight, float eps,
+                          int weight_offset, const void* d_W, void* d_C, int c_dtype, int M,
+                          int N, int K, float alpha, const void* d_residual);
+
 /* out[M,inter] = clamp(act(x.Wgate^T) * (x.Wup^T) * alpha).
  * Replaces runFusedFFN/recordFusedFFN, src/gpu/kernels/fused_ffn.js:501,605
  * (fused_ffn_q4k.wgsl:129-363).  clamp (swigluLimit) applies to DH_ACT_SILU only;
@@ -89,6 +100,14 @@ int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int 
 int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup, float* d_out,
                        int M, int hidden, int inter, int activation, float alpha,
                        float swiglu_limit);
+
+/* dh_q4k_ffn_gate_up over RMSNorm(x): the reference's "fused normed FFN",
+ * src/gpu/kernels/fused_ffn.js:705-745,773-860 (there the inverse RMS comes in as a buffer,
+ * here it is computed in the prologue).  d_norm_weight is f32 [hidden].  M <= 8. */
+int dh_q4k_ffn_gate_up_rmsnorm(const float* d_x, const float* d_norm_weight, float eps,
+                               int weight_offset, const void* d_Wgate, const void* d_Wup,
+                               float* d_out, int M, int hidden, int inter, int activation,
+                               float alpha, float swiglu_limit);
 
 /* ---- dense f16-weight GEMV (LM head) ----
  * C[M,N] = alpha * A[M,K] . f32(W[N,K])^T, W row-major f16.  Replaces the f16-weight branch

@@ -163,6 +163,46 @@ def test_fused_ffn_q4k(M, activation, limit):
     assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
 
 
+@pytest.mark.parametrize("M,N,K,offset", [(1, 6144, 4096, False), (2, 1024, 1024, True), (1, 2048, 640, False),
+                                          (3, 96, 1152, False), (1, 4096, 12288, False), (5, 130, 2048, True)])
+def test_matmul_with_rmsnorm_prologue(M, N, K, offset):
+    """runMatmul with normWeight + useFusedRmsnormWideTile == runRMSNorm followed by runMatmul
+    (reference: src/gpu/kernels/matmul-selection.js:609-620)."""
+    W, wb = q4k_weight(N, K, seed=2100 + M)
+    A = synth.normal_f32((M, K), seed=2101 + N, scale=3.0)
+    nw = (0.0 if offset else 1.0) + synth.normal_f32((K,), seed=2102, scale=0.1)
+    res = synth.normal_f32((M, N), seed=2103)
+    out = ops.runMatmul(ops.tensorFromNumpy(A), wb, M, N, K, alpha=0.75, outputDtype="f32",
+                        residualTensor=ops.tensorFromNumpy(res), normWeight=ops.tensorFromNumpy(nw),
+                        rmsNormEps=1e-6, rmsNormOffset=offset, useFusedRmsnormWideTile=True)
+    normed = oracle.rmsnorm(A, nw, 1e-6, weight_offset=offset)
+    want = oracle.q4k_matmul(normed, W, M, N, K, 0.75) + res
+    assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
+
+
+@pytest.mark.parametrize("M,activation", [(1, "silu"), (2, "gelu")])
+def test_fused_normed_ffn_q4k(M, activation):
+    hidden, inter = 1536, 6144
+    Wg, wg = q4k_weight(inter, hidden, seed=2200)
+    Wu, wu = q4k_weight(inter, hidden, seed=2201)
+    X = synth.normal_f32((M, hidden), seed=2202, scale=5.0)
+    nw = 1.0 + synth.normal_f32((hidden,), seed=2203, scale=0.1)
+    out = ops.runFusedNormedFFN(ops.tensorFromNumpy(X), ops.tensorFromNumpy(nw), 1e-6, wg, wu, hidden, inter,
+                                batchSize=M, activation=activation)
+    normed = oracle.rmsnorm(X, nw, 1e-6)
+    want = oracle.q4k_ffn_gate_up(normed, Wg, Wu, M, hidden, inter, alpha=1.0, activation=activation)
+    assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
+
+
+def test_rmsnorm_prologue_fails_closed_for_large_batches():
+    W, wb = q4k_weight(64, 256, seed=2300)
+    A = ops.tensorFromNumpy(synth.normal_f32((9, 256), seed=2301))
+    nw = ops.tensorFromNumpy(np.ones(256, np.float32))
+    with pytest.raises(DopplerHipError, match="RMSNorm prologue"):
+        ops.runMatmul(A, wb, 9, 64, 256, outputDtype="f32", normWeight=nw, rmsNormEps=1e-6,
+                      useFusedRmsnormWideTile=True)
+
+
 # ----------------------------------------------------------------------------- LM head, argmax, gather
 
 def test_f16_weight_matmul_and_lmhead_argmax():
