@@ -147,6 +147,17 @@ FN(js_q4k_matmul) {
   ARGS(10); P(0, A); I(1, adt); P(2, W); P(3, C); I(4, cdt); I(5, M); I(6, N); I(7, K); F(8, alpha); P(9, res);
   return ret_rc(env, dh_q4k_matmul(A, adt, W, C, cdt, M, N, K, alpha, res));
 }
+FN(js_q4k_matmul_rmsnorm) {
+  ARGS(12); P(0, A); P(1, nw); F(2, eps); I(3, off); P(4, W); P(5, C); I(6, cdt); I(7, M); I(8, N); I(9, K);
+  F(10, alpha); P(11, res);
+  return ret_rc(env, dh_q4k_matmul_rmsnorm((const float*)A, (const float*)nw, eps, off, W, C, cdt, M, N, K, alpha, res));
+}
+FN(js_q4k_ffn_gate_up_rmsnorm) {
+  ARGS(13); P(0, x); P(1, nw); F(2, eps); I(3, off); P(4, wg); P(5, wu); P(6, o); I(7, M); I(8, hid); I(9, inter);
+  I(10, act); F(11, alpha); F(12, lim);
+  return ret_rc(env, dh_q4k_ffn_gate_up_rmsnorm((const float*)x, (const float*)nw, eps, off, wg, wu, (float*)o, M, hid,
+                                                inter, act, alpha, lim));
+}
 FN(js_q4k_ffn_gate_up) {
   ARGS(10); P(0, x); P(1, wg); P(2, wu); P(3, o); I(4, M); I(5, hid); I(6, inter); I(7, act); F(8, alpha); F(9, lim);
   return ret_rc(env, dh_q4k_ffn_gate_up((const float*)x, wg, wu, (float*)o, M, hid, inter, act, alpha, lim));
@@ -210,6 +221,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"eventCreate", js_event_create}, {"eventRecord", js_event_record}, {"eventElapsedMs", js_event_elapsed_ms},
       {"eventDestroy", js_event_destroy}, {"q4kDequant", js_q4k_dequant}, {"q4kMatmul", js_q4k_matmul},
       {"q4kFfnGateUp", js_q4k_ffn_gate_up}, {"f16wMatmul", js_f16w_matmul},
+      {"q4kMatmulRmsnorm", js_q4k_matmul_rmsnorm}, {"q4kFfnGateUpRmsnorm", js_q4k_ffn_gate_up_rmsnorm},
       {"lmheadArgmaxWorkspaceBytes", js_lmhead_argmax_workspace_bytes}, {"lmheadArgmaxF16", js_lmhead_argmax_f16},
       {"attnDecodeWorkspaceBytes", js_attn_decode_workspace_bytes}, {"attnDecode", js_attn_decode},
       {"rmsnorm", js_rmsnorm}, {"rope", js_rope}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},

@@ -2,7 +2,7 @@
 // text pipeline's quantized decode path calls (src/inference/pipelines/text/ops.js:3-30,
 // attention/interpreter.js:6-23).  Same names, argument order and option names.
 export { runMatmul, recordMatmul, runDequantQ4K } from './matmul.js';
-export { runFusedFFN, recordFusedFFN } from './fused_ffn.js';
+export { runFusedFFN, recordFusedFFN, runFusedNormedFFN, recordFusedNormedFFN } from './fused_ffn.js';
 export { runAttention, recordAttention } from './attention.js';
 export { runRMSNorm, recordRMSNorm } from './rmsnorm.js';
 export { runRoPE, recordRoPE } from './rope.js';

@@ -96,7 +96,18 @@ async function executeMatmul(recorder, A, B, M, N, K, options = {}) {
     const aPtr = aBuf.ptr + BigInt(aOffset);
     const bPtr = bBuf.ptr + BigInt(bOffset);
     const cPtr = output.ptr + BigInt(cOffset);
-    if (weightDtype === 'q4k') {
+    if (weightDtype === 'q4k' && options.normWeight != null && options.useFusedRmsnormWideTile === true) {
+      // RMSNorm of A inside the matmul (reference: matmul-selection.js:609-620)
+      if (!Number.isFinite(options.rmsNormEps)) {
+        throw new Error(`[${opLabel}] rmsNormEps is required with normWeight.`);
+      }
+      const normDtype = getWeightDtype(options.normWeight) || options.normWeight.dtype || 'f32';
+      if (normDtype !== 'f32') {
+        throw new Error(`[${opLabel}] the fused RMSNorm prologue takes an f32 norm weight, got ${normDtype}.`);
+      }
+      native.q4kMatmulRmsnorm(aPtr, ptrOf(options.normWeight), options.rmsNormEps, options.rmsNormOffset === true ? 1 : 0,
+        bPtr, cPtr, DTYPE[outputDtype], M, N, K, alpha, ptrOf(residualTensor));
+    } else if (weightDtype === 'q4k') {
       native.q4kMatmul(aPtr, DTYPE.f32, bPtr, cPtr, DTYPE[outputDtype], M, N, K, alpha, ptrOf(residualTensor));
     } else {
       if (outputDtype !== 'f32' || residualTensor) {

@@ -6,7 +6,7 @@
 import {
   createTensor, createWeightBuffer, acquireBuffer, releaseBuffer, uploadData, readBufferSlice,
   createCommandRecorder, recordGather, recordRMSNorm, recordMatmul, recordSplitQKVRMSNormRoPEQK,
-  recordAttention, recordFusedFFN, recordLmHeadArgmaxF16,
+  recordAttention, recordFusedNormedFFN, recordLmHeadArgmaxF16,
 } from '../kernel-selector.js';
 
 function upload(bytes, label) {
@@ -56,9 +56,10 @@ export class HipTextDecoder {
       { embeddingDtype: 'f16', outputDtype: 'f32' }));
     for (let li = 0; li < this.layers.length; li++) {
       const l = this.layers[li];
-      const normed = temp(await recordRMSNorm(recorder, x, l.inputNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden }));
-      const qkv = temp(await recordMatmul(recorder, normed, l.wqkv, 1, this.qSize + 2 * this.kSize, c.hidden,
-        { outputDtype: 'f32', role: 'qkv_proj', layerIdx: li }));
+      // input RMSNorm runs in the prologue of the stacked q/k/v projection
+      const qkv = temp(await recordMatmul(recorder, x, l.wqkv, 1, this.qSize + 2 * this.kSize, c.hidden,
+        { outputDtype: 'f32', role: 'qkv_proj', layerIdx: li,
+          normWeight: l.inputNorm, rmsNormEps: c.eps, useFusedRmsnormWideTile: true }));
       const split = await recordSplitQKVRMSNormRoPEQK(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps, {
         numTokens: 1, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim,
         qSize: this.qSize, kSize: this.kSize, vSize: this.kSize, startPos: pos,
@@ -71,8 +72,7 @@ export class HipTextDecoder {
       const attnFlat = createTensor(attn.buffer, 'f32', [1, this.qSize], 'attn_flat');
       const x2 = temp(await recordMatmul(recorder, attnFlat, l.wo, 1, c.hidden, this.qSize,
         { outputDtype: 'f32', role: 'o_proj', layerIdx: li, residualTensor: x }));
-      const normed2 = temp(await recordRMSNorm(recorder, x2, l.postAttnNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden }));
-      const act = temp(await recordFusedFFN(recorder, normed2, l.wgate, l.wup, c.hidden, c.inter,
+      const act = temp(await recordFusedNormedFFN(recorder, x2, l.postAttnNorm, c.eps, l.wgate, l.wup, c.hidden, c.inter,
         { batchSize: 1, activation: 'silu' }));
       x = temp(await recordMatmul(recorder, act, l.wdown, 1, c.hidden, c.inter,
         { outputDtype: 'f32', role: 'down_proj', layerIdx: li, residualTensor: x2 }));

@@ -49,6 +49,11 @@ async function main() {
       const A = tensor(c.A, 'f32', [c.M, c.K]);
       const opts = { outputDtype: c.outputDtype, alpha: c.alpha, role: 'test' };
       if (c.residual) opts.residualTensor = tensor(c.residual, 'f32', [c.M, c.N]);
+      if (c.normWeight) {
+        opts.normWeight = tensor(c.normWeight, 'f32', [c.K]);
+        opts.rmsNormEps = c.rmsNormEps;
+        opts.useFusedRmsnormWideTile = true;
+      }
       const rec = c.record ? dh.createCommandRecorder('t') : null;
       const t = rec ? await dh.recordMatmul(rec, A, W, c.M, c.N, c.K, opts) : await dh.runMatmul(A, W, c.M, c.N, c.K, opts);
       if (rec) await rec.submitAndWait();
@@ -58,6 +63,12 @@ async function main() {
       const Wu = dh.createWeightBuffer(dev(c.Wu), 'q4k', 'row', [c.inter, c.hidden]);
       const t = await dh.runFusedFFN(tensor(c.X, 'f32', [c.M, c.hidden]), Wg, Wu, c.hidden, c.inter,
         { batchSize: c.M, activation: c.activation, alpha: c.alpha, swigluLimit: c.swigluLimit });
+      await save(out, t.buffer, c.M * c.inter * 4);
+    } else if (c.op === 'fused_normed_ffn') {
+      const Wg = dh.createWeightBuffer(dev(c.Wg), 'q4k', 'row', [c.inter, c.hidden]);
+      const Wu = dh.createWeightBuffer(dev(c.Wu), 'q4k', 'row', [c.inter, c.hidden]);
+      const t = await dh.runFusedNormedFFN(tensor(c.X, 'f32', [c.M, c.hidden]), tensor(c.normWeight, 'f32', [c.hidden]),
+        c.eps, Wg, Wu, c.hidden, c.inter, { batchSize: c.M, activation: c.activation });
       await save(out, t.buffer, c.M * c.inter * 4);
     } else if (c.op === 'rmsnorm') {
       const opts = { batchSize: c.batch, hiddenSize: c.hidden, rmsNormWeightOffset: c.weightOffset };

@@ -70,7 +70,13 @@ def test_js_host_path_parity(tmp_path):
         A = synth.normal_f32((M, K), seed + 1)
         c = dict(name=name, op="matmul", wdtype="q4k", W=put(name + ".W", Wm), A=put(name + ".A", A), M=M, N=N, K=K,
                  outputDtype=kw.get("outputDtype", "f32"), alpha=kw.get("alpha", 1.0), record=kw.get("record", False))
-        want = oracle.q4k_matmul(A, Wm, M, N, K, c["alpha"])
+        if kw.get("normed"):
+            nw = 1.0 + synth.normal_f32((K,), seed + 3, 0.1)
+            c["normWeight"] = put(name + ".nw", nw)
+            c["rmsNormEps"] = 1e-6
+            want = oracle.q4k_matmul(oracle.rmsnorm(A, nw, 1e-6), Wm, M, N, K, c["alpha"])
+        else:
+            want = oracle.q4k_matmul(A, Wm, M, N, K, c["alpha"])
         if kw.get("residual"):
             R = synth.normal_f32((M, N), seed + 2)
             c["residual"] = put(name + ".R", R)
@@ -83,6 +89,7 @@ def test_js_host_path_parity(tmp_path):
     mm("mm_cfg1", 4, 3072, 1024, 9110, record=True)
     mm("mm_res", 2, 512, 1024, 9120, alpha=0.5, residual=True)
     mm("mm_f16", 1, 512, 1024, 9130, outputDtype="f16", alpha=2.0 ** -8)
+    mm("mm_normed", 1, 768, 1024, 9140, normed=True, residual=True)
 
     # f16 weights
     E = synth.normal_f16_bits((3000, 512), 9200, 0.02)
@@ -101,6 +108,13 @@ def test_js_host_path_parity(tmp_path):
                       hidden=768, inter=1024, activation="silu", alpha=1.0, swigluLimit=5.0))
     ffn_want = oracle.q4k_ffn_gate_up(X, Wg, Wu, 2, 768, 1024, activation="silu", swiglu_limit=5.0)
     checks.append(lambda: rel_l2(get("ffn.out.bin", np.float32), ffn_want) <= 1e-3)
+
+    nwf = 1.0 + synth.normal_f32((768,), 9303, 0.1)
+    Xn = synth.normal_f32((2, 768), 9304, 4.0)
+    cases.append(dict(name="ffn_normed", op="fused_normed_ffn", Wg="ffn.Wg", Wu="ffn.Wu", X=put("ffnn.X", Xn),
+                      normWeight=put("ffnn.nw", nwf), eps=1e-6, M=2, hidden=768, inter=1024, activation="gelu"))
+    ffnn_want = oracle.q4k_ffn_gate_up(oracle.rmsnorm(Xn, nwf, 1e-6), Wg, Wu, 2, 768, 1024, activation="gelu")
+    checks.append(lambda: rel_l2(get("ffn_normed.out.bin", np.float32), ffnn_want) <= 1e-3)
 
     # rmsnorm, rope, split qkv, kv write
     x = synth.normal_f32((3, 1152), 9400, 3.0)
