@@ -341,6 +341,7 @@ int env_int(const char* name, int dflt) {
 }
 
 constexpr int kMaxDepth = 4;
+constexpr int kRedSlots = 4;       // tiles a fast wave may run ahead of the slowest one
 
 #ifdef DH_GEMV_TRACE
 __device__ unsigned long long dh_trace_buf[256 * 64];
@@ -497,7 +498,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
   constexpr int NTHR = 64 * WAVES;
   constexpr int XC = 2 * MT, NO = MfmaShape<MT>::NI / 2, NMAT = DUAL ? 2 : 1;
   __shared__ __align__(16) unsigned char xs[XBYTES];        // x fragments | zero row | (sum, 1/scale)
-  __shared__ float red[2][WAVES][NMAT][NO][64];
+  // K-slice partial sums per tile slot; only lanes 0..31 carry activation rows 0..1 (MT <= 2)
+  __shared__ float red[kRedSlots][WAVES][NMAT][NO][32];
+  __shared__ unsigned done[kRedSlots];                       // waves that delivered their partials
   __shared__ float norm_ss[WAVES][MT];
   extern __shared__ __align__(16) unsigned char ring[];     // [WAVES][depth][R*144]
 
@@ -569,12 +572,14 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
   // ---- stage the activations in LDS.  Work item = (sub-block sb, activation row m): 32 floats.
   // The first item's loads go out before the ring loads (loads complete in order), its
   // conversion runs while the ring fills.
+  bool early_ring;
   {
     // Everything this thread needs from memory for its first quarter item is loaded before the
     // ring starts: loads complete in order, so a wait for a later load would also wait for the
     // ring loads in front of it.
     const int total = 4 * MT * nsub;
     const bool norm = a.norm_weight != nullptr;
+    early_ring = wave * 64 >= total || total >= NTHR;
     float v0[8], wn0[8];
     if (tid < total) stage_x_load<MT>(a.A, a.M, a.K, tid, v0);
     float ss = 0.f;
@@ -592,10 +597,18 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
         for (int j = 0; j < 8; j++) ss = fmaf(t[j], t[j], ss);
       }
     }
+    // Waves without staging work start their ring at once.  Waves that stage do so too when
+    // every wave stages; otherwise they convert first and start their ring after the barrier,
+    // so the others can begin computing as early as possible.
     DH_TS();
     DH_WAIT_VM(0);
     DH_TS();
-    for (int d = 0; d < D; d++) DH_ISSUE_NEXT();
+#pragma unroll 1
+    for (int phase = 0; phase < 2; phase++) {     // a loop so that the ring start exists once in the code
+    if ((phase == 0) == early_ring) {
+      for (int d = 0; d < D; d++) DH_ISSUE_NEXT();
+    }
+    if (phase == 1) break;
     DH_TS();
     float inv = 1.f;
     if (norm) {
@@ -631,11 +644,13 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
       }
       stage_x_store<MT>(idx, t, xf, sxi);
     }
+    if (tid < 16) reinterpret_cast<uint32_t*>(xzero)[tid] = 0u;
+    if (tid < kRedSlots) done[tid] = 0u;
+    DH_TS();
+    DH_LDS_BARRIER();
+    DH_TS();
+    }
   }
-  if (tid < 16) reinterpret_cast<uint32_t*>(xzero)[tid] = 0u;
-  DH_TS();
-  DH_LDS_BARRIER();
-  DH_TS();
 
   const _Float16* xfl = xcol < XC ? xf + xcol * 32 + g2 * 16 : xzero;
   const int xf_stride = xcol < XC ? XC * 32 : 0;
@@ -643,10 +658,11 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
   const uint32_t lane_lds =
       (uint32_t)(uintptr_t)DH_LDS_PTR(my_ring) + (uint32_t)min(lane & 31, R - 1) * kBlockBytes;
 
-  int consumed = 0, cstage = 0, par = 0;
+  int consumed = 0, cstage = 0;
 #pragma unroll 1
   for (int tl = 0; tl < ntl; tl++) {
     const int tile = blockIdx.x + tl * gridDim.x;
+    const int slot = tl % kRedSlots;
 #pragma unroll 1
     for (int mat = 0; mat < NMAT; mat++) {
       float acc[NO];
@@ -686,36 +702,52 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
 #endif
         DH_TS();
       }
+      if (lane < 32) {
 #pragma unroll
-      for (int k = 0; k < NO; k++) red[par][wave][mat][k][lane] = acc[k];
+        for (int k = 0; k < NO; k++) red[slot][wave][mat][k][lane] = acc[k];
+      }
     }
-    DH_LDS_BARRIER();
-    // ---- the waves' K slices meet: thread (k, lane) finishes output (row lane & 31, m)
-    const int ln = tid & 63, k = tid >> 6;
-    const int m = (k & 1) + 2 * (ln >> 5) + 4 * (k >> 1);
-    const int64_t row = (int64_t)tile * R + (ln & 31);
-    if (tid < NO * 64 && m < a.M && (ln & 31) < R && row < a.N) {
-      float sg = 0.f, su = 0.f;
+    // ---- tile end.  Nobody waits: each wave reports its partial sums and moves on; the wave
+    // that arrives last adds the K slices in wave order and writes the outputs.  LDS executes a
+    // wave's operations in order, so every earlier arrival's partials are in place by then.
+    // (The counter is bumped with a hand-written LDS atomic: the compiler would put a wait for
+    // all loads in flight in front of its own, because the ring loads write LDS too.)
+    unsigned arrived = 0;
+    if (lane == 0) {
+      const uint32_t cnt_addr = (uint32_t)(uintptr_t)DH_LDS_PTR(&done[slot]);
+      asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                   : "=&v"(arrived) : "v"(cnt_addr), "v"(1u) : "memory");
+    }
+    arrived = __builtin_amdgcn_readfirstlane(arrived);
+    asm volatile("" ::: "memory");
+    if (arrived == WAVES - 1) {
+      const int r = lane & 31, m = lane >> 5;
+      const int64_t row = (int64_t)tile * R + r;
+      if (m < a.M && m < MT && r < R && row < a.N) {
+        float sg = 0.f, su = 0.f;
 #pragma unroll
-      for (int w = 0; w < WAVES; w++) {
-        sg += red[par][w][0][k][ln];
-        if (DUAL) su += red[par][w][NMAT - 1][k][ln];
+        for (int w = 0; w < WAVES; w++) {
+          sg += red[slot][w][0][m][r];
+          if (DUAL) su += red[slot][w][NMAT - 1][m][r];
+        }
+        float v;
+        if (DUAL) {
+          const float act = a.activation == DH_ACT_SILU ? act_silu(sg) : act_gelu(sg);
+          v = act * su * a.alpha;
+          if (a.activation == DH_ACT_SILU && a.clamp_max > 0.f) v = fminf(fmaxf(v, -a.clamp_max), a.clamp_max);
+        } else {
+          v = sg * a.alpha;
+          if (a.residual) v += a.residual[(int64_t)m * a.N + row];
+        }
+        if (a.c_f16)
+          reinterpret_cast<__half*>(a.C)[(int64_t)m * a.N + row] = __float2half(v);
+        else
+          reinterpret_cast<float*>(a.C)[(int64_t)m * a.N + row] = v;
       }
-      float v;
-      if (DUAL) {
-        const float act = a.activation == DH_ACT_SILU ? act_silu(sg) : act_gelu(sg);
-        v = act * su * a.alpha;
-        if (a.activation == DH_ACT_SILU && a.clamp_max > 0.f) v = fminf(fmaxf(v, -a.clamp_max), a.clamp_max);
-      } else {
-        v = sg * a.alpha;
-        if (a.residual) v += a.residual[(int64_t)m * a.N + row];
-      }
-      if (a.c_f16)
-        reinterpret_cast<__half*>(a.C)[(int64_t)m * a.N + row] = __float2half(v);
-      else
-        reinterpret_cast<float*>(a.C)[(int64_t)m * a.N + row] = v;
+      if (lane == 0) done[slot] = 0u;
     }
-    par ^= 1;     // the other half of `red` is free: everyone passed this tile's barrier
+    // more tiles than slots: keep the waves within one tile of each other instead
+    if (ntl > kRedSlots) DH_LDS_BARRIER();
     DH_TS();
   }
 #ifdef DH_GEMV_TRACE
@@ -732,7 +764,7 @@ size_t ring_x_bytes(int mt, int nb) { return (size_t)nb * 8 * mt * (2 * 32 * 2 +
 template <int MT, bool DUAL, int XBYTES, int WAVES>
 int launch_ring_cfg(RingArgs a, const char* op) {
   constexpr int NO = MfmaShape<MT>::NI / 2, NMAT = DUAL ? 2 : 1;
-  const size_t fixed = XBYTES + sizeof(float) * 2 * WAVES * NMAT * NO * 64 + 256;
+  const size_t fixed = XBYTES + sizeof(float) * kRedSlots * WAVES * NMAT * NO * 32 + 512;
   auto kern = q4k_gemv_ring_kernel<MT, DUAL, XBYTES, WAVES>;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
