@@ -425,10 +425,18 @@ __device__ __forceinline__ void stage_norm_weight_load(const float* __restrict__
                                                        float (&wn)[8]) {
   const int item = idx >> 2, grp = idx & 3;
   const int k0 = (item / MT) * 32 + grp * 8, left = K - k0;
+  const float* src = w + k0;
+  if (left >= 8 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+    const float4 t0 = reinterpret_cast<const float4*>(src)[0], t1 = reinterpret_cast<const float4*>(src)[1];
+    wn[0] = t0.x; wn[1] = t0.y; wn[2] = t0.z; wn[3] = t0.w;
+    wn[4] = t1.x; wn[5] = t1.y; wn[6] = t1.z; wn[7] = t1.w;
+  } else {
 #pragma unroll
-  for (int j = 0; j < 8; j++) {
-    const float t = left > 0 ? w[k0 + min(j, left - 1)] : 0.f;
-    wn[j] = j < left ? (offset ? 1.0f + t : t) : 0.f;
+    for (int j = 0; j < 8; j++) wn[j] = j < left ? src[j] : 0.f;
+  }
+  if (offset) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) wn[j] = j < left ? 1.0f + wn[j] : 0.f;
   }
 }
 
@@ -584,11 +592,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     if (tid < total) stage_x_load<MT>(a.A, a.M, a.K, tid, v0);
     float ss = 0.f;
     if (norm) {
-      if (tid < total) {
-        stage_norm_weight_load<MT>(a.norm_weight, a.K, a.norm_weight_offset, tid, wn0);
-#pragma unroll
-        for (int j = 0; j < 8; j++) ss = fmaf(v0[j], v0[j], ss);
-      }
+      if (tid < total) stage_norm_weight_load<MT>(a.norm_weight, a.K, a.norm_weight_offset, tid, wn0);
 #pragma unroll 1
       for (int idx = tid + NTHR; idx < total; idx += NTHR) {   // rows longer than one pass
         float t[8];
@@ -603,15 +607,22 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     DH_TS();
     DH_WAIT_VM(0);
     DH_TS();
-#pragma unroll 1
-    for (int phase = 0; phase < 2; phase++) {     // a loop so that the ring start exists once in the code
-    if ((phase == 0) == early_ring) {
-      for (int d = 0; d < D; d++) DH_ISSUE_NEXT();
+    if (norm && tid < total) {
+#pragma unroll
+      for (int j = 0; j < 8; j++) ss = fmaf(v0[j], v0[j], ss);
     }
-    if (phase == 1) break;
-    DH_TS();
+    // Three phases (a loop, so that the ring-start code exists once): ring stages are put in
+    // flight before the norm reduction, before the conversion and after it.  Early waves start
+    // one stage at once and the rest after the norm barrier (which they would otherwise reach
+    // late, holding up the waves that convert); late waves start after the conversion.
     float inv = 1.f;
-    if (norm) {
+#pragma unroll 1
+    for (int phase = 0; phase < 3; phase++) {
+    const int nstart = early_ring ? (norm ? (phase == 0 ? 1 : (phase == 1 ? D - 1 : 0)) : (phase == 0 ? D : 0))
+                                  : (phase == 2 ? D : 0);
+    for (int d = 0; d < nstart; d++) DH_ISSUE_NEXT();
+    DH_TS();
+    if (phase == 0 && norm) {
       // sum of squares of activation row m = (tid >> 2) % MT: lanes of a quad share a row,
       // lane bit 2 selects the row when MT == 2
       ss += quad_xor_f32(ss, 1);
@@ -628,6 +639,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
       for (int w = 0; w < WAVES; w++) tot += norm_ss[w][my_m];
       inv = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
     }
+    if (phase != 1) continue;
 #pragma unroll 1
     for (int idx = tid; idx < total; idx += NTHR) {
       float t[8], wn[8];
