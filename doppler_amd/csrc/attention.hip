@@ -15,7 +15,6 @@ namespace {
 
 constexpr int kTileKeys = 64;
 constexpr int kMaxG = 8;       // query heads per kv head
-constexpr int kMaxPairs = 4;   // output element pairs per thread (G*D <= 2048)
 
 struct AttnArgs {
   const float* Q;       // [H][D]
@@ -39,171 +38,261 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-template <int D>
+typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
+typedef __attribute__((ext_vector_type(4))) float float4_t;
+
+#ifdef DH_ATTN_TRACE
+__device__ unsigned long long dh_attn_trace_buf[1024 * 32];
+#define DH_ATS() do { if (tid == DH_ATTN_TRACE && tsn < 31) tsbuf[tsn++] = wall_clock64(); } while (0)
+#else
+#define DH_ATS() do {} while (0)
+#endif
+
+// Reductions across the lanes of a 16-lane row with DPP row shifts (no LDS traffic): afterwards
+// the last lane of every aligned group of `span` lanes (span = 2, 4, 8 or 16) holds the
+// group's result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_row(float old, float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(old), __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+template <int SPAN>
+__device__ __forceinline__ float row_group_max(float v) {
+  if (SPAN > 1) v = fmaxf(v, dpp_row<0x111>(v, v));
+  if (SPAN > 2) v = fmaxf(v, dpp_row<0x112>(v, v));
+  if (SPAN > 4) v = fmaxf(v, dpp_row<0x114>(v, v));
+  if (SPAN > 8) v = fmaxf(v, dpp_row<0x118>(v, v));
+  return v;
+}
+template <int SPAN>
+__device__ __forceinline__ float row_group_sum(float v) {
+  if (SPAN > 1) v += dpp_row<0x111>(0.f, v);
+  if (SPAN > 2) v += dpp_row<0x112>(0.f, v);
+  if (SPAN > 4) v += dpp_row<0x114>(0.f, v);
+  if (SPAN > 8) v += dpp_row<0x118>(0.f, v);
+  return v;
+}
+
+// One workgroup = one chunk of 64 keys of one kv head (or several chunks, strided, for long
+// contexts), four waves, two barriers per chunk.
+//   scores   wave w takes keys 16w..16w+15: S = Q.K^T with v_mfma_f32_16x16x32_f16.  The A
+//            operand holds the G query heads of the kv head as rows (2g, 2g+1) = f16 high part
+//            and f16 residual of scale*q (so q keeps ~22 bits); the B operand is loaded from
+//            HBM directly in operand layout (lane (key, kg) reads 16 bytes of its key's row).
+//   softmax  every wave redoes the (tiny) online-softmax update for all heads from the scores
+//            in LDS, so no second exchange is needed: 64/GT lanes per head, GT keys per lane,
+//            DPP row reductions, the per-head maxima and sums travel through scalar registers.
+//   P.V      wave w owns output dims [D/4*w, D/4*(w+1)); lane (dq, kh) holds 4 dims of keys
+//            kh, kh+KH, ... in registers and accumulates them for all heads; the key groups
+//            meet in a wave-private LDS buffer at the end.
+// K and V of the next chunk are requested before the current one is consumed.
+// GT: query heads per kv head rounded up to 1, 2, 4 or 8 (bounds the unrolled per-head code).
+template <int D, int GT>
 __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a) {
-  constexpr int RS = D + 8;             // LDS row stride in halves: 16-byte aligned, bank-skewed
-  constexpr int PART = D / 4;           // halves of a K row handled by one lane
-  __shared__ __align__(16) __half k_tile[kTileKeys * RS];
-  __shared__ __align__(16) __half v_tile[kTileKeys * RS];
-  __shared__ __align__(16) float q_s[kMaxG * D];
-  __shared__ float p_s[kMaxG * kTileKeys];   // scores, then probabilities
-  __shared__ float alpha_s[kMaxG];           // per-head rescale of the running output
-  __shared__ float m_s[kMaxG], l_s[kMaxG];
-  __shared__ float red_s[kMaxPairs * 2 * 256];  // cross key-subset reduction at the end
+  constexpr int STEPS = D / 32;          // MFMAs per 16 keys
+  constexpr int DW = D / 4;              // output dims per wave
+  constexpr int LPK = DW / 4;            // lanes per key in P.V (4 dims each)
+  constexpr int KH = 64 / LPK;           // key groups
+  constexpr int NJ = kTileKeys / KH;     // keys per lane
+  constexpr int LH = 64 / GT;            // softmax: lanes per head (each holds GT keys)
+  constexpr int SPAN = LH < 16 ? LH : 16;
+  __shared__ __align__(16) float s_lds[GT][kTileKeys];        // raw scores of the chunk
+  __shared__ __align__(16) float p_lds[4][GT][kTileKeys];     // per-wave probabilities
+  __shared__ __align__(16) float o_lds[4][KH][GT][DW];        // per-wave partial outputs
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int kvh = blockIdx.x, split = blockIdx.y;
+#ifdef DH_ATTN_TRACE
+  unsigned long long* tsbuf = dh_attn_trace_buf + ((blockIdx.y * gridDim.x + blockIdx.x) & 1023) * 32;
+  int tsn = 0;
+#endif
+  DH_ATS();
   const int G = a.G;
-  const int EP = G * D / 2;                       // output element pairs of this kv head
-  const int KS = EP >= 256 ? 1 : 256 / EP;        // key subsets when threads outnumber pairs
-  const int npairs = EP >= 256 ? (EP + 255) / 256 : 1;
+  const int64_t row_stride = (int64_t)a.Hkv * D;   // halves between consecutive keys
+  const int qrow = lane & 15, kg = lane >> 4;
+  const int dq = lane % LPK, kh = lane / LPK;
+  const int key_s = 16 * wave + (lane & 15);
+  const int nkeys_total = a.kend - a.kbeg;
+  const int nchunks = (nkeys_total + kTileKeys - 1) / kTileKeys;
 
-  for (int i = tid; i < G * D; i += 256) q_s[i] = a.Q[(int64_t)(kvh * G) * D + i];
-  if (tid < G) { m_s[tid] = -FLT_MAX; l_s[tid] = 0.f; }
-  float2 o_acc[kMaxPairs];
+  uint4 kf[STEPS];
+  uint2 vf[NJ], vn[NJ];
+  // Requests this wave's 16 keys of K (into kf) and its dim slice of V (into vn) of chunk c.
+#define DH_ATTN_LOAD(c_)                                                                          \
+  do {                                                                                            \
+    const int kbase_ = a.kbeg + (c_) * kTileKeys;                                                 \
+    const int nk_ = min(kTileKeys, a.kend - kbase_);                                              \
+    /* first cache row of the chunk; in ring layout rows wrap at the window (a chunk never */     \
+    /* spans more keys than the window holds, so one conditional subtraction is enough)    */     \
+    int row0_ = a.kv_start + kbase_, wrap_ = 0x7fffffff;                                          \
+    if (a.ring_window > 0) {                                                                      \
+      row0_ = (int)((unsigned)row0_ % (unsigned)a.ring_window);                                   \
+      wrap_ = a.ring_window;                                                                      \
+    }                                                                                             \
+    int row_ = row0_ + min(key_s, nk_ - 1);                                                       \
+    row_ = row_ >= wrap_ ? row_ - wrap_ : row_;                                                   \
+    const __half* kp_ = a.K + (int64_t)row_ * row_stride + (int64_t)kvh * D + 8 * kg;             \
+    _Pragma("unroll") for (int s = 0; s < STEPS; s++)                                             \
+      kf[s] = *reinterpret_cast<const uint4*>(kp_ + 32 * s);                                      \
+    _Pragma("unroll") for (int j = 0; j < NJ; j++) {                                              \
+      int r_ = row0_ + min(kh + KH * j, nk_ - 1);                                                 \
+      r_ = r_ >= wrap_ ? r_ - wrap_ : r_;                                                         \
+      vn[j] = *reinterpret_cast<const uint2*>(a.V + (int64_t)r_ * row_stride + (int64_t)kvh * D + \
+                                              DW * wave + 4 * dq);                                \
+    }                                                                                             \
+  } while (0)
+
+  if (split < nchunks) DH_ATTN_LOAD(split);
+
+  // ---- query fragments (A operand): row = lane & 15 -> head row>>1, high part / residual
+  half8_t qa[STEPS];
 #pragma unroll
-  for (int i = 0; i < kMaxPairs; i++) o_acc[i] = make_float2(0.f, 0.f);
-  __syncthreads();
-
-  const int tile0 = split * a.tiles_per_split;
-  const int key_lo = a.kbeg + tile0 * kTileKeys;
-  const int key_hi = min(a.kend, key_lo + a.tiles_per_split * kTileKeys);
-
-  for (int kt = key_lo; kt < key_hi; kt += kTileKeys) {
-    const int nkeys = min(kTileKeys, key_hi - kt);
-    // ---- stage K and V tiles: 16 bytes per thread per step, rows are D*2 contiguous bytes
-    constexpr int VEC_PER_ROW = D / 8;
-    for (int i = tid; i < kTileKeys * VEC_PER_ROW; i += 256) {
-      const int r = i / VEC_PER_ROW, cvec = i - r * VEC_PER_ROW;
-      uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-      if (r < nkeys) {
-        int64_t row = (int64_t)a.kv_start + kt + r;
-        if (a.ring_window > 0) row %= a.ring_window;
-        const int64_t off = (row * a.Hkv + kvh) * D + cvec * 8;
-        kv = *reinterpret_cast<const uint4*>(a.K + off);
-        vv = *reinterpret_cast<const uint4*>(a.V + off);
+  for (int s = 0; s < STEPS; s++) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) qa[s][i] = (_Float16)0.f;
+    if ((qrow >> 1) < G) {
+      const float* qp = a.Q + (int64_t)(kvh * G + (qrow >> 1)) * D + 32 * s + 8 * kg;
+      const float4 q0 = reinterpret_cast<const float4*>(qp)[0], q1 = reinterpret_cast<const float4*>(qp)[1];
+      const float qv[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const float xs = qv[i] * a.scale;
+        const _Float16 h = (_Float16)xs;
+        qa[s][i] = (qrow & 1) ? (_Float16)(xs - (float)h) : h;
       }
-      *reinterpret_cast<uint4*>(k_tile + r * RS + cvec * 8) = kv;
-      *reinterpret_cast<uint4*>(v_tile + r * RS + cvec * 8) = vv;
     }
-    __syncthreads();
+  }
+  DH_ATS();
+  float m_run[GT], l_run[GT], acc[GT][4];
+#pragma unroll
+  for (int g = 0; g < GT; g++) {
+    m_run[g] = -FLT_MAX; l_run[g] = 0.f;
+    acc[g][0] = acc[g][1] = acc[g][2] = acc[g][3] = 0.f;
+  }
+  const int sm_g = lane / LH, sm_q = lane % LH;      // softmax role: head, key group
 
-    // ---- scores: lane (key = tid>>2, part = tid&3) covers a quarter of the head dim
+  for (int c = split; c < nchunks; c += a.nsplit) {
+    const int kbase = a.kbeg + c * kTileKeys;
+    const int nk = min(kTileKeys, a.kend - kbase);
+    DH_ATS();
+    // ---- scores of 16 keys x G heads
+    float4_t d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < STEPS; s++)
+      d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[s], __builtin_bit_cast(half8_t, kf[s]), d, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NJ; j++) vf[j] = vn[j];
+    if (c + a.nsplit < nchunks) DH_ATTN_LOAD(c + a.nsplit);
+    // lane (key, kg) holds rows 4kg..4kg+3 = heads 2kg (high + residual), 2kg+1
     {
-      const int key = tid >> 2, part = tid & 3;
-      float kf[PART];
-#pragma unroll
-      for (int v8 = 0; v8 < PART / 8; v8++) {
-        const uint4 raw = *reinterpret_cast<const uint4*>(k_tile + key * RS + part * PART + v8 * 8);
-        const __half2* h2 = reinterpret_cast<const __half2*>(&raw);
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          const float2 f = __half22float2(h2[j]);
-          kf[v8 * 8 + 2 * j] = f.x;
-          kf[v8 * 8 + 2 * j + 1] = f.y;
-        }
+      float sc2[2] = {d[0] + d[1], d[2] + d[3]};
+      if (a.softcap > 0.f) {
+#pragma unroll 1
+        for (int e = 0; e < 2; e++) sc2[e] = tanhf(sc2[e] / a.softcap) * a.softcap;
       }
-      for (int g = 0; g < G; g++) {
-        const float* qg = q_s + g * D + part * PART;
-        float dot = 0.f;
+      const bool valid = key_s < nk;
+      if (2 * kg < GT) s_lds[2 * kg][key_s] = valid ? sc2[0] : -FLT_MAX;
+      if (2 * kg + 1 < GT) s_lds[2 * kg + 1][key_s] = valid ? sc2[1] : -FLT_MAX;
+    }
+    DH_ATS();
+    __syncthreads();
+    DH_ATS();
+    // ---- online softmax: lane (head sm_g, group sm_q) owns keys sm_q*GT .. sm_q*GT + GT - 1
+    {
+      float sc[GT], pr[GT];
 #pragma unroll
-        for (int j = 0; j < PART; j += 4) {
-          const float4 qv = *reinterpret_cast<const float4*>(qg + j);
-          dot = fmaf(qv.x, kf[j], dot);
-          dot = fmaf(qv.y, kf[j + 1], dot);
-          dot = fmaf(qv.z, kf[j + 2], dot);
-          dot = fmaf(qv.w, kf[j + 3], dot);
-        }
-        dot += __shfl_xor(dot, 1, 64);
-        dot += __shfl_xor(dot, 2, 64);
-        if (part == 0) {
-          float s = dot * a.scale;
-          if (a.softcap > 0.f) s = tanhf(s / a.softcap) * a.softcap;
-          p_s[g * kTileKeys + key] = key < nkeys ? s : -FLT_MAX;
-        }
+      for (int i = 0; i < GT; i++) sc[i] = s_lds[sm_g][sm_q * GT + i];
+      float mx = sc[0];
+#pragma unroll
+      for (int i = 1; i < GT; i++) mx = fmaxf(mx, sc[i]);
+      mx = row_group_max<SPAN>(mx);
+      float m_new[GT], alpha[GT], my_m = 0.f;
+#pragma unroll
+      for (int g = 0; g < GT; g++) {
+        float m = m_run[g];
+#pragma unroll
+        for (int r = 0; r < LH / SPAN; r++)       // the head's rows (or its single group)
+          m = fmaxf(m, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx), g * LH + r * SPAN + SPAN - 1)));
+        m_new[g] = m;
+        alpha[g] = __expf(m_run[g] - m);
+        if (g == sm_g) my_m = m;
+      }
+      float ps = 0.f;
+#pragma unroll
+      for (int i = 0; i < GT; i++) {
+        pr[i] = sm_q * GT + i < nk ? __expf(sc[i] - my_m) : 0.f;
+        ps += pr[i];
+        p_lds[wave][sm_g][sm_q * GT + i] = pr[i];
+      }
+      ps = row_group_sum<SPAN>(ps);
+#pragma unroll
+      for (int g = 0; g < GT; g++) {
+        float t = 0.f;
+#pragma unroll
+        for (int r = 0; r < LH / SPAN; r++)
+          t += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ps), g * LH + r * SPAN + SPAN - 1));
+        l_run[g] = l_run[g] * alpha[g] + t;
+        m_run[g] = m_new[g];
+        acc[g][0] *= alpha[g]; acc[g][1] *= alpha[g]; acc[g][2] *= alpha[g]; acc[g][3] *= alpha[g];
       }
     }
-    __syncthreads();
-
-    // ---- online softmax per query head: wave w takes heads w, w+4
-    for (int g = wave; g < G; g += 4) {
-      const float s = p_s[g * kTileKeys + lane];
-      const float m_old = m_s[g];
-      const float m_new = fmaxf(m_old, wave_max(s));
-      const float p = lane < nkeys ? __expf(s - m_new) : 0.f;
-      const float psum = wave_sum(p);
-      p_s[g * kTileKeys + lane] = p;
-      if (lane == 0) {
-        const float alpha = __expf(m_old - m_new);
-        alpha_s[g] = alpha;
-        l_s[g] = l_s[g] * alpha + psum;
-        m_s[g] = m_new;
-      }
-    }
-    __syncthreads();
-
-    // ---- o = o*alpha + P.V : each thread owns pairs of adjacent output dims
+    DH_ATS();
+    // ---- P.V for this wave's dims (p_lds[wave] is private to the wave: program order suffices)
 #pragma unroll
-    for (int i = 0; i < kMaxPairs; i++) {
-      if (i >= npairs) break;
-      const int ep = (EP >= 256 ? tid + i * 256 : tid % EP);
-      const int ks = EP >= 256 ? 0 : tid / EP;
-      if (ep < EP && ks < KS) {
-        const int g = ep / (D / 2), dp = ep - g * (D / 2);
-        const float alpha = alpha_s[g];
-        float2 acc = make_float2(o_acc[i].x * alpha, o_acc[i].y * alpha);
-        const float* pg = p_s + g * kTileKeys;
-        for (int k = ks; k < nkeys; k += KS) {
-          const float2 vf = __half22float2(*reinterpret_cast<const __half2*>(v_tile + k * RS + dp * 2));
-          const float p = pg[k];
-          acc.x = fmaf(p, vf.x, acc.x);
-          acc.y = fmaf(p, vf.y, acc.y);
-        }
-        o_acc[i] = acc;
+    for (int j = 0; j < NJ; j++) {
+      const int key = kh + KH * j;
+      const __half2* h2 = reinterpret_cast<const __half2*>(&vf[j]);
+      const float2 v01 = __half22float2(h2[0]), v23 = __half22float2(h2[1]);
+#pragma unroll
+      for (int g = 0; g < GT; g++) {
+        const float p = p_lds[wave][g][key];
+        acc[g][0] = fmaf(p, v01.x, acc[g][0]);
+        acc[g][1] = fmaf(p, v01.y, acc[g][1]);
+        acc[g][2] = fmaf(p, v23.x, acc[g][2]);
+        acc[g][3] = fmaf(p, v23.y, acc[g][3]);
       }
     }
-    __syncthreads();
+    DH_ATS();
+    __syncthreads();     // s_lds is rewritten by the next chunk
   }
+  DH_ATS();
+#undef DH_ATTN_LOAD
 
-  // ---- combine key subsets, then write the split's (o, m, l)
+  // ---- key groups meet in the wave's LDS buffer, then the split's (o, m, l) go out
 #pragma unroll
-  for (int i = 0; i < kMaxPairs; i++) {
-    red_s[(i * 2) * 256 + tid] = o_acc[i].x;
-    red_s[(i * 2 + 1) * 256 + tid] = o_acc[i].y;
-  }
-  __syncthreads();
-  for (int i = 0; i < npairs; i++) {
-    const int ep = tid + i * 256;
-    if (ep < EP && (EP >= 256 || tid < EP)) {
-      float ox = 0.f, oy = 0.f;
-      if (EP >= 256) {
-        ox = red_s[(i * 2) * 256 + tid];
-        oy = red_s[(i * 2 + 1) * 256 + tid];
-      } else {
-        for (int ks = 0; ks < KS; ks++) {
-          ox += red_s[ks * EP + ep];
-          oy += red_s[256 + ks * EP + ep];
-        }
-      }
-      const int g = ep / (D / 2), dp = ep - g * (D / 2);
+  for (int g = 0; g < GT; g++)
+    *reinterpret_cast<float4*>(&o_lds[wave][kh][g][4 * dq]) = make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+#pragma unroll
+  for (int t = 0; t < (GT * DW + 63) / 64; t++) {
+    const int o = lane + 64 * t, g = min(o / DW, GT - 1), dim = o % DW;
+    float v = 0.f;
+#pragma unroll
+    for (int k = 0; k < KH; k++) v += o_lds[wave][k][g][dim];
+    if (o < GT * DW && g < G) {
       const int h = kvh * G + g;
       if (a.nsplit == 1) {
-        const float l = l_s[g];
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
-        a.O[(int64_t)h * D + 2 * dp] = ox * inv;
-        a.O[(int64_t)h * D + 2 * dp + 1] = oy * inv;
+        float l = 0.f;
+#pragma unroll
+        for (int gg = 0; gg < GT; gg++) l = gg == g ? l_run[gg] : l;
+        a.O[(int64_t)h * D + DW * wave + dim] = l > 0.f ? v / l : 0.f;
       } else {
-        float* w = a.ws + ((int64_t)h * a.nsplit + split) * (D + 2);
-        w[2 * dp] = ox;
-        w[2 * dp + 1] = oy;
+        a.ws[((int64_t)h * a.nsplit + split) * (D + 2) + DW * wave + dim] = v;
       }
     }
   }
-  if (a.nsplit > 1 && tid < G) {
-    float* w = a.ws + ((int64_t)(kvh * G + tid) * a.nsplit + split) * (D + 2);
-    w[D] = m_s[tid];
-    w[D + 1] = l_s[tid];
+  if (a.nsplit > 1 && wave == 0 && lane < G) {
+    float* w = a.ws + ((int64_t)(kvh * G + lane) * a.nsplit + split) * (D + 2);
+    float mv = 0.f, lv = 0.f;
+#pragma unroll
+    for (int g = 0; g < GT; g++) {     // pick this lane's head without dynamic register indexing
+      if (g == lane) { mv = m_run[g]; lv = l_run[g]; }
+    }
+    w[D] = mv;
+    w[D + 1] = lv;
   }
+  DH_ATS();
+#ifdef DH_ATTN_TRACE
+  if (tid == DH_ATTN_TRACE) tsbuf[31] = tsn;
+#endif
 }
 
 // One workgroup per query head: out[d] = sum_s e^{m_s - M} o_s[d] / sum_s e^{m_s - M} l_s.
@@ -250,13 +339,17 @@ int max_splits_for(int kv_len) { return std::max(1, (kv_len + kTileKeys - 1) / k
 
 int choose_splits(int Hkv, int nkeys) {
   const int tiles = std::max(1, (nkeys + kTileKeys - 1) / kTileKeys);
-  const int want = std::max(1, 1024 / std::max(1, Hkv));   // aim for ~4 workgroups per CU
+  const int want = std::max(1, 1024 / std::max(1, Hkv));   // at most ~4 workgroups per CU
   return std::min(tiles, want);
 }
 
 template <int D>
 int launch(const AttnArgs& a, const char* op) {
-  hipLaunchKernelGGL(attn_decode_split_kernel<D>, dim3(a.Hkv, a.nsplit), dim3(256), 0, dh::stream(), a);
+  const dim3 grid(a.Hkv, a.nsplit), block(256);
+  if (a.G <= 1) hipLaunchKernelGGL((attn_decode_split_kernel<D, 1>), grid, block, 0, dh::stream(), a);
+  else if (a.G <= 2) hipLaunchKernelGGL((attn_decode_split_kernel<D, 2>), grid, block, 0, dh::stream(), a);
+  else if (a.G <= 4) hipLaunchKernelGGL((attn_decode_split_kernel<D, 4>), grid, block, 0, dh::stream(), a);
+  else hipLaunchKernelGGL((attn_decode_split_kernel<D, 8>), grid, block, 0, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   if (a.nsplit > 1) {
     hipLaunchKernelGGL(attn_decode_merge_kernel<D>, dim3(a.H), dim3(D), 0, dh::stream(), a.ws, a.O, a.nsplit);
@@ -266,6 +359,12 @@ int launch(const AttnArgs& a, const char* op) {
 }
 
 }  // namespace
+
+#ifdef DH_ATTN_TRACE
+extern "C" int dh_debug_attn_trace(void* host_dst) {
+  return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(dh_attn_trace_buf), sizeof(dh_attn_trace_buf));
+}
+#endif
 
 extern "C" {
 
@@ -314,10 +413,9 @@ int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_
   a.H = H; a.Hkv = Hkv; a.G = G;
   a.kbeg = (int)kbeg; a.kend = (int)kend;
   const int nkeys = (int)(kend - kbeg);
-  int nsplit = choose_splits(Hkv, nkeys);
-  const int tiles = (nkeys + kTileKeys - 1) / kTileKeys;
-  a.tiles_per_split = (tiles + nsplit - 1) / nsplit;
-  nsplit = (tiles + a.tiles_per_split - 1) / a.tiles_per_split;   // no empty splits
+  // workgroup (kv head, split) walks chunks split, split + nsplit, ...: never an empty split
+  const int nsplit = choose_splits(Hkv, nkeys);
+  a.tiles_per_split = 0;
   a.nsplit = nsplit;
   if (nsplit > 1 && !d_workspace) return dh::fail(1, "[%s] workspace is required", op);
   a.scale = scale; a.softcap = softcap;
