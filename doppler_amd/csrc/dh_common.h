@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <type_traits>
 
 #include "../../include/doppler_hip.h"
 
@@ -25,6 +26,25 @@ int num_cus();
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 }  // namespace dh
+
+#ifdef __HIPCC__
+namespace dh {
+// Sum over the 64 lanes of a wave, returned wave-uniform: DPP row shifts inside each 16-lane
+// row (no LDS traffic), then the four row totals travel through scalar registers.
+__device__ __forceinline__ float wave_sum_uniform(float v) {
+  auto shr = [](float x, auto ctrl) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value, 0xF, 0xF, false));
+  };
+  v += shr(v, std::integral_constant<int, 0x111>{});
+  v += shr(v, std::integral_constant<int, 0x112>{});
+  v += shr(v, std::integral_constant<int, 0x114>{});
+  v += shr(v, std::integral_constant<int, 0x118>{});
+  const int b = __float_as_int(v);
+  return (__int_as_float(__builtin_amdgcn_readlane(b, 15)) + __int_as_float(__builtin_amdgcn_readlane(b, 31))) +
+         (__int_as_float(__builtin_amdgcn_readlane(b, 47)) + __int_as_float(__builtin_amdgcn_readlane(b, 63)));
+}
+}  // namespace dh
+#endif
 
 #define DH_REQUIRE_INIT(op)                                                     \
   do {                                                                          \

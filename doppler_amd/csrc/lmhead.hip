@@ -68,6 +68,63 @@ struct F16GemvArgs {
   uint32_t* part_idx;
 };
 
+// M = 1, K <= 4096: every lane meets the same 64 activations in every row (its eight 16-byte
+// chunks sit at fixed k), so they live in registers for the whole kernel: no LDS at all.
+template <bool ARGMAX>
+__global__ __launch_bounds__(256) void f16w_gemv_xreg_kernel(const F16GemvArgs a) {
+  __shared__ float sv[4];
+  __shared__ uint32_t si[4];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int kvec = a.K >> 3;
+  float x[8][8];
+#pragma unroll
+  for (int u = 0; u < 8; u++) {
+    const int v = lane + 64 * u;
+    float4 xa = make_float4(0.f, 0.f, 0.f, 0.f), xb = xa;
+    if (v < kvec) {
+      xa = *reinterpret_cast<const float4*>(a.A + v * 8);
+      xb = *reinterpret_cast<const float4*>(a.A + v * 8 + 4);
+    }
+    x[u][0] = xa.x; x[u][1] = xa.y; x[u][2] = xa.z; x[u][3] = xa.w;
+    x[u][4] = xb.x; x[u][5] = xb.y; x[u][6] = xb.z; x[u][7] = xb.w;
+  }
+  Cand best{-3.402823e+38f, 0xFFFFFFFFu};   // only lane 0 ever updates its candidate
+  for (int r = 0; r < a.rows_per_wave; r++) {
+    const int64_t row = ((int64_t)r * gridDim.x + blockIdx.x) * 4 + wave;
+    if (row >= a.N) break;   // wave-uniform
+    const uint4* wrow = reinterpret_cast<const uint4*>(a.W + row * a.K);
+    uint4 raw[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int v = lane + 64 * u;
+      raw[u] = v < kvec ? wrow[v] : make_uint4(0, 0, 0, 0);
+    }
+    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const __half2* h2 = reinterpret_cast<const __half2*>(&raw[u]);
+      const float2 w0 = __half22float2(h2[0]), w1 = __half22float2(h2[1]);
+      const float2 w2 = __half22float2(h2[2]), w3 = __half22float2(h2[3]);
+      s0 = fmaf(x[u][0], w0.x, s0); s1 = fmaf(x[u][1], w0.y, s1);
+      s0 = fmaf(x[u][2], w1.x, s0); s1 = fmaf(x[u][3], w1.y, s1);
+      s0 = fmaf(x[u][4], w2.x, s0); s1 = fmaf(x[u][5], w2.y, s1);
+      s0 = fmaf(x[u][6], w3.x, s0); s1 = fmaf(x[u][7], w3.y, s1);
+    }
+    const float logit = dh::wave_sum_uniform(s0 + s1) * a.alpha;
+    if (lane == 0) {
+      if (a.C) a.C[row] = logit;
+      if (ARGMAX && row != a.pad_id) {
+        const float v = softcap_f(logit, a.softcap);
+        if (beats(v, (uint32_t)row, best.v, best.i)) { best.v = v; best.i = (uint32_t)row; }
+      }
+    }
+  }
+  if (ARGMAX) {
+    const Cand c = block_best_256(best, sv, si);
+    if (tid == 0) { a.part_val[blockIdx.x] = c.v; a.part_idx[blockIdx.x] = c.i; }
+  }
+}
+
 template <int MT, bool ARGMAX>
 __global__ __launch_bounds__(256) void f16w_gemv_kernel(const F16GemvArgs a) {
   extern __shared__ float xs[];   // [MT][K]
@@ -78,38 +135,46 @@ __global__ __launch_bounds__(256) void f16w_gemv_kernel(const F16GemvArgs a) {
   __syncthreads();
 
   const int kvec = a.K >> 3;
-  const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * a.rows_per_wave;
+  // rows are dealt round-robin over all waves of the grid: at any moment the whole chip reads
+  // one contiguous band of the matrix, which keeps every HBM channel busy
   Cand best{-3.402823e+38f, 0xFFFFFFFFu};   // only lane 0 ever updates its candidate
   for (int r = 0; r < a.rows_per_wave; r++) {
-    const int64_t row = row0 + r;
+    const int64_t row = ((int64_t)r * gridDim.x + blockIdx.x) * 4 + wave;
     if (row >= a.N) break;   // wave-uniform
     const uint4* wrow = reinterpret_cast<const uint4*>(a.W + row * a.K);
     float acc[MT];
 #pragma unroll
     for (int m = 0; m < MT; m++) acc[m] = 0.f;
-    for (int v = lane; v < kvec; v += 64) {
-      const uint4 raw = wrow[v];
-      const __half2* h2 = reinterpret_cast<const __half2*>(&raw);
-      const float2 w0 = __half22float2(h2[0]), w1 = __half22float2(h2[1]);
-      const float2 w2 = __half22float2(h2[2]), w3 = __half22float2(h2[3]);
+    // eight 16-byte loads per lane go out before any of them is used (4 KB of the row per wave)
+    for (int v0 = lane; v0 < kvec; v0 += 8 * 64) {
+      uint4 raw[8];
 #pragma unroll
-      for (int m = 0; m < MT; m++) {
-        const float4 xa = *reinterpret_cast<const float4*>(xs + m * a.K + v * 8);
-        const float4 xb = *reinterpret_cast<const float4*>(xs + m * a.K + v * 8 + 4);
-        float s = acc[m];
-        s = fmaf(xa.x, w0.x, s); s = fmaf(xa.y, w0.y, s);
-        s = fmaf(xa.z, w1.x, s); s = fmaf(xa.w, w1.y, s);
-        s = fmaf(xb.x, w2.x, s); s = fmaf(xb.y, w2.y, s);
-        s = fmaf(xb.z, w3.x, s); s = fmaf(xb.w, w3.y, s);
-        acc[m] = s;
+      for (int u = 0; u < 8; u++) {
+        const int v = v0 + 64 * u;
+        raw[u] = v < kvec ? wrow[v] : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int v = min(v0 + 64 * u, kvec - 1);      // zero weights past the row: any x will do
+        const __half2* h2 = reinterpret_cast<const __half2*>(&raw[u]);
+        const float2 w0 = __half22float2(h2[0]), w1 = __half22float2(h2[1]);
+        const float2 w2 = __half22float2(h2[2]), w3 = __half22float2(h2[3]);
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+          const float4 xa = *reinterpret_cast<const float4*>(xs + m * a.K + v * 8);
+          const float4 xb = *reinterpret_cast<const float4*>(xs + m * a.K + v * 8 + 4);
+          float s = acc[m];
+          s = fmaf(xa.x, w0.x, s); s = fmaf(xa.y, w0.y, s);
+          s = fmaf(xa.z, w1.x, s); s = fmaf(xa.w, w1.y, s);
+          s = fmaf(xb.x, w2.x, s); s = fmaf(xb.y, w2.y, s);
+          s = fmaf(xb.z, w3.x, s); s = fmaf(xb.w, w3.y, s);
+          acc[m] = s;
+        }
       }
     }
 #pragma unroll
     for (int m = 0; m < MT; m++) {
-      float s = acc[m];
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-      acc[m] = s * a.alpha;
+      acc[m] = dh::wave_sum_uniform(acc[m]) * a.alpha;
     }
     if (lane == 0) {
       if (a.C) {
@@ -175,7 +240,10 @@ int launch_gemv(F16GemvArgs a, int* parts_out, const char* op) {
   int grid = (int)dh::ceil_div(a.N, (int64_t)4 * rpw);
   while (grid > kMaxParts) { rpw++; grid = (int)dh::ceil_div(a.N, (int64_t)4 * rpw); }
   a.rows_per_wave = rpw;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, dh::stream(), a);
+  if (MT == 1 && a.K <= 4096 && (reinterpret_cast<uintptr_t>(a.A) & 15) == 0)
+    hipLaunchKernelGGL(f16w_gemv_xreg_kernel<ARGMAX>, dim3(grid), dim3(256), 0, dh::stream(), a);
+  else
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   if (parts_out) *parts_out = grid;
   return 0;
