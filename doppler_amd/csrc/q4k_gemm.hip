@@ -1,0 +1,272 @@
+// Q4_K prefill GEMM for gfx950: C[M,N] = alpha * A[M,K] . dequant(W)[N,K]^T for M >= 16, and
+// the fused gate/up projection with gated activation, on the matrix cores.
+//
+// Tile: 128 (M) x 128 (N) per workgroup of 4 waves, each wave a 64 x 64 quadrant computed with
+// v_mfma_f32_32x32x16_f16 (2 x 2 MFMA tiles, f32 accumulators).  K advances 64 at a time: one
+// 32-byte nibble chunk of a super-block (low nibbles = sub-block 2c, high = 2c+1) per weight row.
+//   weights  thread (row, half) loads 16 nibble bytes + the block header, rebuilds 32 weights
+//            as f16: (w & 0x000F000F) | 0x64006400 is the pair (1024 + q) in f16, one packed
+//            subtract and one packed fma with (d*sc, -dmin*mn) finish them: about 2 vector ops
+//            per weight, paid once per 128 rows of A.
+//   A        f32 -> f16 on the way into LDS.
+// Both tiles sit in LDS as [row][64 k] with a 16-byte pad (conflict-free 16-byte fragment
+// reads) and are double-buffered: the global loads of tile t+1 are issued before tile t is
+// multiplied, one barrier per K step.
+// k order inside every group of 4 is (0, 2, 1, 3) in BOTH tiles: that is the order the masked
+// nibble pairs come out in, and a contraction index may be permuted freely when both operands
+// agree.
+#include <algorithm>
+
+#include "dh_common.h"
+#include "q4k_device.h"
+
+namespace {
+
+using dh::kBlockBytes;
+using dh::kQK;
+
+typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
+typedef __attribute__((ext_vector_type(16))) float float16_t;
+
+constexpr int BK = 64;
+constexpr int LDS_ROW = BK + 8;                    // halves per LDS row (144 bytes)
+
+struct GemmArgs {
+  const float* A;        // [M][K]
+  const uint8_t* W;      // Q4_K rows [N][nb*144]
+  const uint8_t* W2;     // second matrix (DUAL) or null
+  void* C;               // [M][N] f32 or f16
+  const float* residual; // [M][N] or null
+  int M, N, K, nb;
+  float alpha;
+  int c_f16, activation;
+  float clamp_max;
+};
+
+// 16 nibble bytes -> 16 low-nibble and 16 high-nibble weights as f16, k order (0,2,1,3) per dword.
+__device__ __forceinline__ void dequant16(const uint4 q, float sc_lo, float mn_lo, float sc_hi, float mn_hi,
+                                          uint4 (&lo)[2], uint4 (&hi)[2]) {
+  const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+  const half2_t k1024 = {(_Float16)1024.f, (_Float16)1024.f};
+  const half2_t slo = {(_Float16)sc_lo, (_Float16)sc_lo}, mlo = {(_Float16)-mn_lo, (_Float16)-mn_lo};
+  const half2_t shi = {(_Float16)sc_hi, (_Float16)sc_hi}, mhi = {(_Float16)-mn_hi, (_Float16)-mn_hi};
+  uint32_t lo_w[8], hi_w[8];
+#pragma unroll
+  for (int d = 0; d < 4; d++) {
+    const uint32_t p[4] = {(w[d] & 0x000F000Fu) | 0x64006400u, ((w[d] >> 8) & 0x000F000Fu) | 0x64006400u,
+                           ((w[d] >> 4) & 0x000F000Fu) | 0x64006400u, ((w[d] >> 12) & 0x000F000Fu) | 0x64006400u};
+    half2_t v[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[i] = __builtin_bit_cast(half2_t, p[i]) - k1024;     // exact: q
+    lo_w[2 * d] = __builtin_bit_cast(uint32_t, v[0] * slo + mlo);
+    lo_w[2 * d + 1] = __builtin_bit_cast(uint32_t, v[1] * slo + mlo);
+    hi_w[2 * d] = __builtin_bit_cast(uint32_t, v[2] * shi + mhi);
+    hi_w[2 * d + 1] = __builtin_bit_cast(uint32_t, v[3] * shi + mhi);
+  }
+  lo[0] = make_uint4(lo_w[0], lo_w[1], lo_w[2], lo_w[3]);
+  lo[1] = make_uint4(lo_w[4], lo_w[5], lo_w[6], lo_w[7]);
+  hi[0] = make_uint4(hi_w[0], hi_w[1], hi_w[2], hi_w[3]);
+  hi[1] = make_uint4(hi_w[4], hi_w[5], hi_w[6], hi_w[7]);
+}
+
+// tanh-form GELU with tanh(t) = 1 - 2 / (1 + e^{2t}): a handful of instructions, inlined once per
+// accumulator element in the epilogue.
+__device__ __forceinline__ float gelu_tanh_fast(float x) {
+  const float t = fminf(fmaxf(0.7978845608f * (x + 0.044715f * x * x * x), -15.0f), 15.0f);
+  return 0.5f * x * (2.0f - 2.0f / (1.0f + __expf(2.0f * t)));
+}
+
+// T = MFMA tiles per wave along each of M and N: workgroup tile 64T x 64T (T = 2: 128 x 128 for
+// large problems, T = 1: 64 x 64 when a 128-tiling would leave most compute units idle).
+template <bool DUAL, int T>
+__global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
+  constexpr int NMAT = DUAL ? 2 : 1;
+  constexpr int BM = 64 * T, BN = 64 * T;
+  constexpr int A_HALVES = BM * LDS_ROW, B_HALVES = BN * LDS_ROW;
+  extern __shared__ __align__(16) _Float16 lds[];            // [2 buffers][A | B | (B2)]
+  constexpr int BUF_HALVES = A_HALVES + NMAT * B_HALVES;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int wm = (wave >> 1) * 32 * T, wn = (wave & 1) * 32 * T;     // the wave's quadrant
+  const int fr = lane & 31, fg = lane >> 5;                  // fragment row / k half
+  const int64_t row_bytes = (int64_t)a.nb * kBlockBytes;
+  const int nkt = (a.K + BK - 1) / BK;
+
+  // ---- global -> register staging roles
+  // A: 8 float4 per thread, idx = tid + 256 i: row idx >> 4, k 4 * (idx & 15)
+  // W: thread (row tid >> 1, half tid & 1): 16 nibble bytes + header
+  const int w_row = tid >> 1, w_half = tid & 1;
+  const int64_t w_off = (int64_t)min(n0 + w_row, a.N - 1) * row_bytes;
+  constexpr int NA = BM * 16 / 256;                          // float4 loads of A per thread
+  const bool w_active = w_row < BN;
+  float4 a_reg[NA];
+  uint4 q_reg[NMAT], h_reg[NMAT];
+
+  auto load_tile = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < NA; i++) {
+      const int idx = tid + 256 * i, r = idx >> 4, k = kt * BK + 4 * (idx & 15);
+      const int m = min(m0 + r, a.M - 1);
+      a_reg[i] = k < a.K ? *reinterpret_cast<const float4*>(a.A + (int64_t)m * a.K + k)
+                             : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    const int blk = kt >> 2, c = kt & 3;
+#pragma unroll
+    for (int mt = 0; mt < NMAT; mt++) {
+      if (w_active) {
+        const uint8_t* bp = (mt ? a.W2 : a.W) + w_off + (int64_t)blk * kBlockBytes;
+        h_reg[mt] = *reinterpret_cast<const uint4*>(bp);
+        q_reg[mt] = *reinterpret_cast<const uint4*>(bp + 16 + 32 * c + 16 * w_half);
+      }
+    }
+  };
+  auto store_tile = [&](int kt, int buf) {
+    _Float16* At = lds + buf * BUF_HALVES;
+#pragma unroll
+    for (int i = 0; i < NA; i++) {
+      const int idx = tid + 256 * i, r = idx >> 4, kl = 4 * (idx & 15);
+      const half2_t p0 = {(_Float16)a_reg[i].x, (_Float16)a_reg[i].z};    // k order (0, 2, 1, 3)
+      const half2_t p1 = {(_Float16)a_reg[i].y, (_Float16)a_reg[i].w};
+      *reinterpret_cast<uint2*>(At + r * LDS_ROW + kl) =
+          make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+    }
+    const int c = kt & 3;
+#pragma unroll
+    for (int mt = 0; mt < NMAT; mt++) {
+      if (!w_active) break;
+      float sc_lo, sc_hi, mn_lo, mn_hi;
+      q4k_pair_scales(h_reg[mt], c, sc_lo, sc_hi, mn_lo, mn_hi);
+      uint4 lo[2], hi[2];
+      dequant16(q_reg[mt], sc_lo, mn_lo, sc_hi, mn_hi, lo, hi);
+      _Float16* Bt = lds + buf * BUF_HALVES + A_HALVES + mt * B_HALVES + w_row * LDS_ROW;
+      *reinterpret_cast<uint4*>(Bt + 16 * w_half) = lo[0];
+      *reinterpret_cast<uint4*>(Bt + 16 * w_half + 8) = lo[1];
+      *reinterpret_cast<uint4*>(Bt + 32 + 16 * w_half) = hi[0];
+      *reinterpret_cast<uint4*>(Bt + 32 + 16 * w_half + 8) = hi[1];
+    }
+  };
+
+  float16_t acc[NMAT][T][T];
+#pragma unroll
+  for (int mt = 0; mt < NMAT; mt++)
+#pragma unroll
+    for (int i = 0; i < T; i++)
+#pragma unroll
+      for (int j = 0; j < T; j++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[mt][i][j][e] = 0.f;
+
+  load_tile(0);
+  store_tile(0, 0);
+  __syncthreads();
+  for (int kt = 0; kt < nkt; kt++) {
+    const int buf = kt & 1;
+    if (kt + 1 < nkt) load_tile(kt + 1);
+    const _Float16* At = lds + buf * BUF_HALVES;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      half8_t af[T], bf[NMAT][T];
+#pragma unroll
+      for (int i = 0; i < T; i++)
+        af[i] = *reinterpret_cast<const half8_t*>(At + (wm + 32 * i + fr) * LDS_ROW + 16 * ks + 8 * fg);
+#pragma unroll
+      for (int mt = 0; mt < NMAT; mt++)
+#pragma unroll
+        for (int j = 0; j < T; j++)
+          bf[mt][j] = *reinterpret_cast<const half8_t*>(At + A_HALVES + mt * B_HALVES + (wn + 32 * j + fr) * LDS_ROW +
+                                                        16 * ks + 8 * fg);
+#pragma unroll
+      for (int mt = 0; mt < NMAT; mt++)
+#pragma unroll
+        for (int i = 0; i < T; i++)
+#pragma unroll
+          for (int j = 0; j < T; j++)
+            acc[mt][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[mt][j], acc[mt][i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nkt) store_tile(kt + 1, buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds column n = lane & 31 of rows 8 (e / 4) + 4 fg + (e % 4)
+#pragma unroll
+  for (int i = 0; i < T; i++)
+#pragma unroll
+    for (int j = 0; j < T; j++) {
+      const int n = n0 + wn + 32 * j + fr;
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        const int m = m0 + wm + 32 * i + 8 * (e >> 2) + 4 * fg + (e & 3);
+        if (m < a.M && n < a.N) {
+          float v;
+          if (DUAL) {
+            const float g = acc[0][i][j][e], u = acc[NMAT - 1][i][j][e];
+            v = (a.activation == DH_ACT_SILU ? act_silu(g) : gelu_tanh_fast(g)) * u * a.alpha;
+            if (a.activation == DH_ACT_SILU && a.clamp_max > 0.f) v = fminf(fmaxf(v, -a.clamp_max), a.clamp_max);
+          } else {
+            v = acc[0][i][j][e] * a.alpha;
+            if (a.residual) v += a.residual[(int64_t)m * a.N + n];
+          }
+          if (a.c_f16)
+            reinterpret_cast<__half*>(a.C)[(int64_t)m * a.N + n] = __float2half(v);
+          else
+            reinterpret_cast<float*>(a.C)[(int64_t)m * a.N + n] = v;
+        }
+      }
+    }
+}
+
+template <bool DUAL, int T>
+int launch_gemm_cfg(const GemmArgs& a, const char* op) {
+  constexpr int BM = 64 * T, BN = 64 * T;
+  const size_t lds = (size_t)2 * (DUAL ? 3 : 2) * BM * LDS_ROW * sizeof(_Float16);
+  auto kern = q4k_gemm_kernel<DUAL, T>;
+  static bool attr_set = false;   // once per instantiation: the call costs microseconds
+  if (!attr_set) {
+    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attr_set = true;
+  }
+  const dim3 grid((unsigned)dh::ceil_div(a.N, BN), (unsigned)dh::ceil_div(a.M, BM));
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, dh::stream(), a);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+// 128 x 128 tiles when they occupy at least half of the compute units (their higher matrix-core
+// share wins from there on), else 64 x 64.
+template <bool DUAL>
+int launch_gemm(const GemmArgs& a, const char* op) {
+  const int64_t big_tiles = dh::ceil_div(a.M, 128) * dh::ceil_div(a.N, 128);
+  if (2 * big_tiles >= dh::num_cus()) return launch_gemm_cfg<DUAL, 2>(a, op);
+  return launch_gemm_cfg<DUAL, 1>(a, op);
+}
+
+}  // namespace
+
+namespace dh {
+
+bool q4k_gemm_serves(int M, int K, const void* A) {
+  return M >= 16 && (K % 4) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0;
+}
+
+int q4k_gemm(const char* op, const float* A, const uint8_t* W, void* C, int c_f16, int M, int N, int K,
+             float alpha, const float* residual) {
+  GemmArgs a{};
+  a.A = A; a.W = W; a.W2 = nullptr; a.C = C; a.residual = residual;
+  a.M = M; a.N = N; a.K = K; a.nb = (K + kQK - 1) / kQK;
+  a.alpha = alpha; a.c_f16 = c_f16;
+  return launch_gemm<false>(a, op);
+}
+
+int q4k_gemm_gate_up(const char* op, const float* A, const uint8_t* Wg, const uint8_t* Wu, float* C, int M,
+                     int hidden, int inter, int activation, float alpha, float clamp_max) {
+  GemmArgs a{};
+  a.A = A; a.W = Wg; a.W2 = Wu; a.C = C; a.residual = nullptr;
+  a.M = M; a.N = inter; a.K = hidden; a.nb = (hidden + kQK - 1) / kQK;
+  a.alpha = alpha; a.c_f16 = 0; a.activation = activation; a.clamp_max = clamp_max;
+  return launch_gemm<true>(a, op);
+}
+
+}  // namespace dh

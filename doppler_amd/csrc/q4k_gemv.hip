@@ -16,42 +16,12 @@
 #include <cstdlib>
 
 #include "dh_common.h"
+#include "q4k_device.h"
 
 namespace {
 
 using dh::kBlockBytes;
 using dh::kQK;
-
-__device__ __forceinline__ float f16lo(uint32_t v) {
-  return __half2float(__ushort_as_half((unsigned short)(v & 0xffffu)));
-}
-__device__ __forceinline__ float f16hi(uint32_t v) {
-  return __half2float(__ushort_as_half((unsigned short)(v >> 16)));
-}
-
-// Scales and mins of sub-blocks 2c and 2c+1 from the 16-byte block header.
-// Bytes 4..7 (hdr.y): low 6 bits = scale 0..3, top 2 bits = high bits of scale 4..7.
-// Bytes 8..11 (hdr.z): same for mins.  Bytes 12..15 (hdr.w): low nibble = scale 4..7 low
-// bits, high nibble = min 4..7 low bits.
-__device__ __forceinline__ void q4k_pair_scales(const uint4 hdr, const int c, float& sc_lo,
-                                                float& sc_hi, float& mn_lo, float& mn_hi) {
-  const float d = f16lo(hdr.x);
-  const float dmin = f16hi(hdr.x);
-  const int sh = (c & 1) * 16;
-  const uint32_t a1 = hdr.y >> sh, a2 = hdr.z >> sh, a3 = hdr.w >> sh;
-  uint32_t scp, mnp;
-  if (c < 2) {
-    scp = a1 & 0x3F3Fu;
-    mnp = a2 & 0x3F3Fu;
-  } else {
-    scp = (a3 & 0x0F0Fu) | ((a1 >> 2) & 0x3030u);
-    mnp = ((a3 >> 4) & 0x0F0Fu) | ((a2 >> 2) & 0x3030u);
-  }
-  sc_lo = d * (float)(scp & 0xFFu);
-  sc_hi = d * (float)((scp >> 8) & 0xFFu);
-  mn_lo = dmin * (float)(mnp & 0xFFu);
-  mn_hi = dmin * (float)((mnp >> 8) & 0xFFu);
-}
 
 // ---------------------------------------------------------------------------------------
 // Dequantise to f32, bit-exact: w = scale*q - min is the correctly rounded f32 of the exact
@@ -99,12 +69,6 @@ struct GemvArgs {
   int activation;       // DUAL: DH_ACT_SILU / DH_ACT_GELU
   float clamp_max;      // DUAL + silu: 0 = off
 };
-
-__device__ __forceinline__ float act_silu(float x) { return x / (1.0f + __expf(-x)); }
-__device__ __forceinline__ float act_gelu(float x) {
-  const float inner = 0.7978845608f * (x + 0.044715f * x * x * x);
-  return 0.5f * x * (1.0f + tanhf(fminf(fmaxf(inner, -15.0f), 15.0f)));
-}
 
 template <int MT>
 __device__ __forceinline__ void q4k_block_chunk_dot(const uint8_t* __restrict__ blk_ptr, const int c,
@@ -975,6 +939,8 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
   if (normed)
     return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 and K <= 14336 only (M=%d, K=%d); "
                     "run dh_rmsnorm and dh_q4k_matmul instead", op, M, K);
+  if (path != 2 && dh::q4k_gemm_serves(M, K, d_A))
+    return dh::q4k_gemm(op, a.A, a.W, d_C, a.c_f16, M, N, K, alpha, a.residual);
   // tiles of up to 8 activation rows per pass over the weights
   const size_t c_elem = a.c_f16 ? 2 : 4;
   for (int m0 = 0; m0 < M; m0 += 8) {
@@ -1042,6 +1008,8 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
   if (normed)
     return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 and hidden <= 14336 only (M=%d, hidden=%d); "
                     "run dh_rmsnorm and dh_q4k_ffn_gate_up instead", op, M, hidden);
+  if (path != 2 && dh::q4k_gemm_serves(M, hidden, d_x))
+    return dh::q4k_gemm_gate_up(op, d_x, a.W, a.W2, d_out, M, hidden, inter, activation, alpha, swiglu_limit);
   // any batch: tiles of up to 8 activation rows per pass
   for (int m0 = 0; m0 < M; m0 += 8) {
     GemvArgs b = a;
