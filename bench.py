@@ -25,6 +25,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per fused gate/up launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs, scaled
+# by the same counters' readings for a cast kernel of known traffic (x2.000 and x1.000):
+# 55,718 KiB fetched + 48 KiB written.
+GATE_UP_TRAFFIC_BYTES = 57104000
 
 
 def log(*a):
@@ -74,6 +78,9 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="debug only: fewer layers (result is not the metric)")
     ap.add_argument("--prefill", type=int, default=None, help="debug only: shorter prefill")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three f32->f16 casts of 16 Mi elements (64 MiB read, 32 MiB written): a "
+                         "streaming kernel of known traffic to scale rocprofv3 FETCH_SIZE / WRITE_SIZE with")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (single-stream decode has nothing to shard in this tier); "
@@ -142,7 +149,17 @@ def main():
     achieved = launch_bytes / (avg_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": "q4k fused RMSNorm + gate/up GEMV + SiLU [2x12288x4096]", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "bytes_per_launch": launch_bytes, "avg_launch_us": round(avg_ms * 1e3, 2), "traffic": None}
+                "bytes_per_launch": launch_bytes, "avg_launch_us": round(avg_ms * 1e3, 2),
+                "traffic": GATE_UP_TRAFFIC_BYTES if (Hd, I) == (4096, 12288) else None}
+
+    if args.copy_calibration:
+        # a streaming kernel of known traffic: reads 64 MiB of f32, writes 32 MiB of f16
+        from doppler_amd import capi as _capi
+        src = torch.ones(16 << 20, dtype=torch.float32, device="cuda")
+        dst = torch.empty(16 << 20, dtype=torch.float16, device="cuda")
+        for _ in range(3):
+            _capi.check(dec.L.dh_cast_f32_to_f16(src.data_ptr(), dst.data_ptr(), src.numel()))
+        capi_sync()
 
     # ---- CPU baseline: the oracle's decode step (a restatement of the reference's JS per-op
     #      references) on this host, same weights, same KV
