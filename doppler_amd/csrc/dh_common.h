@@ -22,6 +22,12 @@ int fail(int code, const char* fmt, ...);
 hipStream_t stream();
 bool ready();
 int num_cus();
+// State of the chained-GEMV grid barrier, owned by the runtime (allocated by dh_init): eight
+// monotonic counters 256 bytes apart, an error flag the kernel raises when a barrier times out,
+// and the host's copy of the counters' value.  chain_advance(n) returns that value and adds n.
+unsigned* chain_counters();
+unsigned* chain_error_flag();
+unsigned chain_advance(unsigned n);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

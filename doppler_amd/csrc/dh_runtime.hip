@@ -12,6 +12,9 @@ int g_device = -1;
 hipStream_t g_own_stream = nullptr;
 hipStream_t g_stream = nullptr;
 int g_num_cus = 0;
+unsigned* g_chain_mem = nullptr;     // [8 * 64] barrier counters + [1] error flag
+unsigned g_chain_value = 0;          // what every counter reads once the enqueued launches are done
+constexpr size_t kChainWords = 8 * 64 + 64;
 }  // namespace
 
 namespace dh {
@@ -25,6 +28,13 @@ int fail(int code, const char* fmt, ...) {
 hipStream_t stream() { return g_stream; }
 bool ready() { return g_ready; }
 int num_cus() { return g_num_cus; }
+unsigned* chain_counters() { return g_chain_mem; }
+unsigned* chain_error_flag() { return g_chain_mem ? g_chain_mem + 8 * 64 : nullptr; }
+unsigned chain_advance(unsigned n) {
+  const unsigned v = g_chain_value;
+  g_chain_value += n;
+  return v;
+}
 }  // namespace dh
 
 extern "C" {
@@ -51,6 +61,9 @@ int dh_init(int device_ordinal) {
   DH_CHECK_HIP("dh_init", hipStreamCreateWithFlags(&g_own_stream, hipStreamDefault));
   g_stream = g_own_stream;
   g_num_cus = prop.multiProcessorCount;
+  DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_chain_mem), kChainWords * sizeof(unsigned)));
+  DH_CHECK_HIP("dh_init", hipMemset(g_chain_mem, 0, kChainWords * sizeof(unsigned)));
+  g_chain_value = 0;
   g_device = device_ordinal;
   g_ready = true;
   return 0;
@@ -61,6 +74,8 @@ int dh_shutdown(void) {
   if (!g_ready) return 0;
   DH_CHECK_HIP("dh_shutdown", hipStreamSynchronize(g_stream));
   if (g_own_stream) DH_CHECK_HIP("dh_shutdown", hipStreamDestroy(g_own_stream));
+  if (g_chain_mem) DH_CHECK_HIP("dh_shutdown", hipFree(g_chain_mem));
+  g_chain_mem = nullptr;
   g_own_stream = nullptr;
   g_stream = nullptr;
   g_ready = false;
@@ -177,6 +192,17 @@ int dh_event_destroy(void* ev) {
 int dh_sync(void) {
   DH_REQUIRE_INIT("dh_sync");
   DH_CHECK_HIP("dh_sync", hipStreamSynchronize(g_stream));
+  if (g_chain_mem) {
+    // a chained GEMV that could not cross its grid barrier left its outputs incomplete
+    unsigned flag = 0;
+    DH_CHECK_HIP("dh_sync", hipMemcpy(&flag, g_chain_mem + 8 * 64, sizeof(flag), hipMemcpyDeviceToHost));
+    if (flag) {
+      DH_CHECK_HIP("dh_sync", hipMemset(g_chain_mem, 0, kChainWords * sizeof(unsigned)));
+      g_chain_value = 0;
+      return dh::fail(3, "[dh_sync] a chained GEMV launch timed out at its grid barrier (workgroups not all "
+                      "resident); its outputs are invalid");
+    }
+  }
   return 0;
 }
 

@@ -13,6 +13,7 @@ All buffers are allocated once; a step enqueues ~8 launches per layer on the lib
 stream and reads back one token id, the reference's only device->host crossing per token.
 """
 import ctypes
+import os
 import math
 
 import numpy as np
@@ -30,14 +31,22 @@ def _dev_bytes(arr):
     return t
 
 
+def c_hidden_ok(cfg):
+    """The chained kernel holds one activation row in LDS: rows up to 12288 elements."""
+    return max(cfg["hidden"], cfg["inter"], cfg["heads"] * cfg["head_dim"]) <= 12288
+
+
 class HipDecoder:
-    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True):
+    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True, chain=True):
         """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
         layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
         input_norm, post_attn_norm, q_norm, k_norm: f32); embed_bits: uint16 [vocab, hidden]."""
         self.cfg = dict(cfg)
         # RMSNorm runs inside the q/k/v and gate/up GEMVs (their prologue) unless told otherwise
         self.fuse_norm = fuse_norm
+        # the GEMVs between two attentions (o_proj, gate/up, down, next q/k/v) as one persistent launch
+        self.chain = chain and fuse_norm and c_hidden_ok(cfg) and os.environ.get("DH_DECODE_CHAIN", "1") == "1"
+        self._chains = None
         self.L = capi.init(torch.cuda.current_device())
         c = self.cfg
         self.max_seq = max_seq
@@ -99,6 +108,8 @@ class HipDecoder:
         ids = self.token if from_device_token else self.ids
         ck(L.dh_gather_f16(ids.data_ptr(), self.embed.data_ptr(), self.x.data_ptr(), 1, Hd, c["vocab"], 0))
         x, x2 = self.x, self.x2
+        if self.chain:
+            return self._enqueue_chained(pos, want_logits)
         for d in self.layers:
             if self.fuse_norm:
                 ck(L.dh_q4k_matmul_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), c["eps"], 0,
@@ -131,6 +142,57 @@ class HipDecoder:
                                1.0, x2.data_ptr()))
         ck(L.dh_rmsnorm(x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"],
                         0, None, None, None, 1.0))
+        ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
+                                  self.lm_ws.data_ptr(), self.token.data_ptr(), 0,
+                                  self.logits.data_ptr() if want_logits else None))
+
+    def _build_chains(self):
+        """One dh_gemv_phase array per layer: o_proj (+residual) -> RMSNorm + gate/up + SiLU ->
+        down (+residual) -> RMSNorm + the NEXT layer's stacked q/k/v projection."""
+        c = self.cfg
+        Hd, I = c["hidden"], c["inter"]
+        chains = []
+        for li, d in enumerate(self.layers):
+            nxt = self.layers[li + 1] if li + 1 < len(self.layers) else None
+            arr = (capi.GemvPhase * (4 if nxt else 3))()
+
+            def fill(g, A, W, C, N, K, norm=None, W2=None, residual=None):
+                g.d_A, g.d_W, g.d_C, g.N, g.K = A.data_ptr(), W.data_ptr(), C.data_ptr(), N, K
+                g.d_norm_weight = norm.data_ptr() if norm is not None else None
+                g.eps, g.weight_offset = c["eps"], 0
+                g.d_W2 = W2.data_ptr() if W2 is not None else None
+                g.d_residual = residual.data_ptr() if residual is not None else None
+                g.activation, g.alpha, g.swiglu_limit = capi.ACT_SILU, 1.0, 0.0
+            fill(arr[0], self.attn, d["wo"], self.x2, Hd, self.qs, residual=self.x)
+            fill(arr[1], self.x2, d["wgate"], self.act, I, Hd, norm=d["post_attn_norm"], W2=d["wup"])
+            fill(arr[2], self.act, d["wdown"], self.x, Hd, I, residual=self.x2)
+            if nxt:
+                fill(arr[3], self.x, nxt["wqkv"], self.qkv, self.qs + 2 * self.ks, Hd, norm=nxt["input_norm"])
+            chains.append(arr)
+        return chains
+
+    def _enqueue_chained(self, pos, want_logits):
+        """The step with the four GEMVs between two attentions in one persistent launch."""
+        L, c = self.L, self.cfg
+        ck = capi.check
+        H, Hkv, D, Hd = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"]
+        if self._chains is None:
+            self._chains = self._build_chains()
+        first = self.layers[0]
+        ck(L.dh_q4k_matmul_rmsnorm(self.x.data_ptr(), first["input_norm"].data_ptr(), c["eps"], 0,
+                                   first["wqkv"].data_ptr(), self.qkv.data_ptr(), capi.F32, 1,
+                                   self.qs + 2 * self.ks, Hd, 1.0, None))
+        for d, chain in zip(self.layers, self._chains):
+            ck(L.dh_qkv_norm_rope_kvwrite(self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
+                                          self.cos.data_ptr(), self.sin.data_ptr(), self.q.data_ptr(),
+                                          d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), 1, H, Hkv, D, pos, D, 0,
+                                          c["eps"], 0, pos * self.ks, int(c.get("qk_norm", 1))))
+            ck(L.dh_attn_decode(self.q.data_ptr(), d["cache_k"].data_ptr(), d["cache_v"].data_ptr(),
+                                self.attn.data_ptr(), H, Hkv, D, pos + 1, self.scale, 1, pos, 0.0, 0, 0,
+                                capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
+            ck(L.dh_q4k_gemv_chain(chain, len(chain)))
+        ck(L.dh_rmsnorm(self.x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd,
+                        c["eps"], 0, None, None, None, 1.0))
         ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
                                   self.lm_ws.data_ptr(), self.token.data_ptr(), 0,
                                   self.logits.data_ptr() if want_logits else None))
