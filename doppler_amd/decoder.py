@@ -13,7 +13,6 @@ All buffers are allocated once; a step enqueues ~8 launches per layer on the lib
 stream and reads back one token id, the reference's only device->host crossing per token.
 """
 import ctypes
-import os
 import math
 
 import numpy as np
@@ -37,15 +36,17 @@ def c_hidden_ok(cfg):
 
 
 class HipDecoder:
-    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True, chain=True):
+    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True, chain=False):
         """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
         layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
         input_norm, post_attn_norm, q_norm, k_norm: f32); embed_bits: uint16 [vocab, hidden]."""
         self.cfg = dict(cfg)
         # RMSNorm runs inside the q/k/v and gate/up GEMVs (their prologue) unless told otherwise
         self.fuse_norm = fuse_norm
-        # the GEMVs between two attentions (o_proj, gate/up, down, next q/k/v) as one persistent launch
-        self.chain = chain and fuse_norm and c_hidden_ok(cfg) and os.environ.get("DH_DECODE_CHAIN", "1") == "1"
+        # chain=True: the GEMVs between two attentions (o_proj, gate/up, down, next q/k/v) go out as
+        # one persistent launch.  Off by default: on MI355X the in-kernel barrier plus re-staging the
+        # activations under a saturated weight stream costs more than the three kernel boundaries.
+        self.chain = chain and fuse_norm and c_hidden_ok(cfg)
         self._chains = None
         self.L = capi.init(torch.cuda.current_device())
         c = self.cfg
