@@ -307,6 +307,12 @@ int env_int(const char* name, int dflt) {
 constexpr int kMaxDepth = 4;
 constexpr int kRedSlots = 4;       // tiles a fast wave may run ahead of the slowest one
 
+// LDS shape of the partial sums in the streaming kernel: slots (tiles in flight) and lanes kept.
+template <int MT> struct RingShape {
+  static constexpr int RS = MT >= 4 ? 2 : kRedSlots;
+  static constexpr int LW = MT > 2 ? 64 : 32;
+};
+
 #ifdef DH_GEMV_TRACE
 __device__ unsigned long long dh_trace_buf[256 * 64];
 #endif
@@ -469,10 +475,12 @@ template <int MT, bool DUAL, int XBYTES, int WAVES>
 __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(const RingArgs a) {
   constexpr int NTHR = 64 * WAVES;
   constexpr int XC = 2 * MT, NO = MfmaShape<MT>::NI / 2, NMAT = DUAL ? 2 : 1;
+  constexpr int RS = RingShape<MT>::RS, LW = RingShape<MT>::LW;
   __shared__ __align__(16) unsigned char xs[XBYTES];        // x fragments | zero row | (sum, 1/scale)
-  // K-slice partial sums per tile slot; only lanes 0..31 carry activation rows 0..1 (MT <= 2)
-  __shared__ float red[kRedSlots][WAVES][NMAT][NO][32];
-  __shared__ unsigned done[kRedSlots];                       // waves that delivered their partials
+  // K-slice partial sums per tile slot: entry k of lane l belongs to activation row
+  // (k & 1) + 2 * (l >> 5) + 4 * (k >> 1); up to two rows live in lanes 0..31 alone
+  __shared__ float red[RS][WAVES][NMAT][NO][LW];
+  __shared__ unsigned done[RS];                              // waves that delivered their partials
   __shared__ float norm_ss[WAVES][MT];
   extern __shared__ __align__(16) unsigned char ring[];     // [WAVES][depth][R*144]
 
@@ -589,14 +597,15 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     if (phase == 0 && norm) {
       // sum of squares of activation row m = (tid >> 2) % MT: lanes of a quad share a row,
       // lane bit 2 selects the row when MT == 2
+      // (lane bits 2.. select the row: MT consecutive quads hold MT different rows)
       ss += quad_xor_f32(ss, 1);
       ss += quad_xor_f32(ss, 2);
-      if (MT == 1) ss += __shfl_xor(ss, 4);
-      ss += __shfl_xor(ss, 8);
-      ss += __shfl_xor(ss, 16);
+      if (MT <= 1) ss += __shfl_xor(ss, 4);
+      if (MT <= 2) ss += __shfl_xor(ss, 8);
+      if (MT <= 4) ss += __shfl_xor(ss, 16);
       ss += __shfl_xor(ss, 32);
       const int my_m = (tid >> 2) % MT;
-      if ((lane & ~4) == 0 && (lane >> 2) < MT) norm_ss[wave][lane >> 2] = ss;
+      if ((lane & 3) == 0 && (lane >> 2) < MT) norm_ss[wave][lane >> 2] = ss;
       DH_LDS_BARRIER();
       float tot = 0.f;
 #pragma unroll
@@ -621,7 +630,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
       stage_x_store<MT>(idx, t, xf, sxi);
     }
     if (tid < 16) reinterpret_cast<uint32_t*>(xzero)[tid] = 0u;
-    if (tid < kRedSlots) done[tid] = 0u;
+    if (tid < RS) done[tid] = 0u;
     DH_TS();
     DH_LDS_BARRIER();
     DH_TS();
@@ -638,7 +647,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
 #pragma unroll 1
   for (int tl = 0; tl < ntl; tl++) {
     const int tile = blockIdx.x + tl * gridDim.x;
-    const int slot = tl % kRedSlots;
+    const int slot = tl % RS;
 #pragma unroll 1
     for (int mat = 0; mat < NMAT; mat++) {
       float acc[NO];
@@ -678,7 +687,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
 #endif
         DH_TS();
       }
-      if (lane < 32) {
+      if (lane < LW) {
 #pragma unroll
         for (int k = 0; k < NO; k++) red[slot][wave][mat][k][lane] = acc[k];
       }
@@ -697,14 +706,18 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     arrived = __builtin_amdgcn_readfirstlane(arrived);
     asm volatile("" ::: "memory");
     if (arrived == WAVES - 1) {
-      const int r = lane & 31, m = lane >> 5;
+      const int r = lane & 31;
       const int64_t row = (int64_t)tile * R + r;
-      if (m < a.M && m < MT && r < R && row < a.N) {
+#pragma unroll 1
+      for (int m = lane >> 5; m < MT; m += 2) {
+      if (m < a.M && r < R && row < a.N) {
+        // activation row m sits in entry (m & 1) + 2 * (m >> 2) of lane half (m >> 1) & 1
+        const int k = (m & 1) + 2 * (m >> 2), col = (MT > 2 ? 32 * ((m >> 1) & 1) : 0) + r;
         float sg = 0.f, su = 0.f;
 #pragma unroll
         for (int w = 0; w < WAVES; w++) {
-          sg += red[slot][w][0][m][r];
-          if (DUAL) su += red[slot][w][NMAT - 1][m][r];
+          sg += red[slot][w][0][k][col];
+          if (DUAL) su += red[slot][w][NMAT - 1][k][col];
         }
         float v;
         if (DUAL) {
@@ -720,10 +733,11 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
         else
           reinterpret_cast<float*>(a.C)[(int64_t)m * a.N + row] = v;
       }
+      }
       if (lane == 0) done[slot] = 0u;
     }
     // more tiles than slots: keep the waves within one tile of each other instead
-    if (ntl > kRedSlots) DH_LDS_BARRIER();
+    if (ntl > RS) DH_LDS_BARRIER();
     DH_TS();
   }
 #ifdef DH_GEMV_TRACE
@@ -1057,9 +1071,9 @@ constexpr size_t kRingMaxLds = 160 * 1024;
 size_t ring_x_bytes(int mt, int nb) { return (size_t)nb * 8 * mt * (2 * 32 * 2 + 8) + 64; }
 
 template <int MT, bool DUAL, int XBYTES, int WAVES>
-int launch_ring_cfg(RingArgs a, const char* op) {
+int launch_ring_cfg(RingArgs a, const char* op, bool may_shorten_tiles) {
   constexpr int NO = MfmaShape<MT>::NI / 2, NMAT = DUAL ? 2 : 1;
-  const size_t fixed = XBYTES + sizeof(float) * kRedSlots * WAVES * NMAT * NO * 32 + 512;
+  const size_t fixed = XBYTES + sizeof(float) * RingShape<MT>::RS * WAVES * NMAT * NO * RingShape<MT>::LW + 512;
   auto kern = q4k_gemv_ring_kernel<MT, DUAL, XBYTES, WAVES>;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
@@ -1075,6 +1089,9 @@ int launch_ring_cfg(RingArgs a, const char* op) {
   int rows = (int)dh::ceil_div(a.N, (int64_t)ncu * per_cu);
   rows = std::max(4, std::min(32, rows));
   if (env_rows > 0) rows = std::min(32, env_rows);
+  // a two-stage ring must fit beside the activations; shorter tiles (uneven tile counts per
+  // compute unit) only when nothing else is left
+  while (may_shorten_tiles && rows > 8 && fixed + (size_t)WAVES * 2 * rows * kBlockBytes > kRingMaxLds) rows -= 4;
   int depth = kMaxDepth;
   while (depth > 2 && fixed + (size_t)WAVES * depth * rows * kBlockBytes > kRingMaxLds) depth--;
   if (env_depth > 0) depth = std::max(2, std::min(kMaxDepth, env_depth));
@@ -1089,41 +1106,70 @@ int launch_ring_cfg(RingArgs a, const char* op) {
   return 0;
 }
 
-// Returns -1 when the activations of `mt` rows do not fit the kernel's static LDS array.
+// Returns -1 when the activations of MT rows do not fit any of the kernel's static LDS arrays.
+// MT <= 2 run with 16 waves per workgroup where the ring still fits (more loads in flight);
+// four and eight activation rows need the LDS for their fragments and run with 8.
 template <int MT, bool DUAL>
 int launch_ring(const RingArgs& a, const char* op) {
   const size_t xb = ring_x_bytes(MT, a.nb);
   static const int env_waves = env_int("DH_GEMV_WAVES", 16);
-  // 16 waves per workgroup hide more latency; their rings need twice the LDS
-  if (env_waves == 16) {
-    int rc = -1;
-    if (xb <= 20 * 1024) rc = launch_ring_cfg<MT, DUAL, 20 * 1024, 16>(a, op);
-    else if (xb <= 40 * 1024) rc = launch_ring_cfg<MT, DUAL, 40 * 1024, 16>(a, op);
-    else if (xb <= 56 * 1024) rc = launch_ring_cfg<MT, DUAL, 56 * 1024, 16>(a, op);
-    if (rc >= 0) return rc;
+  if constexpr (MT <= 2) {
+    if (env_waves == 16) {
+      int rc = -1;
+      if (xb <= 20 * 1024) rc = launch_ring_cfg<MT, DUAL, 20 * 1024, 16>(a, op, false);
+      else if (xb <= 40 * 1024) rc = launch_ring_cfg<MT, DUAL, 40 * 1024, 16>(a, op, false);
+      else if (xb <= 56 * 1024) rc = launch_ring_cfg<MT, DUAL, 56 * 1024, 16>(a, op, false);
+      if (rc >= 0) return rc;
+    }
+    if (xb <= 20 * 1024) return launch_ring_cfg<MT, DUAL, 20 * 1024, 8>(a, op, true);
+    if (xb <= 40 * 1024) return launch_ring_cfg<MT, DUAL, 40 * 1024, 8>(a, op, true);
+    if (xb <= 56 * 1024) return launch_ring_cfg<MT, DUAL, 56 * 1024, 8>(a, op, true);
+    if constexpr (MT == 2) {
+      if (xb <= 104 * 1024) return launch_ring_cfg<MT, DUAL, 104 * 1024, 8>(a, op, true);
+    }
+  } else {
+    if (xb <= 40 * 1024) return launch_ring_cfg<MT, DUAL, 40 * 1024, 8>(a, op, true);
+    if (xb <= 72 * 1024) return launch_ring_cfg<MT, DUAL, 72 * 1024, 8>(a, op, true);
+    if (xb <= 104 * 1024) return launch_ring_cfg<MT, DUAL, 104 * 1024, 8>(a, op, true);
   }
-  if (xb <= 20 * 1024) return launch_ring_cfg<MT, DUAL, 20 * 1024, 8>(a, op);
-  if (xb <= 40 * 1024) return launch_ring_cfg<MT, DUAL, 40 * 1024, 8>(a, op);
-  if (xb <= 56 * 1024) return launch_ring_cfg<MT, DUAL, 56 * 1024, 8>(a, op);
   return -1;
 }
 
-// M <= 8 activation rows, two at a time when their fragments fit in LDS, else one at a time.
+template <bool DUAL>
+int launch_ring_mt(int mt, const RingArgs& a, const char* op) {
+  switch (mt) {
+    case 8: return launch_ring<8, DUAL>(a, op);
+    case 4: return launch_ring<4, DUAL>(a, op);
+    case 2: return launch_ring<2, DUAL>(a, op);
+    default: return launch_ring<1, DUAL>(a, op);
+  }
+}
+
+// M <= 8 activation rows in as few passes over the weights as the LDS allows: 8, 4, 2 or 1 rows
+// per pass (a pass with fewer rows than its kernel holds zero-fills the rest).
 template <bool DUAL>
 int dispatch_ring(const RingArgs& a, const char* op) {
-  const int mt = (a.M >= 2 && ring_x_bytes(2, a.nb) <= 56 * 1024) ? 2 : 1;
-  if (ring_x_bytes(mt, a.nb) > 56 * 1024) return -1;
+  static const int env_mt = env_int("DH_GEMV_MT", 8);
   const size_t c_elem = a.c_f16 ? 2 : 4;
-  for (int m0 = 0; m0 < a.M; m0 += mt) {
-    RingArgs b = a;
-    b.M = std::min(mt, a.M - m0);
-    b.A = a.A + (int64_t)m0 * a.K;
-    b.C = static_cast<char*>(a.C) + (int64_t)m0 * a.N * c_elem;
-    b.residual = a.residual ? a.residual + (int64_t)m0 * a.N : nullptr;
-    const int rc = b.M == 2 ? launch_ring<2, DUAL>(b, op) : launch_ring<1, DUAL>(b, op);
-    if (rc) return rc;
+  // candidates in order of passes needed, smaller kernels first among equals
+  int order[4] = {1, 2, 4, 8}, n = 0;
+  for (int mt : {1, 2, 4, 8}) n += mt <= env_mt;
+  std::stable_sort(order, order + n, [&](int x, int y) { return (a.M + x - 1) / x < (a.M + y - 1) / y; });
+  for (int c = 0; c < n; c++) {
+    const int mt = order[c];
+    int rc = 0;
+    for (int m0 = 0; m0 < a.M; m0 += mt) {
+      RingArgs b = a;
+      b.M = std::min(mt, a.M - m0);
+      b.A = a.A + (int64_t)m0 * a.K;
+      b.C = static_cast<char*>(a.C) + (int64_t)m0 * a.N * c_elem;
+      b.residual = a.residual ? a.residual + (int64_t)m0 * a.N : nullptr;
+      rc = launch_ring_mt<DUAL>(mt, b, op);
+      if (rc) break;                 // -1 on the first pass: this row count does not fit
+    }
+    if (rc >= 0) return rc;
   }
-  return 0;
+  return -1;
 }
 
 constexpr size_t kMaxLds = 128 * 1024;

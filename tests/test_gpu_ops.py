@@ -98,7 +98,10 @@ def test_matmul_cfg1_block_sweep(name, M):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (1, 1024, 4096), (1, 12288, 4096), (1, 4096, 12288),
-                                   (3, 4096, 4096), (8, 1024, 12288)])
+                                   (3, 4096, 4096), (8, 1024, 12288),
+                                   # four and eight activation rows per pass, and the LDS limits around them
+                                   (4, 6144, 4096), (8, 4096, 4096), (2, 4096, 12288), (4, 2048, 12288),
+                                   (6, 1024, 3072), (7, 512, 6144), (8, 1000, 2048), (5, 4096, 1024)])
 def test_matmul_cfg4_shapes(M, N, K):
     assert _matmul_case(M, N, K, seed=1300 + M) <= REL_L2_F32
 
@@ -176,7 +179,8 @@ def test_matmul_errors_match_reference_behaviour():
 
 # ----------------------------------------------------------------------------- fused FFN gate/up
 
-@pytest.mark.parametrize("M,activation,limit", [(1, "silu", None), (4, "silu", 7.0), (1, "gelu", None), (3, "gelu", None)])
+@pytest.mark.parametrize("M,activation,limit", [(1, "silu", None), (4, "silu", 7.0), (1, "gelu", None), (3, "gelu", None),
+                                                (8, "silu", None), (6, "gelu", 3.0)])
 def test_fused_ffn_q4k(M, activation, limit):
     hidden, inter = 1536, 6144          # the shape of the reference's fused-ffn-q4k parity test
     Wg, wg = q4k_weight(inter, hidden, seed=2000)
@@ -189,7 +193,9 @@ def test_fused_ffn_q4k(M, activation, limit):
 
 
 @pytest.mark.parametrize("M,N,K,offset", [(1, 6144, 4096, False), (2, 1024, 1024, True), (1, 2048, 640, False),
-                                          (3, 96, 1152, False), (1, 4096, 12288, False), (5, 130, 2048, True)])
+                                          (3, 96, 1152, False), (1, 4096, 12288, False), (5, 130, 2048, True),
+                                          (4, 1024, 4096, False), (8, 512, 2048, True), (7, 256, 4096, False),
+                                          (2, 300, 12288, False)])
 def test_matmul_with_rmsnorm_prologue(M, N, K, offset):
     """runMatmul with normWeight + useFusedRmsnormWideTile == runRMSNorm followed by runMatmul
     (reference: src/gpu/kernels/matmul-selection.js:609-620)."""
@@ -205,7 +211,7 @@ def test_matmul_with_rmsnorm_prologue(M, N, K, offset):
     assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
 
 
-@pytest.mark.parametrize("M,activation", [(1, "silu"), (2, "gelu")])
+@pytest.mark.parametrize("M,activation", [(1, "silu"), (2, "gelu"), (4, "silu"), (8, "gelu"), (5, "silu")])
 def test_fused_normed_ffn_q4k(M, activation):
     hidden, inter = 1536, 6144
     Wg, wg = q4k_weight(inter, hidden, seed=2200)
