@@ -26,6 +26,9 @@ int num_cus();
 // monotonic counters 256 bytes apart, an error flag the kernel raises when a barrier times out,
 // and the host's copy of the counters' value.  chain_advance(n) returns that value and adds n.
 unsigned* chain_counters();
+// Scratch for the split-K prefill GEMM's partial products (allocated by dh_init, shared by all
+// launches on the library's stream, which run in order).
+float* splitk_workspace(size_t* bytes);
 unsigned* chain_error_flag();
 unsigned chain_advance(unsigned n);
 

@@ -14,6 +14,8 @@ hipStream_t g_stream = nullptr;
 int g_num_cus = 0;
 unsigned* g_chain_mem = nullptr;     // [8 * 64] barrier counters + [1] error flag
 unsigned g_chain_value = 0;          // what every counter reads once the enqueued launches are done
+float* g_splitk_ws = nullptr;        // partial products of the split-K prefill GEMM
+constexpr size_t kSplitKWsBytes = (size_t)32 << 20;
 constexpr size_t kChainWords = 8 * 64 + 64;
 }  // namespace
 
@@ -28,6 +30,10 @@ int fail(int code, const char* fmt, ...) {
 hipStream_t stream() { return g_stream; }
 bool ready() { return g_ready; }
 int num_cus() { return g_num_cus; }
+float* splitk_workspace(size_t* bytes) {
+  *bytes = g_splitk_ws ? kSplitKWsBytes : 0;
+  return g_splitk_ws;
+}
 unsigned* chain_counters() { return g_chain_mem; }
 unsigned* chain_error_flag() { return g_chain_mem ? g_chain_mem + 8 * 64 : nullptr; }
 unsigned chain_advance(unsigned n) {
@@ -64,6 +70,7 @@ int dh_init(int device_ordinal) {
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_chain_mem), kChainWords * sizeof(unsigned)));
   DH_CHECK_HIP("dh_init", hipMemset(g_chain_mem, 0, kChainWords * sizeof(unsigned)));
   g_chain_value = 0;
+  DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_splitk_ws), kSplitKWsBytes));
   g_device = device_ordinal;
   g_ready = true;
   return 0;
@@ -76,6 +83,8 @@ int dh_shutdown(void) {
   if (g_own_stream) DH_CHECK_HIP("dh_shutdown", hipStreamDestroy(g_own_stream));
   if (g_chain_mem) DH_CHECK_HIP("dh_shutdown", hipFree(g_chain_mem));
   g_chain_mem = nullptr;
+  if (g_splitk_ws) DH_CHECK_HIP("dh_shutdown", hipFree(g_splitk_ws));
+  g_splitk_ws = nullptr;
   g_own_stream = nullptr;
   g_stream = nullptr;
   g_ready = false;

@@ -16,6 +16,7 @@
 // nibble pairs come out in, and a contraction index may be permuted freely when both operands
 // agree.
 #include <algorithm>
+#include <cstdlib>
 
 #include "dh_common.h"
 #include "q4k_device.h"
@@ -28,6 +29,11 @@ using dh::kQK;
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
 typedef __attribute__((ext_vector_type(16))) float float16_t;
+
+int env_ksplit() {
+  const char* e = getenv("DH_GEMM_KSPLIT");
+  return e ? atoi(e) : 0;
+}
 
 constexpr int BK = 64;
 constexpr int LDS_ROW = BK + 8;                    // halves per LDS row (144 bytes)
@@ -42,6 +48,10 @@ struct GemmArgs {
   float alpha;
   int c_f16, activation;
   float clamp_max;
+  // split-K: blockIdx.z takes K steps [z * kt_per_split, ...) and writes its raw partial product to
+  // partial[z][M][N]; splitk_reduce_kernel adds the pieces in order
+  int ksplit, kt_per_split;
+  float* partial;
 };
 
 // 16 nibble bytes -> 16 low-nibble and 16 high-nibble weights as f16, k order (0,2,1,3) per dword.
@@ -92,7 +102,8 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
   const int wm = (wave >> 1) * 32 * T, wn = (wave & 1) * 32 * T;     // the wave's quadrant
   const int fr = lane & 31, fg = lane >> 5;                  // fragment row / k half
   const int64_t row_bytes = (int64_t)a.nb * kBlockBytes;
-  const int nkt = (a.K + BK - 1) / BK;
+  const int kt0 = a.ksplit > 1 ? (int)blockIdx.z * a.kt_per_split : 0;
+  const int nkt = a.ksplit > 1 ? min((a.K + BK - 1) / BK, kt0 + a.kt_per_split) : (a.K + BK - 1) / BK;
 
   // ---- global -> register staging roles
   // A: 8 float4 per thread, idx = tid + 256 i: row idx >> 4, k 4 * (idx & 15)
@@ -158,10 +169,10 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[mt][i][j][e] = 0.f;
 
-  load_tile(0);
-  store_tile(0, 0);
+  load_tile(kt0);
+  store_tile(kt0, kt0 & 1);
   __syncthreads();
-  for (int kt = 0; kt < nkt; kt++) {
+  for (int kt = kt0; kt < nkt; kt++) {
     const int buf = kt & 1;
     if (kt + 1 < nkt) load_tile(kt + 1);
     const _Float16* At = lds + buf * BUF_HALVES;
@@ -200,6 +211,10 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
         const int m = m0 + wm + 32 * i + 8 * (e >> 2) + 4 * fg + (e & 3);
         if (m < a.M && n < a.N) {
           float v;
+          if (!DUAL && a.ksplit > 1) {
+            a.partial[((int64_t)blockIdx.z * a.M + m) * a.N + n] = acc[0][i][j][e];
+            continue;
+          }
           if (DUAL) {
             const float g = acc[0][i][j][e], u = acc[NMAT - 1][i][j][e];
             v = (a.activation == DH_ACT_SILU ? act_silu(g) : gelu_tanh_fast(g)) * u * a.alpha;
@@ -217,6 +232,21 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
     }
 }
 
+// C = alpha * (sum of the split-K pieces, in split order) + residual.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs a) {
+  const int64_t total = (int64_t)a.M * a.N;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  float s = 0.f;
+  for (int z = 0; z < a.ksplit; z++) s += a.partial[(int64_t)z * total + i];
+  float v = s * a.alpha;
+  if (a.residual) v += a.residual[i];
+  if (a.c_f16)
+    reinterpret_cast<__half*>(a.C)[i] = __float2half(v);
+  else
+    reinterpret_cast<float*>(a.C)[i] = v;
+}
+
 template <bool DUAL, int T>
 int launch_gemm_cfg(const GemmArgs& a, const char* op) {
   constexpr int BM = 64 * T, BN = 64 * T;
@@ -228,18 +258,43 @@ int launch_gemm_cfg(const GemmArgs& a, const char* op) {
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attr_set = true;
   }
-  const dim3 grid((unsigned)dh::ceil_div(a.N, BN), (unsigned)dh::ceil_div(a.M, BM));
+  const dim3 grid((unsigned)dh::ceil_div(a.N, BN), (unsigned)dh::ceil_div(a.M, BM), (unsigned)std::max(1, a.ksplit));
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
+  if (a.ksplit > 1) {
+    const int64_t total = (int64_t)a.M * a.N;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)dh::ceil_div(total, 256)), dim3(256), 0, dh::stream(), a);
+    DH_CHECK_LAUNCH(op);
+  }
   return 0;
 }
 
 // 128 x 128 tiles when they occupy at least half of the compute units (their higher matrix-core
 // share wins from there on), else 64 x 64.
 template <bool DUAL>
-int launch_gemm(const GemmArgs& a, const char* op) {
+int launch_gemm(GemmArgs a, const char* op) {
   const int64_t big_tiles = dh::ceil_div(a.M, 128) * dh::ceil_div(a.N, 128);
+  a.ksplit = 1;
   if (2 * big_tiles >= dh::num_cus()) return launch_gemm_cfg<DUAL, 2>(a, op);
+  // Few tiles and a long K: every workgroup would walk K alone at one memory round trip per
+  // step.  Cut K so that about three workgroups share a compute unit and overlap each other's
+  // waits; the pieces meet in the library's scratch buffer.
+  if (!DUAL) {
+    static const int env_split = env_ksplit();
+    const int64_t tiles = dh::ceil_div(a.M, 64) * dh::ceil_div(a.N, 64);
+    const int nkt = (a.K + BK - 1) / BK;
+    size_t ws_bytes = 0;
+    float* ws = dh::splitk_workspace(&ws_bytes);
+    int split = (int)std::min<int64_t>(8, dh::ceil_div(3 * (int64_t)dh::num_cus(), tiles));
+    split = std::min(split, nkt / 8);
+    if (env_split > 0) split = env_split;
+    while (split > 1 && (size_t)split * a.M * a.N * sizeof(float) > ws_bytes) split--;
+    if (split > 1 && ws) {
+      a.kt_per_split = (int)dh::ceil_div(nkt, split);
+      a.ksplit = (int)dh::ceil_div(nkt, a.kt_per_split);
+      a.partial = ws;
+    }
+  }
   return launch_gemm_cfg<DUAL, 1>(a, op);
 }
 

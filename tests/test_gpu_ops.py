@@ -114,7 +114,10 @@ def test_matmul_ragged_shapes(M, N, K):
 
 @pytest.mark.parametrize("M,N,K,kw", [(512, 6912, 1152, {}), (512, 1152, 6912, dict(residual=True)),
                                       (130, 200, 640, dict(alpha=0.5)), (16, 128, 256, dict(outputDtype="f16")),
-                                      (77, 129, 1000, {}), (300, 96, 300, {})])
+                                      (77, 129, 1000, {}), (300, 96, 300, {}),
+                                      # long K, few tiles: the split-K path with its ordered reduction
+                                      (64, 64, 4096, dict(alpha=0.5, outputDtype="f16", residual=True)),
+                                      (100, 70, 8192, dict(residual=True))])
 def test_matmul_prefill_gemm(M, N, K, kw):
     """Config-2 shapes (X[512,1152] against [6912,1152] and [1152,6912]) and ragged tiles."""
     assert _matmul_case(M, N, K, seed=1500 + M, **kw) <= REL_L2_F16_MFMA
