@@ -70,6 +70,23 @@ def gate_up_kernel_bandwidth(dec, reps):
     return total_ms / max(n, 1)
 
 
+def js_reference_timings():
+    """Runs oracle/js/reference_port.mjs (one thread, as the reference's JS is) and returns its
+    timings in milliseconds, or None when node is missing."""
+    import shutil
+    import subprocess
+    node = shutil.which("node")
+    if not node:
+        return None
+    try:
+        r = subprocess.run([node, os.path.join(ROOT, "oracle", "js", "reference_port.mjs"), "time"],
+                           capture_output=True, text=True, timeout=300, check=True)
+        return json.loads(r.stdout.strip().splitlines()[-1])
+    except Exception as e:      # a baseline, never a reason to lose the GPU result
+        log("[bench] JS port timing failed: %r" % (e,))
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -183,9 +200,13 @@ def main():
             n_cpu += 1
             t_cpu = time.perf_counter() - t0
         threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+        js = js_reference_timings()
         cpu = {"value": round(n_cpu / t_cpu, 4), "unit": "tokens/s", "cores": threads, "kind": "port",
                "sample": "%d full decode steps of the same model from the same prefilled KV cache "
-                         "(C restatement of the reference's JS per-op references, f64 accumulate, OpenMP)" % n_cpu}
+                         "(C restatement of the reference's JS per-op references, f64 accumulate, OpenMP)" % n_cpu,
+               # the reference's CPU path is single-threaded JavaScript: the same per-op references
+               # restated in JS and timed under this host's node, per-op, on the small configs
+               "js_port_single_thread_ms": js}
 
     out = {
         "metric": "decode tokens/sec at 9B-class Q4_K, 1 GPU (Q4_K GEMV HBM GB/s in roofline)",

@@ -4,6 +4,9 @@ arithmetic and brute force.  A wrong index, sign, rounding or operand order in
 oracle/doppler_oracle.c fails at least one test here."""
 import hashlib
 import math
+import os
+import shutil
+import subprocess
 from fractions import Fraction
 
 import numpy as np
@@ -201,6 +204,30 @@ def test_q4k_matmul_equals_dequant_then_sequential_f64_dot():
             for k in range(K):
                 s += float(A[m, k]) * float(Wd[n, k])
             assert np.float32(s * 0.5) == C[m, n]
+
+
+@pytest.mark.skipif(shutil.which("node") is None, reason="node is not installed")
+def test_js_port_of_the_reference_agrees_with_the_c_oracle(tmp_path):
+    """oracle/js/reference_port.mjs restates the reference's JS decode + f64 dot a second time,
+    independently of the C oracle (different language, written from the reference's text):
+    both must produce the same f32 results, including a K that is not a multiple of 256 and
+    subnormal / large d, dmin."""
+    M, N, K = 3, 40, 640
+    W = synth.q4k_tensor(N, K, seed=77).copy()
+    blocks = W.reshape(-1, 144)
+    blocks[0, 0:4] = [0x01, 0x00, 0xff, 0x03]        # subnormal d, largest subnormal dmin
+    blocks[1, 0:4] = [0x00, 0x3c, 0x00, 0x44]        # d = 1, dmin = 4
+    A = synth.normal_f32((M, K), seed=78)
+    src, dst = tmp_path / "in.bin", tmp_path / "out.bin"
+    with open(src, "wb") as f:
+        f.write(np.array([M, N, K], np.int32).tobytes())
+        f.write(A.tobytes())
+        f.write(W.tobytes())
+    script = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "js", "reference_port.mjs")
+    subprocess.run(["node", script, "gemv", str(src), str(dst)], check=True, timeout=120)
+    got = np.fromfile(dst, np.float32).reshape(M, N)
+    want = oracle.q4k_matmul(A, W, M, N, K)
+    assert np.array_equal(got, want)
 
 
 def test_q4k_matmul_properties():
