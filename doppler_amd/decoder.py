@@ -14,6 +14,7 @@ stream and reads back one token id, the reference's only device->host crossing p
 """
 import ctypes
 import math
+import warnings
 
 import numpy as np
 import torch
@@ -26,7 +27,10 @@ _P = ctypes.c_void_p
 def _dev_bytes(arr):
     """Upload a numpy array into a fresh torch.uint8 CUDA buffer."""
     arr = np.ascontiguousarray(arr)
-    t = torch.from_numpy(arr.view(np.uint8).reshape(-1)).cuda()
+    with warnings.catch_warnings():
+        # read-only sources (memory-mapped shards) are only read from here
+        warnings.filterwarnings("ignore", message="The given NumPy array is not writable")
+        t = torch.from_numpy(arr.view(np.uint8).reshape(-1)).cuda()
     return t
 
 
