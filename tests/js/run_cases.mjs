@@ -5,6 +5,7 @@ import fs from 'fs';
 import path from 'path';
 import * as dh from '../../doppler_amd/js/kernel-selector.js';
 import { HipTextDecoder } from '../../doppler_amd/js/pipeline/decode-step.js';
+import { loadDecoderWeights, parseManifest } from '../../doppler_amd/js/loader/rdrr-loader.js';
 
 const dir = process.argv[2];
 const manifest = JSON.parse(fs.readFileSync(path.join(dir, 'manifest.json'), 'utf8'));
@@ -144,6 +145,17 @@ async function main() {
         tokens.push(tok);
       }
       fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
+    } else if (c.op === 'rdrr_decoder') {
+      // weights come from an RDRR artifact directory through the JS loader
+      const { config, weights } = loadDecoderWeights(c.dir, c.maxSeq);
+      const dec = new HipTextDecoder(config, weights);
+      const tokens = [];
+      let tok = c.prompt[0];
+      for (let pos = 0; pos < c.prompt.length + c.steps; pos++) {
+        tok = await dec.decodeStep(pos < c.prompt.length ? c.prompt[pos] : tok, pos);
+        tokens.push(tok);
+      }
+      fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
     } else {
       throw new Error(`unknown case op ${c.op}`);
     }
@@ -164,6 +176,11 @@ async function main() {
     await expectThrow(results, 'gather', 'embeddingDtype is required', () => dh.runGather(A.buffer, A.buffer, 1, 8, 8, {}));
     await expectThrow(results, 'kvwrite', 'smaller than requested range', () => dh.runKVCacheWriteF32ToF16(A.buffer, A.buffer, A.buffer, A.buffer, { elementCount: 100000 }));
     await expectThrow(results, 'attn', 'kvLayout', () => dh.runAttention(A, A, A, null, 2, 64, { kvLayout: 'paged' }));
+    await expectThrow(results, 'rdrr-json', 'Failed to parse manifest JSON', async () => parseManifest('{'));
+    await expectThrow(results, 'rdrr-shard', 'missing shard index', async () => parseManifest(JSON.stringify({
+      shards: [{ filename: 'shard_00000.bin', size: 1024 }], tensors: { w: { offset: 0, size: 4, shape: [1], dtype: 'F32' } } })));
+    await expectThrow(results, 'rdrr-size', 'should hold 144 bytes', async () => parseManifest(JSON.stringify({
+      shards: [{ filename: 'shard_00000.bin', size: 1024 }], tensors: { w: { shard: 0, offset: 0, size: 100, shape: [1, 256], dtype: 'Q4_K_M' } } })));
     await expectThrow(results, 'ffn', 'matching gate/up dtypes', () => dh.runFusedFFN(A, W, dh.createWeightBuffer(W.buffer, 'f16', 'row', [8, 256]), 256, 8, {}));
   }
 

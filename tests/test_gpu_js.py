@@ -208,6 +208,27 @@ def test_js_host_path_parity(tmp_path):
         want_tokens.append(tok)
     checks.append(lambda: [int(t) for t in get("decoder.out.bin", np.uint32)] == want_tokens)
 
+    # ---- the same model again, this time written as an RDRR artifact (small shards, so tensors
+    #      span shard boundaries) and read back by the JavaScript loader
+    from doppler_amd import rdrr
+    art_dir = os.path.join(d, "artifact")
+    rdrr.write_artifact(art_dir, cfg, layers, embed, final_norm, shard_bytes=300_000)
+    art_obj = rdrr.Artifact(art_dir)
+    c2, l2, e2, fn2 = rdrr.load_model_arrays(art_obj)        # norms rounded to f16 by the artifact
+    ol2 = []
+    for l in l2:
+        dd = dict(l)
+        dd["cache_k"] = np.zeros((24, 4, 64), np.uint16)
+        dd["cache_v"] = np.zeros((24, 4, 64), np.uint16)
+        ol2.append(dd)
+    cpu2 = oracle.DecoderOracle(cfg, ol2, e2, fn2, mc, ms)
+    want2, tok = [], None
+    for pos in range(len(prompt) + 10):
+        tok = cpu2.step(prompt[pos] if pos < len(prompt) else tok, pos)
+        want2.append(tok)
+    cases.append(dict(name="rdrr_decoder", op="rdrr_decoder", dir=art_dir, maxSeq=24, prompt=prompt, steps=10))
+    checks.append(lambda: [int(t) for t in get("rdrr_decoder.out.bin", np.uint32)] == want2)
+
     json.dump(dict(cases=cases), open(os.path.join(d, "manifest.json"), "w"))
     p = subprocess.run([NODE, os.path.join(ROOT, "tests", "js", "run_cases.mjs"), d], stdout=subprocess.PIPE,
                        stderr=subprocess.STDOUT, text=True, timeout=500)
@@ -217,4 +238,4 @@ def test_js_host_path_parity(tmp_path):
     for i, chk in enumerate(checks):
         assert chk(), "check %d failed" % i
     bad = [e for e in res["errors"] if not e["ok"]]
-    assert not bad and len(res["errors"]) >= 11, bad
+    assert not bad and len(res["errors"]) >= 14, bad
