@@ -1,11 +1,13 @@
 // Decode attention (one query token) over an f16 KV cache with grouped-query heads.
 //
 // Split-K over the context: grid = (kv head, split).  A workgroup walks its slice of keys in
-// tiles of 64, stages the K and V tiles of ONE kv head in LDS and serves all G = H/Hkv query
-// heads that share it from that single copy, so K/V are read from HBM once per kv head
-// rather than once per query head.  Scores and softmax statistics are fp32; each split keeps
-// an online-softmax state (m, l, o) per query head and a second tiny kernel merges the
-// splits with the usual log-sum-exp rescale.
+// tiles of 64 and serves all G = H/Hkv query heads of ONE kv head from a single pass over its
+// K and V rows, so K/V are read from HBM once per kv head rather than once per query head.
+// Scores and softmax statistics are fp32; each split keeps an online-softmax state (m, l, o)
+// per query head and a second tiny kernel merges the splits with the usual log-sum-exp
+// rescale.  (Merging inside the split kernel, by the last workgroup to arrive per kv head, was
+// measured slower: store acknowledgement, arrival atomic and two rounds of agent-scope loads
+// are four dependent memory round trips, more than the kernel boundary costs.)
 #include <algorithm>
 #include <cfloat>
 
