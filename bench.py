@@ -118,7 +118,8 @@ def main():
         c["layers"] = args.layers
     if args.prefill is not None:
         prefill = args.prefill
-    max_seq = prefill + args.warmup + args.steps + 1
+    BATCH = 16                       # extra positions for the batched-decode side measurement
+    max_seq = prefill + args.warmup + args.steps + 2 * BATCH + 1
     cfg = dict(c, max_seq=max_seq)
 
     t0 = time.time()
@@ -158,6 +159,17 @@ def main():
     step_bytes = dec.weight_bytes_per_token(ctx_mid)
     log("[bench] %d steps in %.3f s -> %.1f tok/s (%.0f GB/s of algorithmic traffic)" %
         (args.steps, elapsed, tok_s, step_bytes * tok_s / 1e9))
+
+    # ---- side measurement: the same steps submitted 16 at a time with the token fed back on the
+    #      device (the reference's batched decode); not the headline value, which keeps the
+    #      reference's default of one token readback per step
+    dec.decode_batch(tok, pos, BATCH)
+    capi_sync()
+    t0 = time.perf_counter()
+    dec.decode_batch(tok, pos + BATCH, BATCH)
+    capi_sync()
+    batched_tok_s = BATCH / (time.perf_counter() - t0)
+    log("[bench] batched decode, %d tokens per submit: %.1f tok/s" % (BATCH, batched_tok_s))
 
     # ---- roofline of the dominant kernel
     Hd, I = cfg["hidden"], cfg["inter"]
@@ -216,7 +228,8 @@ def main():
         "config": {"workload": "BASELINE configs[4]: 36-layer 9B-class Q4_K decoder, hidden 4096, FFN 12288, "
                                "32/8 heads x128, vocab 151936, KV prefilled to %d, greedy, batch 1" % prefill,
                    "layers": cfg["layers"], "context": prefill, "algorithmic_bytes_per_step": step_bytes,
-                   "hbm_frac_whole_step": round(step_bytes * tok_s / 1e9 / HBM_PEAK_GBPS, 4)},
+                   "hbm_frac_whole_step": round(step_bytes * tok_s / 1e9 / HBM_PEAK_GBPS, 4),
+                   "batched_decode_16_per_submit_tokens_per_s": round(batched_tok_s, 2)},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "tokens_head": tokens[:4],

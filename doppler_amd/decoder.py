@@ -40,6 +40,8 @@ def c_hidden_ok(cfg):
 
 
 class HipDecoder:
+    TOKEN_RING = 64      # tokens one decode_batch submit can produce
+
     def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True, chain=False):
         """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
         layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
@@ -84,7 +86,7 @@ class HipDecoder:
         self.attn = f32(self.qs)
         self.act = f32(I)
         self.logits = f32(c["vocab"])
-        self.token = torch.zeros(4, dtype=torch.int32, device="cuda")
+        self.token = torch.zeros(self.TOKEN_RING, dtype=torch.int32, device="cuda")
         self.ids = torch.zeros(4, dtype=torch.int32, device="cuda")
         self.attn_ws = torch.zeros(int(self.L.dh_attn_decode_workspace_bytes(H, D, max_seq)), dtype=torch.uint8,
                                    device="cuda")
@@ -104,14 +106,17 @@ class HipDecoder:
             q4 += synth.q4k_nbytes(n, k)
         return c["layers"] * q4 + c["vocab"] * c["hidden"] * 2 + c["layers"] * 2 * self.ks * 2 * ctx
 
-    def enqueue_step(self, pos, want_logits=False, from_device_token=False):
-        """Enqueue one decode step for the token id in self.ids[0] (or the previous step's
-        argmax when from_device_token) at position `pos`.  No host synchronisation."""
+    def enqueue_step(self, pos, want_logits=False, from_device_token=False, in_index=0, out_index=0):
+        """Enqueue one decode step for the token id in self.ids[0] (or, when from_device_token,
+        the argmax an earlier step left in self.token[in_index]) at position `pos`; the new
+        token goes to self.token[out_index].  No host synchronisation."""
         L, c = self.L, self.cfg
         ck = capi.check
         H, Hkv, D, Hd, I = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"], c["inter"]
         ids = self.token if from_device_token else self.ids
-        ck(L.dh_gather_f16(ids.data_ptr(), self.embed.data_ptr(), self.x.data_ptr(), 1, Hd, c["vocab"], 0))
+        ck(L.dh_gather_f16(ids.data_ptr(), self.embed.data_ptr(), self.x.data_ptr(), 1, Hd, c["vocab"],
+                           in_index if from_device_token else 0))
+        self._out_index = out_index
         x, x2 = self.x, self.x2
         if self.chain:
             return self._enqueue_chained(pos, want_logits)
@@ -148,7 +153,7 @@ class HipDecoder:
         ck(L.dh_rmsnorm(x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"],
                         0, None, None, None, 1.0))
         ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
-                                  self.lm_ws.data_ptr(), self.token.data_ptr(), 0,
+                                  self.lm_ws.data_ptr(), self.token.data_ptr(), self._out_index,
                                   self.logits.data_ptr() if want_logits else None))
 
     def _build_chains(self):
@@ -199,7 +204,7 @@ class HipDecoder:
         ck(L.dh_rmsnorm(self.x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd,
                         c["eps"], 0, None, None, None, 1.0))
         ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
-                                  self.lm_ws.data_ptr(), self.token.data_ptr(), 0,
+                                  self.lm_ws.data_ptr(), self.token.data_ptr(), self._out_index,
                                   self.logits.data_ptr() if want_logits else None))
 
     def set_token(self, token):
@@ -215,6 +220,20 @@ class HipDecoder:
         self.set_token(token)
         self.enqueue_step(pos, want_logits)
         return self.read_token()
+
+    def decode_batch(self, token, pos, n):
+        """n greedy steps per submit, as the reference's batched decode does
+        (src/inference/pipelines/text/generator-steps.js `shouldUseBatchDecode`, decode ring):
+        step i reads its input token from the device buffer step i-1 wrote, nothing crosses to
+        the host until all n steps are enqueued, then n token ids come back in one read."""
+        if not 1 <= n <= self.TOKEN_RING:
+            raise ValueError("decode_batch serves 1..%d tokens per submit, got %d" % (self.TOKEN_RING, n))
+        self.set_token(token)
+        for i in range(n):
+            self.enqueue_step(pos + i, from_device_token=i > 0, in_index=i - 1, out_index=i)
+        out = np.empty(n, np.uint32)
+        capi.check(self.L.dh_download(out.ctypes.data, self.token.data_ptr(), 0, 4 * n))
+        return [int(t) for t in out]
 
     def read_logits(self):
         out = np.empty(self.cfg["vocab"], np.float32)

@@ -63,6 +63,29 @@ def test_small_models_prefill_and_greedy(cfg, chain):
         assert rel_l2(v.view(np.float16).astype(np.float64), ev) <= 1e-3
 
 
+def test_batched_decode_matches_step_by_step():
+    """n tokens per submit with the token fed back on the device (the reference's batched decode)
+    gives the tokens of n single steps with a host round trip each."""
+    cfg = dict(layers=3, hidden=1024, inter=3072, heads=16, kv_heads=8, head_dim=128, vocab=2000, eps=1e-6, qk_norm=1,
+               max_seq=64, theta=1e6)
+    layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=31, max_seq=64)
+    a = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 64)
+    b = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 64)
+    prompt = [int(t) for t in synth.rng(32).integers(0, cfg["vocab"], 5)]
+    for pos, t in enumerate(prompt[:-1]):
+        a.step(t, pos)
+        b.step(t, pos)
+    tok, single = prompt[-1], []
+    for i in range(24):
+        tok = a.step(tok, len(prompt) - 1 + i)
+        single.append(tok)
+    batched = b.decode_batch(prompt[-1], len(prompt) - 1, 16)
+    batched += b.decode_batch(batched[-1], len(prompt) - 1 + 16, 8)
+    assert batched == single
+    with pytest.raises(ValueError):
+        b.decode_batch(1, 0, 65)
+
+
 @pytest.mark.timeout(1500)
 def test_9b_class_greedy_64_steps_identical_tokens():
     """BASELINE config 4: 36 layers, hidden 4096, FFN 12288, 32/8 heads of 128, vocab 151936,
