@@ -52,6 +52,7 @@ SIGNATURES = {
     "dh_lmhead_argmax_workspace_bytes": (_SZ, [_I]),
     "dh_lmhead_argmax_f16": (_I, [_P, _P, _I, _I, _I64, _F, _P, _P, _I, _P]),
     "dh_attn_decode_workspace_bytes": (_SZ, [_I, _I, _I]),
+    "dh_attn_prefill": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _F, _I]),
     "dh_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _F, _I, _I, _I, _P]),
     "dh_rmsnorm": (_I, [_P, _P, _I, _P, _I, _I, _F, _I, _P, _P, _P, _F]),
     "dh_rope": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I]),

@@ -1,0 +1,209 @@
+// Prefill attention (T query tokens at once) over an f16 KV cache with grouped-query heads, on the
+// matrix cores: the flash-attention recurrence with v_mfma_f32_16x16x32_f16.
+//
+// Grid = (query tiles of 64 tokens, query heads); a workgroup is 4 waves, wave w owns query rows
+// 16w..16w+15 of the tile.  Keys advance 64 at a time; the K and V tiles of the head's kv head
+// are staged in LDS once per workgroup and shared by the four waves.
+//
+// Everything is computed transposed, so that the softmax statistics of a query live in the lanes
+// that also hold its output column and nothing has to be shuffled between the two products:
+//   S^T = K . Q^T   A = K rows from LDS (16 bytes of a key row per lane), B = Q^T from registers
+//                   (scale folded in, rounded to f16).  D[key][q]: lane (q = l & 15, g = l >> 4)
+//                   gets keys 16j + 4g + i (i < 4) of key subtile j.
+//   softmax         per query = per lane column: maxima and sums over a lane's 16 values, then
+//                   across the four lanes l, l+16, l+32, l+48; fp32, online rescale.
+//   O^T = V^T . P^T B = P^T is exactly the lane's own probabilities (k-slot (g, i') stands for
+//                   key 16 (2 kb + i'/4) + 4g + i'%4 of 32-key block kb: a contraction index may be
+//                   renumbered as long as both operands agree), A = V^T read from LDS, where the
+//                   V tile was stored transposed with its keys in that same slot order.
+// Causal tiles beyond the tile's last query are never visited.
+#include <algorithm>
+#include <cfloat>
+
+#include "dh_common.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
+typedef __attribute__((ext_vector_type(4))) float float4_t;
+
+constexpr int BQ = 64, BKEYS = 64;
+
+struct PrefillArgs {
+  const float* Q;       // [T][H][D]
+  const __half* K;      // [rows][Hkv][D]
+  const __half* V;
+  float* O;             // [T][H][D]
+  int T, H, Hkv, G, kv_len, start_pos, causal, window;
+  float scale, softcap;
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) {
+  constexpr int STEPS = D / 32;            // MFMAs per 16 x 16 score tile
+  constexpr int DT = D / 16;               // output row tiles (of O^T)
+  constexpr int KROW = D + 8;              // halves per K row in LDS (16-byte pad)
+  constexpr int VROW = BKEYS + 8;          // halves per V^T row in LDS
+  constexpr int PIECES = BKEYS * D / 8 / 256;   // 16-byte pieces of a tile per thread
+  __shared__ __align__(16) _Float16 k_lds[BKEYS * KROW];
+  __shared__ __align__(16) _Float16 v_lds[D * VROW];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int q = lane & 15, g = lane >> 4;
+  const int h = blockIdx.y, kvh = h / a.G;
+  const int q0 = blockIdx.x * BQ;
+  const int my_q = q0 + 16 * wave + q;                        // query token of this lane's column
+  const int my_pos = a.start_pos + my_q;                      // its absolute position
+  const int64_t kv_stride = (int64_t)a.Hkv * D;
+
+  // ---- Q^T fragments (B operand): b[i] = scale * Q[my_q][32 s + 8 g + i]
+  half8_t qb[STEPS];
+#pragma unroll
+  for (int s = 0; s < STEPS; s++) {
+    const float* qp = a.Q + ((int64_t)min(my_q, a.T - 1) * a.H + h) * D + 32 * s + 8 * g;
+    const float4 v0 = reinterpret_cast<const float4*>(qp)[0], v1 = reinterpret_cast<const float4*>(qp)[1];
+    const float qv[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++) qb[s][i] = (_Float16)(qv[i] * a.scale);
+  }
+
+  // ---- key range of this query tile
+  const int last_q = min(q0 + BQ, a.T) - 1;
+  int kend = a.kv_len;
+  if (a.causal) kend = min(kend, a.start_pos + last_q + 1);
+  int kbeg = 0;
+  if (a.window > 0) kbeg = max(0, a.start_pos + q0 - a.window + 1);
+  kbeg = kbeg / BKEYS * BKEYS;
+  const int ntiles = (kend - kbeg + BKEYS - 1) / BKEYS;
+
+  float4_t acc[DT];
+#pragma unroll
+  for (int t = 0; t < DT; t++) acc[t] = {0.f, 0.f, 0.f, 0.f};
+  float m_run = -FLT_MAX, l_run = 0.f;
+
+  uint4 kreg[PIECES], vreg[PIECES];
+  // piece p = tid + 256 r of a tile: key p / (D/8), 8 consecutive dims starting at 8 (p % (D/8))
+#define DH_PF_LOAD(tile_)                                                                        \
+  _Pragma("unroll") for (int r = 0; r < PIECES; r++) {                                           \
+    const int p_ = tid + 256 * r, key_ = p_ / (D / 8), c_ = p_ % (D / 8);                        \
+    const int row_ = min(kbeg + (tile_) * BKEYS + key_, a.kv_len - 1);                           \
+    const int64_t off_ = (int64_t)row_ * kv_stride + (int64_t)kvh * D + 8 * c_;                  \
+    kreg[r] = *reinterpret_cast<const uint4*>(a.K + off_);                                       \
+    vreg[r] = *reinterpret_cast<const uint4*>(a.V + off_);                                       \
+  }
+  if (ntiles > 0) { DH_PF_LOAD(0); }
+
+  for (int kt = 0; kt < ntiles; kt++) {
+    __syncthreads();                                   // the previous tile has been consumed
+#pragma unroll
+    for (int r = 0; r < PIECES; r++) {
+      const int p = tid + 256 * r, key = p / (D / 8), c = p % (D / 8);
+      *reinterpret_cast<uint4*>(&k_lds[key * KROW + 8 * c]) = kreg[r];
+      // V^T with the keys in k-slot order: key = 32 kb + 16 jj + 4 gg + ii -> slot 32 kb + 8 gg + 4 jj + ii
+      const int kb = key >> 5, jj = (key >> 4) & 1, gg = (key >> 2) & 3, ii = key & 3;
+      const int slot = 32 * kb + 8 * gg + 4 * jj + ii;
+      const _Float16* hv = reinterpret_cast<const _Float16*>(&vreg[r]);
+#pragma unroll
+      for (int e = 0; e < 8; e++) v_lds[(8 * c + e) * VROW + slot] = hv[e];
+    }
+    __syncthreads();
+    if (kt + 1 < ntiles) { DH_PF_LOAD(kt + 1); }
+
+    // ---- S^T for this wave's 16 queries against the 64 keys
+    const int kbase = kbeg + kt * BKEYS;
+    float4_t st[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      st[j] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < STEPS; s++) {
+        const half8_t ka = *reinterpret_cast<const half8_t*>(&k_lds[(16 * j + q) * KROW + 32 * s + 8 * g]);
+        st[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[s], st[j], 0, 0, 0);
+      }
+    }
+    // ---- mask, soft cap, online softmax (this lane: query my_q, keys kbase + 16 j + 4 g + i)
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int key = kbase + 16 * j + 4 * g + i;
+        float s = st[j][i];
+        if (a.softcap > 0.f) s = tanhf(s / a.softcap) * a.softcap;
+        bool ok = key < a.kv_len;
+        if (a.causal) ok = ok && key <= my_pos;
+        if (a.window > 0) ok = ok && key > my_pos - a.window;
+        s = ok ? s : -INFINITY;
+        st[j][i] = s;
+        mx = fmaxf(mx, s);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);              // finite: m_run starts at -FLT_MAX
+    const float alpha = __expf(m_run - m_new);
+    float ps = 0.f;
+    half8_t pb[2];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const float p = __expf(st[j][i] - m_new);      // exp(-inf) = 0 for masked keys
+        ps += p;
+        pb[j >> 1][4 * (j & 1) + i] = (_Float16)p;
+      }
+    ps += __shfl_xor(ps, 16, 64);
+    ps += __shfl_xor(ps, 32, 64);
+    l_run = l_run * alpha + ps;
+    m_run = m_new;
+    // ---- O^T = alpha O^T + V^T P^T
+#pragma unroll
+    for (int t = 0; t < DT; t++) {
+      acc[t] *= alpha;
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++) {
+        const half8_t va = *reinterpret_cast<const half8_t*>(&v_lds[(16 * t + q) * VROW + 32 * kb + 8 * g]);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[kb], acc[t], 0, 0, 0);
+      }
+    }
+  }
+#undef DH_PF_LOAD
+
+  // ---- lane (q, g) holds O[my_q][16 t + 4 g + i]
+  if (my_q < a.T) {
+    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+    float* op = a.O + ((int64_t)my_q * a.H + h) * D + 4 * g;
+#pragma unroll
+    for (int t = 0; t < DT; t++)
+      *reinterpret_cast<float4*>(op + 16 * t) = make_float4(acc[t][0] * inv, acc[t][1] * inv, acc[t][2] * inv, acc[t][3] * inv);
+  }
+}
+
+}  // namespace
+
+extern "C" int dh_attn_prefill(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int T, int H,
+                               int Hkv, int D, int kv_len, float scale, int causal, int start_pos,
+                               float softcap, int sliding_window) {
+  const char* op = "dh_attn_prefill";
+  DH_REQUIRE_INIT(op);
+  if (T <= 0 || H <= 0 || Hkv <= 0 || D <= 0)
+    return dh::fail(1, "[%s] seqLen/numHeads/numKVHeads/headDim must be positive", op);
+  if (H % Hkv) return dh::fail(1, "[%s] numHeads=%d must be a multiple of numKVHeads=%d", op, H, Hkv);
+  if (D != 64 && D != 128) return dh::fail(1, "[%s] headDim %d not supported (64, 128)", op, D);
+  if (kv_len <= 0 || start_pos < 0 || sliding_window < 0)
+    return dh::fail(1, "[%s] kvLen must be positive, startPos and slidingWindow non-negative", op);
+  if (causal && start_pos + T > kv_len)
+    return dh::fail(1, "[%s] startPos=%d + seqLen=%d exceeds kvLen=%d", op, start_pos, T, kv_len);
+  if (!d_Q || !d_K || !d_V || !d_O) return dh::fail(1, "[%s] null pointer", op);
+  if ((reinterpret_cast<uintptr_t>(d_K) | reinterpret_cast<uintptr_t>(d_V) | reinterpret_cast<uintptr_t>(d_Q) |
+       reinterpret_cast<uintptr_t>(d_O)) & 15)
+    return dh::fail(1, "[%s] Q/K/V/O pointers must be 16-byte aligned", op);
+  PrefillArgs a{};
+  a.Q = d_Q; a.K = static_cast<const __half*>(d_K); a.V = static_cast<const __half*>(d_V); a.O = d_O;
+  a.T = T; a.H = H; a.Hkv = Hkv; a.G = H / Hkv; a.kv_len = kv_len; a.start_pos = start_pos;
+  a.causal = causal ? 1 : 0; a.window = sliding_window; a.scale = scale; a.softcap = softcap;
+  const dim3 grid((unsigned)dh::ceil_div(T, BQ), (unsigned)H);
+  if (D == 64) hipLaunchKernelGGL(attn_prefill_kernel<64>, grid, dim3(256), 0, dh::stream(), a);
+  else hipLaunchKernelGGL(attn_prefill_kernel<128>, grid, dim3(256), 0, dh::stream(), a);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}

@@ -29,6 +29,9 @@ unsigned* chain_counters();
 // Scratch for the split-K prefill GEMM's partial products (allocated by dh_init, shared by all
 // launches on the library's stream, which run in order).
 float* splitk_workspace(size_t* bytes);
+// Per-row scale factors of the prefill GEMM's activations: capacity rows x (multiplier, inverse).
+float* gemm_row_scale();
+int gemm_row_scale_capacity();
 unsigned* chain_error_flag();
 unsigned chain_advance(unsigned n);
 

@@ -16,6 +16,8 @@ unsigned* g_chain_mem = nullptr;     // [8 * 64] barrier counters + [1] error fl
 unsigned g_chain_value = 0;          // what every counter reads once the enqueued launches are done
 float* g_splitk_ws = nullptr;        // partial products of the split-K prefill GEMM
 constexpr size_t kSplitKWsBytes = (size_t)32 << 20;
+float* g_row_scale = nullptr;        // [kRowScaleRows][2] activation row factors of the prefill GEMM
+constexpr int kRowScaleRows = 65536;
 constexpr size_t kChainWords = 8 * 64 + 64;
 }  // namespace
 
@@ -34,6 +36,8 @@ float* splitk_workspace(size_t* bytes) {
   *bytes = g_splitk_ws ? kSplitKWsBytes : 0;
   return g_splitk_ws;
 }
+float* gemm_row_scale() { return g_row_scale; }
+int gemm_row_scale_capacity() { return kRowScaleRows; }
 unsigned* chain_counters() { return g_chain_mem; }
 unsigned* chain_error_flag() { return g_chain_mem ? g_chain_mem + 8 * 64 : nullptr; }
 unsigned chain_advance(unsigned n) {
@@ -71,6 +75,7 @@ int dh_init(int device_ordinal) {
   DH_CHECK_HIP("dh_init", hipMemset(g_chain_mem, 0, kChainWords * sizeof(unsigned)));
   g_chain_value = 0;
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_splitk_ws), kSplitKWsBytes));
+  DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_row_scale), (size_t)kRowScaleRows * 2 * sizeof(float)));
   g_device = device_ordinal;
   g_ready = true;
   return 0;
@@ -85,6 +90,8 @@ int dh_shutdown(void) {
   g_chain_mem = nullptr;
   if (g_splitk_ws) DH_CHECK_HIP("dh_shutdown", hipFree(g_splitk_ws));
   g_splitk_ws = nullptr;
+  if (g_row_scale) DH_CHECK_HIP("dh_shutdown", hipFree(g_row_scale));
+  g_row_scale = nullptr;
   g_own_stream = nullptr;
   g_stream = nullptr;
   g_ready = false;

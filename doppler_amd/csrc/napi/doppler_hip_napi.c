@@ -178,6 +178,11 @@ FN(js_attn_decode) {
   return ret_rc(env, dh_attn_decode((const float*)Q, K, V, (float*)O, H, Hkv, D, kvLen, scale, causal, startPos, cap, win,
                                     kvStart, layout, ws));
 }
+FN(js_attn_prefill) {
+  ARGS(14); P(0, Q); P(1, K); P(2, V); P(3, O); I(4, T); I(5, H); I(6, Hkv); I(7, D); I(8, kvLen); F(9, scale);
+  I(10, causal); I(11, startPos); F(12, cap); I(13, win);
+  return ret_rc(env, dh_attn_prefill((const float*)Q, K, V, (float*)O, T, H, Hkv, D, kvLen, scale, causal, startPos, cap, win));
+}
 FN(js_rmsnorm) {
   ARGS(12); P(0, x); P(1, w); I(2, wdt); P(3, o); I(4, batch); I(5, hid); F(6, eps); I(7, woff); P(8, pre); P(9, post);
   P(10, prenorm); F(11, oscale);
@@ -224,6 +229,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"q4kMatmulRmsnorm", js_q4k_matmul_rmsnorm}, {"q4kFfnGateUpRmsnorm", js_q4k_ffn_gate_up_rmsnorm},
       {"lmheadArgmaxWorkspaceBytes", js_lmhead_argmax_workspace_bytes}, {"lmheadArgmaxF16", js_lmhead_argmax_f16},
       {"attnDecodeWorkspaceBytes", js_attn_decode_workspace_bytes}, {"attnDecode", js_attn_decode},
+      {"attnPrefill", js_attn_prefill},
       {"rmsnorm", js_rmsnorm}, {"rope", js_rope}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},
       {"kvWriteF16", js_kv_write_f16}, {"residualAdd", js_residual_add}, {"gatherF16", js_gather_f16},
       {"actGate", js_act_gate}, {"actGateRowsplit", js_act_gate_rowsplit},

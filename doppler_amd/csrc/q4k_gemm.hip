@@ -8,7 +8,10 @@
 //            as f16: (w & 0x000F000F) | 0x64006400 is the pair (1024 + q) in f16, one packed
 //            subtract and one packed fma with (d*sc, -dmin*mn) finish them: about 2 vector ops
 //            per weight, paid once per 128 rows of A.
-//   A        f32 -> f16 on the way into LDS.
+//   A        f32 -> f16 on the way into LDS, each row scaled by a power of two first so that its
+//            largest element sits at 2^14 (a row-maximum pre-pass writes the factors; the
+//            epilogue divides them out again, exactly): activations beyond the f16 range
+//            (65504) neither overflow nor lose small rows to subnormals.
 // Both tiles sit in LDS as [row][64 k] with a 16-byte pad (conflict-free 16-byte fragment
 // reads) and are double-buffered: the global loads of tile t+1 are issued before tile t is
 // multiplied, one barrier per K step.
@@ -52,7 +55,34 @@ struct GemmArgs {
   // partial[z][M][N]; splitk_reduce_kernel adds the pieces in order
   int ksplit, kt_per_split;
   float* partial;
+  const float2* row_scale;   // [M] (multiplier applied before the f16 rounding, its inverse)
 };
+
+// One wave per activation row (four rows per workgroup): power-of-two factor that puts the row's
+// largest magnitude at 2^14; (1, 1) for an all-zero row.
+__global__ __launch_bounds__(256) void row_scale_kernel(const float* __restrict__ A, int M, int K,
+                                                        float2* __restrict__ out) {
+  const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (m >= M) return;
+  const float* row = A + (int64_t)m * K;
+  float mx = 0.f;
+  if ((K & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    for (int k = 4 * lane; k < K; k += 256) {
+      const float4 v = *reinterpret_cast<const float4*>(row + k);
+      mx = fmaxf(fmaxf(mx, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) mx = fmaxf(mx, fabsf(row[k]));
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  if (lane == 0) {
+    int e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
+    e = max(-100, min(100, e));
+    if (!(mx > 0.f) || !(mx < INFINITY)) e = 14;
+    out[m] = make_float2(__uint_as_float((uint32_t)(127 + 14 - e) << 23), __uint_as_float((uint32_t)(127 - 14 + e) << 23));
+  }
+}
 
 // 16 nibble bytes -> 16 low-nibble and 16 high-nibble weights as f16, k order (0,2,1,3) per dword.
 __device__ __forceinline__ void dequant16(const uint4 q, float sc_lo, float mn_lo, float sc_hi, float mn_hi,
@@ -114,6 +144,13 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
   const bool w_active = w_row < BN;
   float4 a_reg[NA];
   uint4 q_reg[NMAT], h_reg[NMAT];
+  // row factors of this tile's activation rows: one global read each, then LDS
+  __shared__ float2 rs_lds[BM];
+  if (tid < BM) rs_lds[tid] = a.row_scale[min(m0 + tid, a.M - 1)];
+  __syncthreads();
+  float a_mul[NA];
+#pragma unroll
+  for (int i = 0; i < NA; i++) a_mul[i] = rs_lds[(tid + 256 * i) >> 4].x;
 
   auto load_tile = [&](int kt) {
 #pragma unroll
@@ -138,8 +175,9 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
 #pragma unroll
     for (int i = 0; i < NA; i++) {
       const int idx = tid + 256 * i, r = idx >> 4, kl = 4 * (idx & 15);
-      const half2_t p0 = {(_Float16)a_reg[i].x, (_Float16)a_reg[i].z};    // k order (0, 2, 1, 3)
-      const half2_t p1 = {(_Float16)a_reg[i].y, (_Float16)a_reg[i].w};
+      const float ml = a_mul[i];
+      const half2_t p0 = {(_Float16)(a_reg[i].x * ml), (_Float16)(a_reg[i].z * ml)};    // k order (0, 2, 1, 3)
+      const half2_t p1 = {(_Float16)(a_reg[i].y * ml), (_Float16)(a_reg[i].w * ml)};
       *reinterpret_cast<uint2*>(At + r * LDS_ROW + kl) =
           make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
     }
@@ -211,16 +249,17 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
         const int m = m0 + wm + 32 * i + 8 * (e >> 2) + 4 * fg + (e & 3);
         if (m < a.M && n < a.N) {
           float v;
+          const float unscale = rs_lds[wm + 32 * i + 8 * (e >> 2) + 4 * fg + (e & 3)].y;
           if (!DUAL && a.ksplit > 1) {
-            a.partial[((int64_t)blockIdx.z * a.M + m) * a.N + n] = acc[0][i][j][e];
+            a.partial[((int64_t)blockIdx.z * a.M + m) * a.N + n] = acc[0][i][j][e] * unscale;
             continue;
           }
           if (DUAL) {
-            const float g = acc[0][i][j][e], u = acc[NMAT - 1][i][j][e];
+            const float g = acc[0][i][j][e] * unscale, u = acc[NMAT - 1][i][j][e] * unscale;
             v = (a.activation == DH_ACT_SILU ? act_silu(g) : gelu_tanh_fast(g)) * u * a.alpha;
             if (a.activation == DH_ACT_SILU && a.clamp_max > 0.f) v = fminf(fmaxf(v, -a.clamp_max), a.clamp_max);
           } else {
-            v = acc[0][i][j][e] * a.alpha;
+            v = acc[0][i][j][e] * unscale * a.alpha;
             if (a.residual) v += a.residual[(int64_t)m * a.N + n];
           }
           if (a.c_f16)
@@ -273,6 +312,27 @@ int launch_gemm_cfg(const GemmArgs& a, const char* op) {
 // share wins from there on), else 64 x 64.
 template <bool DUAL>
 int launch_gemm(GemmArgs a, const char* op) {
+  // rows beyond the scale buffer's capacity go in further passes
+  const int cap = dh::gemm_row_scale_capacity();
+  if (a.M > cap) {
+    const size_t c_elem = a.c_f16 ? 2 : 4;
+    for (int m0 = 0; m0 < a.M; m0 += cap) {
+      GemmArgs b = a;
+      b.M = std::min(cap, a.M - m0);
+      b.A = a.A + (int64_t)m0 * a.K;
+      b.C = static_cast<char*>(a.C) + (int64_t)m0 * a.N * c_elem;
+      b.residual = a.residual ? a.residual + (int64_t)m0 * a.N : nullptr;
+      const int rc = launch_gemm<DUAL>(b, op);
+      if (rc) return rc;
+    }
+    return 0;
+  }
+  float2* scales = reinterpret_cast<float2*>(dh::gemm_row_scale());
+  if (!scales) return dh::fail(2, "[%s] the library's scratch buffers are missing (dh_init)", op);
+  hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)dh::ceil_div(a.M, 4)), dim3(256), 0, dh::stream(), a.A, a.M, a.K,
+                     scales);
+  DH_CHECK_LAUNCH(op);
+  a.row_scale = scales;
   const int64_t big_tiles = dh::ceil_div(a.M, 128) * dh::ceil_div(a.N, 128);
   a.ksplit = 1;
   if (2 * big_tiles >= dh::num_cus()) return launch_gemm_cfg<DUAL, 2>(a, op);

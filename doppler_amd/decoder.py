@@ -221,6 +221,64 @@ class HipDecoder:
         self.enqueue_step(pos, want_logits)
         return self.read_token()
 
+    def prefill(self, tokens, start_pos=0, chunk=512, want_logits=False):
+        """Pushes a prompt through the batched path, `chunk` tokens at a time: Q4_K prefill GEMMs,
+        the T-token fused QKV-norm-RoPE-KV-write, matrix-core prefill attention.  KV rows
+        start_pos .. start_pos + len(tokens) - 1 are written; returns the greedy token after the
+        last prompt token (the reference's prefill, src/inference/pipelines/text/generator.js)."""
+        L, c, ck = self.L, self.cfg, capi.check
+        H, Hkv, D, Hd, I = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"], c["inter"]
+        tokens = np.asarray(tokens, np.uint32).reshape(-1)
+        if tokens.size == 0 or start_pos + tokens.size > self.max_seq:
+            raise ValueError("prefill of %d tokens at %d does not fit max_seq=%d" % (tokens.size, start_pos, self.max_seq))
+        chunk = max(1, min(chunk, tokens.size))
+        if getattr(self, "_pf_rows", 0) < chunk:
+            f32 = lambda n: torch.zeros(n, dtype=torch.float32, device="cuda")
+            self._pf = dict(x=f32(chunk * Hd), x2=f32(chunk * Hd), normed=f32(chunk * Hd),
+                            qkv=f32(chunk * (self.qs + 2 * self.ks)), q=f32(chunk * self.qs), attn=f32(chunk * self.qs),
+                            act=f32(chunk * I), ids=torch.zeros(chunk, dtype=torch.int32, device="cuda"))
+            self._pf_rows = chunk
+        b = self._pf
+        qkv_n = self.qs + 2 * self.ks
+        for c0 in range(0, tokens.size, chunk):
+            ids = np.ascontiguousarray(tokens[c0:c0 + chunk])
+            T, pos = ids.size, start_pos + c0
+            ck(L.dh_upload(b["ids"].data_ptr(), 0, ids.ctypes.data, 4 * T))
+            ck(L.dh_gather_f16(b["ids"].data_ptr(), self.embed.data_ptr(), b["x"].data_ptr(), T, Hd, c["vocab"], 0))
+            x, x2 = b["x"], b["x2"]
+            for d in self.layers:
+                ck(L.dh_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), capi.F32, b["normed"].data_ptr(), T, Hd,
+                                c["eps"], 0, None, None, None, 1.0))
+                ck(L.dh_q4k_matmul(b["normed"].data_ptr(), capi.F32, d["wqkv"].data_ptr(), b["qkv"].data_ptr(), capi.F32,
+                                   T, qkv_n, Hd, 1.0, None))
+                ck(L.dh_qkv_norm_rope_kvwrite(b["qkv"].data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
+                                              self.cos.data_ptr(), self.sin.data_ptr(), b["q"].data_ptr(),
+                                              d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), T, H, Hkv, D, pos, D, 0,
+                                              c["eps"], 0, pos * self.ks, int(c.get("qk_norm", 1))))
+                if T == 1:
+                    ck(L.dh_attn_decode(b["q"].data_ptr(), d["cache_k"].data_ptr(), d["cache_v"].data_ptr(),
+                                        b["attn"].data_ptr(), H, Hkv, D, pos + 1, self.scale, 1, pos, 0.0, 0, 0,
+                                        capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
+                else:
+                    ck(L.dh_attn_prefill(b["q"].data_ptr(), d["cache_k"].data_ptr(), d["cache_v"].data_ptr(),
+                                         b["attn"].data_ptr(), T, H, Hkv, D, pos + T, self.scale, 1, pos, 0.0, 0))
+                ck(L.dh_q4k_matmul(b["attn"].data_ptr(), capi.F32, d["wo"].data_ptr(), x2.data_ptr(), capi.F32, T, Hd,
+                                   self.qs, 1.0, x.data_ptr()))
+                ck(L.dh_rmsnorm(x2.data_ptr(), d["post_attn_norm"].data_ptr(), capi.F32, b["normed"].data_ptr(), T, Hd,
+                                c["eps"], 0, None, None, None, 1.0))
+                ck(L.dh_q4k_ffn_gate_up(b["normed"].data_ptr(), d["wgate"].data_ptr(), d["wup"].data_ptr(),
+                                        b["act"].data_ptr(), T, Hd, I, capi.ACT_SILU, 1.0, 0.0))
+                ck(L.dh_q4k_matmul(b["act"].data_ptr(), capi.F32, d["wdown"].data_ptr(), x.data_ptr(), capi.F32, T, Hd, I,
+                                   1.0, x2.data_ptr()))
+        # logits of the last prompt token only
+        last = b["x"].data_ptr() + (T - 1) * Hd * 4
+        ck(L.dh_rmsnorm(last, self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"], 0, None,
+                        None, None, 1.0))
+        ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
+                                  self.lm_ws.data_ptr(), self.token.data_ptr(), 0,
+                                  self.logits.data_ptr() if want_logits else None))
+        return self.read_token()
+
     def decode_batch(self, token, pos, n):
         """n greedy steps per submit, as the reference's batched decode does
         (src/inference/pipelines/text/generator-steps.js `shouldUseBatchDecode`, decode ring):

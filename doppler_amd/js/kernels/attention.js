@@ -1,4 +1,4 @@
-// runAttention / recordAttention for decode (seqLen 1) over an f16 KV cache:
+// runAttention / recordAttention over an f16 KV cache, decode (seqLen 1) and prefill (seqLen > 1):
 // reference src/gpu/kernels/attention.js:1047-1310,2007-2030.
 import { getNative, KV_LAYOUT } from '../native.js';
 import { createTensor } from '../tensor.js';
@@ -19,11 +19,11 @@ async function executeAttention(recorder, Q, K, V, mask, numHeads, headDim, opti
     kvStart = 0,
     kvLayout = 'contiguous',
   } = options;
-  if (seqLen !== 1) {
-    throw new Error(`[Attention] the HIP path serves decode (seqLen=1) only, got seqLen=${seqLen}.`);
+  if (!(seqLen >= 1)) {
+    throw new Error(`[Attention] seqLen must be positive, got ${seqLen}.`);
   }
   if (mask) {
-    throw new Error('[Attention] explicit masks are not supported on the decode path.');
+    throw new Error('[Attention] explicit masks are not supported on the HIP path.');
   }
   if (!(kvLayout in KV_LAYOUT)) {
     throw new Error(`[Attention] kvLayout "${kvLayout}" is not supported by the HIP path (contiguous, ring).`);
@@ -37,6 +37,21 @@ async function executeAttention(recorder, Q, K, V, mask, numHeads, headDim, opti
     throw new Error(`[Attention] KV buffers are smaller than kvLen=${kvLen} rows (${kvBytes} bytes).`);
   }
   const native = getNative();
+  if (seqLen > 1) {
+    if (kvLayout !== 'contiguous' || kvStart !== 0) {
+      throw new Error(`[Attention] prefill (seqLen=${seqLen}) needs a contiguous cache with kvStart=0.`);
+    }
+    const out = outputBuffer || acquireBuffer(seqLen * numHeads * headDim * 4, undefined, 'attention_output');
+    try {
+      native.attnPrefill(Q.buffer.ptr, K.buffer.ptr, V.buffer.ptr, out.ptr, seqLen, numHeads, numKVHeads, headDim, kvLen,
+        scale, causal ? 1 : 0, startPos, attnSoftcap, slidingWindow);
+    } catch (error) {
+      if (!outputBuffer) releaseBuffer(out);
+      throw error;
+    }
+    noteDispatch(recorder, 'attention');
+    return createTensor(out, 'f32', [seqLen, numHeads, headDim], 'attention_output');
+  }
   const outputSize = seqLen * padToQ4KBlock(numHeads * headDim) * 4;
   const output = outputBuffer || acquireBuffer(outputSize, undefined, 'attention_output');
   const owned = outputBuffer ? null : output;

@@ -276,19 +276,30 @@ def attentionWorkspaceBytes(numHeads, headDim, kvLen):
 def runAttention(Q, K, V, mask, numHeads, headDim, seqLen=1, kvLen=None, numKVHeads=None, scale=None,
                  causal=True, startPos=0, outputBuffer=None, attnSoftcap=0, slidingWindow=0, kvStart=0,
                  kvLayout="contiguous", workspace=None, **_ignored):
-    """src/gpu/kernels/attention.js:2007 runAttention, decode (seqLen == 1) over an f16 KV cache."""
+    """src/gpu/kernels/attention.js:2007 runAttention over an f16 KV cache: decode (seqLen == 1,
+    split-K kernel) or prefill (seqLen > 1, matrix-core flash kernel)."""
     kvLen = seqLen if kvLen is None else kvLen
     numKVHeads = numHeads if numKVHeads is None else numKVHeads
     scale = 1.0 / math.sqrt(headDim) if scale is None else scale
-    if seqLen != 1:
-        raise DopplerHipError("[Attention] only decode (seqLen=1) runs on the HIP path, got seqLen=%d" % seqLen)
+    if seqLen < 1:
+        raise DopplerHipError("[Attention] seqLen must be positive, got %d" % seqLen)
     if mask is not None:
-        raise DopplerHipError("[Attention] explicit masks are not supported on the decode path")
+        raise DopplerHipError("[Attention] explicit masks are not supported on the HIP path")
     if Q.dtype != "f32" or K.dtype != "f16" or V.dtype != "f16":
-        raise DopplerHipError("[Attention] decode path needs f32 Q and f16 K/V (got %s/%s/%s)" % (Q.dtype, K.dtype, V.dtype))
+        raise DopplerHipError("[Attention] the HIP path needs f32 Q and f16 K/V (got %s/%s/%s)" % (Q.dtype, K.dtype, V.dtype))
     layouts = {"contiguous": capi.KV_CONTIGUOUS, "ring": capi.KV_RING}
     if kvLayout not in layouts:
         raise DopplerHipError("[Attention] kvLayout %r is not supported by the HIP path" % (kvLayout,))
+    if seqLen > 1:
+        if kvLayout != "contiguous" or kvStart != 0:
+            raise DopplerHipError("[Attention] prefill (seqLen=%d) needs a contiguous cache with kvStart=0" % seqLen)
+        if min(_nbytes(K), _nbytes(V)) < kvLen * numKVHeads * headDim * 2:
+            raise DopplerHipError("[Attention] KV buffer smaller than kvLen=%d rows" % kvLen)
+        out = _out(outputBuffer, seqLen * numHeads * headDim * 4)
+        capi.check(_lib().dh_attn_prefill(_ptr(Q), _ptr(K), _ptr(V), out.data_ptr(), seqLen, numHeads, numKVHeads,
+                                          headDim, kvLen, scale, int(bool(causal)), startPos, float(attnSoftcap),
+                                          slidingWindow))
+        return Tensor(out, "f32", (seqLen, numHeads, headDim), "attention_output")
     rows = slidingWindow if kvLayout == "ring" else kvStart + kvLen
     if kvLen > 0 and min(_nbytes(K), _nbytes(V)) < rows * numKVHeads * headDim * 2:
         raise DopplerHipError("[Attention] KV buffer smaller than kvLen=%d rows" % kvLen)

@@ -159,6 +159,14 @@ int dh_lmhead_argmax_f16(const float* d_h, const void* d_E, int vocab, int hidde
  * O f32 [H][D].  kv_layout DH_KV_RING reads row (kv_start+k) % sliding_window.
  * d_workspace needs dh_attn_decode_workspace_bytes(H, D, kv_len) bytes (split-K partials). */
 size_t dh_attn_decode_workspace_bytes(int H, int D, int kv_len);
+/* Prefill attention: T query tokens (Q f32 [T][H][D], already rotated) against the f16 cache rows
+ * [0, kv_len), query t at absolute position start_pos + t; causal and sliding-window masks as in
+ * the decode op; contiguous cache layout.  Replaces runAttention/recordAttention for seqLen > 1,
+ * src/gpu/kernels/attention.js:1047-1310 (attention_streaming_f16kv.wgsl and the tiled prefill
+ * variants).  Scores and P.V run on the matrix cores with f16 inputs and f32 accumulation. */
+int dh_attn_prefill(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int T, int H,
+                    int Hkv, int D, int kv_len, float scale, int causal, int start_pos,
+                    float softcap, int sliding_window);
 int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H,
                    int Hkv, int D, int kv_len, float scale, int causal, int start_pos,
                    float softcap, int sliding_window, int kv_start, int kv_layout,

@@ -63,6 +63,38 @@ def test_small_models_prefill_and_greedy(cfg, chain):
         assert rel_l2(v.view(np.float16).astype(np.float64), ev) <= 1e-3
 
 
+@pytest.mark.parametrize("chunk", [512, 20])
+def test_prefill_path_matches_the_oracle(chunk):
+    """Prompt through the batched path (prefill GEMMs + prefill attention, f16 matrix-core
+    inputs): last-token logits and the KV cache within relative L2 5e-3 of the CPU oracle run
+    token by token, then greedy decode continues from that cache with identical tokens."""
+    cfg = dict(layers=3, hidden=1024, inter=3072, heads=16, kv_heads=8, head_dim=128, vocab=2000, eps=1e-6, qk_norm=1,
+               max_seq=96, theta=1e6)
+    layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=41, max_seq=96)
+    gpu = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 96)
+    ol = oracle_layers(layers, 96, cfg["kv_heads"], cfg["head_dim"])
+    cpu = oracle.DecoderOracle(cfg, ol, embed, final_norm, cos, sin)
+    prompt = [int(t) for t in synth.rng(42).integers(0, cfg["vocab"], 50)]
+    tok = gpu.prefill(prompt, chunk=chunk, want_logits=True)
+    for pos, t in enumerate(prompt):
+        ctok, want = cpu.step(t, pos, want_logits=True)
+    assert rel_l2(gpu.read_logits(), want) <= 5e-3
+    for i in range(cfg["layers"]):
+        k, v = gpu.read_kv(i, len(prompt))
+        ek = ol[i]["cache_k"][:len(prompt)].reshape(-1).view(np.float16).astype(np.float64)
+        ev = ol[i]["cache_v"][:len(prompt)].reshape(-1).view(np.float16).astype(np.float64)
+        assert rel_l2(k.view(np.float16).astype(np.float64), ek) <= 5e-3
+        assert rel_l2(v.view(np.float16).astype(np.float64), ev) <= 5e-3
+    # the top-1 margin of a random model at this size is far above the 5e-3 band
+    assert tok == ctok
+    # continue decoding on the GPU from the prefilled cache; the checker continues from its own
+    for i in range(8):
+        nxt = gpu.step(tok, len(prompt) + i)
+        cn = cpu.step(tok, len(prompt) + i)
+        assert nxt == cn, i
+        tok = nxt
+
+
 def test_batched_decode_matches_step_by_step():
     """n tokens per submit with the token fed back on the device (the reference's batched decode)
     gives the tokens of n single steps with a host round trip each."""

@@ -123,6 +123,24 @@ def test_matmul_prefill_gemm(M, N, K, kw):
     assert _matmul_case(M, N, K, seed=1500 + M, **kw) <= REL_L2_F16_MFMA
 
 
+def test_matmul_prefill_gemm_activation_range():
+    """Rows far outside the f16 range (and far below it) go through the f16 matrix-core path: each
+    row is scaled by its own power of two before rounding."""
+    M, N, K = 64, 192, 1024
+    W, wb = q4k_weight(N, K, seed=1600)
+    A = synth.normal_f32((M, K), seed=1601)
+    A[::3] *= 1e7
+    A[1::3] *= 1e-9
+    A[5] = 0.0
+    out = ops.runMatmul(ops.tensorFromNumpy(A), wb, M, N, K, outputDtype="f32", role="test")
+    got = ops.readTensor(out).reshape(M, N)
+    want = oracle.q4k_matmul(A, W, M, N, K).reshape(M, N)
+    assert np.isfinite(got).all()
+    for m in range(M):
+        assert rel_l2(got[m], want[m]) <= REL_L2_F16_MFMA or not want[m].any(), m
+    assert not got[5].any()
+
+
 @pytest.mark.parametrize("M,activation", [(512, "gelu"), (48, "silu")])
 def test_fused_ffn_prefill_cfg2(M, activation):
     hidden, inter = synth.CFG2["hidden"], synth.CFG2["inter"]
@@ -503,3 +521,65 @@ def test_attention_decode_options():
     assert not got.any()
     with pytest.raises(DopplerHipError, match="kvLayout"):
         ops.runAttention(qt, kt, vt, None, H, D, kvLen=ctx, numKVHeads=Hkv, kvLayout="paged")
+
+
+# ----------------------------------------------------------------------------- prefill attention
+
+def _prefill_oracle(q, kb, vb, T, H, Hkv, D, kv_len, start_pos, causal=True, window=0, softcap=0.0, scale=None):
+    """Oracle for T query rows: each row is one decode-attention problem at its own position."""
+    out = np.empty((T, H, D), np.float32)
+    for t in range(T):
+        out[t] = oracle.attention_decode_f16kv(q[t], kb, vb, H, Hkv, D, kv_len, scale=scale, causal=causal,
+                                               start_pos=start_pos + t, sliding_window=window, softcap=softcap).reshape(H, D)
+    return out
+
+
+@pytest.mark.parametrize("T,start,H,Hkv,D", [(64, 0, 16, 8, 128), (200, 56, 16, 8, 128), (7, 0, 4, 4, 64),
+                                            (130, 300, 8, 2, 64), (512, 0, 32, 8, 128), (33, 1000, 32, 8, 128)])
+def test_attention_prefill_causal(T, start, H, Hkv, D):
+    """seqLen > 1: query t at position start + t sees keys 0..start + t (the reference's causal
+    prefill, attention.js:1047-1080 with createCausalMask semantics).  f16 matrix-core inputs."""
+    kv_len = start + T
+    cos, sin = synth.rope_tables(D, kv_len, 1e6)
+    q = synth.normal_f32((T, H, D), 6000 + T, D ** -0.5)
+    k = synth.normal_f32((kv_len, Hkv, D), 6001 + T, D ** -0.5)
+    v = synth.normal_f32((kv_len, Hkv, D), 6002 + T, D ** -0.5)
+    q = oracle.rope_apply(q, cos, sin, T, H, D, start_pos=start).reshape(T, H, D) * 4.0
+    k = oracle.rope_apply(k, cos, sin, kv_len, Hkv, D, start_pos=0)
+    kb, vb = k.astype(np.float16).view(np.uint16), v.astype(np.float16).view(np.uint16)
+    out = ops.runAttention(ops.tensorFromNumpy(q), ops.tensorFromNumpy(kb), ops.tensorFromNumpy(vb), None, H, D,
+                           seqLen=T, kvLen=kv_len, numKVHeads=Hkv, causal=True, startPos=start)
+    assert out.shape == (T, H, D)
+    got = ops.readTensor(out).reshape(T, H, D)
+    want = _prefill_oracle(q, kb, vb, T, H, Hkv, D, kv_len, start)
+    assert rel_l2(got, want) <= REL_L2_F16_MFMA
+    # row by row as well: early rows see few keys and must not be polluted by masked ones
+    for t in (0, T // 2, T - 1):
+        assert rel_l2(got[t], want[t]) <= REL_L2_F16_MFMA, t
+
+
+def test_attention_prefill_options_and_errors():
+    T, start, H, Hkv, D = 96, 40, 8, 4, 128
+    kv_len = start + T
+    q = synth.normal_f32((T, H, D), 6100, 1.0)
+    kb = synth.normal_f32((kv_len, Hkv, D), 6101, D ** -0.5).astype(np.float16).view(np.uint16)
+    vb = synth.normal_f32((kv_len, Hkv, D), 6102, 1.0).astype(np.float16).view(np.uint16)
+    qt, kt, vt = ops.tensorFromNumpy(q), ops.tensorFromNumpy(kb), ops.tensorFromNumpy(vb)
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, seqLen=T, kvLen=kv_len, numKVHeads=Hkv, startPos=start,
+                                          slidingWindow=50, scale=0.2))
+    want = _prefill_oracle(q, kb, vb, T, H, Hkv, D, kv_len, start, window=50, scale=0.2)
+    assert rel_l2(got, want) <= REL_L2_F16_MFMA
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, seqLen=T, kvLen=kv_len, numKVHeads=Hkv, startPos=start,
+                                          attnSoftcap=3.0, scale=0.5))
+    want = _prefill_oracle(q, kb, vb, T, H, Hkv, D, kv_len, start, softcap=3.0, scale=0.5)
+    assert rel_l2(got, want) <= REL_L2_F16_MFMA
+    # not causal: every query sees every key
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, seqLen=T, kvLen=kv_len, numKVHeads=Hkv, causal=False,
+                                          startPos=start, scale=0.2))
+    want = _prefill_oracle(q, kb, vb, T, H, Hkv, D, kv_len, start, causal=False, scale=0.2)
+    assert rel_l2(got, want) <= REL_L2_F16_MFMA
+    with pytest.raises(DopplerHipError, match="exceeds kvLen"):
+        ops.runAttention(qt, kt, vt, None, H, D, seqLen=T, kvLen=kv_len - 1, numKVHeads=Hkv, startPos=start)
+    with pytest.raises(DopplerHipError, match="contiguous cache"):
+        ops.runAttention(qt, kt, vt, None, H, D, seqLen=T, kvLen=kv_len, numKVHeads=Hkv, startPos=start, kvLayout="ring",
+                         slidingWindow=64)
