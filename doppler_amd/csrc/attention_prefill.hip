@@ -102,9 +102,19 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
       // V^T with the keys in k-slot order: key = 32 kb + 16 jj + 4 gg + ii -> slot 32 kb + 8 gg + 4 jj + ii
       const int kb = key >> 5, jj = (key >> 4) & 1, gg = (key >> 2) & 3, ii = key & 3;
       const int slot = 32 * kb + 8 * gg + 4 * jj + ii;
-      const _Float16* hv = reinterpret_cast<const _Float16*>(&vreg[r]);
+      // the 16 lanes that hold one key write different dims in the same step (lane c starts at
+      // dim c): their LDS rows would otherwise all fall into one bank
+      const uint32_t vw[4] = {vreg[r].x, vreg[r].y, vreg[r].z, vreg[r].w};
 #pragma unroll
-      for (int e = 0; e < 8; e++) v_lds[(8 * c + e) * VROW + slot] = hv[e];
+      for (int e = 0; e < 8; e++) {
+        const int ee = (e + c) & 7;
+        uint32_t w = vw[0];
+        w = (ee >> 1) == 1 ? vw[1] : w;
+        w = (ee >> 1) == 2 ? vw[2] : w;
+        w = (ee >> 1) == 3 ? vw[3] : w;
+        const uint16_t hbits = (uint16_t)((ee & 1) ? (w >> 16) : (w & 0xFFFFu));
+        reinterpret_cast<uint16_t*>(v_lds)[(8 * c + ee) * VROW + slot] = hbits;
+      }
     }
     __syncthreads();
     if (kt + 1 < ntiles) { DH_PF_LOAD(kt + 1); }

@@ -1,6 +1,6 @@
 """Per-kernel measurements of the HIP path on the benchmark configurations.
 
-    python -m doppler_amd.kernel_bench [--only gemv,gemm,attn,lmhead] [--json out.jsonl]
+    python -m doppler_amd.kernel_bench [--only gemv,gemm,attn,prefill_attn,lmhead] [--json out.jsonl]
 
 Every case is timed with events around back-to-back launches on the library's stream.  Weights
 (and KV caches) rotate through enough copies that their total exceeds the 256 MB Infinity Cache
@@ -180,6 +180,21 @@ def attn_cases(L, T, rows, reps):
             del K, V
 
 
+def attn_prefill_cases(L, T, rows, reps):
+    """Causal prefill attention from an empty cache: flops = 4 H D sum_t (t + 1)."""
+    D = 128
+    for (H, Hkv, Tq, cfg) in ((16, 8, 512, 3), (16, 8, 4096, 3), (32, 8, 2048, 4)):
+        K = torch.randn(Tq, Hkv, D, device="cuda", dtype=torch.float16) * (1.0 / D ** 0.5)
+        V = torch.randn(Tq, Hkv, D, device="cuda", dtype=torch.float16) * (1.0 / D ** 0.5)
+        q = torch.randn(Tq, H, D, device="cuda")
+        o = torch.zeros(Tq, H, D, device="cuda")
+        us = T.us(lambda i: capi.check(L.dh_attn_prefill(q.data_ptr(), K.data_ptr(), V.data_ptr(), o.data_ptr(), Tq, H, Hkv,
+                                                         D, Tq, 1.0 / D ** 0.5, 1, 0, 0.0, 0)), max(8, reps // 4))
+        flops = 4 * H * D * Tq * (Tq + 1) // 2
+        emit(rows, config=cfg, kernel="attn_prefill causal (cfg%d heads)" % cfg, shape="H=%d/%d D=128 T=%d" % (H, Hkv, Tq),
+             mode="warm", us=round(us, 2), achieved=round(flops / us / 1e6, 1), unit="TFLOP/s", flops=flops)
+
+
 def lmhead_cases(L, T, rows, reps):
     vocab, hidden = 151936, 4096
     E = (torch.randn(vocab, hidden, device="cuda") * 0.02).half()
@@ -195,7 +210,7 @@ def lmhead_cases(L, T, rows, reps):
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="gemv,gemm,attn,lmhead")
+    ap.add_argument("--only", default="gemv,gemm,attn,prefill_attn,lmhead")
     ap.add_argument("--reps", type=int, default=96)
     ap.add_argument("--json", default=None, help="also write one JSON object per case to this file")
     args = ap.parse_args(argv)
@@ -211,6 +226,8 @@ def main(argv=None):
         gemm_cases(L, T, rows, max(8, args.reps // 4))
     if "attn" in which:
         attn_cases(L, T, rows, args.reps)
+    if "prefill_attn" in which:
+        attn_prefill_cases(L, T, rows, args.reps)
     if "lmhead" in which:
         lmhead_cases(L, T, rows, args.reps)
     if args.json:
