@@ -31,6 +31,8 @@ unsigned* chain_counters();
 float* splitk_workspace(size_t* bytes);
 // Per-row scale factors of the prefill GEMM's activations: capacity rows x (multiplier, inverse).
 float* gemm_row_scale();
+// Packed f16 activations of the prefill GEMM (rows x K rounded up to 64 halves).
+void* gemm_packed_a(size_t* bytes);
 int gemm_row_scale_capacity();
 unsigned* chain_error_flag();
 unsigned chain_advance(unsigned n);

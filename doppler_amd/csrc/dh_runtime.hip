@@ -18,6 +18,8 @@ float* g_splitk_ws = nullptr;        // partial products of the split-K prefill 
 constexpr size_t kSplitKWsBytes = (size_t)32 << 20;
 float* g_row_scale = nullptr;        // [kRowScaleRows][2] activation row factors of the prefill GEMM
 constexpr int kRowScaleRows = 65536;
+void* g_packed_a = nullptr;          // packed f16 activations of the prefill GEMM
+constexpr size_t kPackedABytes = (size_t)64 << 20;
 constexpr size_t kChainWords = 8 * 64 + 64;
 }  // namespace
 
@@ -37,6 +39,10 @@ float* splitk_workspace(size_t* bytes) {
   return g_splitk_ws;
 }
 float* gemm_row_scale() { return g_row_scale; }
+void* gemm_packed_a(size_t* bytes) {
+  *bytes = g_packed_a ? kPackedABytes : 0;
+  return g_packed_a;
+}
 int gemm_row_scale_capacity() { return kRowScaleRows; }
 unsigned* chain_counters() { return g_chain_mem; }
 unsigned* chain_error_flag() { return g_chain_mem ? g_chain_mem + 8 * 64 : nullptr; }
@@ -76,6 +82,7 @@ int dh_init(int device_ordinal) {
   g_chain_value = 0;
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_splitk_ws), kSplitKWsBytes));
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_row_scale), (size_t)kRowScaleRows * 2 * sizeof(float)));
+  DH_CHECK_HIP("dh_init", hipMalloc(&g_packed_a, kPackedABytes));
   g_device = device_ordinal;
   g_ready = true;
   return 0;
@@ -92,6 +99,8 @@ int dh_shutdown(void) {
   g_splitk_ws = nullptr;
   if (g_row_scale) DH_CHECK_HIP("dh_shutdown", hipFree(g_row_scale));
   g_row_scale = nullptr;
+  if (g_packed_a) DH_CHECK_HIP("dh_shutdown", hipFree(g_packed_a));
+  g_packed_a = nullptr;
   g_own_stream = nullptr;
   g_stream = nullptr;
   g_ready = false;

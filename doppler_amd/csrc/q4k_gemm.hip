@@ -8,10 +8,12 @@
 //            as f16: (w & 0x000F000F) | 0x64006400 is the pair (1024 + q) in f16, one packed
 //            subtract and one packed fma with (d*sc, -dmin*mn) finish them: about 2 vector ops
 //            per weight, paid once per 128 rows of A.
-//   A        f32 -> f16 on the way into LDS, each row scaled by a power of two first so that its
-//            largest element sits at 2^14 (a row-maximum pre-pass writes the factors; the
-//            epilogue divides them out again, exactly): activations beyond the f16 range
-//            (65504) neither overflow nor lose small rows to subnormals.
+//   A        packed once per product by a pre-pass (pack_a_kernel): each row scaled by the power
+//            of two that puts its largest element at 2^14, rounded to f16, k-permuted, rows
+//            zero-padded to a multiple of 64.  The GEMM tiles then copy 16-byte pieces into
+//            LDS, no conversion in the K loop (every column tile used to redo it), and the
+//            epilogue divides the row factor out again, exactly: activations beyond the f16
+//            range (65504) neither overflow nor lose small rows to subnormals.
 // Both tiles sit in LDS as [row][64 k] with a 16-byte pad (conflict-free 16-byte fragment
 // reads) and are double-buffered: the global loads of tile t+1 are issued before tile t is
 // multiplied, one barrier per K step.
@@ -32,6 +34,7 @@ using dh::kQK;
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
 typedef __attribute__((ext_vector_type(16))) float float16_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
 int env_ksplit() {
   const char* e = getenv("DH_GEMM_KSPLIT");
@@ -43,6 +46,8 @@ constexpr int LDS_ROW = BK + 8;                    // halves per LDS row (144 by
 
 struct GemmArgs {
   const float* A;        // [M][K]
+  const _Float16* Apk;   // [M][kpad] packed activations (see pack_a_kernel)
+  int kpad;              // K rounded up to a multiple of 64
   const uint8_t* W;      // Q4_K rows [N][nb*144]
   const uint8_t* W2;     // second matrix (DUAL) or null
   void* C;               // [M][N] f32 or f16
@@ -58,15 +63,19 @@ struct GemmArgs {
   const float2* row_scale;   // [M] (multiplier applied before the f16 rounding, its inverse)
 };
 
-// One wave per activation row (four rows per workgroup): power-of-two factor that puts the row's
-// largest magnitude at 2^14; (1, 1) for an all-zero row.
-__global__ __launch_bounds__(256) void row_scale_kernel(const float* __restrict__ A, int M, int K,
-                                                        float2* __restrict__ out) {
+// Packs the activations for the matrix cores, one wave per row (four rows per workgroup):
+// finds the row's largest magnitude, scales by the power of two that puts it at 2^14 ((1, 1) for
+// an all-zero row), rounds to f16 and writes the row with its k in (0, 2, 1, 3) order inside
+// every group of four (the order the masked nibble pairs of the weights come out in), zero-padded
+// to kpad.  out_scale[m] = (factor, 1 / factor).
+__global__ __launch_bounds__(256) void pack_a_kernel(const float* __restrict__ A, int M, int K, int kpad,
+                                                     _Float16* __restrict__ Apk, float2* __restrict__ out_scale) {
   const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (m >= M) return;
   const float* row = A + (int64_t)m * K;
+  const bool vec = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0;
   float mx = 0.f;
-  if ((K & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+  if (vec) {
     for (int k = 4 * lane; k < K; k += 256) {
       const float4 v = *reinterpret_cast<const float4*>(row + k);
       mx = fmaxf(fmaxf(mx, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
@@ -76,11 +85,24 @@ __global__ __launch_bounds__(256) void row_scale_kernel(const float* __restrict_
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-  if (lane == 0) {
-    int e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
-    e = max(-100, min(100, e));
-    if (!(mx > 0.f) || !(mx < INFINITY)) e = 14;
-    out[m] = make_float2(__uint_as_float((uint32_t)(127 + 14 - e) << 23), __uint_as_float((uint32_t)(127 - 14 + e) << 23));
+  int e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
+  e = max(-100, min(100, e));
+  if (!(mx > 0.f) || !(mx < INFINITY)) e = 14;
+  const float mul = __uint_as_float((uint32_t)(127 + 14 - e) << 23);
+  if (lane == 0) out_scale[m] = make_float2(mul, __uint_as_float((uint32_t)(127 - 14 + e) << 23));
+  _Float16* dst = Apk + (int64_t)m * kpad;
+  for (int k = 4 * lane; k < kpad; k += 256) {
+    float v[4];
+    if (vec && k + 3 < K) {
+      const float4 t = *reinterpret_cast<const float4*>(row + k);      // second read: cache hit
+      v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[j] = k + j < K ? row[k + j] : 0.f;
+    }
+    const half2_t p0 = {(_Float16)(v[0] * mul), (_Float16)(v[2] * mul)};
+    const half2_t p1 = {(_Float16)(v[1] * mul), (_Float16)(v[3] * mul)};
+    *reinterpret_cast<uint2*>(dst + k) = make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
   }
 }
 
@@ -136,29 +158,24 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
   const int nkt = a.ksplit > 1 ? min((a.K + BK - 1) / BK, kt0 + a.kt_per_split) : (a.K + BK - 1) / BK;
 
   // ---- global -> register staging roles
-  // A: 8 float4 per thread, idx = tid + 256 i: row idx >> 4, k 4 * (idx & 15)
+  // A: 16-byte pieces of the packed rows, idx = tid + 256 i: row idx >> 3, halves 8 * (idx & 7)
   // W: thread (row tid >> 1, half tid & 1): 16 nibble bytes + header
   const int w_row = tid >> 1, w_half = tid & 1;
   const int64_t w_off = (int64_t)min(n0 + w_row, a.N - 1) * row_bytes;
-  constexpr int NA = BM * 16 / 256;                          // float4 loads of A per thread
+  constexpr int NA = BM * 8 / 256;                           // 16-byte loads of A per thread
   const bool w_active = w_row < BN;
-  float4 a_reg[NA];
+  u32x4_t a_reg[NA];
   uint4 q_reg[NMAT], h_reg[NMAT];
   // row factors of this tile's activation rows: one global read each, then LDS
   __shared__ float2 rs_lds[BM];
   if (tid < BM) rs_lds[tid] = a.row_scale[min(m0 + tid, a.M - 1)];
-  __syncthreads();
-  float a_mul[NA];
-#pragma unroll
-  for (int i = 0; i < NA; i++) a_mul[i] = rs_lds[(tid + 256 * i) >> 4].x;
 
   auto load_tile = [&](int kt) {
 #pragma unroll
     for (int i = 0; i < NA; i++) {
-      const int idx = tid + 256 * i, r = idx >> 4, k = kt * BK + 4 * (idx & 15);
+      const int idx = tid + 256 * i, r = idx >> 3;
       const int m = min(m0 + r, a.M - 1);
-      a_reg[i] = k < a.K ? *reinterpret_cast<const float4*>(a.A + (int64_t)m * a.K + k)
-                             : make_float4(0.f, 0.f, 0.f, 0.f);
+      a_reg[i] = *reinterpret_cast<const u32x4_t*>(a.Apk + (int64_t)m * a.kpad + kt * BK + 8 * (idx & 7));
     }
     const int blk = kt >> 2, c = kt & 3;
 #pragma unroll
@@ -174,12 +191,8 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
     _Float16* At = lds + buf * BUF_HALVES;
 #pragma unroll
     for (int i = 0; i < NA; i++) {
-      const int idx = tid + 256 * i, r = idx >> 4, kl = 4 * (idx & 15);
-      const float ml = a_mul[i];
-      const half2_t p0 = {(_Float16)(a_reg[i].x * ml), (_Float16)(a_reg[i].z * ml)};    // k order (0, 2, 1, 3)
-      const half2_t p1 = {(_Float16)(a_reg[i].y * ml), (_Float16)(a_reg[i].w * ml)};
-      *reinterpret_cast<uint2*>(At + r * LDS_ROW + kl) =
-          make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+      const int idx = tid + 256 * i, r = idx >> 3;
+      *reinterpret_cast<u32x4_t*>(At + r * LDS_ROW + 8 * (idx & 7)) = a_reg[i];
     }
     const int c = kt & 3;
 #pragma unroll
@@ -312,8 +325,14 @@ int launch_gemm_cfg(const GemmArgs& a, const char* op) {
 // share wins from there on), else 64 x 64.
 template <bool DUAL>
 int launch_gemm(GemmArgs a, const char* op) {
-  // rows beyond the scale buffer's capacity go in further passes
-  const int cap = dh::gemm_row_scale_capacity();
+  // rows beyond the capacity of the packed-activation scratch go in further passes
+  a.kpad = (a.K + BK - 1) / BK * BK;
+  size_t pk_bytes = 0;
+  _Float16* packed = reinterpret_cast<_Float16*>(dh::gemm_packed_a(&pk_bytes));
+  float2* scales = reinterpret_cast<float2*>(dh::gemm_row_scale());
+  if (!packed || !scales) return dh::fail(2, "[%s] the library's scratch buffers are missing (dh_init)", op);
+  const int cap = (int)std::min<size_t>((size_t)dh::gemm_row_scale_capacity(), pk_bytes / ((size_t)a.kpad * 2));
+  if (cap < 16) return dh::fail(1, "[%s] K=%d is too long for the prefill GEMM's activation scratch", op, a.K);
   if (a.M > cap) {
     const size_t c_elem = a.c_f16 ? 2 : 4;
     for (int m0 = 0; m0 < a.M; m0 += cap) {
@@ -327,12 +346,11 @@ int launch_gemm(GemmArgs a, const char* op) {
     }
     return 0;
   }
-  float2* scales = reinterpret_cast<float2*>(dh::gemm_row_scale());
-  if (!scales) return dh::fail(2, "[%s] the library's scratch buffers are missing (dh_init)", op);
-  hipLaunchKernelGGL(row_scale_kernel, dim3((unsigned)dh::ceil_div(a.M, 4)), dim3(256), 0, dh::stream(), a.A, a.M, a.K,
-                     scales);
+  hipLaunchKernelGGL(pack_a_kernel, dim3((unsigned)dh::ceil_div(a.M, 4)), dim3(256), 0, dh::stream(), a.A, a.M, a.K,
+                     a.kpad, packed, scales);
   DH_CHECK_LAUNCH(op);
   a.row_scale = scales;
+  a.Apk = packed;
   const int64_t big_tiles = dh::ceil_div(a.M, 128) * dh::ceil_div(a.N, 128);
   a.ksplit = 1;
   if (2 * big_tiles >= dh::num_cus()) return launch_gemm_cfg<DUAL, 2>(a, op);
@@ -363,7 +381,8 @@ int launch_gemm(GemmArgs a, const char* op) {
 namespace dh {
 
 bool q4k_gemm_serves(int M, int K, const void* A) {
-  return M >= 16 && (K % 4) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0;
+  (void)K; (void)A;          // any K and alignment: the packing pre-pass has a scalar path
+  return M >= 16;
 }
 
 int q4k_gemm(const char* op, const float* A, const uint8_t* W, void* C, int c_f16, int M, int N, int K,
