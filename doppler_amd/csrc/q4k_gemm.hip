@@ -15,8 +15,14 @@
 //            epilogue divides the row factor out again, exactly: activations beyond the f16
 //            range (65504) neither overflow nor lose small rows to subnormals.
 // Both tiles sit in LDS as [row][64 k] with a 16-byte pad (conflict-free 16-byte fragment
-// reads) and are double-buffered: the global loads of tile t+1 are issued before tile t is
-// multiplied, one barrier per K step.
+// reads) and are double-buffered, one barrier per K step.
+// SPEC (used where only one workgroup fits a compute unit, the fused gate/up tile): the
+// workgroup has eight waves, waves 0..3 only multiply (fragment reads + matrix-core
+// instructions), waves 4..7 only produce (global loads two tiles ahead, dequantise, write the
+// next LDS buffer).  Each SIMD then holds one wave of either kind, so the vector ALU work of the
+// dequantisation runs under the matrix-core work instead of in front of it; with all waves doing
+// both in turn (one barrier per step keeps them in phase) the two never overlap.  Where two or
+// more four-wave workgroups share a compute unit they overlap each other and that is faster.
 // k order inside every group of 4 is (0, 2, 1, 3) in BOTH tiles: that is the order the masked
 // nibble pairs come out in, and a contraction index may be permuted freely when both operands
 // agree.
@@ -139,17 +145,30 @@ __device__ __forceinline__ float gelu_tanh_fast(float x) {
   return 0.5f * x * (2.0f - 2.0f / (1.0f + __expf(2.0f * t)));
 }
 
+#ifdef DH_GEMM_TRACE
+__device__ unsigned long long dh_gemm_trace_buf[8 * 128];
+#define DH_GTS() do { if (lane == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 0 && tsn < 127) \
+                        dh_gemm_trace_buf[wave * 128 + tsn++] = wall_clock64(); } while (0)
+#else
+#define DH_GTS() do {} while (0)
+#endif
+
 // T = MFMA tiles per wave along each of M and N: workgroup tile 64T x 64T (T = 2: 128 x 128 for
 // large problems, T = 1: 64 x 64 when a 128-tiling would leave most compute units idle).
-template <bool DUAL, int T>
-__global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
+template <bool DUAL, int T, bool SPEC>
+__global__ __launch_bounds__(SPEC ? 512 : 256) void q4k_gemm_kernel(const GemmArgs a) {
   constexpr int NMAT = DUAL ? 2 : 1;
   constexpr int BM = 64 * T, BN = 64 * T;
   constexpr int A_HALVES = BM * LDS_ROW, B_HALVES = BN * LDS_ROW;
   extern __shared__ __align__(16) _Float16 lds[];            // [2 buffers][A | B | (B2)]
   constexpr int BUF_HALVES = A_HALVES + NMAT * B_HALVES;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const bool producer = !SPEC || wave >= 4, multiplier = !SPEC || wave < 4;
+  const int tid = threadIdx.x & 255;            // index inside the role's 256 threads
+#ifdef DH_GEMM_TRACE
+  int tsn = 0;
+#endif
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   const int wm = (wave >> 1) * 32 * T, wn = (wave & 1) * 32 * T;     // the wave's quadrant
   const int fr = lane & 31, fg = lane >> 5;                  // fragment row / k half
@@ -164,44 +183,51 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
   const int64_t w_off = (int64_t)min(n0 + w_row, a.N - 1) * row_bytes;
   constexpr int NA = BM * 8 / 256;                           // 16-byte loads of A per thread
   const bool w_active = w_row < BN;
-  u32x4_t a_reg[NA];
-  uint4 q_reg[NMAT], h_reg[NMAT];
+  // Two register sets: while tile kt is multiplied, tile kt+1 waits in one set and the loads of
+  // tile kt+2 are in flight into the other, so a load has two K steps to arrive.
+  struct Staged {
+    u32x4_t a[NA];
+    u32x4_t q[NMAT], h[NMAT];
+  };
+  Staged st0, st1;
   // row factors of this tile's activation rows: one global read each, then LDS
   __shared__ float2 rs_lds[BM];
-  if (tid < BM) rs_lds[tid] = a.row_scale[min(m0 + tid, a.M - 1)];
+  if (threadIdx.x < BM) rs_lds[threadIdx.x] = a.row_scale[min(m0 + (int)threadIdx.x, a.M - 1)];
 
-  auto load_tile = [&](int kt) {
+  auto load_tile = [&](int kt, Staged& st) {
 #pragma unroll
     for (int i = 0; i < NA; i++) {
       const int idx = tid + 256 * i, r = idx >> 3;
       const int m = min(m0 + r, a.M - 1);
-      a_reg[i] = *reinterpret_cast<const u32x4_t*>(a.Apk + (int64_t)m * a.kpad + kt * BK + 8 * (idx & 7));
+      st.a[i] = *reinterpret_cast<const u32x4_t*>(a.Apk + (int64_t)m * a.kpad + kt * BK + 8 * (idx & 7));
     }
     const int blk = kt >> 2, c = kt & 3;
 #pragma unroll
     for (int mt = 0; mt < NMAT; mt++) {
       if (w_active) {
         const uint8_t* bp = (mt ? a.W2 : a.W) + w_off + (int64_t)blk * kBlockBytes;
-        h_reg[mt] = *reinterpret_cast<const uint4*>(bp);
-        q_reg[mt] = *reinterpret_cast<const uint4*>(bp + 16 + 32 * c + 16 * w_half);
+        st.h[mt] = *reinterpret_cast<const u32x4_t*>(bp);
+        st.q[mt] = *reinterpret_cast<const u32x4_t*>(bp + 16 + 32 * c + 16 * w_half);
       }
     }
   };
-  auto store_tile = [&](int kt, int buf) {
+  auto store_tile = [&](int kt, int buf, const Staged& st) {
     _Float16* At = lds + buf * BUF_HALVES;
 #pragma unroll
     for (int i = 0; i < NA; i++) {
       const int idx = tid + 256 * i, r = idx >> 3;
-      *reinterpret_cast<u32x4_t*>(At + r * LDS_ROW + 8 * (idx & 7)) = a_reg[i];
+      *reinterpret_cast<u32x4_t*>(At + r * LDS_ROW + 8 * (idx & 7)) = st.a[i];
     }
     const int c = kt & 3;
 #pragma unroll
     for (int mt = 0; mt < NMAT; mt++) {
       if (!w_active) break;
       float sc_lo, sc_hi, mn_lo, mn_hi;
-      q4k_pair_scales(h_reg[mt], c, sc_lo, sc_hi, mn_lo, mn_hi);
+      const uint4 hdr = make_uint4(st.h[mt][0], st.h[mt][1], st.h[mt][2], st.h[mt][3]);
+      const uint4 qv = make_uint4(st.q[mt][0], st.q[mt][1], st.q[mt][2], st.q[mt][3]);
+      q4k_pair_scales(hdr, c, sc_lo, sc_hi, mn_lo, mn_hi);
       uint4 lo[2], hi[2];
-      dequant16(q_reg[mt], sc_lo, mn_lo, sc_hi, mn_hi, lo, hi);
+      dequant16(qv, sc_lo, mn_lo, sc_hi, mn_hi, lo, hi);
       _Float16* Bt = lds + buf * BUF_HALVES + A_HALVES + mt * B_HALVES + w_row * LDS_ROW;
       *reinterpret_cast<uint4*>(Bt + 16 * w_half) = lo[0];
       *reinterpret_cast<uint4*>(Bt + 16 * w_half + 8) = lo[1];
@@ -220,13 +246,13 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[mt][i][j][e] = 0.f;
 
-  load_tile(kt0);
-  store_tile(kt0, kt0 & 1);
-  __syncthreads();
-  for (int kt = kt0; kt < nkt; kt++) {
+  // One K step.  Multipliers: the tile in LDS buffer kt & 1.  Producers: move tile kt+1 from `nxt`
+  // into the other buffer and start the loads of tile kt+3 into `nxt`.
+  auto k_step = [&](int kt, Staged& nxt) {
+    DH_GTS();
     const int buf = kt & 1;
-    if (kt + 1 < nkt) load_tile(kt + 1);
     const _Float16* At = lds + buf * BUF_HALVES;
+    if (multiplier) {
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ks++) {
       half8_t af[T], bf[NMAT][T];
@@ -245,12 +271,36 @@ __global__ __launch_bounds__(256) void q4k_gemm_kernel(const GemmArgs a) {
         for (int i = 0; i < T; i++)
 #pragma unroll
           for (int j = 0; j < T; j++)
-            acc[mt][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[mt][j], acc[mt][i][j], 0, 0, 0);
+            // accumulators pinned to the accumulation registers: left to itself the compiler keeps
+            // them in vector registers and copies all of them aside and back every K step
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[mt][i][j]) : "v"(af[i]), "v"(bf[mt][j]));
     }
-    if (kt + 1 < nkt) store_tile(kt + 1, buf ^ 1);
+    }
+    DH_GTS();
+    if (producer) {
+      if (kt + 1 < nkt) store_tile(kt + 1, buf ^ 1, nxt);
+      if (kt + 3 < nkt) load_tile(kt + 3, nxt);
+    }
     __syncthreads();
+  };
+
+  if (producer) {
+    load_tile(kt0, st0);
+    store_tile(kt0, kt0 & 1, st0);
+    if (kt0 + 1 < nkt) load_tile(kt0 + 1, st0);
+    if (kt0 + 2 < nkt) load_tile(kt0 + 2, st1);
+  }
+  __syncthreads();
+  for (int kt = kt0; kt < nkt; kt += 2) {
+    k_step(kt, st0);
+    if (kt + 1 < nkt) k_step(kt + 1, st1);
   }
 
+  DH_GTS();
+#ifdef DH_GEMM_TRACE
+  if (lane == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 0) dh_gemm_trace_buf[wave * 128 + 127] = tsn;
+#endif
+  if (!multiplier) return;
   // ---- epilogue: lane holds column n = lane & 31 of rows 8 (e / 4) + 4 fg + (e % 4)
 #pragma unroll
   for (int i = 0; i < T; i++)
@@ -301,9 +351,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs a) {
 
 template <bool DUAL, int T>
 int launch_gemm_cfg(const GemmArgs& a, const char* op) {
+  constexpr bool SPEC = DUAL && T == 2;      // 110 KB of LDS: one workgroup per compute unit
   constexpr int BM = 64 * T, BN = 64 * T;
   const size_t lds = (size_t)2 * (DUAL ? 3 : 2) * BM * LDS_ROW * sizeof(_Float16);
-  auto kern = q4k_gemm_kernel<DUAL, T>;
+  auto kern = q4k_gemm_kernel<DUAL, T, SPEC>;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
     DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -311,7 +362,7 @@ int launch_gemm_cfg(const GemmArgs& a, const char* op) {
     attr_set = true;
   }
   const dim3 grid((unsigned)dh::ceil_div(a.N, BN), (unsigned)dh::ceil_div(a.M, BM), (unsigned)std::max(1, a.ksplit));
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds, dh::stream(), a);
+  hipLaunchKernelGGL(kern, grid, dim3(SPEC ? 512 : 256), lds, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   if (a.ksplit > 1) {
     const int64_t total = (int64_t)a.M * a.N;
@@ -377,6 +428,12 @@ int launch_gemm(GemmArgs a, const char* op) {
 }
 
 }  // namespace
+
+#ifdef DH_GEMM_TRACE
+extern "C" int dh_debug_gemm_trace(void* host_dst) {
+  return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(dh_gemm_trace_buf), sizeof(dh_gemm_trace_buf));
+}
+#endif
 
 namespace dh {
 
