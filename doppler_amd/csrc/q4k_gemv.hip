@@ -575,7 +575,11 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     }
     // Waves without staging work start their ring at once.  Waves that stage do so too when
     // every wave stages; otherwise they convert first and start their ring after the barrier,
-    // so the others can begin computing as early as possible.
+    // so the others can begin computing as early as possible.  (Putting every wave's whole ring
+    // in flight right behind the activation loads was measured slower, 9.3 vs 7.7 us on the
+    // 6144 x 4096 product: the activation loads of the staging waves then queue behind the
+    // other waves' weight loads in the memory system, and nothing can be consumed before the
+    // activations are staged.)
     DH_TS();
     DH_WAIT_VM(0);
     DH_TS();
