@@ -587,36 +587,28 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
 #pragma unroll
       for (int j = 0; j < 8; j++) ss = fmaf(v0[j], v0[j], ss);
     }
-    // Three phases (a loop, so that the ring-start code exists once): ring stages are put in
-    // flight before the norm reduction, before the conversion and after it.  Early waves start
-    // one stage at once and the rest after the norm barrier (which they would otherwise reach
-    // late, holding up the waves that convert); late waves start after the conversion.
-    float inv = 1.f;
-#pragma unroll 1
-    for (int phase = 0; phase < 3; phase++) {
-    const int nstart = early_ring ? (norm ? (phase == 0 ? 1 : (phase == 1 ? D - 1 : 0)) : (phase == 0 ? D : 0))
-                                  : (phase == 2 ? D : 0);
-    for (int d = 0; d < nstart; d++) DH_ISSUE_NEXT();
-    DH_TS();
-    if (phase == 0 && norm) {
-      // sum of squares of activation row m = (tid >> 2) % MT: lanes of a quad share a row,
-      // lane bit 2 selects the row when MT == 2
-      // (lane bits 2.. select the row: MT consecutive quads hold MT different rows)
+    // RMSNorm prologue: the row's 1/rms is one factor per activation row, so it is applied to
+    // the outputs at the tile end instead of to the activations here; the conversion below
+    // does not have to wait for the sum of squares, only the tile ends do.  Per wave: sum of
+    // squares of activation row m = (tid >> 2) % MT (lanes of a quad share a row, the lane
+    // bits above select among MT rows).
+    if (norm) {
       ss += quad_xor_f32(ss, 1);
       ss += quad_xor_f32(ss, 2);
       if (MT <= 1) ss += __shfl_xor(ss, 4);
       if (MT <= 2) ss += __shfl_xor(ss, 8);
       if (MT <= 4) ss += __shfl_xor(ss, 16);
       ss += __shfl_xor(ss, 32);
-      const int my_m = (tid >> 2) % MT;
       if ((lane & 3) == 0 && (lane >> 2) < MT) norm_ss[wave][lane >> 2] = ss;
-      DH_LDS_BARRIER();
-      float tot = 0.f;
-#pragma unroll
-      for (int w = 0; w < WAVES; w++) tot += norm_ss[w][my_m];
-      inv = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
     }
-    if (phase != 1) continue;
+    // Two places where ring stages are put in flight (a loop, so that the code exists once):
+    // early waves before the conversion, late waves after it.
+#pragma unroll 1
+    for (int phase = 0; phase < 2; phase++) {
+    const int nstart = early_ring == (phase == 0) ? D : 0;
+    for (int d = 0; d < nstart; d++) DH_ISSUE_NEXT();
+    DH_TS();
+    if (phase != 0) continue;
 #pragma unroll 1
     for (int idx = tid; idx < total; idx += NTHR) {
       float t[8], wn[8];
@@ -629,7 +621,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
       }
       if (norm) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) t[j] = t[j] * inv * wn[j];
+        for (int j = 0; j < 8; j++) t[j] = t[j] * wn[j];
       }
       stage_x_store<MT>(idx, t, xf, sxi);
     }
@@ -722,6 +714,14 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
         for (int w = 0; w < WAVES; w++) {
           sg += red[slot][w][0][k][col];
           if (DUAL) su += red[slot][w][NMAT - 1][k][col];
+        }
+        if (a.norm_weight) {
+          float tot = 0.f;
+#pragma unroll
+          for (int w = 0; w < WAVES; w++) tot += norm_ss[w][m];
+          const float inv = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
+          sg *= inv;
+          su *= inv;
         }
         float v;
         if (DUAL) {
