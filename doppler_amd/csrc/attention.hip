@@ -298,17 +298,26 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
 }
 
 // One workgroup per query head: out[d] = sum_s e^{m_s - M} o_s[d] / sum_s e^{m_s - M} l_s.
-// The per-split factors are computed once, in parallel over splits, and kept in LDS; the
-// D threads then walk the splits with independent (prefetchable) loads.
+// Every load the kernel needs for the first 32 splits (a thread's 32 partial outputs, and one
+// (m, l) pair per thread) is issued before anything is waited for, so the kernel costs one memory
+// round trip, not one per dependent phase; splits beyond 32 follow in a pipelined loop.
 template <int D>
 __global__ __launch_bounds__(D) void attn_decode_merge_kernel(const float* __restrict__ ws,
                                                               float* __restrict__ O, int nsplit) {
+  constexpr int CH = 32;
   __shared__ float f_s[1024];
   __shared__ float red[4];
   const int h = blockIdx.x, d = threadIdx.x;
   const float* base = ws + (int64_t)h * nsplit * (D + 2);
-  float M = -FLT_MAX;
-  for (int s = d; s < nsplit; s += D) M = fmaxf(M, base[s * (D + 2) + D]);
+  float ov[CH];
+#pragma unroll
+  for (int i = 0; i < CH; i++) ov[i] = base[(int64_t)min(i, nsplit - 1) * (D + 2) + d];
+  // (m, l) of split d, d + D, ...: registers for the first, reloaded (cache hits) beyond
+  const bool has = d < nsplit;
+  const float m0 = has ? base[d * (D + 2) + D] : -FLT_MAX;
+  const float l0 = has ? base[d * (D + 2) + D + 1] : 0.f;
+  float M = m0;
+  for (int s = d + D; s < nsplit; s += D) M = fmaxf(M, base[s * (D + 2) + D]);
   M = wave_max(M);
   if ((d & 63) == 0) red[d >> 6] = M;
   __syncthreads();
@@ -316,7 +325,12 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(const float* __res
   for (int w = 1; w < D / 64; w++) M = fmaxf(M, red[w]);
   __syncthreads();
   float den = 0.f;
-  for (int s = d; s < nsplit; s += D) {
+  if (has) {
+    const float f = __expf(m0 - M);
+    f_s[d] = f;
+    den = f * l0;
+  }
+  for (int s = d + D; s < nsplit; s += D) {
     const float f = __expf(base[s * (D + 2) + D] - M);
     f_s[s] = f;
     den = fmaf(f, base[s * (D + 2) + D + 1], den);
@@ -327,8 +341,10 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(const float* __res
   den = 0.f;
   for (int w = 0; w < D / 64; w++) den += red[w];
   float num = 0.f;
+#pragma unroll
+  for (int i = 0; i < CH; i++) num = i < nsplit ? fmaf(f_s[i], ov[i], num) : num;
 #pragma unroll 8
-  for (int s = 0; s < nsplit; s++) num = fmaf(f_s[s], base[s * (D + 2) + d], num);
+  for (int s = CH; s < nsplit; s++) num = fmaf(f_s[s], base[s * (D + 2) + d], num);
   O[(int64_t)h * D + d] = den > 0.f ? num / den : 0.f;
 }
 
