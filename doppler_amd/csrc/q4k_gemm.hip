@@ -301,6 +301,9 @@ __global__ __launch_bounds__(SPEC ? 512 : 256) void q4k_gemm_kernel(const GemmAr
   if (lane == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 0) dh_gemm_trace_buf[wave * 128 + 127] = tsn;
 #endif
   if (!multiplier) return;
+  // the matrix-core instructions above are inline asm, invisible to the compiler's hazard
+  // checks: give the last one time to retire before its accumulators are read
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   // ---- epilogue: lane holds column n = lane & 31 of rows 8 (e / 4) + 4 fg + (e % 4)
 #pragma unroll
   for (int i = 0; i < T; i++)
