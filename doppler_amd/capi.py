@@ -65,6 +65,8 @@ SIGNATURES = {
     "dh_act_gate_rowsplit": (_I, [_P, _P, _I, _I, _I, _F]),
     "dh_argmax_workspace_bytes": (_SZ, []),
     "dh_argmax": (_I, [_P, _I, _I64, _F, _P, _P, _I]),
+    "dh_sample_topk_workspace_bytes": (_SZ, [_I, _I]),
+    "dh_sample_topk": (_I, [_P, _I, ctypes.c_double, _I, ctypes.c_double, _I64, _F, _P, _P, _I]),
     "dh_cast_f32_to_f16": (_I, [_P, _P, _I64]),
     "dh_cast_f16_to_f32": (_I, [_P, _P, _I64]),
 }

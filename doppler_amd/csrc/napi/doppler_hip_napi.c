@@ -216,6 +216,16 @@ FN(js_argmax) {
   ARGS(7); P(0, lg); I(1, vocab); L(2, pad); F(3, cap); P(4, ws); P(5, tok); I(6, idx);
   return ret_rc(env, dh_argmax((const float*)lg, vocab, pad, cap, ws, (uint32_t*)tok, idx));
 }
+FN(js_sample_topk_workspace_bytes) { ARGS(2); I(0, vocab); I(1, k); return ret_num(env, (double)dh_sample_topk_workspace_bytes(vocab, k)); }
+FN(js_sample_topk) {
+  ARGS(10); P(0, lg); I(1, vocab); I(3, k); L(5, pad); F(6, cap); P(7, ws); P(8, tok); I(9, idx);
+  double temperature, random_value;
+  if (napi_get_value_double(env, a[2], &temperature) != napi_ok || napi_get_value_double(env, a[4], &random_value) != napi_ok) {
+    napi_throw_type_error(env, NULL, "doppler_hip: number expected");
+    return NULL;
+  }
+  return ret_rc(env, dh_sample_topk((const float*)lg, vocab, temperature, k, random_value, pad, cap, ws, (uint32_t*)tok, idx));
+}
 FN(js_cast_f32_to_f16) { ARGS(3); P(0, i); P(1, o); L(2, n); return ret_rc(env, dh_cast_f32_to_f16((const float*)i, o, n)); }
 FN(js_cast_f16_to_f32) { ARGS(3); P(0, i); P(1, o); L(2, n); return ret_rc(env, dh_cast_f16_to_f32(i, (float*)o, n)); }
 
@@ -234,6 +244,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"kvWriteF16", js_kv_write_f16}, {"residualAdd", js_residual_add}, {"gatherF16", js_gather_f16},
       {"actGate", js_act_gate}, {"actGateRowsplit", js_act_gate_rowsplit},
       {"argmaxWorkspaceBytes", js_argmax_workspace_bytes}, {"argmax", js_argmax},
+      {"sampleTopkWorkspaceBytes", js_sample_topk_workspace_bytes}, {"sampleTopk", js_sample_topk},
       {"castF32ToF16", js_cast_f32_to_f16}, {"castF16ToF32", js_cast_f16_to_f32},
   };
   for (size_t i = 0; i < sizeof(table) / sizeof(table[0]); i++) {

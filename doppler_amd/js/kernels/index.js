@@ -12,6 +12,6 @@ export { runSiLU, recordSiLU, runSiLURowSplit, recordSiLURowSplit } from './silu
 export { runGeLU, recordGeLU } from './gelu.js';
 export { runResidualAdd, recordResidualAdd } from './residual.js';
 export { runGather, recordGather } from './gather.js';
-export { runArgmax, recordArgmax } from './sample.js';
+export { runArgmax, recordArgmax, runGPUSample, recordGPUSample, seededRandom } from './sample.js';
 export { recordLmHeadArgmax, recordLmHeadArgmaxF16 } from './lm-head-argmax.js';
 export { castF32ToF16, castF16ToF32, recordCastF32ToF16, recordCastF16ToF32 } from './cast.js';

@@ -472,6 +472,37 @@ def runArgmax(logits, vocabSize, padTokenId=None, logitSoftcap=0.0, logitsDtype=
     return int(readBuffer(out, (outputIndex + 1) * 4, np.uint32)[outputIndex])
 
 
+def seededRandom(seed):
+    """src/gpu/kernels/sample.js:569-572: the reference's Math.sin based uniform number."""
+    x = math.sin(seed) * 10000.0
+    return x - math.floor(x)
+
+
+def runGPUSample(logits, vocabSize, temperature=1.0, topK=40, randomSeed=None, randomValue=None, padTokenId=None,
+                 logitSoftcap=0.0, greedyThreshold=0.01, logitsDtype="f32", outputBuffer=None, outputIndex=0,
+                 readback=True):
+    """src/gpu/kernels/sample.js:343 runGPUSample: top-k temperature sampling; below the greedy
+    threshold or with topK <= 1 it is runArgmax.  randomValue overrides the seeded draw."""
+    if logitsDtype != "f32":
+        raise DopplerHipError("[Sample] logitsDtype %r is not supported on the HIP path" % (logitsDtype,))
+    if temperature < greedyThreshold or topK <= 1:
+        return runArgmax(logits, vocabSize, padTokenId=padTokenId, logitSoftcap=logitSoftcap, outputBuffer=outputBuffer,
+                         outputIndex=outputIndex, readback=readback)
+    if randomValue is None:
+        if randomSeed is None:
+            raise DopplerHipError("[Sample] randomSeed (or randomValue) is required on the HIP path")
+        randomValue = seededRandom(randomSeed)
+    L = _lib()
+    ws = acquireBuffer(int(L.dh_sample_topk_workspace_bytes(vocabSize, topK)))
+    out = _out(outputBuffer, max(4, (outputIndex + 1) * 4))
+    capi.check(L.dh_sample_topk(_ptr(logits), vocabSize, float(temperature), int(topK), float(randomValue),
+                                -1 if padTokenId is None else padTokenId, logitSoftcap, ws.data_ptr(), out.data_ptr(),
+                                outputIndex))
+    if not readback:
+        return out
+    return int(readBuffer(out, (outputIndex + 1) * 4, np.uint32)[outputIndex])
+
+
 def recordLmHeadArgmaxF16(recorder, inputTensor, lmHead, vocabSize=None, hiddenSize=None, padTokenId=None,
                           logitSoftcap=0.0, outputBuffer=None, outputIndex=0, logitsOutput=None):
     """src/gpu/kernels/lm-head-argmax.js:304 recordLmHeadArgmaxF16: returns the output buffer

@@ -235,6 +235,19 @@ size_t dh_argmax_workspace_bytes(void);
 int dh_argmax(const float* d_logits, int vocab, int64_t pad_token_id, float logit_softcap,
               void* d_workspace, uint32_t* d_token_out, int output_index);
 
+/* Top-k temperature sampling: the top_k (<= 256) logits by value (ties to the lower index),
+ * softmax of value / temperature over them, first candidate whose running probability reaches
+ * random_value.  Replaces runGPUSample/recordGPUSample, src/gpu/kernels/sample.js:343-568
+ * (sample.wgsl:66-243), with the selection of the reference's sampler oracle
+ * (tests/kernels/reference/sample.js:62-92: exact top-k; the WGSL keeps one candidate per
+ * workgroup).  The caller draws random_value (seededRandom, sample.js:569-572) and routes
+ * temperature below its greedy threshold to dh_argmax.  d_workspace needs
+ * dh_sample_topk_workspace_bytes(vocab, top_k) bytes. */
+size_t dh_sample_topk_workspace_bytes(int vocab, int top_k);
+int dh_sample_topk(const float* d_logits, int vocab, double temperature, int top_k,
+                   double random_value, int64_t pad_token_id, float logit_softcap,
+                   void* d_workspace, uint32_t* d_token_out, int output_index);
+
 /* f32 <-> f16 casts.  Replaces castF32ToF16/castF16ToF32, src/gpu/kernels/cast.js:98-116. */
 int dh_cast_f32_to_f16(const float* d_in, void* d_out, int64_t n);
 int dh_cast_f16_to_f32(const void* d_in, float* d_out, int64_t n);

@@ -90,6 +90,10 @@ def _declare(L):
     L.dor_gather_f16.argtypes = [_P, _P, _I64, _I64, _I64, _P]
     L.dor_argmax.restype = _I64
     L.dor_argmax.argtypes = [_P, _I64, _I64, _F]
+    L.dor_sample_topk.restype = _I64
+    L.dor_sample_topk.argtypes = [_P, _I64, ctypes.c_double, _I64, ctypes.c_double, _I64, _F]
+    L.dor_seeded_random.restype = ctypes.c_double
+    L.dor_seeded_random.argtypes = [ctypes.c_double]
     L.dor_decode_step.restype = _I64
     L.dor_decode_step.argtypes = [_P, _P, _P, _P, _P, _P, ctypes.c_uint32, _I64, _P]
 
@@ -353,6 +357,16 @@ def argmax(logits, pad_id=None, softcap=0.0):
     logits = _c(logits, np.float32).reshape(-1)
     return int(lib().dor_argmax(_ptr(logits), logits.size, -1 if pad_id is None else pad_id,
                                 softcap))
+
+
+def sample_topk(logits, temperature, top_k, random_value, pad_id=None, softcap=0.0):
+    logits = _c(logits, np.float32).reshape(-1)
+    return int(lib().dor_sample_topk(_ptr(logits), logits.size, float(temperature), int(top_k), float(random_value),
+                                     -1 if pad_id is None else pad_id, softcap))
+
+
+def seeded_random(seed):
+    return float(lib().dor_seeded_random(float(seed)))
 
 
 # --------------------------------------------------------------------------- decode step

@@ -718,6 +718,63 @@ int64_t dor_argmax(const float* logits, int64_t vocab, int64_t pad_id, float sof
   return best;
 }
 
+/* Top-k temperature sampling.  tests/kernels/reference/sample.js:62-92 (sampleTopKRef):
+ * below temperature 0.01 plain argmax; otherwise the top_k logits by value (stable: among
+ * equal values the lower index first, as Array.prototype.sort on {val, idx} gives), softmax of
+ * value / temperature over those in f64, then the first candidate at which the running sum of
+ * probabilities reaches random_value (last candidate if none does).  Soft cap and pad id as in
+ * dor_argmax (the kernel's extras). */
+int64_t dor_sample_topk(const float* logits, int64_t vocab, double temperature, int64_t top_k,
+                        double random_value, int64_t pad_id, float softcap) {
+  if (temperature < 0.01) return dor_argmax(logits, vocab, pad_id, softcap);
+  if (top_k > vocab) top_k = vocab;
+  int64_t* idx = (int64_t*)malloc((size_t)top_k * sizeof(int64_t));
+  double* val = (double*)malloc((size_t)top_k * sizeof(double));
+  int64_t n = 0;
+  for (int64_t i = 0; i < vocab; i++) {            /* insertion into the sorted top-k list */
+    if (i == pad_id) continue;
+    float v = logits[i];
+    if (softcap > 0.0f) v = (float)((double)softcap * tanh((double)v / (double)softcap));
+    if (n == top_k && !((double)v > val[n - 1])) continue;   /* equal to the last: later index loses */
+    int64_t p = n < top_k ? n : top_k - 1;
+    while (p > 0 && (double)v > val[p - 1]) {
+      val[p] = val[p - 1];
+      idx[p] = idx[p - 1];
+      p--;
+    }
+    val[p] = (double)v;
+    idx[p] = i;
+    if (n < top_k) n++;
+  }
+  double mx = -INFINITY, sum = 0.0;
+  for (int64_t i = 0; i < n; i++) {
+    val[i] = val[i] / temperature;
+    if (val[i] > mx) mx = val[i];
+  }
+  for (int64_t i = 0; i < n; i++) {
+    val[i] = exp(val[i] - mx);
+    sum += val[i];
+  }
+  int64_t pick = n > 0 ? idx[n - 1] : 0;
+  double cum = 0.0;
+  for (int64_t i = 0; i < n; i++) {
+    cum += val[i] / sum;
+    if (cum >= random_value) {
+      pick = idx[i];
+      break;
+    }
+  }
+  free(idx);
+  free(val);
+  return pick;
+}
+
+/* Math.sin based generator of the reference, tests/kernels/reference/sample.js:94-97. */
+double dor_seeded_random(double seed) {
+  const double x = sin(seed) * 10000.0;
+  return x - floor(x);
+}
+
 /* ------------------------------------------------------------------------- */
 /* Whole decoder step (test/bench driver; op order follows the execution graph */
 /* src/config/conversion/qwen3/qwen-3-embedding-0-6b-q4k-ehf16-af32.json       */

@@ -145,6 +145,9 @@ async function main() {
         tokens.push(tok);
       }
       fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
+    } else if (c.op === 'sample') {
+      const tok = await dh.runGPUSample(dev(c.logits), c.vocab, { temperature: c.temperature, topK: c.topK, randomSeed: c.seed });
+      fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array([tok]).buffer));
     } else if (c.op === 'rdrr_decoder') {
       // weights come from an RDRR artifact directory through the JS loader
       const { config, weights } = loadDecoderWeights(c.dir, c.maxSeq);

@@ -208,6 +208,12 @@ def test_js_host_path_parity(tmp_path):
         want_tokens.append(tok)
     checks.append(lambda: [int(t) for t in get("decoder.out.bin", np.uint32)] == want_tokens)
 
+    # ---- top-k temperature sampling through the JS op (seeded draw as in the reference)
+    slog = (synth.rng(79).standard_normal(4000) * 3).astype(np.float32)
+    cases.append(dict(name="sample", op="sample", logits=put("s.logits", slog), vocab=4000, temperature=0.9, topK=40, seed=42))
+    want_sample = oracle.sample_topk(slog, 0.9, 40, oracle.seeded_random(42))
+    checks.append(lambda: int(get("sample.out.bin", np.uint32)[0]) == want_sample)
+
     # ---- the same model again, this time written as an RDRR artifact (small shards, so tensors
     #      span shard boundaries) and read back by the JavaScript loader
     from doppler_amd import rdrr

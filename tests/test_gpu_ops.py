@@ -339,6 +339,41 @@ def test_argmax_exact_ties_pad_softcap():
     assert ops.runArgmax(ops.tensorFromNumpy(x), 4096, logitSoftcap=30.0) == oracle.argmax(x, softcap=30.0)
 
 
+def test_gpu_sample_topk_matches_oracle():
+    """runGPUSample against the sampler oracle (exact top-k, f64 softmax, inverse CDF): vocabulary
+    sizes on both sides of one sort tile and at the 9B-class size, ties, top_k from 2 to 256."""
+    g = synth.rng(7100)
+    cases = [(64, 4), (1000, 40), (1024, 256), (1025, 7), (5000, 50), (151936, 40), (151936, 256), (151936, 2)]
+    for ci, (V, k) in enumerate(cases):
+        logits = (g.standard_normal(V) * 3).astype(np.float32)
+        if ci % 2 == 1:
+            logits = (np.round(logits * 4) / 4).astype(np.float32)        # exact ties everywhere
+        lt = ops.tensorFromNumpy(logits)
+        for T in (0.7, 1.0, 1.8):
+            for seed in (1, 42, 977):
+                r = ops.seededRandom(seed + ci)
+                assert r == oracle.seeded_random(seed + ci)
+                got = ops.runGPUSample(lt, V, temperature=T, topK=k, randomSeed=seed + ci)
+                assert got == oracle.sample_topk(logits, T, k, r), (V, k, T, seed)
+    # extremes of the uniform draw, pad id, greedy fallbacks
+    V = 3000
+    logits = (g.standard_normal(V) * 2).astype(np.float32)
+    lt = ops.tensorFromNumpy(logits)
+    order = np.argsort(-logits, kind="stable")
+    assert ops.runGPUSample(lt, V, temperature=1.0, topK=5, randomValue=0.0) == int(order[0])
+    assert ops.runGPUSample(lt, V, temperature=1.0, topK=5, randomValue=1.0) == oracle.sample_topk(logits, 1.0, 5, 1.0)
+    assert ops.runGPUSample(lt, V, temperature=1.0, topK=5, randomValue=0.0, padTokenId=int(order[0])) == int(order[1])
+    assert ops.runGPUSample(lt, V, temperature=0.001, topK=5, randomSeed=3) == int(order[0])
+    assert ops.runGPUSample(lt, V, temperature=1.0, topK=1, randomSeed=3) == int(order[0])
+    buf = ops.acquireBuffer(16)
+    ops.runGPUSample(lt, V, temperature=1.0, topK=8, randomValue=0.3, outputBuffer=buf, outputIndex=2, readback=False)
+    assert int(ops.readBuffer(buf, 16, np.uint32)[2]) == oracle.sample_topk(logits, 1.0, 8, 0.3)
+    with pytest.raises(DopplerHipError, match="topK must be in 1..256"):
+        ops.runGPUSample(lt, V, temperature=1.0, topK=300, randomSeed=1)
+    with pytest.raises(DopplerHipError, match="randomSeed"):
+        ops.runGPUSample(lt, V, temperature=1.0, topK=5)
+
+
 def test_gather_f16_exact():
     vocab, hidden = 300, 640
     E = synth.normal_f16_bits((vocab, hidden), seed=3200, scale=0.02)

@@ -519,6 +519,45 @@ def tiny_model(seed=200, layers=2, hidden=256, inter=512, heads=4, kv_heads=2, h
     return cfg, L, embed, final_norm, cos, sin
 
 
+def test_sample_topk_matches_a_direct_restatement_of_the_js_reference():
+    """dor_sample_topk against the reference's sampleTopKRef written out with Python's stable
+    sort and math.exp (tests/kernels/reference/sample.js:62-92), including ties, top_k = 1 and
+    the sub-0.01 temperature that falls back to argmax; seededRandom against Math.sin."""
+    g = synth.rng(900)
+
+    def ref(logits, T, k, r):
+        if T < 0.01:
+            return int(np.argmax(logits))
+        order = sorted(range(len(logits)), key=lambda i: (-float(logits[i]), i))[:k]
+        vals = [float(logits[i]) / T for i in order]
+        mx = max(vals)
+        ex = [math.exp(v - mx) for v in vals]
+        tot = sum(ex)
+        c = 0.0
+        for i, e in zip(order, ex):
+            c += e / tot
+            if c >= r:
+                return i
+        return order[-1]
+
+    for t in range(200):
+        V = int(g.integers(3, 500))
+        logits = g.standard_normal(V).astype(np.float32)
+        if t % 3 == 0:
+            logits = (np.round(logits * 2) / 2).astype(np.float32)      # many exact ties
+        k = int(g.integers(1, min(V, 64) + 1))
+        T = float(g.choice([0.001, 0.3, 1.0, 2.5]))
+        r = float(g.random())
+        assert oracle.sample_topk(logits, T, k, r) == ref(logits, T, k, r), (t, V, k, T, r)
+    # the running sum never reaches 1.0 + : last candidate
+    assert oracle.sample_topk(np.array([0.0, 1.0, 2.0], np.float32), 1.0, 2, 1.5) == 1
+    # pad id can never be drawn
+    assert oracle.sample_topk(np.array([5.0, 1.0, 0.0], np.float32), 1.0, 2, 0.0, pad_id=0) == 1
+    for seed in (0, 1, 42, 12345.5):
+        x = math.sin(seed) * 10000
+        assert oracle.seeded_random(seed) == x - math.floor(x)
+
+
 def test_decode_step_wiring_matches_op_by_op():
     cfg, L, embed, final_norm, cos, sin = tiny_model()
     dec = oracle.DecoderOracle(cfg, L, embed, final_norm, cos, sin)
