@@ -208,6 +208,19 @@ def lmhead_cases(L, T, rows, reps):
          us=round(us, 2), achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
 
 
+def sample_cases(L, T, rows, reps):
+    vocab = 151936
+    logits = torch.randn(vocab, device="cuda") * 3
+    tok = torch.zeros(4, dtype=torch.int32, device="cuda")
+    for k in (40, 256):
+        ws = torch.zeros(int(L.dh_sample_topk_workspace_bytes(vocab, k)), dtype=torch.uint8, device="cuda")
+        us = T.us(lambda i: capi.check(L.dh_sample_topk(logits.data_ptr(), vocab, 0.8, k, 0.37, -1, 0.0, ws.data_ptr(),
+                                                        tok.data_ptr(), 0)), max(8, reps // 4))
+        algo = vocab * 4
+        emit(rows, config=4, kernel="sample top-k (vocab 151936)", shape="topK=%d T=0.8" % k, mode="warm", us=round(us, 2),
+             achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--only", default="gemv,gemm,attn,prefill_attn,lmhead")
@@ -230,6 +243,7 @@ def main(argv=None):
         attn_prefill_cases(L, T, rows, args.reps)
     if "lmhead" in which:
         lmhead_cases(L, T, rows, args.reps)
+        sample_cases(L, T, rows, args.reps)
     if args.json:
         with open(args.json, "w") as f:
             for r in rows:
