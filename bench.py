@@ -215,7 +215,8 @@ def main():
             t_cpu = time.perf_counter() - t0
         threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
         js = js_reference_timings()
-        cpu = {"value": round(n_cpu / t_cpu, 4), "unit": "tokens/s", "cores": threads, "kind": "port",
+        cpu = {"value": round(n_cpu / t_cpu, 4), "unit": "tokens/s", "cores": threads, "host_cpus": os.cpu_count(),
+               "kind": "port",
                "sample": "%d full decode steps of the same model from the same prefilled KV cache "
                          "(C restatement of the reference's JS per-op references, f64 accumulate, OpenMP)" % n_cpu,
                # the reference's CPU path is single-threaded JavaScript: the same per-op references
