@@ -215,13 +215,42 @@ class HipDecoder:
         capi.check(self.L.dh_download(self._host_token.ctypes.data, self.token.data_ptr(), 0, 4))
         return int(self._host_token[0])
 
-    def step(self, token, pos, want_logits=False):
-        """One full step with the reference's single device->host crossing (the token id)."""
+    def step(self, token, pos, want_logits=False, sampling=None):
+        """One full step with the reference's single device->host crossing (the token id).
+        sampling = dict(temperature, topK, randomSeed): top-k temperature sampling from the
+        step's logits instead of the fused greedy argmax."""
         self.set_token(token)
-        self.enqueue_step(pos, want_logits)
+        self.enqueue_step(pos, want_logits or sampling is not None)
+        if sampling is not None:
+            self._enqueue_sample(sampling)
         return self.read_token()
 
-    def prefill(self, tokens, start_pos=0, chunk=512, want_logits=False):
+    def _enqueue_sample(self, sampling, out_index=0):
+        from . import ops
+        L, c = self.L, self.cfg
+        k = int(sampling["topK"])
+        if float(sampling["temperature"]) < sampling.get("greedyThreshold", 0.01) or k <= 1:
+            return                                  # the fused argmax already left the greedy token
+        r = sampling["randomValue"] if "randomValue" in sampling else ops.seededRandom(sampling["randomSeed"])
+        need = int(L.dh_sample_topk_workspace_bytes(c["vocab"], k))
+        if getattr(self, "_sample_ws", None) is None or self._sample_ws.numel() < need:
+            self._sample_ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+        capi.check(L.dh_sample_topk(self.logits.data_ptr(), c["vocab"], float(sampling["temperature"]), k, float(r), -1, 0.0,
+                                    self._sample_ws.data_ptr(), self.token.data_ptr(), out_index))
+
+    def generate(self, prompt, max_tokens, sampling=None, chunk=512):
+        """prefill + decode loop; sampling = dict(temperature, topK, seed) draws token i with
+        randomSeed seed + i (greedy when None)."""
+        draw = (lambda i: dict(temperature=sampling["temperature"], topK=sampling["topK"], randomSeed=sampling["seed"] + i)) \
+            if sampling else (lambda i: None)
+        tok = self.prefill(prompt, chunk=chunk, sampling=draw(0))
+        out = [tok]
+        for i in range(1, max_tokens):
+            tok = self.step(tok, len(prompt) + i - 1, sampling=draw(i))
+            out.append(tok)
+        return out
+
+    def prefill(self, tokens, start_pos=0, chunk=512, want_logits=False, sampling=None):
         """Pushes a prompt through the batched path, `chunk` tokens at a time: Q4_K prefill GEMMs,
         the T-token fused QKV-norm-RoPE-KV-write, matrix-core prefill attention.  KV rows
         start_pos .. start_pos + len(tokens) - 1 are written; returns the greedy token after the
@@ -276,7 +305,9 @@ class HipDecoder:
                         None, None, 1.0))
         ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
                                   self.lm_ws.data_ptr(), self.token.data_ptr(), 0,
-                                  self.logits.data_ptr() if want_logits else None))
+                                  self.logits.data_ptr() if (want_logits or sampling is not None) else None))
+        if sampling is not None:
+            self._enqueue_sample(sampling)
         return self.read_token()
 
     def decode_batch(self, token, pos, n):

@@ -6,8 +6,13 @@
 import {
   createTensor, createWeightBuffer, acquireBuffer, releaseBuffer, uploadData, readBufferSlice,
   createCommandRecorder, recordGather, recordRMSNorm, recordMatmul, recordSplitQKVRMSNormRoPEQK,
-  recordAttention, recordFusedNormedFFN, recordLmHeadArgmaxF16,
+  recordAttention, recordFusedNormedFFN, recordFusedFFN, recordLmHeadArgmaxF16, recordGPUSample,
 } from '../kernel-selector.js';
+
+// A window of a device buffer starting `offset` bytes in (no ownership: never released).
+function bufferWindow(buffer, offset, size) {
+  return { ptr: buffer.ptr + BigInt(offset), size, capacity: size, label: buffer.label };
+}
 
 function upload(bytes, label) {
   const buf = acquireBuffer(bytes.byteLength, undefined, label);
@@ -43,6 +48,91 @@ export class HipTextDecoder {
     this.sin = createTensor(upload(weights.sin), 'f32', [c.maxSeq, c.headDim / 2], 'rope_sin');
     this.ids = acquireBuffer(16, undefined, 'token_ids');
     this.tokenOut = acquireBuffer(16, undefined, 'sampled_token');
+    this.logits = null;
+  }
+
+  // Final RMSNorm + LM head for one hidden row; greedy, or top-k temperature sampling when
+  // `sampling` = {temperature, topK, randomSeed} is given (the logits then go through memory).
+  async recordHead(recorder, temps, hiddenRow, sampling) {
+    const c = this.config;
+    const normed = await recordRMSNorm(recorder, hiddenRow, this.finalNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden });
+    temps.push(normed.buffer);
+    if (sampling && !this.logits) this.logits = acquireBuffer(c.vocab * 4, undefined, 'logits');
+    await recordLmHeadArgmaxF16(recorder, normed, this.embed, {
+      vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: this.tokenOut, outputIndex: 0,
+      logitsOutput: sampling ? this.logits : null,
+    });
+    if (sampling) {
+      await recordGPUSample(recorder, this.logits, c.vocab, Object.assign({ outputBuffer: this.tokenOut, outputIndex: 0 }, sampling));
+    }
+  }
+
+  // Pushes prompt tokens through the batched path (prefill GEMMs + prefill attention), `chunk`
+  // tokens per pass, writing KV rows startPos.. ; returns the token after the last prompt token.
+  // Mirrors the reference's prefill (src/inference/pipelines/text/generator.js) on the HIP ops.
+  async prefill(tokens, startPos = 0, options = {}) {
+    const c = this.config;
+    const chunk = Math.max(1, Math.min(options.chunk || 512, tokens.length));
+    if (tokens.length === 0 || startPos + tokens.length > c.maxSeq) {
+      throw new Error(`[prefill] ${tokens.length} tokens at ${startPos} do not fit maxSeq=${c.maxSeq}`);
+    }
+    const recorder = createCommandRecorder('prefill');
+    const temps = [];
+    const temp = (t) => { temps.push(t.buffer); return t; };
+    const ids = acquireBuffer(chunk * 4, undefined, 'prefill_ids');
+    temps.push(ids);
+    let x = null, T = 0;
+    for (let c0 = 0; c0 < tokens.length; c0 += chunk) {
+      const part = tokens.slice(c0, c0 + chunk);
+      T = part.length;
+      const pos = startPos + c0;
+      uploadData(ids, new Uint32Array(part));
+      x = temp(await recordGather(recorder, ids, this.embed, T, c.hidden, c.vocab, { embeddingDtype: 'f16', outputDtype: 'f32' }));
+      for (let li = 0; li < this.layers.length; li++) {
+        const l = this.layers[li];
+        const normed = temp(await recordRMSNorm(recorder, x, l.inputNorm, c.eps, { batchSize: T, hiddenSize: c.hidden }));
+        const qkv = temp(await recordMatmul(recorder, normed, l.wqkv, T, this.qSize + 2 * this.kSize, c.hidden,
+          { outputDtype: 'f32', role: 'qkv_proj', layerIdx: li }));
+        const split = await recordSplitQKVRMSNormRoPEQK(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps, {
+          numTokens: T, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim,
+          qSize: this.qSize, kSize: this.kSize, vSize: this.kSize, startPos: pos,
+          f16KVCacheWrite: { keysBuffer: l.cacheK.buffer, valuesBuffer: l.cacheV.buffer, dstOffset: pos * this.kSize },
+        });
+        temp(split.Q);
+        const attn = temp(await recordAttention(recorder, split.Q, l.cacheK, l.cacheV, null, c.heads, c.headDim, {
+          seqLen: T, kvLen: pos + T, numKVHeads: c.kvHeads, causal: true, startPos: pos, layerIdx: li,
+        }));
+        const attnFlat = createTensor(attn.buffer, 'f32', [T, this.qSize], 'attn_flat');
+        const x2 = temp(await recordMatmul(recorder, attnFlat, l.wo, T, c.hidden, this.qSize,
+          { outputDtype: 'f32', role: 'o_proj', layerIdx: li, residualTensor: x }));
+        const normed2 = temp(await recordRMSNorm(recorder, x2, l.postAttnNorm, c.eps, { batchSize: T, hiddenSize: c.hidden }));
+        const act = temp(await recordFusedFFN(recorder, normed2, l.wgate, l.wup, c.hidden, c.inter,
+          { batchSize: T, activation: 'silu' }));
+        x = temp(await recordMatmul(recorder, act, l.wdown, T, c.hidden, c.inter,
+          { outputDtype: 'f32', role: 'down_proj', layerIdx: li, residualTensor: x2 }));
+      }
+    }
+    const lastRow = createTensor(bufferWindow(x.buffer, (T - 1) * c.hidden * 4, c.hidden * 4), 'f32', [1, c.hidden], 'last_hidden');
+    await this.recordHead(recorder, temps, lastRow, options.sampling || null);
+    for (const b of temps) recorder.trackTemporaryBuffer(b);
+    recorder.submit();
+    const bytes = await readBufferSlice(this.tokenOut, 0, 4);
+    return new Uint32Array(bytes)[0];
+  }
+
+  // prefill + decode loop: returns the generated token ids.  sampling = {temperature, topK, seed}
+  // draws token i with randomSeed seed + i (greedy when absent), as the reference's generator
+  // advances its seed per step.
+  async generate(promptTokens, maxTokens, sampling = null) {
+    const draw = (i) => (sampling ? { temperature: sampling.temperature, topK: sampling.topK, randomSeed: sampling.seed + i } : null);
+    const out = [];
+    let tok = await this.prefill(promptTokens, 0, { sampling: draw(0) });
+    out.push(tok);
+    for (let i = 1; i < maxTokens; i++) {
+      tok = await this.decodeStep(tok, promptTokens.length + i - 1, { sampling: draw(i) });
+      out.push(tok);
+    }
+    return out;
   }
 
   // Returns the greedy token for `token` at position `pos` (KV rows 0..pos-1 present).
@@ -77,11 +167,15 @@ export class HipTextDecoder {
       x = temp(await recordMatmul(recorder, act, l.wdown, 1, c.hidden, c.inter,
         { outputDtype: 'f32', role: 'down_proj', layerIdx: li, residualTensor: x2 }));
     }
-    const finalNormed = temp(await recordRMSNorm(recorder, x, this.finalNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden }));
-    await recordLmHeadArgmaxF16(recorder, finalNormed, this.embed, {
-      vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: this.tokenOut, outputIndex: 0,
-      logitsOutput: options.logitsOutput || null,
-    });
+    if (options.sampling) {
+      await this.recordHead(recorder, temps, x, options.sampling);
+    } else {
+      const finalNormed = temp(await recordRMSNorm(recorder, x, this.finalNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden }));
+      await recordLmHeadArgmaxF16(recorder, finalNormed, this.embed, {
+        vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: this.tokenOut, outputIndex: 0,
+        logitsOutput: options.logitsOutput || null,
+      });
+    }
     for (const b of temps) recorder.trackTemporaryBuffer(b);
     recorder.submit();
     const bytes = await readBufferSlice(this.tokenOut, 0, 4);   // the only device->host crossing

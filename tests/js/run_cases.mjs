@@ -145,6 +145,12 @@ async function main() {
         tokens.push(tok);
       }
       fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
+    } else if (c.op === 'generate') {
+      // RDRR artifact -> JS loader -> prefill path -> decode loop, greedy or sampled
+      const { config, weights } = loadDecoderWeights(c.dir, c.maxSeq);
+      const dec = new HipTextDecoder(config, weights);
+      const tokens = await dec.generate(c.prompt, c.maxTokens, c.sampling || null);
+      fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
     } else if (c.op === 'sample') {
       const tok = await dh.runGPUSample(dev(c.logits), c.vocab, { temperature: c.temperature, topK: c.topK, randomSeed: c.seed });
       fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array([tok]).buffer));

@@ -95,6 +95,28 @@ def test_prefill_path_matches_the_oracle(chunk):
         tok = nxt
 
 
+def test_sampled_generation_follows_the_sampler_oracle():
+    """generate() with seeded top-k sampling: every drawn token is what the sampler oracle picks from
+    the GPU's own logits of that step with the same seed."""
+    cfg = dict(layers=2, hidden=512, inter=1024, heads=8, kv_heads=4, head_dim=64, vocab=900, eps=1e-6, qk_norm=1,
+               max_seq=40, theta=1e6)
+    layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=51, max_seq=40)
+    gpu = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 40)
+    prompt = [int(t) for t in synth.rng(52).integers(0, cfg["vocab"], 9)]
+    samp = dict(temperature=1.3, topK=12, seed=100)
+    tok = gpu.prefill(prompt, sampling=dict(temperature=1.3, topK=12, randomSeed=100))
+    assert tok == oracle.sample_topk(gpu.read_logits(), 1.3, 12, oracle.seeded_random(100))
+    picked = [tok]
+    for i in range(1, 10):
+        tok = gpu.step(tok, len(prompt) + i - 1, sampling=dict(temperature=1.3, topK=12, randomSeed=100 + i))
+        assert tok == oracle.sample_topk(gpu.read_logits(), 1.3, 12, oracle.seeded_random(100 + i)), i
+        picked.append(tok)
+    again = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 40)
+    assert again.generate(prompt, 10, sampling=samp) == picked
+    greedy = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 40).generate(prompt, 10)
+    assert greedy != picked            # temperature 1.3 over 12 candidates does leave the greedy path
+
+
 def test_batched_decode_matches_step_by_step():
     """n tokens per submit with the token fed back on the device (the reference's batched decode)
     gives the tokens of n single steps with a host round trip each."""

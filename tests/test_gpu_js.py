@@ -235,6 +235,20 @@ def test_js_host_path_parity(tmp_path):
     cases.append(dict(name="rdrr_decoder", op="rdrr_decoder", dir=art_dir, maxSeq=24, prompt=prompt, steps=10))
     checks.append(lambda: [int(t) for t in get("rdrr_decoder.out.bin", np.uint32)] == want2)
 
+    # ---- generate(): prompt through the prefill path, then the decode loop, greedy and with seeded
+    #      top-k sampling; the Python host runs the same kernels on the same artifact
+    from doppler_amd import rdrr as _rdrr
+    pyd = _rdrr.load_decoder(art_dir, 24)
+    want_greedy = pyd.generate(prompt, 8)
+    pyd2 = _rdrr.load_decoder(art_dir, 24)
+    samp = dict(temperature=0.9, topK=20, seed=5)
+    want_sampled = pyd2.generate(prompt, 8, sampling=samp)
+    assert want_greedy[0] == want2[len(prompt) - 1]            # prefill path agrees with the checker's token
+    cases.append(dict(name="gen_greedy", op="generate", dir=art_dir, maxSeq=24, prompt=prompt, maxTokens=8))
+    cases.append(dict(name="gen_sampled", op="generate", dir=art_dir, maxSeq=24, prompt=prompt, maxTokens=8, sampling=samp))
+    checks.append(lambda: [int(t) for t in get("gen_greedy.out.bin", np.uint32)] == want_greedy)
+    checks.append(lambda: [int(t) for t in get("gen_sampled.out.bin", np.uint32)] == want_sampled)
+
     json.dump(dict(cases=cases), open(os.path.join(d, "manifest.json"), "w"))
     p = subprocess.run([NODE, os.path.join(ROOT, "tests", "js", "run_cases.mjs"), d], stdout=subprocess.PIPE,
                        stderr=subprocess.STDOUT, text=True, timeout=500)
