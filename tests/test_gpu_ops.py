@@ -112,6 +112,27 @@ def test_matmul_ragged_shapes(M, N, K):
     assert _matmul_case(M, N, K, seed=1400 + M + N) <= matmul_bar(M)
 
 
+def test_matmul_random_shape_sweep():
+    """Seeded sweep over the dispatch boundaries: M across the 1/2/4/8-row GEMV passes and the GEMM
+    threshold, K with and without a 256 tail and across the LDS limits of the passes, N off the
+    tile sizes, with and without residual / alpha / f16 output."""
+    g = synth.rng(1700)
+    ks = [256, 300, 640, 1024, 1152, 2048, 2304, 3072, 4096, 4352, 6144, 6400, 8192, 12288]
+    for t in range(48):
+        M = int(g.choice([1, 2, 3, 4, 5, 6, 7, 8, 9, 15, 16, 17, 33, 64, 100]))
+        K = int(g.choice(ks))
+        N = int(g.choice([1, 7, 31, 32, 33, 64, 100, 129, 257, 500, 1000]))
+        kw = {}
+        if g.random() < 0.4:
+            kw["residual"] = True
+        if g.random() < 0.3:
+            kw["alpha"] = 0.5
+        if g.random() < 0.2:
+            kw["outputDtype"] = "f16"
+        bar = 2e-3 if kw.get("outputDtype") == "f16" else matmul_bar(M)
+        assert _matmul_case(M, N, K, seed=1701 + t, **kw) <= max(bar, matmul_bar(M)), (M, N, K, kw)
+
+
 @pytest.mark.parametrize("M,N,K,kw", [(512, 6912, 1152, {}), (512, 1152, 6912, dict(residual=True)),
                                       (130, 200, 640, dict(alpha=0.5)), (16, 128, 256, dict(outputDtype="f16")),
                                       (77, 129, 1000, {}), (300, 96, 300, {}),
@@ -211,6 +232,32 @@ def test_fused_ffn_q4k(M, activation, limit):
                           alpha=0.5, swigluLimit=limit)
     want = oracle.q4k_ffn_gate_up(X, Wg, Wu, M, hidden, inter, alpha=0.5, activation=activation, swiglu_limit=limit or 0.0)
     assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
+
+
+def test_fused_ffn_random_shape_sweep():
+    """Seeded sweep of the fused gate/up product (plain and with the RMSNorm prologue) over batch
+    sizes on both sides of every GEMV pass size and of the GEMM threshold, hidden sizes with and
+    without a 256 tail, odd intermediate sizes, both activations."""
+    g = synth.rng(2600)
+    for t in range(24):
+        M = int(g.choice([1, 2, 3, 4, 5, 8, 9, 16, 17, 40]))
+        hidden = int(g.choice([256, 640, 1024, 1152, 2048, 4096, 4352]))
+        inter = int(g.choice([64, 100, 257, 1000, 1536]))
+        act = str(g.choice(["silu", "gelu"]))
+        normed = M <= 8 and g.random() < 0.5
+        Wg, wg = q4k_weight(inter, hidden, seed=2601 + 3 * t)
+        Wu, wu = q4k_weight(inter, hidden, seed=2602 + 3 * t)
+        X = synth.normal_f32((M, hidden), seed=2603 + 3 * t, scale=0.05)
+        if normed:
+            nw = 1.0 + synth.normal_f32((hidden,), seed=2604 + t, scale=0.1)
+            out = ops.runFusedNormedFFN(ops.tensorFromNumpy(X), ops.tensorFromNumpy(nw), 1e-6, wg, wu, hidden, inter,
+                                        batchSize=M, activation=act)
+            xin = oracle.rmsnorm(X, nw, 1e-6)
+        else:
+            out = ops.runFusedFFN(ops.tensorFromNumpy(X), wg, wu, hidden, inter, batchSize=M, activation=act)
+            xin = X
+        want = oracle.q4k_ffn_gate_up(xin, Wg, Wu, M, hidden, inter, alpha=1.0, activation=act)
+        assert rel_l2(ops.readTensor(out), want) <= matmul_bar(M), (M, hidden, inter, act, normed)
 
 
 @pytest.mark.parametrize("M,N,K,offset", [(1, 6144, 4096, False), (2, 1024, 1024, True), (1, 2048, 640, False),
