@@ -3,10 +3,12 @@
 // uniform number.  Follows the reference's sampler oracle, tests/kernels/reference/sample.js:62-92,
 // with the kernel's extras (soft cap, pad id) of src/gpu/kernels/sample.wgsl:35-51.
 //
-// Selection is a tournament of 1024-element bitonic sorts in LDS: round 0 sorts slices of the
-// vocabulary and keeps the best k of each, later rounds sort 1024 surviving candidates at a time,
-// until one workgroup holds them all; that workgroup also draws the token.  k <= 256, so a round
-// shrinks the field at least four-fold.
+// Selection is a tournament of 1024-element bitonic sorts (registers + lane shuffles, LDS only
+// for the widest exchanges): round 0 sorts slices of the vocabulary and keeps the best k of
+// each, later rounds sort 1024 surviving candidates at a time, until one workgroup holds them
+// all; that workgroup also draws the token.  k <= 256, so a round shrinks the field at least
+// four-fold.  A round costs ~25 us whatever its grid: the 55 dependent exchange steps of the
+// network set its length (3 rounds at k = 40 over 151,936 logits, 5 at k = 256).
 #include <algorithm>
 #include <cfloat>
 
@@ -37,56 +39,105 @@ __device__ __forceinline__ bool ranks_before(float av, uint32_t ai, float bv, ui
   return av > bv || (av == bv && ai < bi);
 }
 
+// Sorts 1024 (value, id) pairs best first, four per thread: element i = 4 * tid + r.  A bitonic
+// network; exchanges at distance 1 and 2 stay inside a thread's registers, distances 4..128 are
+// lane shuffles inside a wave, only the three steps at distance 256 and 512 go through LDS and
+// a barrier.
+__device__ __forceinline__ void sort1024(float (&v)[4], uint32_t (&id)[4], float* s_val, uint32_t* s_idx, int tid) {
+#pragma unroll 1
+  for (int k = 2; k <= kSortN; k <<= 1) {
+#pragma unroll 1
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      if (j >= 4) {
+        float pv[4];
+        uint32_t pi[4];
+        if (j >= 256) {
+          __syncthreads();
+#pragma unroll
+          for (int r = 0; r < 4; r++) { s_val[4 * tid + r] = v[r]; s_idx[4 * tid + r] = id[r]; }
+          __syncthreads();
+#pragma unroll
+          for (int r = 0; r < 4; r++) { pv[r] = s_val[(4 * tid + r) ^ j]; pi[r] = s_idx[(4 * tid + r) ^ j]; }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            pv[r] = __shfl_xor(v[r], j >> 2, 64);
+            pi[r] = (uint32_t)__shfl_xor((int)id[r], j >> 2, 64);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int i = 4 * tid + r;
+          const bool keep_better = ((i & j) == 0) == ((i & k) == 0);
+          const bool partner_better = ranks_before(pv[r], pi[r], v[r], id[r]);
+          if (partner_better == keep_better) { v[r] = pv[r]; id[r] = pi[r]; }
+        }
+      } else {
+        // pairs (r, r + j) inside the thread: j = 2 -> (0,2) (1,3); j = 1 -> (0,1) (2,3)
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+          const int lo = j == 2 ? p : 2 * p, hi = lo + j;
+          const bool best_first = ((4 * tid + lo) & k) == 0;
+          float av = v[0], bv = v[0];
+          uint32_t ai = id[0], bi = id[0];
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            if (r == lo) { av = v[r]; ai = id[r]; }
+            if (r == hi) { bv = v[r]; bi = id[r]; }
+          }
+          const bool swap = best_first ? ranks_before(bv, bi, av, ai) : ranks_before(av, ai, bv, bi);
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            if (swap && r == lo) { v[r] = bv; id[r] = bi; }
+            if (swap && r == hi) { v[r] = av; id[r] = ai; }
+          }
+        }
+      }
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void topk_round_kernel(const SampleArgs a) {
   __shared__ float val[kSortN];
   __shared__ uint32_t idx[kSortN];
   __shared__ double prob[kMaxTopK];
   const int tid = threadIdx.x;
   const int base = blockIdx.x * kSortN;
-  for (int i = tid; i < kSortN; i += 256) {
-    const int g = base + i;
-    float v = -INFINITY;                      // padding never ranks before a real entry
-    uint32_t id = 0xFFFFFFFFu;
+  float v[4];
+  uint32_t id[4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    const int g = base + 4 * tid + r;
+    v[r] = -INFINITY;                         // padding never ranks before a real entry
+    id[r] = 0xFFFFFFFFu;
     if (g < a.n_in) {
       if (a.logits) {
-        id = (uint32_t)g;
-        v = a.logits[g];
-        if (a.softcap > 0.f) v = a.softcap * tanhf(v / a.softcap);
-        if ((int64_t)g == a.pad_id || !(v == v)) { v = -INFINITY; id = 0xFFFFFFFFu; }   // pad id, NaN: out
+        float x = a.logits[g];
+        if (a.softcap > 0.f) x = a.softcap * tanhf(x / a.softcap);
+        if ((int64_t)g != a.pad_id && x == x) { v[r] = x; id[r] = (uint32_t)g; }   // pad id, NaN: out
       } else {
-        v = a.in_val[g];
-        id = a.in_idx[g];
+        v[r] = a.in_val[g];
+        id[r] = a.in_idx[g];
       }
     }
-    val[i] = v;
-    idx[i] = id;
   }
-  __syncthreads();
-  // bitonic sort, best first
-  for (int k = 2; k <= kSortN; k <<= 1) {
-    for (int j = k >> 1; j > 0; j >>= 1) {
-      for (int t = tid; t < kSortN / 2; t += 256) {
-        const int lo = 2 * t - (t & (j - 1)), hi = lo + j;       // pair (lo, lo + j)
-        const bool descending = (lo & k) == 0;
-        const float av = val[lo], bv = val[hi];
-        const uint32_t ai = idx[lo], bi = idx[hi];
-        const bool swap = descending ? ranks_before(bv, bi, av, ai) : ranks_before(av, ai, bv, bi);
-        if (swap) {
-          val[lo] = bv; idx[lo] = bi;
-          val[hi] = av; idx[hi] = ai;
-        }
-      }
-      __syncthreads();
-    }
-  }
+  sort1024(v, id, val, idx, tid);
   if (gridDim.x > 1) {
-    for (int i = tid; i < a.top_k; i += 256) {
-      a.out_val[blockIdx.x * a.top_k + i] = val[i];
-      a.out_idx[blockIdx.x * a.top_k + i] = idx[i];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const int i = 4 * tid + r;
+      if (i < a.top_k) {
+        a.out_val[blockIdx.x * a.top_k + i] = v[r];
+        a.out_idx[blockIdx.x * a.top_k + i] = id[r];
+      }
     }
     return;
   }
   // ---- the field is down to one workgroup: softmax over the candidates and the draw
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 4; r++) { val[4 * tid + r] = v[r]; idx[4 * tid + r] = id[r]; }
+  __syncthreads();
   int n = min(a.top_k, a.n_in);
   while (n > 0 && idx[n - 1] == 0xFFFFFFFFu) n--;               // padding / excluded entries
   const double mx = n > 0 ? (double)val[0] / a.temperature : 0.0;
