@@ -8,7 +8,15 @@
 // rescale.  (Merging inside the split kernel, by the last workgroup to arrive per kv head, was
 // measured slower: store acknowledgement, arrival atomic and two rounds of agent-scope loads
 // are four dependent memory round trips, more than the kernel boundary costs.)
+//
+// The decode step's own q/k/v can be taken raw from the stacked projection (QKV variant): the
+// per-head RMSNorm and the rotary embedding of the query heads are redone in the prologue of
+// every workgroup (a few hundred elements), and the workgroup whose chunk holds the new
+// position also norms and rotates the new key, narrows key and value to f16, appends them to
+// the cache and uses them straight from registers.  That removes the split-QKV/norm/RoPE/
+// KV-write kernel (one launch, ~4.5 us per layer) from the decode step.
 #include <algorithm>
+#include <type_traits>
 #include <cfloat>
 
 #include "dh_common.h"
@@ -27,6 +35,18 @@ struct AttnArgs {
   int H, Hkv, G, kbeg, kend, nsplit, tiles_per_split;
   float scale, softcap;
   int kv_start, ring_window;  // ring_window > 0: row = (kv_start + k) % ring_window
+  // ---- QKV variant only
+  const float* qkv;     // [(H + 2 Hkv) * D]: raw q heads, k heads, v heads of the step's token
+  const float* qw;      // per-head RMSNorm weights [D] (null when use_norm == 0)
+  const float* kw;
+  const float* cos_row; // rotary tables at the row of this position: [rotary_dim / 2]
+  const float* sin_row;
+  __half* Kw;           // the caches again, writable
+  __half* Vw;
+  int64_t new_row;      // first element of the appended row in the caches
+  int rotary_half, interleaved, w_offset, use_norm;
+  float eps;
+  int c_new, j_new;     // chunk, and key within the chunk, of the appended position
 };
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -88,7 +108,10 @@ __device__ __forceinline__ float row_group_sum(float v) {
 //            meet in a wave-private LDS buffer at the end.
 // K and V of the next chunk are requested before the current one is consumed.
 // GT: query heads per kv head rounded up to 1, 2, 4 or 8 (bounds the unrolled per-head code).
-template <int D, int GT>
+// QKV: the step's q, k, v arrive raw (see the top of the file); the appended key is the last
+// visible one, so the lanes that would read its row, or a clamped copy of it, from the not yet
+// written cache are patched from registers.
+template <int D, int GT, bool QKV>
 __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a) {
   constexpr int STEPS = D / 32;          // MFMAs per 16 keys
   constexpr int DW = D / 4;              // output dims per wave
@@ -143,23 +166,146 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
     }                                                                                             \
   } while (0)
 
-  if (split < nchunks) DH_ATTN_LOAD(split);
+  // The appended key/value in fragment form (QKV variant, owner workgroup): lanes whose key, or
+  // whose clamped stand-in for a key past the end, is the appended one take it from here.
+  uint4 knew[STEPS] = {};
+  uint2 vnew = make_uint2(0u, 0u);
+#define DH_ATTN_PATCH(c_)                                                                         \
+  do {                                                                                            \
+    if (QKV && (c_) == a.c_new) {                                                                 \
+      if (key_s >= a.j_new) {                                                                     \
+        _Pragma("unroll") for (int s = 0; s < STEPS; s++) kf[s] = knew[s];                        \
+      }                                                                                           \
+      _Pragma("unroll") for (int j = 0; j < NJ; j++)                                              \
+        if (kh + KH * j >= a.j_new) vn[j] = vnew;                                                 \
+    }                                                                                             \
+  } while (0)
+
+  if (!QKV && split < nchunks) DH_ATTN_LOAD(split);
 
   // ---- query fragments (A operand): row = lane & 15 -> head row>>1, high part / residual
   half8_t qa[STEPS];
+  if constexpr (QKV) {
+    // The rows of the step (G query heads; where the appended position is met, also the new key
+    // and value) are prepared once per workgroup, one row per half wave (32 lanes x D/32
+    // consecutive elements, so the loads are coalesced and tiny), and handed to the fragment
+    // layout through LDS.  Their loads go out before those of the first K/V chunk, so they
+    // return first and the preparation runs under the latency of the cache reads.
+    constexpr int EPL = D / 32;                       // elements per lane
+    constexpr int ROUNDS = (GT + 2 + 7) / 8;          // 8 half waves per round
+    __shared__ __align__(16) float q_rows[GT][D];
+    __shared__ __align__(16) __half k_row[D];
+    __shared__ __align__(16) __half v_row[D];
+    const bool owner = split == a.c_new % a.nsplit;
+    const int hl = lane & 31;
+    const int rotary_dim = 2 * a.rotary_half;
+    float rx[ROUNDS][EPL], rw[ROUNDS][EPL], rc[ROUNDS][EPL], rs[ROUNDS][EPL];
+    int role[ROUNDS];                                  // 0 idle, 1 query head, 2 new key, 3 new value
 #pragma unroll
-  for (int s = 0; s < STEPS; s++) {
+    for (int r = 0; r < ROUNDS; r++) {
+      const int slot = 8 * r + 2 * wave + (lane >> 5);
+      role[r] = slot < G ? 1 : (owner && slot == G) ? 2 : (owner && slot == G + 1) ? 3 : 0;
+      const int64_t row = role[r] == 1 ? kvh * G + slot : role[r] == 2 ? a.H + kvh : role[r] == 3 ? a.H + a.Hkv + kvh : 0;
+      const float* src = a.qkv + row * D + EPL * hl;
+      const float* wsrc = !a.use_norm ? nullptr : role[r] == 1 ? a.qw : role[r] == 2 ? a.kw : nullptr;
+      typedef __attribute__((ext_vector_type(EPL))) float row_vec_t;
+      const row_vec_t xv = *reinterpret_cast<const row_vec_t*>(src);
+      const row_vec_t wv = *reinterpret_cast<const row_vec_t*>((wsrc ? wsrc : a.qkv) + EPL * hl);
 #pragma unroll
-    for (int i = 0; i < 8; i++) qa[s][i] = (_Float16)0.f;
-    if ((qrow >> 1) < G) {
-      const float* qp = a.Q + (int64_t)(kvh * G + (qrow >> 1)) * D + 32 * s + 8 * kg;
+      for (int i = 0; i < EPL; i++) {
+        const int e = EPL * hl + i;
+        const bool rotated = (role[r] == 1 || role[r] == 2) && e < rotary_dim;
+        const int p = a.interleaved ? e >> 1 : e & (a.rotary_half - 1);
+        rx[r][i] = xv[i];
+        rw[r][i] = wsrc ? wv[i] : 1.0f;
+        rc[r][i] = a.cos_row[rotated ? p : 0];
+        rs[r][i] = a.sin_row[rotated ? p : 0];
+      }
+    }
+    DH_ATTN_LOAD(split);        // never empty: there are no more splits than chunks
+#pragma unroll
+    for (int r = 0; r < ROUNDS; r++) {
+      const int slot = 8 * r + 2 * wave + (lane >> 5);
+      float y[EPL];
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < EPL; i++) ss = fmaf(rx[r][i], rx[r][i], ss);
+#pragma unroll
+      for (int off = 1; off < 32; off <<= 1) ss += __shfl_xor(ss, off, 64);
+      const bool normed = a.use_norm && (role[r] == 1 || role[r] == 2);
+      const float inv = normed ? 1.0f / sqrtf(ss / (float)D + a.eps) : 1.0f;
+#pragma unroll
+      for (int i = 0; i < EPL; i++)
+        y[i] = normed ? rx[r][i] * inv * (a.w_offset ? 1.0f + rw[r][i] : rw[r][i]) : rx[r][i];
+      const bool rotates = role[r] == 1 || role[r] == 2;
+      if (a.interleaved) {
+#pragma unroll
+        for (int i = 0; i < EPL; i += 2) {
+          const float x0 = y[i], x1 = y[i + 1];
+          const bool on = rotates && EPL * hl + i < rotary_dim;
+          y[i] = on ? x0 * rc[r][i] - x1 * rs[r][i] : x0;
+          y[i + 1] = on ? x0 * rs[r][i + 1] + x1 * rc[r][i + 1] : x1;
+        }
+      } else {
+        const int pd = a.rotary_half / EPL;           // lanes between the partners (p, p + half)
+        const bool low = EPL * hl < a.rotary_half;
+#pragma unroll
+        for (int i = 0; i < EPL; i++) {
+          const float other = __shfl_xor(y[i], pd, 64);
+          const float x0 = low ? y[i] : other, x1 = low ? other : y[i];
+          const float rot = low ? x0 * rc[r][i] - x1 * rs[r][i] : x0 * rs[r][i] + x1 * rc[r][i];
+          y[i] = rotates && EPL * hl + i < rotary_dim ? rot : y[i];
+        }
+      }
+      if (role[r] == 1) {
+#pragma unroll
+        for (int i = 0; i < EPL; i++) q_rows[min(slot, GT - 1)][EPL * hl + i] = y[i];
+      } else if (role[r] == 2 || role[r] == 3) {
+        __half* lrow = role[r] == 2 ? k_row : v_row;
+        __half* grow = (role[r] == 2 ? a.Kw : a.Vw) + a.new_row + (int64_t)kvh * D;
+#pragma unroll
+        for (int i = 0; i < EPL; i += 2) {
+          const __half2 h2 = __floats2half2_rn(y[i], y[i + 1]);
+          *reinterpret_cast<__half2*>(lrow + EPL * hl + i) = h2;
+          *reinterpret_cast<__half2*>(grow + EPL * hl + i) = h2;
+        }
+      }
+    }
+    __syncthreads();
+    const bool live = (qrow >> 1) < G;
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+      const float* qp = &q_rows[min(qrow >> 1, GT - 1)][32 * s + 8 * kg];
       const float4 q0 = reinterpret_cast<const float4*>(qp)[0], q1 = reinterpret_cast<const float4*>(qp)[1];
       const float qv[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
 #pragma unroll
       for (int i = 0; i < 8; i++) {
-        const float xs = qv[i] * a.scale;
+        const float xs = live ? qv[i] * a.scale : 0.f;
         const _Float16 h = (_Float16)xs;
         qa[s][i] = (qrow & 1) ? (_Float16)(xs - (float)h) : h;
+      }
+    }
+    if (owner) {
+#pragma unroll
+      for (int s = 0; s < STEPS; s++) knew[s] = *reinterpret_cast<const uint4*>(k_row + 32 * s + 8 * kg);
+      vnew = *reinterpret_cast<const uint2*>(v_row + DW * wave + 4 * dq);
+      DH_ATTN_PATCH(split);
+    }
+  } else {
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) qa[s][i] = (_Float16)0.f;
+      if ((qrow >> 1) < G) {
+        const float* qp = a.Q + (int64_t)(kvh * G + (qrow >> 1)) * D + 32 * s + 8 * kg;
+        const float4 q0 = reinterpret_cast<const float4*>(qp)[0], q1 = reinterpret_cast<const float4*>(qp)[1];
+        const float qv[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const float xs = qv[i] * a.scale;
+          const _Float16 h = (_Float16)xs;
+          qa[s][i] = (qrow & 1) ? (_Float16)(xs - (float)h) : h;
+        }
       }
     }
   }
@@ -183,7 +329,10 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
       d = __builtin_amdgcn_mfma_f32_16x16x32_f16(qa[s], __builtin_bit_cast(half8_t, kf[s]), d, 0, 0, 0);
 #pragma unroll
     for (int j = 0; j < NJ; j++) vf[j] = vn[j];
-    if (c + a.nsplit < nchunks) DH_ATTN_LOAD(c + a.nsplit);
+    if (c + a.nsplit < nchunks) {
+      DH_ATTN_LOAD(c + a.nsplit);
+      DH_ATTN_PATCH(c + a.nsplit);
+    }
     // lane (key, kg) holds rows 4kg..4kg+3 = heads 2kg (high + residual), 2kg+1
     {
       float sc2[2] = {d[0] + d[1], d[2] + d[3]};
@@ -258,6 +407,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
   }
   DH_ATS();
 #undef DH_ATTN_LOAD
+#undef DH_ATTN_PATCH
 
   // ---- key groups meet in the wave's LDS buffer, then the split's (o, m, l) go out
 #pragma unroll
@@ -361,13 +511,13 @@ int choose_splits(int Hkv, int nkeys) {
   return std::min(tiles, want);
 }
 
-template <int D>
+template <int D, bool QKV>
 int launch(const AttnArgs& a, const char* op) {
   const dim3 grid(a.Hkv, a.nsplit), block(256);
-  if (a.G <= 1) hipLaunchKernelGGL((attn_decode_split_kernel<D, 1>), grid, block, 0, dh::stream(), a);
-  else if (a.G <= 2) hipLaunchKernelGGL((attn_decode_split_kernel<D, 2>), grid, block, 0, dh::stream(), a);
-  else if (a.G <= 4) hipLaunchKernelGGL((attn_decode_split_kernel<D, 4>), grid, block, 0, dh::stream(), a);
-  else hipLaunchKernelGGL((attn_decode_split_kernel<D, 8>), grid, block, 0, dh::stream(), a);
+  if (a.G <= 1) hipLaunchKernelGGL((attn_decode_split_kernel<D, 1, QKV>), grid, block, 0, dh::stream(), a);
+  else if (a.G <= 2) hipLaunchKernelGGL((attn_decode_split_kernel<D, 2, QKV>), grid, block, 0, dh::stream(), a);
+  else if (a.G <= 4) hipLaunchKernelGGL((attn_decode_split_kernel<D, 4, QKV>), grid, block, 0, dh::stream(), a);
+  else hipLaunchKernelGGL((attn_decode_split_kernel<D, 8, QKV>), grid, block, 0, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   if (a.nsplit > 1) {
     hipLaunchKernelGGL(attn_decode_merge_kernel<D>, dim3(a.H), dim3(D), 0, dh::stream(), a.ws, a.O, a.nsplit);
@@ -439,7 +589,70 @@ int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_
   a.scale = scale; a.softcap = softcap;
   a.kv_start = kv_start;
   a.ring_window = kv_layout == DH_KV_RING ? sliding_window : 0;
-  return D == 64 ? launch<64>(a, op) : launch<128>(a, op);
+  return D == 64 ? launch<64, false>(a, op) : launch<128, false>(a, op);
+}
+
+int dh_attn_decode_qkv_supported(int H, int Hkv, int D, int rotary_dim, int interleaved) {
+  if (H <= 0 || Hkv <= 0 || H % Hkv || H / Hkv > kMaxG || (D != 64 && D != 128)) return 0;
+  if (rotary_dim <= 0 || rotary_dim > D || rotary_dim % 2) return 0;
+  if (interleaved) return 1;                       // pairs (2p, 2p + 1): always inside one lane
+  // pairs (p, p + half): half a power of two and at least one lane's D/32 elements
+  return (rotary_dim & (rotary_dim - 1)) == 0 && rotary_dim / 2 >= D / 32;
+}
+
+int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float* d_k_weight, const float* d_cos,
+                       const float* d_sin, void* d_cache_k, void* d_cache_v, float* d_O, int H, int Hkv, int D,
+                       int start_pos, int rotary_dim, int interleaved, float eps, int weight_offset, int use_norm,
+                       float scale, float softcap, int sliding_window, int kv_start, int kv_layout,
+                       void* d_workspace) {
+  const char* op = "dh_attn_decode_qkv";
+  DH_REQUIRE_INIT(op);
+  if (H <= 0 || Hkv <= 0 || D <= 0) return dh::fail(1, "[%s] numHeads/numKVHeads/headDim must be positive", op);
+  if (H % Hkv) return dh::fail(1, "[%s] numHeads=%d must be a multiple of numKVHeads=%d", op, H, Hkv);
+  if (!dh_attn_decode_qkv_supported(H, Hkv, D, rotary_dim, interleaved))
+    return dh::fail(1, "[%s] shape not served (heads %d/%d, headDim %d, rotaryDim %d, interleaved %d): use "
+                       "dh_qkv_norm_rope_kvwrite + dh_attn_decode", op, H, Hkv, D, rotary_dim, interleaved);
+  if (start_pos < 0 || sliding_window < 0 || kv_start < 0 || kv_start > start_pos)
+    return dh::fail(1, "[%s] need 0 <= kvStart <= startPos and slidingWindow >= 0", op);
+  if (kv_layout != DH_KV_CONTIGUOUS && kv_layout != DH_KV_RING)
+    return dh::fail(1, "[%s] kvLayout %d not supported (contiguous, ring)", op, kv_layout);
+  if (kv_layout == DH_KV_RING && sliding_window <= 0)
+    return dh::fail(1, "[%s] ring layout needs slidingWindow > 0", op);
+  if (!d_qkv || !d_cos || !d_sin || !d_cache_k || !d_cache_v || !d_O) return dh::fail(1, "[%s] null pointer", op);
+  if (use_norm && (!d_q_weight || !d_k_weight)) return dh::fail(1, "[%s] q/k norm weights are required", op);
+  const int half = rotary_dim / 2;
+  const float* cos_row = d_cos + (int64_t)start_pos * half;
+  const float* sin_row = d_sin + (int64_t)start_pos * half;
+  if ((reinterpret_cast<uintptr_t>(d_cache_k) | reinterpret_cast<uintptr_t>(d_cache_v) |
+       reinterpret_cast<uintptr_t>(d_qkv) | reinterpret_cast<uintptr_t>(d_q_weight) |
+       reinterpret_cast<uintptr_t>(d_k_weight)) & 15)
+    return dh::fail(1, "[%s] qkv, the norm weights and the caches must be 16-byte aligned", op);
+
+  // visible keys [kbeg, kend) in cache-relative indices; the appended position is kend - 1
+  const int64_t kend = (int64_t)start_pos - kv_start + 1;
+  int64_t kbeg = 0;
+  if (sliding_window > 0 && start_pos >= sliding_window)
+    kbeg = std::max<int64_t>(0, (int64_t)start_pos - sliding_window + 1 - kv_start);
+  AttnArgs a{};
+  a.K = static_cast<const __half*>(d_cache_k); a.V = static_cast<const __half*>(d_cache_v);
+  a.Kw = static_cast<__half*>(d_cache_k); a.Vw = static_cast<__half*>(d_cache_v);
+  a.O = d_O; a.ws = static_cast<float*>(d_workspace);
+  a.H = H; a.Hkv = Hkv; a.G = H / Hkv;
+  a.kbeg = (int)kbeg; a.kend = (int)kend;
+  const int nkeys = (int)(kend - kbeg);
+  a.nsplit = choose_splits(Hkv, nkeys);
+  if (a.nsplit > 1 && !d_workspace) return dh::fail(1, "[%s] workspace is required", op);
+  a.scale = scale; a.softcap = softcap;
+  a.kv_start = kv_start;
+  a.ring_window = kv_layout == DH_KV_RING ? sliding_window : 0;
+  a.qkv = d_qkv; a.qw = d_q_weight; a.kw = d_k_weight; a.cos_row = cos_row; a.sin_row = sin_row;
+  a.rotary_half = half; a.interleaved = interleaved; a.w_offset = weight_offset; a.use_norm = use_norm;
+  a.eps = eps;
+  const int64_t row = a.ring_window > 0 ? start_pos % a.ring_window : start_pos;
+  a.new_row = row * Hkv * D;
+  a.c_new = (nkeys - 1) / kTileKeys;
+  a.j_new = (nkeys - 1) % kTileKeys;
+  return D == 64 ? launch<64, true>(a, op) : launch<128, true>(a, op);
 }
 
 }  // extern "C"

@@ -42,7 +42,8 @@ def c_hidden_ok(cfg):
 class HipDecoder:
     TOKEN_RING = 64      # tokens one decode_batch submit can produce
 
-    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True, chain=False):
+    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True, chain=False,
+                 fuse_qkv_attention=True):
         """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
         layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
         input_norm, post_attn_norm, q_norm, k_norm: f32); embed_bits: uint16 [vocab, hidden]."""
@@ -56,6 +57,10 @@ class HipDecoder:
         self._chains = None
         self.L = capi.init(torch.cuda.current_device())
         c = self.cfg
+        # decode steps: q/k norm + RoPE + KV append run inside the attention kernel when the head
+        # geometry allows it (one launch fewer per layer)
+        self.fuse_qkv_attention = bool(fuse_qkv_attention and self.L.dh_attn_decode_qkv_supported(
+            c["heads"], c["kv_heads"], c["head_dim"], c["head_dim"], 0))
         self.max_seq = max_seq
         H, Hkv, D, Hd, I = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"], c["inter"]
         self.qs, self.ks = H * D, Hkv * D
@@ -130,13 +135,7 @@ class HipDecoder:
                                 c["eps"], 0, None, None, None, 1.0))
                 ck(L.dh_q4k_matmul(self.normed.data_ptr(), capi.F32, d["wqkv"].data_ptr(), self.qkv.data_ptr(),
                                    capi.F32, 1, self.qs + 2 * self.ks, Hd, 1.0, None))
-            ck(L.dh_qkv_norm_rope_kvwrite(self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
-                                          self.cos.data_ptr(), self.sin.data_ptr(), self.q.data_ptr(),
-                                          d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), 1, H, Hkv, D, pos, D, 0,
-                                          c["eps"], 0, pos * self.ks, int(c.get("qk_norm", 1))))
-            ck(L.dh_attn_decode(self.q.data_ptr(), d["cache_k"].data_ptr(), d["cache_v"].data_ptr(),
-                                self.attn.data_ptr(), H, Hkv, D, pos + 1, self.scale, 1, pos, 0.0, 0, 0,
-                                capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
+            self._enqueue_attention(d, pos)
             ck(L.dh_q4k_matmul(self.attn.data_ptr(), capi.F32, d["wo"].data_ptr(), x2.data_ptr(), capi.F32, 1, Hd,
                                self.qs, 1.0, x.data_ptr()))
             if self.fuse_norm:
@@ -155,6 +154,26 @@ class HipDecoder:
         ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
                                   self.lm_ws.data_ptr(), self.token.data_ptr(), self._out_index,
                                   self.logits.data_ptr() if want_logits else None))
+
+    def _enqueue_attention(self, d, pos):
+        """self.qkv (raw stacked projection of the step's token) -> self.attn, appending the
+        token's key/value to the layer's cache."""
+        L, c, ck = self.L, self.cfg, capi.check
+        H, Hkv, D = c["heads"], c["kv_heads"], c["head_dim"]
+        use_norm = int(c.get("qk_norm", 1))
+        if self.fuse_qkv_attention:
+            ck(L.dh_attn_decode_qkv(self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
+                                    self.cos.data_ptr(), self.sin.data_ptr(), d["cache_k"].data_ptr(),
+                                    d["cache_v"].data_ptr(), self.attn.data_ptr(), H, Hkv, D, pos, D, 0, c["eps"], 0,
+                                    use_norm, self.scale, 0.0, 0, 0, capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
+            return
+        ck(L.dh_qkv_norm_rope_kvwrite(self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
+                                      self.cos.data_ptr(), self.sin.data_ptr(), self.q.data_ptr(),
+                                      d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), 1, H, Hkv, D, pos, D, 0,
+                                      c["eps"], 0, pos * self.ks, use_norm))
+        ck(L.dh_attn_decode(self.q.data_ptr(), d["cache_k"].data_ptr(), d["cache_v"].data_ptr(),
+                            self.attn.data_ptr(), H, Hkv, D, pos + 1, self.scale, 1, pos, 0.0, 0, 0,
+                            capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
 
     def _build_chains(self):
         """One dh_gemv_phase array per layer: o_proj (+residual) -> RMSNorm + gate/up + SiLU ->
@@ -193,13 +212,7 @@ class HipDecoder:
                                    first["wqkv"].data_ptr(), self.qkv.data_ptr(), capi.F32, 1,
                                    self.qs + 2 * self.ks, Hd, 1.0, None))
         for d, chain in zip(self.layers, self._chains):
-            ck(L.dh_qkv_norm_rope_kvwrite(self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
-                                          self.cos.data_ptr(), self.sin.data_ptr(), self.q.data_ptr(),
-                                          d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), 1, H, Hkv, D, pos, D, 0,
-                                          c["eps"], 0, pos * self.ks, int(c.get("qk_norm", 1))))
-            ck(L.dh_attn_decode(self.q.data_ptr(), d["cache_k"].data_ptr(), d["cache_v"].data_ptr(),
-                                self.attn.data_ptr(), H, Hkv, D, pos + 1, self.scale, 1, pos, 0.0, 0, 0,
-                                capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
+            self._enqueue_attention(d, pos)
             ck(L.dh_q4k_gemv_chain(chain, len(chain)))
         ck(L.dh_rmsnorm(self.x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd,
                         c["eps"], 0, None, None, None, 1.0))

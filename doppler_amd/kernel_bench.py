@@ -177,6 +177,20 @@ def attn_cases(L, T, rows, reps):
                 algo = kv_bytes + H * D * 8
                 emit(rows, config=cfg, kernel="attn_decode (cfg%d)" % cfg, shape="H=%d/%d D=128 ctx=%d" % (H, Hkv, ctx),
                      mode=mode, us=round(us, 3), achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
+            if ctx >= 2048:
+                # the same step taken straight from the stacked projection (q/k norm, RoPE and KV append inside)
+                qkv = torch.randn((H + 2 * Hkv) * D, device="cuda")
+                w = torch.ones(D, device="cuda")
+                cs = torch.rand(ctx, D // 2, device="cuda")
+                for mode in ("rotating", "warm"):
+                    n = copies if mode == "rotating" else 1
+                    us = T.us(lambda i: capi.check(L.dh_attn_decode_qkv(
+                        qkv.data_ptr(), w.data_ptr(), w.data_ptr(), cs.data_ptr(), cs.data_ptr(),
+                        K.data_ptr() + (i % n) * step, V.data_ptr() + (i % n) * step, o.data_ptr(), H, Hkv, D, ctx - 1, D, 0,
+                        1e-6, 0, 1, 1.0 / D ** 0.5, 0.0, 0, 0, 0, ws.data_ptr())), reps)
+                    algo = kv_bytes + (H + 2 * Hkv) * D * 4 + H * D * 4
+                    emit(rows, config=cfg, kernel="attn_decode_qkv (cfg%d)" % cfg, shape="H=%d/%d D=128 ctx=%d" % (H, Hkv, ctx),
+                         mode=mode, us=round(us, 3), achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
             del K, V
 
 

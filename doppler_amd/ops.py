@@ -401,6 +401,46 @@ def runSplitQKVRMSNormRoPEQK(qkvTensor, qWeight, kWeight, freqsCos, freqsSin, ep
                 wroteF16KVCache=True)
 
 
+def decodeAttentionFromQKVSupported(numHeads, numKVHeads, headDim, rotaryDim=None, interleaved=False):
+    rotaryDim = headDim if rotaryDim is None else rotaryDim
+    return bool(_lib().dh_attn_decode_qkv_supported(numHeads, numKVHeads, headDim, rotaryDim, int(bool(interleaved))))
+
+
+def runDecodeAttentionFromQKV(qkvTensor, qWeight, kWeight, freqsCos, freqsSin, eps, keysBuffer, valuesBuffer, numHeads,
+                              numKVHeads, headDim, startPos, rotaryDim=None, interleaved=False,
+                              rmsNormWeightOffset=False, useNorm=True, scale=None, attnSoftcap=0, slidingWindow=0,
+                              kvStart=0, kvLayout="contiguous", outputBuffer=None, workspace=None, **_ignored):
+    """One decode step of runSplitQKVRMSNormRoPEQK (f16KVCacheWrite at the row of startPos,
+    src/gpu/kernels/split-qkv-rmsnorm-rope-qk.js:244) followed by runAttention with seqLen == 1
+    (src/gpu/kernels/attention.js:2007) in one launch: the new key/value are appended to the cache
+    and the token attends to rows up to and including its own."""
+    rotaryDim = headDim if rotaryDim is None else rotaryDim
+    scale = 1.0 / math.sqrt(headDim) if scale is None else scale
+    if qkvTensor.dtype != "f32":
+        raise DopplerHipError("[Attention] fused decode requires f32 QKV input, got %s." % qkvTensor.dtype)
+    layouts = {"contiguous": capi.KV_CONTIGUOUS, "ring": capi.KV_RING}
+    if kvLayout not in layouts:
+        raise DopplerHipError("[Attention] kvLayout %r is not supported by the HIP path" % (kvLayout,))
+    if _nbytes(qkvTensor) < (numHeads + 2 * numKVHeads) * headDim * 4:
+        raise DopplerHipError("[Attention] fused decode: qkv tensor smaller than (H + 2 Hkv) * headDim floats")
+    rows = slidingWindow if kvLayout == "ring" else startPos + 1
+    if min(_nbytes(keysBuffer), _nbytes(valuesBuffer)) < rows * numKVHeads * headDim * 2:
+        raise DopplerHipError("[Attention] KV buffer smaller than %d rows" % rows)
+    if min(_nbytes(freqsCos), _nbytes(freqsSin)) < (startPos + 1) * (rotaryDim // 2) * 4:
+        raise DopplerHipError("[Attention] rotary tables end before position %d" % startPos)
+    out = _out(outputBuffer, padToQ4KBlock(numHeads * headDim) * 4)
+    if workspace is None:
+        workspace = acquireBuffer(attentionWorkspaceBytes(numHeads, headDim, max(startPos - kvStart + 1, 1)))
+    capi.check(_lib().dh_attn_decode_qkv(_ptr(qkvTensor), _ptr(qWeight) if useNorm else None,
+                                         _ptr(kWeight) if useNorm else None, _ptr(freqsCos), _ptr(freqsSin),
+                                         _ptr(keysBuffer), _ptr(valuesBuffer), out.data_ptr(), numHeads, numKVHeads,
+                                         headDim, startPos, rotaryDim, int(bool(interleaved)), eps,
+                                         int(bool(rmsNormWeightOffset)), int(bool(useNorm)), scale,
+                                         float(attnSoftcap), slidingWindow, kvStart, layouts[kvLayout],
+                                         _ptr(workspace)))
+    return Tensor(out, "f32", (1, numHeads, headDim), "attention_output")
+
+
 # ------------------------------------------------------------------ elementwise
 
 def runResidualAdd(a, b, size, outputBuffer=None, outputScale=None, **_ignored):

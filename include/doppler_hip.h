@@ -171,6 +171,24 @@ int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_
                    int Hkv, int D, int kv_len, float scale, int causal, int start_pos,
                    float softcap, int sliding_window, int kv_start, int kv_layout,
                    void* d_workspace);
+/* One decode step's attention straight from the stacked projection qkv[(H+2Hkv)*D] (f32): per-head
+ * RMSNorm (use_norm) and rotary embedding of q and k, k and v narrowed to f16 and appended to the
+ * caches at the row of start_pos, then causal attention of the new token over rows up to and
+ * including its own.  Same results as dh_qkv_norm_rope_kvwrite (T = 1, dst row of start_pos)
+ * followed by dh_attn_decode (kv_len = start_pos - kv_start + 1, causal), in one launch fewer;
+ * i.e. recordSplitQKVRMSNormRoPEQK with f16KVCacheWrite,
+ * src/gpu/kernels/split-qkv-rmsnorm-rope-qk.js:244-250, followed by recordAttention for
+ * seqLen == 1, src/gpu/kernels/attention.js:2007-2030.  d_cos/d_sin are the whole tables
+ * [max_seq][rotary_dim/2].  dh_attn_decode_qkv_supported tells whether a head geometry is served
+ * (head_dim 64 or 128; rotary_dim even when interleaved, else a power of two of at least
+ * head_dim/16); workspace as for dh_attn_decode. */
+int dh_attn_decode_qkv_supported(int H, int Hkv, int D, int rotary_dim, int interleaved);
+int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float* d_k_weight,
+                       const float* d_cos, const float* d_sin, void* d_cache_k, void* d_cache_v,
+                       float* d_O, int H, int Hkv, int D, int start_pos, int rotary_dim,
+                       int interleaved, float eps, int weight_offset, int use_norm, float scale,
+                       float softcap, int sliding_window, int kv_start, int kv_layout,
+                       void* d_workspace);
 
 /* ---- normalisation / rotary / KV ---- */
 

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import oracle
-from doppler_amd import ops, synth
+from doppler_amd import capi, ops, synth
 from doppler_amd.capi import DopplerHipError
 
 pytestmark = pytest.mark.gpu
@@ -603,6 +603,111 @@ def test_attention_decode_options():
     assert not got.any()
     with pytest.raises(DopplerHipError, match="kvLayout"):
         ops.runAttention(qt, kt, vt, None, H, D, kvLen=ctx, numKVHeads=Hkv, kvLayout="paged")
+
+
+# ------------------------------------------------- decode attention straight from the stacked q/k/v
+
+def _fused_case(H, Hkv, D, pos, seed, rotary=None, interleaved=False, window=0, ring=False, softcap=0.0,
+                weight_offset=False):
+    """History of `pos` cached rows, then one step at `pos` through the fused entry point; checks the
+    attention output and the appended cache row against the oracle's two separate ops."""
+    rotary = rotary or D
+    max_seq = pos + 1
+    cos, sin = synth.rope_tables(rotary, max_seq, 1e6)
+    rows = window if ring else max_seq
+    hist_k = synth.normal_f32((max_seq, Hkv, D), seed, D ** -0.5).astype(np.float16).view(np.uint16)
+    hist_v = synth.normal_f32((max_seq, Hkv, D), seed + 1, D ** -0.5).astype(np.float16).view(np.uint16)
+    ck = np.zeros((rows, Hkv, D), np.uint16)
+    cv = np.zeros((rows, Hkv, D), np.uint16)
+    for p_ in range(max(0, pos - rows), pos):
+        ck[p_ % rows], cv[p_ % rows] = hist_k[p_], hist_v[p_]
+    new_row = pos % rows
+    ck[new_row], cv[new_row] = 0x7E00, 0x7E00          # stale NaN where the new row goes: must never be used
+    qkv = synth.normal_f32((1, (H + 2 * Hkv) * D), seed + 2)
+    qw = 1 + synth.normal_f32(D, seed + 3, scale=0.1) - (1.0 if weight_offset else 0.0)
+    kw = 1 + synth.normal_f32(D, seed + 4, scale=0.1) - (1.0 if weight_offset else 0.0)
+    kbuf, vbuf = ops.tensorFromNumpy(ck), ops.tensorFromNumpy(cv)
+    kv_start = max(0, pos + 1 - rows) if ring else 0
+    out = ops.runDecodeAttentionFromQKV(ops.tensorFromNumpy(qkv), ops.tensorFromNumpy(qw), ops.tensorFromNumpy(kw),
+                                        ops.tensorFromNumpy(cos), ops.tensorFromNumpy(sin), 1e-6, kbuf.buffer,
+                                        vbuf.buffer, H, Hkv, D, pos, rotaryDim=rotary, interleaved=interleaved,
+                                        rmsNormWeightOffset=weight_offset, attnSoftcap=softcap, slidingWindow=window,
+                                        kvStart=kv_start, kvLayout="ring" if ring else "contiguous")
+    wk, wv = ck.copy(), cv.copy()
+    q = oracle.qkv_norm_rope_kvwrite(qkv, qw, kw, cos, sin, 1, H, Hkv, D, pos, wk.reshape(-1), wv.reshape(-1),
+                                     new_row * Hkv * D, rotary_dim=rotary, interleaved=interleaved,
+                                     weight_offset=weight_offset)
+    want = oracle.attention_decode_f16kv(q, wk, wv, H, Hkv, D, pos - kv_start + 1, start_pos=pos, softcap=softcap,
+                                         sliding_window=window, kv_start=kv_start, kv_layout=1 if ring else 0)
+    got_k = ops.readBuffer(kbuf.buffer, dtype=np.uint16).reshape(rows, Hkv, D)
+    got_v = ops.readBuffer(vbuf.buffer, dtype=np.uint16).reshape(rows, Hkv, D)
+    assert np.array_equal(got_v, wv)                    # V: a pure narrowing, and no other row touched
+    others = np.arange(rows) != new_row
+    assert np.array_equal(got_k[others], wk[others])
+    gk, ek = got_k[new_row].view(np.float16).astype(np.float64), wk[new_row].view(np.float16).astype(np.float64)
+    assert rel_l2(gk, ek) <= 5e-4 and np.mean(got_k[new_row] != wk[new_row]) < 0.02
+    # the oracle attends to ITS f16 key; ours may differ from it by an f16 ulp in a few elements
+    assert rel_l2(ops.readTensor(out), want) <= 2e-4, (H, Hkv, D, pos)
+
+
+@pytest.mark.parametrize("pos", [0, 1, 63, 64, 65, 575, 640, 2047, 9000])
+def test_attention_decode_from_qkv_positions(pos):
+    _fused_case(32, 8, 128, pos, seed=5300 + pos)
+
+
+@pytest.mark.parametrize("H,Hkv,D,rotary,interleaved", [(8, 8, 128, 128, False), (16, 2, 128, 64, False),
+                                                        (8, 1, 64, 64, False), (6, 2, 64, 64, True),
+                                                        (16, 8, 128, 96, True), (4, 4, 64, 16, True),
+                                                        (16, 8, 128, 32, False), (4, 4, 64, 4, False),
+                                                        (8, 1, 128, 8, False), (12, 4, 128, 6, True)])
+def test_attention_decode_from_qkv_geometries(H, Hkv, D, rotary, interleaved):
+    assert ops.decodeAttentionFromQKVSupported(H, Hkv, D, rotary, interleaved)
+    _fused_case(H, Hkv, D, 333, seed=5400 + H + rotary, rotary=rotary, interleaved=interleaved)
+
+
+def test_attention_decode_from_qkv_options():
+    _fused_case(32, 32, 128, 2500, seed=5500)                       # more chunks than splits: the owner loops
+    _fused_case(16, 8, 128, 1499, seed=5501, window=200)            # sliding window, contiguous rows
+    _fused_case(16, 8, 128, 1499, seed=5502, window=256, ring=True) # ring rows, wrapped
+    _fused_case(16, 8, 128, 100, seed=5503, window=256, ring=True)  # ring not yet full
+    _fused_case(16, 8, 128, 900, seed=5504, softcap=3.0, weight_offset=True)
+    assert not ops.decodeAttentionFromQKVSupported(16, 8, 128, 96, False)     # partners not a lane apart
+    assert not ops.decodeAttentionFromQKVSupported(16, 8, 128, 4, False)
+    assert not ops.decodeAttentionFromQKVSupported(16, 8, 256, 256, False)
+    z = ops.tensorFromNumpy(np.zeros(64, np.float32))
+    with pytest.raises(DopplerHipError, match="not served"):
+        ops.runDecodeAttentionFromQKV(ops.tensorFromNumpy(np.zeros(32 * 128, np.float32)), z, z, z, z, 1e-6,
+                                      ops.acquireBuffer(4096), ops.acquireBuffer(4096), 16, 8, 128, 0, rotaryDim=96)
+
+
+def test_attention_decode_from_qkv_matches_separate_ops_without_norm():
+    H, Hkv, D, pos = 32, 8, 128, 700
+    cos, sin = synth.rope_tables(D, pos + 1, 1e6)
+    ck = synth.normal_f32((pos + 1, Hkv, D), 5600, D ** -0.5).astype(np.float16).view(np.uint16)
+    cv = synth.normal_f32((pos + 1, Hkv, D), 5601, D ** -0.5).astype(np.float16).view(np.uint16)
+    qkv = synth.normal_f32((1, (H + 2 * Hkv) * D), 5602, D ** -0.5)
+    L = capi.load()
+    t = {k_: ops.tensorFromNumpy(v_) for k_, v_ in dict(qkv=qkv, cos=cos, sin=sin).items()}
+    outs = []
+    for fused in (False, True):
+        kb, vb = ops.tensorFromNumpy(ck), ops.tensorFromNumpy(cv)
+        if fused:
+            o = ops.runDecodeAttentionFromQKV(t["qkv"], None, None, t["cos"], t["sin"], 1e-6, kb.buffer, vb.buffer, H,
+                                              Hkv, D, pos, useNorm=False)
+        else:
+            qb = ops.acquireBuffer(H * D * 4)
+            capi.check(L.dh_qkv_norm_rope_kvwrite(t["qkv"].buffer.data_ptr(), None, None, t["cos"].buffer.data_ptr(),
+                                                  t["sin"].buffer.data_ptr(), qb.data_ptr(), kb.buffer.data_ptr(),
+                                                  vb.buffer.data_ptr(), 1, H, Hkv, D, pos, D, 0, 1e-6, 0,
+                                                  pos * Hkv * D, 0))
+            o = ops.runAttention(ops.Tensor(qb, "f32", (H, D), "q"), kb, vb, None, H, D, kvLen=pos + 1, numKVHeads=Hkv,
+                                 startPos=pos)
+        outs.append((ops.readTensor(o), ops.readBuffer(kb.buffer, dtype=np.uint16), ops.readBuffer(vb.buffer, dtype=np.uint16)))
+    assert np.array_equal(outs[0][2], outs[1][2])
+    # K: the two kernels may contract the rotation into fused multiply-adds differently
+    assert np.mean(outs[0][1] != outs[1][1]) < 1e-4
+    assert rel_l2(outs[1][1].view(np.float16).astype(np.float64), outs[0][1].view(np.float16).astype(np.float64)) <= 1e-4
+    assert rel_l2(outs[1][0], outs[0][0]) <= 1e-5
 
 
 # ----------------------------------------------------------------------------- prefill attention
