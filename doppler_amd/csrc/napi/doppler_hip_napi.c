@@ -13,7 +13,7 @@
 
 #include "doppler_hip.h"
 
-#define MAX_ARGS 20
+#define MAX_ARGS 24
 
 static napi_value fail(napi_env env, const char* msg) {
   napi_throw_error(env, NULL, msg);
@@ -178,6 +178,18 @@ FN(js_attn_decode) {
   return ret_rc(env, dh_attn_decode((const float*)Q, K, V, (float*)O, H, Hkv, D, kvLen, scale, causal, startPos, cap, win,
                                     kvStart, layout, ws));
 }
+FN(js_attn_decode_qkv_supported) {
+  ARGS(5); I(0, H); I(1, Hkv); I(2, D); I(3, rd); I(4, inter);
+  return ret_num(env, (double)dh_attn_decode_qkv_supported(H, Hkv, D, rd, inter));
+}
+FN(js_attn_decode_qkv) {
+  ARGS(23); P(0, qkv); P(1, qw); P(2, kw); P(3, c); P(4, s); P(5, ck); P(6, cv); P(7, O); I(8, H); I(9, Hkv); I(10, D);
+  I(11, start); I(12, rd); I(13, inter); F(14, eps); I(15, woff); I(16, useNorm); F(17, scale); F(18, cap); I(19, win);
+  I(20, kvStart); I(21, layout); P(22, ws);
+  return ret_rc(env, dh_attn_decode_qkv((const float*)qkv, (const float*)qw, (const float*)kw, (const float*)c,
+                                        (const float*)s, ck, cv, (float*)O, H, Hkv, D, start, rd, inter, eps, woff,
+                                        useNorm, scale, cap, win, kvStart, layout, ws));
+}
 FN(js_attn_prefill) {
   ARGS(14); P(0, Q); P(1, K); P(2, V); P(3, O); I(4, T); I(5, H); I(6, Hkv); I(7, D); I(8, kvLen); F(9, scale);
   I(10, causal); I(11, startPos); F(12, cap); I(13, win);
@@ -239,6 +251,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"q4kMatmulRmsnorm", js_q4k_matmul_rmsnorm}, {"q4kFfnGateUpRmsnorm", js_q4k_ffn_gate_up_rmsnorm},
       {"lmheadArgmaxWorkspaceBytes", js_lmhead_argmax_workspace_bytes}, {"lmheadArgmaxF16", js_lmhead_argmax_f16},
       {"attnDecodeWorkspaceBytes", js_attn_decode_workspace_bytes}, {"attnDecode", js_attn_decode},
+      {"attnDecodeQkvSupported", js_attn_decode_qkv_supported}, {"attnDecodeQkv", js_attn_decode_qkv},
       {"attnPrefill", js_attn_prefill},
       {"rmsnorm", js_rmsnorm}, {"rope", js_rope}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},
       {"kvWriteF16", js_kv_write_f16}, {"residualAdd", js_residual_add}, {"gatherF16", js_gather_f16},

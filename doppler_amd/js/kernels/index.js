@@ -4,6 +4,7 @@
 export { runMatmul, recordMatmul, runDequantQ4K } from './matmul.js';
 export { runFusedFFN, recordFusedFFN, runFusedNormedFFN, recordFusedNormedFFN } from './fused_ffn.js';
 export { runAttention, recordAttention } from './attention.js';
+export { runDecodeAttentionFromQKV, recordDecodeAttentionFromQKV, decodeAttentionFromQKVSupported } from './attention-from-qkv.js';
 export { runRMSNorm, recordRMSNorm } from './rmsnorm.js';
 export { runRoPE, recordRoPE } from './rope.js';
 export { runKVCacheWriteF32ToF16, recordKVCacheWriteF32ToF16 } from './kv-cache-write.js';

@@ -7,6 +7,7 @@ import {
   createTensor, createWeightBuffer, acquireBuffer, releaseBuffer, uploadData, readBufferSlice,
   createCommandRecorder, recordGather, recordRMSNorm, recordMatmul, recordSplitQKVRMSNormRoPEQK,
   recordAttention, recordFusedNormedFFN, recordFusedFFN, recordLmHeadArgmaxF16, recordGPUSample,
+  recordDecodeAttentionFromQKV, decodeAttentionFromQKVSupported,
 } from '../kernel-selector.js';
 
 // A window of a device buffer starting `offset` bytes in (no ownership: never released).
@@ -46,6 +47,10 @@ export class HipTextDecoder {
     this.finalNorm = createTensor(upload(weights.finalNorm), 'f32', [c.hidden], 'final_norm');
     this.cos = createTensor(upload(weights.cos), 'f32', [c.maxSeq, c.headDim / 2], 'rope_cos');
     this.sin = createTensor(upload(weights.sin), 'f32', [c.maxSeq, c.headDim / 2], 'rope_sin');
+    // decode steps: q/k norm, RoPE and the KV append run inside the attention kernel when the head
+    // geometry allows it (one launch fewer per layer)
+    this.fuseQkvAttention = config.fuseQkvAttention !== false &&
+      decodeAttentionFromQKVSupported(c.heads, c.kvHeads, c.headDim, c.headDim, false);
     this.ids = acquireBuffer(16, undefined, 'token_ids');
     this.tokenOut = acquireBuffer(16, undefined, 'sampled_token');
     this.logits = null;
@@ -150,15 +155,21 @@ export class HipTextDecoder {
       const qkv = temp(await recordMatmul(recorder, x, l.wqkv, 1, this.qSize + 2 * this.kSize, c.hidden,
         { outputDtype: 'f32', role: 'qkv_proj', layerIdx: li,
           normWeight: l.inputNorm, rmsNormEps: c.eps, useFusedRmsnormWideTile: true }));
-      const split = await recordSplitQKVRMSNormRoPEQK(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps, {
-        numTokens: 1, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim,
-        qSize: this.qSize, kSize: this.kSize, vSize: this.kSize, startPos: pos,
-        f16KVCacheWrite: { keysBuffer: l.cacheK.buffer, valuesBuffer: l.cacheV.buffer, dstOffset: pos * this.kSize },
-      });
-      temp(split.Q);
-      const attn = temp(await recordAttention(recorder, split.Q, l.cacheK, l.cacheV, null, c.heads, c.headDim, {
-        seqLen: 1, kvLen: pos + 1, numKVHeads: c.kvHeads, causal: true, startPos: pos, layerIdx: li,
-      }));
+      let attn;
+      if (this.fuseQkvAttention) {
+        attn = temp(await recordDecodeAttentionFromQKV(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps,
+          l.cacheK, l.cacheV, { numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim, startPos: pos, layerIdx: li }));
+      } else {
+        const split = await recordSplitQKVRMSNormRoPEQK(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps, {
+          numTokens: 1, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim,
+          qSize: this.qSize, kSize: this.kSize, vSize: this.kSize, startPos: pos,
+          f16KVCacheWrite: { keysBuffer: l.cacheK.buffer, valuesBuffer: l.cacheV.buffer, dstOffset: pos * this.kSize },
+        });
+        temp(split.Q);
+        attn = temp(await recordAttention(recorder, split.Q, l.cacheK, l.cacheV, null, c.heads, c.headDim, {
+          seqLen: 1, kvLen: pos + 1, numKVHeads: c.kvHeads, causal: true, startPos: pos, layerIdx: li,
+        }));
+      }
       const attnFlat = createTensor(attn.buffer, 'f32', [1, this.qSize], 'attn_flat');
       const x2 = temp(await recordMatmul(recorder, attnFlat, l.wo, 1, c.hidden, this.qSize,
         { outputDtype: 'f32', role: 'o_proj', layerIdx: li, residualTensor: x }));

@@ -105,6 +105,17 @@ async function main() {
         tensor(c.V, 'f16', [c.kvLen, c.kvHeads, c.headDim]), null, c.heads, c.headDim,
         { seqLen: 1, kvLen: c.kvLen, numKVHeads: c.kvHeads, causal: true, startPos: c.kvLen - 1 });
       await save(out, t.buffer, c.heads * c.headDim * 4);
+    } else if (c.op === 'attention_from_qkv') {
+      // cache pre-filled with history rows; the op appends the row of startPos itself
+      const keys = tensor(c.K, 'f16', [c.maxSeq, c.kvHeads, c.headDim]);
+      const values = tensor(c.V, 'f16', [c.maxSeq, c.kvHeads, c.headDim]);
+      if (!dh.decodeAttentionFromQKVSupported(c.heads, c.kvHeads, c.headDim)) throw new Error('fused decode attention should serve this geometry');
+      const t = await dh.runDecodeAttentionFromQKV(tensor(c.qkv, 'f32', [1, (c.heads + 2 * c.kvHeads) * c.headDim]),
+        tensor(c.qw, 'f32', [c.headDim]), tensor(c.kw, 'f32', [c.headDim]), tensor(c.cos, 'f32', [1]), tensor(c.sin, 'f32', [1]),
+        c.eps, keys, values, { numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim, startPos: c.startPos });
+      await save(out, t.buffer, c.heads * c.headDim * 4);
+      await save(`${c.name}.k.bin`, keys.buffer, c.maxSeq * c.kvHeads * c.headDim * 2);
+      await save(`${c.name}.v.bin`, values.buffer, c.maxSeq * c.kvHeads * c.headDim * 2);
     } else if (c.op === 'residual') {
       const t = await dh.runResidualAdd(tensor(c.a, 'f32', [c.n]), tensor(c.b, 'f32', [c.n]), c.n, { outputScale: c.outputScale });
       await save(out, t.buffer, c.n * 4);

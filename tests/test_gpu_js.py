@@ -38,7 +38,7 @@ def test_addon_is_built_and_exports_the_op_api():
               "recordRoPE", "runKVCacheWriteF32ToF16", "recordKVCacheWriteF32ToF16", "runSplitQKVRMSNormRoPEQK",
               "recordSplitQKVRMSNormRoPEQK", "runSiLU", "recordSiLU", "runSiLURowSplit", "recordSiLURowSplit", "runGeLU",
               "recordGeLU", "runResidualAdd", "recordResidualAdd", "runGather", "recordGather", "runFusedFFN",
-              "recordFusedFFN", "runArgmax", "recordArgmax", "recordLmHeadArgmax", "recordLmHeadArgmaxF16",
+              "recordFusedFFN", "runDecodeAttentionFromQKV", "recordDecodeAttentionFromQKV", "runArgmax", "recordArgmax", "recordLmHeadArgmax", "recordLmHeadArgmaxF16",
               "createTensor", "createWeightBuffer", "acquireBuffer", "releaseBuffer", "uploadData", "readBuffer",
               "createCommandRecorder", "CommandRecorder"):
         assert n in names, n
@@ -143,6 +143,21 @@ def test_js_host_path_parity(tmp_path):
     checks.append(lambda: np.array_equal(get("split.v.bin", np.uint16), wv.reshape(-1)))
     checks.append(lambda: rel_l2(get("split.k.bin", np.float16).astype(np.float32), wk.reshape(-1).view(np.float16).astype(np.float32)) <= 5e-4)
 
+    # one decode step straight from the stacked projection: norm + RoPE + KV append inside the attention kernel
+    fpos = start + T
+    hk = synth.normal_f16_bits((max_seq, Hkv, D), 9610, D ** -0.5)
+    hv = synth.normal_f16_bits((max_seq, Hkv, D), 9611, D ** -0.5)
+    fq = synth.normal_f32((1, (H + 2 * Hkv) * D), 9612)
+    cases.append(dict(name="fattn", op="attention_from_qkv", qkv=put("fattn.qkv", fq), qw="split.qw", kw="split.kw", cos="cos",
+                      sin="sin", eps=1e-6, K=put("fattn.k", hk), V=put("fattn.v", hv), heads=H, kvHeads=Hkv, headDim=D,
+                      startPos=fpos, maxSeq=max_seq))
+    fk, fv = hk.copy().reshape(max_seq, Hkv, D), hv.copy().reshape(max_seq, Hkv, D)
+    fqn = oracle.qkv_norm_rope_kvwrite(fq, qw, kw, cos, sin, 1, H, Hkv, D, fpos, fk.reshape(-1), fv.reshape(-1), fpos * Hkv * D)
+    fwant = oracle.attention_decode_f16kv(fqn, fk, fv, H, Hkv, D, fpos + 1)
+    checks.append(lambda: rel_l2(get("fattn.out.bin", np.float32), fwant) <= 2e-4)
+    checks.append(lambda: np.array_equal(get("fattn.v.bin", np.uint16), fv.reshape(-1)))
+    checks.append(lambda: rel_l2(get("fattn.k.bin", np.float16).astype(np.float32), fk.reshape(-1).view(np.float16).astype(np.float32)) <= 5e-4)
+
     kk, vv = synth.normal_f32(2048, 9700), synth.normal_f32(2048, 9701)
     cases.append(dict(name="kvw", op="kv_write", k=put("kvw.k", kk), v=put("kvw.v", vv), cacheElems=4096, srcOffset=64,
                       dstOffset=1024, count=1500))
@@ -195,6 +210,8 @@ def test_js_host_path_parity(tmp_path):
     cases.append(dict(name="decoder", op="decoder", layers=jl, embed=put("m.embed", embed), finalNorm=put("m.fn", final_norm),
                       cos=put("m.cos", mc), sin=put("m.sin", ms), prompt=prompt, steps=10,
                       config=dict(layers=2, hidden=512, inter=1024, heads=8, kvHeads=4, headDim=64, vocab=700, eps=1e-6, maxSeq=24)))
+    cases.append(dict(cases[-1], name="decoder_separate_qkv_kernel",
+                      config=dict(cases[-1]["config"], fuseQkvAttention=False)))
     ol = []
     for l in layers:
         dd = dict(l)
@@ -207,6 +224,7 @@ def test_js_host_path_parity(tmp_path):
         tok = cpu.step(prompt[pos] if pos < len(prompt) else tok, pos)
         want_tokens.append(tok)
     checks.append(lambda: [int(t) for t in get("decoder.out.bin", np.uint32)] == want_tokens)
+    checks.append(lambda: [int(t) for t in get("decoder_separate_qkv_kernel.out.bin", np.uint32)] == want_tokens)
 
     # ---- top-k temperature sampling through the JS op (seeded draw as in the reference)
     slog = (synth.rng(79).standard_normal(4000) * 3).astype(np.float32)
