@@ -130,12 +130,12 @@ def main():
     log("[bench] uploaded in %.1f s" % (time.time() - t0))
 
     # ---- KV prefill (outside the timed region): the prompt goes through the batched path, Q4_K
-    #      prefill GEMMs and matrix-core prefill attention, 512 tokens at a time
+    #      prefill GEMMs and matrix-core prefill attention, up to 2048 tokens at a time
     ids = synth.rng(40).integers(0, cfg["vocab"], max(prefill, 1))
-    dec.prefill(ids[:min(64, prefill)], chunk=512)          # warms code; rows are rewritten below
+    dec.prefill(ids[:prefill], chunk=2048)                   # warms code and buffers; rows are rewritten below
     dec.L.dh_sync()
     t0 = time.perf_counter()
-    tok = dec.prefill(ids[:prefill], chunk=512)
+    tok = dec.prefill(ids[:prefill], chunk=2048)
     dec.L.dh_sync()
     prefill_s = time.perf_counter() - t0
     log("[bench] prefill of %d positions in %.3f s (%.0f tokens/s)" % (prefill, prefill_s, prefill / prefill_s))

@@ -315,6 +315,8 @@ template <int MT> struct RingShape {
 
 #ifdef DH_GEMV_TRACE
 __device__ unsigned long long dh_trace_buf[256 * 64];
+__device__ unsigned long long dh_trace_span[64][256][16][2];     // per launch (mod 64), workgroup, wave: in, out
+unsigned dh_trace_launches = 0;
 #endif
 
 struct RingArgs {
@@ -333,6 +335,9 @@ struct RingArgs {
   const float* norm_weight;   // [K]
   float norm_eps;
   int norm_weight_offset;     // 1: scale by (1 + w)
+#ifdef DH_GEMV_TRACE
+  unsigned trace_seq;
+#endif
 };
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -490,6 +495,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
   unsigned long long* tsbuf = reinterpret_cast<unsigned long long*>(dh_trace_buf) + blockIdx.x * 64;
   int tsn = 0;
 #define DH_TS() do { if (tid == DH_GEMV_TRACE && tsn < 63) tsbuf[tsn++] = wall_clock64(); } while (0)
+  if (lane == 0) dh_trace_span[a.trace_seq & 63][blockIdx.x & 255][wave & 15][0] = wall_clock64();
 #else
 #define DH_TS() do {} while (0)
 #endif
@@ -579,7 +585,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     // in flight right behind the activation loads was measured slower, 9.3 vs 7.7 us on the
     // 6144 x 4096 product: the activation loads of the staging waves then queue behind the
     // other waves' weight loads in the memory system, and nothing can be consumed before the
-    // activations are staged.)
+    // activations are staged.  Starting the staging waves' rings after their activations have
+    // arrived but before they convert them gains nothing either: 8.7 vs 7.4 us there, 20.7 vs
+    // 20.6 us on the fused gate/up product.)
     DH_TS();
     DH_WAIT_VM(0);
     DH_TS();
@@ -746,6 +754,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
   }
 #ifdef DH_GEMV_TRACE
   if (tid == DH_GEMV_TRACE) tsbuf[63] = tsn;
+  if (lane == 0) dh_trace_span[a.trace_seq & 63][blockIdx.x & 255][wave & 15][1] = wall_clock64();
 #endif
 #undef DH_TS
 #undef DH_ISSUE_NEXT
@@ -1103,6 +1112,9 @@ int launch_ring_cfg(RingArgs a, const char* op, bool may_shorten_tiles) {
   if (fixed + dyn > kRingMaxLds) return -1;
   a.rows_per_tile = rows;
   a.depth = depth;
+#ifdef DH_GEMV_TRACE
+  a.trace_seq = dh_trace_launches++;
+#endif
   const int64_t ntiles = dh::ceil_div(a.N, rows);
   const int grid = (int)std::min<int64_t>(ntiles, ncu);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), dyn, dh::stream(), a);
@@ -1255,6 +1267,13 @@ int chain_rows(int N, int ncu) {
 }  // namespace
 
 #ifdef DH_GEMV_TRACE
+extern "C" int dh_debug_span(void* host_io, int reset) {
+  if (reset) {
+    dh_trace_launches = 0;
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(dh_trace_span), host_io, sizeof(dh_trace_span));
+  }
+  return (int)hipMemcpyFromSymbol(host_io, HIP_SYMBOL(dh_trace_span), sizeof(dh_trace_span));
+}
 extern "C" int dh_debug_trace(void* host_dst) {
   return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(dh_trace_buf), sizeof(dh_trace_buf));
 }

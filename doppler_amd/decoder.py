@@ -251,7 +251,7 @@ class HipDecoder:
         capi.check(L.dh_sample_topk(self.logits.data_ptr(), c["vocab"], float(sampling["temperature"]), k, float(r), -1, 0.0,
                                     self._sample_ws.data_ptr(), self.token.data_ptr(), out_index))
 
-    def generate(self, prompt, max_tokens, sampling=None, chunk=512):
+    def generate(self, prompt, max_tokens, sampling=None, chunk=2048):
         """prefill + decode loop; sampling = dict(temperature, topK, seed) draws token i with
         randomSeed seed + i (greedy when None)."""
         draw = (lambda i: dict(temperature=sampling["temperature"], topK=sampling["topK"], randomSeed=sampling["seed"] + i)) \
@@ -263,7 +263,7 @@ class HipDecoder:
             out.append(tok)
         return out
 
-    def prefill(self, tokens, start_pos=0, chunk=512, want_logits=False, sampling=None):
+    def prefill(self, tokens, start_pos=0, chunk=2048, want_logits=False, sampling=None):
         """Pushes a prompt through the batched path, `chunk` tokens at a time: Q4_K prefill GEMMs,
         the T-token fused QKV-norm-RoPE-KV-write, matrix-core prefill attention.  KV rows
         start_pos .. start_pos + len(tokens) - 1 are written; returns the greedy token after the

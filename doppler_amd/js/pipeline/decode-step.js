@@ -77,7 +77,7 @@ export class HipTextDecoder {
   // Mirrors the reference's prefill (src/inference/pipelines/text/generator.js) on the HIP ops.
   async prefill(tokens, startPos = 0, options = {}) {
     const c = this.config;
-    const chunk = Math.max(1, Math.min(options.chunk || 512, tokens.length));
+    const chunk = Math.max(1, Math.min(options.chunk || 2048, tokens.length));
     if (tokens.length === 0 || startPos + tokens.length > c.maxSeq) {
       throw new Error(`[prefill] ${tokens.length} tokens at ${startPos} do not fit maxSeq=${c.maxSeq}`);
     }
