@@ -26,6 +26,7 @@ namespace {
 
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(4))) float float4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;   // plain vector type: arrays of it stay in registers
 
 constexpr int BQ = 64, BKEYS = 64;
 
@@ -56,7 +57,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
   const int my_pos = a.start_pos + my_q;                      // its absolute position
   const int64_t kv_stride = (int64_t)a.Hkv * D;
 
-  // ---- Q^T fragments (B operand): b[i] = scale * Q[my_q][32 s + 8 g + i]
+  // ---- Q^T fragments (B operand): b[i] = scale * Q[my_q][32 s + 8 g + i].  Scores are kept in
+  // units of log2(e), so that the softmax needs v_exp_f32 alone (with a soft cap the factor is
+  // applied after the cap instead).
+  constexpr float kLog2e = 1.4426950408889634f;
+  const float qscale = a.softcap > 0.f ? a.scale : a.scale * kLog2e;
   half8_t qb[STEPS];
 #pragma unroll
   for (int s = 0; s < STEPS; s++) {
@@ -64,7 +69,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
     const float4 v0 = reinterpret_cast<const float4*>(qp)[0], v1 = reinterpret_cast<const float4*>(qp)[1];
     const float qv[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
-    for (int i = 0; i < 8; i++) qb[s][i] = (_Float16)(qv[i] * a.scale);
+    for (int i = 0; i < 8; i++) qb[s][i] = (_Float16)(qv[i] * qscale);
   }
 
   // ---- key range of this query tile
@@ -81,15 +86,21 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
   for (int t = 0; t < DT; t++) acc[t] = {0.f, 0.f, 0.f, 0.f};
   float m_run = -FLT_MAX, l_run = 0.f;
 
-  uint4 kreg[PIECES], vreg[PIECES];
-  // piece p = tid + 256 r of a tile: key p / (D/8), 8 consecutive dims starting at 8 (p % (D/8))
+  u32x4_t kreg[PIECES], vreg[PIECES];
+  // K piece p = tid + 256 r of a tile: key p / (D/8), 8 consecutive dims starting at 8 (p % (D/8)).
+  // V is fetched by key PAIRS, so that the transposed tile can be written in 32-bit words: item j
+  // of a thread is keys 2 (tid % 32), 2 (tid % 32) + 1 and dims 8 c .. 8 c + 7, c = tid / 32 + 8 j
+  // (vreg[2 j + s] holds key s of the pair).  The 32 pairs of a half wave land in 32 different
+  // LDS banks.
+  const int vpair = tid & 31, vcol = tid >> 5;
 #define DH_PF_LOAD(tile_)                                                                        \
   _Pragma("unroll") for (int r = 0; r < PIECES; r++) {                                           \
     const int p_ = tid + 256 * r, key_ = p_ / (D / 8), c_ = p_ % (D / 8);                        \
     const int row_ = min(kbeg + (tile_) * BKEYS + key_, a.kv_len - 1);                           \
-    const int64_t off_ = (int64_t)row_ * kv_stride + (int64_t)kvh * D + 8 * c_;                  \
-    kreg[r] = *reinterpret_cast<const uint4*>(a.K + off_);                                       \
-    vreg[r] = *reinterpret_cast<const uint4*>(a.V + off_);                                       \
+    kreg[r] = *reinterpret_cast<const u32x4_t*>(a.K + (int64_t)row_ * kv_stride + (int64_t)kvh * D + 8 * c_); \
+    const int vrow_ = min(kbeg + (tile_) * BKEYS + 2 * vpair + (r & 1), a.kv_len - 1);           \
+    vreg[r] = *reinterpret_cast<const u32x4_t*>(a.V + (int64_t)vrow_ * kv_stride + (int64_t)kvh * D + \
+                                              8 * (vcol + 8 * (r >> 1)));                        \
   }
   if (ntiles > 0) { DH_PF_LOAD(0); }
 
@@ -98,22 +109,23 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
 #pragma unroll
     for (int r = 0; r < PIECES; r++) {
       const int p = tid + 256 * r, key = p / (D / 8), c = p % (D / 8);
-      *reinterpret_cast<uint4*>(&k_lds[key * KROW + 8 * c]) = kreg[r];
-      // V^T with the keys in k-slot order: key = 32 kb + 16 jj + 4 gg + ii -> slot 32 kb + 8 gg + 4 jj + ii
-      const int kb = key >> 5, jj = (key >> 4) & 1, gg = (key >> 2) & 3, ii = key & 3;
-      const int slot = 32 * kb + 8 * gg + 4 * jj + ii;
-      // the 16 lanes that hold one key write different dims in the same step (lane c starts at
-      // dim c): their LDS rows would otherwise all fall into one bank
-      const uint32_t vw[4] = {vreg[r].x, vreg[r].y, vreg[r].z, vreg[r].w};
+      *reinterpret_cast<u32x4_t*>(&k_lds[key * KROW + 8 * c]) = kreg[r];
+    }
+    // V^T with the keys in k-slot order: key = 32 kb + 16 jj + 4 gg + ii -> slot 32 kb + 8 gg + 4 jj + ii;
+    // the two keys of a pair are neighbours there, one 32-bit word per dim
+    {
+      const int key0 = 2 * vpair;
+      const int slot = 32 * (key0 >> 5) + 8 * ((key0 >> 2) & 3) + 4 * ((key0 >> 4) & 1) + (key0 & 3);
 #pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const int ee = (e + c) & 7;
-        uint32_t w = vw[0];
-        w = (ee >> 1) == 1 ? vw[1] : w;
-        w = (ee >> 1) == 2 ? vw[2] : w;
-        w = (ee >> 1) == 3 ? vw[3] : w;
-        const uint16_t hbits = (uint16_t)((ee & 1) ? (w >> 16) : (w & 0xFFFFu));
-        reinterpret_cast<uint16_t*>(v_lds)[(8 * c + ee) * VROW + slot] = hbits;
+      for (int j = 0; j < PIECES / 2; j++) {
+        const int c = vcol + 8 * j;
+        const u32x4_t aw = vreg[2 * j];
+        const u32x4_t bw = vreg[2 * j + 1];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const uint32_t word = __builtin_amdgcn_perm(bw[e >> 1], aw[e >> 1], (e & 1) ? 0x07060302u : 0x05040100u);
+          reinterpret_cast<uint32_t*>(v_lds)[((8 * c + e) * VROW + slot) >> 1] = word;
+        }
       }
     }
     __syncthreads();
@@ -131,33 +143,44 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
         st[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[s], st[j], 0, 0, 0);
       }
     }
-    // ---- mask, soft cap, online softmax (this lane: query my_q, keys kbase + 16 j + 4 g + i)
+    // ---- mask, soft cap, online softmax (this lane: query my_q, keys kbase + 16 j + 4 g + i).
+    // A tile that every query of this wave sees completely needs no per-element masks.
+    const int wave_lo = a.start_pos + q0 + 16 * wave, wave_hi = wave_lo + 15;
+    const bool full = kbase + BKEYS <= a.kv_len && (!a.causal || kbase + BKEYS - 1 <= wave_lo) &&
+                      (a.window <= 0 || kbase > wave_hi - a.window);
     float mx = -FLT_MAX;
+    if (full && !(a.softcap > 0.f)) {
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+      for (int j = 0; j < 4; j++)
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int key = kbase + 16 * j + 4 * g + i;
-        float s = st[j][i];
-        if (a.softcap > 0.f) s = tanhf(s / a.softcap) * a.softcap;
-        bool ok = key < a.kv_len;
-        if (a.causal) ok = ok && key <= my_pos;
-        if (a.window > 0) ok = ok && key > my_pos - a.window;
-        s = ok ? s : -INFINITY;
-        st[j][i] = s;
-        mx = fmaxf(mx, s);
-      }
+        for (int i = 0; i < 4; i++) mx = fmaxf(mx, st[j][i]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int key = kbase + 16 * j + 4 * g + i;
+          float s = st[j][i];
+          if (a.softcap > 0.f) s = tanhf(s / a.softcap) * (a.softcap * kLog2e);
+          bool ok = key < a.kv_len;
+          if (a.causal) ok = ok && key <= my_pos;
+          if (a.window > 0) ok = ok && key > my_pos - a.window;
+          s = ok ? s : -INFINITY;
+          st[j][i] = s;
+          mx = fmaxf(mx, s);
+        }
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx);              // finite: m_run starts at -FLT_MAX
-    const float alpha = __expf(m_run - m_new);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float ps = 0.f;
     half8_t pb[2];
 #pragma unroll
     for (int j = 0; j < 4; j++)
 #pragma unroll
       for (int i = 0; i < 4; i++) {
-        const float p = __expf(st[j][i] - m_new);      // exp(-inf) = 0 for masked keys
+        const float p = __builtin_amdgcn_exp2f(st[j][i] - m_new);   // 2^-inf = 0 for masked keys
         ps += p;
         pb[j >> 1][4 * (j & 1) + i] = (_Float16)p;
       }
@@ -165,10 +188,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
     ps += __shfl_xor(ps, 32, 64);
     l_run = l_run * alpha + ps;
     m_run = m_new;
+    const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;   // no new maximum: nothing to scale
     // ---- O^T = alpha O^T + V^T P^T
 #pragma unroll
     for (int t = 0; t < DT; t++) {
-      acc[t] *= alpha;
+      if (rescale) acc[t] *= alpha;
 #pragma unroll
       for (int kb = 0; kb < 2; kb++) {
         const half8_t va = *reinterpret_cast<const half8_t*>(&v_lds[(16 * t + q) * VROW + 32 * kb + 8 * g]);
