@@ -8,7 +8,7 @@
 //            as f16: (w & 0x000F000F) | 0x64006400 is the pair (1024 + q) in f16, one packed
 //            subtract and one packed fma with (d*sc, -dmin*mn) finish them: about 2 vector ops
 //            per weight, paid once per 128 rows of A.
-//   A        packed once per product by a pre-pass (pack_a_kernel): each row scaled by the power
+//   A        packed once per product by a pre-pass (pack_a_row_kernel / pack_a_kernel): each row scaled by the power
 //            of two that puts its largest element at 2^14, rounded to f16, k-permuted, rows
 //            zero-padded to a multiple of 64.  The GEMM tiles then copy 16-byte pieces into
 //            LDS, no conversion in the K loop (every column tile used to redo it), and the
@@ -109,6 +109,55 @@ __global__ __launch_bounds__(256) void pack_a_kernel(const float* __restrict__ A
     const half2_t p0 = {(_Float16)(v[0] * mul), (_Float16)(v[2] * mul)};
     const half2_t p1 = {(_Float16)(v[1] * mul), (_Float16)(v[3] * mul)};
     *reinterpret_cast<uint2*>(dst + k) = make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+  }
+}
+
+// The same packing with one workgroup per row and the row held in registers (NV float4 per
+// thread, K <= 1024 NV): every load of a row is in flight at once and the row is read once.  One
+// wave per row walks its row in dependent steps and is latency-bound (14.5 us for 512 x 6912).
+template <int NV>
+__global__ __launch_bounds__(256) void pack_a_row_kernel(const float* __restrict__ A, int M, int K, int kpad,
+                                                         _Float16* __restrict__ Apk, float2* __restrict__ out_scale) {
+  __shared__ float wave_max[4];
+  const int tid = threadIdx.x, m = blockIdx.x;
+  const float* row = A + (int64_t)m * K;
+  const bool vec = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+  float v[NV][4];
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int k = 4 * tid + 1024 * i;
+    if (vec && k + 3 < K) {
+      const float4 t = *reinterpret_cast<const float4*>(row + k);
+      v[i][0] = t.x; v[i][1] = t.y; v[i][2] = t.z; v[i][3] = t.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[i][j] = k + j < K ? row[k + j] : 0.f;
+    }
+  }
+  float mx = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) mx = fmaxf(mx, fabsf(v[i][j]));
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+  if ((tid & 63) == 0) wave_max[tid >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+  int e = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;
+  e = max(-100, min(100, e));
+  if (!(mx > 0.f) || !(mx < INFINITY)) e = 14;
+  const float mul = __uint_as_float((uint32_t)(127 + 14 - e) << 23);
+  if (tid == 0) out_scale[m] = make_float2(mul, __uint_as_float((uint32_t)(127 - 14 + e) << 23));
+  _Float16* dst = Apk + (int64_t)m * kpad;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int k = 4 * tid + 1024 * i;
+    if (k < kpad) {
+      const half2_t p0 = {(_Float16)(v[i][0] * mul), (_Float16)(v[i][2] * mul)};
+      const half2_t p1 = {(_Float16)(v[i][1] * mul), (_Float16)(v[i][3] * mul)};
+      *reinterpret_cast<uint2*>(dst + k) = make_uint2(__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1));
+    }
   }
 }
 
@@ -400,7 +449,16 @@ int launch_gemm(GemmArgs a, const char* op) {
     }
     return 0;
   }
-  hipLaunchKernelGGL(pack_a_kernel, dim3((unsigned)dh::ceil_div(a.M, 4)), dim3(256), 0, dh::stream(), a.A, a.M, a.K,
+  if (a.K <= 2048)
+    hipLaunchKernelGGL(pack_a_row_kernel<2>, dim3((unsigned)a.M), dim3(256), 0, dh::stream(), a.A, a.M, a.K, a.kpad, packed, scales);
+  else if (a.K <= 4096)
+    hipLaunchKernelGGL(pack_a_row_kernel<4>, dim3((unsigned)a.M), dim3(256), 0, dh::stream(), a.A, a.M, a.K, a.kpad, packed, scales);
+  else if (a.K <= 8192)
+    hipLaunchKernelGGL(pack_a_row_kernel<8>, dim3((unsigned)a.M), dim3(256), 0, dh::stream(), a.A, a.M, a.K, a.kpad, packed, scales);
+  else if (a.K <= 16384)
+    hipLaunchKernelGGL(pack_a_row_kernel<16>, dim3((unsigned)a.M), dim3(256), 0, dh::stream(), a.A, a.M, a.K, a.kpad, packed, scales);
+  else
+    hipLaunchKernelGGL(pack_a_kernel, dim3((unsigned)dh::ceil_div(a.M, 4)), dim3(256), 0, dh::stream(), a.A, a.M, a.K,
                      a.kpad, packed, scales);
   DH_CHECK_LAUNCH(op);
   a.row_scale = scales;
