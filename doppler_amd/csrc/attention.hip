@@ -16,6 +16,7 @@
 // the cache and uses them straight from registers.  That removes the split-QKV/norm/RoPE/
 // KV-write kernel (one launch, ~4.5 us per layer) from the decode step.
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 #include <cfloat>
 
@@ -451,6 +452,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
 // Every load the kernel needs for the first 32 splits (a thread's 32 partial outputs, and one
 // (m, l) pair per thread) is issued before anything is waited for, so the kernel costs one memory
 // round trip, not one per dependent phase; splits beyond 32 follow in a pipelined loop.
+// (Preloading 64 made short contexts slower, 8.9 vs 8.1 us at 512 keys.)
 template <int D>
 __global__ __launch_bounds__(D) void attn_decode_merge_kernel(const float* __restrict__ ws,
                                                               float* __restrict__ O, int nsplit) {
@@ -505,10 +507,18 @@ __global__ void zero_f32_kernel(float* p, int n) {
 
 int max_splits_for(int kv_len) { return std::max(1, (kv_len + kTileKeys - 1) / kTileKeys); }
 
+// Splits of the key range per kv head.  Fewer, longer workgroups beat more splits once every CU
+// has one: a workgroup's next chunk costs well under 1 us, every extra split costs the merge
+// kernel and the dispatch more (measured, 32/8 heads, four workgroups per CU against one:
+// 3000 keys 12.9 vs 10.4 us, 6000 keys 17.1 vs 12.6, 16384 keys 24.4 vs 20.4, 32768 keys 37.1 vs
+// 33.4).  One workgroup per CU, two once that would mean more than 16 chunks each.
 int choose_splits(int Hkv, int nkeys) {
   const int tiles = std::max(1, (nkeys + kTileKeys - 1) / kTileKeys);
-  const int want = std::max(1, 1024 / std::max(1, Hkv));   // at most ~4 workgroups per CU
-  return std::min(tiles, want);
+  static const double env_per_cu = getenv("DH_ATTN_WG_PER_CU") ? atof(getenv("DH_ATTN_WG_PER_CU")) : 0.0;
+  const int one_per_cu = std::max(1, dh::num_cus() / std::max(1, Hkv));
+  if (env_per_cu > 0.0) return std::min(tiles, std::max(1, (int)(one_per_cu * env_per_cu)));
+  if (tiles <= 16 * one_per_cu) return std::min(tiles, one_per_cu);
+  return std::min(tiles, 2 * one_per_cu);
 }
 
 template <int D, bool QKV>
