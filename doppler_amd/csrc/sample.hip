@@ -7,8 +7,9 @@
 // for the widest exchanges): round 0 sorts slices of the vocabulary and keeps the best k of
 // each, later rounds sort 1024 surviving candidates at a time, until one workgroup holds them
 // all; that workgroup also draws the token.  k <= 256, so a round shrinks the field at least
-// four-fold.  A round costs ~25 us whatever its grid: the 55 dependent exchange steps of the
-// network set its length (3 rounds at k = 40 over 151,936 logits, 5 at k = 256).
+// four-fold.  A round costs ~16 us whatever its grid: the 55 dependent exchange steps of the
+// network set its length (3 rounds at k = 40 over 151,936 logits, 5 at k = 256); as a rolled
+// loop with run-time distances it cost 25.
 #include <algorithm>
 #include <cfloat>
 
@@ -39,14 +40,24 @@ __device__ __forceinline__ bool ranks_before(float av, uint32_t ai, float bv, ui
   return av > bv || (av == bv && ai < bi);
 }
 
+// Value of lane (l ^ dist).  The network below is fully unrolled, so dist is a constant where this
+// is called: partners inside a quad and 8 lanes apart come through the DPP path of the vector ALU
+// (quad_perm, row_ror:8), the rest through the LDS crossbar.
+__device__ __forceinline__ uint32_t lane_xor(uint32_t x, int dist) {
+  if (dist == 1) return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0xB1, 0xF, 0xF, false);
+  if (dist == 2) return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x4E, 0xF, 0xF, false);
+  if (dist == 8) return (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, 0x128, 0xF, 0xF, false);
+  return (uint32_t)__shfl_xor((int)x, dist, 64);
+}
+
 // Sorts 1024 (value, id) pairs best first, four per thread: element i = 4 * tid + r.  A bitonic
 // network; exchanges at distance 1 and 2 stay inside a thread's registers, distances 4..128 are
 // lane shuffles inside a wave, only the three steps at distance 256 and 512 go through LDS and
 // a barrier.
 __device__ __forceinline__ void sort1024(float (&v)[4], uint32_t (&id)[4], float* s_val, uint32_t* s_idx, int tid) {
-#pragma unroll 1
+#pragma unroll
   for (int k = 2; k <= kSortN; k <<= 1) {
-#pragma unroll 1
+#pragma unroll
     for (int j = k >> 1; j > 0; j >>= 1) {
       if (j >= 4) {
         float pv[4];
@@ -61,8 +72,8 @@ __device__ __forceinline__ void sort1024(float (&v)[4], uint32_t (&id)[4], float
         } else {
 #pragma unroll
           for (int r = 0; r < 4; r++) {
-            pv[r] = __shfl_xor(v[r], j >> 2, 64);
-            pi[r] = (uint32_t)__shfl_xor((int)id[r], j >> 2, 64);
+            pv[r] = __uint_as_float(lane_xor(__float_as_uint(v[r]), j >> 2));
+            pi[r] = lane_xor(id[r], j >> 2);
           }
         }
 #pragma unroll
