@@ -519,8 +519,12 @@ int choose_splits(int Hkv, int nkeys) {
   static const double env_per_cu = getenv("DH_ATTN_WG_PER_CU") ? atof(getenv("DH_ATTN_WG_PER_CU")) : 0.0;
   const int one_per_cu = std::max(1, dh::num_cus() / std::max(1, Hkv));
   if (env_per_cu > 0.0) return std::min(tiles, std::max(1, (int)(one_per_cu * env_per_cu)));
-  if (tiles <= 16 * one_per_cu) return std::min(tiles, one_per_cu);
-  return std::min(tiles, 2 * one_per_cu);
+  const int wgs = tiles <= 16 * one_per_cu ? one_per_cu : 2 * one_per_cu;
+  if (tiles <= wgs) return tiles;
+  // every workgroup the same number of chunks (the slowest one sets the time), in as few splits
+  // as that allows (the merge kernel pays per split)
+  const int chunks_each = (tiles + wgs - 1) / wgs;
+  return (tiles + chunks_each - 1) / chunks_each;
 }
 
 template <int D, bool QKV>
