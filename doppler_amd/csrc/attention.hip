@@ -108,8 +108,10 @@ __device__ __forceinline__ float row_group_sum(float v) {
 //            kh, kh+KH, ... in registers and accumulates them for all heads; the key groups
 //            meet in a wave-private LDS buffer at the end.
 // K and V of the next chunk are requested before the current one is consumed.
-// (Keeping two chunks in flight instead of one changed nothing, 34.1 vs 33.3 us at 32768 keys: a
-// workgroup's ~2 us per chunk is its own barrier-and-LDS latency, not the wait for memory.)
+// (Keeping two chunks in flight instead of one changed nothing, 34.1 vs 33.3 us at 32768 keys, and
+// neither did 128-key chunks, 33.5 us: a workgroup's ~2 us per 64 keys is its own softmax and
+// P.V arithmetic plus LDS round trips with one wave per SIMD, not the wait for memory or the
+// barriers.)
 // GT: query heads per kv head rounded up to 1, 2, 4 or 8 (bounds the unrolled per-head code).
 // QKV: the step's q, k, v arrive raw (see the top of the file); the appended key is the last
 // visible one, so the lanes that would read its row, or a clamped copy of it, from the not yet
