@@ -42,10 +42,14 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // Matrix-core GEMM for prefill-sized batches (q4k_gemm.hip).  `serves`: M >= 16, K a multiple
 // of 4, A 16-byte aligned.
 bool q4k_gemm_serves(int M, int K, const void* A);
+// norm_weight != null: every row of A goes through RMSNorm (weights norm_weight, or 1 + them) on its
+// way into the packed operand.
 int q4k_gemm(const char* op, const float* A, const uint8_t* W, void* C, int c_f16, int M, int N, int K,
-             float alpha, const float* residual);
+             float alpha, const float* residual, const float* norm_weight = nullptr, float norm_eps = 0.f,
+             int norm_weight_offset = 0);
 int q4k_gemm_gate_up(const char* op, const float* A, const uint8_t* Wg, const uint8_t* Wu, float* C, int M,
-                     int hidden, int inter, int activation, float alpha, float clamp_max);
+                     int hidden, int inter, int activation, float alpha, float clamp_max,
+                     const float* norm_weight = nullptr, float norm_eps = 0.f, int norm_weight_offset = 0);
 
 }  // namespace dh
 

@@ -67,6 +67,10 @@ struct GemmArgs {
   int ksplit, kt_per_split;
   float* partial;
   const float2* row_scale;   // [M] (multiplier applied before the f16 rounding, its inverse)
+  // RMSNorm prologue (norm_weight null = off): rows are normalised while they are packed
+  const float* norm_weight;  // [K]
+  float norm_eps;
+  int norm_weight_offset;    // 1: scale by (1 + w)
 };
 
 // Packs the activations for the matrix cores, one wave per row (four rows per workgroup):
@@ -117,8 +121,11 @@ __global__ __launch_bounds__(256) void pack_a_kernel(const float* __restrict__ A
 // wave per row walks its row in dependent steps and is latency-bound (14.5 us for 512 x 6912).
 template <int NV>
 __global__ __launch_bounds__(256) void pack_a_row_kernel(const float* __restrict__ A, int M, int K, int kpad,
-                                                         _Float16* __restrict__ Apk, float2* __restrict__ out_scale) {
+                                                         _Float16* __restrict__ Apk, float2* __restrict__ out_scale,
+                                                         const float* __restrict__ norm_w, float norm_eps,
+                                                         int norm_w_offset) {
   __shared__ float wave_max[4];
+  __shared__ float wave_ss[4];
   const int tid = threadIdx.x, m = blockIdx.x;
   const float* row = A + (int64_t)m * K;
   const bool vec = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0;
@@ -133,6 +140,36 @@ __global__ __launch_bounds__(256) void pack_a_row_kernel(const float* __restrict
 #pragma unroll
       for (int j = 0; j < 4; j++) v[i][j] = k + j < K ? row[k + j] : 0.f;
     }
+  }
+  if (norm_w) {
+    // RMSNorm of the row, same arithmetic as the stand-alone kernel: x * rsqrt(mean x^2 + eps) * w
+    float wn[NV][4];
+    const bool wvec = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(norm_w) & 15) == 0;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int k = 4 * tid + 1024 * i;
+      if (wvec && k + 3 < K) {
+        const float4 t = *reinterpret_cast<const float4*>(norm_w + k);
+        wn[i][0] = t.x; wn[i][1] = t.y; wn[i][2] = t.z; wn[i][3] = t.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) wn[i][j] = k + j < K ? norm_w[k + j] : 0.f;
+      }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) ss = fmaf(v[i][j], v[i][j], ss);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    if ((tid & 63) == 0) wave_ss[tid >> 6] = ss;
+    __syncthreads();
+    const float inv = 1.0f / sqrtf((wave_ss[0] + wave_ss[1] + wave_ss[2] + wave_ss[3]) / (float)K + norm_eps);
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) v[i][j] = v[i][j] * inv * (norm_w_offset ? 1.0f + wn[i][j] : wn[i][j]);
   }
   float mx = 0.f;
 #pragma unroll
@@ -449,17 +486,19 @@ int launch_gemm(GemmArgs a, const char* op) {
     }
     return 0;
   }
-  if (a.K <= 2048)
-    hipLaunchKernelGGL(pack_a_row_kernel<2>, dim3((unsigned)a.M), dim3(256), 0, dh::stream(), a.A, a.M, a.K, a.kpad, packed, scales);
-  else if (a.K <= 4096)
-    hipLaunchKernelGGL(pack_a_row_kernel<4>, dim3((unsigned)a.M), dim3(256), 0, dh::stream(), a.A, a.M, a.K, a.kpad, packed, scales);
-  else if (a.K <= 8192)
-    hipLaunchKernelGGL(pack_a_row_kernel<8>, dim3((unsigned)a.M), dim3(256), 0, dh::stream(), a.A, a.M, a.K, a.kpad, packed, scales);
-  else if (a.K <= 16384)
-    hipLaunchKernelGGL(pack_a_row_kernel<16>, dim3((unsigned)a.M), dim3(256), 0, dh::stream(), a.A, a.M, a.K, a.kpad, packed, scales);
+#define DH_PACK_ROWS(NV_)                                                                          \
+  hipLaunchKernelGGL(pack_a_row_kernel<NV_>, dim3((unsigned)a.M), dim3(256), 0, dh::stream(), a.A, a.M, a.K, \
+                     a.kpad, packed, scales, a.norm_weight, a.norm_eps, a.norm_weight_offset)
+  if (a.K <= 2048) DH_PACK_ROWS(2);
+  else if (a.K <= 4096) DH_PACK_ROWS(4);
+  else if (a.K <= 8192) DH_PACK_ROWS(8);
+  else if (a.K <= 16384) DH_PACK_ROWS(16);
+  else if (a.norm_weight)
+    return dh::fail(1, "[%s] the RMSNorm prologue serves K <= 16384 at M >= 16 (K=%d)", op, a.K);
   else
     hipLaunchKernelGGL(pack_a_kernel, dim3((unsigned)dh::ceil_div(a.M, 4)), dim3(256), 0, dh::stream(), a.A, a.M, a.K,
-                     a.kpad, packed, scales);
+                       a.kpad, packed, scales);
+#undef DH_PACK_ROWS
   DH_CHECK_LAUNCH(op);
   a.row_scale = scales;
   a.Apk = packed;
@@ -504,20 +543,23 @@ bool q4k_gemm_serves(int M, int K, const void* A) {
 }
 
 int q4k_gemm(const char* op, const float* A, const uint8_t* W, void* C, int c_f16, int M, int N, int K,
-             float alpha, const float* residual) {
+             float alpha, const float* residual, const float* norm_weight, float norm_eps, int norm_weight_offset) {
   GemmArgs a{};
   a.A = A; a.W = W; a.W2 = nullptr; a.C = C; a.residual = residual;
   a.M = M; a.N = N; a.K = K; a.nb = (K + kQK - 1) / kQK;
   a.alpha = alpha; a.c_f16 = c_f16;
+  a.norm_weight = norm_weight; a.norm_eps = norm_eps; a.norm_weight_offset = norm_weight_offset;
   return launch_gemm<false>(a, op);
 }
 
 int q4k_gemm_gate_up(const char* op, const float* A, const uint8_t* Wg, const uint8_t* Wu, float* C, int M,
-                     int hidden, int inter, int activation, float alpha, float clamp_max) {
+                     int hidden, int inter, int activation, float alpha, float clamp_max,
+                     const float* norm_weight, float norm_eps, int norm_weight_offset) {
   GemmArgs a{};
   a.A = A; a.W = Wg; a.W2 = Wu; a.C = C; a.residual = nullptr;
   a.M = M; a.N = inter; a.K = hidden; a.nb = (hidden + kQK - 1) / kQK;
   a.alpha = alpha; a.c_f16 = 0; a.activation = activation; a.clamp_max = clamp_max;
+  a.norm_weight = norm_weight; a.norm_eps = norm_eps; a.norm_weight_offset = norm_weight_offset;
   return launch_gemm<true>(a, op);
 }
 

@@ -1334,11 +1334,12 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
     const int rc = dispatch_ring<false>(g, op);
     if (rc >= 0) return rc;
   }
-  if (normed)
-    return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 and K <= 14336 only (M=%d, K=%d); "
-                    "run dh_rmsnorm and dh_q4k_matmul instead", op, M, K);
   if (path != 2 && dh::q4k_gemm_serves(M, K, d_A))
-    return dh::q4k_gemm(op, a.A, a.W, d_C, a.c_f16, M, N, K, alpha, a.residual);
+    return dh::q4k_gemm(op, a.A, a.W, d_C, a.c_f16, M, N, K, alpha, a.residual, normed ? d_norm_weight : nullptr, eps,
+                        weight_offset);
+  if (normed)
+    return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 with K <= 14336 and M >= 16 (M=%d, K=%d); "
+                    "run dh_rmsnorm and dh_q4k_matmul instead", op, M, K);
   // tiles of up to 8 activation rows per pass over the weights
   const size_t c_elem = a.c_f16 ? 2 : 4;
   for (int m0 = 0; m0 < M; m0 += 8) {
@@ -1403,11 +1404,12 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
     const int rc = dispatch_ring<true>(g, op);
     if (rc >= 0) return rc;
   }
-  if (normed)
-    return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 and hidden <= 14336 only (M=%d, hidden=%d); "
-                    "run dh_rmsnorm and dh_q4k_ffn_gate_up instead", op, M, hidden);
   if (path != 2 && dh::q4k_gemm_serves(M, hidden, d_x))
-    return dh::q4k_gemm_gate_up(op, d_x, a.W, a.W2, d_out, M, hidden, inter, activation, alpha, swiglu_limit);
+    return dh::q4k_gemm_gate_up(op, d_x, a.W, a.W2, d_out, M, hidden, inter, activation, alpha, swiglu_limit,
+                                normed ? d_norm_weight : nullptr, eps, weight_offset);
+  if (normed)
+    return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 with hidden <= 14336 and M >= 16 (M=%d, hidden=%d); "
+                    "run dh_rmsnorm and dh_q4k_ffn_gate_up instead", op, M, hidden);
   // any batch: tiles of up to 8 activation rows per pass
   for (int m0 = 0; m0 < M; m0 += 8) {
     GemvArgs b = a;

@@ -289,10 +289,18 @@ class HipDecoder:
             ck(L.dh_gather_f16(b["ids"].data_ptr(), self.embed.data_ptr(), b["x"].data_ptr(), T, Hd, c["vocab"], 0))
             x, x2 = b["x"], b["x2"]
             for d in self.layers:
-                ck(L.dh_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), capi.F32, b["normed"].data_ptr(), T, Hd,
-                                c["eps"], 0, None, None, None, 1.0))
-                ck(L.dh_q4k_matmul(b["normed"].data_ptr(), capi.F32, d["wqkv"].data_ptr(), b["qkv"].data_ptr(), capi.F32,
-                                   T, qkv_n, Hd, 1.0, None))
+                # chunks of 1..8 or 16+ tokens: the input RMSNorm runs inside the product (GEMV prologue,
+                # or the GEMM's activation packing); 9..15 tokens take the separate norm kernel
+                fused_norm = self.fuse_norm and (T <= 8 or T >= 16)
+                if fused_norm:
+                    ck(L.dh_q4k_matmul_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), c["eps"], 0,
+                                               d["wqkv"].data_ptr(), b["qkv"].data_ptr(), capi.F32, T, qkv_n, Hd, 1.0,
+                                               None))
+                else:
+                    ck(L.dh_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), capi.F32, b["normed"].data_ptr(), T, Hd,
+                                    c["eps"], 0, None, None, None, 1.0))
+                    ck(L.dh_q4k_matmul(b["normed"].data_ptr(), capi.F32, d["wqkv"].data_ptr(), b["qkv"].data_ptr(),
+                                       capi.F32, T, qkv_n, Hd, 1.0, None))
                 ck(L.dh_qkv_norm_rope_kvwrite(b["qkv"].data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
                                               self.cos.data_ptr(), self.sin.data_ptr(), b["q"].data_ptr(),
                                               d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), T, H, Hkv, D, pos, D, 0,
@@ -306,10 +314,15 @@ class HipDecoder:
                                          b["attn"].data_ptr(), T, H, Hkv, D, pos + T, self.scale, 1, pos, 0.0, 0))
                 ck(L.dh_q4k_matmul(b["attn"].data_ptr(), capi.F32, d["wo"].data_ptr(), x2.data_ptr(), capi.F32, T, Hd,
                                    self.qs, 1.0, x.data_ptr()))
-                ck(L.dh_rmsnorm(x2.data_ptr(), d["post_attn_norm"].data_ptr(), capi.F32, b["normed"].data_ptr(), T, Hd,
-                                c["eps"], 0, None, None, None, 1.0))
-                ck(L.dh_q4k_ffn_gate_up(b["normed"].data_ptr(), d["wgate"].data_ptr(), d["wup"].data_ptr(),
-                                        b["act"].data_ptr(), T, Hd, I, capi.ACT_SILU, 1.0, 0.0))
+                if fused_norm:
+                    ck(L.dh_q4k_ffn_gate_up_rmsnorm(x2.data_ptr(), d["post_attn_norm"].data_ptr(), c["eps"], 0,
+                                                    d["wgate"].data_ptr(), d["wup"].data_ptr(), b["act"].data_ptr(), T,
+                                                    Hd, I, capi.ACT_SILU, 1.0, 0.0))
+                else:
+                    ck(L.dh_rmsnorm(x2.data_ptr(), d["post_attn_norm"].data_ptr(), capi.F32, b["normed"].data_ptr(), T,
+                                    Hd, c["eps"], 0, None, None, None, 1.0))
+                    ck(L.dh_q4k_ffn_gate_up(b["normed"].data_ptr(), d["wgate"].data_ptr(), d["wup"].data_ptr(),
+                                            b["act"].data_ptr(), T, Hd, I, capi.ACT_SILU, 1.0, 0.0))
                 ck(L.dh_q4k_matmul(b["act"].data_ptr(), capi.F32, d["wdown"].data_ptr(), x.data_ptr(), capi.F32, T, Hd, I,
                                    1.0, x2.data_ptr()))
         # logits of the last prompt token only

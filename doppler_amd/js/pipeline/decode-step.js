@@ -95,9 +95,19 @@ export class HipTextDecoder {
       x = temp(await recordGather(recorder, ids, this.embed, T, c.hidden, c.vocab, { embeddingDtype: 'f16', outputDtype: 'f32' }));
       for (let li = 0; li < this.layers.length; li++) {
         const l = this.layers[li];
-        const normed = temp(await recordRMSNorm(recorder, x, l.inputNorm, c.eps, { batchSize: T, hiddenSize: c.hidden }));
-        const qkv = temp(await recordMatmul(recorder, normed, l.wqkv, T, this.qSize + 2 * this.kSize, c.hidden,
-          { outputDtype: 'f32', role: 'qkv_proj', layerIdx: li }));
+        // chunks of 1..8 or 16+ tokens: the input RMSNorm runs inside the product (GEMV prologue, or the
+        // GEMM's activation packing); 9..15 tokens take the separate norm kernel
+        const fusedNorm = T <= 8 || T >= 16;
+        let qkv;
+        if (fusedNorm) {
+          qkv = temp(await recordMatmul(recorder, x, l.wqkv, T, this.qSize + 2 * this.kSize, c.hidden,
+            { outputDtype: 'f32', role: 'qkv_proj', layerIdx: li,
+              normWeight: l.inputNorm, rmsNormEps: c.eps, useFusedRmsnormWideTile: true }));
+        } else {
+          const normed = temp(await recordRMSNorm(recorder, x, l.inputNorm, c.eps, { batchSize: T, hiddenSize: c.hidden }));
+          qkv = temp(await recordMatmul(recorder, normed, l.wqkv, T, this.qSize + 2 * this.kSize, c.hidden,
+            { outputDtype: 'f32', role: 'qkv_proj', layerIdx: li }));
+        }
         const split = await recordSplitQKVRMSNormRoPEQK(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps, {
           numTokens: T, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim,
           qSize: this.qSize, kSize: this.kSize, vSize: this.kSize, startPos: pos,
@@ -110,9 +120,15 @@ export class HipTextDecoder {
         const attnFlat = createTensor(attn.buffer, 'f32', [T, this.qSize], 'attn_flat');
         const x2 = temp(await recordMatmul(recorder, attnFlat, l.wo, T, c.hidden, this.qSize,
           { outputDtype: 'f32', role: 'o_proj', layerIdx: li, residualTensor: x }));
-        const normed2 = temp(await recordRMSNorm(recorder, x2, l.postAttnNorm, c.eps, { batchSize: T, hiddenSize: c.hidden }));
-        const act = temp(await recordFusedFFN(recorder, normed2, l.wgate, l.wup, c.hidden, c.inter,
-          { batchSize: T, activation: 'silu' }));
+        let act;
+        if (fusedNorm) {
+          act = temp(await recordFusedNormedFFN(recorder, x2, l.postAttnNorm, c.eps, l.wgate, l.wup, c.hidden, c.inter,
+            { batchSize: T, activation: 'silu' }));
+        } else {
+          const normed2 = temp(await recordRMSNorm(recorder, x2, l.postAttnNorm, c.eps, { batchSize: T, hiddenSize: c.hidden }));
+          act = temp(await recordFusedFFN(recorder, normed2, l.wgate, l.wup, c.hidden, c.inter,
+            { batchSize: T, activation: 'silu' }));
+        }
         x = temp(await recordMatmul(recorder, act, l.wdown, T, c.hidden, c.inter,
           { outputDtype: 'f32', role: 'down_proj', layerIdx: li, residualTensor: x2 }));
       }

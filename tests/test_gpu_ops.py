@@ -244,7 +244,7 @@ def test_fused_ffn_random_shape_sweep():
         hidden = int(g.choice([256, 640, 1024, 1152, 2048, 4096, 4352]))
         inter = int(g.choice([64, 100, 257, 1000, 1536]))
         act = str(g.choice(["silu", "gelu"]))
-        normed = M <= 8 and g.random() < 0.5
+        normed = (M <= 8 or M >= 16) and g.random() < 0.5
         Wg, wg = q4k_weight(inter, hidden, seed=2601 + 3 * t)
         Wu, wu = q4k_weight(inter, hidden, seed=2602 + 3 * t)
         X = synth.normal_f32((M, hidden), seed=2603 + 3 * t, scale=0.05)
@@ -293,13 +293,30 @@ def test_fused_normed_ffn_q4k(M, activation):
     assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
 
 
-def test_rmsnorm_prologue_fails_closed_for_large_batches():
+def test_rmsnorm_prologue_fails_closed_between_gemv_and_gemm_batches():
     W, wb = q4k_weight(64, 256, seed=2300)
     A = ops.tensorFromNumpy(synth.normal_f32((9, 256), seed=2301))
     nw = ops.tensorFromNumpy(np.ones(256, np.float32))
     with pytest.raises(DopplerHipError, match="RMSNorm prologue"):
         ops.runMatmul(A, wb, 9, 64, 256, outputDtype="f32", normWeight=nw, rmsNormEps=1e-6,
                       useFusedRmsnormWideTile=True)
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 300, 1024), (40, 512, 1152), (512, 1024, 4096), (130, 200, 12288), (33, 96, 640)])
+def test_matmul_rmsnorm_prologue_on_the_gemm_path(M, N, K):
+    """M >= 16: the rows are normalised while the GEMM's activations are packed."""
+    W, wb = q4k_weight(N, K, seed=2310 + M)
+    X = synth.normal_f32((M, K), seed=2311 + M, scale=3.0)
+    nw = 1.0 + synth.normal_f32((K,), seed=2312 + M, scale=0.1)
+    res = synth.normal_f32((M, N), seed=2313 + M)
+    out = ops.runMatmul(ops.tensorFromNumpy(X), wb, M, N, K, outputDtype="f32", normWeight=ops.tensorFromNumpy(nw),
+                        rmsNormEps=1e-6, useFusedRmsnormWideTile=True, residualTensor=ops.tensorFromNumpy(res))
+    want = oracle.q4k_matmul(oracle.rmsnorm(X, nw, 1e-6), W, M, N, K) + res
+    assert rel_l2(ops.readTensor(out), want) <= matmul_bar(M)
+    # weights given as offsets from one, as Gemma-style checkpoints store them
+    out = ops.runMatmul(ops.tensorFromNumpy(X), wb, M, N, K, outputDtype="f32", normWeight=ops.tensorFromNumpy(nw - 1.0),
+                        rmsNormEps=1e-6, useFusedRmsnormWideTile=True, rmsNormOffset=True)
+    assert rel_l2(ops.readTensor(out), want - res) <= matmul_bar(M)
 
 
 @pytest.mark.parametrize("hidden,inter,qkv_rows", [(4096, 12288, 6144), (1024, 3072, 2048), (640, 1500, 700)])
