@@ -1325,21 +1325,28 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
   a.alpha = alpha;
   a.c_f16 = c_dtype == DH_F16;
   const int path = gemv_path();
-  if ((path == 0 || normed) && M <= 8) {
-    RingArgs g{};
-    g.A = a.A; g.W = a.W; g.W2 = nullptr; g.C = d_C; g.residual = a.residual;
-    g.M = M; g.N = N; g.K = K; g.nb = a.nb; g.alpha = alpha; g.c_f16 = a.c_f16;
-    g.norm_weight = normed ? d_norm_weight : nullptr;
-    g.norm_eps = eps; g.norm_weight_offset = weight_offset;
-    const int rc = dispatch_ring<false>(g, op);
+  if ((path == 0 || normed) && M < 16) {
+    // below the GEMM's batch size: passes of up to 8 rows through the streaming GEMV
+    int rc = 0;
+    for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
+      RingArgs g{};
+      g.A = a.A + (int64_t)m0 * K; g.W = a.W; g.W2 = nullptr;
+      g.C = static_cast<char*>(d_C) + (int64_t)m0 * N * (a.c_f16 ? 2 : 4);
+      g.residual = a.residual ? a.residual + (int64_t)m0 * N : nullptr;
+      g.M = std::min(8, M - m0); g.N = N; g.K = K; g.nb = a.nb; g.alpha = alpha; g.c_f16 = a.c_f16;
+      g.norm_weight = normed ? d_norm_weight : nullptr;
+      g.norm_eps = eps; g.norm_weight_offset = weight_offset;
+      rc = dispatch_ring<false>(g, op);
+      if (rc < 0 && m0 > 0) return dh::fail(2, "[%s] internal: GEMV pass %d did not fit after pass 0 did", op, m0 / 8);
+    }
     if (rc >= 0) return rc;
   }
   if (path != 2 && dh::q4k_gemm_serves(M, K, d_A))
     return dh::q4k_gemm(op, a.A, a.W, d_C, a.c_f16, M, N, K, alpha, a.residual, normed ? d_norm_weight : nullptr, eps,
                         weight_offset);
   if (normed)
-    return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 with K <= 14336 and M >= 16 (M=%d, K=%d); "
-                    "run dh_rmsnorm and dh_q4k_matmul instead", op, M, K);
+    return dh::fail(1, "[%s] the RMSNorm prologue serves K <= 14336 below 16 rows and K <= 16384 from 16 rows on "
+                    "(M=%d, K=%d); run dh_rmsnorm and dh_q4k_matmul instead", op, M, K);
   // tiles of up to 8 activation rows per pass over the weights
   const size_t c_elem = a.c_f16 ? 2 : 4;
   for (int m0 = 0; m0 < M; m0 += 8) {
@@ -1394,22 +1401,26 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
   a.activation = activation;
   a.clamp_max = swiglu_limit;
   const int path = gemv_path();
-  if ((path == 0 || normed) && M <= 8) {
-    RingArgs g{};
-    g.A = d_x; g.W = a.W; g.W2 = a.W2; g.C = d_out; g.residual = nullptr;
-    g.M = M; g.N = inter; g.K = hidden; g.nb = a.nb; g.alpha = alpha; g.c_f16 = 0;
-    g.activation = activation; g.clamp_max = swiglu_limit;
-    g.norm_weight = normed ? d_norm_weight : nullptr;
-    g.norm_eps = eps; g.norm_weight_offset = weight_offset;
-    const int rc = dispatch_ring<true>(g, op);
+  if ((path == 0 || normed) && M < 16) {
+    int rc = 0;
+    for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
+      RingArgs g{};
+      g.A = d_x + (int64_t)m0 * hidden; g.W = a.W; g.W2 = a.W2; g.C = d_out + (int64_t)m0 * inter; g.residual = nullptr;
+      g.M = std::min(8, M - m0); g.N = inter; g.K = hidden; g.nb = a.nb; g.alpha = alpha; g.c_f16 = 0;
+      g.activation = activation; g.clamp_max = swiglu_limit;
+      g.norm_weight = normed ? d_norm_weight : nullptr;
+      g.norm_eps = eps; g.norm_weight_offset = weight_offset;
+      rc = dispatch_ring<true>(g, op);
+      if (rc < 0 && m0 > 0) return dh::fail(2, "[%s] internal: GEMV pass %d did not fit after pass 0 did", op, m0 / 8);
+    }
     if (rc >= 0) return rc;
   }
   if (path != 2 && dh::q4k_gemm_serves(M, hidden, d_x))
     return dh::q4k_gemm_gate_up(op, d_x, a.W, a.W2, d_out, M, hidden, inter, activation, alpha, swiglu_limit,
                                 normed ? d_norm_weight : nullptr, eps, weight_offset);
   if (normed)
-    return dh::fail(1, "[%s] the RMSNorm prologue serves M <= 8 with hidden <= 14336 and M >= 16 (M=%d, hidden=%d); "
-                    "run dh_rmsnorm and dh_q4k_ffn_gate_up instead", op, M, hidden);
+    return dh::fail(1, "[%s] the RMSNorm prologue serves hidden <= 14336 below 16 rows and hidden <= 16384 from 16 "
+                    "rows on (M=%d, hidden=%d); run dh_rmsnorm and dh_q4k_ffn_gate_up instead", op, M, hidden);
   // any batch: tiles of up to 8 activation rows per pass
   for (int m0 = 0; m0 < M; m0 += 8) {
     GemvArgs b = a;

@@ -289,9 +289,9 @@ class HipDecoder:
             ck(L.dh_gather_f16(b["ids"].data_ptr(), self.embed.data_ptr(), b["x"].data_ptr(), T, Hd, c["vocab"], 0))
             x, x2 = b["x"], b["x2"]
             for d in self.layers:
-                # chunks of 1..8 or 16+ tokens: the input RMSNorm runs inside the product (GEMV prologue,
-                # or the GEMM's activation packing); 9..15 tokens take the separate norm kernel
-                fused_norm = self.fuse_norm and (T <= 8 or T >= 16)
+                # the input RMSNorm runs inside the product (GEMV prologue below 16 tokens, the GEMM's
+                # activation packing from 16 on)
+                fused_norm = self.fuse_norm
                 if fused_norm:
                     ck(L.dh_q4k_matmul_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), c["eps"], 0,
                                                d["wqkv"].data_ptr(), b["qkv"].data_ptr(), capi.F32, T, qkv_n, Hd, 1.0,

@@ -95,9 +95,9 @@ export class HipTextDecoder {
       x = temp(await recordGather(recorder, ids, this.embed, T, c.hidden, c.vocab, { embeddingDtype: 'f16', outputDtype: 'f32' }));
       for (let li = 0; li < this.layers.length; li++) {
         const l = this.layers[li];
-        // chunks of 1..8 or 16+ tokens: the input RMSNorm runs inside the product (GEMV prologue, or the
-        // GEMM's activation packing); 9..15 tokens take the separate norm kernel
-        const fusedNorm = T <= 8 || T >= 16;
+        // the input RMSNorm runs inside the product (GEMV prologue below 16 tokens, the GEMM's activation
+        // packing from 16 on) unless the model asks for separate norm launches
+        const fusedNorm = c.fuseNorm !== false;
         let qkv;
         if (fusedNorm) {
           qkv = temp(await recordMatmul(recorder, x, l.wqkv, T, this.qSize + 2 * this.kSize, c.hidden,

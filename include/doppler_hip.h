@@ -87,9 +87,9 @@ int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int 
  * standalone norm dispatch in front of the q/k/v and gate/up projections disappears.
  * Replaces runMatmul with `normWeight` + `useFusedRmsnormWideTile`,
  * src/gpu/kernels/matmul-selection.js:609-620 (fused_rmsnorm_q4_widetile.wgsl:4-24,189-215).
- * d_norm_weight is f32 [K].  Served for M <= 8 (in the GEMV's prologue) and M >= 16 (while the
- * GEMM's activations are packed, K <= 16384); other shapes fail with a message (run
- * dh_rmsnorm + dh_q4k_matmul). */
+ * d_norm_weight is f32 [K].  Below 16 rows the norm runs in the GEMV's prologue (K <= 14336), from
+ * 16 rows on while the GEMM's activations are packed (K <= 16384); longer rows fail with a message
+ * (run dh_rmsnorm + dh_q4k_matmul). */
 int dh_q4k_matmul_rmsnorm(const float* d_A, const float* d_norm_weight, float eps,
                           int weight_offset, const void* d_W, void* d_C, int c_dtype, int M,
                           int N, int K, float alpha, const void* d_residual);
@@ -131,7 +131,8 @@ int dh_q4k_gemv_chain(const dh_gemv_phase* phases, int count);
 
 /* dh_q4k_ffn_gate_up over RMSNorm(x): the reference's "fused normed FFN",
  * src/gpu/kernels/fused_ffn.js:705-745,773-860 (there the inverse RMS comes in as a buffer,
- * here it is computed in the prologue).  d_norm_weight is f32 [hidden].  M <= 8 or M >= 16. */
+ * here it is computed in the prologue).  d_norm_weight is f32 [hidden]; limits as for
+ * dh_q4k_matmul_rmsnorm. */
 int dh_q4k_ffn_gate_up_rmsnorm(const float* d_x, const float* d_norm_weight, float eps,
                                int weight_offset, const void* d_Wgate, const void* d_Wup,
                                float* d_out, int M, int hidden, int inter, int activation,

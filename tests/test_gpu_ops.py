@@ -244,7 +244,7 @@ def test_fused_ffn_random_shape_sweep():
         hidden = int(g.choice([256, 640, 1024, 1152, 2048, 4096, 4352]))
         inter = int(g.choice([64, 100, 257, 1000, 1536]))
         act = str(g.choice(["silu", "gelu"]))
-        normed = (M <= 8 or M >= 16) and g.random() < 0.5
+        normed = g.random() < 0.5
         Wg, wg = q4k_weight(inter, hidden, seed=2601 + 3 * t)
         Wu, wu = q4k_weight(inter, hidden, seed=2602 + 3 * t)
         X = synth.normal_f32((M, hidden), seed=2603 + 3 * t, scale=0.05)
@@ -293,13 +293,29 @@ def test_fused_normed_ffn_q4k(M, activation):
     assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
 
 
-def test_rmsnorm_prologue_fails_closed_between_gemv_and_gemm_batches():
-    W, wb = q4k_weight(64, 256, seed=2300)
-    A = ops.tensorFromNumpy(synth.normal_f32((9, 256), seed=2301))
-    nw = ops.tensorFromNumpy(np.ones(256, np.float32))
+def test_rmsnorm_prologue_fails_closed_for_rows_too_long_for_the_gemv():
+    K = 20480                                   # fragments of one row no longer fit beside the weight ring
+    W, wb = q4k_weight(32, K, seed=2300)
+    A = ops.tensorFromNumpy(synth.normal_f32((2, K), seed=2301))
+    nw = ops.tensorFromNumpy(np.ones(K, np.float32))
     with pytest.raises(DopplerHipError, match="RMSNorm prologue"):
-        ops.runMatmul(A, wb, 9, 64, 256, outputDtype="f32", normWeight=nw, rmsNormEps=1e-6,
+        ops.runMatmul(A, wb, 2, 32, K, outputDtype="f32", normWeight=nw, rmsNormEps=1e-6,
                       useFusedRmsnormWideTile=True)
+
+
+@pytest.mark.parametrize("M", [9, 12, 15])
+def test_rmsnorm_prologue_between_gemv_and_gemm_batches(M):
+    """9..15 rows: two passes of the streaming GEMV."""
+    N, K = 200, 1024
+    W, wb = q4k_weight(N, K, seed=2305 + M)
+    X = synth.normal_f32((M, K), seed=2306 + M, scale=2.0)
+    nw = 1.0 + synth.normal_f32((K,), seed=2307 + M, scale=0.1)
+    res = synth.normal_f32((M, N), seed=2308 + M)
+    out = ops.runMatmul(ops.tensorFromNumpy(X), wb, M, N, K, outputDtype="f32", normWeight=ops.tensorFromNumpy(nw),
+                        rmsNormEps=1e-6, useFusedRmsnormWideTile=True, residualTensor=ops.tensorFromNumpy(res))
+    assert rel_l2(ops.readTensor(out), oracle.q4k_matmul(oracle.rmsnorm(X, nw, 1e-6), W, M, N, K) + res) <= REL_L2_F32
+    out = ops.runMatmul(ops.tensorFromNumpy(X), wb, M, N, K, outputDtype="f32")
+    assert rel_l2(ops.readTensor(out), oracle.q4k_matmul(X, W, M, N, K)) <= REL_L2_F32
 
 
 @pytest.mark.parametrize("M,N,K", [(16, 300, 1024), (40, 512, 1152), (512, 1024, 4096), (130, 200, 12288), (33, 96, 640)])
