@@ -591,7 +591,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     // ring stage first (a counter in LDS, per-unit partial sums added in super-block order by
     // the wave that completes a tile): waves of a workgroup end up to 5 us apart under fixed
     // ownership, but the workgroup as a whole is limited by what the memory system delivers,
-    // 17.2 vs 17.7 us for gate/up and 13.8 vs 13.0 us for the down projection, no change per step.)
+    // 17.2 vs 17.7 us for gate/up and 13.8 vs 13.0 us for the down projection, no change per step.
+    // Nor letting the staging waves only stage and the other half own the whole weight stream:
+    // 8.4 vs 7.5 us on the 6144 x 4096 product.)
     DH_TS();
     DH_WAIT_VM(0);
     DH_TS();
