@@ -143,6 +143,34 @@ def test_batched_decode_matches_step_by_step():
         b.decode_batch(1, 0, 65)
 
 
+def test_long_context_decode_fused_and_separate_attention_agree():
+    """4,500 cached positions: a kv head has more 64-key chunks than workgroups, so workgroups walk
+    several chunks and the one that appends the new key meets it late in its walk.  The decoder
+    with the q/k-norm + RoPE + KV append inside the attention kernel must give the tokens, logits
+    and cache rows of the one that runs them as a separate kernel."""
+    cfg = dict(layers=2, hidden=512, inter=1024, heads=16, kv_heads=2, head_dim=64, vocab=900, eps=1e-6, qk_norm=1,
+               max_seq=4608, theta=1e6)
+    layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=41, max_seq=cfg["max_seq"])
+    prompt = synth.rng(42).integers(0, cfg["vocab"], 4500)
+    runs = []
+    for fused in (True, False):
+        d = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, cfg["max_seq"], fuse_qkv_attention=fused)
+        assert d.fuse_qkv_attention == fused
+        tok = d.prefill(prompt)
+        toks, logits = [tok], []
+        for i in range(6):
+            tok = d.step(tok, len(prompt) + i, want_logits=True)
+            toks.append(tok)
+            logits.append(d.read_logits())
+        runs.append((toks, logits, d.read_kv(1, len(prompt) + 6)))
+    assert runs[0][0] == runs[1][0]
+    for la, lb in zip(runs[0][1], runs[1][1]):
+        assert rel_l2(la, lb) <= 1e-4
+    for x, y in zip(runs[0][2], runs[1][2]):
+        assert np.mean(x != y) < 1e-3                  # f16 cache rows: the odd last-bit difference in K
+        assert rel_l2(x.view(np.float16).astype(np.float64), y.view(np.float16).astype(np.float64)) <= 1e-3
+
+
 @pytest.mark.timeout(1500)
 def test_9b_class_greedy_64_steps_identical_tokens():
     """BASELINE config 4: 36 layers, hidden 4096, FFN 12288, 32/8 heads of 128, vocab 151936,
