@@ -23,6 +23,9 @@
 // dequantisation runs under the matrix-core work instead of in front of it; with all waves doing
 // both in turn (one barrier per step keeps them in phase) the two never overlap.  Where two or
 // more four-wave workgroups share a compute unit they overlap each other and that is faster.
+// A 256 (M) x 128 (N) tile with the same split (two A tiles against one weight tile, half the
+// dequantisation per output) was measured too: 368 against 326 us at M = 2048, N = 12288,
+// K = 4096; one workgroup of it per compute unit loses to two 128 x 128 workgroups.
 // k order inside every group of 4 is (0, 2, 1, 3) in BOTH tiles: that is the order the masked
 // nibble pairs come out in, and a contraction index may be permuted freely when both operands
 // agree.
