@@ -57,13 +57,33 @@ extern "C" {
 
 const char* dh_last_error(void) { return g_err; }
 
-int dh_init(int device_ordinal) {
-  std::lock_guard<std::mutex> lock(g_mu);
-  if (g_ready) {
-    if (device_ordinal != g_device)
-      return dh::fail(1, "[dh_init] already initialised on device %d", g_device);
-    return 0;
-  }
+// Frees whatever dh_init has allocated so far and returns the runtime to its unset state; the
+// first failing call is the one reported.
+static int release_all(const char* op) {
+  hipError_t first = hipSuccess;
+  auto note = [&](hipError_t e) {
+    if (first == hipSuccess) first = e;
+  };
+  if (g_own_stream) note(hipStreamDestroy(g_own_stream));
+  if (g_chain_mem) note(hipFree(g_chain_mem));
+  if (g_splitk_ws) note(hipFree(g_splitk_ws));
+  if (g_row_scale) note(hipFree(g_row_scale));
+  if (g_packed_a) note(hipFree(g_packed_a));
+  g_own_stream = nullptr;
+  g_stream = nullptr;
+  g_chain_mem = nullptr;
+  g_splitk_ws = nullptr;
+  g_row_scale = nullptr;
+  g_packed_a = nullptr;
+  g_chain_value = 0;
+  g_num_cus = 0;
+  g_ready = false;
+  g_device = -1;
+  if (first != hipSuccess) return dh::fail(2, "[%s] releasing the runtime failed: %s", op, hipGetErrorString(first));
+  return 0;
+}
+
+static int init_locked(int device_ordinal) {
   int count = 0;
   DH_CHECK_HIP("dh_init", hipGetDeviceCount(&count));
   if (device_ordinal < 0 || device_ordinal >= count)
@@ -88,24 +108,29 @@ int dh_init(int device_ordinal) {
   return 0;
 }
 
+int dh_init(int device_ordinal) {
+  std::lock_guard<std::mutex> lock(g_mu);
+  if (g_ready) {
+    if (device_ordinal != g_device)
+      return dh::fail(1, "[dh_init] already initialised on device %d", g_device);
+    return 0;
+  }
+  const int rc = init_locked(device_ordinal);
+  if (rc != 0) {
+    // keep the message of the step that failed; a second attempt starts from nothing
+    char msg[sizeof(g_err)];
+    memcpy(msg, g_err, sizeof(msg));
+    release_all("dh_init");
+    memcpy(g_err, msg, sizeof(msg));
+  }
+  return rc;
+}
+
 int dh_shutdown(void) {
   std::lock_guard<std::mutex> lock(g_mu);
   if (!g_ready) return 0;
   DH_CHECK_HIP("dh_shutdown", hipStreamSynchronize(g_stream));
-  if (g_own_stream) DH_CHECK_HIP("dh_shutdown", hipStreamDestroy(g_own_stream));
-  if (g_chain_mem) DH_CHECK_HIP("dh_shutdown", hipFree(g_chain_mem));
-  g_chain_mem = nullptr;
-  if (g_splitk_ws) DH_CHECK_HIP("dh_shutdown", hipFree(g_splitk_ws));
-  g_splitk_ws = nullptr;
-  if (g_row_scale) DH_CHECK_HIP("dh_shutdown", hipFree(g_row_scale));
-  g_row_scale = nullptr;
-  if (g_packed_a) DH_CHECK_HIP("dh_shutdown", hipFree(g_packed_a));
-  g_packed_a = nullptr;
-  g_own_stream = nullptr;
-  g_stream = nullptr;
-  g_ready = false;
-  g_device = -1;
-  return 0;
+  return release_all("dh_shutdown");
 }
 
 int dh_set_stream(void* hip_stream) {

@@ -1,31 +1,40 @@
 // Q4_K prefill GEMM for gfx950: C[M,N] = alpha * A[M,K] . dequant(W)[N,K]^T for M >= 16, and
 // the fused gate/up projection with gated activation, on the matrix cores.
 //
-// Tile: 128 (M) x 128 (N) per workgroup of 4 waves, each wave a 64 x 64 quadrant computed with
-// v_mfma_f32_32x32x16_f16 (2 x 2 MFMA tiles, f32 accumulators).  K advances 64 at a time: one
-// 32-byte nibble chunk of a super-block (low nibbles = sub-block 2c, high = 2c+1) per weight row.
-//   weights  thread (row, half) loads 16 nibble bytes + the block header, rebuilds 32 weights
-//            as f16: (w & 0x000F000F) | 0x64006400 is the pair (1024 + q) in f16, one packed
-//            subtract and one packed fma with (d*sc, -dmin*mn) finish them: about 2 vector ops
-//            per weight, paid once per 128 rows of A.
-//   A        packed once per product by a pre-pass (pack_a_row_kernel / pack_a_kernel): each row scaled by the power
-//            of two that puts its largest element at 2^14, rounded to f16, k-permuted, rows
-//            zero-padded to a multiple of 64.  The GEMM tiles then copy 16-byte pieces into
-//            LDS, no conversion in the K loop (every column tile used to redo it), and the
-//            epilogue divides the row factor out again, exactly: activations beyond the f16
-//            range (65504) neither overflow nor lose small rows to subnormals.
+// Tiles: a wave computes a 64 x 64 (or 32 x 32) quadrant with v_mfma_f32_32x32x16_f16 (f32
+// accumulators), four waves a 128 x 128 (64 x 64) tile, and a workgroup is one or two such groups
+// stacked along M against the same weight tile: 256 x 128 with eight waves for large problems.
+// K advances 64 at a time: one 32-byte nibble chunk of a super-block (low nibbles = sub-block
+// 2c, high = 2c+1) per weight row.
+//   weights  a thread loads 8 or 16 nibble bytes of a row + the block header and rebuilds the
+//            weights as f16: (w & 0x000F000F) | 0x64006400 is the pair (1024 + q) in f16, one
+//            packed subtract and one packed fma with (d*sc, -dmin*mn) finish them: about 2
+//            vector ops per weight, paid once per workgroup tile (hence the tall tiles).
+//   A        packed once per product by a pre-pass (pack_a_row_kernel / pack_a_kernel): each
+//            row scaled by the power of two that puts its largest element at 2^14, rounded to
+//            f16, k-permuted, rows zero-padded to a multiple of 64.  The GEMM tiles then copy
+//            16-byte pieces into LDS, no conversion in the K loop, and the epilogue divides the
+//            row factor out again, exactly: activations beyond the f16 range (65504) neither
+//            overflow nor lose small rows to subnormals.
 // Both tiles sit in LDS as [row][64 k] with a 16-byte pad (conflict-free 16-byte fragment
 // reads) and are double-buffered, one barrier per K step.
-// SPEC (used where only one workgroup fits a compute unit, the fused gate/up tile): the
-// workgroup has eight waves, waves 0..3 only multiply (fragment reads + matrix-core
-// instructions), waves 4..7 only produce (global loads two tiles ahead, dequantise, write the
-// next LDS buffer).  Each SIMD then holds one wave of either kind, so the vector ALU work of the
-// dequantisation runs under the matrix-core work instead of in front of it; with all waves doing
-// both in turn (one barrier per step keeps them in phase) the two never overlap.  Where two or
-// more four-wave workgroups share a compute unit they overlap each other and that is faster.
-// A 256 (M) x 128 (N) tile with the same split (two A tiles against one weight tile, half the
-// dequantisation per output) was measured too: 368 against 326 us at M = 2048, N = 12288,
-// K = 4096; one workgroup of it per compute unit loses to two 128 x 128 workgroups.
+// The K loop is bound by instruction issue, not by memory (with every load served from the
+// first-level cache it runs 3 % faster) and not by the matrix cores alone (they are busy for
+// half of the loop's cycles at the 1.84 GHz the part holds under this load).  Measured on this
+// part: a wave issues an independent vector instruction every 5 cycles and a dependent one every
+// 8, a matrix-core instruction occupies its pipe for 32, and a wave may issue 4 vector
+// instructions behind a matrix-core instruction at no cost.  Hence:
+//   * every wave both multiplies and produces, and the producer's work of a step (LDS stores of
+//     the A tile, scale unpack, nibble dwords, the loads two tiles ahead) is dealt out in pieces
+//     behind the matrix-core instructions of the same step, in program order pinned with
+//     scheduling barriers;
+//   * fragments are double-buffered in registers, so LDS latency runs under the previous slice;
+//   * all global loads are unconditional: one conditional load makes the compiler wait for every
+//     outstanding load before a tile is used, which halves the lookahead.
+// Tried and measured slower: producer / multiplier wave specialisation (four waves each: the
+// producers' 250 vector instructions per step at one wave per SIMD took longer than the
+// multipliers' step, 1.3 us per K step against 1.0 us for eight symmetric waves on the same
+// 256 x 128 x 2 problem), two A sub-tiles per wave (one wave per SIMD), 256 x 64 blocks.
 // k order inside every group of 4 is (0, 2, 1, 3) in BOTH tiles: that is the order the masked
 // nibble pairs come out in, and a contraction index may be permuted freely when both operands
 // agree.
@@ -201,30 +210,37 @@ __global__ __launch_bounds__(256) void pack_a_row_kernel(const float* __restrict
   }
 }
 
-// 16 nibble bytes -> 16 low-nibble and 16 high-nibble weights as f16, k order (0,2,1,3) per dword.
-__device__ __forceinline__ void dequant16(const uint4 q, float sc_lo, float mn_lo, float sc_hi, float mn_hi,
-                                          uint4 (&lo)[2], uint4 (&hi)[2]) {
-  const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+// Dequantisation in pieces, for the K loop that spreads it between the matrix-core
+// instructions.  Scales of sub-blocks 2c, 2c+1 as broadcastable f16 pairs, without a branch on c:
+struct PairScales {
+  half2_t slo, mlo, shi, mhi;     // (scale, scale), (-min, -min) of the low- and high-nibble sub-block
+};
+__device__ __forceinline__ PairScales pair_scales_f16(const u32x4_t hdr, const int c) {
+  const float d = f16lo(hdr[0]), dmin = f16hi(hdr[0]);
+  const int sh = (c & 1) * 16;
+  const uint32_t a1 = hdr[1] >> sh, a2 = hdr[2] >> sh, a3 = hdr[3] >> sh;
+  const bool low = c < 2;
+  const uint32_t scp = low ? (a1 & 0x3F3Fu) : ((a3 & 0x0F0Fu) | ((a1 >> 2) & 0x3030u));
+  const uint32_t mnp = low ? (a2 & 0x3F3Fu) : (((a3 >> 4) & 0x0F0Fu) | ((a2 >> 2) & 0x3030u));
+  const _Float16 sl = (_Float16)(d * (float)(scp & 0xFFu)), sh_ = (_Float16)(d * (float)((scp >> 8) & 0xFFu));
+  const _Float16 ml = (_Float16)(-dmin * (float)(mnp & 0xFFu)), mh = (_Float16)(-dmin * (float)((mnp >> 8) & 0xFFu));
+  PairScales r;
+  r.slo = half2_t{sl, sl}; r.mlo = half2_t{ml, ml};
+  r.shi = half2_t{sh_, sh_}; r.mhi = half2_t{mh, mh};
+  return r;
+}
+// One dword of nibbles (8 weights) -> two low-nibble and two high-nibble f16 pairs.
+__device__ __forceinline__ void dequant_dword(const uint32_t w, const PairScales& ps, uint32_t& lo0, uint32_t& lo1,
+                                              uint32_t& hi0, uint32_t& hi1) {
   const half2_t k1024 = {(_Float16)1024.f, (_Float16)1024.f};
-  const half2_t slo = {(_Float16)sc_lo, (_Float16)sc_lo}, mlo = {(_Float16)-mn_lo, (_Float16)-mn_lo};
-  const half2_t shi = {(_Float16)sc_hi, (_Float16)sc_hi}, mhi = {(_Float16)-mn_hi, (_Float16)-mn_hi};
-  uint32_t lo_w[8], hi_w[8];
-#pragma unroll
-  for (int d = 0; d < 4; d++) {
-    const uint32_t p[4] = {(w[d] & 0x000F000Fu) | 0x64006400u, ((w[d] >> 8) & 0x000F000Fu) | 0x64006400u,
-                           ((w[d] >> 4) & 0x000F000Fu) | 0x64006400u, ((w[d] >> 12) & 0x000F000Fu) | 0x64006400u};
-    half2_t v[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) v[i] = __builtin_bit_cast(half2_t, p[i]) - k1024;     // exact: q
-    lo_w[2 * d] = __builtin_bit_cast(uint32_t, v[0] * slo + mlo);
-    lo_w[2 * d + 1] = __builtin_bit_cast(uint32_t, v[1] * slo + mlo);
-    hi_w[2 * d] = __builtin_bit_cast(uint32_t, v[2] * shi + mhi);
-    hi_w[2 * d + 1] = __builtin_bit_cast(uint32_t, v[3] * shi + mhi);
-  }
-  lo[0] = make_uint4(lo_w[0], lo_w[1], lo_w[2], lo_w[3]);
-  lo[1] = make_uint4(lo_w[4], lo_w[5], lo_w[6], lo_w[7]);
-  hi[0] = make_uint4(hi_w[0], hi_w[1], hi_w[2], hi_w[3]);
-  hi[1] = make_uint4(hi_w[4], hi_w[5], hi_w[6], hi_w[7]);
+  const half2_t v0 = __builtin_bit_cast(half2_t, (w & 0x000F000Fu) | 0x64006400u) - k1024;
+  const half2_t v1 = __builtin_bit_cast(half2_t, ((w >> 8) & 0x000F000Fu) | 0x64006400u) - k1024;
+  const half2_t v2 = __builtin_bit_cast(half2_t, ((w >> 4) & 0x000F000Fu) | 0x64006400u) - k1024;
+  const half2_t v3 = __builtin_bit_cast(half2_t, ((w >> 12) & 0x000F000Fu) | 0x64006400u) - k1024;
+  lo0 = __builtin_bit_cast(uint32_t, v0 * ps.slo + ps.mlo);
+  lo1 = __builtin_bit_cast(uint32_t, v1 * ps.slo + ps.mlo);
+  hi0 = __builtin_bit_cast(uint32_t, v2 * ps.shi + ps.mhi);
+  hi1 = __builtin_bit_cast(uint32_t, v3 * ps.shi + ps.mhi);
 }
 
 // tanh-form GELU with tanh(t) = 1 - 2 / (1 + e^{2t}): a handful of instructions, inlined once per
@@ -235,93 +251,100 @@ __device__ __forceinline__ float gelu_tanh_fast(float x) {
 }
 
 #ifdef DH_GEMM_TRACE
-__device__ unsigned long long dh_gemm_trace_buf[8 * 128];
-#define DH_GTS() do { if (lane == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 0 && tsn < 127) \
+__device__ unsigned long long dh_gemm_trace_buf[12 * 128];
+#define DH_GTS() do { if (lane == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 0 && tsn < 124) \
                         dh_gemm_trace_buf[wave * 128 + tsn++] = wall_clock64(); } while (0)
 #else
 #define DH_GTS() do {} while (0)
 #endif
 
-// T = MFMA tiles per wave along each of M and N: workgroup tile 64T x 64T (T = 2: 128 x 128 for
-// large problems, T = 1: 64 x 64 when a 128-tiling would leave most compute units idle).
-template <bool DUAL, int T, bool SPEC>
-__global__ __launch_bounds__(SPEC ? 512 : 256) void q4k_gemm_kernel(const GemmArgs a) {
+// T = MFMA tiles per wave along each of M and N (T = 2: a 64 x 64 quadrant per wave, T = 1:
+// 32 x 32 when larger tiles would leave most compute units idle).  Four waves cover a
+// 64T x 64T tile; MG = groups of four waves stacked along M, all multiplying against the same
+// weight tile.  Workgroup tile: 64T MG x 64T.  The weights of a tile are dequantised once per
+// workgroup, so MG = 2 halves that work per matrix-core instruction.
+template <bool DUAL, int T, int MG>
+__global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
   constexpr int NMAT = DUAL ? 2 : 1;
-  constexpr int BM = 64 * T, BN = 64 * T;
+  constexpr int SUBM = 64 * T;                               // rows of one group's A tile
+  constexpr int BM = SUBM * MG, BN = 64 * T;
   constexpr int A_HALVES = BM * LDS_ROW, B_HALVES = BN * LDS_ROW;
   extern __shared__ __align__(16) _Float16 lds[];            // [2 buffers][A | B | (B2)]
   constexpr int BUF_HALVES = A_HALVES + NMAT * B_HALVES;
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const bool producer = !SPEC || wave >= 4, multiplier = !SPEC || wave < 4;
-  const int tid = threadIdx.x & 255;            // index inside the role's 256 threads
+  constexpr int PT = 256 * MG;                               // threads of the workgroup
+  const int tid = threadIdx.x;
 #ifdef DH_GEMM_TRACE
   int tsn = 0;
 #endif
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  const int wm = (wave >> 1) * 32 * T, wn = (wave & 1) * 32 * T;     // the wave's quadrant
+  const int wm = (wave >> 2) * SUBM + ((wave >> 1) & 1) * 32 * T, wn = (wave & 1) * 32 * T;
   const int fr = lane & 31, fg = lane >> 5;                  // fragment row / k half
   const int64_t row_bytes = (int64_t)a.nb * kBlockBytes;
   const int kt0 = a.ksplit > 1 ? (int)blockIdx.z * a.kt_per_split : 0;
   const int nkt = a.ksplit > 1 ? min((a.K + BK - 1) / BK, kt0 + a.kt_per_split) : (a.K + BK - 1) / BK;
 
-  // ---- global -> register staging roles
-  // A: 16-byte pieces of the packed rows, idx = tid + 256 i: row idx >> 3, halves 8 * (idx & 7)
-  // W: thread (row tid >> 1, half tid & 1): 16 nibble bytes + header
-  const int w_row = tid >> 1, w_half = tid & 1;
-  const int64_t w_off = (int64_t)min(n0 + w_row, a.N - 1) * row_bytes;
-  constexpr int NA = BM * 8 / 256;                           // 16-byte loads of A per thread
-  const bool w_active = w_row < BN;
+  // ---- global -> register staging
+  // A: 16-byte pieces of the packed rows, idx = tid + PT i: row idx >> 3, halves 8 * (idx & 7)
+  // W: item (matrix, row, half) = 16 nibble bytes of one row + its block header; SPLIT threads
+  //    share an item (QD dwords each) when there are more threads than items
+  constexpr int NA = BM * 8 / PT;                            // 16-byte loads of A per thread
+  constexpr int ITEMS = 2 * BN * NMAT;
+  constexpr int SPLIT = PT > ITEMS ? (PT / ITEMS > 2 ? 2 : PT / ITEMS) : 1;
+  constexpr int QD = 4 / SPLIT;                              // dwords of nibbles per thread and item
+  constexpr int UNITS = ITEMS * SPLIT;
+  constexpr int NW = UNITS > PT ? UNITS / PT : 1;            // units per thread
+  constexpr bool ALL_ACTIVE = UNITS >= PT;                   // every producer thread has its units
+  static_assert(BM * 8 % PT == 0 && (UNITS % PT == 0 || UNITS < PT), "producer threads must tile the work");
+  const uint8_t* w_ptr[NW];
+  int w_lds[NW], w_qoff[NW];
+  bool w_active[NW];
+#pragma unroll
+  for (int j = 0; j < NW; j++) {
+    const int u = tid + PT * j, it = u / SPLIT, sub = u % SPLIT;
+    const int mt = it / (2 * BN), rem = it % (2 * BN), row = rem >> 1, half = rem & 1;
+    w_active[j] = u < UNITS;
+    w_qoff[j] = 16 + 16 * half + 8 * sub;
+    // rows past the tile or the matrix re-read row N - 1: the loads stay unconditional
+    w_ptr[j] = ((mt & 1) && NMAT > 1 ? a.W2 : a.W) + (int64_t)min(n0 + row, a.N - 1) * row_bytes;
+    w_lds[j] = A_HALVES + (mt % NMAT) * B_HALVES + row * LDS_ROW + 16 * half + 8 * sub;
+  }
   // Two register sets: while tile kt is multiplied, tile kt+1 waits in one set and the loads of
   // tile kt+2 are in flight into the other, so a load has two K steps to arrive.
   struct Staged {
     u32x4_t a[NA];
-    u32x4_t q[NMAT], h[NMAT];
+    u32x4_t q[NW], h[NW];
   };
   Staged st0, st1;
   // row factors of this tile's activation rows: one global read each, then LDS
   __shared__ float2 rs_lds[BM];
-  if (threadIdx.x < BM) rs_lds[threadIdx.x] = a.row_scale[min(m0 + (int)threadIdx.x, a.M - 1)];
+  for (int r = threadIdx.x; r < BM; r += blockDim.x) rs_lds[r] = a.row_scale[min(m0 + r, a.M - 1)];
 
+  // Every load is unconditional (past the end of K the last tile is loaded again and never used,
+  // rows past the matrix re-read its last row): loads complete in order, so with exactly one
+  // tile's loads issued per step the wait in front of the older tile leaves the younger tile's
+  // loads in flight.  A load under a condition turns that wait into "all loads", and a load then
+  // has one K step to arrive instead of two.
   auto load_tile = [&](int kt, Staged& st) {
 #pragma unroll
     for (int i = 0; i < NA; i++) {
-      const int idx = tid + 256 * i, r = idx >> 3;
+      const int idx = tid + PT * i, r = idx >> 3;
       const int m = min(m0 + r, a.M - 1);
       st.a[i] = *reinterpret_cast<const u32x4_t*>(a.Apk + (int64_t)m * a.kpad + kt * BK + 8 * (idx & 7));
     }
     const int blk = kt >> 2, c = kt & 3;
 #pragma unroll
-    for (int mt = 0; mt < NMAT; mt++) {
-      if (w_active) {
-        const uint8_t* bp = (mt ? a.W2 : a.W) + w_off + (int64_t)blk * kBlockBytes;
-        st.h[mt] = *reinterpret_cast<const u32x4_t*>(bp);
-        st.q[mt] = *reinterpret_cast<const u32x4_t*>(bp + 16 + 32 * c + 16 * w_half);
+    for (int j = 0; j < NW; j++) {
+      const uint8_t* bp = w_ptr[j] + (int64_t)blk * kBlockBytes;
+      st.h[j] = *reinterpret_cast<const u32x4_t*>(bp);
+      if constexpr (QD == 4) {
+        st.q[j] = *reinterpret_cast<const u32x4_t*>(bp + 32 * c + w_qoff[j]);
+      } else {
+        const uint2 v = *reinterpret_cast<const uint2*>(bp + 32 * c + w_qoff[j]);
+        st.q[j][0] = v.x;
+        st.q[j][1] = v.y;
       }
-    }
-  };
-  auto store_tile = [&](int kt, int buf, const Staged& st) {
-    _Float16* At = lds + buf * BUF_HALVES;
-#pragma unroll
-    for (int i = 0; i < NA; i++) {
-      const int idx = tid + 256 * i, r = idx >> 3;
-      *reinterpret_cast<u32x4_t*>(At + r * LDS_ROW + 8 * (idx & 7)) = st.a[i];
-    }
-    const int c = kt & 3;
-#pragma unroll
-    for (int mt = 0; mt < NMAT; mt++) {
-      if (!w_active) break;
-      float sc_lo, sc_hi, mn_lo, mn_hi;
-      const uint4 hdr = make_uint4(st.h[mt][0], st.h[mt][1], st.h[mt][2], st.h[mt][3]);
-      const uint4 qv = make_uint4(st.q[mt][0], st.q[mt][1], st.q[mt][2], st.q[mt][3]);
-      q4k_pair_scales(hdr, c, sc_lo, sc_hi, mn_lo, mn_hi);
-      uint4 lo[2], hi[2];
-      dequant16(qv, sc_lo, mn_lo, sc_hi, mn_hi, lo, hi);
-      _Float16* Bt = lds + buf * BUF_HALVES + A_HALVES + mt * B_HALVES + w_row * LDS_ROW;
-      *reinterpret_cast<uint4*>(Bt + 16 * w_half) = lo[0];
-      *reinterpret_cast<uint4*>(Bt + 16 * w_half + 8) = lo[1];
-      *reinterpret_cast<uint4*>(Bt + 32 + 16 * w_half) = hi[0];
-      *reinterpret_cast<uint4*>(Bt + 32 + 16 * w_half + 8) = hi[1];
     }
   };
 
@@ -335,61 +358,121 @@ __global__ __launch_bounds__(SPEC ? 512 : 256) void q4k_gemm_kernel(const GemmAr
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[mt][i][j][e] = 0.f;
 
-  // One K step.  Multipliers: the tile in LDS buffer kt & 1.  Producers: move tile kt+1 from `nxt`
-  // into the other buffer and start the loads of tile kt+3 into `nxt`.
-  auto k_step = [&](int kt, Staged& nxt) {
-    DH_GTS();
-    const int buf = kt & 1;
-    const _Float16* At = lds + buf * BUF_HALVES;
-    if (multiplier) {
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ks++) {
-      half8_t af[T], bf[NMAT][T];
+  // Multiplies the tile in LDS buffer kt & 1.  Fragments are double-buffered in registers: the
+  // reads of k slice ks+1 are issued before the matrix-core instructions of slice ks, so the LDS
+  // latency runs under them.  after(slot) is called behind every matrix-core instruction
+  // (slot = its index within the K step).
+  constexpr int NMFMA = (BK / 16) * NMAT * T * T;
+  auto multiply_step = [&](int kt, auto&& after) {
+    const _Float16* At = lds + (kt & 1) * BUF_HALVES;
+    half8_t af[2][T], bf[2][NMAT][T];
+    auto read_frags = [&](int ks, half8_t (&fa)[T], half8_t (&fb)[NMAT][T]) {
 #pragma unroll
       for (int i = 0; i < T; i++)
-        af[i] = *reinterpret_cast<const half8_t*>(At + (wm + 32 * i + fr) * LDS_ROW + 16 * ks + 8 * fg);
+        fa[i] = *reinterpret_cast<const half8_t*>(At + (wm + 32 * i + fr) * LDS_ROW + 16 * ks + 8 * fg);
 #pragma unroll
       for (int mt = 0; mt < NMAT; mt++)
 #pragma unroll
         for (int j = 0; j < T; j++)
-          bf[mt][j] = *reinterpret_cast<const half8_t*>(At + A_HALVES + mt * B_HALVES + (wn + 32 * j + fr) * LDS_ROW +
+          fb[mt][j] = *reinterpret_cast<const half8_t*>(At + A_HALVES + mt * B_HALVES + (wn + 32 * j + fr) * LDS_ROW +
                                                         16 * ks + 8 * fg);
+    };
+    read_frags(0, af[0], bf[0]);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      if (ks + 1 < BK / 16) read_frags(ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
 #pragma unroll
       for (int mt = 0; mt < NMAT; mt++)
 #pragma unroll
         for (int i = 0; i < T; i++)
 #pragma unroll
-          for (int j = 0; j < T; j++)
+          for (int j = 0; j < T; j++) {
             // accumulators pinned to the accumulation registers: left to itself the compiler keeps
             // them in vector registers and copies all of them aside and back every K step
-            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[mt][i][j]) : "v"(af[i]), "v"(bf[mt][j]));
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0"
+                         : "+a"(acc[mt][i][j])
+                         : "v"(af[ks & 1][i]), "v"(bf[ks & 1][mt][j]));
+            after(((ks * NMAT + mt) * T + i) * T + j);
+          }
     }
+  };
+  auto no_hook = [](int) {};
+
+  // The producer's work of one K step in NPARTS pieces, so that it can be dealt out between the
+  // matrix-core instructions of the same wave (each runs for 32 cycles while the wave is free to
+  // issue vector instructions): piece 0 stores the A tile, then per weight unit the scales and
+  // its dwords of nibbles, and the last piece issues the loads two tiles ahead.
+  constexpr int NPARTS = 2 + (1 + QD) * NW;
+  PairScales ps[NW];
+  uint32_t lo_w[NW][2 * QD], hi_w[NW][2 * QD];
+  auto produce_part = [&](int part, int kt, Staged& nxt) {      // moves tile kt + 1
+    _Float16* At = lds + ((kt & 1) ^ 1) * BUF_HALVES;
+    if (part == 0) {
+#pragma unroll
+      for (int i = 0; i < NA; i++) {
+        const int idx = tid + PT * i, r = idx >> 3;
+        *reinterpret_cast<u32x4_t*>(At + r * LDS_ROW + 8 * (idx & 7)) = nxt.a[i];
+      }
+    } else if (part == NPARTS - 1) {
+      load_tile(min(kt + 3, nkt - 1), nxt);
+    } else {
+      const int j = (part - 1) / (1 + QD), d = (part - 1) % (1 + QD) - 1;
+      if (ALL_ACTIVE || w_active[j]) {
+        if (d < 0) {
+          ps[j] = pair_scales_f16(nxt.h[j], (kt + 1) & 3);
+        } else {
+          dequant_dword(nxt.q[j][d], ps[j], lo_w[j][2 * d], lo_w[j][2 * d + 1], hi_w[j][2 * d], hi_w[j][2 * d + 1]);
+          if (d & 1) {
+            _Float16* Bt = At + w_lds[j] + 4 * (d - 1);
+            *reinterpret_cast<uint4*>(Bt) = make_uint4(lo_w[j][2 * d - 2], lo_w[j][2 * d - 1], lo_w[j][2 * d], lo_w[j][2 * d + 1]);
+            *reinterpret_cast<uint4*>(Bt + 32) = make_uint4(hi_w[j][2 * d - 2], hi_w[j][2 * d - 1], hi_w[j][2 * d], hi_w[j][2 * d + 1]);
+          }
+        }
+      }
     }
-    DH_GTS();
-    if (producer) {
-      if (kt + 1 < nkt) store_tile(kt + 1, buf ^ 1, nxt);
-      if (kt + 3 < nkt) load_tile(kt + 3, nxt);
-    }
-    __syncthreads();
+  };
+  auto produce_first = [&]() {
+    load_tile(kt0, st0);
+#pragma unroll
+    for (int part = 0; part < NPARTS - 1; part++) produce_part(part, kt0 - 1, st0);   // tile kt0 into its buffer
+    load_tile(min(kt0 + 1, nkt - 1), st0);
+    load_tile(min(kt0 + 2, nkt - 1), st1);
+  };
+  // Multiplies tile kt and, between its matrix-core instructions, moves tile kt+1 out of `nxt`
+  // into the other LDS buffer and reloads `nxt` with tile kt+3.
+  auto fused_step = [&](int kt, Staged& nxt) {
+    multiply_step(kt, [&](int slot) {
+#pragma unroll
+      for (int part = 0; part < NPARTS; part++)
+        if (part * NMFMA / NPARTS == slot) produce_part(part, kt, nxt);
+      __builtin_amdgcn_sched_barrier(0);
+    });
   };
 
-  if (producer) {
-    load_tile(kt0, st0);
-    store_tile(kt0, kt0 & 1, st0);
-    if (kt0 + 1 < nkt) load_tile(kt0 + 1, st0);
-    if (kt0 + 2 < nkt) load_tile(kt0 + 2, st1);
-  }
+  produce_first();
   __syncthreads();
-  for (int kt = kt0; kt < nkt; kt += 2) {
-    k_step(kt, st0);
-    if (kt + 1 < nkt) k_step(kt + 1, st1);
+  int kt = kt0;
+  for (; kt + 2 < nkt; kt += 2) {        // st0 holds the tiles at odd distance from kt0, st1 the even ones
+    DH_GTS();
+    fused_step(kt, st0);
+    DH_GTS();
+    __syncthreads();
+    DH_GTS();
+    fused_step(kt + 1, st1);
+    DH_GTS();
+    __syncthreads();
   }
+  if (kt + 1 < nkt) {
+    fused_step(kt, st0);
+    __syncthreads();
+    kt++;
+  }
+  multiply_step(kt, no_hook);
 
   DH_GTS();
 #ifdef DH_GEMM_TRACE
   if (lane == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 0) dh_gemm_trace_buf[wave * 128 + 127] = tsn;
 #endif
-  if (!multiplier) return;
   // the matrix-core instructions above are inline asm, invisible to the compiler's hazard
   // checks: give the last one time to retire before its accumulators are read
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
@@ -401,10 +484,11 @@ __global__ __launch_bounds__(SPEC ? 512 : 256) void q4k_gemm_kernel(const GemmAr
       const int n = n0 + wn + 32 * j + fr;
 #pragma unroll
       for (int e = 0; e < 16; e++) {
-        const int m = m0 + wm + 32 * i + 8 * (e >> 2) + 4 * fg + (e & 3);
+        const int rl = wm + 32 * i + 8 * (e >> 2) + 4 * fg + (e & 3);
+        const int m = m0 + rl;
         if (m < a.M && n < a.N) {
           float v;
-          const float unscale = rs_lds[wm + 32 * i + 8 * (e >> 2) + 4 * fg + (e & 3)].y;
+          const float unscale = rs_lds[rl].y;
           if (!DUAL && a.ksplit > 1) {
             a.partial[((int64_t)blockIdx.z * a.M + m) * a.N + n] = acc[0][i][j][e] * unscale;
             continue;
@@ -441,12 +525,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs a) {
     reinterpret_cast<float*>(a.C)[i] = v;
 }
 
-template <bool DUAL, int T>
+template <bool DUAL, int T, int MG>
 int launch_gemm_cfg(const GemmArgs& a, const char* op) {
-  constexpr bool SPEC = DUAL && T == 2;      // 110 KB of LDS: one workgroup per compute unit
-  constexpr int BM = 64 * T, BN = 64 * T;
-  const size_t lds = (size_t)2 * (DUAL ? 3 : 2) * BM * LDS_ROW * sizeof(_Float16);
-  auto kern = q4k_gemm_kernel<DUAL, T, SPEC>;
+  constexpr int BM = 64 * T * MG, BN = 64 * T;
+  const size_t lds = (size_t)2 * (BM + (DUAL ? 2 : 1) * BN) * LDS_ROW * sizeof(_Float16);
+  auto kern = q4k_gemm_kernel<DUAL, T, MG>;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
     DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -454,7 +537,7 @@ int launch_gemm_cfg(const GemmArgs& a, const char* op) {
     attr_set = true;
   }
   const dim3 grid((unsigned)dh::ceil_div(a.N, BN), (unsigned)dh::ceil_div(a.M, BM), (unsigned)std::max(1, a.ksplit));
-  hipLaunchKernelGGL(kern, grid, dim3(SPEC ? 512 : 256), lds, dh::stream(), a);
+  hipLaunchKernelGGL(kern, grid, dim3(256 * MG), lds, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   if (a.ksplit > 1) {
     const int64_t total = (int64_t)a.M * a.N;
@@ -505,9 +588,20 @@ int launch_gemm(GemmArgs a, const char* op) {
   DH_CHECK_LAUNCH(op);
   a.row_scale = scales;
   a.Apk = packed;
+  // Tile choice, largest first: 256 x 128 (eight waves) when such tiles fill the compute units,
+  // for the fused gate/up pair 128 x 64 (eight waves) next, then 128 x 128 (four waves, two
+  // workgroups per compute unit) when those occupy at least half of them, else 64 x 64.
   const int64_t big_tiles = dh::ceil_div(a.M, 128) * dh::ceil_div(a.N, 128);
+  const int64_t tall_tiles = dh::ceil_div(a.M, 256) * dh::ceil_div(a.N, 128);
   a.ksplit = 1;
-  if (2 * big_tiles >= dh::num_cus()) return launch_gemm_cfg<DUAL, 2>(a, op);
+  if (tall_tiles >= dh::num_cus()) return launch_gemm_cfg<DUAL, 2, 2>(a, op);
+  if (2 * big_tiles >= dh::num_cus()) {
+    if constexpr (DUAL) {
+      return launch_gemm_cfg<true, 1, 2>(a, op);
+    } else {
+      return launch_gemm_cfg<false, 2, 1>(a, op);
+    }
+  }
   // Few tiles and a long K: every workgroup would walk K alone at one memory round trip per
   // step.  Cut K so that about three workgroups share a compute unit and overlap each other's
   // waits; the pieces meet in the library's scratch buffer.
@@ -527,7 +621,7 @@ int launch_gemm(GemmArgs a, const char* op) {
       a.partial = ws;
     }
   }
-  return launch_gemm_cfg<DUAL, 1>(a, op);
+  return launch_gemm_cfg<DUAL, 1, 1>(a, op);
 }
 
 }  // namespace
