@@ -230,17 +230,25 @@ __device__ __forceinline__ PairScales pair_scales_f16(const u32x4_t hdr, const i
   return r;
 }
 // One dword of nibbles (8 weights) -> two low-nibble and two high-nibble f16 pairs.
-__device__ __forceinline__ void dequant_dword(const uint32_t w, const PairScales& ps, uint32_t& lo0, uint32_t& lo1,
-                                              uint32_t& hi0, uint32_t& hi1) {
+// `magic` is 0x64006400 held in a vector register (see magic_1024): with the constant visible the
+// compiler emits v_and + v_or, since one instruction may read only one literal or scalar.
+__device__ __forceinline__ void dequant_dword(const uint32_t w, const PairScales& ps, const uint32_t magic, uint32_t& lo0,
+                                              uint32_t& lo1, uint32_t& hi0, uint32_t& hi1) {
   const half2_t k1024 = {(_Float16)1024.f, (_Float16)1024.f};
-  const half2_t v0 = __builtin_bit_cast(half2_t, (w & 0x000F000Fu) | 0x64006400u) - k1024;
-  const half2_t v1 = __builtin_bit_cast(half2_t, ((w >> 8) & 0x000F000Fu) | 0x64006400u) - k1024;
-  const half2_t v2 = __builtin_bit_cast(half2_t, ((w >> 4) & 0x000F000Fu) | 0x64006400u) - k1024;
-  const half2_t v3 = __builtin_bit_cast(half2_t, ((w >> 12) & 0x000F000Fu) | 0x64006400u) - k1024;
+  const half2_t v0 = __builtin_bit_cast(half2_t, (w & 0x000F000Fu) | magic) - k1024;
+  const half2_t v1 = __builtin_bit_cast(half2_t, ((w >> 8) & 0x000F000Fu) | magic) - k1024;
+  const half2_t v2 = __builtin_bit_cast(half2_t, ((w >> 4) & 0x000F000Fu) | magic) - k1024;
+  const half2_t v3 = __builtin_bit_cast(half2_t, ((w >> 12) & 0x000F000Fu) | magic) - k1024;
   lo0 = __builtin_bit_cast(uint32_t, v0 * ps.slo + ps.mlo);
   lo1 = __builtin_bit_cast(uint32_t, v1 * ps.slo + ps.mlo);
   hi0 = __builtin_bit_cast(uint32_t, v2 * ps.shi + ps.mhi);
   hi1 = __builtin_bit_cast(uint32_t, v3 * ps.shi + ps.mhi);
+}
+
+__device__ __forceinline__ uint32_t magic_1024() {
+  uint32_t m;
+  asm("v_mov_b32 %0, 0x64006400" : "=v"(m));
+  return m;
 }
 
 // tanh-form GELU with tanh(t) = 1 - 2 / (1 + e^{2t}): a handful of instructions, inlined once per
@@ -297,7 +305,9 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
   constexpr int NW = UNITS > PT ? UNITS / PT : 1;            // units per thread
   constexpr bool ALL_ACTIVE = UNITS >= PT;                   // every producer thread has its units
   static_assert(BM * 8 % PT == 0 && (UNITS % PT == 0 || UNITS < PT), "producer threads must tile the work");
-  const uint8_t* w_ptr[NW];
+  // per-thread byte offsets of the loads (the host checks that both operands stay below 2 GB)
+  uint32_t w_off[NW], a_off[NA];
+  bool w_second[NW];
   int w_lds[NW], w_qoff[NW];
   bool w_active[NW];
 #pragma unroll
@@ -307,7 +317,9 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
     w_active[j] = u < UNITS;
     w_qoff[j] = 16 + 16 * half + 8 * sub;
     // rows past the tile or the matrix re-read row N - 1: the loads stay unconditional
-    w_ptr[j] = ((mt & 1) && NMAT > 1 ? a.W2 : a.W) + (int64_t)min(n0 + row, a.N - 1) * row_bytes;
+    // a matrix's units are a multiple of 64 threads: uniform per wave, so the base stays scalar
+    w_second[j] = NMAT > 1 && __builtin_amdgcn_readfirstlane(mt & 1) != 0;
+    w_off[j] = (uint32_t)((int64_t)min(n0 + row, a.N - 1) * row_bytes);
     w_lds[j] = A_HALVES + (mt % NMAT) * B_HALVES + row * LDS_ROW + 16 * half + 8 * sub;
   }
   // Two register sets: while tile kt is multiplied, tile kt+1 waits in one set and the loads of
@@ -326,24 +338,35 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
   // tile's loads issued per step the wait in front of the older tile leaves the younger tile's
   // loads in flight.  A load under a condition turns that wait into "all loads", and a load then
   // has one K step to arrive instead of two.
+#pragma unroll
+  for (int i = 0; i < NA; i++) {
+    const int idx = tid + PT * i, r = idx >> 3;
+    a_off[i] = (uint32_t)(((int64_t)min(m0 + r, a.M - 1) * a.kpad + 8 * (idx & 7)) * 2);
+  }
+  // Buffer loads: address = descriptor base + per-thread 32-bit offset + per-step scalar offset,
+  // so the loop holds no vector address arithmetic (and a read past a tensor would return 0).
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<_Float16*>(a.Apk), 0, (int)min((int64_t)a.M * a.kpad * 2, (int64_t)0x7fffffff), 0x00020000);
+  const int w_bytes = (int)min((int64_t)a.N * row_bytes, (int64_t)0x7fffffff);
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.W), 0, w_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t w2_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(NMAT > 1 ? a.W2 : a.W), 0, w_bytes, 0x00020000);
   auto load_tile = [&](int kt, Staged& st) {
 #pragma unroll
-    for (int i = 0; i < NA; i++) {
-      const int idx = tid + PT * i, r = idx >> 3;
-      const int m = min(m0 + r, a.M - 1);
-      st.a[i] = *reinterpret_cast<const u32x4_t*>(a.Apk + (int64_t)m * a.kpad + kt * BK + 8 * (idx & 7));
-    }
+    for (int i = 0; i < NA; i++)
+      st.a[i] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, a_off[i], kt * (BK * 2), 0));
     const int blk = kt >> 2, c = kt & 3;
 #pragma unroll
     for (int j = 0; j < NW; j++) {
-      const uint8_t* bp = w_ptr[j] + (int64_t)blk * kBlockBytes;
-      st.h[j] = *reinterpret_cast<const u32x4_t*>(bp);
+      const __amdgpu_buffer_rsrc_t r = w_second[j] ? w2_rsrc : w_rsrc;
+      st.h[j] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(r, w_off[j], blk * kBlockBytes, 0));
       if constexpr (QD == 4) {
-        st.q[j] = *reinterpret_cast<const u32x4_t*>(bp + 32 * c + w_qoff[j]);
+        st.q[j] = __builtin_bit_cast(u32x4_t, __builtin_amdgcn_raw_buffer_load_b128(r, w_off[j] + w_qoff[j],
+                                                                                  blk * kBlockBytes + 32 * c, 0));
       } else {
-        const uint2 v = *reinterpret_cast<const uint2*>(bp + 32 * c + w_qoff[j]);
-        st.q[j][0] = v.x;
-        st.q[j][1] = v.y;
+        const auto v = __builtin_amdgcn_raw_buffer_load_b64(r, w_off[j] + w_qoff[j], blk * kBlockBytes + 32 * c, 0);
+        st.q[j][0] = v[0];
+        st.q[j][1] = v[1];
       }
     }
   };
@@ -404,6 +427,7 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
   // its dwords of nibbles, and the last piece issues the loads two tiles ahead.
   constexpr int NPARTS = 2 + (1 + QD) * NW;
   PairScales ps[NW];
+  const uint32_t magic = magic_1024();
   uint32_t lo_w[NW][2 * QD], hi_w[NW][2 * QD];
   auto produce_part = [&](int part, int kt, Staged& nxt) {      // moves tile kt + 1
     _Float16* At = lds + ((kt & 1) ^ 1) * BUF_HALVES;
@@ -421,7 +445,7 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
         if (d < 0) {
           ps[j] = pair_scales_f16(nxt.h[j], (kt + 1) & 3);
         } else {
-          dequant_dword(nxt.q[j][d], ps[j], lo_w[j][2 * d], lo_w[j][2 * d + 1], hi_w[j][2 * d], hi_w[j][2 * d + 1]);
+          dequant_dword(nxt.q[j][d], ps[j], magic, lo_w[j][2 * d], lo_w[j][2 * d + 1], hi_w[j][2 * d], hi_w[j][2 * d + 1]);
           if (d & 1) {
             _Float16* Bt = At + w_lds[j] + 4 * (d - 1);
             *reinterpret_cast<uint4*>(Bt) = make_uint4(lo_w[j][2 * d - 2], lo_w[j][2 * d - 1], lo_w[j][2 * d], lo_w[j][2 * d + 1]);
@@ -559,6 +583,10 @@ int launch_gemm(GemmArgs a, const char* op) {
   if (!packed || !scales) return dh::fail(2, "[%s] the library's scratch buffers are missing (dh_init)", op);
   const int cap = (int)std::min<size_t>((size_t)dh::gemm_row_scale_capacity(), pk_bytes / ((size_t)a.kpad * 2));
   if (cap < 16) return dh::fail(1, "[%s] K=%d is too long for the prefill GEMM's activation scratch", op, a.K);
+  // the kernel addresses a weight row as a 32-bit byte offset into a buffer descriptor
+  if ((int64_t)a.N * a.nb * kBlockBytes >= ((int64_t)1 << 31))
+    return dh::fail(1, "[%s] a weight tensor of %d x %d (2 GB or more) is beyond the prefill GEMM; split it by rows", op,
+                    a.N, a.K);
   if (a.M > cap) {
     const size_t c_elem = a.c_f16 ? 2 : 4;
     for (int m0 = 0; m0 < a.M; m0 += cap) {
