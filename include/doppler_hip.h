@@ -78,7 +78,8 @@ int dh_q4k_dequant(const void* d_W, int64_t num_blocks, float* d_out);
  * f16 (c_dtype).  K need not be a multiple of 256: the padded tail of each row's last
  * block is ignored.  d_residual (may be NULL) is added after alpha, as the reference's
  * `residualTensor` option does.  M = 1..8 takes the HBM-bound GEMV path, larger M the
- * MFMA GEMM path. */
+ * MFMA GEMM path (from 16 rows on a weight tensor must be smaller than 2 GB, as the kernel
+ * addresses it through one buffer descriptor; a larger one fails with a message). */
 int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int c_dtype,
                   int M, int N, int K, float alpha, const void* d_residual);
 

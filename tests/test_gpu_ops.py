@@ -318,6 +318,17 @@ def test_rmsnorm_prologue_between_gemv_and_gemm_batches(M):
     assert rel_l2(ops.readTensor(out), oracle.q4k_matmul(X, W, M, N, K)) <= REL_L2_F32
 
 
+def test_prefill_gemm_rejects_a_weight_tensor_its_descriptor_cannot_address():
+    """From 16 rows on the kernel reaches a weight row through a 32-bit offset: 2 GB or more fails before any launch
+    (so the small buffers handed over here are never touched)."""
+    lib = capi.load()
+    A = ops.tensorFromNumpy(np.zeros((16, 1024), np.float32))
+    small = ops.tensorFromNumpy(np.zeros(1024, np.float32))
+    N = 4_000_000                               # 4e6 rows x 4 blocks x 144 bytes = 2.3 GB
+    rc = lib.dh_q4k_matmul(A.buffer.data_ptr(), 0, small.buffer.data_ptr(), small.buffer.data_ptr(), 0, 16, N, 1024, 1.0, None)
+    assert rc != 0 and b"2 GB" in lib.dh_last_error()
+
+
 @pytest.mark.parametrize("M,N,K", [(16, 300, 1024), (40, 512, 1152), (512, 1024, 4096), (130, 200, 12288), (33, 96, 640)])
 def test_matmul_rmsnorm_prologue_on_the_gemm_path(M, N, K):
     """M >= 16: the rows are normalised while the GEMM's activations are packed."""
