@@ -144,6 +144,26 @@ def test_matmul_prefill_gemm(M, N, K, kw):
     assert _matmul_case(M, N, K, seed=1500 + M, **kw) <= REL_L2_F16_MFMA
 
 
+@pytest.mark.parametrize("M,N,K,kw", [(1000, 8200, 320, dict(residual=True)), (1024, 8192, 256, dict(outputDtype="f16")),
+                                      (2048, 4224, 192, dict(alpha=0.5))])
+def test_matmul_prefill_gemm_tall_tiles(M, N, K, kw):
+    """Enough 256 x 128 tiles to fill 256 compute units: the eight-wave tall-tile kernel, with ragged edges in M
+    and N, an odd number of K steps and a K that ends inside a super-block."""
+    assert -(-M // 256) * -(-N // 128) >= 256
+    assert _matmul_case(M, N, K, seed=1560 + K, **kw) <= REL_L2_F16_MFMA
+
+
+@pytest.mark.parametrize("M,hidden,inter,activation", [(1000, 320, 8200, "silu"), (1024, 256, 8192, "gelu")])
+def test_fused_ffn_prefill_tall_tiles(M, hidden, inter, activation):
+    """The fused gate/up pair on 256 x 128 x 2 tiles."""
+    Wg, wg = q4k_weight(inter, hidden, seed=2410)
+    Wu, wu = q4k_weight(inter, hidden, seed=2411)
+    X = synth.normal_f32((M, hidden), seed=2412, scale=0.05)
+    out = ops.runFusedFFN(ops.tensorFromNumpy(X), wg, wu, hidden, inter, batchSize=M, activation=activation)
+    want = oracle.q4k_ffn_gate_up(X, Wg, Wu, M, hidden, inter, alpha=1.0, activation=activation)
+    assert rel_l2(ops.readTensor(out), want) <= REL_L2_F16_MFMA
+
+
 def test_matmul_prefill_gemm_activation_range():
     """Rows far outside the f16 range (and far below it) go through the f16 matrix-core path: each
     row is scaled by its own power of two before rounding."""
