@@ -10,8 +10,9 @@
 //   S^T = K . Q^T   A = K rows from LDS (16 bytes of a key row per lane), B = Q^T from registers
 //                   (scale folded in, rounded to f16).  D[key][q]: lane (q = l & 15, g = l >> 4)
 //                   gets keys 16j + 4g + i (i < 4) of key subtile j.
-//   softmax         per query = per lane column: maxima and sums over a lane's 16 values, then
-//                   across the four lanes l, l+16, l+32, l+48; fp32, online rescale.
+//   softmax         per query = per lane column: maxima and sums over a lane's 16 values, the
+//                   maxima then across the four lanes l, l+16, l+32, l+48 (lane-swap
+//                   instructions), the sums only once after the last tile; fp32, online rescale.
 //   O^T = V^T . P^T B = P^T is exactly the lane's own probabilities (k-slot (g, i') stands for
 //                   key 16 (2 kb + i'/4) + 4g + i'%4 of 32-key block kb: a contraction index may be
 //                   renumbered as long as both operands agree), A = V^T read from LDS, where the
@@ -31,6 +32,23 @@ typedef __attribute__((ext_vector_type(4))) float float4_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;   // plain vector type: arrays of it stay in registers
 
 constexpr int BQ = 64, BKEYS = 64;
+
+// The four lanes l, l ^ 16, l ^ 32, l ^ 48 hold one query's scores.  v_permlane32_swap and
+// v_permlane16_swap (gfx950) hand a lane its partner's value through the vector ALU: with both
+// operands the same register, one result holds the lane's own half (row) pair and the other the
+// partner's.  No LDS round trip, and no wait that would also stall on outstanding fragment reads.
+__device__ __forceinline__ float quad_rows_max(float v) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_rows_sum(float v) {
+  auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
 
 struct PrefillArgs {
   const float* Q;       // [T][H][D]
@@ -172,8 +190,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
           mx = fmaxf(mx, s);
         }
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = quad_rows_max(mx);
     const float m_new = fmaxf(m_run, mx);              // finite: m_run starts at -FLT_MAX
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float ps = 0.f;
@@ -186,9 +203,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
         ps += p;
         pb[j >> 1][4 * (j & 1) + i] = (_Float16)p;
       }
-    ps += __shfl_xor(ps, 16, 64);
-    ps += __shfl_xor(ps, 32, 64);
-    l_run = l_run * alpha + ps;
+    l_run = l_run * alpha + ps;                        // this lane's share: alpha is the query's, the sum is taken once at the end
     m_run = m_new;
     const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;   // no new maximum: nothing to scale
     // ---- O^T = alpha O^T + V^T P^T
@@ -204,6 +219,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
   }
 #undef DH_PF_LOAD
 
+  l_run = quad_rows_sum(l_run);
   // ---- lane (q, g) holds O[my_q][16 t + 4 g + i]
   if (my_q < a.T) {
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
