@@ -1,9 +1,12 @@
 // Prefill attention (T query tokens at once) over an f16 KV cache with grouped-query heads, on the
 // matrix cores: the flash-attention recurrence with v_mfma_f32_16x16x32_f16.
 //
-// Grid = (query tiles of 64 tokens, query heads); a workgroup is 4 waves, wave w owns query rows
-// 16w..16w+15 of the tile.  Keys advance 64 at a time; the K and V tiles of the head's kv head
-// are staged in LDS once per workgroup and shared by the four waves.
+// Grid = (query tiles of 64 QT tokens, query heads); a workgroup is 4 waves, wave w owns QT
+// groups of 16 consecutive query rows of the tile.  Keys advance 64 at a time; the K and V tiles
+// of the head's kv head are staged in LDS once per workgroup and shared by the four waves, and
+// every fragment a wave reads from there feeds QT matrix-core instructions (QT = 2 for prompts
+// long enough to fill the compute units with 128-query tiles: the kernel is bound by LDS
+// traffic and instruction issue, not by the matrix cores; 118 -> 102 us at T = 2048, 32 heads).
 //
 // Everything is computed transposed, so that the softmax statistics of a query live in the lanes
 // that also hold its output column and nothing has to be shuffled between the two products:
@@ -22,6 +25,7 @@
 // tile instead of two, and dispatching the long late-query tiles first.)
 #include <algorithm>
 #include <cfloat>
+#include <cstdlib>
 
 #include "dh_common.h"
 
@@ -31,7 +35,7 @@ typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(4))) float float4_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;   // plain vector type: arrays of it stay in registers
 
-constexpr int BQ = 64, BKEYS = 64;
+constexpr int BKEYS = 64;
 
 // The four lanes l, l ^ 16, l ^ 32, l ^ 48 hold one query's scores.  v_permlane32_swap and
 // v_permlane16_swap (gfx950) hand a lane its partner's value through the vector ALU: with both
@@ -59,8 +63,11 @@ struct PrefillArgs {
   float scale, softcap;
 };
 
-template <int D>
+// QT = 16-query groups per wave: every K and V fragment read from LDS feeds QT matrix-core
+// instructions, and a workgroup tile (64 QT queries) stages each key tile once.
+template <int D, int QT>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) {
+  constexpr int BQ = 64 * QT;
   constexpr int STEPS = D / 32;            // MFMAs per 16 x 16 score tile
   constexpr int DT = D / 16;               // output row tiles (of O^T)
   constexpr int KROW = D + 8;              // halves per K row in LDS (16-byte pad)
@@ -73,24 +80,30 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
   const int q = lane & 15, g = lane >> 4;
   const int h = blockIdx.y, kvh = h / a.G;
   const int q0 = blockIdx.x * BQ;
-  const int my_q = q0 + 16 * wave + q;                        // query token of this lane's column
-  const int my_pos = a.start_pos + my_q;                      // its absolute position
   const int64_t kv_stride = (int64_t)a.Hkv * D;
+  int my_q[QT], my_pos[QT];                                   // query token of this lane's column, its absolute position
+#pragma unroll
+  for (int u = 0; u < QT; u++) {
+    my_q[u] = q0 + 16 * (QT * wave + u) + q;
+    my_pos[u] = a.start_pos + my_q[u];
+  }
 
   // ---- Q^T fragments (B operand): b[i] = scale * Q[my_q][32 s + 8 g + i].  Scores are kept in
   // units of log2(e), so that the softmax needs v_exp_f32 alone (with a soft cap the factor is
   // applied after the cap instead).
   constexpr float kLog2e = 1.4426950408889634f;
   const float qscale = a.softcap > 0.f ? a.scale : a.scale * kLog2e;
-  half8_t qb[STEPS];
+  half8_t qb[QT][STEPS];
 #pragma unroll
-  for (int s = 0; s < STEPS; s++) {
-    const float* qp = a.Q + ((int64_t)min(my_q, a.T - 1) * a.H + h) * D + 32 * s + 8 * g;
-    const float4 v0 = reinterpret_cast<const float4*>(qp)[0], v1 = reinterpret_cast<const float4*>(qp)[1];
-    const float qv[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+  for (int u = 0; u < QT; u++)
 #pragma unroll
-    for (int i = 0; i < 8; i++) qb[s][i] = (_Float16)(qv[i] * qscale);
-  }
+    for (int s = 0; s < STEPS; s++) {
+      const float* qp = a.Q + ((int64_t)min(my_q[u], a.T - 1) * a.H + h) * D + 32 * s + 8 * g;
+      const float4 v0 = reinterpret_cast<const float4*>(qp)[0], v1 = reinterpret_cast<const float4*>(qp)[1];
+      const float qv[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+      for (int i = 0; i < 8; i++) qb[u][s][i] = (_Float16)(qv[i] * qscale);
+    }
 
   // ---- key range of this query tile
   const int last_q = min(q0 + BQ, a.T) - 1;
@@ -101,10 +114,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
   kbeg = kbeg / BKEYS * BKEYS;
   const int ntiles = (kend - kbeg + BKEYS - 1) / BKEYS;
 
-  float4_t acc[DT];
+  float4_t acc[QT][DT];
+  float m_run[QT], l_run[QT];
 #pragma unroll
-  for (int t = 0; t < DT; t++) acc[t] = {0.f, 0.f, 0.f, 0.f};
-  float m_run = -FLT_MAX, l_run = 0.f;
+  for (int u = 0; u < QT; u++) {
+#pragma unroll
+    for (int t = 0; t < DT; t++) acc[u][t] = {0.f, 0.f, 0.f, 0.f};
+    m_run[u] = -FLT_MAX;
+    l_run[u] = 0.f;
+  }
 
   u32x4_t kreg[PIECES], vreg[PIECES];
   // K piece p = tid + 256 r of a tile: key p / (D/8), 8 consecutive dims starting at 8 (p % (D/8)).
@@ -151,82 +169,97 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const PrefillArgs a) 
     __syncthreads();
     if (kt + 1 < ntiles) { DH_PF_LOAD(kt + 1); }
 
-    // ---- S^T for this wave's 16 queries against the 64 keys
+    // ---- S^T for this wave's 16 QT queries against the 64 keys
     const int kbase = kbeg + kt * BKEYS;
-    float4_t st[4];
+    float4_t st[QT][4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      st[j] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < QT; u++) st[u][j] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < STEPS; s++) {
         const half8_t ka = *reinterpret_cast<const half8_t*>(&k_lds[(16 * j + q) * KROW + 32 * s + 8 * g]);
-        st[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[s], st[j], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < QT; u++) st[u][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[u][s], st[u][j], 0, 0, 0);
       }
     }
     // ---- mask, soft cap, online softmax (this lane: query my_q, keys kbase + 16 j + 4 g + i).
-    // A tile that every query of this wave sees completely needs no per-element masks.
-    const int wave_lo = a.start_pos + q0 + 16 * wave, wave_hi = wave_lo + 15;
-    const bool full = kbase + BKEYS <= a.kv_len && (!a.causal || kbase + BKEYS - 1 <= wave_lo) &&
-                      (a.window <= 0 || kbase > wave_hi - a.window);
-    float mx = -FLT_MAX;
-    if (full && !(a.softcap > 0.f)) {
+    // A tile that every query of a 16-query group sees completely needs no per-element masks.
+    half8_t pb[QT][2];
+    float alpha[QT];
+    bool rescale = false;
 #pragma unroll
-      for (int j = 0; j < 4; j++)
+    for (int u = 0; u < QT; u++) {
+      const int grp_lo = a.start_pos + q0 + 16 * (QT * wave + u), grp_hi = grp_lo + 15;
+      const bool full = kbase + BKEYS <= a.kv_len && (!a.causal || kbase + BKEYS - 1 <= grp_lo) &&
+                        (a.window <= 0 || kbase > grp_hi - a.window);
+      float mx = -FLT_MAX;
+      if (full && !(a.softcap > 0.f)) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) mx = fmaxf(mx, st[j][i]);
-    } else {
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) mx = fmaxf(mx, st[u][j][i]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int key = kbase + 16 * j + 4 * g + i;
+            float s = st[u][j][i];
+            if (a.softcap > 0.f) s = tanhf(s / a.softcap) * (a.softcap * kLog2e);
+            bool ok = key < a.kv_len;
+            if (a.causal) ok = ok && key <= my_pos[u];
+            if (a.window > 0) ok = ok && key > my_pos[u] - a.window;
+            s = ok ? s : -INFINITY;
+            st[u][j][i] = s;
+            mx = fmaxf(mx, s);
+          }
+      }
+      mx = quad_rows_max(mx);
+      const float m_new = fmaxf(m_run[u], mx);              // finite: m_run starts at -FLT_MAX
+      alpha[u] = __builtin_amdgcn_exp2f(m_run[u] - m_new);
+      float ps = 0.f;
 #pragma unroll
       for (int j = 0; j < 4; j++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          const int key = kbase + 16 * j + 4 * g + i;
-          float s = st[j][i];
-          if (a.softcap > 0.f) s = tanhf(s / a.softcap) * (a.softcap * kLog2e);
-          bool ok = key < a.kv_len;
-          if (a.causal) ok = ok && key <= my_pos;
-          if (a.window > 0) ok = ok && key > my_pos - a.window;
-          s = ok ? s : -INFINITY;
-          st[j][i] = s;
-          mx = fmaxf(mx, s);
+          const float p = __builtin_amdgcn_exp2f(st[u][j][i] - m_new);   // 2^-inf = 0 for masked keys
+          ps += p;
+          pb[u][j >> 1][4 * (j & 1) + i] = (_Float16)p;
         }
+      l_run[u] = l_run[u] * alpha[u] + ps;               // this lane's share: alpha is the query's, the sum is taken once at the end
+      m_run[u] = m_new;
+      rescale = rescale || __builtin_amdgcn_ballot_w64(alpha[u] != 1.0f) != 0;   // no new maximum: nothing to scale
     }
-    mx = quad_rows_max(mx);
-    const float m_new = fmaxf(m_run, mx);              // finite: m_run starts at -FLT_MAX
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    float ps = 0.f;
-    half8_t pb[2];
-#pragma unroll
-    for (int j = 0; j < 4; j++)
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const float p = __builtin_amdgcn_exp2f(st[j][i] - m_new);   // 2^-inf = 0 for masked keys
-        ps += p;
-        pb[j >> 1][4 * (j & 1) + i] = (_Float16)p;
-      }
-    l_run = l_run * alpha + ps;                        // this lane's share: alpha is the query's, the sum is taken once at the end
-    m_run = m_new;
-    const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;   // no new maximum: nothing to scale
     // ---- O^T = alpha O^T + V^T P^T
 #pragma unroll
     for (int t = 0; t < DT; t++) {
-      if (rescale) acc[t] *= alpha;
+      if (rescale) {
+#pragma unroll
+        for (int u = 0; u < QT; u++) acc[u][t] *= alpha[u];
+      }
 #pragma unroll
       for (int kb = 0; kb < 2; kb++) {
         const half8_t va = *reinterpret_cast<const half8_t*>(&v_lds[(16 * t + q) * VROW + 32 * kb + 8 * g]);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[kb], acc[t], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < QT; u++) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb[u][kb], acc[u][t], 0, 0, 0);
       }
     }
   }
 #undef DH_PF_LOAD
 
-  l_run = quad_rows_sum(l_run);
   // ---- lane (q, g) holds O[my_q][16 t + 4 g + i]
-  if (my_q < a.T) {
-    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-    float* op = a.O + ((int64_t)my_q * a.H + h) * D + 4 * g;
 #pragma unroll
-    for (int t = 0; t < DT; t++)
-      *reinterpret_cast<float4*>(op + 16 * t) = make_float4(acc[t][0] * inv, acc[t][1] * inv, acc[t][2] * inv, acc[t][3] * inv);
+  for (int u = 0; u < QT; u++) {
+    const float l = quad_rows_sum(l_run[u]);
+    if (my_q[u] < a.T) {
+      const float inv = l > 0.f ? 1.0f / l : 0.f;
+      float* op = a.O + ((int64_t)my_q[u] * a.H + h) * D + 4 * g;
+#pragma unroll
+      for (int t = 0; t < DT; t++)
+        *reinterpret_cast<float4*>(op + 16 * t) =
+            make_float4(acc[u][t][0] * inv, acc[u][t][1] * inv, acc[u][t][2] * inv, acc[u][t][3] * inv);
+    }
   }
 }
 
@@ -253,9 +286,18 @@ extern "C" int dh_attn_prefill(const float* d_Q, const void* d_K, const void* d_
   a.Q = d_Q; a.K = static_cast<const __half*>(d_K); a.V = static_cast<const __half*>(d_V); a.O = d_O;
   a.T = T; a.H = H; a.Hkv = Hkv; a.G = H / Hkv; a.kv_len = kv_len; a.start_pos = start_pos;
   a.causal = causal ? 1 : 0; a.window = sliding_window; a.scale = scale; a.softcap = softcap;
-  const dim3 grid((unsigned)dh::ceil_div(T, BQ), (unsigned)H);
-  if (D == 64) hipLaunchKernelGGL(attn_prefill_kernel<64>, grid, dim3(256), 0, dh::stream(), a);
-  else hipLaunchKernelGGL(attn_prefill_kernel<128>, grid, dim3(256), 0, dh::stream(), a);
+  // Two 16-query groups per wave (128 queries per workgroup) halve the LDS traffic per product;
+  // short prompts keep 64-query tiles so that the grid still covers the compute units.
+  static const int env_qt = getenv("DH_ATTN_PREFILL_QT") ? atoi(getenv("DH_ATTN_PREFILL_QT")) : 0;
+  const int qt = env_qt ? env_qt : ((int64_t)dh::ceil_div(T, 128) * H >= 2 * dh::num_cus() ? 2 : 1);
+  const dim3 grid((unsigned)dh::ceil_div(T, 64 * qt), (unsigned)H);
+  if (D == 64) {
+    if (qt == 2) hipLaunchKernelGGL((attn_prefill_kernel<64, 2>), grid, dim3(256), 0, dh::stream(), a);
+    else hipLaunchKernelGGL((attn_prefill_kernel<64, 1>), grid, dim3(256), 0, dh::stream(), a);
+  } else {
+    if (qt == 2) hipLaunchKernelGGL((attn_prefill_kernel<128, 2>), grid, dim3(256), 0, dh::stream(), a);
+    else hipLaunchKernelGGL((attn_prefill_kernel<128, 1>), grid, dim3(256), 0, dh::stream(), a);
+  }
   DH_CHECK_LAUNCH(op);
   return 0;
 }
