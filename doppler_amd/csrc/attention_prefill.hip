@@ -5,8 +5,9 @@
 // groups of 16 consecutive query rows of the tile.  Keys advance 64 at a time; the K and V tiles
 // of the head's kv head are staged in LDS once per workgroup and shared by the four waves, and
 // every fragment a wave reads from there feeds QT matrix-core instructions (QT = 2 for prompts
-// long enough to fill the compute units with 128-query tiles: the kernel is bound by LDS
-// traffic and instruction issue, not by the matrix cores; 118 -> 102 us at T = 2048, 32 heads).
+// long enough to fill the compute units with 128-query tiles: the kernel is bound by
+// instruction issue and LDS round trips per product, not by the matrix cores or by LDS
+// bandwidth; 118 -> 102 us at T = 2048, 32 heads).
 //
 // Everything is computed transposed, so that the softmax statistics of a query live in the lanes
 // that also hold its output column and nothing has to be shuffled between the two products:

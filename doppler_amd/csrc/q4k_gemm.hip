@@ -386,9 +386,10 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
   // latency runs under them.  after(slot) is called behind every matrix-core instruction
   // (slot = its index within the K step).
   constexpr int NMFMA = (BK / 16) * NMAT * T * T;
+  constexpr int FD = 2;                                      // fragment sets in flight (3 and 4 measured: no gain)
   auto multiply_step = [&](int kt, auto&& after) {
     const _Float16* At = lds + (kt & 1) * BUF_HALVES;
-    half8_t af[2][T], bf[2][NMAT][T];
+    half8_t af[FD][T], bf[FD][NMAT][T];
     auto read_frags = [&](int ks, half8_t (&fa)[T], half8_t (&fb)[NMAT][T]) {
 #pragma unroll
       for (int i = 0; i < T; i++)
@@ -400,10 +401,11 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
           fb[mt][j] = *reinterpret_cast<const half8_t*>(At + A_HALVES + mt * B_HALVES + (wn + 32 * j + fr) * LDS_ROW +
                                                         16 * ks + 8 * fg);
     };
-    read_frags(0, af[0], bf[0]);
+#pragma unroll
+    for (int ks = 0; ks < FD - 1; ks++) read_frags(ks, af[ks], bf[ks]);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ks++) {
-      if (ks + 1 < BK / 16) read_frags(ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
+      if (ks + FD - 1 < BK / 16) read_frags(ks + FD - 1, af[(ks + FD - 1) % FD], bf[(ks + FD - 1) % FD]);
 #pragma unroll
       for (int mt = 0; mt < NMAT; mt++)
 #pragma unroll
@@ -414,7 +416,7 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
             // them in vector registers and copies all of them aside and back every K step
             asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0"
                          : "+a"(acc[mt][i][j])
-                         : "v"(af[ks & 1][i]), "v"(bf[ks & 1][mt][j]));
+                         : "v"(af[ks % FD][i]), "v"(bf[ks % FD][mt][j]));
             after(((ks * NMAT + mt) * T + i) * T + j);
           }
     }
