@@ -114,6 +114,29 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const float* __restric
   }
 }
 
+// Per-head RMSNorm of the q rows and the k rows in one launch: one wave per row of head_dim
+// elements (rows q_rows.. are k rows with their own weight).
+__global__ __launch_bounds__(256) void rmsnorm_qk_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                         const void* __restrict__ qw, int qw_f16,
+                                                         const void* __restrict__ kw, int kw_f16,
+                                                         float* __restrict__ q_out, float* __restrict__ k_out, int q_rows,
+                                                         int k_rows, int head_dim, float eps, int w_offset) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= (int64_t)q_rows + k_rows) return;
+  const bool is_q = row < q_rows;
+  const int64_t base = (is_q ? row : row - q_rows) * head_dim;
+  const float* src = (is_q ? q : k) + base;
+  float* dst = (is_q ? q_out : k_out) + base;
+  const void* w = is_q ? qw : kw;
+  const int w_f16 = is_q ? qw_f16 : kw_f16;
+  float ss = 0.f;
+  for (int i = lane; i < head_dim; i += 64) ss = fmaf(src[i], src[i], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)head_dim + eps);
+  for (int i = lane; i < head_dim; i += 64) dst[i] = src[i] * inv * load_norm_weight(w, w_f16, i, w_offset);
+}
+
 // ---------------------------------------------------------------------------------------
 // RoPE in place: one thread per rotated pair.
 // ---------------------------------------------------------------------------------------
@@ -318,6 +341,24 @@ int dh_rmsnorm(const float* d_x, const void* d_weight, int weight_dtype, float* 
     hipLaunchKernelGGL(rmsnorm_kernel, dim3(batch), dim3(256), 0, dh::stream(), DH_RMS_ARGS);
   }
 #undef DH_RMS_ARGS
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_rmsnorm_qk(const float* d_q, const float* d_k, const void* d_q_weight, int q_weight_dtype,
+                  const void* d_k_weight, int k_weight_dtype, float* d_q_out, float* d_k_out, int q_rows,
+                  int k_rows, int head_dim, float eps, int weight_offset) {
+  const char* op = "dh_rmsnorm_qk";
+  DH_REQUIRE_INIT(op);
+  if (q_rows <= 0 || k_rows <= 0 || head_dim <= 0)
+    return dh::fail(1, "[%s] qRows=%d kRows=%d headDim=%d must be positive", op, q_rows, k_rows, head_dim);
+  if (!d_q || !d_k || !d_q_out || !d_k_out || !d_q_weight || !d_k_weight) return dh::fail(1, "[%s] null pointer", op);
+  if ((q_weight_dtype != DH_F32 && q_weight_dtype != DH_F16) || (k_weight_dtype != DH_F32 && k_weight_dtype != DH_F16))
+    return dh::fail(1, "[%s] weight dtype must be f32 or f16", op);
+  const int64_t rows = (int64_t)q_rows + k_rows;
+  hipLaunchKernelGGL(rmsnorm_qk_kernel, dim3((unsigned)dh::ceil_div(rows, 4)), dim3(256), 0, dh::stream(), d_q, d_k,
+                     d_q_weight, q_weight_dtype == DH_F16, d_k_weight, k_weight_dtype == DH_F16, d_q_out, d_k_out,
+                     q_rows, k_rows, head_dim, eps, weight_offset);
   DH_CHECK_LAUNCH(op);
   return 0;
 }

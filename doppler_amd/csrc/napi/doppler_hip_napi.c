@@ -201,6 +201,12 @@ FN(js_rmsnorm) {
   return ret_rc(env, dh_rmsnorm((const float*)x, w, wdt, (float*)o, batch, hid, eps, woff, (const float*)pre,
                                 (const float*)post, (float*)prenorm, oscale));
 }
+FN(js_rmsnorm_qk) {
+  ARGS(13); P(0, q); P(1, k); P(2, qw); I(3, qwdt); P(4, kw); I(5, kwdt); P(6, qo); P(7, ko); I(8, qrows); I(9, krows);
+  I(10, hd); F(11, eps); I(12, woff);
+  return ret_rc(env, dh_rmsnorm_qk((const float*)q, (const float*)k, qw, qwdt, kw, kwdt, (float*)qo, (float*)ko, qrows,
+                                   krows, hd, eps, woff));
+}
 FN(js_rope) {
   ARGS(10); P(0, x); P(1, c); P(2, s); I(3, seq); I(4, heads); I(5, hd); I(6, rd); I(7, span); I(8, inter); I(9, start);
   return ret_rc(env, dh_rope((float*)x, (const float*)c, (const float*)s, seq, heads, hd, rd, span, inter, start));
@@ -253,7 +259,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"attnDecodeWorkspaceBytes", js_attn_decode_workspace_bytes}, {"attnDecode", js_attn_decode},
       {"attnDecodeQkvSupported", js_attn_decode_qkv_supported}, {"attnDecodeQkv", js_attn_decode_qkv},
       {"attnPrefill", js_attn_prefill},
-      {"rmsnorm", js_rmsnorm}, {"rope", js_rope}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},
+      {"rmsnorm", js_rmsnorm}, {"rmsnormQK", js_rmsnorm_qk}, {"rope", js_rope}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},
       {"kvWriteF16", js_kv_write_f16}, {"residualAdd", js_residual_add}, {"gatherF16", js_gather_f16},
       {"actGate", js_act_gate}, {"actGateRowsplit", js_act_gate_rowsplit},
       {"argmaxWorkspaceBytes", js_argmax_workspace_bytes}, {"argmax", js_argmax},

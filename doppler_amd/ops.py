@@ -338,6 +338,45 @@ def runRMSNorm(input, weight, eps, batchSize=1, hiddenSize=None, residual=None, 
     return Tensor(out, "f32", (batchSize, hidden), "rmsnorm_output")
 
 
+def canUseRMSNormQK(qTensor, kTensor, skipKNorm=False):
+    """src/gpu/kernels/rmsnorm-qk.js:29 canUseRMSNormQK (f32 tensors on this path)."""
+    if skipKNorm or qTensor is None or kTensor is None or qTensor.buffer is kTensor.buffer:
+        return False
+    return qTensor.dtype == kTensor.dtype == "f32"
+
+
+def runRMSNormQK(qTensor, kTensor, qWeight, kWeight, eps, numTokens=None, numHeads=None, numKVHeads=None,
+                 headDim=None, rmsNormWeightOffset=False, **_ignored):
+    """src/gpu/kernels/rmsnorm-qk.js:122 runRMSNormQK: per-head RMSNorm of q and k in one launch; returns
+    {"q": Tensor [numTokens*numHeads, headDim], "k": Tensor [numTokens*numKVHeads, headDim]}."""
+    for name, v in (("numTokens", numTokens), ("numHeads", numHeads), ("numKVHeads", numKVHeads), ("headDim", headDim)):
+        if not isinstance(v, (int, np.integer)) or v <= 0:
+            raise DopplerHipError("RMSNorm QK requires a positive integer %s, got %r." % (name, v))
+    if qTensor.dtype != kTensor.dtype:
+        raise DopplerHipError("RMSNorm QK requires matching Q/K dtypes, got %s and %s." % (qTensor.dtype, kTensor.dtype))
+    if qTensor.dtype != "f32":
+        raise DopplerHipError("RMSNorm QK: the HIP path takes f32 tensors, got %s." % qTensor.dtype)
+    q_rows, k_rows = numTokens * numHeads, numTokens * numKVHeads
+    if _nbytes(qTensor) < q_rows * headDim * 4:
+        raise DopplerHipError("RMSNorm QK: Q input buffer smaller than %d bytes" % (q_rows * headDim * 4))
+    if _nbytes(kTensor) < k_rows * headDim * 4:
+        raise DopplerHipError("RMSNorm QK: K input buffer smaller than %d bytes" % (k_rows * headDim * 4))
+    dts = []
+    for name, w in (("q", qWeight), ("k", kWeight)):
+        wd = w.dtype if isinstance(w, (Tensor, WeightBuffer)) else "f32"
+        dt = capi.F16 if wd == "f16" else capi.F32
+        if _nbytes(w) < headDim * (2 if dt == capi.F16 else 4):
+            raise DopplerHipError("RMSNorm QK: %s weight buffer smaller than headDim=%d" % (name, headDim))
+        dts.append(dt)
+    q_out = _out(None, q_rows * padToQ4KBlock(headDim) * 4)
+    k_out = _out(None, k_rows * padToQ4KBlock(headDim) * 4)
+    capi.check(_lib().dh_rmsnorm_qk(_ptr(qTensor), _ptr(kTensor), _ptr(qWeight), dts[0], _ptr(kWeight), dts[1],
+                                    q_out.data_ptr(), k_out.data_ptr(), q_rows, k_rows, headDim, eps,
+                                    int(bool(rmsNormWeightOffset))))
+    return {"q": Tensor(q_out, "f32", (q_rows, headDim), "rmsnorm_qk_q_output"),
+            "k": Tensor(k_out, "f32", (k_rows, headDim), "rmsnorm_qk_k_output")}
+
+
 def runRoPE(input, freqsCos, freqsSin, seqLen, numHeads=1, headDim=64, rotaryDim=None, pairSpanDim=None,
             interleaved=False, startPos=0, **_ignored):
     """src/gpu/kernels/rope.js:108 runRoPE: in place, returns a Tensor aliasing the input."""

@@ -203,6 +203,14 @@ int dh_rmsnorm(const float* d_x, const void* d_weight, int weight_dtype, float* 
                int batch, int hidden, float eps, int weight_offset, const float* d_pre_residual,
                const float* d_post_residual, float* d_prenorm_out, float output_scale);
 
+/* Per-head RMSNorm of q [q_rows, head_dim] and k [k_rows, head_dim] in one launch, each with its
+ * own weight [head_dim] (f32 or f16; 1 + w with weight_offset).  Replaces
+ * runRMSNormQK/recordRMSNormQK, src/gpu/kernels/rmsnorm-qk.js:122-128 (rmsnorm_qk.wgsl:74-118);
+ * q_rows = numTokens * numHeads, k_rows = numTokens * numKVHeads.  Outputs may alias the inputs. */
+int dh_rmsnorm_qk(const float* d_q, const float* d_k, const void* d_q_weight, int q_weight_dtype,
+                  const void* d_k_weight, int k_weight_dtype, float* d_q_out, float* d_k_out,
+                  int q_rows, int k_rows, int head_dim, float eps, int weight_offset);
+
 /* In-place rotary embedding on x[seq][heads][head_dim] with host-built tables
  * cos/sin[max_seq][rotary_dim/2].  Replaces runRoPE/recordRoPE,
  * src/gpu/kernels/rope.js:108-114 (rope.wgsl:63-106). */

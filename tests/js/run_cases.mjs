@@ -77,6 +77,14 @@ async function main() {
       if (c.outputScale) opts.outputScale = c.outputScale;
       const t = await dh.runRMSNorm(tensor(c.x, 'f32', [c.batch, c.hidden]), tensor(c.w, 'f32', [c.hidden]), c.eps, opts);
       await save(out, t.buffer, c.batch * c.hidden * 4);
+    } else if (c.op === 'rmsnorm_qk') {
+      const q = tensor(c.q, 'f32', [c.T * c.heads, c.headDim]);
+      const k = tensor(c.k, 'f32', [c.T * c.kvHeads, c.headDim]);
+      if (!dh.canUseRMSNormQK(q, k) || dh.canUseRMSNormQK(q, q)) throw new Error('canUseRMSNormQK');
+      const r = await dh.runRMSNormQK(q, k, tensor(c.qw, 'f32', [c.headDim]), tensor(c.kw, 'f32', [c.headDim]), c.eps,
+        { numTokens: c.T, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim, rmsNormWeightOffset: true });
+      await save(c.name + '.q.out.bin', r.q.buffer, c.T * c.heads * c.headDim * 4);
+      await save(c.name + '.k.out.bin', r.k.buffer, c.T * c.kvHeads * c.headDim * 4);
     } else if (c.op === 'rope') {
       const x = tensor(c.x, 'f32', [c.seq, c.heads, c.headDim]);
       const t = await dh.runRoPE(x, tensor(c.cos, 'f32', [1]), tensor(c.sin, 'f32', [1]), c.seq,

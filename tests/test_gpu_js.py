@@ -34,7 +34,7 @@ def test_addon_is_built_and_exports_the_op_api():
     out = subprocess.run([NODE, "-e", code], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
     assert out.returncode == 0, out.stderr
     names = set(json.loads(out.stdout))
-    for n in ("runMatmul", "recordMatmul", "runAttention", "recordAttention", "runRMSNorm", "recordRMSNorm", "runRoPE",
+    for n in ("runMatmul", "recordMatmul", "runAttention", "recordAttention", "runRMSNorm", "recordRMSNorm", "runRMSNormQK", "recordRMSNormQK", "canUseRMSNormQK", "runRoPE",
               "recordRoPE", "runKVCacheWriteF32ToF16", "recordKVCacheWriteF32ToF16", "runSplitQKVRMSNormRoPEQK",
               "recordSplitQKVRMSNormRoPEQK", "runSiLU", "recordSiLU", "runSiLURowSplit", "recordSiLURowSplit", "runGeLU",
               "recordGeLU", "runResidualAdd", "recordResidualAdd", "runGather", "recordGather", "runFusedFFN",
@@ -124,6 +124,15 @@ def test_js_host_path_parity(tmp_path):
                       hidden=1152, eps=1e-6, weightOffset=True, outputScale=0.5))
     rms_want = oracle.rmsnorm(x, w, 1e-6, weight_offset=True, post_residual=r, output_scale=0.5)
     checks.append(lambda: rel_l2(get("rms.out.bin", np.float32), rms_want) <= 1e-5)
+
+    qn = synth.normal_f32((2 * 16, 128), 9410, 2.0)
+    kn = synth.normal_f32((2 * 8, 128), 9411, 0.5)
+    qnw, knw = synth.normal_f32(128, 9412, 0.1), synth.normal_f32(128, 9413, 0.1)
+    cases.append(dict(name="rmsqk", op="rmsnorm_qk", q=put("rmsqk.q", qn), k=put("rmsqk.k", kn), qw=put("rmsqk.qw", qnw),
+                      kw=put("rmsqk.kw", knw), T=2, heads=16, kvHeads=8, headDim=128, eps=1e-6))
+    rmsqk_q, rmsqk_k = oracle.rmsnorm(qn, qnw, 1e-6, weight_offset=True), oracle.rmsnorm(kn, knw, 1e-6, weight_offset=True)
+    checks.append(lambda: rel_l2(get("rmsqk.q.out.bin", np.float32), rmsqk_q) <= 1e-5)
+    checks.append(lambda: rel_l2(get("rmsqk.k.out.bin", np.float32), rmsqk_k) <= 1e-5)
 
     cos, sin = synth.rope_tables(128, 64, 1e6)
     xr = synth.normal_f32((2, 16, 128), 9500)

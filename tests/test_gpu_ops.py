@@ -522,6 +522,31 @@ def test_rmsnorm_options(hidden):
     assert rel_l2(got, oracle.rmsnorm(x, w16.astype(np.float32), 1e-6)) <= 1e-5
 
 
+@pytest.mark.parametrize("T,H,Hkv,D,offset", [(3, 16, 8, 128, False), (1, 32, 8, 128, True), (5, 4, 2, 64, False),
+                                              (2, 3, 1, 80, True)])
+def test_rmsnorm_qk_one_launch(T, H, Hkv, D, offset):
+    """Per-head RMSNorm of q and k together (rmsnorm-qk.js): equals the oracle's RMSNorm row by row, f32 and f16 weights."""
+    q = synth.normal_f32((T * H, D), seed=4100 + D, scale=2.0)
+    k = synth.normal_f32((T * Hkv, D), seed=4101 + D, scale=0.5)
+    qw = synth.normal_f32(D, seed=4102, scale=0.1) + (0.0 if offset else 1.0)
+    kw16 = (synth.normal_f32(D, seed=4103, scale=0.1) + (0.0 if offset else 1.0)).astype(np.float16)
+    qt, kt = ops.tensorFromNumpy(q), ops.tensorFromNumpy(k)
+    assert ops.canUseRMSNormQK(qt, kt) and not ops.canUseRMSNormQK(qt, qt) and not ops.canUseRMSNormQK(qt, kt, skipKNorm=True)
+    r = ops.runRMSNormQK(qt, kt, ops.tensorFromNumpy(qw), ops.tensorFromNumpy(kw16.view(np.uint16), "f16"), 1e-6,
+                         numTokens=T, numHeads=H, numKVHeads=Hkv, headDim=D, rmsNormWeightOffset=offset)
+    assert r["q"].shape == (T * H, D) and r["k"].shape == (T * Hkv, D)
+    assert rel_l2(ops.readTensor(r["q"]), oracle.rmsnorm(q, qw, 1e-6, weight_offset=offset)) <= 1e-5
+    assert rel_l2(ops.readTensor(r["k"]), oracle.rmsnorm(k, kw16.astype(np.float32), 1e-6, weight_offset=offset)) <= 1e-5
+    # the inputs are left alone
+    assert np.array_equal(ops.readTensor(qt), q.reshape(-1)) or np.array_equal(ops.readTensor(qt).reshape(q.shape), q)
+    with pytest.raises(DopplerHipError, match="positive integer numHeads"):
+        ops.runRMSNormQK(qt, kt, ops.tensorFromNumpy(qw), ops.tensorFromNumpy(qw), 1e-6, numTokens=T, numHeads=0,
+                         numKVHeads=Hkv, headDim=D)
+    with pytest.raises(DopplerHipError, match="Q input buffer"):
+        ops.runRMSNormQK(qt, kt, ops.tensorFromNumpy(qw), ops.tensorFromNumpy(qw), 1e-6, numTokens=T + 1, numHeads=H,
+                         numKVHeads=Hkv, headDim=D)
+
+
 def test_rope_variants():
     S, H, D, start = 5, 16, 128, 32000
     cos, sin = synth.rope_tables(D, start + S, 1e6)
