@@ -58,6 +58,8 @@ SIGNATURES = {
     "dh_attn_decode_qkv": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _F, _I, _I,
                                 _I, _P]),
     "dh_rmsnorm": (_I, [_P, _P, _I, _P, _I, _I, _F, _I, _P, _P, _P, _F]),
+    "dh_rmsnorm_sandwich_pair": (_I, [_P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _F, _I]),
+    "dh_residual_rmsnorm_pair": (_I, [_P, _P, _P, _I, _P, _P, _I, _I, _F, _I, _F]),
     "dh_rmsnorm_qk": (_I, [_P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _F, _I]),
     "dh_rope": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I]),
     "dh_qkv_norm_rope_kvwrite": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F,

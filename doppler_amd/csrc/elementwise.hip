@@ -114,6 +114,43 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const float* __restric
   }
 }
 
+// Two chained normalisations of a token in one launch, one workgroup per token.
+//   sandwich (mode 0):      post = rmsnorm(x, w_a) (+ residual);  second = rmsnorm(post, w_b)
+//   residual-next (mode 1): post = (x + residual) * scale;        second = rmsnorm(post, w_a)
+// Outputs: first_out = post, second_out = second.  A thread re-reads only what it wrote itself, and
+// first_out may alias x or residual (each element is read before the same thread overwrites it).
+__global__ __launch_bounds__(256) void rmsnorm_pair_kernel(const float* x, const float* residual,
+                                                           const void* __restrict__ wa, int wa_f16,
+                                                           const void* __restrict__ wb, int wb_f16, float* first_out,
+                                                           float* second_out, int hidden, float eps, int w_offset,
+                                                           int mode, float scale) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * hidden;
+  float ss = 0.f;
+  if (mode == 0) {
+    for (int i = threadIdx.x; i < hidden; i += 256) ss = fmaf(x[base + i], x[base + i], ss);
+    const float inv_in = 1.0f / sqrtf(block_sum_256(ss, red) / (float)hidden + eps);
+    ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += 256) {
+      float post = x[base + i] * inv_in * load_norm_weight(wa, wa_f16, i, w_offset);
+      if (residual) post += residual[base + i];
+      first_out[base + i] = post;
+      ss = fmaf(post, post, ss);
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += 256) {
+      const float v = (x[base + i] + residual[base + i]) * scale;
+      first_out[base + i] = v;
+      ss = fmaf(v, v, ss);
+    }
+  }
+  const float inv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)hidden + eps);
+  const void* w2 = mode == 0 ? wb : wa;
+  const int w2_f16 = mode == 0 ? wb_f16 : wa_f16;
+  for (int i = threadIdx.x; i < hidden; i += 256)
+    second_out[base + i] = first_out[base + i] * inv * load_norm_weight(w2, w2_f16, i, w_offset);
+}
+
 // Per-head RMSNorm of the q rows and the k rows in one launch: one wave per row of head_dim
 // elements (rows q_rows.. are k rows with their own weight).
 __global__ __launch_bounds__(256) void rmsnorm_qk_kernel(const float* __restrict__ q, const float* __restrict__ k,
@@ -341,6 +378,44 @@ int dh_rmsnorm(const float* d_x, const void* d_weight, int weight_dtype, float* 
     hipLaunchKernelGGL(rmsnorm_kernel, dim3(batch), dim3(256), 0, dh::stream(), DH_RMS_ARGS);
   }
 #undef DH_RMS_ARGS
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_rmsnorm_sandwich_pair(const float* d_x, const float* d_residual, const void* d_post_weight,
+                             int post_weight_dtype, const void* d_pre_weight, int pre_weight_dtype,
+                             float* d_post_out, float* d_pre_out, int batch, int hidden, float eps,
+                             int weight_offset) {
+  const char* op = "dh_rmsnorm_sandwich_pair";
+  DH_REQUIRE_INIT(op);
+  if (batch <= 0 || hidden <= 0) return dh::fail(1, "[%s] batch=%d hidden=%d must be positive", op, batch, hidden);
+  if (!d_x || !d_post_weight || !d_pre_weight || !d_post_out || !d_pre_out) return dh::fail(1, "[%s] null pointer", op);
+  if ((post_weight_dtype != DH_F32 && post_weight_dtype != DH_F16) ||
+      (pre_weight_dtype != DH_F32 && pre_weight_dtype != DH_F16))
+    return dh::fail(1, "[%s] weight dtype must be f32 or f16", op);
+  if (d_post_out == d_pre_out) return dh::fail(1, "[%s] the two outputs must be different buffers", op);
+  hipLaunchKernelGGL(rmsnorm_pair_kernel, dim3(batch), dim3(256), 0, dh::stream(), d_x, d_residual, d_post_weight,
+                     post_weight_dtype == DH_F16, d_pre_weight, pre_weight_dtype == DH_F16, d_post_out, d_pre_out, hidden,
+                     eps, weight_offset, 0, 1.0f);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_residual_rmsnorm_pair(const float* d_x, const float* d_residual, const void* d_norm_weight,
+                             int norm_weight_dtype, float* d_residual_out, float* d_norm_out, int batch,
+                             int hidden, float eps, int weight_offset, float output_scale) {
+  const char* op = "dh_residual_rmsnorm_pair";
+  DH_REQUIRE_INIT(op);
+  if (batch <= 0 || hidden <= 0) return dh::fail(1, "[%s] batch=%d hidden=%d must be positive", op, batch, hidden);
+  if (!d_x || !d_residual || !d_norm_weight || !d_residual_out || !d_norm_out) return dh::fail(1, "[%s] null pointer", op);
+  if (norm_weight_dtype != DH_F32 && norm_weight_dtype != DH_F16)
+    return dh::fail(1, "[%s] weight dtype must be f32 or f16", op);
+  if (!(output_scale == output_scale) || output_scale > 3.0e38f || output_scale < -3.0e38f)
+    return dh::fail(1, "[residual_rmsnorm_pair] outputScale must be finite");
+  if (d_residual_out == d_norm_out) return dh::fail(1, "[%s] the two outputs must be different buffers", op);
+  hipLaunchKernelGGL(rmsnorm_pair_kernel, dim3(batch), dim3(256), 0, dh::stream(), d_x, d_residual, d_norm_weight,
+                     norm_weight_dtype == DH_F16, nullptr, 0, d_residual_out, d_norm_out, hidden, eps, weight_offset, 1,
+                     output_scale);
   DH_CHECK_LAUNCH(op);
   return 0;
 }

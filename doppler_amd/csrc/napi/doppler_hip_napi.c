@@ -207,6 +207,18 @@ FN(js_rmsnorm_qk) {
   return ret_rc(env, dh_rmsnorm_qk((const float*)q, (const float*)k, qw, qwdt, kw, kwdt, (float*)qo, (float*)ko, qrows,
                                    krows, hd, eps, woff));
 }
+FN(js_rmsnorm_sandwich_pair) {
+  ARGS(12); P(0, x); P(1, r); P(2, pw); I(3, pwdt); P(4, qw); I(5, qwdt); P(6, po); P(7, qo); I(8, batch); I(9, hid);
+  F(10, eps); I(11, woff);
+  return ret_rc(env, dh_rmsnorm_sandwich_pair((const float*)x, (const float*)r, pw, pwdt, qw, qwdt, (float*)po, (float*)qo,
+                                              batch, hid, eps, woff));
+}
+FN(js_residual_rmsnorm_pair) {
+  ARGS(11); P(0, x); P(1, r); P(2, w); I(3, wdt); P(4, ro); P(5, no); I(6, batch); I(7, hid); F(8, eps); I(9, woff);
+  F(10, scale);
+  return ret_rc(env, dh_residual_rmsnorm_pair((const float*)x, (const float*)r, w, wdt, (float*)ro, (float*)no, batch, hid,
+                                              eps, woff, scale));
+}
 FN(js_rope) {
   ARGS(10); P(0, x); P(1, c); P(2, s); I(3, seq); I(4, heads); I(5, hd); I(6, rd); I(7, span); I(8, inter); I(9, start);
   return ret_rc(env, dh_rope((float*)x, (const float*)c, (const float*)s, seq, heads, hd, rd, span, inter, start));
@@ -259,7 +271,8 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"attnDecodeWorkspaceBytes", js_attn_decode_workspace_bytes}, {"attnDecode", js_attn_decode},
       {"attnDecodeQkvSupported", js_attn_decode_qkv_supported}, {"attnDecodeQkv", js_attn_decode_qkv},
       {"attnPrefill", js_attn_prefill},
-      {"rmsnorm", js_rmsnorm}, {"rmsnormQK", js_rmsnorm_qk}, {"rope", js_rope}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},
+      {"rmsnorm", js_rmsnorm}, {"rmsnormQK", js_rmsnorm_qk}, {"rmsnormSandwichPair", js_rmsnorm_sandwich_pair},
+      {"residualRmsnormPair", js_residual_rmsnorm_pair}, {"rope", js_rope}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},
       {"kvWriteF16", js_kv_write_f16}, {"residualAdd", js_residual_add}, {"gatherF16", js_gather_f16},
       {"actGate", js_act_gate}, {"actGateRowsplit", js_act_gate_rowsplit},
       {"argmaxWorkspaceBytes", js_argmax_workspace_bytes}, {"argmax", js_argmax},

@@ -7,6 +7,9 @@ export { runAttention, recordAttention } from './attention.js';
 export { runDecodeAttentionFromQKV, recordDecodeAttentionFromQKV, decodeAttentionFromQKVSupported } from './attention-from-qkv.js';
 export { runRMSNorm, recordRMSNorm } from './rmsnorm.js';
 export { runRMSNormQK, recordRMSNormQK, canUseRMSNormQK } from './rmsnorm-qk.js';
+export {
+  runSandwichRMSNormPair, recordSandwichRMSNormPair, runResidualNextRMSNormPair, recordResidualNextRMSNormPair,
+} from './rmsnorm-pair.js';
 export { runRoPE, recordRoPE } from './rope.js';
 export { runKVCacheWriteF32ToF16, recordKVCacheWriteF32ToF16 } from './kv-cache-write.js';
 export { runSplitQKVRMSNormRoPEQK, recordSplitQKVRMSNormRoPEQK } from './split-qkv-rmsnorm-rope-qk.js';

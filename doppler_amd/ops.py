@@ -338,6 +338,60 @@ def runRMSNorm(input, weight, eps, batchSize=1, hiddenSize=None, residual=None, 
     return Tensor(out, "f32", (batchSize, hidden), "rmsnorm_output")
 
 
+def _norm_weight_dtype(weight, hidden, what):
+    wd = weight.dtype if isinstance(weight, (Tensor, WeightBuffer)) else "f32"
+    dt = capi.F16 if wd == "f16" else capi.F32
+    if _nbytes(weight) < hidden * (2 if dt == capi.F16 else 4):
+        raise DopplerHipError("%s weight buffer smaller than hiddenSize=%d" % (what, hidden))
+    return dt
+
+
+def _pair_inputs(tag, input, residual, hiddenSize):
+    if input.dtype != "f32":
+        raise DopplerHipError('[%s] input dtype must be f32; got "%s".' % (tag, input.dtype))
+    if residual is not None and isinstance(residual, Tensor) and residual.dtype != "f32":
+        raise DopplerHipError('[%s] residual dtype must be f32; got "%s".' % (tag, residual.dtype))
+    hidden = hiddenSize if hiddenSize else input.shape[-1]
+    if not isinstance(hidden, (int, np.integer)) or hidden <= 0:
+        raise DopplerHipError("[%s] hiddenSize must be a positive integer." % tag)
+    return int(hidden)
+
+
+def runSandwichRMSNormPair(input, residual, postWeight, preWeight, eps, batchSize=1, hiddenSize=None,
+                           rmsNormWeightOffset=False, postOutputBuffer=None, preOutputBuffer=None, **_ignored):
+    """src/gpu/kernels/rmsnorm-pair.js:147 runSandwichRMSNormPair: postAttn = residual + rmsnorm(input, postWeight),
+    ffnInput = rmsnorm(postAttn, preWeight), one launch."""
+    hidden = _pair_inputs("rmsnorm_pair", input, residual, hiddenSize)
+    pdt = _norm_weight_dtype(postWeight, hidden, "[rmsnorm_pair] post")
+    qdt = _norm_weight_dtype(preWeight, hidden, "[rmsnorm_pair] pre")
+    nbytes = batchSize * padToQ4KBlock(hidden) * 4
+    post, pre = _out(postOutputBuffer, nbytes), _out(preOutputBuffer, nbytes)
+    capi.check(_lib().dh_rmsnorm_sandwich_pair(_ptr(input), _ptr(residual), _ptr(postWeight), pdt, _ptr(preWeight), qdt,
+                                               post.data_ptr(), pre.data_ptr(), batchSize, hidden, eps,
+                                               int(bool(rmsNormWeightOffset))))
+    return {"postAttn": Tensor(post, "f32", (batchSize, hidden), "rmsnorm_pair_post_output"),
+            "ffnInput": Tensor(pre, "f32", (batchSize, hidden), "rmsnorm_pair_pre_output")}
+
+
+def runResidualNextRMSNormPair(input, residual, normWeight, eps, batchSize=1, hiddenSize=None, rmsNormWeightOffset=False,
+                               residualOutputBuffer=None, normOutputBuffer=None, outputScale=1, **_ignored):
+    """src/gpu/kernels/rmsnorm-pair.js:246 runResidualNextRMSNormPair: residual = (input + residual) * outputScale,
+    nextInput = rmsnorm(residual, normWeight), one launch."""
+    hidden = _pair_inputs("rmsnorm_pair", input, residual, hiddenSize)
+    if residual is None:
+        raise DopplerHipError("[residual_rmsnorm_pair] a residual tensor is required.")
+    scale = float(outputScale)
+    if not math.isfinite(scale):
+        raise DopplerHipError('[residual_rmsnorm_pair] outputScale must be finite; got "%s".' % outputScale)
+    wdt = _norm_weight_dtype(normWeight, hidden, "[residual_rmsnorm_pair] norm")
+    nbytes = batchSize * padToQ4KBlock(hidden) * 4
+    res, nrm = _out(residualOutputBuffer, nbytes), _out(normOutputBuffer, nbytes)
+    capi.check(_lib().dh_residual_rmsnorm_pair(_ptr(input), _ptr(residual), _ptr(normWeight), wdt, res.data_ptr(),
+                                               nrm.data_ptr(), batchSize, hidden, eps, int(bool(rmsNormWeightOffset)), scale))
+    return {"residual": Tensor(res, "f32", (batchSize, hidden), "residual_rmsnorm_pair_residual_output"),
+            "nextInput": Tensor(nrm, "f32", (batchSize, hidden), "residual_rmsnorm_pair_norm_output")}
+
+
 def canUseRMSNormQK(qTensor, kTensor, skipKNorm=False):
     """src/gpu/kernels/rmsnorm-qk.js:29 canUseRMSNormQK (f32 tensors on this path)."""
     if skipKNorm or qTensor is None or kTensor is None or qTensor.buffer is kTensor.buffer:

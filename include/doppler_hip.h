@@ -211,6 +211,22 @@ int dh_rmsnorm_qk(const float* d_q, const float* d_k, const void* d_q_weight, in
                   const void* d_k_weight, int k_weight_dtype, float* d_q_out, float* d_k_out,
                   int q_rows, int k_rows, int head_dim, float eps, int weight_offset);
 
+/* post = rmsnorm(x, post_weight) (+ residual, may be NULL); pre = rmsnorm(post, pre_weight), one
+ * launch.  Replaces runSandwichRMSNormPair/recordSandwichRMSNormPair,
+ * src/gpu/kernels/rmsnorm-pair.js:147-167 (rmsnorm_pair.wgsl:4-5,109-166).  d_post_out may alias
+ * d_x or d_residual (each element is read before it is written); the two outputs must differ. */
+int dh_rmsnorm_sandwich_pair(const float* d_x, const float* d_residual, const void* d_post_weight,
+                             int post_weight_dtype, const void* d_pre_weight, int pre_weight_dtype,
+                             float* d_post_out, float* d_pre_out, int batch, int hidden, float eps,
+                             int weight_offset);
+
+/* residual_out = (x + residual) * output_scale; norm_out = rmsnorm(residual_out, norm_weight), one
+ * launch.  Replaces runResidualNextRMSNormPair/recordResidualNextRMSNormPair,
+ * src/gpu/kernels/rmsnorm-pair.js:246-266 (residual_rmsnorm_pair.wgsl:75-119). */
+int dh_residual_rmsnorm_pair(const float* d_x, const float* d_residual, const void* d_norm_weight,
+                             int norm_weight_dtype, float* d_residual_out, float* d_norm_out, int batch,
+                             int hidden, float eps, int weight_offset, float output_scale);
+
 /* In-place rotary embedding on x[seq][heads][head_dim] with host-built tables
  * cos/sin[max_seq][rotary_dim/2].  Replaces runRoPE/recordRoPE,
  * src/gpu/kernels/rope.js:108-114 (rope.wgsl:63-106). */

@@ -85,6 +85,18 @@ async function main() {
         { numTokens: c.T, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim, rmsNormWeightOffset: true });
       await save(c.name + '.q.out.bin', r.q.buffer, c.T * c.heads * c.headDim * 4);
       await save(c.name + '.k.out.bin', r.k.buffer, c.T * c.kvHeads * c.headDim * 4);
+    } else if (c.op === 'rmsnorm_pair') {
+      const x = tensor(c.x, 'f32', [c.batch, c.hidden]);
+      const r = tensor(c.r, 'f32', [c.batch, c.hidden]);
+      const wa = tensor(c.wa, 'f32', [c.hidden]);
+      const wb = tensor(c.wb, 'f32', [c.hidden]);
+      const opts = { batchSize: c.batch, hiddenSize: c.hidden, rmsNormWeightOffset: true };
+      const s = await dh.runSandwichRMSNormPair(x, r, wa, wb, c.eps, opts);
+      await save(c.name + '.post.out.bin', s.postAttn.buffer, c.batch * c.hidden * 4);
+      await save(c.name + '.pre.out.bin', s.ffnInput.buffer, c.batch * c.hidden * 4);
+      const n = await dh.runResidualNextRMSNormPair(x, r, wa, c.eps, Object.assign({ outputScale: c.outputScale }, opts));
+      await save(c.name + '.res.out.bin', n.residual.buffer, c.batch * c.hidden * 4);
+      await save(c.name + '.next.out.bin', n.nextInput.buffer, c.batch * c.hidden * 4);
     } else if (c.op === 'rope') {
       const x = tensor(c.x, 'f32', [c.seq, c.heads, c.headDim]);
       const t = await dh.runRoPE(x, tensor(c.cos, 'f32', [1]), tensor(c.sin, 'f32', [1]), c.seq,

@@ -34,7 +34,8 @@ def test_addon_is_built_and_exports_the_op_api():
     out = subprocess.run([NODE, "-e", code], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
     assert out.returncode == 0, out.stderr
     names = set(json.loads(out.stdout))
-    for n in ("runMatmul", "recordMatmul", "runAttention", "recordAttention", "runRMSNorm", "recordRMSNorm", "runRMSNormQK", "recordRMSNormQK", "canUseRMSNormQK", "runRoPE",
+    for n in ("runMatmul", "recordMatmul", "runAttention", "recordAttention", "runRMSNorm", "recordRMSNorm", "runRMSNormQK", "recordRMSNormQK", "canUseRMSNormQK", "runSandwichRMSNormPair", "recordSandwichRMSNormPair",
+              "runResidualNextRMSNormPair", "recordResidualNextRMSNormPair", "runRoPE",
               "recordRoPE", "runKVCacheWriteF32ToF16", "recordKVCacheWriteF32ToF16", "runSplitQKVRMSNormRoPEQK",
               "recordSplitQKVRMSNormRoPEQK", "runSiLU", "recordSiLU", "runSiLURowSplit", "recordSiLURowSplit", "runGeLU",
               "recordGeLU", "runResidualAdd", "recordResidualAdd", "runGather", "recordGather", "runFusedFFN",
@@ -133,6 +134,19 @@ def test_js_host_path_parity(tmp_path):
     rmsqk_q, rmsqk_k = oracle.rmsnorm(qn, qnw, 1e-6, weight_offset=True), oracle.rmsnorm(kn, knw, 1e-6, weight_offset=True)
     checks.append(lambda: rel_l2(get("rmsqk.q.out.bin", np.float32), rmsqk_q) <= 1e-5)
     checks.append(lambda: rel_l2(get("rmsqk.k.out.bin", np.float32), rmsqk_k) <= 1e-5)
+
+    px, pr = synth.normal_f32((3, 1152), 9420, 3.0), synth.normal_f32((3, 1152), 9421)
+    pwa, pwb = synth.normal_f32(1152, 9422, 0.1), synth.normal_f32(1152, 9423, 0.1)
+    cases.append(dict(name="pair", op="rmsnorm_pair", x=put("pair.x", px), r=put("pair.r", pr), wa=put("pair.wa", pwa),
+                      wb=put("pair.wb", pwb), batch=3, hidden=1152, eps=1e-6, outputScale=0.5))
+    pair_post = oracle.rmsnorm(px, pwa, 1e-6, weight_offset=True, post_residual=pr)
+    pair_pre = oracle.rmsnorm(pair_post.reshape(3, 1152), pwb, 1e-6, weight_offset=True)
+    pair_res = ((px + pr) * np.float32(0.5)).astype(np.float32)
+    pair_next = oracle.rmsnorm(pair_res, pwa, 1e-6, weight_offset=True)
+    checks.append(lambda: rel_l2(get("pair.post.out.bin", np.float32), pair_post) <= 1e-5)
+    checks.append(lambda: rel_l2(get("pair.pre.out.bin", np.float32), pair_pre) <= 1e-5)
+    checks.append(lambda: np.array_equal(get("pair.res.out.bin", np.float32), pair_res.reshape(-1)))
+    checks.append(lambda: rel_l2(get("pair.next.out.bin", np.float32), pair_next) <= 1e-5)
 
     cos, sin = synth.rope_tables(128, 64, 1e6)
     xr = synth.normal_f32((2, 16, 128), 9500)

@@ -547,6 +547,38 @@ def test_rmsnorm_qk_one_launch(T, H, Hkv, D, offset):
                          numKVHeads=Hkv, headDim=D)
 
 
+@pytest.mark.parametrize("hidden,B,with_residual,offset", [(1152, 3, True, True), (4096, 2, False, False), (100, 5, True, False)])
+def test_rmsnorm_sandwich_pair(hidden, B, with_residual, offset):
+    """rmsnorm-pair.js sandwich form: post = residual + rmsnorm(x, w_post), pre = rmsnorm(post, w_pre)."""
+    x = synth.normal_f32((B, hidden), seed=4200 + hidden, scale=3.0)
+    r = synth.normal_f32((B, hidden), seed=4201)
+    wp = synth.normal_f32(hidden, seed=4202, scale=0.1) + (0.0 if offset else 1.0)
+    wq16 = (synth.normal_f32(hidden, seed=4203, scale=0.1) + (0.0 if offset else 1.0)).astype(np.float16)
+    out = ops.runSandwichRMSNormPair(ops.tensorFromNumpy(x), ops.tensorFromNumpy(r) if with_residual else None,
+                                     ops.tensorFromNumpy(wp), ops.tensorFromNumpy(wq16.view(np.uint16), "f16"), 1e-6,
+                                     batchSize=B, hiddenSize=hidden, rmsNormWeightOffset=offset)
+    want_post = oracle.rmsnorm(x, wp, 1e-6, weight_offset=offset, post_residual=r if with_residual else None)
+    want_pre = oracle.rmsnorm(want_post.reshape(B, hidden), wq16.astype(np.float32), 1e-6, weight_offset=offset)
+    assert rel_l2(ops.readTensor(out["postAttn"]), want_post) <= 1e-5
+    assert rel_l2(ops.readTensor(out["ffnInput"]), want_pre) <= 1e-5
+
+
+@pytest.mark.parametrize("hidden,B,scale", [(1152, 3, 1.0), (4096, 1, 0.5), (100, 4, 2.0)])
+def test_residual_next_rmsnorm_pair(hidden, B, scale):
+    """rmsnorm-pair.js residual-next form: residual = (x + r) * scale (bit exact), next = rmsnorm(residual, w)."""
+    x = synth.normal_f32((B, hidden), seed=4300 + hidden, scale=2.0)
+    r = synth.normal_f32((B, hidden), seed=4301)
+    w = synth.normal_f32(hidden, seed=4302, scale=0.1)
+    out = ops.runResidualNextRMSNormPair(ops.tensorFromNumpy(x), ops.tensorFromNumpy(r), ops.tensorFromNumpy(w), 1e-6,
+                                         batchSize=B, hiddenSize=hidden, rmsNormWeightOffset=True, outputScale=scale)
+    want_res = ((x + r) * np.float32(scale)).astype(np.float32)
+    assert np.array_equal(ops.readTensor(out["residual"]).reshape(B, hidden), want_res)
+    assert rel_l2(ops.readTensor(out["nextInput"]), oracle.rmsnorm(want_res, w, 1e-6, weight_offset=True)) <= 1e-5
+    with pytest.raises(DopplerHipError, match="outputScale must be finite"):
+        ops.runResidualNextRMSNormPair(ops.tensorFromNumpy(x), ops.tensorFromNumpy(r), ops.tensorFromNumpy(w), 1e-6,
+                                       batchSize=B, hiddenSize=hidden, outputScale=float("inf"))
+
+
 def test_rope_variants():
     S, H, D, start = 5, 16, 128, 32000
     cos, sin = synth.rope_tables(D, start + S, 1e6)
