@@ -62,6 +62,7 @@ SIGNATURES = {
     "dh_residual_rmsnorm_pair": (_I, [_P, _P, _P, _I, _P, _P, _I, _I, _F, _I, _F]),
     "dh_rmsnorm_qk": (_I, [_P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _F, _I]),
     "dh_rope": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I]),
+    "dh_rope_qk": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I]),
     "dh_qkv_norm_rope_kvwrite": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F,
                                       _I, _I64, _I]),
     "dh_kv_write_f16": (_I, [_P, _P, _P, _P, _I64, _I64, _I64]),

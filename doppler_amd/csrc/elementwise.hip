@@ -196,6 +196,30 @@ __global__ __launch_bounds__(256) void rope_kernel(float* __restrict__ x, const 
   row[i1] = x0 * s + x1 * c;
 }
 
+// RoPE in place on separate q [seq][q_heads][head_dim] and k [seq][kv_heads][head_dim] buffers in one
+// launch: pairs 0 .. q_pairs-1 belong to q, the rest to k; both read the same tables.
+__global__ __launch_bounds__(256) void rope_qk_kernel(float* __restrict__ q, float* __restrict__ k,
+                                                      const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                      int64_t q_pairs, int64_t total_pairs, int q_heads, int kv_heads,
+                                                      int head_dim, int half, int partner, int interleaved,
+                                                      int start_pos) {
+  int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total_pairs) return;
+  const bool is_k = idx >= q_pairs;
+  if (is_k) idx -= q_pairs;
+  const int heads = is_k ? kv_heads : q_heads;
+  const int pair = (int)(idx % half);
+  const int64_t th = idx / half;  // token * heads + head
+  const int64_t pos = start_pos + th / heads;
+  const float c = cos_t[pos * half + pair], s = sin_t[pos * half + pair];
+  float* row = (is_k ? k : q) + th * head_dim;
+  const int i0 = interleaved ? 2 * pair : pair;
+  const int i1 = interleaved ? 2 * pair + 1 : pair + partner;
+  const float x0 = row[i0], x1 = row[i1];
+  row[i0] = x0 * c - x1 * s;
+  row[i1] = x0 * s + x1 * c;
+}
+
 // ---------------------------------------------------------------------------------------
 // Fused split-QKV + per-head RMSNorm + RoPE + f16 KV write.  One wave per (token, head)
 // row for Q and K rows; the trailing workgroups narrow V.  D <= 512.
@@ -457,6 +481,37 @@ int dh_rope(float* d_x, const float* d_cos, const float* d_sin, int seq, int hea
   const int64_t pairs = (int64_t)seq * heads * half;
   hipLaunchKernelGGL(rope_kernel, dim3(grid_for(pairs)), dim3(256), 0, dh::stream(), d_x, d_cos, d_sin,
                      pairs, heads, head_dim, half, pair_span_dim / 2, interleaved, start_pos);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_rope_qk(float* d_q, float* d_k, const float* d_cos, const float* d_sin, int seq, int q_heads, int kv_heads,
+               int head_dim, int rotary_dim, int pair_span_dim, int interleaved, int start_pos) {
+  const char* op = "dh_rope_qk";
+  DH_REQUIRE_INIT(op);
+  if (seq < 0) return dh::fail(1, "RoPE QK requires seqLen to be a non-negative integer.");
+  if (start_pos < 0) return dh::fail(1, "RoPE QK requires startPos to be a non-negative integer.");
+  if (q_heads <= 0) return dh::fail(1, "RoPE QK requires numQHeads to be a positive integer.");
+  if (kv_heads <= 0) return dh::fail(1, "RoPE QK requires numKVHeads to be a positive integer.");
+  if (head_dim <= 0) return dh::fail(1, "RoPE QK requires headDim to be a positive integer.");
+  if (head_dim % 2) return dh::fail(1, "RoPE QK headDim must be even, got %d.", head_dim);
+  if (rotary_dim <= 0) return dh::fail(1, "RoPE QK requires rotaryDim to be a positive integer.");
+  if (rotary_dim % 2) return dh::fail(1, "RoPE QK rotaryDim must be even, got %d.", rotary_dim);
+  if (rotary_dim > head_dim)
+    return dh::fail(1, "RoPE QK rotaryDim must be <= headDim; got %d for headDim %d.", rotary_dim, head_dim);
+  if (pair_span_dim <= 0) return dh::fail(1, "RoPE QK requires pairSpanDim to be a positive integer.");
+  if (pair_span_dim % 2) return dh::fail(1, "RoPE QK pairSpanDim must be even, got %d.", pair_span_dim);
+  if (pair_span_dim < rotary_dim || pair_span_dim > head_dim)
+    return dh::fail(1, "RoPE QK pairSpanDim must be in [rotaryDim, headDim]; got %d for rotaryDim %d and headDim %d.",
+                    pair_span_dim, rotary_dim, head_dim);
+  if (seq == 0) return 0;
+  if (!d_q || !d_k || !d_cos || !d_sin) return dh::fail(1, "[%s] null pointer", op);
+  if (d_q == d_k) return dh::fail(1, "[%s] q and k must be different buffers", op);
+  const int half = rotary_dim / 2;
+  const int64_t q_pairs = (int64_t)seq * q_heads * half;
+  const int64_t total = q_pairs + (int64_t)seq * kv_heads * half;
+  hipLaunchKernelGGL(rope_qk_kernel, dim3(grid_for(total)), dim3(256), 0, dh::stream(), d_q, d_k, d_cos, d_sin, q_pairs,
+                     total, q_heads, kv_heads, head_dim, half, pair_span_dim / 2, interleaved, start_pos);
   DH_CHECK_LAUNCH(op);
   return 0;
 }

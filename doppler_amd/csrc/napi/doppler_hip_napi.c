@@ -223,6 +223,12 @@ FN(js_rope) {
   ARGS(10); P(0, x); P(1, c); P(2, s); I(3, seq); I(4, heads); I(5, hd); I(6, rd); I(7, span); I(8, inter); I(9, start);
   return ret_rc(env, dh_rope((float*)x, (const float*)c, (const float*)s, seq, heads, hd, rd, span, inter, start));
 }
+FN(js_rope_qk) {
+  ARGS(12); P(0, q); P(1, k); P(2, c); P(3, s); I(4, seq); I(5, qh); I(6, kvh); I(7, hd); I(8, rd); I(9, span); I(10, inter);
+  I(11, start);
+  return ret_rc(env, dh_rope_qk((float*)q, (float*)k, (const float*)c, (const float*)s, seq, qh, kvh, hd, rd, span, inter,
+                                start));
+}
 FN(js_qkv_norm_rope_kvwrite) {
   ARGS(19); P(0, qkv); P(1, qw); P(2, kw); P(3, c); P(4, s); P(5, qo); P(6, ck); P(7, cv); I(8, T); I(9, H); I(10, Hkv);
   I(11, D); I(12, start); I(13, rd); I(14, inter); F(15, eps); I(16, woff); L(17, dst); I(18, useNorm);
@@ -272,7 +278,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"attnDecodeQkvSupported", js_attn_decode_qkv_supported}, {"attnDecodeQkv", js_attn_decode_qkv},
       {"attnPrefill", js_attn_prefill},
       {"rmsnorm", js_rmsnorm}, {"rmsnormQK", js_rmsnorm_qk}, {"rmsnormSandwichPair", js_rmsnorm_sandwich_pair},
-      {"residualRmsnormPair", js_residual_rmsnorm_pair}, {"rope", js_rope}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},
+      {"residualRmsnormPair", js_residual_rmsnorm_pair}, {"rope", js_rope}, {"ropeQK", js_rope_qk}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},
       {"kvWriteF16", js_kv_write_f16}, {"residualAdd", js_residual_add}, {"gatherF16", js_gather_f16},
       {"actGate", js_act_gate}, {"actGateRowsplit", js_act_gate_rowsplit},
       {"argmaxWorkspaceBytes", js_argmax_workspace_bytes}, {"argmax", js_argmax},

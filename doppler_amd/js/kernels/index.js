@@ -11,6 +11,7 @@ export {
   runSandwichRMSNormPair, recordSandwichRMSNormPair, runResidualNextRMSNormPair, recordResidualNextRMSNormPair,
 } from './rmsnorm-pair.js';
 export { runRoPE, recordRoPE } from './rope.js';
+export { runRoPEQK, recordRoPEQK, canUseRoPEQK } from './rope-qk.js';
 export { runKVCacheWriteF32ToF16, recordKVCacheWriteF32ToF16 } from './kv-cache-write.js';
 export { runSplitQKVRMSNormRoPEQK, recordSplitQKVRMSNormRoPEQK } from './split-qkv-rmsnorm-rope-qk.js';
 export { runSiLU, recordSiLU, runSiLURowSplit, recordSiLURowSplit } from './silu.js';

@@ -446,6 +446,45 @@ def runRoPE(input, freqsCos, freqsSin, seqLen, numHeads=1, headDim=64, rotaryDim
     return Tensor(input.buffer, input.dtype, input.shape, "rope_output")
 
 
+def canUseRoPEQK(qTensor, kTensor, reusesSharedKV=False, **_ignored):
+    """src/gpu/kernels/rope-qk.js:56-64 canUseRoPEQK (the HIP kernel rotates f32 activations only)."""
+    if reusesSharedKV or qTensor is None or kTensor is None or qTensor.buffer is kTensor.buffer:
+        return False
+    return qTensor.dtype == "f32" and kTensor.dtype == "f32"
+
+
+def runRoPEQK(qTensor, kTensor, freqsCos, freqsSin, seqLen, numQHeads=None, numKVHeads=None, headDim=None,
+              rotaryDim=None, pairSpanDim=None, interleaved=False, startPos=0, **_ignored):
+    """src/gpu/kernels/rope-qk.js:136 runRoPEQK: q and k rotated in place by one launch; returns Tensors
+    aliasing the inputs."""
+    rotaryDim = headDim if rotaryDim is None else rotaryDim
+    pairSpanDim = rotaryDim if pairSpanDim is None else pairSpanDim
+    for label, v, low, kind in (("seqLen", seqLen, 0, "non-negative"), ("startPos", startPos, 0, "non-negative"),
+                                ("numQHeads", numQHeads, 1, "positive"), ("numKVHeads", numKVHeads, 1, "positive"),
+                                ("headDim", headDim, 1, "positive"), ("rotaryDim", rotaryDim, 1, "positive"),
+                                ("pairSpanDim", pairSpanDim, 1, "positive")):
+        if not isinstance(v, (int, np.integer)) or isinstance(v, bool) or v < low:
+            raise DopplerHipError("RoPE QK requires %s to be a %s integer." % (label, kind))
+    if qTensor.dtype != kTensor.dtype:
+        raise DopplerHipError("RoPE QK requires matching Q/K dtypes, got %s and %s." % (qTensor.dtype, kTensor.dtype))
+    if qTensor.dtype != "f32":
+        raise DopplerHipError("RoPE QK on the HIP path takes f32 tensors, got %s." % qTensor.dtype)
+    result = {"q": Tensor(qTensor.buffer, qTensor.dtype, qTensor.shape, "rope_q_output"),
+              "k": Tensor(kTensor.buffer, kTensor.dtype, kTensor.shape, "rope_k_output")}
+    if seqLen == 0:
+        return result
+    table = (startPos + seqLen) * (rotaryDim // 2) * 4
+    for buf, need, label in ((qTensor, seqLen * numQHeads * headDim * 4, "Q input"),
+                             (kTensor, seqLen * numKVHeads * headDim * 4, "K input"),
+                             (freqsCos, table, "cos frequencies"), (freqsSin, table, "sin frequencies")):
+        if need > _nbytes(buf):
+            raise DopplerHipError("RoPE QK %s buffer is smaller than requested range (%d > %d bytes)."
+                                  % (label, need, _nbytes(buf)))
+    capi.check(_lib().dh_rope_qk(_ptr(qTensor), _ptr(kTensor), _ptr(freqsCos), _ptr(freqsSin), seqLen, numQHeads,
+                                 numKVHeads, headDim, rotaryDim, pairSpanDim, int(bool(interleaved)), startPos))
+    return result
+
+
 def runKVCacheWriteF32ToF16(keys, values, outputKeys, outputValues, srcOffset=0, dstOffset=0, elementCount=None):
     """src/gpu/kernels/kv-cache-write.js:107 runKVCacheWriteF32ToF16."""
     for name, v in (("srcOffset", srcOffset), ("dstOffset", dstOffset), ("elementCount", elementCount)):

@@ -233,6 +233,12 @@ int dh_residual_rmsnorm_pair(const float* d_x, const float* d_residual, const vo
 int dh_rope(float* d_x, const float* d_cos, const float* d_sin, int seq, int heads,
             int head_dim, int rotary_dim, int pair_span_dim, int interleaved, int start_pos);
 
+/* In-place rotary embedding of q[seq][q_heads][head_dim] and k[seq][kv_heads][head_dim] in one
+ * launch, same tables and pairing rules as dh_rope; seq == 0 is a no-op.  Replaces
+ * runRoPEQK/recordRoPEQK, src/gpu/kernels/rope-qk.js:67-143 (rope_qk.wgsl:41-95). */
+int dh_rope_qk(float* d_q, float* d_k, const float* d_cos, const float* d_sin, int seq, int q_heads, int kv_heads,
+               int head_dim, int rotary_dim, int pair_span_dim, int interleaved, int start_pos);
+
 /* From fused qkv[T][(H+2Hkv)*D]: per-head RMSNorm (q/k weights) -> RoPE -> Q out f32,
  * K and V narrowed to f16 straight into the caches at element kv_dst_offset.  Replaces
  * recordSplitQKVRMSNormRoPEQK with f16KVCacheWrite,

@@ -103,6 +103,15 @@ async function main() {
         { numHeads: c.heads, headDim: c.headDim, startPos: c.startPos, interleaved: c.interleaved });
       if (t.buffer !== x.buffer) throw new Error('runRoPE must alias its input');
       await save(out, t.buffer, c.seq * c.heads * c.headDim * 4);
+    } else if (c.op === 'rope_qk') {
+      const q = tensor(c.q, 'f32', [c.seq, c.heads, c.headDim]);
+      const k = tensor(c.k, 'f32', [c.seq, c.kvHeads, c.headDim]);
+      if (!dh.canUseRoPEQK(q, k) || dh.canUseRoPEQK(q, q)) throw new Error('canUseRoPEQK');
+      const r = await dh.runRoPEQK(q, k, tensor(c.cos, 'f32', [1]), tensor(c.sin, 'f32', [1]), c.seq,
+        { numQHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim, startPos: c.startPos });
+      if (r.q.buffer !== q.buffer || r.k.buffer !== k.buffer) throw new Error('runRoPEQK must alias its inputs');
+      await save(c.name + '.q.out.bin', r.q.buffer, c.seq * c.heads * c.headDim * 4);
+      await save(c.name + '.k.out.bin', r.k.buffer, c.seq * c.kvHeads * c.headDim * 4);
     } else if (c.op === 'split_qkv') {
       const ck = dh.acquireBuffer(c.maxSeq * c.kvHeads * c.headDim * 2);
       const cv = dh.acquireBuffer(c.maxSeq * c.kvHeads * c.headDim * 2);
@@ -212,6 +221,7 @@ async function main() {
     await expectThrow(results, 'asmall', 'A buffer too small', () => dh.runMatmul(A, W, 2, 8, 256, { outputDtype: 'f32' }));
     await expectThrow(results, 'bdtype', 'B dtype is required', () => dh.runMatmul(A, W.buffer, 1, 8, 256, { outputDtype: 'f32' }));
     await expectThrow(results, 'offsets', '256-byte aligned', () => dh.runMatmul(A, W, 1, 8, 256, { outputDtype: 'f32', aOffset: 4 }));
+    await expectThrow(results, 'rope_qk', 'RoPE QK rotaryDim must be even', () => dh.runRoPEQK(A, dh.createTensor(dh.acquireBuffer(1024), 'f32', [1, 256], 'b'), A, A, 1, { numQHeads: 1, numKVHeads: 1, headDim: 64, rotaryDim: 31 }));
     await expectThrow(results, 'rope', 'rotaryDim must be even', () => dh.runRoPE(A, A, A, 1, { numHeads: 1, headDim: 64, rotaryDim: 31 }));
     await expectThrow(results, 'gather', 'embeddingDtype is required', () => dh.runGather(A.buffer, A.buffer, 1, 8, 8, {}));
     await expectThrow(results, 'kvwrite', 'smaller than requested range', () => dh.runKVCacheWriteF32ToF16(A.buffer, A.buffer, A.buffer, A.buffer, { elementCount: 100000 }));

@@ -599,6 +599,38 @@ def test_rope_variants():
         ops.runRoPE(xt, ct, st, S, numHeads=H, headDim=D, rotaryDim=31)
 
 
+def test_rope_qk_one_launch_equals_two_single_buffer_calls():
+    """rope-qk.js: q and k rotated by one launch; bit-identical to runRoPE on each buffer, oracle-close."""
+    S, H, Hkv, D, start = 3, 16, 8, 128, 2047
+    cos, sin = synth.rope_tables(D, start + S, 1e6)
+    c32, s32 = synth.rope_tables(32, start + S, 1e4)
+    q, k = synth.normal_f32((S, H, D), seed=4150), synth.normal_f32((S, Hkv, D), seed=4151)
+    for tables, kw in (((cos, sin), {}), ((cos, sin), {"interleaved": True}),
+                       ((c32, s32), {"rotaryDim": 32, "pairSpanDim": 128})):
+        ct, st = ops.tensorFromNumpy(tables[0]), ops.tensorFromNumpy(tables[1])
+        qt, kt = ops.tensorFromNumpy(q), ops.tensorFromNumpy(k)
+        assert ops.canUseRoPEQK(qt, kt) and not ops.canUseRoPEQK(qt, qt)
+        out = ops.runRoPEQK(qt, kt, ct, st, S, numQHeads=H, numKVHeads=Hkv, headDim=D, startPos=start, **kw)
+        assert out["q"].buffer is qt.buffer and out["k"].buffer is kt.buffer
+        one_q = ops.readTensor(ops.runRoPE(ops.tensorFromNumpy(q), ct, st, S, numHeads=H, headDim=D, startPos=start, **kw))
+        one_k = ops.readTensor(ops.runRoPE(ops.tensorFromNumpy(k), ct, st, S, numHeads=Hkv, headDim=D, startPos=start, **kw))
+        assert np.array_equal(ops.readTensor(out["q"]), one_q) and np.array_equal(ops.readTensor(out["k"]), one_k)
+        okw = {"interleaved": kw.get("interleaved", False)}
+        if "rotaryDim" in kw:
+            okw.update(rotary_dim=32, pair_span_dim=128)
+        assert rel_l2(ops.readTensor(out["q"]), oracle.rope_apply(q, tables[0], tables[1], S, H, D, start, **okw)) <= 1e-6
+        assert rel_l2(ops.readTensor(out["k"]), oracle.rope_apply(k, tables[0], tables[1], S, Hkv, D, start, **okw)) <= 1e-6
+    qt, kt = ops.tensorFromNumpy(q), ops.tensorFromNumpy(k)
+    ops.runRoPEQK(qt, kt, ct, st, 0, numQHeads=H, numKVHeads=Hkv, headDim=D)       # seqLen 0: nothing is touched
+    assert np.array_equal(ops.readTensor(qt).reshape(q.shape), q)
+    with pytest.raises(DopplerHipError, match="pairSpanDim must be in"):
+        ops.runRoPEQK(qt, kt, ct, st, S, numQHeads=H, numKVHeads=Hkv, headDim=D, rotaryDim=64, pairSpanDim=32)
+    with pytest.raises(DopplerHipError, match="numKVHeads to be a positive integer"):
+        ops.runRoPEQK(qt, kt, ct, st, S, numQHeads=H, numKVHeads=0, headDim=D)
+    with pytest.raises(DopplerHipError, match="cos frequencies buffer is smaller"):
+        ops.runRoPEQK(qt, kt, ct, st, S, numQHeads=H, numKVHeads=Hkv, headDim=D, startPos=start + 1)
+
+
 def test_kv_cache_write_bit_exact():
     n = 8 * 128 * 3
     k = synth.normal_f32(n + 64, seed=4200)
