@@ -67,6 +67,8 @@ SIGNATURES = {
                                       _I, _I64, _I]),
     "dh_kv_write_f16": (_I, [_P, _P, _P, _P, _I64, _I64, _I64]),
     "dh_residual_add": (_I, [_P, _P, _P, _I64, _F]),
+    "dh_bias_add": (_I, [_P, _P, _I, _I64, _I, _I64, _I64]),
+    "dh_scale": (_I, [_P, _P, _I64, _F]),
     "dh_gather_f16": (_I, [_P, _P, _P, _I, _I, _I, _I]),
     "dh_act_gate": (_I, [_P, _P, _P, _I64, _I, _F]),
     "dh_act_gate_rowsplit": (_I, [_P, _P, _I, _I, _I, _F]),

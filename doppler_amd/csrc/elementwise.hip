@@ -314,6 +314,22 @@ __global__ __launch_bounds__(256) void residual_kernel(const float* __restrict__
   if (i < n) out[i] = (a[i] + b[i]) * scale;
 }
 
+// data[t][d] += bias[d] in place; bias is f32 or f16.
+__global__ __launch_bounds__(256) void bias_add_kernel(float* __restrict__ data, const void* __restrict__ bias,
+                                                       int bias_f16, int64_t total, int dim) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int d = (int)(i % dim);
+  const float b = bias_f16 ? __half2float(((const __half*)bias)[d]) : ((const float*)bias)[d];
+  data[i] += b;
+}
+
+// out = in * scale; out may be the input itself.
+__global__ __launch_bounds__(256) void scale_kernel(const float* in, float* out, int64_t n, float scale) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = in[i] * scale;
+}
+
 __global__ __launch_bounds__(256) void gather_f16_kernel(const uint32_t* __restrict__ ids,
                                                          const __half* __restrict__ table,
                                                          float* __restrict__ out, int64_t total, int hidden,
@@ -569,6 +585,38 @@ int dh_residual_add(const float* d_a, const float* d_b, float* d_out, int64_t n,
   if (!(scale == scale) || scale > 3.0e38f || scale < -3.0e38f)
     return dh::fail(1, "[Residual] outputScale must be finite");
   hipLaunchKernelGGL(residual_kernel, dim3(grid_for(n)), dim3(256), 0, dh::stream(), d_a, d_b, d_out, n, scale);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_bias_add(float* d_data, const void* d_bias, int bias_dtype, int64_t num_tokens, int dim,
+                int64_t data_offset_bytes, int64_t bias_offset_bytes) {
+  const char* op = "dh_bias_add";
+  DH_REQUIRE_INIT(op);
+  if (num_tokens < 0 || dim <= 0)
+    return dh::fail(1, "[%s] numTokens=%lld dim=%d: need numTokens >= 0 and dim > 0", op, (long long)num_tokens, dim);
+  if (bias_dtype != DH_F32 && bias_dtype != DH_F16) return dh::fail(1, "[%s] bias dtype must be f32 or f16", op);
+  const int64_t bias_elem = bias_dtype == DH_F16 ? 2 : 4;
+  if (data_offset_bytes < 0 || data_offset_bytes % 4 || bias_offset_bytes < 0 || bias_offset_bytes % bias_elem)
+    return dh::fail(1, "[%s] dataOffset=%lld / biasOffset=%lld must be non-negative multiples of the element size", op,
+                    (long long)data_offset_bytes, (long long)bias_offset_bytes);
+  if (num_tokens == 0) return 0;
+  if (!d_data || !d_bias) return dh::fail(1, "[%s] null pointer", op);
+  const int64_t total = num_tokens * dim;
+  hipLaunchKernelGGL(bias_add_kernel, dim3(grid_for(total)), dim3(256), 0, dh::stream(),
+                     (float*)((char*)d_data + data_offset_bytes), (const void*)((const char*)d_bias + bias_offset_bytes),
+                     bias_dtype == DH_F16, total, dim);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_scale(const float* d_in, float* d_out, int64_t n, float scale) {
+  const char* op = "dh_scale";
+  DH_REQUIRE_INIT(op);
+  if (n < 0) return dh::fail(1, "[%s] count must be non-negative", op);
+  if (n == 0) return 0;
+  if (!d_in || !d_out) return dh::fail(1, "[%s] null pointer", op);
+  hipLaunchKernelGGL(scale_kernel, dim3(grid_for(n)), dim3(256), 0, dh::stream(), d_in, d_out, n, scale);
   DH_CHECK_LAUNCH(op);
   return 0;
 }

@@ -585,6 +585,35 @@ def runResidualAdd(a, b, size, outputBuffer=None, outputScale=None, **_ignored):
     return Tensor(out, "f32", (size,), "residual_output")
 
 
+def runBiasAdd(data, bias, numTokens, dim, dataOffset=0, biasOffset=0, **_ignored):
+    """src/gpu/kernels/residual.js:218 runBiasAdd: data[t, :] += bias in place (offsets in bytes); the returned
+    Tensor aliases data.  The bias may be f32 or f16 and is widened on the fly."""
+    if data.dtype != "f32":
+        raise DopplerHipError("[BiasAdd] the HIP path takes f32 data, got %s." % data.dtype)
+    bias_dtype = getattr(bias, "dtype", "f32")
+    if bias_dtype not in ("f32", "f16"):
+        raise DopplerHipError("[BiasAdd] bias dtype must be f32 or f16, got %s." % bias_dtype)
+    if dataOffset + numTokens * dim * 4 > _nbytes(data):
+        raise DopplerHipError("[BiasAdd] data buffer is smaller than numTokens=%d x dim=%d at offset %d."
+                              % (numTokens, dim, dataOffset))
+    if biasOffset + dim * (2 if bias_dtype == "f16" else 4) > _nbytes(bias):
+        raise DopplerHipError("[BiasAdd] bias buffer is smaller than dim=%d at offset %d." % (dim, biasOffset))
+    capi.check(_lib().dh_bias_add(_ptr(data), _ptr(bias), capi.F16 if bias_dtype == "f16" else capi.F32, numTokens, dim, dataOffset, biasOffset))
+    return Tensor(data.buffer, data.dtype, (numTokens, dim), "bias_add_output")
+
+
+def runScale(input, scale, count=None, outputBuffer=None, inplace=False, **_ignored):
+    """src/gpu/kernels/scale.js:44 runScale: out = input * scale, into a new buffer, outputBuffer or in place."""
+    if input.dtype != "f32":
+        raise DopplerHipError("[Scale] the HIP path takes f32 tensors, got %s." % input.dtype)
+    n = _nbytes(input) // 4 if count is None else count
+    if n * 4 > _nbytes(input):
+        raise DopplerHipError("[Scale] count=%d exceeds the input buffer." % n)
+    out = input.buffer if inplace else _out(outputBuffer, n * 4)
+    capi.check(_lib().dh_scale(_ptr(input), _ptr(out), n, float(scale)))
+    return Tensor(out, input.dtype, input.shape, "scale_output")
+
+
 def runGather(indices, embeddings, numTokens, hiddenSize, vocabSize, outputBuffer=None, embeddingDtype=None,
               outputDtype=None, transpose=False, indexOffset=0, **_ignored):
     """src/gpu/kernels/gather.js:370 runGather for f16 tables -> f32 rows."""

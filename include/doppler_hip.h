@@ -263,6 +263,16 @@ int dh_kv_write_f16(const float* d_k, const float* d_v, void* d_cache_k, void* d
  * (residual.wgsl:24-31). */
 int dh_residual_add(const float* d_a, const float* d_b, float* d_out, int64_t n, float scale);
 
+/* data[t][d] += bias[d] in place for t < num_tokens, d < dim; the byte offsets select the start
+ * inside each buffer; bias is DH_F32 or DH_F16.  Replaces runBiasAdd/recordBiasAdd,
+ * src/gpu/kernels/residual.js:165-224 (bias_add.wgsl:27-39). */
+int dh_bias_add(float* d_data, const void* d_bias, int bias_dtype, int64_t num_tokens, int dim,
+                int64_t data_offset_bytes, int64_t bias_offset_bytes);
+
+/* out = in * scale over n elements; d_out may equal d_in (the reference's inplace variant).
+ * Replaces runScale/recordScale, src/gpu/kernels/scale.js:13-46. */
+int dh_scale(const float* d_in, float* d_out, int64_t n, float scale);
+
 /* out[t,:] = f32(E[ids[t + index_offset], :]) (zero row when the id is outside the
  * vocabulary).  Replaces runGather for f16 tables, src/gpu/kernels/gather.js:370-391
  * (gather_f16.wgsl:35-66). */

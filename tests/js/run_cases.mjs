@@ -112,6 +112,13 @@ async function main() {
       if (r.q.buffer !== q.buffer || r.k.buffer !== k.buffer) throw new Error('runRoPEQK must alias its inputs');
       await save(c.name + '.q.out.bin', r.q.buffer, c.seq * c.heads * c.headDim * 4);
       await save(c.name + '.k.out.bin', r.k.buffer, c.seq * c.kvHeads * c.headDim * 4);
+    } else if (c.op === 'bias_scale') {
+      const x = tensor(c.x, 'f32', [c.tokens, c.dim]);
+      const b = await dh.runBiasAdd(x, tensor(c.bias, 'f32', [2, c.dim]), c.tokens, c.dim, { biasOffset: c.dim * 4 });
+      if (b.buffer !== x.buffer) throw new Error('runBiasAdd must alias its data');
+      const s = await dh.runScale(b, c.scale);
+      await save(c.name + '.bias.out.bin', b.buffer, c.tokens * c.dim * 4);
+      await save(c.name + '.scale.out.bin', s.buffer, c.tokens * c.dim * 4);
     } else if (c.op === 'split_qkv') {
       const ck = dh.acquireBuffer(c.maxSeq * c.kvHeads * c.headDim * 2);
       const cv = dh.acquireBuffer(c.maxSeq * c.kvHeads * c.headDim * 2);

@@ -35,7 +35,7 @@ def test_addon_is_built_and_exports_the_op_api():
     assert out.returncode == 0, out.stderr
     names = set(json.loads(out.stdout))
     for n in ("runMatmul", "recordMatmul", "runAttention", "recordAttention", "runRMSNorm", "recordRMSNorm", "runRMSNormQK", "recordRMSNormQK", "canUseRMSNormQK", "runSandwichRMSNormPair", "recordSandwichRMSNormPair",
-              "runResidualNextRMSNormPair", "recordResidualNextRMSNormPair", "runRoPE", "runRoPEQK", "recordRoPEQK", "canUseRoPEQK",
+              "runResidualNextRMSNormPair", "recordResidualNextRMSNormPair", "runRoPE", "runBiasAdd", "recordBiasAdd", "runScale", "recordScale", "runRoPEQK", "recordRoPEQK", "canUseRoPEQK",
               "recordRoPE", "runKVCacheWriteF32ToF16", "recordKVCacheWriteF32ToF16", "runSplitQKVRMSNormRoPEQK",
               "recordSplitQKVRMSNormRoPEQK", "runSiLU", "recordSiLU", "runSiLURowSplit", "recordSiLURowSplit", "runGeLU",
               "recordGeLU", "runResidualAdd", "recordResidualAdd", "runGather", "recordGather", "runFusedFFN",
@@ -154,6 +154,10 @@ def test_js_host_path_parity(tmp_path):
                       heads=16, headDim=128, startPos=40, interleaved=False))
     rope_want = oracle.rope_apply(xr, cos, sin, 2, 16, 128, 40)
     checks.append(lambda: rel_l2(get("rope.out.bin", np.float32), rope_want) <= 1e-6)
+    bx, bb = synth.normal_f32((3, 1024), 9510, 2.0), synth.normal_f32((2, 1024), 9511)
+    cases.append(dict(name="biasscale", op="bias_scale", x=put("bs.x", bx), bias=put("bs.b", bb), tokens=3, dim=1024, scale=0.125))
+    checks.append(lambda: np.array_equal(get("biasscale.bias.out.bin", np.float32).reshape(3, 1024), bx + bb[1]))
+    checks.append(lambda: np.array_equal(get("biasscale.scale.out.bin", np.float32).reshape(3, 1024), (bx + bb[1]) * np.float32(0.125)))
     kr = synth.normal_f32((2, 8, 128), 9501)
     cases.append(dict(name="ropeqk", op="rope_qk", q=put("ropeqk.q", xr), k=put("ropeqk.k", kr), cos=put("cos", cos),
                       sin=put("sin", sin), seq=2, heads=16, kvHeads=8, headDim=128, startPos=40))

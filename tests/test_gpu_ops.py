@@ -676,6 +676,33 @@ def test_split_qkv_rmsnorm_rope_kvwrite(T, H, Hkv, D):
     assert np.mean(got_k != wk) < 0.02
 
 
+def test_bias_add_and_scale_bit_exact():
+    """residual.js runBiasAdd (in place, byte offsets, f32 or f16 bias) and scale.js runScale: one IEEE add or
+    multiply per element, so the f32 results are fixed bit for bit."""
+    T, dim = 5, 1536
+    x = synth.normal_f32((T + 1, dim), seed=4450, scale=3.0)
+    bias = synth.normal_f32((2, dim), seed=4451)
+    xt = ops.tensorFromNumpy(x)
+    out = ops.runBiasAdd(xt, ops.tensorFromNumpy(bias), T, dim, dataOffset=dim * 4, biasOffset=dim * 4)
+    assert out.buffer is xt.buffer and tuple(out.shape) == (T, dim)
+    want = x.copy()
+    want[1:] += bias[1]
+    assert np.array_equal(ops.readTensor(xt).reshape(T + 1, dim), want)
+    b16 = bias[0].astype(np.float16)
+    xt = ops.tensorFromNumpy(x)
+    ops.runBiasAdd(xt, ops.tensorFromNumpy(b16.view(np.uint16), "f16"), T + 1, dim)
+    assert np.array_equal(ops.readTensor(xt).reshape(T + 1, dim), x + b16.astype(np.float32))
+    with pytest.raises(DopplerHipError, match="data buffer is smaller"):
+        ops.runBiasAdd(xt, ops.tensorFromNumpy(bias), T + 2, dim)
+    s = np.float32(1536 ** 0.5)
+    xt = ops.tensorFromNumpy(x)
+    assert np.array_equal(ops.readTensor(ops.runScale(xt, float(s))).reshape(x.shape), x * s)
+    part = ops.runScale(xt, 0.3, count=dim)
+    assert np.array_equal(ops.readTensor(part).reshape(-1)[:dim], x[0] * np.float32(0.3))
+    same = ops.runScale(xt, float(s), inplace=True)
+    assert same.buffer is xt.buffer and np.array_equal(ops.readTensor(xt).reshape(x.shape), x * s)
+
+
 def test_residual_and_gated_activations():
     n = 12288
     a, b = synth.normal_f32(n, seed=4400, scale=4.0), synth.normal_f32(n, seed=4401)
