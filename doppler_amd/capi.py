@@ -69,6 +69,7 @@ SIGNATURES = {
     "dh_residual_add": (_I, [_P, _P, _P, _I64, _F]),
     "dh_bias_add": (_I, [_P, _P, _I, _I64, _I, _I64, _I64]),
     "dh_scale": (_I, [_P, _P, _I64, _F]),
+    "dh_split_qkv": (_I, [_P, _P, _P, _P, _I, _I, _I, _I]),
     "dh_gather_f16": (_I, [_P, _P, _P, _I, _I, _I, _I]),
     "dh_act_gate": (_I, [_P, _P, _P, _I64, _I, _F]),
     "dh_act_gate_rowsplit": (_I, [_P, _P, _I, _I, _I, _F]),

@@ -314,6 +314,21 @@ __global__ __launch_bounds__(256) void residual_kernel(const float* __restrict__
   if (i < n) out[i] = (a[i] + b[i]) * scale;
 }
 
+// Rows of [q | k | v] copied apart into three dense buffers, one element per thread.
+__global__ __launch_bounds__(256) void split_qkv_kernel(const float* __restrict__ qkv, float* __restrict__ q,
+                                                        float* __restrict__ k, float* __restrict__ v, int64_t total,
+                                                        int q_size, int k_size, int v_size) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int row_len = q_size + k_size + v_size;
+  const int64_t t = i / row_len;
+  const int c = (int)(i % row_len);
+  const float x = qkv[i];
+  if (c < q_size) q[t * q_size + c] = x;
+  else if (c < q_size + k_size) k[t * k_size + (c - q_size)] = x;
+  else v[t * v_size + (c - q_size - k_size)] = x;
+}
+
 // data[t][d] += bias[d] in place; bias is f32 or f16.
 __global__ __launch_bounds__(256) void bias_add_kernel(float* __restrict__ data, const void* __restrict__ bias,
                                                        int bias_f16, int64_t total, int dim) {
@@ -585,6 +600,22 @@ int dh_residual_add(const float* d_a, const float* d_b, float* d_out, int64_t n,
   if (!(scale == scale) || scale > 3.0e38f || scale < -3.0e38f)
     return dh::fail(1, "[Residual] outputScale must be finite");
   hipLaunchKernelGGL(residual_kernel, dim3(grid_for(n)), dim3(256), 0, dh::stream(), d_a, d_b, d_out, n, scale);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_split_qkv(const float* d_qkv, float* d_q, float* d_k, float* d_v, int num_tokens, int q_size, int k_size,
+                 int v_size) {
+  const char* op = "dh_split_qkv";
+  DH_REQUIRE_INIT(op);
+  if (num_tokens < 0 || q_size <= 0 || k_size <= 0 || v_size <= 0)
+    return dh::fail(1, "[%s] numTokens=%d qSize=%d kSize=%d vSize=%d: need numTokens >= 0 and positive sizes", op,
+                    num_tokens, q_size, k_size, v_size);
+  if (num_tokens == 0) return 0;
+  if (!d_qkv || !d_q || !d_k || !d_v) return dh::fail(1, "[%s] null pointer", op);
+  const int64_t total = (int64_t)num_tokens * ((int64_t)q_size + k_size + v_size);
+  hipLaunchKernelGGL(split_qkv_kernel, dim3(grid_for(total)), dim3(256), 0, dh::stream(), d_qkv, d_q, d_k, d_v, total,
+                     q_size, k_size, v_size);
   DH_CHECK_LAUNCH(op);
   return 0;
 }

@@ -241,6 +241,10 @@ FN(js_kv_write_f16) {
   return ret_rc(env, dh_kv_write_f16((const float*)k, (const float*)v, ck, cv, so, dof, n));
 }
 FN(js_residual_add) { ARGS(5); P(0, x); P(1, y); P(2, o); L(3, n); F(4, s); return ret_rc(env, dh_residual_add((const float*)x, (const float*)y, (float*)o, n, s)); }
+FN(js_split_qkv) {
+  ARGS(8); P(0, x); P(1, q); P(2, k); P(3, v); I(4, t); I(5, qs); I(6, ks); I(7, vs);
+  return ret_rc(env, dh_split_qkv((const float*)x, (float*)q, (float*)k, (float*)v, t, qs, ks, vs));
+}
 FN(js_bias_add) {
   ARGS(7); P(0, d); P(1, b); I(2, bdt); L(3, t); I(4, dim); L(5, doff); L(6, boff);
   return ret_rc(env, dh_bias_add((float*)d, b, bdt, t, dim, doff, boff));
@@ -284,7 +288,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"attnPrefill", js_attn_prefill},
       {"rmsnorm", js_rmsnorm}, {"rmsnormQK", js_rmsnorm_qk}, {"rmsnormSandwichPair", js_rmsnorm_sandwich_pair},
       {"residualRmsnormPair", js_residual_rmsnorm_pair}, {"rope", js_rope}, {"ropeQK", js_rope_qk}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},
-      {"kvWriteF16", js_kv_write_f16}, {"residualAdd", js_residual_add}, {"biasAdd", js_bias_add}, {"scale", js_scale}, {"gatherF16", js_gather_f16},
+      {"kvWriteF16", js_kv_write_f16}, {"residualAdd", js_residual_add}, {"biasAdd", js_bias_add}, {"splitQKV", js_split_qkv}, {"scale", js_scale}, {"gatherF16", js_gather_f16},
       {"actGate", js_act_gate}, {"actGateRowsplit", js_act_gate_rowsplit},
       {"argmaxWorkspaceBytes", js_argmax_workspace_bytes}, {"argmax", js_argmax},
       {"sampleTopkWorkspaceBytes", js_sample_topk_workspace_bytes}, {"sampleTopk", js_sample_topk},

@@ -17,6 +17,7 @@ export { runSplitQKVRMSNormRoPEQK, recordSplitQKVRMSNormRoPEQK } from './split-q
 export { runSiLU, recordSiLU, runSiLURowSplit, recordSiLURowSplit } from './silu.js';
 export { runGeLU, recordGeLU } from './gelu.js';
 export { runResidualAdd, recordResidualAdd } from './residual.js';
+export { runSplitQKV, recordSplitQKV } from './split_qkv.js';
 export { runBiasAdd, recordBiasAdd, runScale, recordScale } from './bias-scale.js';
 export { runGather, recordGather } from './gather.js';
 export { runArgmax, recordArgmax, runGPUSample, recordGPUSample, seededRandom } from './sample.js';

@@ -585,6 +585,25 @@ def runResidualAdd(a, b, size, outputBuffer=None, outputScale=None, **_ignored):
     return Tensor(out, "f32", (size,), "residual_output")
 
 
+def runSplitQKV(qkvTensor, numTokens=None, qSize=None, kSize=None, vSize=None, qTensor=None, kTensor=None,
+                vTensor=None, **_ignored):
+    """src/gpu/kernels/split_qkv.js:40 runSplitQKV: the stacked projection copied apart into Q, K, V (new buffers
+    unless the caller passes tensors to fill)."""
+    if qkvTensor.dtype != "f32":
+        raise DopplerHipError("[SplitQKV] the HIP path takes f32 tensors, got %s." % qkvTensor.dtype)
+    if numTokens * (qSize + kSize + vSize) * 4 > _nbytes(qkvTensor):
+        raise DopplerHipError("[SplitQKV] qkv buffer is smaller than numTokens=%d x %d elements."
+                              % (numTokens, qSize + kSize + vSize))
+    outs = []
+    for given, size, name in ((qTensor, qSize, "Q"), (kTensor, kSize, "K"), (vTensor, vSize, "V")):
+        if given is not None and _nbytes(given) < numTokens * size * 4:
+            raise DopplerHipError("[SplitQKV] %s tensor is smaller than numTokens=%d x %d elements." % (name, numTokens, size))
+        outs.append(given if given is not None else Tensor(_out(None, numTokens * size * 4), "f32", (numTokens, size), name))
+    capi.check(_lib().dh_split_qkv(_ptr(qkvTensor), _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), numTokens, qSize,
+                                   kSize, vSize))
+    return {"Q": outs[0], "K": outs[1], "V": outs[2]}
+
+
 def runBiasAdd(data, bias, numTokens, dim, dataOffset=0, biasOffset=0, **_ignored):
     """src/gpu/kernels/residual.js:218 runBiasAdd: data[t, :] += bias in place (offsets in bytes); the returned
     Tensor aliases data.  The bias may be f32 or f16 and is widened on the fly."""

@@ -263,6 +263,12 @@ int dh_kv_write_f16(const float* d_k, const float* d_v, void* d_cache_k, void* d
  * (residual.wgsl:24-31). */
 int dh_residual_add(const float* d_a, const float* d_b, float* d_out, int64_t n, float scale);
 
+/* Rows of qkv[num_tokens][q_size + k_size + v_size] copied apart into q[num_tokens][q_size],
+ * k[num_tokens][k_size], v[num_tokens][v_size].  Replaces runSplitQKV/recordSplitQKV,
+ * src/gpu/kernels/split_qkv.js:6-45. */
+int dh_split_qkv(const float* d_qkv, float* d_q, float* d_k, float* d_v, int num_tokens, int q_size, int k_size,
+                 int v_size);
+
 /* data[t][d] += bias[d] in place for t < num_tokens, d < dim; the byte offsets select the start
  * inside each buffer; bias is DH_F32 or DH_F16.  Replaces runBiasAdd/recordBiasAdd,
  * src/gpu/kernels/residual.js:165-224 (bias_add.wgsl:27-39). */

@@ -112,6 +112,12 @@ async function main() {
       if (r.q.buffer !== q.buffer || r.k.buffer !== k.buffer) throw new Error('runRoPEQK must alias its inputs');
       await save(c.name + '.q.out.bin', r.q.buffer, c.seq * c.heads * c.headDim * 4);
       await save(c.name + '.k.out.bin', r.k.buffer, c.seq * c.kvHeads * c.headDim * 4);
+    } else if (c.op === 'split_plain') {
+      const r = await dh.runSplitQKV(tensor(c.x, 'f32', [c.tokens, c.q + c.k + c.v]),
+        { numTokens: c.tokens, qSize: c.q, kSize: c.k, vSize: c.v });
+      await save(c.name + '.q.out.bin', r.Q.buffer, c.tokens * c.q * 4);
+      await save(c.name + '.k.out.bin', r.K.buffer, c.tokens * c.k * 4);
+      await save(c.name + '.v.out.bin', r.V.buffer, c.tokens * c.v * 4);
     } else if (c.op === 'bias_scale') {
       const x = tensor(c.x, 'f32', [c.tokens, c.dim]);
       const b = await dh.runBiasAdd(x, tensor(c.bias, 'f32', [2, c.dim]), c.tokens, c.dim, { biasOffset: c.dim * 4 });

@@ -35,7 +35,7 @@ def test_addon_is_built_and_exports_the_op_api():
     assert out.returncode == 0, out.stderr
     names = set(json.loads(out.stdout))
     for n in ("runMatmul", "recordMatmul", "runAttention", "recordAttention", "runRMSNorm", "recordRMSNorm", "runRMSNormQK", "recordRMSNormQK", "canUseRMSNormQK", "runSandwichRMSNormPair", "recordSandwichRMSNormPair",
-              "runResidualNextRMSNormPair", "recordResidualNextRMSNormPair", "runRoPE", "runBiasAdd", "recordBiasAdd", "runScale", "recordScale", "runRoPEQK", "recordRoPEQK", "canUseRoPEQK",
+              "runResidualNextRMSNormPair", "recordResidualNextRMSNormPair", "runRoPE", "runSplitQKV", "recordSplitQKV", "runBiasAdd", "recordBiasAdd", "runScale", "recordScale", "runRoPEQK", "recordRoPEQK", "canUseRoPEQK",
               "recordRoPE", "runKVCacheWriteF32ToF16", "recordKVCacheWriteF32ToF16", "runSplitQKVRMSNormRoPEQK",
               "recordSplitQKVRMSNormRoPEQK", "runSiLU", "recordSiLU", "runSiLURowSplit", "recordSiLURowSplit", "runGeLU",
               "recordGeLU", "runResidualAdd", "recordResidualAdd", "runGather", "recordGather", "runFusedFFN",
@@ -158,6 +158,11 @@ def test_js_host_path_parity(tmp_path):
     cases.append(dict(name="biasscale", op="bias_scale", x=put("bs.x", bx), bias=put("bs.b", bb), tokens=3, dim=1024, scale=0.125))
     checks.append(lambda: np.array_equal(get("biasscale.bias.out.bin", np.float32).reshape(3, 1024), bx + bb[1]))
     checks.append(lambda: np.array_equal(get("biasscale.scale.out.bin", np.float32).reshape(3, 1024), (bx + bb[1]) * np.float32(0.125)))
+    sx = synth.normal_f32((3, 1024 + 256 + 256), 9520)
+    cases.append(dict(name="splitplain", op="split_plain", x=put("sp.x", sx), tokens=3, q=1024, k=256, v=256))
+    checks.append(lambda: np.array_equal(get("splitplain.q.out.bin", np.float32).reshape(3, 1024), sx[:, :1024]))
+    checks.append(lambda: np.array_equal(get("splitplain.k.out.bin", np.float32).reshape(3, 256), sx[:, 1024:1280]))
+    checks.append(lambda: np.array_equal(get("splitplain.v.out.bin", np.float32).reshape(3, 256), sx[:, 1280:]))
     kr = synth.normal_f32((2, 8, 128), 9501)
     cases.append(dict(name="ropeqk", op="rope_qk", q=put("ropeqk.q", xr), k=put("ropeqk.k", kr), cos=put("cos", cos),
                       sin=put("sin", sin), seq=2, heads=16, kvHeads=8, headDim=128, startPos=40))

@@ -703,6 +703,21 @@ def test_bias_add_and_scale_bit_exact():
     assert same.buffer is xt.buffer and np.array_equal(ops.readTensor(xt).reshape(x.shape), x * s)
 
 
+def test_split_qkv_exact():
+    """split_qkv.js: a pure copy, so every output element equals its source bit for bit."""
+    T, qs, ks, vs = 7, 2048, 512, 384
+    x = synth.normal_f32((T, qs + ks + vs), seed=4460)
+    out = ops.runSplitQKV(ops.tensorFromNumpy(x), numTokens=T, qSize=qs, kSize=ks, vSize=vs)
+    assert np.array_equal(ops.readTensor(out["Q"]).reshape(T, qs), x[:, :qs])
+    assert np.array_equal(ops.readTensor(out["K"]).reshape(T, ks), x[:, qs:qs + ks])
+    assert np.array_equal(ops.readTensor(out["V"]).reshape(T, vs), x[:, qs + ks:])
+    mine = ops.tensorFromNumpy(np.zeros((T, ks), np.float32))
+    again = ops.runSplitQKV(ops.tensorFromNumpy(x), numTokens=T, qSize=qs, kSize=ks, vSize=vs, kTensor=mine)
+    assert again["K"] is mine and np.array_equal(ops.readTensor(mine).reshape(T, ks), x[:, qs:qs + ks])
+    with pytest.raises(DopplerHipError, match="qkv buffer is smaller"):
+        ops.runSplitQKV(ops.tensorFromNumpy(x), numTokens=T + 1, qSize=qs, kSize=ks, vSize=vs)
+
+
 def test_residual_and_gated_activations():
     n = 12288
     a, b = synth.normal_f32(n, seed=4400, scale=4.0), synth.normal_f32(n, seed=4401)
