@@ -1327,6 +1327,11 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
   a.alpha = alpha;
   a.c_f16 = c_dtype == DH_F16;
   const int path = gemv_path();
+  if ((path == 0 || normed) && M <= 2) {
+    const int rc = dh::q4k_gemv_i8(op, a.A, a.W, nullptr, d_C, a.c_f16, a.residual, M, N, K, alpha, 0, 0.f,
+                                   normed ? d_norm_weight : nullptr, eps, weight_offset);
+    if (rc >= 0) return rc;
+  }
   if ((path == 0 || normed) && M < 16) {
     // below the GEMM's batch size: passes of up to 8 rows through the streaming GEMV
     int rc = 0;
@@ -1403,6 +1408,11 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
   a.activation = activation;
   a.clamp_max = swiglu_limit;
   const int path = gemv_path();
+  if ((path == 0 || normed) && M <= 2) {
+    const int rc = dh::q4k_gemv_i8(op, d_x, a.W, a.W2, d_out, 0, nullptr, M, inter, hidden, alpha, activation,
+                                   swiglu_limit, normed ? d_norm_weight : nullptr, eps, weight_offset);
+    if (rc >= 0) return rc;
+  }
   if ((path == 0 || normed) && M < 16) {
     int rc = 0;
     for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
