@@ -45,7 +45,6 @@ typedef float v2f __attribute__((ext_vector_type(2)));
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 16;
-constexpr int kSetupWaves = 8;                    // waves that prepare the activation operands
 constexpr int kTileRows = 16;
 constexpr int kStage = kTileRows * kBlockBytes;   // 2304 bytes per ring stage
 constexpr int kUnitLoads = 3;                     // load instructions of a full unit: ceil(16 rows * 9 pieces / 64 lanes)
@@ -147,7 +146,7 @@ __device__ unsigned long long dh_i8_trace[256 * 16 * 32];
 //   red    [nslots][upt][MT][16] partial sums of a tile's units
 //   ctr    [0] next unit to draw, [1 + s] units delivered to slot s, [1 + nslots + s] tiles completed
 //          in slot s, [1 + 2 nslots + c] column c's operands are in place
-template <int MT, bool DUAL>
+template <int MT, bool DUAL, bool VEC>
 __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Args a) {
   constexpr int NMAT = DUAL ? 2 : 1;
 #ifdef DH_I8_TRACE
@@ -226,35 +225,32 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     }                                                                                             \
   } while (0)
 
-  // ---- 1. the first kSetupWaves waves prepare the activation operands: wave w takes columns
-  // w, w + kSetupWaves, ..; lane t holds elements 4t .. 4t+3 of a column.  Per (column, row):
-  // three digit planes, the sub-block sums, 2^-E and the sum of squares, then the column's flag.
-  // Their activation loads go out BEFORE the workgroup barrier and the other waves' weight loads
-  // after it, so the activations are at the head of the compute unit's memory queue.
+  // ---- 1. every wave prepares the activation operands of columns wave, wave + 16, ..; lane t
+  // holds elements 4t .. 4t+3 of a column.  Per (column, row): three digit planes, the sub-block
+  // sums, 2^-E and the sum of squares, then the column's flag.  The activation loads go out BEFORE
+  // the workgroup barrier and every weight load after it, so the activations are at the head of the
+  // compute unit's memory queue.  (Fast path, K a multiple of 4 and 16-byte aligned rows: the loads
+  // are hand-issued so that the first weight unit can follow them and only THEY are waited for.)
   const int kg = lane >> 4;
-  constexpr int SC = MT == 1 ? 6 : 3;                    // columns per pass (all loads of a pass in flight at once)
-  const bool setup_wave = wave < kSetupWaves;
-  const int my_cols = (setup_wave && wave < nb) ? (nb - wave + kSetupWaves - 1) / kSetupWaves : 0;
-  const bool vec_ok = (a.K & 3) == 0 && (reinterpret_cast<uintptr_t>(a.A) & 15) == 0 &&
-                      (!norm || (reinterpret_cast<uintptr_t>(a.norm_weight) & 15) == 0);
+  constexpr int SC = MT == 1 ? 3 : 2;                    // columns per pass (all loads of a pass in flight at once)
+  const int my_cols = wave < nb ? (nb - wave + kWaves - 1) >> 4 : 0;
   v4f xr[SC][MT], wr[SC];
-  // All loads of a pass go out back to back, from addresses clamped into the row (what lies past
-  // K is dropped afterwards).
 #define DH_LOAD_X(c0_)                                                                            \
   do {                                                                                            \
-    if (vec_ok) {                                                                                 \
-      _Pragma("unroll") for (int i = 0; i < SC; i++) {                                            \
-        if ((c0_) + i < my_cols) {                                                                \
-          const int k0 = (wave + kSetupWaves * ((c0_) + i)) * kQK + 4 * lane, kc = k0 < a.K ? k0 : 0; \
-          _Pragma("unroll") for (int m = 0; m < MT; m++)                                          \
-            xr[i][m] = *reinterpret_cast<const v4f*>(a.A + (int64_t)min(m, a.M - 1) * a.K + kc);  \
-          if (norm) wr[i] = *reinterpret_cast<const v4f*>(a.norm_weight + kc);                    \
-        }                                                                                         \
-      }                                                                                           \
-    } else {                                                                                      \
-      _Pragma("unroll") for (int i = 0; i < SC; i++) {                                            \
-        if ((c0_) + i < my_cols) {                                                                \
-          const int k0 = (wave + kSetupWaves * ((c0_) + i)) * kQK + 4 * lane;                     \
+    _Pragma("unroll") for (int i = 0; i < SC; i++) {                                              \
+      if ((c0_) + i < my_cols) {                                                                  \
+        const int k0 = (wave + kWaves * ((c0_) + i)) * kQK + 4 * lane;                            \
+        if constexpr (VEC) {                                                                      \
+          const int kc = k0 < a.K ? k0 : 0;                                                       \
+          _Pragma("unroll") for (int m = 0; m < MT; m++) {                                        \
+            const float* p_ = a.A + (int64_t)min(m, a.M - 1) * a.K + kc;                          \
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(xr[i][m]) : "v"(p_) : "memory"); \
+          }                                                                                       \
+          if (norm) {                                                                             \
+            const float* p_ = a.norm_weight + kc;                                                 \
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(wr[i]) : "v"(p_) : "memory");  \
+          }                                                                                       \
+        } else {                                                                                  \
           _Pragma("unroll") for (int e = 0; e < 4; e++) {                                         \
             const int kc = min(k0 + e, a.K - 1);                                                  \
             _Pragma("unroll") for (int m = 0; m < MT; m++)                                        \
@@ -265,19 +261,55 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
       }                                                                                           \
     }                                                                                             \
   } while (0)
+  // makes the loaded registers depend on the wait in front of it
+#define DH_TIE_X()                                                                                \
+  do {                                                                                            \
+    _Pragma("unroll") for (int i = 0; i < SC; i++) {                                              \
+      _Pragma("unroll") for (int m = 0; m < MT; m++) asm volatile("" : "+v"(xr[i][m]));           \
+      if (norm) asm volatile("" : "+v"(wr[i]));                                                   \
+    }                                                                                             \
+  } while (0)
   DH_LOAD_X(0);
+  if constexpr (!VEC) {
+    DH_WAIT_VM(0);
+    DH_TIE_X();
+  }
   // counters, flags and the zero area are in place; costs little more than the skew of the wave launches
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   DH_TS(1);
-  if (setup_wave) {
+
+  // Draws the next unit of the workgroup (wave-uniform result).
+  const uint32_t ctr_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(ctr);
+  auto draw = [&]() -> int {
+    unsigned v = 0;
+    if (lane == 0)
+      asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(ctr_abs), "v"(1u) : "memory");
+    return (int)__builtin_amdgcn_readfirstlane(v);
+  };
+  // ---- 2. the first unit's loads go out before anything else is waited for
+  int u_ring[kMaxDepth];                   // units in the ring stages (>= total: none)
+#pragma unroll
+  for (int d = 0; d < kMaxDepth; d++) u_ring[d] = 0x7fffffff;
+  int inflight = 0;
+  u_ring[0] = draw();
+  if (u_ring[0] < total) {
+    DH_ISSUE(u_ring[0], 0);
+    inflight = 1;
+  }
+  DH_TS(2);
+  {
 #pragma unroll 1
     for (int c0 = 0; c0 < my_cols; c0 += SC) {
       if (c0 > 0) DH_LOAD_X(c0);
-      DH_TS(2);
+      if constexpr (VEC) {
+        // only the activations are waited for (the unit's loads were issued behind them)
+        if (c0 == 0 && inflight) wait_vm_at_most(a.nlw); else DH_WAIT_VM(0);
+        DH_TIE_X();
+      }
 #pragma unroll
       for (int i = 0; i < SC; i++) {
         if (c0 + i < my_cols) {
-          const int col = wave + kSetupWaves * (c0 + i);
+          const int col = wave + kWaves * (c0 + i);
 #pragma unroll
           for (int m = 0; m < MT; m++) {
             float v[4], ss = 0.f;
@@ -331,6 +363,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     DH_TS(3);
   }
 #undef DH_LOAD_X
+#undef DH_TIE_X
   DH_TS(4);
 
   // ---- 5. stream the units
@@ -354,7 +387,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     }
   }
   const uint32_t xq_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(xq);
-  const uint32_t ctr_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(ctr);
   const uint32_t red_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(red);
   // LDS byte address of this lane's header inside stage 0, and of its 16 nibble bytes of chunk
   // (kg >> 1) (chunk 2 + (kg >> 1) is 64 bytes further)
@@ -362,24 +394,13 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
   const uint32_t lane_q = lane_hdr + 16 + 32 * (kg >> 1) + 16 * (kg & 1);
   const uint32_t sh_lo = 8 * kg;           // bit offset of this lane's byte in the header words
 
-  // Draws the next unit of the workgroup (wave-uniform result).
-  auto draw = [&]() -> int {
-    unsigned v = 0;
-    if (lane == 0)
-      asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(ctr_abs), "v"(1u) : "memory");
-    return (int)__builtin_amdgcn_readfirstlane(v);
-  };
-
   float inv_rms[MT];                       // RMSNorm prologue: filled by the first tile end this wave meets
   bool have_rms = false;
 #pragma unroll
   for (int m = 0; m < MT; m++) inv_rms[m] = 1.f;
 
-  int u_ring[kMaxDepth];                   // units in the ring stages (>= total: none)
-#pragma unroll
-  for (int d = 0; d < kMaxDepth; d++) u_ring[d] = 0x7fffffff;
-  int inflight = 0;
-  for (int d = 0; d < D; d++) {
+  for (int d = 1; d < D; d++) {
+    if (u_ring[0] >= total) break;
     const int u = draw();
 #pragma unroll
     for (int q = 0; q < kMaxDepth; q++) if (q == d) u_ring[q] = u;
@@ -594,14 +615,14 @@ int env_int(const char* name, int dflt) {
   return e ? atoi(e) : dflt;
 }
 
-template <int MT, bool DUAL>
-int launch_i8(I8Args a, const char* op) {
+template <int MT, bool DUAL, bool VEC>
+int launch_i8_vec(I8Args a, const char* op) {
   constexpr int NMAT = DUAL ? 2 : 1;
   size_t cap = kMaxLds;
 #ifdef DH_I8_TRACE
   cap -= 4096;
 #endif
-  auto kern = q4k_gemv_i8_kernel<MT, DUAL>;
+  auto kern = q4k_gemv_i8_kernel<MT, DUAL, VEC>;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
     DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -646,6 +667,14 @@ int launch_i8(I8Args a, const char* op) {
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kWaves), lds_for(depth), dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   return 0;
+}
+
+// Fast path: K a multiple of 4 and 16-byte aligned rows (vector loads of the activations).
+template <int MT, bool DUAL>
+int launch_i8(const I8Args& a, const char* op) {
+  const bool vec = (a.K & 3) == 0 && (reinterpret_cast<uintptr_t>(a.A) & 15) == 0 &&
+                   (!a.norm_weight || (reinterpret_cast<uintptr_t>(a.norm_weight) & 15) == 0);
+  return vec ? launch_i8_vec<MT, DUAL, true>(a, op) : launch_i8_vec<MT, DUAL, false>(a, op);
 }
 
 template <bool DUAL>
