@@ -54,6 +54,8 @@ SIGNATURES = {
     "dh_attn_decode_workspace_bytes": (_SZ, [_I, _I, _I]),
     "dh_attn_prefill": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _F, _I]),
     "dh_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _F, _I, _I, _I, _P]),
+    "dh_attn_decode_static_max_bytes": (_SZ, []),
+    "dh_attn_decode_static": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _F, _I, _I, _I]),
     "dh_attn_decode_qkv_supported": (_I, [_I, _I, _I, _I, _I]),
     "dh_attn_decode_qkv": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _F, _I, _I,
                                 _I, _P]),

@@ -546,6 +546,29 @@ int launch(const AttnArgs& a, const char* op) {
 
 }  // namespace
 
+// ---------------------------------------------------------------------------------------
+// Split-K partials for callers that may not allocate (dh_attn_decode_static): a fixed array in
+// device memory that belongs to the library.  Each GPU holds its own copy at its own address, so
+// the address is asked for once per device (dh_init) and kept; host code only ever passes that
+// address, never the symbol, to kernels.
+// ---------------------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = (size_t)4 << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+namespace dh {
+int attn_static_scratch_init(int device) {
+  if (device < 0 || device >= kMaxDevices)
+    return fail(1, "[dh_init] device ordinal %d is beyond the %d the static attention scratch tracks", device, kMaxDevices);
+  if (g_scratch_ptr[device]) return 0;
+  void* ptr = nullptr;
+  DH_CHECK_HIP("dh_init", hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  g_scratch_ptr[device] = ptr;
+  return 0;
+}
+}  // namespace dh
+
 #ifdef DH_ATTN_TRACE
 extern "C" int dh_debug_attn_trace(void* host_dst) {
   return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(dh_attn_trace_buf), sizeof(dh_attn_trace_buf));
@@ -560,10 +583,11 @@ size_t dh_attn_decode_workspace_bytes(int H, int D, int kv_len) {
   return std::max<size_t>(256, (size_t)H * splits * (D + 2) * sizeof(float));
 }
 
-int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H, int Hkv, int D,
-                   int kv_len, float scale, int causal, int start_pos, float softcap, int sliding_window,
-                   int kv_start, int kv_layout, void* d_workspace) {
-  const char* op = "dh_attn_decode";
+// Shared body of dh_attn_decode and dh_attn_decode_static.  ws_capacity: bytes behind d_workspace when
+// the caller of this function knows them (0: the public contract, dh_attn_decode_workspace_bytes, holds).
+static int attn_decode_impl(const char* op, const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H,
+                            int Hkv, int D, int kv_len, float scale, int causal, int start_pos, float softcap,
+                            int sliding_window, int kv_start, int kv_layout, void* d_workspace, size_t ws_capacity) {
   DH_REQUIRE_INIT(op);
   if (H <= 0 || Hkv <= 0 || D <= 0) return dh::fail(1, "[%s] numHeads/numKVHeads/headDim must be positive", op);
   if (H % Hkv) return dh::fail(1, "[%s] numHeads=%d must be a multiple of numKVHeads=%d", op, H, Hkv);
@@ -604,10 +628,38 @@ int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_
   a.tiles_per_split = 0;
   a.nsplit = nsplit;
   if (nsplit > 1 && !d_workspace) return dh::fail(1, "[%s] workspace is required", op);
+  const size_t ws_need = nsplit > 1 ? (size_t)H * nsplit * (D + 2) * sizeof(float) : 0;
+  if (ws_capacity && ws_need > ws_capacity)
+    return dh::fail(1, "[%s] numHeads=%d, headDim=%d with %d key splits needs %zu bytes of split partials, the "
+                       "scratch holds %zu: use dh_attn_decode with a workspace", op, H, D, nsplit, ws_need, ws_capacity);
   a.scale = scale; a.softcap = softcap;
   a.kv_start = kv_start;
   a.ring_window = kv_layout == DH_KV_RING ? sliding_window : 0;
   return D == 64 ? launch<64, false>(a, op) : launch<128, false>(a, op);
+}
+
+int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H, int Hkv, int D,
+                   int kv_len, float scale, int causal, int start_pos, float softcap, int sliding_window,
+                   int kv_start, int kv_layout, void* d_workspace) {
+  return attn_decode_impl("dh_attn_decode", d_Q, d_K, d_V, d_O, H, Hkv, D, kv_len, scale, causal, start_pos, softcap,
+                          sliding_window, kv_start, kv_layout, d_workspace, 0);
+}
+
+size_t dh_attn_decode_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int dh_attn_decode_static(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H, int Hkv, int D,
+                          int kv_len, float scale, int causal, int start_pos, float softcap, int sliding_window,
+                          int kv_start, int kv_layout) {
+  const char* op = "dh_attn_decode_static";
+  DH_REQUIRE_INIT(op);
+  int device = -1;
+  DH_CHECK_HIP(op, hipGetDevice(&device));
+  if (device < 0 || device >= kMaxDevices || !g_scratch_ptr[device])
+    return dh::fail(1, "[%s] the static scratch of device %d was not set up by dh_init", op, device);
+  // nothing in the scratch has to start at zero: every (head, split) slot the merge reads is
+  // written by the split kernel of the same call
+  return attn_decode_impl(op, d_Q, d_K, d_V, d_O, H, Hkv, D, kv_len, scale, causal, start_pos, softcap,
+                          sliding_window, kv_start, kv_layout, g_scratch_ptr[device], kStaticScratchBytes);
 }
 
 int dh_attn_decode_qkv_supported(int H, int Hkv, int D, int rotary_dim, int interleaved) {

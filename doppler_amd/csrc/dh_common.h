@@ -51,6 +51,10 @@ int q4k_gemm_gate_up(const char* op, const float* A, const uint8_t* Wg, const ui
                      int hidden, int inter, int activation, float alpha, float clamp_max,
                      const float* norm_weight = nullptr, float norm_eps = 0.f, int norm_weight_offset = 0);
 
+// Looks up, once per device, the address of the fixed device array that dh_attn_decode_static uses
+// for its split partials (attention.hip).  Called by dh_init with the device current.
+int attn_static_scratch_init(int device);
+
 // Decode GEMV on the int8 matrix cores (q4k_gemv_i8.hip): C = alpha * A . W^T + residual, or with W2
 // the gated pair act(A . W^T) * (A . W2^T) * alpha; norm_weight != null normalises A's rows first.
 // Returns -1 when the shape is not served (the caller then takes another kernel), 0 on success.

@@ -103,6 +103,7 @@ static int init_locked(int device_ordinal) {
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_splitk_ws), kSplitKWsBytes));
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_row_scale), (size_t)kRowScaleRows * 2 * sizeof(float)));
   DH_CHECK_HIP("dh_init", hipMalloc(&g_packed_a, kPackedABytes));
+  if (int rc = dh::attn_static_scratch_init(device_ordinal)) return rc;
   g_device = device_ordinal;
   g_ready = true;
   return 0;

@@ -174,6 +174,17 @@ int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_
                    int Hkv, int D, int kv_len, float scale, int causal, int start_pos,
                    float softcap, int sliding_window, int kv_start, int kv_layout,
                    void* d_workspace);
+/* dh_attn_decode for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the split-K partials go to a fixed 4 MiB
+ * device array inside the library instead of a caller's workspace, and the call allocates nothing.
+ * It has no counterpart in the reference.  Arguments and results as dh_attn_decode; a shape whose
+ * partials (numHeads * key splits * (headDim + 2) floats) exceed
+ * dh_attn_decode_static_max_bytes() fails with a message.  Every call on a GPU shares that GPU's
+ * array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not. */
+size_t dh_attn_decode_static_max_bytes(void);
+int dh_attn_decode_static(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H,
+                          int Hkv, int D, int kv_len, float scale, int causal, int start_pos,
+                          float softcap, int sliding_window, int kv_start, int kv_layout);
 /* One decode step's attention straight from the stacked projection qkv[(H+2Hkv)*D] (f32): per-head
  * RMSNorm (use_norm) and rotary embedding of q and k, k and v narrowed to f16 and appended to the
  * caches at the row of start_pos, then causal attention of the new token over rows up to and
