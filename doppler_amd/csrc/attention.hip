@@ -34,6 +34,7 @@ struct AttnArgs {
   float* O;             // [H][D]
   float* ws;            // [H][nsplit][D + 2]  (o..., m, l)
   int H, Hkv, G, kbeg, kend, nsplit, tiles_per_split;
+  int direct;           // one split and no merge launch behind it: the split kernel writes O itself
   float scale, softcap;
   int kv_start, ring_window;  // ring_window > 0: row = (kv_start + k) % ring_window
   // ---- QKV variant only
@@ -426,7 +427,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
     for (int k = 0; k < KH; k++) v += o_lds[wave][k][g][dim];
     if (o < GT * DW && g < G) {
       const int h = kvh * G + g;
-      if (a.nsplit == 1) {
+      if (a.direct) {
         float l = 0.f;
 #pragma unroll
         for (int gg = 0; gg < GT; gg++) l = gg == g ? l_run[gg] : l;
@@ -436,7 +437,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
       }
     }
   }
-  if (a.nsplit > 1 && wave == 0 && lane < G) {
+  if (!a.direct && wave == 0 && lane < G) {
     float* w = a.ws + ((int64_t)(kvh * G + lane) * a.nsplit + split) * (D + 2);
     float mv = 0.f, lv = 0.f;
 #pragma unroll
@@ -529,17 +530,73 @@ int choose_splits(int Hkv, int nkeys) {
   return (tiles + chunks_each - 1) / chunks_each;
 }
 
+typedef void (*SplitKernel)(const AttnArgs);
+typedef void (*MergeKernel)(const float*, float*, int);
+
 template <int D, bool QKV>
-int launch(const AttnArgs& a, const char* op) {
-  const dim3 grid(a.Hkv, a.nsplit), block(256);
-  if (a.G <= 1) hipLaunchKernelGGL((attn_decode_split_kernel<D, 1, QKV>), grid, block, 0, dh::stream(), a);
-  else if (a.G <= 2) hipLaunchKernelGGL((attn_decode_split_kernel<D, 2, QKV>), grid, block, 0, dh::stream(), a);
-  else if (a.G <= 4) hipLaunchKernelGGL((attn_decode_split_kernel<D, 4, QKV>), grid, block, 0, dh::stream(), a);
-  else hipLaunchKernelGGL((attn_decode_split_kernel<D, 8, QKV>), grid, block, 0, dh::stream(), a);
+SplitKernel split_kernel_for(int G) {
+  if (G <= 1) return attn_decode_split_kernel<D, 1, QKV>;
+  if (G <= 2) return attn_decode_split_kernel<D, 2, QKV>;
+  if (G <= 4) return attn_decode_split_kernel<D, 4, QKV>;
+  return attn_decode_split_kernel<D, 8, QKV>;
+}
+SplitKernel split_kernel_for(int D, bool qkv, int G) {
+  if (D == 64) return qkv ? split_kernel_for<64, true>(G) : split_kernel_for<64, false>(G);
+  return qkv ? split_kernel_for<128, true>(G) : split_kernel_for<128, false>(G);
+}
+MergeKernel merge_kernel_for(int D) { return D == 64 ? attn_decode_merge_kernel<64> : attn_decode_merge_kernel<128>; }
+
+int launch(const AttnArgs& a, int D, bool qkv, const char* op) {
+  hipLaunchKernelGGL(split_kernel_for(D, qkv, a.G), dim3(a.Hkv, a.nsplit), dim3(256), 0, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
-  if (a.nsplit > 1) {
-    hipLaunchKernelGGL(attn_decode_merge_kernel<D>, dim3(a.H), dim3(D), 0, dh::stream(), a.ws, a.O, a.nsplit);
+  if (!a.direct) {
+    hipLaunchKernelGGL(merge_kernel_for(D), dim3(a.H), dim3(D), 0, dh::stream(), a.ws, a.O, a.nsplit);
     DH_CHECK_LAUNCH(op);
+  }
+  return 0;
+}
+
+// Host-side arithmetic of one decode attention call at position shift `delta` from the recorded one:
+// visible key range, key splits, and for the stacked-projection form the rotary rows and the
+// appended cache row.  Returns 1 when no key is visible (the caller zero-fills O), 0 otherwise.
+int build_args(const dh::GraphAttnCall& c, int delta, bool force_merge, AttnArgs& a) {
+  const int start_pos = c.start_pos + delta;
+  const int kv_len = c.kv_len + delta;
+  int64_t kbeg = 0, kend;
+  if (c.qkv) {
+    kend = (int64_t)start_pos - c.kv_start + 1;
+  } else {
+    kend = kv_len;
+    if (c.causal) kend = std::min<int64_t>(kend, (int64_t)start_pos - c.kv_start + 1);
+  }
+  if (c.sliding_window > 0 && start_pos >= c.sliding_window)
+    kbeg = std::max<int64_t>(0, (int64_t)start_pos - c.sliding_window + 1 - c.kv_start);
+  if (kend <= kbeg) return 1;
+  a = AttnArgs{};
+  a.K = static_cast<const __half*>(c.K); a.V = static_cast<const __half*>(c.V);
+  a.O = c.O; a.ws = static_cast<float*>(c.ws);
+  a.H = c.H; a.Hkv = c.Hkv; a.G = c.H / c.Hkv;
+  a.kbeg = (int)kbeg; a.kend = (int)kend;
+  const int nkeys = (int)(kend - kbeg);
+  a.nsplit = choose_splits(c.Hkv, nkeys);
+  a.direct = (a.nsplit == 1 && !force_merge) ? 1 : 0;
+  a.scale = c.scale; a.softcap = c.softcap;
+  a.kv_start = c.kv_start;
+  a.ring_window = c.kv_layout == DH_KV_RING ? c.sliding_window : 0;
+  if (c.qkv) {
+    const int half = c.rotary_dim / 2;
+    a.Kw = static_cast<__half*>(c.K); a.Vw = static_cast<__half*>(c.V);
+    a.qkv = c.q; a.qw = c.qw; a.kw = c.kw;
+    a.cos_row = c.cos + (int64_t)start_pos * half;
+    a.sin_row = c.sin + (int64_t)start_pos * half;
+    a.rotary_half = half; a.interleaved = c.interleaved; a.w_offset = c.weight_offset; a.use_norm = c.use_norm;
+    a.eps = c.eps;
+    const int64_t row = a.ring_window > 0 ? start_pos % a.ring_window : start_pos;
+    a.new_row = row * c.Hkv * c.D;
+    a.c_new = (nkeys - 1) / kTileKeys;
+    a.j_new = (nkeys - 1) % kTileKeys;
+  } else {
+    a.Q = c.q;
   }
   return 0;
 }
@@ -558,6 +615,104 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 static void* g_scratch_ptr[kMaxDevices] = {};
 
 namespace dh {
+// The captured graph is a chain (one stream): walking it from its root visits the kernel nodes in
+// launch order.  Every recorded attention call owns the next node that runs its split kernel and
+// the merge node behind it.
+int attn_graph_bind(Graph* g) {
+  if (g->n_attn == 0) return 0;
+  size_t n = 0;
+  DH_CHECK_HIP("dh_graph_end", hipGraphGetNodes(g->graph, nullptr, &n));
+  hipGraphNode_t* nodes = new hipGraphNode_t[n ? n : 1];
+  hipError_t e = hipGraphGetNodes(g->graph, nodes, &n);
+  if (e != hipSuccess) {
+    delete[] nodes;
+    return fail(2, "[dh_graph_end] hipGraphGetNodes failed: %s", hipGetErrorString(e));
+  }
+  // order the nodes along the chain: repeatedly take the node whose dependencies are all placed
+  hipGraphNode_t* order = new hipGraphNode_t[n ? n : 1];
+  size_t placed = 0;
+  {
+    size_t nroot = 0;
+    e = hipGraphGetRootNodes(g->graph, nullptr, &nroot);
+    hipGraphNode_t cur = nullptr;
+    if (e == hipSuccess && nroot == 1) e = hipGraphGetRootNodes(g->graph, &cur, &nroot);
+    if (e != hipSuccess || nroot != 1) {
+      delete[] nodes; delete[] order;
+      return fail(2, "[dh_graph_end] the captured graph is not a single chain (%zu roots)", nroot);
+    }
+    while (cur && placed < n) {
+      order[placed++] = cur;
+      size_t nd = 0;
+      if (hipGraphNodeGetDependentNodes(cur, nullptr, &nd) != hipSuccess || nd > 1) {
+        delete[] nodes; delete[] order;
+        return fail(2, "[dh_graph_end] the captured graph is not a single chain");
+      }
+      hipGraphNode_t next = nullptr;
+      if (nd == 1 && hipGraphNodeGetDependentNodes(cur, &next, &nd) != hipSuccess) next = nullptr;
+      cur = nd == 1 ? next : nullptr;
+    }
+  }
+  delete[] nodes;
+  int ci = 0;
+  bool want_merge = false;
+  for (size_t i = 0; i < placed && ci <= g->n_attn; i++) {
+    hipGraphNodeType type;
+    if (hipGraphNodeGetType(order[i], &type) != hipSuccess || type != hipGraphNodeTypeKernel) continue;
+    hipKernelNodeParams kp{};
+    if (hipGraphKernelNodeGetParams(order[i], &kp) != hipSuccess) continue;
+    if (want_merge) {
+      if (kp.func == reinterpret_cast<void*>(merge_kernel_for(g->attn[ci].D))) {
+        g->attn[ci].merge_node = order[i];
+        want_merge = false;
+        ci++;
+      }
+      continue;
+    }
+    if (ci < g->n_attn) {
+      const GraphAttnCall& c = g->attn[ci];
+      if (kp.func == reinterpret_cast<void*>(split_kernel_for(c.D, c.qkv != 0, c.H / c.Hkv))) {
+        g->attn[ci].split_node = order[i];
+        want_merge = true;
+      }
+    }
+  }
+  delete[] order;
+  if (ci != g->n_attn || want_merge)
+    return fail(2, "[dh_graph_end] found the kernel nodes of %d of %d attention calls in the captured graph", ci, g->n_attn);
+  return 0;
+}
+
+int attn_graph_set_position(Graph* g, int position) {
+  const int delta = position - g->captured_position;
+  for (int i = 0; i < g->n_attn; i++) {
+    const GraphAttnCall& c = g->attn[i];
+    AttnArgs a;
+    if (build_args(c, delta, true, a))
+      return fail(1, "[dh_graph_launch] position %d leaves attention call %d without a visible key", position, i);
+    AttnArgs* ap = &a;
+    void* split_args[] = {ap};
+    hipKernelNodeParams sp{};
+    sp.func = reinterpret_cast<void*>(split_kernel_for(c.D, c.qkv != 0, a.G));
+    sp.gridDim = dim3(a.Hkv, a.nsplit);
+    sp.blockDim = dim3(256);
+    sp.sharedMemBytes = 0;
+    sp.kernelParams = split_args;
+    DH_CHECK_HIP("dh_graph_launch", hipGraphExecKernelNodeSetParams(g->exec, c.split_node, &sp));
+    const float* ws = a.ws;
+    float* O = a.O;
+    int nsplit = a.nsplit;
+    void* merge_args[] = {&ws, &O, &nsplit};
+    hipKernelNodeParams mp{};
+    mp.func = reinterpret_cast<void*>(merge_kernel_for(c.D));
+    mp.gridDim = dim3(a.H);
+    mp.blockDim = dim3(c.D);
+    mp.sharedMemBytes = 0;
+    mp.kernelParams = merge_args;
+    DH_CHECK_HIP("dh_graph_launch", hipGraphExecKernelNodeSetParams(g->exec, c.merge_node, &mp));
+  }
+  return 0;
+}
+
 int attn_static_scratch_init(int device) {
   if (device < 0 || device >= kMaxDevices)
     return fail(1, "[dh_init] device ordinal %d is beyond the %d the static attention scratch tracks", device, kMaxDevices);
@@ -603,12 +758,15 @@ static int attn_decode_impl(const char* op, const float* d_Q, const void* d_K, c
     return dh::fail(1, "[%s] ring layout needs slidingWindow > 0", op);
   if (!d_Q || !d_O) return dh::fail(1, "[%s] null pointer", op);
 
-  // visible key range [kbeg, kend) in cache-relative indices (abs_key = kv_start + k)
-  int64_t kbeg = 0, kend = kv_len;
-  if (causal) kend = std::min<int64_t>(kend, (int64_t)start_pos - kv_start + 1);
-  if (sliding_window > 0 && start_pos >= sliding_window)
-    kbeg = std::max<int64_t>(0, (int64_t)start_pos - sliding_window + 1 - kv_start);
-  if (kend <= kbeg) {
+  dh::GraphAttnCall c{};
+  c.qkv = 0; c.q = d_Q; c.K = const_cast<void*>(d_K); c.V = const_cast<void*>(d_V); c.O = d_O;
+  c.H = H; c.Hkv = Hkv; c.D = D; c.kv_len = kv_len; c.start_pos = start_pos; c.causal = causal;
+  c.scale = scale; c.softcap = softcap; c.sliding_window = sliding_window; c.kv_start = kv_start;
+  c.kv_layout = kv_layout; c.ws = d_workspace;
+  const bool capturing = dh::capturing_graph() != nullptr;
+  AttnArgs a;
+  if (build_args(c, 0, capturing, a)) {
+    if (capturing) return dh::fail(1, "[%s] a captured step needs at least one visible key", op);
     hipLaunchKernelGGL(zero_f32_kernel, dim3((H * D + 255) / 256), dim3(256), 0, dh::stream(), d_O, H * D);
     DH_CHECK_LAUNCH(op);
     return 0;
@@ -616,26 +774,13 @@ static int attn_decode_impl(const char* op, const float* d_Q, const void* d_K, c
   if (!d_K || !d_V) return dh::fail(1, "[%s] null pointer", op);
   if ((reinterpret_cast<uintptr_t>(d_K) | reinterpret_cast<uintptr_t>(d_V)) & 15)
     return dh::fail(1, "[%s] K/V pointers must be 16-byte aligned", op);
-
-  AttnArgs a{};
-  a.Q = d_Q; a.K = static_cast<const __half*>(d_K); a.V = static_cast<const __half*>(d_V);
-  a.O = d_O; a.ws = static_cast<float*>(d_workspace);
-  a.H = H; a.Hkv = Hkv; a.G = G;
-  a.kbeg = (int)kbeg; a.kend = (int)kend;
-  const int nkeys = (int)(kend - kbeg);
-  // workgroup (kv head, split) walks chunks split, split + nsplit, ...: never an empty split
-  const int nsplit = choose_splits(Hkv, nkeys);
-  a.tiles_per_split = 0;
-  a.nsplit = nsplit;
-  if (nsplit > 1 && !d_workspace) return dh::fail(1, "[%s] workspace is required", op);
-  const size_t ws_need = nsplit > 1 ? (size_t)H * nsplit * (D + 2) * sizeof(float) : 0;
+  if (!a.direct && !d_workspace) return dh::fail(1, "[%s] workspace is required", op);
+  const size_t ws_need = a.direct ? 0 : (size_t)H * a.nsplit * (D + 2) * sizeof(float);
   if (ws_capacity && ws_need > ws_capacity)
     return dh::fail(1, "[%s] numHeads=%d, headDim=%d with %d key splits needs %zu bytes of split partials, the "
-                       "scratch holds %zu: use dh_attn_decode with a workspace", op, H, D, nsplit, ws_need, ws_capacity);
-  a.scale = scale; a.softcap = softcap;
-  a.kv_start = kv_start;
-  a.ring_window = kv_layout == DH_KV_RING ? sliding_window : 0;
-  return D == 64 ? launch<64, false>(a, op) : launch<128, false>(a, op);
+                       "scratch holds %zu: use dh_attn_decode with a workspace", op, H, D, a.nsplit, ws_need, ws_capacity);
+  dh::graph_note_attention(c);
+  return launch(a, D, false, op);
 }
 
 int dh_attn_decode(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H, int Hkv, int D,
@@ -690,39 +835,23 @@ int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float*
     return dh::fail(1, "[%s] ring layout needs slidingWindow > 0", op);
   if (!d_qkv || !d_cos || !d_sin || !d_cache_k || !d_cache_v || !d_O) return dh::fail(1, "[%s] null pointer", op);
   if (use_norm && (!d_q_weight || !d_k_weight)) return dh::fail(1, "[%s] q/k norm weights are required", op);
-  const int half = rotary_dim / 2;
-  const float* cos_row = d_cos + (int64_t)start_pos * half;
-  const float* sin_row = d_sin + (int64_t)start_pos * half;
   if ((reinterpret_cast<uintptr_t>(d_cache_k) | reinterpret_cast<uintptr_t>(d_cache_v) |
        reinterpret_cast<uintptr_t>(d_qkv) | reinterpret_cast<uintptr_t>(d_q_weight) |
        reinterpret_cast<uintptr_t>(d_k_weight)) & 15)
     return dh::fail(1, "[%s] qkv, the norm weights and the caches must be 16-byte aligned", op);
-
-  // visible keys [kbeg, kend) in cache-relative indices; the appended position is kend - 1
-  const int64_t kend = (int64_t)start_pos - kv_start + 1;
-  int64_t kbeg = 0;
-  if (sliding_window > 0 && start_pos >= sliding_window)
-    kbeg = std::max<int64_t>(0, (int64_t)start_pos - sliding_window + 1 - kv_start);
-  AttnArgs a{};
-  a.K = static_cast<const __half*>(d_cache_k); a.V = static_cast<const __half*>(d_cache_v);
-  a.Kw = static_cast<__half*>(d_cache_k); a.Vw = static_cast<__half*>(d_cache_v);
-  a.O = d_O; a.ws = static_cast<float*>(d_workspace);
-  a.H = H; a.Hkv = Hkv; a.G = H / Hkv;
-  a.kbeg = (int)kbeg; a.kend = (int)kend;
-  const int nkeys = (int)(kend - kbeg);
-  a.nsplit = choose_splits(Hkv, nkeys);
-  if (a.nsplit > 1 && !d_workspace) return dh::fail(1, "[%s] workspace is required", op);
-  a.scale = scale; a.softcap = softcap;
-  a.kv_start = kv_start;
-  a.ring_window = kv_layout == DH_KV_RING ? sliding_window : 0;
-  a.qkv = d_qkv; a.qw = d_q_weight; a.kw = d_k_weight; a.cos_row = cos_row; a.sin_row = sin_row;
-  a.rotary_half = half; a.interleaved = interleaved; a.w_offset = weight_offset; a.use_norm = use_norm;
-  a.eps = eps;
-  const int64_t row = a.ring_window > 0 ? start_pos % a.ring_window : start_pos;
-  a.new_row = row * Hkv * D;
-  a.c_new = (nkeys - 1) / kTileKeys;
-  a.j_new = (nkeys - 1) % kTileKeys;
-  return D == 64 ? launch<64, true>(a, op) : launch<128, true>(a, op);
+  dh::GraphAttnCall c{};
+  c.qkv = 1; c.q = d_qkv; c.qw = d_q_weight; c.kw = d_k_weight; c.cos = d_cos; c.sin = d_sin;
+  c.K = d_cache_k; c.V = d_cache_v; c.O = d_O;
+  c.H = H; c.Hkv = Hkv; c.D = D; c.kv_len = start_pos - kv_start + 1; c.start_pos = start_pos; c.causal = 1;
+  c.rotary_dim = rotary_dim; c.interleaved = interleaved; c.weight_offset = weight_offset; c.use_norm = use_norm;
+  c.eps = eps; c.scale = scale; c.softcap = softcap; c.sliding_window = sliding_window; c.kv_start = kv_start;
+  c.kv_layout = kv_layout; c.ws = d_workspace;
+  const bool capturing = dh::capturing_graph() != nullptr;
+  AttnArgs a;
+  if (build_args(c, 0, capturing, a)) return dh::fail(2, "[%s] internal: no visible key", op);
+  if (!a.direct && !d_workspace) return dh::fail(1, "[%s] workspace is required", op);
+  dh::graph_note_attention(c);
+  return launch(a, D, true, op);
 }
 
 }  // extern "C"

@@ -51,6 +51,45 @@ int q4k_gemm_gate_up(const char* op, const float* A, const uint8_t* Wg, const ui
                      int hidden, int inter, int activation, float alpha, float clamp_max,
                      const float* norm_weight = nullptr, float norm_eps = 0.f, int norm_weight_offset = 0);
 
+// ---- captured decode steps (dh_graph_*, dh_runtime.hip) ---------------------------------------
+// One decode attention call made while a graph was being captured: everything needed to redo its
+// host-side arithmetic (visible key range, key splits, rotary table row, appended cache row) for
+// another position and patch the two kernel nodes it became.
+struct GraphAttnCall {
+  int qkv;                 // 1: dh_attn_decode_qkv, 0: dh_attn_decode
+  const float* q;          // Q [H][D], or the stacked qkv projection
+  const float* qw;
+  const float* kw;
+  const float* cos;
+  const float* sin;
+  void* K;
+  void* V;
+  float* O;
+  int H, Hkv, D;
+  int kv_len, start_pos;   // at capture time
+  int causal;
+  int rotary_dim, interleaved, weight_offset, use_norm;
+  float eps, scale, softcap;
+  int sliding_window, kv_start, kv_layout;
+  void* ws;
+  hipGraphNode_t split_node, merge_node;
+};
+struct Graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  int position = 0;                       // position the node parameters currently stand at
+  int captured_position = 0;
+  GraphAttnCall* attn = nullptr;
+  int n_attn = 0, cap_attn = 0;
+};
+// The graph being captured on the op stream, or null.
+Graph* capturing_graph();
+// attention.hip: records a call for the graph being captured (no-op outside a capture).
+void graph_note_attention(const GraphAttnCall& call);
+// attention.hip: finds the kernel nodes of the recorded calls in the captured graph / patches them for `position`.
+int attn_graph_bind(Graph* g);
+int attn_graph_set_position(Graph* g, int position);
+
 // Looks up, once per device, the address of the fixed device array that dh_attn_decode_static uses
 // for its split partials (attention.hip).  Called by dh_init with the device current.
 int attn_static_scratch_init(int device);

@@ -12,6 +12,7 @@ int g_device = -1;
 hipStream_t g_own_stream = nullptr;
 hipStream_t g_stream = nullptr;
 int g_num_cus = 0;
+dh::Graph* g_capturing = nullptr;     // graph being captured on g_stream
 unsigned* g_chain_mem = nullptr;     // [8 * 64] barrier counters + [1] error flag
 unsigned g_chain_value = 0;          // what every counter reads once the enqueued launches are done
 float* g_splitk_ws = nullptr;        // partial products of the split-K prefill GEMM
@@ -34,6 +35,20 @@ int fail(int code, const char* fmt, ...) {
 hipStream_t stream() { return g_stream; }
 bool ready() { return g_ready; }
 int num_cus() { return g_num_cus; }
+Graph* capturing_graph() { return g_capturing; }
+void graph_note_attention(const GraphAttnCall& call) {
+  Graph* g = g_capturing;
+  if (!g) return;
+  if (g->n_attn == g->cap_attn) {
+    const int cap = g->cap_attn ? 2 * g->cap_attn : 64;
+    GraphAttnCall* grown = new GraphAttnCall[cap];
+    for (int i = 0; i < g->n_attn; i++) grown[i] = g->attn[i];
+    delete[] g->attn;
+    g->attn = grown;
+    g->cap_attn = cap;
+  }
+  g->attn[g->n_attn++] = call;
+}
 float* splitk_workspace(size_t* bytes) {
   *bytes = g_splitk_ws ? kSplitKWsBytes : 0;
   return g_splitk_ws;
@@ -153,6 +168,7 @@ int dh_malloc(size_t bytes, void** d_out) {
 
 int dh_free(void* d_ptr) {
   DH_REQUIRE_INIT("dh_free");
+  if (g_capturing) return dh::fail(1, "[dh_free] not possible while a graph is being captured (it waits for the stream)");
   if (!d_ptr) return 0;
   DH_CHECK_HIP("dh_free", hipStreamSynchronize(g_stream));
   DH_CHECK_HIP("dh_free", hipFree(d_ptr));
@@ -161,6 +177,7 @@ int dh_free(void* d_ptr) {
 
 int dh_upload(void* d_dst, size_t dst_offset, const void* host_src, size_t bytes) {
   DH_REQUIRE_INIT("dh_upload");
+  if (g_capturing) return dh::fail(1, "[dh_upload] not possible while a graph is being captured (it waits for the stream)");
   if (bytes == 0) return 0;
   if (!d_dst || !host_src) return dh::fail(1, "[dh_upload] null pointer");
   // Pageable host memory: hipMemcpyAsync stages it before returning, so the caller may
@@ -173,6 +190,7 @@ int dh_upload(void* d_dst, size_t dst_offset, const void* host_src, size_t bytes
 
 int dh_download(void* host_dst, const void* d_src, size_t src_offset, size_t bytes) {
   DH_REQUIRE_INIT("dh_download");
+  if (g_capturing) return dh::fail(1, "[dh_download] not possible while a graph is being captured (it waits for the stream)");
   if (bytes == 0) return 0;
   if (!host_dst || !d_src) return dh::fail(1, "[dh_download] null pointer");
   DH_CHECK_HIP("dh_download", hipMemcpyAsync(host_dst, static_cast<const char*>(d_src) + src_offset,
@@ -240,8 +258,80 @@ int dh_event_destroy(void* ev) {
   return 0;
 }
 
+// ---- captured decode steps -------------------------------------------------------------------
+int dh_graph_begin(void) {
+  DH_REQUIRE_INIT("dh_graph_begin");
+  if (g_capturing) return dh::fail(1, "[dh_graph_begin] a capture is already in progress");
+  DH_CHECK_HIP("dh_graph_begin", hipStreamSynchronize(g_stream));
+  g_capturing = new dh::Graph();
+  const hipError_t e = hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal);
+  if (e != hipSuccess) {
+    delete g_capturing;
+    g_capturing = nullptr;
+    return dh::fail(2, "[dh_graph_begin] hipStreamBeginCapture failed: %s", hipGetErrorString(e));
+  }
+  return 0;
+}
+
+static void graph_free(dh::Graph* g) {
+  if (!g) return;
+  if (g->exec) (void)hipGraphExecDestroy(g->exec);
+  if (g->graph) (void)hipGraphDestroy(g->graph);
+  delete[] g->attn;
+  delete g;
+}
+
+int dh_graph_end(int position, void** graph_out) {
+  DH_REQUIRE_INIT("dh_graph_end");
+  if (!graph_out) return dh::fail(1, "[dh_graph_end] output pointer is null");
+  *graph_out = nullptr;
+  if (!g_capturing) return dh::fail(1, "[dh_graph_end] no capture in progress");
+  dh::Graph* g = g_capturing;
+  g_capturing = nullptr;
+  hipError_t e = hipStreamEndCapture(g_stream, &g->graph);
+  if (e != hipSuccess || !g->graph) {
+    graph_free(g);
+    return dh::fail(2, "[dh_graph_end] hipStreamEndCapture failed: %s", hipGetErrorString(e));
+  }
+  e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    graph_free(g);
+    return dh::fail(2, "[dh_graph_end] hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  }
+  g->position = g->captured_position = position;
+  if (int rc = dh::attn_graph_bind(g)) {
+    graph_free(g);
+    return rc;
+  }
+  *graph_out = g;
+  return 0;
+}
+
+int dh_graph_launch(void* graph, int position) {
+  DH_REQUIRE_INIT("dh_graph_launch");
+  dh::Graph* g = static_cast<dh::Graph*>(graph);
+  if (!g || !g->exec) return dh::fail(1, "[dh_graph_launch] null graph");
+  if (g_capturing) return dh::fail(1, "[dh_graph_launch] a capture is in progress");
+  if (position < 0) return dh::fail(1, "[dh_graph_launch] position must be non-negative");
+  if (position != g->position) {
+    if (int rc = dh::attn_graph_set_position(g, position)) return rc;
+    g->position = position;
+  }
+  DH_CHECK_HIP("dh_graph_launch", hipGraphLaunch(g->exec, g_stream));
+  return 0;
+}
+
+int dh_graph_destroy(void* graph) {
+  DH_REQUIRE_INIT("dh_graph_destroy");
+  if (!graph) return 0;
+  DH_CHECK_HIP("dh_graph_destroy", hipStreamSynchronize(g_stream));
+  graph_free(static_cast<dh::Graph*>(graph));
+  return 0;
+}
+
 int dh_sync(void) {
   DH_REQUIRE_INIT("dh_sync");
+  if (g_capturing) return dh::fail(1, "[dh_sync] not possible while a graph is being captured (it waits for the stream)");
   DH_CHECK_HIP("dh_sync", hipStreamSynchronize(g_stream));
   if (g_chain_mem) {
     // a chained GEMV that could not cross its grid barrier left its outputs incomplete

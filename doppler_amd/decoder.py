@@ -118,6 +118,10 @@ class HipDecoder:
         L, c = self.L, self.cfg
         ck = capi.check
         H, Hkv, D, Hd, I = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"], c["inter"]
+        if not 0 <= pos < self.max_seq:
+            # the ops take no cache capacity: a position past the caches would write K/V and read
+            # the rotary tables out of bounds
+            raise ValueError("decode position %d is outside the KV cache (max_seq=%d)" % (pos, self.max_seq))
         ids = self.token if from_device_token else self.ids
         ck(L.dh_gather_f16(ids.data_ptr(), self.embed.data_ptr(), self.x.data_ptr(), 1, Hd, c["vocab"],
                            in_index if from_device_token else 0))
@@ -238,6 +242,41 @@ class HipDecoder:
             self._enqueue_sample(sampling)
         return self.read_token()
 
+    def capture_step(self, pos, want_logits=False):
+        """Captures one decode step (enqueued for position `pos`) into a HIP graph, the
+        counterpart of the reference's one-submit-per-step recorder
+        (src/inference/pipelines/text/generator-steps.js:605,814).  The step is run once
+        normally first so that every kernel's one-time set-up is done outside the capture."""
+        if not self.fuse_qkv_attention or self.chain:
+            raise ValueError("capture_step serves the fused-attention, unchained step")
+        self.enqueue_step(pos, want_logits)
+        capi.check(self.L.dh_sync())
+        capi.check(self.L.dh_graph_begin())
+        try:
+            self.enqueue_step(pos, want_logits)
+        finally:
+            g = ctypes.c_void_p()
+            rc = self.L.dh_graph_end(pos, ctypes.byref(g))
+        capi.check(rc)
+        self._graph = g
+        return g
+
+    def step_graph(self, token, pos):
+        """One decode step by replaying the captured graph at position `pos`: one graph launch
+        and the 4-byte token readback."""
+        if not 0 <= pos < self.max_seq:
+            raise ValueError("decode position %d is outside the KV cache (max_seq=%d)" % (pos, self.max_seq))
+        if getattr(self, "_graph", None) is None:
+            self.capture_step(pos)
+        self.set_token(token)
+        capi.check(self.L.dh_graph_launch(self._graph, pos))
+        return self.read_token()
+
+    def release_graph(self):
+        if getattr(self, "_graph", None) is not None:
+            capi.check(self.L.dh_graph_destroy(self._graph))
+            self._graph = None
+
     def _enqueue_sample(self, sampling, out_index=0):
         from . import ops
         L, c = self.L, self.cfg
@@ -256,6 +295,9 @@ class HipDecoder:
         randomSeed seed + i (greedy when None)."""
         draw = (lambda i: dict(temperature=sampling["temperature"], topK=sampling["topK"], randomSeed=sampling["seed"] + i)) \
             if sampling else (lambda i: None)
+        if len(prompt) + max_tokens - 1 > self.max_seq:
+            raise ValueError("prompt of %d tokens plus %d generated does not fit max_seq=%d" %
+                             (len(prompt), max_tokens, self.max_seq))
         tok = self.prefill(prompt, chunk=chunk, sampling=draw(0))
         out = [tok]
         for i in range(1, max_tokens):

@@ -65,6 +65,23 @@ int dh_event_record(void* ev);
 int dh_event_elapsed_ms(void* start, void* stop, float* ms_out);
 int dh_event_destroy(void* ev);
 
+/* ---- captured decode steps ----
+ * The reference records a whole decode step into one command encoder and submits it once
+ * (src/inference/pipelines/text/generator-steps.js:588-820 decodeStep: recorder at :605, submit at
+ * :814; the pre-allocated per-step buffers of src/inference/decode-ring.js make the step replayable).
+ * Here: every op enqueued between dh_graph_begin and dh_graph_end is captured into a HIP graph
+ * instead of running; dh_graph_launch replays the whole step with one call.  `position` is the
+ * token position the captured step was enqueued for; dh_graph_launch(graph, p) first moves the
+ * decode attention calls of the step (dh_attn_decode, dh_attn_decode_qkv: start_pos, kv_len, key
+ * splits, rotary row, appended cache row) to position p by patching their kernel nodes, everything
+ * else (pointers, shapes) replays as captured.  Captured steps must keep at least one key visible.
+ * Calls that wait for the stream (dh_upload, dh_download, dh_sync, dh_free) fail during a capture;
+ * ops never allocate and dh_fill_zero is a kernel, so nothing in a step is unsuitable for capture. */
+int dh_graph_begin(void);
+int dh_graph_end(int position, void** graph_out);
+int dh_graph_launch(void* graph, int position);
+int dh_graph_destroy(void* graph);
+
 /* ---- Q4_K ---- */
 
 /* Dequantize `num_blocks` super-blocks to f32 (bit-exact with
