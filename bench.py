@@ -87,6 +87,42 @@ def js_reference_timings():
         return None
 
 
+def js_host_decode(cfg, layers, embed, final_norm, prefill, warmup, steps):
+    """Decode tokens/s of the JavaScript host on the same model: node subprocess over
+    doppler_amd/js/bench/decode_bench.mjs (loader -> prefill -> decodeStep loop, then the
+    captured-graph loop).  Returns its JSON, or None when node or the addon is missing."""
+    import shutil
+    import subprocess
+    import tempfile
+    from doppler_amd import rdrr
+    node = shutil.which("node")
+    addon = os.path.join(ROOT, "doppler_amd", "js", "doppler_hip.node")
+    if not node or not os.path.exists(addon):
+        log("[bench] JS host skipped (node or the addon missing)")
+        return None
+    base = "/dev/shm" if os.path.isdir("/dev/shm") and os.access("/dev/shm", os.W_OK) else None
+    d = tempfile.mkdtemp(prefix="doppler_amd_bench_", dir=base)
+    try:
+        t0 = time.time()
+        rdrr.write_artifact(d, cfg, layers, embed, final_norm, shard_bytes=256 << 20)
+        log("[bench] artifact for the JS host written in %.1f s" % (time.time() - t0))
+        r = subprocess.run([node, os.path.join(ROOT, "doppler_amd", "js", "bench", "decode_bench.mjs"), d, str(prefill),
+                            str(warmup), str(steps), "graph"], capture_output=True, text=True, timeout=600)
+        if r.returncode != 0:
+            log("[bench] JS host failed: %s" % r.stderr[-2000:])
+            return None
+        res = json.loads(r.stdout.strip().splitlines()[-1])
+        for k in ("tokens_per_s", "ms_per_step", "graph_tokens_per_s", "graph_ms_per_step"):
+            if k in res:
+                res[k] = round(res[k], 3)
+        return res
+    except Exception as e:      # a side measurement, never a reason to lose the GPU result
+        log("[bench] JS host failed: %r" % (e,))
+        return None
+    finally:
+        shutil.rmtree(d, ignore_errors=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,6 +131,7 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="debug only: fewer layers (result is not the metric)")
     ap.add_argument("--prefill", type=int, default=None, help="debug only: shorter prefill")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-js-host", action="store_true", help="skip the JavaScript-host side measurement")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three f32->f16 casts of 16 Mi elements (64 MiB read, 32 MiB written): a "
                          "streaming kernel of known traffic to scale rocprofv3 FETCH_SIZE / WRITE_SIZE with")
@@ -119,7 +156,7 @@ def main():
     if args.prefill is not None:
         prefill = args.prefill
     BATCH = 16                       # extra positions for the batched-decode side measurement
-    max_seq = prefill + args.warmup + args.steps + 2 * BATCH + 1
+    max_seq = prefill + args.warmup + args.steps + 2 * BATCH + 40
     cfg = dict(c, max_seq=max_seq)
 
     t0 = time.time()
@@ -173,6 +210,22 @@ def main():
     batched_tok_s = BATCH / (time.perf_counter() - t0)
     log("[bench] batched decode, %d tokens per submit: %.1f tok/s" % (BATCH, batched_tok_s))
 
+    # ---- side measurement: the step captured once into a HIP graph and replayed (one launch per
+    #      token instead of ~220); same kernels, same readback
+    pos_g = pos + 2 * BATCH
+    gtok = dec.step_graph(tok, pos_g)                 # eager run + capture + first replay
+    for i in range(1, 4):
+        gtok = dec.step_graph(gtok, pos_g + i)
+    capi_sync()
+    n_graph = min(32, max_seq - (pos_g + 4))
+    t0 = time.perf_counter()
+    for i in range(n_graph):
+        gtok = dec.step_graph(gtok, pos_g + 4 + i)
+    capi_sync()
+    graph_tok_s = n_graph / (time.perf_counter() - t0)
+    dec.release_graph()
+    log("[bench] graph replay: %.1f tok/s" % graph_tok_s)
+
     # ---- roofline of the dominant kernel
     Hd, I = cfg["hidden"], cfg["inter"]
     launch_bytes = 2 * synth.q4k_nbytes(I, Hd) + 2 * Hd * 4 + I * 4      # weights, x + norm weight, output
@@ -181,7 +234,9 @@ def main():
     roofline = {"bound": "hbm", "kernel": "q4k fused RMSNorm + gate/up GEMV + SiLU [2x12288x4096]", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "bytes_per_launch": launch_bytes, "avg_launch_us": round(avg_ms * 1e3, 2),
-                "traffic": GATE_UP_TRAFFIC_BYTES if (Hd, I) == (4096, 12288) else None}
+                "traffic": GATE_UP_TRAFFIC_BYTES if (Hd, I) == (4096, 12288) else None,
+                "traffic_source": "stored figure from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised under "
+                                  "profiles/ (not measured in this run)"}
 
     if args.copy_calibration:
         # a streaming kernel of known traffic: reads 64 MiB of f32, writes 32 MiB of f16
@@ -223,6 +278,12 @@ def main():
                # restated in JS and timed under this host's node, per-op, on the small configs
                "js_port_single_thread_ms": js}
 
+    # ---- the same model through the JavaScript host (the reference's host language): RDRR artifact
+    #      written to memory-backed storage, read by the JS loader, decoded through the N-API addon
+    js_host = None
+    if not args.no_js_host:
+        js_host = js_host_decode(cfg, layers, embed, final_norm, prefill, args.warmup, min(args.steps, 48))
+
     out = {
         "metric": "decode tokens/sec at 9B-class Q4_K, 1 GPU (Q4_K GEMV HBM GB/s in roofline)",
         "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -233,6 +294,8 @@ def main():
                    "layers": cfg["layers"], "context": prefill, "algorithmic_bytes_per_step": step_bytes,
                    "hbm_frac_whole_step": round(step_bytes * tok_s / 1e9 / HBM_PEAK_GBPS, 4),
                    "batched_decode_16_per_submit_tokens_per_s": round(batched_tok_s, 2),
+                   "graph_replay_tokens_per_s": round(graph_tok_s, 2),
+                   "js_host": js_host,
                    "prefill_tokens_per_s": round(prefill / prefill_s, 1)},
         "roofline": roofline,
         "cpu_baseline": cpu,

@@ -45,6 +45,7 @@ SIGNATURES = {
     "dh_graph_begin": (_I, []),
     "dh_graph_end": (_I, [_I, ctypes.POINTER(_P)]),
     "dh_graph_launch": (_I, [_P, _I]),
+    "dh_graph_prepare": (_I, [_P, _I]),
     "dh_graph_destroy": (_I, [_P]),
     "dh_q4k_dequant": (_I, [_P, _I64, _P]),
     "dh_q4k_matmul": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _F, _P]),

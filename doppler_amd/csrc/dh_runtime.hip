@@ -321,6 +321,18 @@ int dh_graph_launch(void* graph, int position) {
   return 0;
 }
 
+int dh_graph_prepare(void* graph, int position) {
+  DH_REQUIRE_INIT("dh_graph_prepare");
+  dh::Graph* g = static_cast<dh::Graph*>(graph);
+  if (!g || !g->exec) return dh::fail(1, "[dh_graph_prepare] null graph");
+  if (position < 0) return dh::fail(1, "[dh_graph_prepare] position must be non-negative");
+  if (position != g->position) {
+    if (int rc = dh::attn_graph_set_position(g, position)) return rc;
+    g->position = position;
+  }
+  return 0;
+}
+
 int dh_graph_destroy(void* graph) {
   DH_REQUIRE_INIT("dh_graph_destroy");
   if (!graph) return 0;

@@ -84,6 +84,18 @@ static napi_value ret_num(napi_env env, double d) {
 #define L(i, var) int64_t var; if (!arg_i64(env, a[i], &var)) return NULL
 #define F(i, var) float var; if (!arg_f32(env, a[i], &var)) return NULL
 
+/* ---- captured decode steps ---- */
+FN(js_graph_begin) { (void)info; return ret_rc(env, dh_graph_begin()); }
+FN(js_graph_end) {
+  ARGS(1); I(0, position);
+  void* g = NULL;
+  if (dh_graph_end(position, &g) != 0) return fail(env, dh_last_error());
+  return ret_ptr(env, g);
+}
+FN(js_graph_launch) { ARGS(2); P(0, g); I(1, position); return ret_rc(env, dh_graph_launch(g, position)); }
+FN(js_graph_prepare) { ARGS(2); P(0, g); I(1, position); return ret_rc(env, dh_graph_prepare(g, position)); }
+FN(js_graph_destroy) { ARGS(1); P(0, g); return ret_rc(env, dh_graph_destroy(g)); }
+
 /* ---- device / memory ---- */
 FN(js_init) { ARGS(1); I(0, dev); return ret_rc(env, dh_init(dev)); }
 FN(js_shutdown) { (void)info; return ret_rc(env, dh_shutdown()); }
@@ -178,6 +190,13 @@ FN(js_attn_decode) {
   return ret_rc(env, dh_attn_decode((const float*)Q, K, V, (float*)O, H, Hkv, D, kvLen, scale, causal, startPos, cap, win,
                                     kvStart, layout, ws));
 }
+FN(js_attn_decode_static) {
+  ARGS(15); P(0, Q); P(1, K); P(2, V); P(3, O); I(4, H); I(5, Hkv); I(6, D); I(7, kvLen); F(8, scale); I(9, causal);
+  I(10, startPos); F(11, cap); I(12, win); I(13, kvStart); I(14, layout);
+  return ret_rc(env, dh_attn_decode_static((const float*)Q, K, V, (float*)O, H, Hkv, D, kvLen, scale, causal, startPos, cap,
+                                           win, kvStart, layout));
+}
+FN(js_attn_decode_static_max_bytes) { (void)info; return ret_num(env, (double)dh_attn_decode_static_max_bytes()); }
 FN(js_attn_decode_qkv_supported) {
   ARGS(5); I(0, H); I(1, Hkv); I(2, D); I(3, rd); I(4, inter);
   return ret_num(env, (double)dh_attn_decode_qkv_supported(H, Hkv, D, rd, inter));
@@ -276,6 +295,8 @@ FN(js_cast_f16_to_f32) { ARGS(3); P(0, i); P(1, o); L(2, n); return ret_rc(env, 
 
 static napi_value module_init(napi_env env, napi_value exports) {
   static const struct { const char* name; napi_callback fn; } table[] = {
+      {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end}, {"graphLaunch", js_graph_launch}, {"graphPrepare", js_graph_prepare},
+      {"graphDestroy", js_graph_destroy},
       {"init", js_init}, {"shutdown", js_shutdown}, {"sync", js_sync}, {"malloc", js_malloc}, {"free", js_free},
       {"upload", js_upload}, {"download", js_download}, {"copy", js_copy}, {"fillZero", js_fill_zero},
       {"eventCreate", js_event_create}, {"eventRecord", js_event_record}, {"eventElapsedMs", js_event_elapsed_ms},
@@ -284,6 +305,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"q4kMatmulRmsnorm", js_q4k_matmul_rmsnorm}, {"q4kFfnGateUpRmsnorm", js_q4k_ffn_gate_up_rmsnorm},
       {"lmheadArgmaxWorkspaceBytes", js_lmhead_argmax_workspace_bytes}, {"lmheadArgmaxF16", js_lmhead_argmax_f16},
       {"attnDecodeWorkspaceBytes", js_attn_decode_workspace_bytes}, {"attnDecode", js_attn_decode},
+      {"attnDecodeStatic", js_attn_decode_static}, {"attnDecodeStaticMaxBytes", js_attn_decode_static_max_bytes},
       {"attnDecodeQkvSupported", js_attn_decode_qkv_supported}, {"attnDecodeQkv", js_attn_decode_qkv},
       {"attnPrefill", js_attn_prefill},
       {"rmsnorm", js_rmsnorm}, {"rmsnormQK", js_rmsnorm_qk}, {"rmsnormSandwichPair", js_rmsnorm_sandwich_pair},

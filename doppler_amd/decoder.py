@@ -270,6 +270,9 @@ class HipDecoder:
             self.capture_step(pos)
         self.set_token(token)
         capi.check(self.L.dh_graph_launch(self._graph, pos))
+        if pos + 1 < self.max_seq:
+            # the next position's node parameters are set while the GPU runs this one
+            capi.check(self.L.dh_graph_prepare(self._graph, pos + 1))
         return self.read_token()
 
     def release_graph(self):

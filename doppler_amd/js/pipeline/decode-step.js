@@ -9,6 +9,7 @@ import {
   recordAttention, recordFusedNormedFFN, recordFusedFFN, recordLmHeadArgmaxF16, recordGPUSample,
   recordDecodeAttentionFromQKV, decodeAttentionFromQKVSupported,
 } from '../kernel-selector.js';
+import { getNative } from '../native.js';
 
 // A window of a device buffer starting `offset` bytes in (no ownership: never released).
 function bufferWindow(buffer, offset, size) {
@@ -156,13 +157,15 @@ export class HipTextDecoder {
     return out;
   }
 
-  // Returns the greedy token for `token` at position `pos` (KV rows 0..pos-1 present).
-  async decodeStep(token, pos, options = {}) {
+  // Records the ops of one decode step for the token id in this.ids at position `pos`; the new
+  // token id goes to this.tokenOut.  Temporaries are pushed onto `temps`.
+  async recordDecodeStep(recorder, temps, pos, options = {}) {
     const c = this.config;
-    const recorder = createCommandRecorder('decode');
-    const temps = [];
+    if (!(pos >= 0 && pos < c.maxSeq)) {
+      // the ops take no cache capacity: a position past the caches would write K/V out of bounds
+      throw new Error(`[decodeStep] position ${pos} is outside the KV cache (maxSeq=${c.maxSeq})`);
+    }
     const temp = (t) => { temps.push(t.buffer); return t; };
-    uploadData(this.ids, new Uint32Array([token]));
     let x = temp(await recordGather(recorder, this.ids, this.embed, 1, c.hidden, c.vocab,
       { embeddingDtype: 'f16', outputDtype: 'f32' }));
     for (let li = 0; li < this.layers.length; li++) {
@@ -203,13 +206,67 @@ export class HipTextDecoder {
         logitsOutput: options.logitsOutput || null,
       });
     }
+  }
+
+  // Returns the greedy token for `token` at position `pos` (KV rows 0..pos-1 present).
+  // options.recorder: a recorder of the caller's (e.g. a profiling one) instead of a fresh one.
+  async decodeStep(token, pos, options = {}) {
+    const recorder = options.recorder || createCommandRecorder('decode');
+    const temps = [];
+    uploadData(this.ids, new Uint32Array([token]));
+    await this.recordDecodeStep(recorder, temps, pos, options);
     for (const b of temps) recorder.trackTemporaryBuffer(b);
     recorder.submit();
     const bytes = await readBufferSlice(this.tokenOut, 0, 4);   // the only device->host crossing
     return new Uint32Array(bytes)[0];
   }
 
+  // Captures the decode step into a HIP graph, the counterpart of the reference's
+  // one-submit-per-step recorder (generator-steps.js:605,814).  The step runs once normally first
+  // (every kernel's one-time set-up then lies outside the capture); the buffers the captured step
+  // uses stay allocated for the graph's life.
+  async captureDecodeStep(token, pos) {
+    if (!this.fuseQkvAttention) throw new Error('[captureDecodeStep] serves the fused-attention step');
+    const first = await this.decodeStep(token, pos);
+    getNative().graphBegin();
+    let graph = null;
+    const temps = [];
+    try {
+      await this.recordDecodeStep(createCommandRecorder('decode_capture'), temps, pos, {});
+    } finally {
+      graph = getNative().graphEnd(pos);
+    }
+    this.graph = graph;
+    this.graphBuffers = temps;
+    return first;
+  }
+
+  // One decode step by replaying the captured graph at position `pos`.
+  async decodeStepGraph(token, pos) {
+    const c = this.config;
+    if (!(pos >= 0 && pos < c.maxSeq)) {
+      throw new Error(`[decodeStepGraph] position ${pos} is outside the KV cache (maxSeq=${c.maxSeq})`);
+    }
+    if (!this.graph) return this.captureDecodeStep(token, pos);
+    uploadData(this.ids, new Uint32Array([token]));
+    getNative().graphLaunch(this.graph, pos);
+    // the next position's node parameters are set while the GPU runs this one
+    if (pos + 1 < c.maxSeq) getNative().graphPrepare(this.graph, pos + 1);
+    const bytes = await readBufferSlice(this.tokenOut, 0, 4);
+    return new Uint32Array(bytes)[0];
+  }
+
+  releaseGraph() {
+    if (this.graph) {
+      getNative().graphDestroy(this.graph);
+      for (const b of this.graphBuffers) releaseBuffer(b);
+      this.graph = null;
+      this.graphBuffers = [];
+    }
+  }
+
   destroy() {
+    this.releaseGraph();
     for (const l of this.layers) {
       for (const key of Object.keys(l)) releaseBuffer(l[key].buffer);
     }

@@ -80,6 +80,10 @@ int dh_event_destroy(void* ev);
 int dh_graph_begin(void);
 int dh_graph_end(int position, void** graph_out);
 int dh_graph_launch(void* graph, int position);
+/* Moves the step to `position` without launching it: a later dh_graph_launch at that position
+ * then has nothing left to patch.  Launches already enqueued keep the position they were launched
+ * at, so a host can prepare position p + 1 while the GPU still runs position p. */
+int dh_graph_prepare(void* graph, int position);
 int dh_graph_destroy(void* graph);
 
 /* ---- Q4_K ---- */

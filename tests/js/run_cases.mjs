@@ -194,9 +194,21 @@ async function main() {
       let tok = c.prompt[0];
       for (let pos = 0; pos < c.prompt.length + c.steps; pos++) {
         const inp = pos < c.prompt.length ? c.prompt[pos] : tok;
-        tok = await dec.decodeStep(inp, pos);
+        if (c.graphFrom !== undefined && pos >= c.graphFrom && pos % 5 !== 4) {
+          // replay of the captured step (captured at the first such position), an eager step now and then
+          tok = await dec.decodeStepGraph(inp, pos);
+        } else if (c.profileAt === pos) {
+          // per-label HIP-event timings of one step (reference: createProfilingRecorder + resolveProfileTimings)
+          const rec = dh.createProfilingRecorder('profiled_step');
+          tok = await dec.decodeStep(inp, pos, { recorder: rec });
+          results.profile = await rec.resolveProfileTimings();
+          results.profileOps = rec.opCount;
+        } else {
+          tok = await dec.decodeStep(inp, pos);
+        }
         tokens.push(tok);
       }
+      dec.releaseGraph();
       fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
     } else if (c.op === 'generate') {
       // RDRR artifact -> JS loader -> prefill path -> decode loop, greedy or sampled

@@ -250,6 +250,9 @@ def test_js_host_path_parity(tmp_path):
                       config=dict(layers=2, hidden=512, inter=1024, heads=8, kvHeads=4, headDim=64, vocab=700, eps=1e-6, maxSeq=24)))
     cases.append(dict(cases[-1], name="decoder_separate_qkv_kernel",
                       config=dict(cases[-1]["config"], fuseQkvAttention=False)))
+    # the same steps with the decode step captured into a HIP graph at position 3 and replayed from
+    # there on, and one step under a profiling recorder (per-label HIP-event timings)
+    cases.append(dict(cases[-2], name="decoder_graph_replay", graphFrom=3, profileAt=4))
     ol = []
     for l in layers:
         dd = dict(l)
@@ -263,6 +266,7 @@ def test_js_host_path_parity(tmp_path):
         want_tokens.append(tok)
     checks.append(lambda: [int(t) for t in get("decoder.out.bin", np.uint32)] == want_tokens)
     checks.append(lambda: [int(t) for t in get("decoder_separate_qkv_kernel.out.bin", np.uint32)] == want_tokens)
+    checks.append(lambda: [int(t) for t in get("decoder_graph_replay.out.bin", np.uint32)] == want_tokens)
 
     # ---- top-k temperature sampling through the JS op (seeded draw as in the reference)
     slog = (synth.rng(79).standard_normal(4000) * 3).astype(np.float32)
@@ -313,5 +317,12 @@ def test_js_host_path_parity(tmp_path):
     assert res["cases"] == [c["name"] for c in cases]
     for i, chk in enumerate(checks):
         assert chk(), "check %d failed" % i
+    # the profiled step: every op of the step carries a label with a positive time (2 layers x 5 ops
+    # + gather + final norm + LM head)
+    prof = res["profile"]
+    assert res["profileOps"] == 13, res["profileOps"]
+    assert set(prof) == {"gather", "matmul:qkv_proj", "attention:from_qkv", "matmul:o_proj", "fused_normed_ffn",
+                         "matmul:down_proj", "rmsnorm", "lm_head_argmax"}, prof
+    assert all(0.0 < ms < 50.0 for ms in prof.values()), prof
     bad = [e for e in res["errors"] if not e["ok"]]
     assert not bad and len(res["errors"]) >= 14, bad
