@@ -50,7 +50,6 @@ SIGNATURES = {
     "dh_q4k_dequant": (_I, [_P, _I64, _P]),
     "dh_q4k_matmul": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
     "dh_q4k_matmul_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
-    "dh_q4k_gemv_chain": (_I, [_P, _I]),
     "dh_q4k_ffn_gate_up": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
     "dh_q4k_ffn_gate_up_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
     "dh_f16w_matmul": (_I, [_P, _P, _P, _I, _I, _I, _F]),
@@ -88,13 +87,6 @@ SIGNATURES = {
     "dh_cast_f16_to_f32": (_I, [_P, _P, _I64]),
 }
 
-
-
-class GemvPhase(ctypes.Structure):
-    """dh_gemv_phase of include/doppler_hip.h."""
-    _fields_ = [("d_A", _P), ("d_norm_weight", _P), ("eps", _F), ("weight_offset", _I), ("d_W", _P), ("d_W2", _P),
-                ("d_C", _P), ("d_residual", _P), ("N", _I), ("K", _I), ("activation", _I), ("alpha", _F),
-                ("swiglu_limit", _F)]
 
 
 _lib = None

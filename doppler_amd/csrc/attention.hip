@@ -65,12 +65,6 @@ __device__ __forceinline__ float wave_sum(float v) {
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
 typedef __attribute__((ext_vector_type(4))) float float4_t;
 
-#ifdef DH_ATTN_TRACE
-__device__ unsigned long long dh_attn_trace_buf[1024 * 32];
-#define DH_ATS() do { if (tid == DH_ATTN_TRACE && tsn < 31) tsbuf[tsn++] = wall_clock64(); } while (0)
-#else
-#define DH_ATS() do {} while (0)
-#endif
 
 // Reductions across the lanes of a 16-lane row with DPP row shifts (no LDS traffic): afterwards
 // the last lane of every aligned group of `span` lanes (span = 2, 4, 8 or 16) holds the
@@ -132,11 +126,6 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int kvh = blockIdx.x, split = blockIdx.y;
-#ifdef DH_ATTN_TRACE
-  unsigned long long* tsbuf = dh_attn_trace_buf + ((blockIdx.y * gridDim.x + blockIdx.x) & 1023) * 32;
-  int tsn = 0;
-#endif
-  DH_ATS();
   const int G = a.G;
   const int64_t row_stride = (int64_t)a.Hkv * D;   // halves between consecutive keys
   const int qrow = lane & 15, kg = lane >> 4;
@@ -315,7 +304,6 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
       }
     }
   }
-  DH_ATS();
   float m_run[GT], l_run[GT], acc[GT][4];
 #pragma unroll
   for (int g = 0; g < GT; g++) {
@@ -327,7 +315,6 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
   for (int c = split; c < nchunks; c += a.nsplit) {
     const int kbase = a.kbeg + c * kTileKeys;
     const int nk = min(kTileKeys, a.kend - kbase);
-    DH_ATS();
     // ---- scores of 16 keys x G heads
     float4_t d = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -350,9 +337,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
       if (2 * kg < GT) s_lds[2 * kg][key_s] = valid ? sc2[0] : -FLT_MAX;
       if (2 * kg + 1 < GT) s_lds[2 * kg + 1][key_s] = valid ? sc2[1] : -FLT_MAX;
     }
-    DH_ATS();
     __syncthreads();
-    DH_ATS();
     // ---- online softmax: lane (head sm_g, group sm_q) owns keys sm_q*GT .. sm_q*GT + GT - 1
     {
       float sc[GT], pr[GT];
@@ -392,7 +377,6 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
         acc[g][0] *= alpha[g]; acc[g][1] *= alpha[g]; acc[g][2] *= alpha[g]; acc[g][3] *= alpha[g];
       }
     }
-    DH_ATS();
     // ---- P.V for this wave's dims (p_lds[wave] is private to the wave: program order suffices)
 #pragma unroll
     for (int j = 0; j < NJ; j++) {
@@ -408,10 +392,8 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
         acc[g][3] = fmaf(p, v23.y, acc[g][3]);
       }
     }
-    DH_ATS();
     __syncthreads();     // s_lds is rewritten by the next chunk
   }
-  DH_ATS();
 #undef DH_ATTN_LOAD
 #undef DH_ATTN_PATCH
 
@@ -447,10 +429,6 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
     w[D] = mv;
     w[D + 1] = lv;
   }
-  DH_ATS();
-#ifdef DH_ATTN_TRACE
-  if (tid == DH_ATTN_TRACE) tsbuf[31] = tsn;
-#endif
 }
 
 // One workgroup per query head: out[d] = sum_s e^{m_s - M} o_s[d] / sum_s e^{m_s - M} l_s.
@@ -724,11 +702,6 @@ int attn_static_scratch_init(int device) {
 }
 }  // namespace dh
 
-#ifdef DH_ATTN_TRACE
-extern "C" int dh_debug_attn_trace(void* host_dst) {
-  return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(dh_attn_trace_buf), sizeof(dh_attn_trace_buf));
-}
-#endif
 
 extern "C" {
 

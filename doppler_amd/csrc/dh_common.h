@@ -22,10 +22,6 @@ int fail(int code, const char* fmt, ...);
 hipStream_t stream();
 bool ready();
 int num_cus();
-// State of the chained-GEMV grid barrier, owned by the runtime (allocated by dh_init): eight
-// monotonic counters 256 bytes apart, an error flag the kernel raises when a barrier times out,
-// and the host's copy of the counters' value.  chain_advance(n) returns that value and adds n.
-unsigned* chain_counters();
 // Scratch for the split-K prefill GEMM's partial products (allocated by dh_init, shared by all
 // launches on the library's stream, which run in order).
 float* splitk_workspace(size_t* bytes);
@@ -34,8 +30,6 @@ float* gemm_row_scale();
 // Packed f16 activations of the prefill GEMM (rows x K rounded up to 64 halves).
 void* gemm_packed_a(size_t* bytes);
 int gemm_row_scale_capacity();
-unsigned* chain_error_flag();
-unsigned chain_advance(unsigned n);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

@@ -13,15 +13,12 @@ hipStream_t g_own_stream = nullptr;
 hipStream_t g_stream = nullptr;
 int g_num_cus = 0;
 dh::Graph* g_capturing = nullptr;     // graph being captured on g_stream
-unsigned* g_chain_mem = nullptr;     // [8 * 64] barrier counters + [1] error flag
-unsigned g_chain_value = 0;          // what every counter reads once the enqueued launches are done
 float* g_splitk_ws = nullptr;        // partial products of the split-K prefill GEMM
 constexpr size_t kSplitKWsBytes = (size_t)32 << 20;
 float* g_row_scale = nullptr;        // [kRowScaleRows][2] activation row factors of the prefill GEMM
 constexpr int kRowScaleRows = 65536;
 void* g_packed_a = nullptr;          // packed f16 activations of the prefill GEMM
 constexpr size_t kPackedABytes = (size_t)64 << 20;
-constexpr size_t kChainWords = 8 * 64 + 64;
 }  // namespace
 
 namespace dh {
@@ -59,13 +56,6 @@ void* gemm_packed_a(size_t* bytes) {
   return g_packed_a;
 }
 int gemm_row_scale_capacity() { return kRowScaleRows; }
-unsigned* chain_counters() { return g_chain_mem; }
-unsigned* chain_error_flag() { return g_chain_mem ? g_chain_mem + 8 * 64 : nullptr; }
-unsigned chain_advance(unsigned n) {
-  const unsigned v = g_chain_value;
-  g_chain_value += n;
-  return v;
-}
 }  // namespace dh
 
 extern "C" {
@@ -80,17 +70,14 @@ static int release_all(const char* op) {
     if (first == hipSuccess) first = e;
   };
   if (g_own_stream) note(hipStreamDestroy(g_own_stream));
-  if (g_chain_mem) note(hipFree(g_chain_mem));
   if (g_splitk_ws) note(hipFree(g_splitk_ws));
   if (g_row_scale) note(hipFree(g_row_scale));
   if (g_packed_a) note(hipFree(g_packed_a));
   g_own_stream = nullptr;
   g_stream = nullptr;
-  g_chain_mem = nullptr;
   g_splitk_ws = nullptr;
   g_row_scale = nullptr;
   g_packed_a = nullptr;
-  g_chain_value = 0;
   g_num_cus = 0;
   g_ready = false;
   g_device = -1;
@@ -112,9 +99,6 @@ static int init_locked(int device_ordinal) {
   DH_CHECK_HIP("dh_init", hipStreamCreateWithFlags(&g_own_stream, hipStreamDefault));
   g_stream = g_own_stream;
   g_num_cus = prop.multiProcessorCount;
-  DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_chain_mem), kChainWords * sizeof(unsigned)));
-  DH_CHECK_HIP("dh_init", hipMemset(g_chain_mem, 0, kChainWords * sizeof(unsigned)));
-  g_chain_value = 0;
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_splitk_ws), kSplitKWsBytes));
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_row_scale), (size_t)kRowScaleRows * 2 * sizeof(float)));
   DH_CHECK_HIP("dh_init", hipMalloc(&g_packed_a, kPackedABytes));
@@ -345,17 +329,6 @@ int dh_sync(void) {
   DH_REQUIRE_INIT("dh_sync");
   if (g_capturing) return dh::fail(1, "[dh_sync] not possible while a graph is being captured (it waits for the stream)");
   DH_CHECK_HIP("dh_sync", hipStreamSynchronize(g_stream));
-  if (g_chain_mem) {
-    // a chained GEMV that could not cross its grid barrier left its outputs incomplete
-    unsigned flag = 0;
-    DH_CHECK_HIP("dh_sync", hipMemcpy(&flag, g_chain_mem + 8 * 64, sizeof(flag), hipMemcpyDeviceToHost));
-    if (flag) {
-      DH_CHECK_HIP("dh_sync", hipMemset(g_chain_mem, 0, kChainWords * sizeof(unsigned)));
-      g_chain_value = 0;
-      return dh::fail(3, "[dh_sync] a chained GEMV launch timed out at its grid barrier (workgroups not all "
-                      "resident); its outputs are invalid");
-    }
-  }
   return 0;
 }
 

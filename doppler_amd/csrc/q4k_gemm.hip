@@ -258,13 +258,6 @@ __device__ __forceinline__ float gelu_tanh_fast(float x) {
   return 0.5f * x * (2.0f - 2.0f / (1.0f + __expf(2.0f * t)));
 }
 
-#ifdef DH_GEMM_TRACE
-__device__ unsigned long long dh_gemm_trace_buf[12 * 128];
-#define DH_GTS() do { if (lane == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 0 && tsn < 124) \
-                        dh_gemm_trace_buf[wave * 128 + tsn++] = wall_clock64(); } while (0)
-#else
-#define DH_GTS() do {} while (0)
-#endif
 
 // T = MFMA tiles per wave along each of M and N (T = 2: a 64 x 64 quadrant per wave, T = 1:
 // 32 x 32 when larger tiles would leave most compute units idle).  Four waves cover a
@@ -283,9 +276,6 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   constexpr int PT = 256 * MG;                               // threads of the workgroup
   const int tid = threadIdx.x;
-#ifdef DH_GEMM_TRACE
-  int tsn = 0;
-#endif
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   const int wm = (wave >> 2) * SUBM + ((wave >> 1) & 1) * 32 * T, wn = (wave & 1) * 32 * T;
   const int fr = lane & 31, fg = lane >> 5;                  // fragment row / k half
@@ -479,13 +469,9 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
   __syncthreads();
   int kt = kt0;
   for (; kt + 2 < nkt; kt += 2) {        // st0 holds the tiles at odd distance from kt0, st1 the even ones
-    DH_GTS();
     fused_step(kt, st0);
-    DH_GTS();
     __syncthreads();
-    DH_GTS();
     fused_step(kt + 1, st1);
-    DH_GTS();
     __syncthreads();
   }
   if (kt + 1 < nkt) {
@@ -495,10 +481,6 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
   }
   multiply_step(kt, no_hook);
 
-  DH_GTS();
-#ifdef DH_GEMM_TRACE
-  if (lane == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 0) dh_gemm_trace_buf[wave * 128 + 127] = tsn;
-#endif
   // the matrix-core instructions above are inline asm, invisible to the compiler's hazard
   // checks: give the last one time to retire before its accumulators are read
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
@@ -656,11 +638,6 @@ int launch_gemm(GemmArgs a, const char* op) {
 
 }  // namespace
 
-#ifdef DH_GEMM_TRACE
-extern "C" int dh_debug_gemm_trace(void* host_dst) {
-  return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(dh_gemm_trace_buf), sizeof(dh_gemm_trace_buf));
-}
-#endif
 
 namespace dh {
 

@@ -313,12 +313,6 @@ template <int MT> struct RingShape {
   static constexpr int LW = MT > 2 ? 64 : 32;
 };
 
-#ifdef DH_GEMV_TRACE
-__device__ unsigned long long dh_trace_buf[256 * 64];
-__device__ unsigned long long dh_trace_span[64][256][16][2];     // per launch (mod 64), workgroup, wave: in, out
-unsigned dh_trace_launches = 0;
-#endif
-
 struct RingArgs {
   const float* A;        // [M][K]
   const uint8_t* W;      // Q4_K rows
@@ -335,9 +329,6 @@ struct RingArgs {
   const float* norm_weight;   // [K]
   float norm_eps;
   int norm_weight_offset;     // 1: scale by (1 + w)
-#ifdef DH_GEMV_TRACE
-  unsigned trace_seq;
-#endif
 };
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
@@ -491,15 +482,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // provably wave-uniform
-#ifdef DH_GEMV_TRACE
-  unsigned long long* tsbuf = reinterpret_cast<unsigned long long*>(dh_trace_buf) + blockIdx.x * 64;
-  int tsn = 0;
-#define DH_TS() do { if (tid == DH_GEMV_TRACE && tsn < 63) tsbuf[tsn++] = wall_clock64(); } while (0)
-  if (lane == 0) dh_trace_span[a.trace_seq & 63][blockIdx.x & 255][wave & 15][0] = wall_clock64();
-#else
-#define DH_TS() do {} while (0)
-#endif
-  DH_TS();
   const int g2 = lane >> 5, xcol = lane & 31;
   const int R = a.rows_per_tile, D = a.depth;
   const int nsub = a.nb * 8;
@@ -594,9 +576,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     // 17.2 vs 17.7 us for gate/up and 13.8 vs 13.0 us for the down projection, no change per step.
     // Nor letting the staging waves only stage and the other half own the whole weight stream:
     // 8.4 vs 7.5 us on the 6144 x 4096 product.)
-    DH_TS();
     DH_WAIT_VM(0);
-    DH_TS();
     if (norm && tid < total) {
 #pragma unroll
       for (int j = 0; j < 8; j++) ss = fmaf(v0[j], v0[j], ss);
@@ -621,7 +601,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     for (int phase = 0; phase < 2; phase++) {
     const int nstart = early_ring == (phase == 0) ? D : 0;
     for (int d = 0; d < nstart; d++) DH_ISSUE_NEXT();
-    DH_TS();
     if (phase != 0) continue;
 #pragma unroll 1
     for (int idx = tid; idx < total; idx += NTHR) {
@@ -641,9 +620,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     }
     if (tid < 16) reinterpret_cast<uint32_t*>(xzero)[tid] = 0u;
     if (tid < RS) done[tid] = 0u;
-    DH_TS();
     DH_LDS_BARRIER();
-    DH_TS();
     }
   }
 
@@ -667,8 +644,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
       for (int i = 0; i < bpw; i++) {
         // units issued after this one: each put nlw load instructions behind ours
         wait_vm_at_most((issued - consumed - 1) * nlw);
-        DH_TS();
-        const uint32_t hp = lane_lds + cstage * stage_bytes, qp = hp + 16 + 16 * g2;
+            const uint32_t hp = lane_lds + cstage * stage_bytes, qp = hp + 16 + 16 * g2;
         u32x4 h, q0, q1, q2, q3;
         asm volatile(
             "ds_read_b128 %0, %5\n\t"
@@ -682,21 +658,15 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
             : "memory");
         consumed++;
         cstage = cstage + 1 == D ? 0 : cstage + 1;
-        DH_TS();
-        DH_ISSUE_NEXT();            // the stage just read is free again
-        DH_TS();
-        WBlock w;
+            DH_ISSUE_NEXT();            // the stage just read is free again
+            WBlock w;
         w.hdr = make_uint4(h.x, h.y, h.z, h.w);
         w.q[0] = make_uint4(q0.x, q0.y, q0.z, q0.w);
         w.q[1] = make_uint4(q1.x, q1.y, q1.z, q1.w);
         w.q[2] = make_uint4(q2.x, q2.y, q2.z, q2.w);
         w.q[3] = make_uint4(q3.x, q3.y, q3.z, q3.w);
         mfma_block<MT>(w, xfl, xf_stride, sxi, (wave + WAVES * i) * 8, g2, acc);
-#ifdef DH_GEMV_TRACE
-        asm volatile("" :: "v"(acc[0]));
-#endif
-        DH_TS();
-      }
+          }
       if (lane < LW) {
 #pragma unroll
         for (int k = 0; k < NO; k++) red[slot][wave][mat][k][lane] = acc[k];
@@ -756,333 +726,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES / 4) void q4k_gemv_ring_kernel(co
     }
     // more tiles than slots: keep the waves within one tile of each other instead
     if (ntl > RS) DH_LDS_BARRIER();
-    DH_TS();
   }
-#ifdef DH_GEMV_TRACE
-  if (tid == DH_GEMV_TRACE) tsbuf[63] = tsn;
-  if (lane == 0) dh_trace_span[a.trace_seq & 63][blockIdx.x & 255][wave & 15][1] = wall_clock64();
-#endif
-#undef DH_TS
 #undef DH_ISSUE_NEXT
-}
-
-// ---------------------------------------------------------------------------------------
-// Chained GEMVs: up to four dependent M = 1 products (e.g. o_proj -> RMSNorm + gate/up ->
-// down -> RMSNorm + next layer's qkv) in ONE persistent launch of one workgroup per compute
-// unit.  Between two products the workgroups meet at a grid-wide barrier; what the chain buys
-// is that the weight stream never stops: a wave's ring cursor runs across the boundary, so the
-// first stages of the next product are already in flight (they do not depend on the
-// activations) while the barrier is crossed and the new activations are staged.
-//
-// Values handed from one product to the next go through memory with agent-scope stores and
-// loads (they bypass the per-XCD caches, which are not coherent with each other inside a
-// kernel); no cache-wide fences are used: those cost ~6 us each on this part, the barrier ~1.6.
-// The barrier is a set of 8 monotonic counters (workgroup b bumps counter b & 7, lanes 0..7 of
-// every workgroup poll one each); polling is bounded, a time-out raises *err and ends the
-// kernel, so a launch that is not fully resident cannot hang.
-// ---------------------------------------------------------------------------------------
-constexpr int kChainMaxPhases = 4;
-constexpr int kChainWaves = 16;
-constexpr int kChainXBytes = 56 * 1024;      // fragments of the longest activation row (K <= 12288)
-constexpr int kChainRows = 16;               // rows per tile (ring stage = 16 x 144 bytes)
-constexpr int kChainDepth = 2;
-constexpr unsigned kChainSpinLimit = 400000u;
-
-struct ChainPhase {
-  const float* A;             // [K] input (an earlier phase's C, or a buffer written before the launch)
-  const float* norm_weight;   // [K] RMSNorm prologue weights or null
-  const uint8_t* W;           // Q4_K [N][K]
-  const uint8_t* W2;          // second matrix: C = act(W x) * (W2 x); null: C = alpha W x + residual
-  float* C;                   // [N]
-  const float* residual;      // [N] or null
-  int N, K, nb, rows;         // rows per tile (<= kChainRows)
-  int activation, norm_offset;
-  float alpha, eps, clamp_max;
-};
-
-struct ChainArgs {
-  ChainPhase ph[kChainMaxPhases];
-  int nph;
-  unsigned* counters;         // 8 counters, 64 uint apart
-  unsigned base;              // value of every counter when the launch starts
-  unsigned* err;
-};
-
-__device__ __forceinline__ float ld_agent(const float* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Geometry of one phase as one wave sees it.
-struct ChainGeo {
-  const uint8_t* W;
-  const uint8_t* W2;
-  int R, nb, N, ntl, bpw, nmat, nlw;
-  int64_t row_bytes;
-};
-
-__device__ __forceinline__ ChainGeo chain_geo(const ChainArgs& a, int p, int wave) {
-  ChainGeo g;
-  g.W = a.ph[p].W; g.W2 = a.ph[p].W2;
-  g.R = a.ph[p].rows; g.nb = a.ph[p].nb; g.N = a.ph[p].N;
-  g.row_bytes = (int64_t)g.nb * kBlockBytes;
-  const int ntiles = (g.N + g.R - 1) / g.R;
-  g.ntl = (ntiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-  g.bpw = (g.nb - wave + kChainWaves - 1) / kChainWaves;
-  g.nmat = g.W2 ? 2 : 1;
-  g.nlw = (9 * g.R + 63) >> 6;
-  return g;
-}
-
-__global__ __launch_bounds__(64 * kChainWaves, kChainWaves / 4) void q4k_chain_kernel(const ChainArgs a) {
-  constexpr int WAVES = kChainWaves, NTHR = 64 * WAVES, D = kChainDepth;
-  constexpr int STAGE = kChainRows * kBlockBytes;
-  __shared__ __align__(16) unsigned char xs[kChainXBytes];
-  __shared__ float red[kRedSlots][WAVES][2][32];
-  __shared__ unsigned done[kRedSlots];
-  __shared__ float norm_ss[WAVES];
-  __shared__ int bar_ok;
-  extern __shared__ __align__(16) unsigned char ring[];     // [WAVES][D][STAGE]
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int g2 = lane >> 5, xcol = lane & 31;
-  unsigned char* my_ring = ring + (size_t)wave * D * STAGE;
-#ifdef DH_GEMV_TRACE
-  unsigned long long* tsbuf = reinterpret_cast<unsigned long long*>(dh_trace_buf) + blockIdx.x * 64;
-  int tsn = 0;
-#define DH_CTS() do { if (tid == DH_GEMV_TRACE && tsn < 63) tsbuf[tsn++] = wall_clock64(); } while (0)
-#else
-#define DH_CTS() do {} while (0)
-#endif
-  DH_CTS();
-
-  // ---- issue side: a cursor over (phase, tile, matrix, block) that runs ahead of the consumer
-  int ip = 0;
-  ChainGeo ig = chain_geo(a, 0, wave);
-  UnitCursor ic = {0, 0, 0};
-  uint32_t goff[3];
-#define DH_CHAIN_GOFF()                                                                      \
-  _Pragma("unroll") for (int t = 0; t < 3; t++) {                                            \
-    const int q = t * 64 + lane, r = q / 9;                                                  \
-    goff[t] = q < 9 * ig.R ? (uint32_t)(r * ig.row_bytes + (q - r * 9) * 16) : 0xFFFFFFFFu;  \
-  }
-  DH_CHAIN_GOFF();
-  int issue_stage = 0, loads_issued = 0;
-  int loads_at[D];                     // loads_issued right after each stage's unit went out
-#pragma unroll
-  for (int d = 0; d < D; d++) loads_at[d] = 0;
-#define DH_CHAIN_ISSUE()                                                                          \
-  do {                                                                                            \
-    while (ip < a.nph && (ic.tl >= ig.ntl || ig.bpw == 0)) {                                      \
-      if (++ip < a.nph) { ig = chain_geo(a, ip, wave); ic = {0, 0, 0}; DH_CHAIN_GOFF(); }         \
-    }                                                                                             \
-    if (ip < a.nph) {                                                                             \
-      const int tile_ = blockIdx.x + ic.tl * gridDim.x;                                           \
-      const uint8_t* base_ = (ic.mat ? ig.W2 : ig.W) + (int64_t)tile_ * ig.R * ig.row_bytes +     \
-                             (int64_t)(wave + WAVES * ic.i) * kBlockBytes;                        \
-      unsigned char* st_ = my_ring + issue_stage * STAGE;                                         \
-      const int rows_left_ = ig.N - tile_ * ig.R;                                                 \
-      _Pragma("unroll") for (int t = 0; t < 3; t++) {                                             \
-        const int q_ = t * 64 + lane, r_ = q_ / 9;                                                \
-        const int64_t o_ = rows_left_ >= ig.R ? (int64_t)goff[t]                                  \
-                                              : (int64_t)min(r_, rows_left_ - 1) * ig.row_bytes + (q_ - r_ * 9) * 16; \
-        if (goff[t] != 0xFFFFFFFFu)                                                               \
-          __builtin_amdgcn_global_load_lds(base_ + o_, DH_LDS_PTR(st_ + t * 1024), 16, 0, 0);     \
-      }                                                                                           \
-      loads_issued += ig.nlw;                                                                     \
-      _Pragma("unroll") for (int d = 0; d < D; d++) if (d == issue_stage) loads_at[d] = loads_issued; \
-      issue_stage = issue_stage + 1 == D ? 0 : issue_stage + 1;                                   \
-      if (++ic.i == ig.bpw) {                                                                     \
-        ic.i = 0;                                                                                 \
-        if (++ic.mat == ig.nmat) { ic.mat = 0; ic.tl++; }                                         \
-      }                                                                                           \
-    }                                                                                             \
-  } while (0)
-
-  for (int d = 0; d < D; d++) DH_CHAIN_ISSUE();
-  if (tid < kRedSlots) done[tid] = 0u;
-  DH_CTS();
-
-  int cstage = 0;
-  unsigned bar_target = a.base;
-#pragma unroll 1
-  for (int p = 0; p < a.nph; p++) {
-    const ChainGeo cg = chain_geo(a, p, wave);
-    const int nsub = cg.nb * 8, K = a.ph[p].K;
-    _Float16* xf = reinterpret_cast<_Float16*>(xs);                       // [nsub][2][32]
-    _Float16* xzero = xf + (size_t)nsub * 2 * 32;
-    float2* sxi = reinterpret_cast<float2*>(xzero + 32);                  // [nsub]
-
-    // ---- grid barrier: every workgroup has written the previous product's outputs
-    DH_CTS();
-    if (p > 0) {
-      DH_LDS_BARRIER();                                   // this workgroup's waves are done with p - 1
-      DH_CTS();
-      bar_target += gridDim.x / 8;
-      if (tid < 64) {
-        if (tid == 0) atomicAdd(a.counters + 64 * (blockIdx.x & 7), 1u);
-        bool ok = true;
-        if (tid < 8) {
-          unsigned spins = 0;
-          // counters only grow; the difference is taken modulo 2^32
-          while ((int)(__hip_atomic_load(a.counters + 64 * tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) -
-                       bar_target) < 0) {
-            if (++spins > kChainSpinLimit) { ok = false; break; }
-          }
-        }
-        const bool all_ok = __all(ok);
-        if (tid == 0) {
-          bar_ok = all_ok;
-          if (!all_ok) atomicExch(a.err, 1u);
-        }
-      }
-      DH_LDS_BARRIER();
-      if (!bar_ok) {                                      // not fully resident (or a peer failed): give up,
-        DH_WAIT_VM(0);                                    // but only once no load can still land in LDS
-        return;
-      }
-    }
-
-    DH_CTS();
-    // ---- stage this product's activations (quarter items, as in the stand-alone kernel)
-    {
-      const float* A = a.ph[p].A;
-      const float* nw = a.ph[p].norm_weight;
-      const int total = 4 * nsub;
-      float ss = 0.f;
-#pragma unroll 1
-      for (int pass = 0; pass < (nw ? 2 : 1); pass++) {    // with a norm: first pass sums squares
-        float inv = 1.f;
-        if (pass == 1 || !nw) {
-          if (nw) {
-            ss += quad_xor_f32(ss, 1);
-            ss += quad_xor_f32(ss, 2);
-            ss += __shfl_xor(ss, 4);
-            ss += __shfl_xor(ss, 8);
-            ss += __shfl_xor(ss, 16);
-            ss += __shfl_xor(ss, 32);
-            if (lane == 0) norm_ss[wave] = ss;
-            DH_LDS_BARRIER();
-            float tot = 0.f;
-#pragma unroll
-            for (int w = 0; w < WAVES; w++) tot += norm_ss[w];
-            inv = 1.0f / sqrtf(tot / (float)K + a.ph[p].eps);
-          }
-        }
-#pragma unroll 1
-        for (int idx = tid; idx < total; idx += NTHR) {
-          const int item = idx >> 2, grp = idx & 3;
-          const int k0 = item * 32 + grp * 8, left = K - k0;
-          float v[8];
-#pragma unroll
-          for (int j = 0; j < 8; j++) v[j] = j < left ? ld_agent(A + k0 + j) : 0.f;
-          if (nw && pass == 0) {
-#pragma unroll
-            for (int j = 0; j < 8; j++) ss = fmaf(v[j], v[j], ss);
-            continue;
-          }
-          if (nw) {
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-              const float wj = j < left ? nw[k0 + j] : 0.f;
-              v[j] = v[j] * inv * (a.ph[p].norm_offset ? 1.0f + wj : wj);
-            }
-          }
-          stage_x_store<1>(idx, v, xf, sxi);
-        }
-      }
-      if (tid < 16) reinterpret_cast<uint32_t*>(xzero)[tid] = 0u;
-      DH_LDS_BARRIER();
-    }
-    const _Float16* xfl = xcol < 2 ? xf + xcol * 32 + g2 * 16 : xzero;
-    const int xf_stride = xcol < 2 ? 2 * 32 : 0;
-    const uint32_t lane_lds =
-        (uint32_t)(uintptr_t)DH_LDS_PTR(my_ring) + (uint32_t)min(lane & 31, cg.R - 1) * kBlockBytes;
-
-    DH_CTS();
-    // ---- consume this product's units
-#pragma unroll 1
-    for (int tl = 0; tl < cg.ntl; tl++) {
-      const int tile = blockIdx.x + tl * gridDim.x;
-      const int slot = tl % kRedSlots;
-#pragma unroll 1
-      for (int mat = 0; mat < cg.nmat; mat++) {
-        float acc[1] = {0.f};
-#pragma unroll 1
-        for (int i = 0; i < cg.bpw; i++) {
-          int at = loads_at[0];
-#pragma unroll
-          for (int d = 1; d < D; d++) at = d == cstage ? loads_at[d] : at;
-          wait_vm_at_most(loads_issued - at);
-          const uint32_t hp = lane_lds + cstage * STAGE, qp = hp + 16 + 16 * g2;
-          u32x4 h, q0, q1, q2, q3;
-          asm volatile(
-              "ds_read_b128 %0, %5\n\t"
-              "ds_read_b128 %1, %6\n\t"
-              "ds_read_b128 %2, %6 offset:32\n\t"
-              "ds_read_b128 %3, %6 offset:64\n\t"
-              "ds_read_b128 %4, %6 offset:96\n\t"
-              "s_waitcnt lgkmcnt(0)"
-              : "=&v"(h), "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3)
-              : "v"(hp), "v"(qp)
-              : "memory");
-          cstage = cstage + 1 == D ? 0 : cstage + 1;
-          DH_CHAIN_ISSUE();           // the stage just read is free again (may belong to the next product)
-          WBlock w;
-          w.hdr = make_uint4(h.x, h.y, h.z, h.w);
-          w.q[0] = make_uint4(q0.x, q0.y, q0.z, q0.w);
-          w.q[1] = make_uint4(q1.x, q1.y, q1.z, q1.w);
-          w.q[2] = make_uint4(q2.x, q2.y, q2.z, q2.w);
-          w.q[3] = make_uint4(q3.x, q3.y, q3.z, q3.w);
-          mfma_block<1>(w, xfl, xf_stride, sxi, (wave + WAVES * i) * 8, g2, acc);
-        }
-        if (lane < 32) red[slot][wave][mat][lane] = acc[0];
-      }
-      // ---- tile end: the last wave to arrive adds the K slices and writes the outputs
-      unsigned arrived = 0;
-      if (lane == 0) {
-        const uint32_t cnt_addr = (uint32_t)(uintptr_t)DH_LDS_PTR(&done[slot]);
-        asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
-                     : "=&v"(arrived) : "v"(cnt_addr), "v"(1u) : "memory");
-      }
-      arrived = __builtin_amdgcn_readfirstlane(arrived);
-      asm volatile("" ::: "memory");
-      if (arrived == WAVES - 1) {
-        const int r = lane;
-        const int64_t row = (int64_t)tile * cg.R + r;
-        if (r < cg.R && row < cg.N) {
-          float sg = 0.f, su = 0.f;
-#pragma unroll
-          for (int w = 0; w < WAVES; w++) {
-            sg += red[slot][w][0][r];
-            su += red[slot][w][1][r];
-          }
-          float v;
-          if (cg.nmat == 2) {
-            const float act = a.ph[p].activation == DH_ACT_SILU ? act_silu(sg) : act_gelu(sg);
-            v = act * su * a.ph[p].alpha;
-            if (a.ph[p].activation == DH_ACT_SILU && a.ph[p].clamp_max > 0.f)
-              v = fminf(fmaxf(v, -a.ph[p].clamp_max), a.ph[p].clamp_max);
-          } else {
-            v = sg * a.ph[p].alpha;
-            if (a.ph[p].residual) v += ld_agent(a.ph[p].residual + row);
-          }
-          __hip_atomic_store(a.ph[p].C + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        if (lane == 0) done[slot] = 0u;
-        // the outputs must have left this wave before the workgroup reports at the barrier
-        DH_WAIT_VM(0);
-      }
-      if (cg.ntl > kRedSlots) DH_LDS_BARRIER();
-    }
-    DH_CTS();
-  }
-#ifdef DH_GEMV_TRACE
-  if (tid == DH_GEMV_TRACE) tsbuf[63] = tsn;
-#endif
-#undef DH_CTS
-#undef DH_CHAIN_ISSUE
-#undef DH_CHAIN_GOFF
 }
 
 constexpr size_t kRingMaxLds = 160 * 1024;
@@ -1118,9 +763,6 @@ int launch_ring_cfg(RingArgs a, const char* op, bool may_shorten_tiles) {
   if (fixed + dyn > kRingMaxLds) return -1;
   a.rows_per_tile = rows;
   a.depth = depth;
-#ifdef DH_GEMV_TRACE
-  a.trace_seq = dh_trace_launches++;
-#endif
   const int64_t ntiles = dh::ceil_div(a.N, rows);
   const int grid = (int)std::min<int64_t>(ntiles, ncu);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), dyn, dh::stream(), a);
@@ -1264,26 +906,7 @@ int gemv_path() {
   return path;
 }
 
-// Rows per tile for a chained product: whole tiles per compute unit, at most kChainRows rows.
-int chain_rows(int N, int ncu) {
-  const int per_cu = (int)dh::ceil_div(N, (int64_t)ncu * kChainRows);
-  return std::max(1, std::min(kChainRows, (int)dh::ceil_div(N, (int64_t)ncu * per_cu)));
-}
-
 }  // namespace
-
-#ifdef DH_GEMV_TRACE
-extern "C" int dh_debug_span(void* host_io, int reset) {
-  if (reset) {
-    dh_trace_launches = 0;
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(dh_trace_span), host_io, sizeof(dh_trace_span));
-  }
-  return (int)hipMemcpyFromSymbol(host_io, HIP_SYMBOL(dh_trace_span), sizeof(dh_trace_span));
-}
-extern "C" int dh_debug_trace(void* host_dst) {
-  return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(dh_trace_buf), sizeof(dh_trace_buf));
-}
-#endif
 
 extern "C" {
 
@@ -1442,51 +1065,6 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
     const int rc = dispatch_lds<true>(b, op);
     if (rc) return rc;
   }
-  return 0;
-}
-
-int dh_q4k_gemv_chain(const dh_gemv_phase* phases, int count) {
-  const char* op = "dh_q4k_gemv_chain";
-  DH_REQUIRE_INIT(op);
-  if (!phases || count < 1 || count > kChainMaxPhases)
-    return dh::fail(1, "[%s] between 1 and %d phases are supported, got %d", op, kChainMaxPhases, count);
-  const int ncu = dh::num_cus() & ~7;
-  if (ncu < 8 || !dh::chain_counters()) return dh::fail(1, "[%s] not available on this device", op);
-  ChainArgs a{};
-  a.nph = count;
-  for (int p = 0; p < count; p++) {
-    const dh_gemv_phase& h = phases[p];
-    if (h.N <= 0 || h.K <= 0) return dh::fail(1, "[%s] phase %d: Dimensions must be positive: N=%d, K=%d", op, p, h.N, h.K);
-    if (!h.d_A || !h.d_W || !h.d_C) return dh::fail(1, "[%s] phase %d: null pointer", op, p);
-    if ((reinterpret_cast<uintptr_t>(h.d_W) | reinterpret_cast<uintptr_t>(h.d_W2)) & 15)
-      return dh::fail(1, "[%s] phase %d: weight pointers must be 16-byte aligned", op, p);
-    const int nb = (h.K + kQK - 1) / kQK;
-    if (ring_x_bytes(1, nb) > (size_t)kChainXBytes)
-      return dh::fail(1, "[%s] phase %d: K=%d exceeds the chained kernel's limit of %d", op, p, h.K,
-                      (kChainXBytes - 64) / 136 * 32);
-    if (h.d_W2 && h.activation != DH_ACT_SILU && h.activation != DH_ACT_GELU)
-      return dh::fail(1, "[%s] phase %d: unknown activation %d", op, p, h.activation);
-    if (h.d_W2 && h.d_residual) return dh::fail(1, "[%s] phase %d: a gated product takes no residual", op, p);
-    ChainPhase& q = a.ph[p];
-    q.A = h.d_A; q.norm_weight = h.d_norm_weight; q.W = static_cast<const uint8_t*>(h.d_W);
-    q.W2 = static_cast<const uint8_t*>(h.d_W2); q.C = h.d_C; q.residual = h.d_residual;
-    q.N = h.N; q.K = h.K; q.nb = nb; q.rows = chain_rows(h.N, ncu);
-    q.activation = h.activation; q.norm_offset = h.weight_offset;
-    q.alpha = h.alpha; q.eps = h.eps; q.clamp_max = h.swiglu_limit;
-  }
-  a.counters = dh::chain_counters();
-  a.err = dh::chain_error_flag();
-  a.base = dh::chain_advance((unsigned)(count - 1) * (unsigned)(ncu / 8));
-  static bool attr_set = false;
-  const size_t dyn = (size_t)kChainWaves * kChainDepth * kChainRows * kBlockBytes;
-  if (!attr_set) {
-    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(q4k_chain_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn));
-    attr_set = true;
-  }
-  // one workgroup per compute unit, all resident at once (the kernel's barrier relies on it)
-  hipLaunchKernelGGL(q4k_chain_kernel, dim3(ncu), dim3(64 * kChainWaves), dyn, dh::stream(), a);
-  DH_CHECK_LAUNCH(op);
   return 0;
 }
 

@@ -232,7 +232,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
   // compute unit's memory queue.  (Fast path, K a multiple of 4 and 16-byte aligned rows: the loads
   // are hand-issued so that the first weight unit can follow them and only THEY are waited for.)
   const int kg = lane >> 4;
-  constexpr int SC = MT == 1 ? 3 : 2;                    // columns per pass (all loads of a pass in flight at once)
+  constexpr int SC = MT == 1 ? 3 : (MT == 2 ? 2 : 1);    // columns per pass (all loads of a pass in flight at once)
   const int my_cols = wave < nb ? (nb - wave + kWaves - 1) >> 4 : 0;
   v4f xr[SC][MT], wr[SC];
 #define DH_LOAD_X(c0_)                                                                            \
@@ -428,10 +428,13 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     const uint32_t rec = xq_abs + (uint32_t)(col * MT) * kRec;
     const uint32_t gen_addr = ctr_abs + 4 * (1 + nslots + slot);
     const uint32_t flag_addr = ctr_abs + 4 * (1 + 2 * nslots + col);
+    // activation rows are handled MP at a time (their operands share the registers); the first
+    // batch is read together with the weights
+    constexpr int MP = MT < 2 ? MT : 2;
     v4u h, q0, q1;
-    v4i ax[MT][2][2];
-    v2f sx[MT];
-    float xinv[MT];
+    v4i ax[MP][2][2];
+    v2f sx[MP];
+    float xinv[MP];
     uint32_t gen, flag;
     asm volatile(
         "ds_read_b32 %4, %8\n\t"
@@ -444,9 +447,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
         : "memory");
     // the column's operands, read at once on the expectation that its flag is up (it is, except
     // in the first microseconds of a launch); re-read below if it was not
-#define DH_READ_OPERANDS()                                                                        \
-    _Pragma("unroll") for (int m = 0; m < MT; m++) {                                              \
-      const uint32_t rm = rec + m * kRec;                                                         \
+#define DH_READ_OPERANDS(m0_)                                                                     \
+    _Pragma("unroll") for (int m = 0; m < MP; m++) {                                              \
+      const uint32_t rm = rec + ((m0_) + m) * kRec;                                               \
       const uint32_t pa = rm * a_mul[0] + a_off[0], pb = rm * a_mul[1] + a_off[1], ps = rm + 768 + 4 * kg; \
       asm volatile(                                                                               \
           "ds_read_b128 %0, %6\n\t"                                                               \
@@ -460,9 +463,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
           : "memory");                                                                            \
     }
 #define DH_TIE_OPERANDS()                                                                         \
-    _Pragma("unroll") for (int m = 0; m < MT; m++)                                                \
+    _Pragma("unroll") for (int m = 0; m < MP; m++)                                                \
       asm volatile("" : "+v"(ax[m][0][0]), "+v"(ax[m][0][1]), "+v"(ax[m][1][0]), "+v"(ax[m][1][1]), "+v"(sx[m]), "+v"(xinv[m]))
-    DH_READ_OPERANDS()
+    DH_READ_OPERANDS(0)
     // everything above has landed (one wait for all of it; the registers are tied to it)
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(h), "+v"(q0), "+v"(q1), "+v"(gen), "+v"(flag), "+v"(nxt) :: "memory");
     DH_TIE_OPERANDS();
@@ -471,12 +474,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
         __builtin_amdgcn_s_sleep(2);
         flag = lds_read_u32(flag_addr);
       } while (__builtin_amdgcn_readfirstlane(flag) == 0u);
-      DH_READ_OPERANDS()
+      DH_READ_OPERANDS(0)
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       DH_TIE_OPERANDS();
     }
-#undef DH_READ_OPERANDS
-#undef DH_TIE_OPERANDS
     // the stage is free again: put the loads of the unit drawn above in flight
     inflight--;
     {
@@ -493,19 +494,14 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     const float mn_a = (float)((h.z >> sh_lo) & 63u);
     const float mn_b = (float)(((h.w >> (sh_lo + 4)) & 15u) | (((h.z >> (sh_lo + 6)) & 3u) << 4));
     const float d = f16lo(h.x), dmin = f16hi(h.x);
-    v4i dd[2][MT];
+    v4i blo[2], bhi[2];
 #pragma unroll
     for (int cc = 0; cc < 2; cc++) {
       const v4u q = cc ? q1 : q0;
-      const v4i blo = {(int)(q.x & 0x0F0F0F0Fu), (int)(q.y & 0x0F0F0F0Fu), (int)(q.z & 0x0F0F0F0Fu),
-                       (int)(q.w & 0x0F0F0F0Fu)};
-      const v4i bhi = {(int)((q.x >> 4) & 0x0F0F0F0Fu), (int)((q.y >> 4) & 0x0F0F0F0Fu),
-                       (int)((q.z >> 4) & 0x0F0F0F0Fu), (int)((q.w >> 4) & 0x0F0F0F0Fu)};
-#pragma unroll
-      for (int m = 0; m < MT; m++) {
-        v4i t = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[m][cc][0], blo, v4i{0, 0, 0, 0}, 0, 0, 0);
-        dd[cc][m] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[m][cc][1], bhi, t, 0, 0, 0);
-      }
+      blo[cc] = v4i{(int)(q.x & 0x0F0F0F0Fu), (int)(q.y & 0x0F0F0F0Fu), (int)(q.z & 0x0F0F0F0Fu),
+                    (int)(q.w & 0x0F0F0F0Fu)};
+      bhi[cc] = v4i{(int)((q.x >> 4) & 0x0F0F0F0Fu), (int)((q.y >> 4) & 0x0F0F0F0Fu),
+                    (int)((q.z >> 4) & 0x0F0F0F0Fu), (int)((q.w >> 4) & 0x0F0F0F0Fu)};
     }
     // wait (never, in practice) until the tile that used this slot nslots tiles ago is written out
     {
@@ -516,17 +512,33 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
       }
     }
 #pragma unroll
-    for (int m = 0; m < MT; m++) {
-      // |digit sum| <= 32*15*64 and the scale is 6 bits: 24-bit multiplies are exact
-      const int p0 = __mul24(sc_a, dd[0][m][0]) + __mul24(sc_b, dd[1][m][0]);
-      const int p1 = __mul24(sc_a, dd[0][m][1]) + __mul24(sc_b, dd[1][m][1]);
-      const int p2 = __mul24(sc_a, dd[0][m][2]) + __mul24(sc_b, dd[1][m][2]);
-      const float t = fmaf((float)p0, 16384.f, fmaf((float)p1, 128.f, (float)p2));
-      const float mins = fmaf(mn_a, sx[m][0], mn_b * sx[m][1]);
-      // the four lane groups hold different sub-blocks of the same 16 rows
-      const float s = sum_lane_groups(fmaf(d * xinv[m], t, -dmin * mins));
-      if (lane < 16) red[(((size_t)slot * upt + (mat * nb + col)) * MT + m) * 16 + lane] = s;
+    for (int m0 = 0; m0 < MT; m0 += MP) {
+      if (m0 > 0) {
+        DH_READ_OPERANDS(m0)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        DH_TIE_OPERANDS();
+      }
+#pragma unroll
+      for (int m = 0; m < MP; m++) {
+        v4i dd[2];
+#pragma unroll
+        for (int cc = 0; cc < 2; cc++) {
+          v4i t = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[m][cc][0], blo[cc], v4i{0, 0, 0, 0}, 0, 0, 0);
+          dd[cc] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[m][cc][1], bhi[cc], t, 0, 0, 0);
+        }
+        // |digit sum| <= 32*15*64 and the scale is 6 bits: 24-bit multiplies are exact
+        const int p0 = __mul24(sc_a, dd[0][0]) + __mul24(sc_b, dd[1][0]);
+        const int p1 = __mul24(sc_a, dd[0][1]) + __mul24(sc_b, dd[1][1]);
+        const int p2 = __mul24(sc_a, dd[0][2]) + __mul24(sc_b, dd[1][2]);
+        const float t = fmaf((float)p0, 16384.f, fmaf((float)p1, 128.f, (float)p2));
+        const float mins = fmaf(mn_a, sx[m][0], mn_b * sx[m][1]);
+        // the four lane groups hold different sub-blocks of the same 16 rows
+        const float sres = sum_lane_groups(fmaf(d * xinv[m], t, -dmin * mins));
+        if (lane < 16) red[(((size_t)slot * upt + (mat * nb + col)) * MT + m0 + m) * 16 + lane] = sres;
+      }
     }
+#undef DH_READ_OPERANDS
+#undef DH_TIE_OPERANDS
     // ---- deliver.  LDS executes a wave's operations in order, so the partial sums above are in
     // place before the count below is; the wave that delivers a tile's last unit finishes it.
     unsigned arrived = 0;
@@ -677,11 +689,41 @@ int launch_i8(const I8Args& a, const char* op) {
   return vec ? launch_i8_vec<MT, DUAL, true>(a, op) : launch_i8_vec<MT, DUAL, false>(a, op);
 }
 
+// Bytes of LDS a launch with MT activation rows needs at ring depth 1 (what launch_i8_vec computes).
+size_t i8_lds_bytes(int mt, int nb, int nmat) {
+  const int upt = nb * nmat;
+  const int need = (kWaves * (kMaxDepth + 1) + upt - 1) / upt + 2;
+  int nslots = 2;
+  while (nslots < need) nslots *= 2;
+  return (size_t)kWaves * kStage + (size_t)nb * mt * kRec + kZeroBytes + sizeof(float) * nslots * upt * mt * 16 +
+         sizeof(unsigned) * (1 + 2 * nslots + nb);
+}
+
+template <bool DUAL>
+int launch_mt(int mt, const I8Args& a, const char* op) {
+  return mt == 2 ? launch_i8<2, DUAL>(a, op) : launch_i8<1, DUAL>(a, op);
+}
+
+// M activation rows in as few passes over the weights as the LDS allows: 2 or 1 rows per pass (the
+// rows' operands, 832 bytes per row and super-block column, must fit beside the ring).
 template <bool DUAL>
 int dispatch_i8(const I8Args& a, const char* op) {
-  if (a.M == 1) return launch_i8<1, DUAL>(a, op);
-  if (a.M == 2) return launch_i8<2, DUAL>(a, op);
-  return -1;
+  const size_t c_elem = a.c_f16 ? 2 : 4;
+  int mt = 1;
+  for (int cand : {2}) {
+    if (cand / 2 < a.M && i8_lds_bytes(cand, a.nb, DUAL ? 2 : 1) <= kMaxLds - 4096) mt = cand;
+  }
+  if (i8_lds_bytes(mt, a.nb, DUAL ? 2 : 1) > kMaxLds - 4096) return -1;
+  for (int m0 = 0; m0 < a.M; m0 += mt) {
+    I8Args b = a;
+    b.M = std::min(mt, a.M - m0);
+    b.A = a.A + (int64_t)m0 * a.K;
+    b.C = static_cast<char*>(a.C) + (int64_t)m0 * a.N * c_elem;
+    b.residual = a.residual ? a.residual + (int64_t)m0 * a.N : nullptr;
+    const int rc = launch_mt<DUAL>(mt, b, op);
+    if (rc != 0) return m0 == 0 ? rc : dh::fail(2, "[%s] internal: GEMV pass %d did not launch after pass 0 did", op, m0 / mt);
+  }
+  return 0;
 }
 
 }  // namespace
@@ -698,6 +740,9 @@ int q4k_gemv_i8(const char* op, const float* A, const uint8_t* W, const uint8_t*
                 const float* residual, int M, int N, int K, float alpha, int activation, float clamp_max,
                 const float* norm_weight, float norm_eps, int norm_weight_offset) {
   static const int off = env_int("DH_GEMV_I8_OFF", 0);
+  // three and more activation rows stay with the f16 matrix-core kernel of q4k_gemv.hip: their
+  // operands (832 bytes per row and column) crowd the LDS and the per-row epilogue outweighs the
+  // weight stream (measured: 24 against 21 us for the fused gate/up product at M = 4)
   if (off || M < 1 || M > 2) return -1;
   I8Args a{};
   a.A = A; a.W = W; a.W2 = W2; a.C = C; a.residual = residual;

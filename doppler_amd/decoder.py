@@ -34,15 +34,10 @@ def _dev_bytes(arr):
     return t
 
 
-def c_hidden_ok(cfg):
-    """The chained kernel holds one activation row in LDS: rows up to 12288 elements."""
-    return max(cfg["hidden"], cfg["inter"], cfg["heads"] * cfg["head_dim"]) <= 12288
-
-
 class HipDecoder:
     TOKEN_RING = 64      # tokens one decode_batch submit can produce
 
-    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True, chain=False,
+    def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True,
                  fuse_qkv_attention=True):
         """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
         layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
@@ -50,11 +45,6 @@ class HipDecoder:
         self.cfg = dict(cfg)
         # RMSNorm runs inside the q/k/v and gate/up GEMVs (their prologue) unless told otherwise
         self.fuse_norm = fuse_norm
-        # chain=True: the GEMVs between two attentions (o_proj, gate/up, down, next q/k/v) go out as
-        # one persistent launch.  Off by default: on MI355X the in-kernel barrier plus re-staging the
-        # activations under a saturated weight stream costs more than the three kernel boundaries.
-        self.chain = chain and fuse_norm and c_hidden_ok(cfg)
-        self._chains = None
         self.L = capi.init(torch.cuda.current_device())
         c = self.cfg
         # decode steps: q/k norm + RoPE + KV append run inside the attention kernel when the head
@@ -127,8 +117,6 @@ class HipDecoder:
                            in_index if from_device_token else 0))
         self._out_index = out_index
         x, x2 = self.x, self.x2
-        if self.chain:
-            return self._enqueue_chained(pos, want_logits)
         for d in self.layers:
             if self.fuse_norm:
                 ck(L.dh_q4k_matmul_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), c["eps"], 0,
@@ -179,51 +167,6 @@ class HipDecoder:
                             self.attn.data_ptr(), H, Hkv, D, pos + 1, self.scale, 1, pos, 0.0, 0, 0,
                             capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
 
-    def _build_chains(self):
-        """One dh_gemv_phase array per layer: o_proj (+residual) -> RMSNorm + gate/up + SiLU ->
-        down (+residual) -> RMSNorm + the NEXT layer's stacked q/k/v projection."""
-        c = self.cfg
-        Hd, I = c["hidden"], c["inter"]
-        chains = []
-        for li, d in enumerate(self.layers):
-            nxt = self.layers[li + 1] if li + 1 < len(self.layers) else None
-            arr = (capi.GemvPhase * (4 if nxt else 3))()
-
-            def fill(g, A, W, C, N, K, norm=None, W2=None, residual=None):
-                g.d_A, g.d_W, g.d_C, g.N, g.K = A.data_ptr(), W.data_ptr(), C.data_ptr(), N, K
-                g.d_norm_weight = norm.data_ptr() if norm is not None else None
-                g.eps, g.weight_offset = c["eps"], 0
-                g.d_W2 = W2.data_ptr() if W2 is not None else None
-                g.d_residual = residual.data_ptr() if residual is not None else None
-                g.activation, g.alpha, g.swiglu_limit = capi.ACT_SILU, 1.0, 0.0
-            fill(arr[0], self.attn, d["wo"], self.x2, Hd, self.qs, residual=self.x)
-            fill(arr[1], self.x2, d["wgate"], self.act, I, Hd, norm=d["post_attn_norm"], W2=d["wup"])
-            fill(arr[2], self.act, d["wdown"], self.x, Hd, I, residual=self.x2)
-            if nxt:
-                fill(arr[3], self.x, nxt["wqkv"], self.qkv, self.qs + 2 * self.ks, Hd, norm=nxt["input_norm"])
-            chains.append(arr)
-        return chains
-
-    def _enqueue_chained(self, pos, want_logits):
-        """The step with the four GEMVs between two attentions in one persistent launch."""
-        L, c = self.L, self.cfg
-        ck = capi.check
-        H, Hkv, D, Hd = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"]
-        if self._chains is None:
-            self._chains = self._build_chains()
-        first = self.layers[0]
-        ck(L.dh_q4k_matmul_rmsnorm(self.x.data_ptr(), first["input_norm"].data_ptr(), c["eps"], 0,
-                                   first["wqkv"].data_ptr(), self.qkv.data_ptr(), capi.F32, 1,
-                                   self.qs + 2 * self.ks, Hd, 1.0, None))
-        for d, chain in zip(self.layers, self._chains):
-            self._enqueue_attention(d, pos)
-            ck(L.dh_q4k_gemv_chain(chain, len(chain)))
-        ck(L.dh_rmsnorm(self.x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd,
-                        c["eps"], 0, None, None, None, 1.0))
-        ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
-                                  self.lm_ws.data_ptr(), self.token.data_ptr(), self._out_index,
-                                  self.logits.data_ptr() if want_logits else None))
-
     def set_token(self, token):
         self._host_token[0] = token
         capi.check(self.L.dh_upload(self.ids.data_ptr(), 0, self._host_token.ctypes.data, 4))
@@ -247,8 +190,8 @@ class HipDecoder:
         counterpart of the reference's one-submit-per-step recorder
         (src/inference/pipelines/text/generator-steps.js:605,814).  The step is run once
         normally first so that every kernel's one-time set-up is done outside the capture."""
-        if not self.fuse_qkv_attention or self.chain:
-            raise ValueError("capture_step serves the fused-attention, unchained step")
+        if not self.fuse_qkv_attention:
+            raise ValueError("capture_step serves the step with the fused attention kernel")
         self.enqueue_step(pos, want_logits)
         capi.check(self.L.dh_sync())
         capi.check(self.L.dh_graph_begin())

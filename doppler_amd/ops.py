@@ -222,29 +222,6 @@ def runFusedFFN(input, W_gate, W_up, hiddenSize, intermediateSize, batchSize=1, 
     return Tensor(out, "f32", (batchSize, intermediateSize), "fused_ffn_output")
 
 
-def runGemvChain(phases):
-    """Several dependent M = 1 Q4_K products in one persistent launch (dh_q4k_gemv_chain).
-    `phases`: list of dicts with keys input, weight, output (Tensors / WeightBuffer), N, K and
-    optionally normWeight, eps, rmsNormWeightOffset, weight2, activation, residual, alpha,
-    swigluLimit.  Equivalent to the matching sequence of runMatmul / runFusedFFN calls."""
-    arr = (capi.GemvPhase * len(phases))()
-    for i, ph in enumerate(phases):
-        g = arr[i]
-        g.d_A = _ptr(ph["input"])
-        g.d_norm_weight = _ptr(ph.get("normWeight"))
-        g.eps = float(ph.get("eps", 0.0))
-        g.weight_offset = 1 if ph.get("rmsNormWeightOffset") else 0
-        g.d_W = _ptr(ph["weight"])
-        g.d_W2 = _ptr(ph.get("weight2"))
-        g.d_C = _ptr(ph["output"])
-        g.d_residual = _ptr(ph.get("residual"))
-        g.N, g.K = int(ph["N"]), int(ph["K"])
-        g.activation = _act_code(ph.get("activation", "silu"), "GemvChain")
-        g.alpha = float(ph.get("alpha", 1.0))
-        g.swiglu_limit = float(ph.get("swigluLimit") or 0.0)
-    capi.check(_lib().dh_q4k_gemv_chain(arr, len(phases)))
-
-
 def runFusedNormedFFN(input, normWeight, eps, W_gate, W_up, hiddenSize, intermediateSize, batchSize=1,
                       activation="silu", alpha=1.0, outputBuffer=None, swigluLimit=None,
                       rmsNormWeightOffset=False, **_ignored):

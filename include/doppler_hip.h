@@ -124,33 +124,6 @@ int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup,
                        int M, int hidden, int inter, int activation, float alpha,
                        float swiglu_limit);
 
-/* Up to four dependent M = 1 products in one persistent launch (decode only): phase p computes
- *   C = alpha * W . norm(A) + residual            (d_W2 NULL), or
- *   C = act(W . norm(A)) * (W2 . norm(A)) * alpha (d_W2 given, activation DH_ACT_*),
- * norm = RMSNorm with d_norm_weight (NULL: none), and a later phase may read an earlier
- * phase's d_C as its d_A or d_residual.  Same arithmetic as the corresponding sequence of
- * dh_q4k_matmul[_rmsnorm] / dh_q4k_ffn_gate_up[_rmsnorm] calls, i.e. of the reference's
- * recordMatmul / recordFusedFFN calls of one decoder layer
- * (src/inference/pipelines/text/ffn/standard.js, attention/interpreter.js); what changes is
- * that the weight stream of phase p+1 starts while phase p finishes.  All buffers f32, K <=
- * 12288.  A launch that cannot get all its workgroups resident at once gives up at its first
- * grid barrier; dh_sync then reports the failure. */
-typedef struct dh_gemv_phase {
-  const float* d_A;            /* [K] */
-  const float* d_norm_weight;  /* [K] or NULL */
-  float eps;
-  int weight_offset;           /* 1: scale by (1 + w) */
-  const void* d_W;             /* Q4_K [N][K] */
-  const void* d_W2;            /* Q4_K [N][K] or NULL */
-  float* d_C;                  /* [N] */
-  const float* d_residual;     /* [N] or NULL */
-  int N, K;
-  int activation;
-  float alpha;
-  float swiglu_limit;
-} dh_gemv_phase;
-int dh_q4k_gemv_chain(const dh_gemv_phase* phases, int count);
-
 /* dh_q4k_ffn_gate_up over RMSNorm(x): the reference's "fused normed FFN",
  * src/gpu/kernels/fused_ffn.js:705-745,773-860 (there the inverse RMS comes in as a buffer,
  * here it is computed in the prologue).  d_norm_weight is f32 [hidden]; limits as for

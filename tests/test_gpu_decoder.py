@@ -1,4 +1,4 @@
-"""Whole-step parity: the HIP decoder (C-ABI ops chained by doppler_amd.decoder) against the
+"""Whole-step parity: the HIP decoder (C-ABI ops strung together by doppler_amd.decoder) against the
 CPU oracle's decode step on the same random-init weights.
 
 Bars: logits within relative L2 1e-3 at every checked position; greedy token ids identical.
@@ -34,19 +34,16 @@ def oracle_layers(layers, max_seq, kv_heads, head_dim):
     dict(layers=3, hidden=1024, inter=3072, heads=16, kv_heads=8, head_dim=128, vocab=2000, eps=1e-6, qk_norm=1),
     dict(layers=2, hidden=640, inter=2048, heads=4, kv_heads=1, head_dim=128, vocab=500, eps=1e-6, qk_norm=0),
 ])
-@pytest.mark.parametrize("chain,fuse_attn", [(False, True), (True, True), (False, False)],
-                         ids=["separate", "chained", "qkv-kernel-then-attention"])
-def test_small_models_prefill_and_greedy(cfg, chain, fuse_attn):
+@pytest.mark.parametrize("fuse_attn", [True, False], ids=["attention-from-qkv", "qkv-kernel-then-attention"])
+def test_small_models_prefill_and_greedy(cfg, fuse_attn):
     """Both sides start from an empty cache, consume 12 prompt tokens one at a time, then
-    decode 20 greedy tokens.  KV rows written on the way are compared too.  `chain` selects the
-    persistent chained-GEMV launch per layer instead of one kernel per projection; `fuse_attn`
+    decode 20 greedy tokens.  KV rows written on the way are compared too.  `fuse_attn` selects
     the attention kernel that norms, rotates and appends the step's q/k/v itself."""
     max_seq = 40
     cfg = dict(cfg, max_seq=max_seq, theta=1e6)
     layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=11, max_seq=max_seq)
-    gpu = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, max_seq, chain=chain,
-                             fuse_qkv_attention=fuse_attn)
-    assert gpu.chain == chain and gpu.fuse_qkv_attention == fuse_attn
+    gpu = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, max_seq, fuse_qkv_attention=fuse_attn)
+    assert gpu.fuse_qkv_attention == fuse_attn
     ol = oracle_layers(layers, max_seq, cfg["kv_heads"], cfg["head_dim"])
     cpu = oracle.DecoderOracle(cfg, ol, embed, final_norm, cos, sin)
     prompt = synth.rng(12).integers(0, cfg["vocab"], 12)

@@ -366,55 +366,6 @@ def test_matmul_rmsnorm_prologue_on_the_gemm_path(M, N, K):
     assert rel_l2(ops.readTensor(out), want - res) <= matmul_bar(M)
 
 
-@pytest.mark.parametrize("hidden,inter,qkv_rows", [(4096, 12288, 6144), (1024, 3072, 2048), (640, 1500, 700)])
-def test_gemv_chain_matches_separate_ops(hidden, inter, qkv_rows):
-    """o_proj(+residual) -> RMSNorm + gate/up -> down(+residual) -> RMSNorm + next qkv in one
-    persistent launch equals the four separate ops (checked against the oracle), and a second
-    launch right after gives the same bits (the grid-barrier counters carry over)."""
-    attn = synth.normal_f32((1, hidden), seed=2500)
-    x = synth.normal_f32((1, hidden), seed=2501)
-    Wo, wo = q4k_weight(hidden, hidden, seed=2502)
-    Wg, wg = q4k_weight(inter, hidden, seed=2503)
-    Wu, wu = q4k_weight(inter, hidden, seed=2504)
-    Wd, wd = q4k_weight(hidden, inter, seed=2505)
-    Wq, wq = q4k_weight(qkv_rows, hidden, seed=2506)
-    n1 = 1 + synth.normal_f32((hidden,), seed=2507, scale=0.1)
-    n2 = 1 + synth.normal_f32((hidden,), seed=2508, scale=0.1)
-    scale = 1.0 / 64.0          # keeps the synthetic activations O(1) through the chain
-    t = ops.tensorFromNumpy
-    x2, act, x3, qkv = (ops.createTensor(ops.acquireBuffer(n * 4), "f32", (1, n)) for n in (hidden, inter, hidden, qkv_rows))
-    phases = [
-        dict(input=t(attn), weight=wo, output=x2, residual=t(x), N=hidden, K=hidden, alpha=scale),
-        dict(input=x2, normWeight=t(n1), eps=1e-6, weight=wg, weight2=wu, output=act, N=inter, K=hidden,
-             activation="silu", alpha=scale),
-        dict(input=act, weight=wd, output=x3, residual=x2, N=hidden, K=inter, alpha=scale),
-        dict(input=x3, normWeight=t(n2), eps=1e-6, weight=wq, output=qkv, N=qkv_rows, K=hidden),
-    ]
-    ops.runGemvChain(phases)
-    got = [ops.readTensor(z).copy() for z in (x2, act, x3, qkv)]
-    ops.runGemvChain(phases)
-    again = [ops.readTensor(z) for z in (x2, act, x3, qkv)]
-    w_x2 = oracle.q4k_matmul(attn, Wo, 1, hidden, hidden, scale) + x
-    w_act = oracle.q4k_ffn_gate_up(oracle.rmsnorm(w_x2, n1, 1e-6), Wg, Wu, 1, hidden, inter, alpha=scale, activation="silu")
-    w_x3 = oracle.q4k_matmul(w_act, Wd, 1, hidden, inter, scale) + w_x2
-    w_qkv = oracle.q4k_matmul(oracle.rmsnorm(w_x3, n2, 1e-6), Wq, 1, qkv_rows, hidden, 1.0)
-    for g, a2, w in zip(got, again, (w_x2, w_act, w_x3, w_qkv)):
-        assert rel_l2(g, w) <= REL_L2_F32
-        assert g.tobytes() == a2.tobytes()
-
-
-def test_gemv_chain_rejects_bad_input():
-    W, wb = q4k_weight(64, 256, seed=2600)
-    a = ops.tensorFromNumpy(synth.normal_f32((1, 256), seed=2601))
-    out = ops.createTensor(ops.acquireBuffer(64 * 4), "f32", (1, 64))
-    with pytest.raises(DopplerHipError, match="between 1 and 4 phases"):
-        ops.runGemvChain([dict(input=a, weight=wb, output=out, N=64, K=256)] * 5)
-    with pytest.raises(DopplerHipError, match="exceeds the chained kernel's limit"):
-        ops.runGemvChain([dict(input=a, weight=wb, output=out, N=64, K=20000)])
-
-
-# ----------------------------------------------------------------------------- LM head, argmax, gather
-
 def test_f16_weight_matmul_and_lmhead_argmax():
     vocab, hidden = 5000, 1024
     E = synth.normal_f16_bits((vocab, hidden), seed=3000, scale=0.02)
