@@ -975,8 +975,8 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
     return dh::q4k_gemm(op, a.A, a.W, d_C, a.c_f16, M, N, K, alpha, a.residual, normed ? d_norm_weight : nullptr, eps,
                         weight_offset);
   if (normed)
-    return dh::fail(1, "[%s] the RMSNorm prologue serves K <= 14336 below 16 rows and K <= 16384 from 16 rows on "
-                    "(M=%d, K=%d); run dh_rmsnorm and dh_q4k_matmul instead", op, M, K);
+    return dh::fail(1, "[%s] the RMSNorm prologue serves K <= 28672 up to 2 rows, K <= 14336 up to 15 and K <= 16384 "
+                    "from 16 rows on (M=%d, K=%d); run dh_rmsnorm and dh_q4k_matmul instead", op, M, K);
   // tiles of up to 8 activation rows per pass over the weights
   const size_t c_elem = a.c_f16 ? 2 : 4;
   for (int m0 = 0; m0 < M; m0 += 8) {
@@ -1054,8 +1054,9 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
     return dh::q4k_gemm_gate_up(op, d_x, a.W, a.W2, d_out, M, hidden, inter, activation, alpha, swiglu_limit,
                                 normed ? d_norm_weight : nullptr, eps, weight_offset);
   if (normed)
-    return dh::fail(1, "[%s] the RMSNorm prologue serves hidden <= 14336 below 16 rows and hidden <= 16384 from 16 "
-                    "rows on (M=%d, hidden=%d); run dh_rmsnorm and dh_q4k_ffn_gate_up instead", op, M, hidden);
+    return dh::fail(1, "[%s] the RMSNorm prologue serves hidden <= 28672 up to 2 rows, hidden <= 14336 up to 15 and "
+                    "hidden <= 16384 from 16 rows on (M=%d, hidden=%d); run dh_rmsnorm and dh_q4k_ffn_gate_up instead", op, M,
+                    hidden);
   // any batch: tiles of up to 8 activation rows per pass
   for (int m0 = 0; m0 < M; m0 += 8) {
     GemvArgs b = a;

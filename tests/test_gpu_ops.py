@@ -283,7 +283,7 @@ def test_fused_ffn_random_shape_sweep():
 @pytest.mark.parametrize("M,N,K,offset", [(1, 6144, 4096, False), (2, 1024, 1024, True), (1, 2048, 640, False),
                                           (3, 96, 1152, False), (1, 4096, 12288, False), (5, 130, 2048, True),
                                           (4, 1024, 4096, False), (8, 512, 2048, True), (7, 256, 4096, False),
-                                          (2, 300, 12288, False)])
+                                          (2, 300, 12288, False), (2, 40, 20480, True), (1, 33, 28672, False)])
 def test_matmul_with_rmsnorm_prologue(M, N, K, offset):
     """runMatmul with normWeight + useFusedRmsnormWideTile == runRMSNorm followed by runMatmul
     (reference: src/gpu/kernels/matmul-selection.js:609-620)."""
@@ -314,7 +314,7 @@ def test_fused_normed_ffn_q4k(M, activation):
 
 
 def test_rmsnorm_prologue_fails_closed_for_rows_too_long_for_the_gemv():
-    K = 20480                                   # fragments of one row no longer fit beside the weight ring
+    K = 32768                                   # the row's operands no longer fit beside the weight ring
     W, wb = q4k_weight(32, K, seed=2300)
     A = ops.tensorFromNumpy(synth.normal_f32((2, K), seed=2301))
     nw = ops.tensorFromNumpy(np.ones(K, np.float32))
