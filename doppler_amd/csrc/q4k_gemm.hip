@@ -619,6 +619,23 @@ int launch_gemm(GemmArgs a, const char* op) {
   // waits; the pieces meet in the library's scratch buffer.
   if (!DUAL) {
     static const int env_split = env_ksplit();
+    static const int env_big = getenv("DH_GEMM_BIGSPLIT") ? atoi(getenv("DH_GEMM_BIGSPLIT")) : 1;
+    // 128 x 128 tiles with K cut into pieces when that fills the compute units: their matrix-core
+    // share is higher than that of 64 x 64 tiles
+    if (env_big) {
+      const int nkt = (a.K + BK - 1) / BK;
+      size_t ws_bytes = 0;
+      float* ws = dh::splitk_workspace(&ws_bytes);
+      int split = (int)std::min<int64_t>(8, dh::num_cus() / std::max<int64_t>(1, big_tiles));
+      split = std::min(split, nkt / 8);
+      while (split > 1 && (size_t)split * a.M * a.N * sizeof(float) > ws_bytes) split--;
+      if (split > 1 && ws && big_tiles * split * 2 >= dh::num_cus()) {
+        a.kt_per_split = (int)dh::ceil_div(nkt, split);
+        a.ksplit = (int)dh::ceil_div(nkt, a.kt_per_split);
+        a.partial = ws;
+        return launch_gemm_cfg<false, 2, 1>(a, op);
+      }
+    }
     const int64_t tiles = dh::ceil_div(a.M, 64) * dh::ceil_div(a.N, 64);
     const int nkt = (a.K + BK - 1) / BK;
     size_t ws_bytes = 0;
