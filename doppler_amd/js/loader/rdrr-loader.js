@@ -9,7 +9,9 @@
 //   f16 norm weights         widened to f32 on the host (tensor-loader.js:520-533)
 //   RoPE tables              frequency rounded to f32, angle and cos/sin in f64, stored f32
 //                            (src/inference/pipelines/text/init-rope.js:21-26,120-133)
-// Unsupported model features fail closed with the field named in the message.
+// Unsupported model features fail closed with the field named in the message.  A shard that
+// carries a sha256 hash is checked against it when first opened.
+import crypto from 'crypto';
 import fs from 'fs';
 import path from 'path';
 
@@ -48,6 +50,9 @@ export function parseManifest(jsonString) {
       offset: shard.offset !== undefined ? shard.offset : offset,
     };
     if (typeof shard.size !== 'number' || shard.size <= 0) errors.push(`Shard ${i} has invalid size`);
+    if (normalized.filename && (path.basename(normalized.filename) !== normalized.filename || normalized.filename === '.' || normalized.filename === '..')) {
+      errors.push(`Shard ${i} filename '${normalized.filename}' must be a plain file name inside the artifact directory`);
+    }
     offset += shard.size;
     return normalized;
   });
@@ -118,6 +123,15 @@ export function decoderConfig(manifest, maxSeq) {
   if (out.tieWordEmbeddings === false) unsupported('untied LM head');
   if (out.finalLogitSoftcapping || out.scaleEmbeddings) unsupported('logit soft cap / embedding scale');
   if (((inf.layerPattern || {}).type || 'uniform') !== 'uniform') unsupported('non-uniform layer pattern');
+  // scalars the decoder hard-wires: attention scale 1/sqrt(headDim), no logit or residual-branch scale
+  if (att.queryPreAttnScalar !== undefined && att.queryPreAttnScalar !== null && att.queryPreAttnScalar !== a.headDim) {
+    unsupported(`inference.attention.queryPreAttnScalar ${att.queryPreAttnScalar} != headDim ${a.headDim}`);
+  }
+  if (out.logitInputScale !== undefined && out.logitInputScale !== null && out.logitInputScale !== 1) {
+    unsupported(`inference.output.logitInputScale ${out.logitInputScale}`);
+  }
+  const rbs = (inf.layerPattern || {}).residualBranchScale;
+  if (rbs !== undefined && rbs !== null && rbs !== 1) unsupported(`inference.layerPattern.residualBranchScale ${rbs}`);
   return {
     layers: a.numLayers, hidden: a.hiddenSize, inter: a.intermediateSize, heads: a.numAttentionHeads,
     kvHeads: a.numKeyValueHeads, headDim: a.headDim, vocab: a.vocabSize,
@@ -147,8 +161,11 @@ function halfToFloat(bits) {
 }
 
 export class RdrrArtifact {
-  constructor(dir) {
+  // verifyHashes: check each shard that carries a hash against it when first opened (sha256 only;
+  // a hashed shard under another algorithm is refused unless this is off).
+  constructor(dir, { verifyHashes = true } = {}) {
     this.dir = dir;
+    this.verifyHashes = verifyHashes;
     this.manifest = parseManifest(fs.readFileSync(path.join(dir, 'manifest.json'), 'utf8'));
     if (!this.manifest.tensors || typeof this.manifest.tensors !== 'object') {
       let raw;
@@ -170,7 +187,27 @@ export class RdrrArtifact {
       if (!fs.existsSync(p)) throw new Error(`Shard file ${p} is missing`);
       const onDisk = fs.statSync(p).size;
       if (onDisk !== info.size) throw new Error(`Shard ${index} is ${onDisk} bytes on disk, manifest says ${info.size}`);
-      this.fds.set(index, fs.openSync(p, 'r'));
+      const fd = fs.openSync(p, 'r');
+      if (this.verifyHashes && info.hash) {
+        const algorithm = this.manifest.hashAlgorithm;
+        if (algorithm !== 'sha256') {
+          fs.closeSync(fd);
+          throw new Error(`Shard ${index} carries a ${algorithm} hash, which this loader cannot check (pass verifyHashes: false to load it unchecked)`);
+        }
+        const h = crypto.createHash('sha256'), buf = Buffer.allocUnsafe(16 << 20);
+        for (let at = 0; at < info.size;) {
+          const n = fs.readSync(fd, buf, 0, Math.min(buf.length, info.size - at), at);
+          if (n <= 0) break;
+          h.update(buf.subarray(0, n));
+          at += n;
+        }
+        const got = h.digest('hex');
+        if (got !== String(info.hash).toLowerCase()) {
+          fs.closeSync(fd);
+          throw new Error(`Shard ${index} fails its sha256 check (manifest ${info.hash}, file ${got})`);
+        }
+      }
+      this.fds.set(index, fd);
     }
     return this.fds.get(index);
   }

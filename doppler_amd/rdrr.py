@@ -12,10 +12,12 @@ Mirrors what the reference's loader does for the tensors this path consumes:
 Q4_K bytes are never repacked: a tensor's bytes in the shard are exactly what the GEMV kernels
 read.  Anything this path cannot run (MoE, non-row Q4_K layout, other weight dtypes, sliding
 windows, soft caps, per-layer patterns) fails closed with an error that names the field.
+A shard that carries a sha256 hash is checked against it when first opened; a mismatch is an error.
 
 write_artifact() produces the same on-disk format from arrays; tests and examples use it to make
 synthetic artifacts (the reference ships manifests, not shards).
 """
+import hashlib
 import json
 import mmap
 import os
@@ -63,6 +65,8 @@ def normalize_manifest(manifest):
             errors.append("Shard %d has invalid size" % i)
             continue
         fn = s.get("filename") or s.get("fileName") or ""
+        if os.path.basename(fn) != fn or fn in (".", ".."):
+            errors.append("Shard %d filename %r must be a plain file name inside the artifact directory" % (i, fn))
         if not fn:
             errors.append("Shard %d missing filename" % i)
         norm.append({"index": s.get("index", i), "filename": fn, "size": s["size"],
@@ -140,8 +144,11 @@ def parse_manifest(text):
 class Artifact:
     """A directory with manifest.json (+ optional tensors file) and its shards, memory-mapped."""
 
-    def __init__(self, directory):
+    def __init__(self, directory, verify_hashes=True):
+        """`verify_hashes`: check each shard that carries a hash against it when the shard is first
+        opened (sha256 only; a hashed shard under another algorithm is refused unless this is off)."""
         self.dir = directory
+        self.verify_hashes = verify_hashes
         with open(os.path.join(directory, "manifest.json"), "r") as f:
             self.manifest = parse_manifest(f.read())
         if "tensors" not in self.manifest or not isinstance(self.manifest["tensors"], dict):
@@ -166,6 +173,17 @@ class Artifact:
                                 (index, os.path.getsize(path), info["size"]))
             f = open(path, "rb")
             m = (f, mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_READ))
+            if self.verify_hashes and info["hash"]:
+                algorithm = self.manifest.get("hashAlgorithm")
+                if algorithm != "sha256":
+                    raise RdrrError("Shard %d carries a %r hash, which this loader cannot check "
+                                    "(pass verify_hashes=False to load it unchecked)" % (index, algorithm))
+                h = hashlib.sha256()
+                for at in range(0, info["size"], 64 << 20):
+                    h.update(m[1][at:at + (64 << 20)])
+                if h.hexdigest() != info["hash"].lower():
+                    raise RdrrError("Shard %d fails its sha256 check (manifest %s, file %s)" %
+                                    (index, info["hash"], h.hexdigest()))
             self._maps[index] = m
         return m[1]
 
@@ -225,6 +243,12 @@ def decoder_config(manifest):
     _require(outp.get("tieWordEmbeddings", True), "untied LM head")
     _require(not outp.get("finalLogitSoftcapping") and not outp.get("scaleEmbeddings"), "logit soft cap / embedding scale")
     _require((inf.get("layerPattern") or {}).get("type", "uniform") == "uniform", "non-uniform layer pattern")
+    # scalars the decoder hard-wires: attention scale 1/sqrt(headDim), no logit or residual-branch scale
+    qpas = att.get("queryPreAttnScalar")
+    _require(qpas in (None, a["headDim"]), "inference.attention.queryPreAttnScalar %r != headDim %d" % (qpas, a["headDim"]))
+    _require(outp.get("logitInputScale") in (None, 1, 1.0), "inference.output.logitInputScale %r" % outp.get("logitInputScale"))
+    rbs = (inf.get("layerPattern") or {}).get("residualBranchScale")
+    _require(rbs in (None, 1, 1.0), "inference.layerPattern.residualBranchScale %r" % rbs)
     return dict(layers=a["numLayers"], hidden=a["hiddenSize"], inter=a["intermediateSize"],
                 heads=a["numAttentionHeads"], kv_heads=a["numKeyValueHeads"], head_dim=a["headDim"],
                 vocab=a["vocabSize"], eps=float(nrm.get("rmsNormEps", 1e-6)),
@@ -302,11 +326,12 @@ def load_decoder(directory, max_seq, **decoder_kwargs):
 
 
 def write_artifact(directory, cfg, layers, embed_bits, final_norm, shard_bytes=64 << 20, model_id="synthetic-q4k",
-                   layout=None):
+                   layout=None, hash_shards=None):
     """Writes manifest.json and shards for a dense Q4_K decoder.  Tensors are laid out in name
     order into shards of `shard_bytes`; a tensor that does not fit the rest of a shard is split
     into spans, as the reference's converter does for large embeddings.  `layout`, if given,
-    maps tensor name -> spans to write at (used to reproduce an existing manifest's placement)."""
+    maps tensor name -> spans to write at (used to reproduce an existing manifest's placement).
+    `hash_shards`: record each shard's sha256 (default: only when the artifact is under 1 GiB)."""
     os.makedirs(directory, exist_ok=True)
     items = {"embed_tokens.weight": (np.ascontiguousarray(embed_bits).view(np.uint8).reshape(-1),
                                      [cfg["vocab"], cfg["hidden"]], "F16", "embedding", "embed"),
@@ -367,8 +392,17 @@ def write_artifact(directory, cfg, layers, embed_bits, final_norm, shard_bytes=6
     for f in files.values():
         f.close()
     offset, shards = 0, []
+    if hash_shards is None:
+        hash_shards = sum(shard_sizes) < (1 << 30)
     for i, size in enumerate(shard_sizes):
-        shards.append({"index": i, "filename": shard_filename(i), "size": int(size), "hash": "", "offset": offset})
+        digest = ""
+        if hash_shards:
+            h = hashlib.sha256()
+            with open(os.path.join(directory, shard_filename(i)), "rb") as f:
+                for chunk in iter(lambda: f.read(64 << 20), b""):
+                    h.update(chunk)
+            digest = h.hexdigest()
+        shards.append({"index": i, "filename": shard_filename(i), "size": int(size), "hash": digest, "offset": offset})
         offset += size
     manifest = {
         "version": RDRR_VERSION, "modelId": model_id, "modelType": "transformer", "quantization": "Q4_K_M",

@@ -98,6 +98,8 @@ def _manifest_with(tmp_path, mutate):
     (lambda m: m["tensors"]["layers.0.mlp.up_proj.weight"].update(offset=10 ** 9), "past the end of shard"),
     (lambda m: m.pop("shards"), "Missing or empty shards"),
     (lambda m: m.pop("tensors"), "Missing tensorsFile and tensors"),
+    (lambda m: m["shards"][0].update(filename="../shard_00000.bin"), "plain file name"),
+    (lambda m: m["shards"][0].update(filename="/etc/passwd"), "plain file name"),
 ])
 def test_manifest_errors_fail_closed(tmp_path, mutate, match):
     _manifest_with(tmp_path, mutate)
@@ -113,6 +115,9 @@ def test_manifest_errors_fail_closed(tmp_path, mutate, match):
     (lambda m: m["tensors"]["layers.1.self_attn.q_proj.weight"].update(layout="column"), "row layout"),
     (lambda m: m["tensors"].pop("layers.1.mlp.down_proj.weight"), "is not in the manifest"),
     (lambda m: m["architecture"].pop("headDim"), "architecture.headDim"),
+    (lambda m: m["inference"]["attention"].update(queryPreAttnScalar=256), "queryPreAttnScalar"),
+    (lambda m: m["inference"]["output"].update(logitInputScale=0.5), "logitInputScale"),
+    (lambda m: m["inference"].setdefault("layerPattern", {}).update(residualBranchScale=0.22), "residualBranchScale"),
 ])
 def test_unsupported_models_fail_closed(tmp_path, mutate, match):
     _manifest_with(tmp_path, mutate)
@@ -132,3 +137,70 @@ def test_truncated_shard_is_detected(tmp_path):
     with pytest.raises(rdrr.RdrrError, match="bytes on disk"):
         rdrr.load_model_arrays(art)
     art.close()
+
+
+def test_corrupted_shard_fails_its_hash_check(tmp_path):
+    layers, embed, final_norm = tiny_model()
+    man = rdrr.write_artifact(str(tmp_path), TINY, layers, embed, final_norm, shard_bytes=1 << 20)
+    import hashlib
+    for s in man["shards"]:
+        with open(os.path.join(str(tmp_path), s["filename"]), "rb") as f:
+            assert hashlib.sha256(f.read()).hexdigest() == s["hash"]
+    p = os.path.join(str(tmp_path), rdrr.shard_filename(0))
+    with open(p, "r+b") as f:
+        f.seek(1000)
+        b = f.read(1)
+        f.seek(1000)
+        f.write(bytes([b[0] ^ 0x10]))
+    art = rdrr.Artifact(str(tmp_path))
+    with pytest.raises(rdrr.RdrrError, match="fails its sha256 check"):
+        rdrr.load_model_arrays(art)
+    art.close()
+    art = rdrr.Artifact(str(tmp_path), verify_hashes=False)
+    rdrr.load_model_arrays(art)
+    art.close()
+
+
+def test_a_hash_this_loader_cannot_check_is_refused(tmp_path):
+    _manifest_with(tmp_path, lambda m: m.update(hashAlgorithm="blake3"))
+    art = rdrr.Artifact(str(tmp_path))
+    with pytest.raises(rdrr.RdrrError, match="cannot check"):
+        rdrr.load_model_arrays(art)
+    art.close()
+
+
+@pytest.mark.skipif(__import__("shutil").which("node") is None, reason="node is not installed")
+def test_js_loader_checks_hashes_and_shard_names(tmp_path):
+    import subprocess
+    layers, embed, final_norm = tiny_model()
+    rdrr.write_artifact(str(tmp_path), TINY, layers, embed, final_norm, shard_bytes=1 << 20)
+    loader = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                          "doppler_amd", "js", "loader", "rdrr-loader.js")
+    script = """
+import fs from 'fs';
+import { RdrrArtifact, parseManifest } from %r;
+const dir = %r;
+const name = Object.keys(new RdrrArtifact(dir).tensors)[0];
+new RdrrArtifact(dir).tensorBytes(name);
+const text = fs.readFileSync(dir + '/manifest.json', 'utf8');
+const m = JSON.parse(text);
+m.shards[0].filename = '../x.bin';
+let caught = '';
+try { parseManifest(JSON.stringify(m)); } catch (e) { caught = e.message; }
+if (!/plain file name/.test(caught)) throw new Error('path component accepted: ' + caught);
+const p = dir + '/shard_00000.bin';
+const bytes = fs.readFileSync(p);
+bytes[1000] ^= 0x10;
+fs.writeFileSync(p, bytes);
+caught = '';
+try { const a = new RdrrArtifact(dir); for (const n of Object.keys(a.tensors)) a.tensorBytes(n); } catch (e) { caught = e.message; }
+if (!/fails its sha256 check/.test(caught)) throw new Error('corruption accepted: ' + caught);
+const a = new RdrrArtifact(dir, { verifyHashes: false });
+for (const n of Object.keys(a.tensors)) a.tensorBytes(n);
+console.log('ok');
+""" % (loader, str(tmp_path))
+    src = tmp_path / "check.mjs"
+    src.write_text(script)
+    out = subprocess.run(["node", str(src)], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.strip() == "ok"
