@@ -94,6 +94,11 @@ int attn_static_scratch_init(int device);
 int q4k_gemv_i8(const char* op, const float* A, const uint8_t* W, const uint8_t* W2, void* C, int c_f16,
                 const float* residual, int M, int N, int K, float alpha, int activation, float clamp_max,
                 const float* norm_weight, float norm_eps, int norm_weight_offset);
+// The same product for up to 8 activation rows in one pass over the weights, on the f16 matrix cores
+// (q4k_gemv_rows.hip).  Same arguments and return values.
+int q4k_gemv_rows(const char* op, const float* A, const uint8_t* W, const uint8_t* W2, void* C, int c_f16,
+                  const float* residual, int M, int N, int K, float alpha, int activation, float clamp_max,
+                  const float* norm_weight, float norm_eps, int norm_weight_offset);
 
 }  // namespace dh
 

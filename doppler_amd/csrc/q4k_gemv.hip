@@ -956,6 +956,17 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
     if (rc >= 0) return rc;
   }
   if ((path == 0 || normed) && M < 16) {
+    // below the GEMM's batch size: passes of up to 8 rows, each one sweep over the weights
+    int rc = 0;
+    for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
+      rc = dh::q4k_gemv_rows(op, a.A + (int64_t)m0 * K, a.W, nullptr, static_cast<char*>(d_C) + (int64_t)m0 * N * (a.c_f16 ? 2 : 4),
+                             a.c_f16, a.residual ? a.residual + (int64_t)m0 * N : nullptr, std::min(8, M - m0), N, K, alpha, 0,
+                             0.f, normed ? d_norm_weight : nullptr, eps, weight_offset);
+      if (rc < 0 && m0 > 0) return dh::fail(2, "[%s] internal: GEMV pass %d did not launch after pass 0 did", op, m0 / 8);
+    }
+    if (rc >= 0) return rc;
+  }
+  if ((path == 0 || normed) && M < 16) {
     // below the GEMM's batch size: passes of up to 8 rows through the streaming GEMV
     int rc = 0;
     for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
@@ -975,8 +986,9 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
     return dh::q4k_gemm(op, a.A, a.W, d_C, a.c_f16, M, N, K, alpha, a.residual, normed ? d_norm_weight : nullptr, eps,
                         weight_offset);
   if (normed)
-    return dh::fail(1, "[%s] the RMSNorm prologue serves K <= 28672 up to 2 rows, K <= 14336 up to 15 and K <= 16384 "
-                    "from 16 rows on (M=%d, K=%d); run dh_rmsnorm and dh_q4k_matmul instead", op, M, K);
+    return dh::fail(1, "[%s] the RMSNorm prologue serves any K up to 15 rows (K <= 14336 for matrices of more than "
+                    "61440 rows) and K <= 16384 from 16 rows on (M=%d, K=%d); run dh_rmsnorm and dh_q4k_matmul instead", op,
+                    M, K);
   // tiles of up to 8 activation rows per pass over the weights
   const size_t c_elem = a.c_f16 ? 2 : 4;
   for (int m0 = 0; m0 < M; m0 += 8) {
@@ -1039,6 +1051,16 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
   if ((path == 0 || normed) && M < 16) {
     int rc = 0;
     for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
+      rc = dh::q4k_gemv_rows(op, d_x + (int64_t)m0 * hidden, a.W, a.W2, d_out + (int64_t)m0 * inter, 0, nullptr,
+                             std::min(8, M - m0), inter, hidden, alpha, activation, swiglu_limit,
+                             normed ? d_norm_weight : nullptr, eps, weight_offset);
+      if (rc < 0 && m0 > 0) return dh::fail(2, "[%s] internal: GEMV pass %d did not launch after pass 0 did", op, m0 / 8);
+    }
+    if (rc >= 0) return rc;
+  }
+  if ((path == 0 || normed) && M < 16) {
+    int rc = 0;
+    for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
       RingArgs g{};
       g.A = d_x + (int64_t)m0 * hidden; g.W = a.W; g.W2 = a.W2; g.C = d_out + (int64_t)m0 * inter; g.residual = nullptr;
       g.M = std::min(8, M - m0); g.N = inter; g.K = hidden; g.nb = a.nb; g.alpha = alpha; g.c_f16 = 0;
@@ -1054,9 +1076,9 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
     return dh::q4k_gemm_gate_up(op, d_x, a.W, a.W2, d_out, M, hidden, inter, activation, alpha, swiglu_limit,
                                 normed ? d_norm_weight : nullptr, eps, weight_offset);
   if (normed)
-    return dh::fail(1, "[%s] the RMSNorm prologue serves hidden <= 28672 up to 2 rows, hidden <= 14336 up to 15 and "
-                    "hidden <= 16384 from 16 rows on (M=%d, hidden=%d); run dh_rmsnorm and dh_q4k_ffn_gate_up instead", op, M,
-                    hidden);
+    return dh::fail(1, "[%s] the RMSNorm prologue serves any hidden size up to 15 rows (hidden <= 14336 for more than "
+                    "30720 intermediate rows) and hidden <= 16384 from 16 rows on (M=%d, hidden=%d); run dh_rmsnorm and "
+                    "dh_q4k_ffn_gate_up instead", op, M, hidden);
   // any batch: tiles of up to 8 activation rows per pass
   for (int m0 = 0; m0 < M; m0 += 8) {
     GemvArgs b = a;

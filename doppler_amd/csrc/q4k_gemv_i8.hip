@@ -21,9 +21,8 @@
 // wave draws the next unit of the workgroup from a counter in LDS, has the load unit fetch it
 // straight into its private LDS ring (global_load_lds, 16 bytes per lane, 9 lanes per row), and
 // reads the activation operands of the unit's column from LDS.  Those are prepared once per
-// launch by the first eight waves (wave w quantises columns w, w+8, .. and raises a flag per
-// column) while the other eight already stream weights; a wave that meets a column whose flag
-// is not up yet waits for it.  Waves that get the memory pipeline first (the hardware favours the
+// launch: wave w quantises columns w, w+16, .. and raises a flag per column, with its first
+// weight unit already in flight; a wave that meets a column whose flag is not up yet waits for it.  Waves that get the memory pipeline first (the hardware favours the
 // oldest) simply draw more units, so all sixteen finish together and the pipeline stays full until
 // the end.  A unit's 16 partial sums go to LDS; the wave that delivers the last unit of a tile
 // adds them in column order (deterministic) and writes the outputs.  The only workgroup barrier
@@ -131,13 +130,6 @@ __device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
   return v;
 }
 
-#ifdef DH_I8_TRACE
-__device__ unsigned long long dh_i8_trace[256 * 16 * 32];
-#define DH_TS(k) do { if (lane == 0) ts_lds[wave][(k) & 31] = wall_clock64(); } while (0)
-#else
-#define DH_TS(k) do {} while (0)
-#endif
-
 // Layout of the dynamic LDS block, in this order:
 //   ring   [16 waves][depth][2304]
 //   xq     [nb][MT][kRec]: per column and activation row, digit plane p at 256 p (byte e = digit p
@@ -149,17 +141,10 @@ __device__ unsigned long long dh_i8_trace[256 * 16 * 32];
 template <int MT, bool DUAL, bool VEC>
 __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Args a) {
   constexpr int NMAT = DUAL ? 2 : 1;
-#ifdef DH_I8_TRACE
-  __shared__ unsigned long long ts_lds[kWaves][32];
-#endif
   extern __shared__ __align__(16) unsigned char lds[];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-#ifdef DH_I8_TRACE
-  if (lane < 32) ts_lds[wave][lane] = 0ull;
-#endif
-  DH_TS(0);
   // Every kernel argument is fetched in one batch here (left alone the compiler fetches some of
   // them only where they are first used: a second, dependent trip to memory).
   asm volatile("" :: "s"(a.A), "s"(a.W), "s"(a.W2), "s"(a.C), "s"(a.residual), "s"(a.norm_weight));
@@ -276,7 +261,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
   }
   // counters, flags and the zero area are in place; costs little more than the skew of the wave launches
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  DH_TS(1);
 
   // Draws the next unit of the workgroup (wave-uniform result).
   const uint32_t ctr_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(ctr);
@@ -296,7 +280,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     DH_ISSUE(u_ring[0], 0);
     inflight = 1;
   }
-  DH_TS(2);
   {
 #pragma unroll 1
     for (int c0 = 0; c0 < my_cols; c0 += SC) {
@@ -360,11 +343,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
         }
       }
     }
-    DH_TS(3);
   }
 #undef DH_LOAD_X
 #undef DH_TIE_X
-  DH_TS(4);
 
   // ---- 5. stream the units
   // MFMA pair cc (sub-blocks 4cc .. 4cc+3): the first MFMA takes the low nibbles of the 16 bytes
@@ -423,7 +404,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     unsigned nxt = 0;
     if (lane == 0) asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=&v"(nxt) : "v"(ctr_abs), "v"(1u) : "memory");
     wait_vm_at_most((inflight - 1) * a.nlw);
-    DH_TS(5 + (cur >> 4));
     const uint32_t hp = lane_hdr + cstage * kStage, qp = lane_q + cstage * kStage;
     const uint32_t rec = xq_abs + (uint32_t)(col * MT) * kRec;
     const uint32_t gen_addr = ctr_abs + 4 * (1 + nslots + slot);
@@ -614,10 +594,6 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
       }
     }
   }
-  DH_TS(31);
-#ifdef DH_I8_TRACE
-  if (lane < 32 && blockIdx.x < 256) dh_i8_trace[(blockIdx.x * 16 + wave) * 32 + lane] = ts_lds[wave][lane];
-#endif
 #undef DH_ISSUE
 #undef DH_DECODE
 }
@@ -631,9 +607,6 @@ template <int MT, bool DUAL, bool VEC>
 int launch_i8_vec(I8Args a, const char* op) {
   constexpr int NMAT = DUAL ? 2 : 1;
   size_t cap = kMaxLds;
-#ifdef DH_I8_TRACE
-  cap -= 4096;
-#endif
   auto kern = q4k_gemv_i8_kernel<MT, DUAL, VEC>;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
@@ -727,12 +700,6 @@ int dispatch_i8(const I8Args& a, const char* op) {
 }
 
 }  // namespace
-
-#ifdef DH_I8_TRACE
-extern "C" int dh_debug_i8_trace(void* host_dst) {
-  return (int)hipMemcpyFromSymbol(host_dst, HIP_SYMBOL(dh_i8_trace), sizeof(dh_i8_trace));
-}
-#endif
 
 namespace dh {
 

@@ -109,9 +109,9 @@ int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int 
  * standalone norm dispatch in front of the q/k/v and gate/up projections disappears.
  * Replaces runMatmul with `normWeight` + `useFusedRmsnormWideTile`,
  * src/gpu/kernels/matmul-selection.js:609-620 (fused_rmsnorm_q4_widetile.wgsl:4-24,189-215).
- * d_norm_weight is f32 [K].  Below 16 rows the norm runs in the GEMV's prologue (K <= 14336; K <= 28672 for one or two rows), from
- * 16 rows on while the GEMM's activations are packed (K <= 16384); longer rows fail with a message
- * (run dh_rmsnorm + dh_q4k_matmul). */
+ * d_norm_weight is f32 [K].  Below 16 rows the norm runs in the GEMV's prologue (any K; K <= 14336
+ * for matrices of more than 61440 rows), from 16 rows on while the GEMM's activations are packed
+ * (K <= 16384); longer rows fail with a message (run dh_rmsnorm + dh_q4k_matmul). */
 int dh_q4k_matmul_rmsnorm(const float* d_A, const float* d_norm_weight, float eps,
                           int weight_offset, const void* d_W, void* d_C, int c_dtype, int M,
                           int N, int K, float alpha, const void* d_residual);

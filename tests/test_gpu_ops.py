@@ -313,14 +313,26 @@ def test_fused_normed_ffn_q4k(M, activation):
     assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
 
 
-def test_rmsnorm_prologue_fails_closed_for_rows_too_long_for_the_gemv():
-    K = 32768                                   # the row's operands no longer fit beside the weight ring
+def test_rmsnorm_prologue_fails_closed_for_rows_too_long_for_the_gemm():
+    K = 32768                                   # from 16 rows on the product is the GEMM's, whose prologue stops at 16384
     W, wb = q4k_weight(32, K, seed=2300)
-    A = ops.tensorFromNumpy(synth.normal_f32((2, K), seed=2301))
+    A = ops.tensorFromNumpy(synth.normal_f32((16, K), seed=2301))
     nw = ops.tensorFromNumpy(np.ones(K, np.float32))
     with pytest.raises(DopplerHipError, match="RMSNorm prologue"):
-        ops.runMatmul(A, wb, 2, 32, K, outputDtype="f32", normWeight=nw, rmsNormEps=1e-6,
+        ops.runMatmul(A, wb, 16, 32, K, outputDtype="f32", normWeight=nw, rmsNormEps=1e-6,
                       useFusedRmsnormWideTile=True)
+
+
+@pytest.mark.parametrize("M,N,K", [(2, 32, 32768), (7, 40, 32768), (12, 33, 20480)])
+def test_rmsnorm_prologue_long_rows_below_the_gemm_batch(M, N, K):
+    """Up to 15 rows the few-row kernel converts the activations column by column: no limit on K."""
+    W, wb = q4k_weight(N, K, seed=2310 + M)
+    A = synth.normal_f32((M, K), seed=2311 + M, scale=2.0)
+    nw = 1.0 + synth.normal_f32((K,), seed=2312 + M, scale=0.1)
+    out = ops.runMatmul(ops.tensorFromNumpy(A), wb, M, N, K, outputDtype="f32", normWeight=ops.tensorFromNumpy(nw),
+                        rmsNormEps=1e-6, useFusedRmsnormWideTile=True)
+    want = oracle.q4k_matmul(oracle.rmsnorm(A, nw, 1e-6), W, M, N, K, 1.0)
+    assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
 
 
 @pytest.mark.parametrize("M", [9, 12, 15])
