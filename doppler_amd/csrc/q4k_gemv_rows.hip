@@ -142,11 +142,11 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  // every kernel argument is fetched in one batch
-  asm volatile("" :: "s"(a.A), "s"(a.W), "s"(a.W2), "s"(a.C), "s"(a.residual), "s"(a.norm_weight));
+  // the arguments the streaming loop uses are fetched in one batch (left alone the compiler fetches
+  // some of them only where they are first used: a second, dependent trip to memory)
+  asm volatile("" :: "s"(a.A), "s"(a.W), "s"(a.W2), "s"(a.norm_weight));
   asm volatile("" :: "s"(a.M), "s"(a.N), "s"(a.K), "s"(a.nb), "s"(a.depth), "s"(a.rows), "s"(a.nlw), "s"(a.grid),
-               "s"(a.tiles_base), "s"(a.tiles_rem), "s"(a.acc_max), "s"(a.c_f16), "s"(a.activation), "s"(a.norm_weight_offset));
-  asm volatile("" :: "s"(a.alpha), "s"(a.clamp_max), "s"(a.norm_eps));
+               "s"(a.tiles_base), "s"(a.tiles_rem), "s"(a.acc_max));
 
   const int D = a.depth, nb = a.nb;
   const bool norm = a.norm_weight != nullptr;
@@ -277,9 +277,12 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
         for (int e = 0; e < 4; e++)
           if (col * kQK + 32 * s + xk + e >= a.K) xr[s][e] = 0.f;
     }
+    // (one instruction per two elements; written through fmaxf/fabsf the compiler spends four)
 #pragma unroll
-    for (int s = 0; s < 8; s++)
-      mx = fmaxf(fmaxf(mx, fmaxf(fabsf(xr[s][0]), fabsf(xr[s][1]))), fmaxf(fabsf(xr[s][2]), fabsf(xr[s][3])));
+    for (int s = 0; s < 8; s++) {
+      asm("v_max3_f32 %0, %0, |%1|, |%2|" : "+v"(mx) : "v"(xr[s][0]), "v"(xr[s][1]));
+      asm("v_max3_f32 %0, %0, |%1|, |%2|" : "+v"(mx) : "v"(xr[s][2]), "v"(xr[s][3]));
+    }
     mx = row_lanes_max(mx);
     int ex = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;      // mx < 2^(ex+1)
     ex = max(-100, min(100, ex));
