@@ -555,8 +555,10 @@ int launch_rows(RowsArgs a, const char* op) {
   a.tiles_base = (int)(ntiles / grid);
   a.tiles_rem = (int)(ntiles % grid);
   a.acc_max = (a.tiles_base + (a.tiles_rem ? 1 : 0)) * NMAT;
-  // a run per wave: with fewer units than waves most of the workgroup would idle
-  if ((int64_t)a.nb * a.tiles_base * NMAT < kWaves) return -1;
+  // about a run per wave: with far fewer units than waves most of the workgroup idles, and the
+  // kernel that spreads a tile's columns over the waves is faster (measured on 1024 x 3072 and smaller)
+  static const int env_min_units = env_int("DH_GEMV_ROWS_MIN_UNITS", 12);
+  if ((int64_t)a.nb * a.tiles_base * NMAT < env_min_units) return -1;
   auto lds_for = [&](int dep) {
     return (size_t)kWaves * dep * kStage + (a.norm_weight ? sizeof(float) * kWaves * kQK : 0) +
            sizeof(float) * kWaves * kSsqFloats + (size_t)kWaves * a.acc_max * kAccBytes;
