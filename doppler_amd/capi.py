@@ -85,6 +85,8 @@ SIGNATURES = {
     "dh_sample_topk": (_I, [_P, _I, ctypes.c_double, _I, ctypes.c_double, _I64, _F, _P, _P, _I]),
     "dh_cast_f32_to_f16": (_I, [_P, _P, _I64]),
     "dh_cast_f16_to_f32": (_I, [_P, _P, _I64]),
+    "dh_matmul_rmsnorm_f32": (_I, [_P, _P, _I, _P, _I, _F, _I, _P, _P, _I, _I]),
+    "dh_check_finiteness": (_I, [_P, _I, _I64, _P, ctypes.c_uint32, ctypes.c_uint32, _F]),
 }
 
 

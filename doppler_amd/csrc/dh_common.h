@@ -30,6 +30,9 @@ float* gemm_row_scale();
 // Packed f16 activations of the prefill GEMM (rows x K rounded up to 64 halves).
 void* gemm_packed_a(size_t* bytes);
 int gemm_row_scale_capacity();
+// f32 copy of f16 activations handed to dh_q4k_matmul (allocated by dh_init; one matmul at a time
+// uses it, in stream order).
+float* widened_activations(size_t* bytes);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

@@ -19,6 +19,8 @@ float* g_row_scale = nullptr;        // [kRowScaleRows][2] activation row factor
 constexpr int kRowScaleRows = 65536;
 void* g_packed_a = nullptr;          // packed f16 activations of the prefill GEMM
 constexpr size_t kPackedABytes = (size_t)64 << 20;
+float* g_widened_a = nullptr;        // f16 activations of dh_q4k_matmul widened to f32
+constexpr size_t kWidenedABytes = (size_t)64 << 20;
 }  // namespace
 
 namespace dh {
@@ -56,6 +58,10 @@ void* gemm_packed_a(size_t* bytes) {
   return g_packed_a;
 }
 int gemm_row_scale_capacity() { return kRowScaleRows; }
+float* widened_activations(size_t* bytes) {
+  *bytes = g_widened_a ? kWidenedABytes : 0;
+  return g_widened_a;
+}
 }  // namespace dh
 
 extern "C" {
@@ -73,11 +79,13 @@ static int release_all(const char* op) {
   if (g_splitk_ws) note(hipFree(g_splitk_ws));
   if (g_row_scale) note(hipFree(g_row_scale));
   if (g_packed_a) note(hipFree(g_packed_a));
+  if (g_widened_a) note(hipFree(g_widened_a));
   g_own_stream = nullptr;
   g_stream = nullptr;
   g_splitk_ws = nullptr;
   g_row_scale = nullptr;
   g_packed_a = nullptr;
+  g_widened_a = nullptr;
   g_num_cus = 0;
   g_ready = false;
   g_device = -1;
@@ -102,6 +110,7 @@ static int init_locked(int device_ordinal) {
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_splitk_ws), kSplitKWsBytes));
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_row_scale), (size_t)kRowScaleRows * 2 * sizeof(float)));
   DH_CHECK_HIP("dh_init", hipMalloc(&g_packed_a, kPackedABytes));
+  DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_widened_a), kWidenedABytes));
   if (int rc = dh::attn_static_scratch_init(device_ordinal)) return rc;
   g_device = device_ordinal;
   g_ready = true;

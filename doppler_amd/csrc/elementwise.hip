@@ -2,6 +2,7 @@
 // All of these move a few KB per token: they are launch-bound, so each is one launch with
 // 16-byte accesses where alignment allows and no intermediate buffers.
 #include <algorithm>
+#include <cmath>
 
 #include "dh_common.h"
 
@@ -400,6 +401,26 @@ __global__ __launch_bounds__(256) void cast_f16_f32_kernel(const __half* __restr
   if (i < n) out[i] = __half2float(in[i]);
 }
 
+// status[0] goes 0 -> 1 for the first element that is not finite or whose magnitude exceeds the
+// threshold; the launch that wins the exchange records its layer and step beside it.
+template <typename T>
+__global__ __launch_bounds__(256) void check_finiteness_kernel(const T* __restrict__ in, int64_t n,
+                                                               uint32_t* __restrict__ status, uint32_t layer,
+                                                               uint32_t step, float abs_threshold) {
+  int bad = 0;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const float v = static_cast<float>(in[i]);
+    const uint32_t bits = __float_as_uint(v);
+    bad |= ((bits & 0x7F800000u) == 0x7F800000u) | (fabsf(v) > abs_threshold);
+  }
+  if (__syncthreads_or(bad) && threadIdx.x == 0) {
+    if (atomicCAS(&status[0], 0u, 1u) == 0u) {
+      __hip_atomic_store(&status[1], layer, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&status[2], step, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
 unsigned grid_for(int64_t n) { return (unsigned)dh::ceil_div(n, 256); }
 
 }  // namespace
@@ -713,6 +734,27 @@ int dh_cast_f16_to_f32(const void* d_in, float* d_out, int64_t n) {
   if (!d_in || !d_out) return dh::fail(1, "[%s] null pointer", op);
   hipLaunchKernelGGL(cast_f16_f32_kernel, dim3(grid_for(n)), dim3(256), 0, dh::stream(),
                      static_cast<const __half*>(d_in), d_out, n);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+int dh_check_finiteness(const void* d_input, int dtype, int64_t size, uint32_t* d_status, uint32_t layer,
+                        uint32_t step, float abs_threshold) {
+  const char* op = "dh_check_finiteness";
+  DH_REQUIRE_INIT(op);
+  if (size < 0) return dh::fail(1, "[%s] size must be non-negative", op);
+  if (dtype != DH_F32 && dtype != DH_F16) return dh::fail(1, "[%s] input dtype must be f32 or f16", op);
+  if (!d_status) return dh::fail(1, "[%s] status pointer is null", op);
+  if (size == 0) return 0;
+  if (!d_input) return dh::fail(1, "[%s] null pointer", op);
+  if (!(abs_threshold > 0.f) || !std::isfinite(abs_threshold)) abs_threshold = 65500.f;
+  const unsigned grid = (unsigned)std::min<int64_t>(dh::ceil_div(size, 256), 4096);
+  if (dtype == DH_F16)
+    hipLaunchKernelGGL(check_finiteness_kernel<__half>, dim3(grid), dim3(256), 0, dh::stream(),
+                       static_cast<const __half*>(d_input), size, d_status, layer, step, abs_threshold);
+  else
+    hipLaunchKernelGGL(check_finiteness_kernel<float>, dim3(grid), dim3(256), 0, dh::stream(),
+                       static_cast<const float*>(d_input), size, d_status, layer, step, abs_threshold);
   DH_CHECK_LAUNCH(op);
   return 0;
 }

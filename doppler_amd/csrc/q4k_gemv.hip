@@ -933,7 +933,7 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
   if (M <= 0 || N <= 0 || K <= 0)
     return dh::fail(1, "[%s] Dimensions must be positive: M=%d, N=%d, K=%d", op, M, N, K);
   if (!d_A || !d_W || !d_C) return dh::fail(1, "[%s] null pointer", op);
-  if (a_dtype != DH_F32) return dh::fail(1, "[%s] activations must be f32 (a_dtype=%d)", op, a_dtype);
+  if (a_dtype != DH_F32) return dh::fail(1, "[%s] activations must be f32 or f16 (a_dtype=%d)", op, a_dtype);
   if (c_dtype != DH_F32 && c_dtype != DH_F16)
     return dh::fail(1, "[%s] output dtype must be f32 or f16 (c_dtype=%d)", op, c_dtype);
   if (reinterpret_cast<uintptr_t>(d_W) & 15)
@@ -1005,6 +1005,34 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
 
 int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int c_dtype, int M,
                   int N, int K, float alpha, const void* d_residual) {
+  if (a_dtype == DH_F16) {
+    // f16 activations: widened (exactly) into the library's f32 staging rows, as many rows per
+    // pass as the staging holds; the product accumulates in f32 like the f32-activation path
+    const char* op = "dh_q4k_matmul";
+    DH_REQUIRE_INIT(op);
+    if (M <= 0 || N <= 0 || K <= 0)
+      return dh::fail(1, "[%s] Dimensions must be positive: M=%d, N=%d, K=%d", op, M, N, K);
+    if (!d_A || !d_W || !d_C) return dh::fail(1, "[%s] null pointer", op);
+    if (c_dtype != DH_F32 && c_dtype != DH_F16)
+      return dh::fail(1, "[%s] output dtype must be f32 or f16 (c_dtype=%d)", op, c_dtype);
+    size_t bytes = 0;
+    float* wide = dh::widened_activations(&bytes);
+    int64_t rows_per_pass = (int64_t)(bytes / sizeof(float)) / K;
+    if (rows_per_pass >= 16) rows_per_pass &= ~(int64_t)15;
+    if (rows_per_pass < 1)
+      return dh::fail(1, "[%s] K=%d is too long for f16 activations (at most %zu)", op, K, bytes / sizeof(float));
+    const size_t c_elem = c_dtype == DH_F16 ? 2 : 4;
+    for (int64_t m0 = 0; m0 < M; m0 += rows_per_pass) {
+      const int rows = (int)std::min<int64_t>(rows_per_pass, M - m0);
+      int rc = dh_cast_f16_to_f32(static_cast<const uint16_t*>(d_A) + m0 * K, wide, (int64_t)rows * K);
+      if (rc) return rc;
+      rc = q4k_matmul_impl(op, wide, DH_F32, nullptr, 0.f, 0, false, d_W, static_cast<char*>(d_C) + m0 * N * c_elem,
+                           c_dtype, rows, N, K, alpha,
+                           d_residual ? static_cast<const float*>(d_residual) + m0 * N : nullptr);
+      if (rc) return rc;
+    }
+    return 0;
+  }
   return q4k_matmul_impl("dh_q4k_matmul", d_A, a_dtype, nullptr, 0.f, 0, false, d_W, d_C, c_dtype, M, N, K,
                          alpha, d_residual);
 }

@@ -34,15 +34,26 @@ def _dev_bytes(arr):
     return t
 
 
+class FinitenessError(RuntimeError):
+    """An activation left the f16 range (or the configured bound) during a decode step:
+    src/inference/pipelines/text/generator-steps.js:164-169."""
+
+
 class HipDecoder:
     TOKEN_RING = 64      # tokens one decode_batch submit can produce
 
     def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True,
-                 fuse_qkv_attention=True):
+                 fuse_qkv_attention=True, finiteness_guard=False, finiteness_abs_threshold=None):
         """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
         layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
-        input_norm, post_attn_norm, q_norm, k_norm: f32); embed_bits: uint16 [vocab, hidden]."""
+        input_norm, post_attn_norm, q_norm, k_norm: f32); embed_bits: uint16 [vocab, hidden].
+        finiteness_guard: check every layer's output against the overflow bound (one more launch
+        per layer) and read the 4-word status back beside the token, as the reference does when
+        activations are f16 (src/inference/pipelines/text/layer.js:1237-1252,
+        generator-steps.js:786-798, :837-843); off by default, the activations here are f32."""
         self.cfg = dict(cfg)
+        self.finiteness_guard = bool(finiteness_guard)
+        self.finiteness_abs_threshold = float(finiteness_abs_threshold) if finiteness_abs_threshold else 65500.0
         # RMSNorm runs inside the q/k/v and gate/up GEMVs (their prologue) unless told otherwise
         self.fuse_norm = fuse_norm
         self.L = capi.init(torch.cuda.current_device())
@@ -81,7 +92,10 @@ class HipDecoder:
         self.attn = f32(self.qs)
         self.act = f32(I)
         self.logits = f32(c["vocab"])
-        self.token = torch.zeros(self.TOKEN_RING, dtype=torch.int32, device="cuda")
+        # sampled tokens, then the finiteness status [status, layer, step, pad]: a single step
+        # with the guard on puts its token in the ring's last slot, so that one 20-byte read
+        # brings token and status back together
+        self.token = torch.zeros(self.TOKEN_RING + 4, dtype=torch.int32, device="cuda")
         self.ids = torch.zeros(4, dtype=torch.int32, device="cuda")
         self.attn_ws = torch.zeros(int(self.L.dh_attn_decode_workspace_bytes(H, D, max_seq)), dtype=torch.uint8,
                                    device="cuda")
@@ -117,7 +131,7 @@ class HipDecoder:
                            in_index if from_device_token else 0))
         self._out_index = out_index
         x, x2 = self.x, self.x2
-        for d in self.layers:
+        for li, d in enumerate(self.layers):
             if self.fuse_norm:
                 ck(L.dh_q4k_matmul_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), c["eps"], 0,
                                            d["wqkv"].data_ptr(), self.qkv.data_ptr(), capi.F32, 1,
@@ -141,6 +155,9 @@ class HipDecoder:
                                         self.act.data_ptr(), 1, Hd, I, capi.ACT_SILU, 1.0, 0.0))
             ck(L.dh_q4k_matmul(self.act.data_ptr(), capi.F32, d["wdown"].data_ptr(), x.data_ptr(), capi.F32, 1, Hd, I,
                                1.0, x2.data_ptr()))
+            if self.finiteness_guard:
+                ck(L.dh_check_finiteness(x.data_ptr(), capi.F32, Hd, self.token.data_ptr() + 4 * self.TOKEN_RING, li,
+                                         pos, self.finiteness_abs_threshold))
         ck(L.dh_rmsnorm(x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"],
                         0, None, None, None, 1.0))
         ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
@@ -175,15 +192,35 @@ class HipDecoder:
         capi.check(self.L.dh_download(self._host_token.ctypes.data, self.token.data_ptr(), 0, 4))
         return int(self._host_token[0])
 
+    def _reset_finiteness(self):
+        capi.check(self.L.dh_fill_zero(self.token.data_ptr(), 4 * self.TOKEN_RING, 16))
+
+    def _raise_if_triggered(self, words, offset, what):
+        from . import ops
+        st = ops.parseFinitenessStatusWords(words, offset)
+        if st["triggered"]:
+            raise FinitenessError("F16 bounds exceeded during %s%s" % (what, st["metadata"]))
+
     def step(self, token, pos, want_logits=False, sampling=None):
-        """One full step with the reference's single device->host crossing (the token id).
+        """One full step with the reference's single device->host crossing (the token id, with
+        the finiteness status beside it when the guard is on).
         sampling = dict(temperature, topK, randomSeed): top-k temperature sampling from the
         step's logits instead of the fused greedy argmax."""
         self.set_token(token)
-        self.enqueue_step(pos, want_logits or sampling is not None)
+        out_index = 0
+        if self.finiteness_guard:
+            self._reset_finiteness()
+            out_index = self.TOKEN_RING - 1
+        self.enqueue_step(pos, want_logits or sampling is not None, out_index=out_index)
         if sampling is not None:
-            self._enqueue_sample(sampling)
-        return self.read_token()
+            self._enqueue_sample(sampling, out_index)
+        if not self.finiteness_guard:
+            return self.read_token()
+        # staging layout of the reference: [token, status, layer, step, pad]
+        words = np.empty(5, np.uint32)
+        capi.check(self.L.dh_download(words.ctypes.data, self.token.data_ptr(), 4 * out_index, 20))
+        self._raise_if_triggered(words, 1, "generation")
+        return int(words[0])
 
     def capture_step(self, pos, want_logits=False):
         """Captures one decode step (enqueued for position `pos`) into a HIP graph, the
@@ -192,6 +229,9 @@ class HipDecoder:
         normally first so that every kernel's one-time set-up is done outside the capture."""
         if not self.fuse_qkv_attention:
             raise ValueError("capture_step serves the step with the fused attention kernel")
+        if self.finiteness_guard:
+            # the guard's step number is a launch argument: a replayed graph would report the capture's
+            raise ValueError("capture_step does not serve a decoder with the finiteness guard on")
         self.enqueue_step(pos, want_logits)
         capi.check(self.L.dh_sync())
         capi.check(self.L.dh_graph_begin())
@@ -332,8 +372,16 @@ class HipDecoder:
         if not 1 <= n <= self.TOKEN_RING:
             raise ValueError("decode_batch serves 1..%d tokens per submit, got %d" % (self.TOKEN_RING, n))
         self.set_token(token)
+        if self.finiteness_guard:
+            self._reset_finiteness()
         for i in range(n):
             self.enqueue_step(pos + i, from_device_token=i > 0, in_index=i - 1, out_index=i)
+        if self.finiteness_guard:
+            # ring and status in one read (src/inference/pipelines/text/generator-steps.js:1734-1740)
+            words = np.empty(self.TOKEN_RING + 4, np.uint32)
+            capi.check(self.L.dh_download(words.ctypes.data, self.token.data_ptr(), 0, words.nbytes))
+            self._raise_if_triggered(words, self.TOKEN_RING, "batch generation")
+            return [int(t) for t in words[:n]]
         out = np.empty(n, np.uint32)
         capi.check(self.L.dh_download(out.ctypes.data, self.token.data_ptr(), 0, 4 * n))
         return [int(t) for t in out]

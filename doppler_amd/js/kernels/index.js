@@ -23,3 +23,10 @@ export { runGather, recordGather } from './gather.js';
 export { runArgmax, recordArgmax, runGPUSample, recordGPUSample, seededRandom } from './sample.js';
 export { recordLmHeadArgmax, recordLmHeadArgmaxF16 } from './lm-head-argmax.js';
 export { castF32ToF16, castF16ToF32, recordCastF32ToF16, recordCastF16ToF32 } from './cast.js';
+export {
+  runMatmulRMSNormFused, recordMatmulRMSNormFused, shouldUseFusedMatmulRMSNorm, selectMatmulRMSNormFusedVariant,
+} from './fused_matmul_rmsnorm.js';
+export {
+  recordCheckFiniteness, createFinitenessStatusBuffer, parseFinitenessStatusWords, resolveFinitenessAbsThreshold,
+  shouldTriggerFinitenessValue, DEFAULT_FINITENESS_ABS_THRESHOLD, FINITENESS_STATUS_BYTES,
+} from './check-finiteness.js';

@@ -58,14 +58,19 @@ async function executeMatmul(recorder, A, B, M, N, K, options = {}) {
   }
   const outputDtype = requireOutputDtype(options.outputDtype, opLabel);
   validateOffsets(opLabel, aOffset, bOffset, cOffset);
-  if (A.dtype !== 'f32') {
-    throw new Error(`[${opLabel}] the HIP path takes f32 activations, got ${A.dtype}.`);
+  if (A.dtype !== 'f32' && A.dtype !== 'f16') {
+    throw new Error(`[${opLabel}] the HIP path takes f32 or f16 activations, got ${A.dtype}.`);
+  }
+  const fusedNorm = weightDtype === 'q4k' && options.normWeight != null && options.useFusedRmsnormWideTile === true;
+  if (A.dtype === 'f16' && (weightDtype !== 'q4k' || fusedNorm)) {
+    // reference: the f16-activation Q4_K kernels (fused_matmul_q4_f16a.wgsl and its batched forms)
+    throw new Error(`[${opLabel}] f16 activations are served for q4k weights without the fused RMSNorm only.`);
   }
   const aBuf = getBuffer(A);
   const bBuf = getBuffer(B);
-  const aRequired = aOffset + M * K * 4;
+  const aRequired = aOffset + M * K * (A.dtype === 'f16' ? 2 : 4);
   if (aBuf.size < aRequired) {
-    throw new Error(`[${opLabel}] A buffer too small: ${aBuf.size} < ${aRequired} (M=${M}, K=${K}, aDtype=f32)`);
+    throw new Error(`[${opLabel}] A buffer too small: ${aBuf.size} < ${aRequired} (M=${M}, K=${K}, aDtype=${A.dtype})`);
   }
   let bRequired;
   if (weightDtype === 'q4k') {
@@ -96,7 +101,7 @@ async function executeMatmul(recorder, A, B, M, N, K, options = {}) {
     const aPtr = aBuf.ptr + BigInt(aOffset);
     const bPtr = bBuf.ptr + BigInt(bOffset);
     const cPtr = output.ptr + BigInt(cOffset);
-    if (weightDtype === 'q4k' && options.normWeight != null && options.useFusedRmsnormWideTile === true) {
+    if (fusedNorm) {
       // RMSNorm of A inside the matmul (reference: matmul-selection.js:609-620)
       if (!Number.isFinite(options.rmsNormEps)) {
         throw new Error(`[${opLabel}] rmsNormEps is required with normWeight.`);
@@ -108,7 +113,7 @@ async function executeMatmul(recorder, A, B, M, N, K, options = {}) {
       native.q4kMatmulRmsnorm(aPtr, ptrOf(options.normWeight), options.rmsNormEps, options.rmsNormOffset === true ? 1 : 0,
         bPtr, cPtr, DTYPE[outputDtype], M, N, K, alpha, ptrOf(residualTensor));
     } else if (weightDtype === 'q4k') {
-      native.q4kMatmul(aPtr, DTYPE.f32, bPtr, cPtr, DTYPE[outputDtype], M, N, K, alpha, ptrOf(residualTensor));
+      native.q4kMatmul(aPtr, DTYPE[A.dtype], bPtr, cPtr, DTYPE[outputDtype], M, N, K, alpha, ptrOf(residualTensor));
     } else {
       if (outputDtype !== 'f32' || residualTensor) {
         throw new Error(`[${opLabel}] f16-weight matmul produces f32 without a fused residual on the HIP path.`);

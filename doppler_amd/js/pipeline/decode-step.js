@@ -8,12 +8,22 @@ import {
   createCommandRecorder, recordGather, recordRMSNorm, recordMatmul, recordSplitQKVRMSNormRoPEQK,
   recordAttention, recordFusedNormedFFN, recordFusedFFN, recordLmHeadArgmaxF16, recordGPUSample,
   recordDecodeAttentionFromQKV, decodeAttentionFromQKVSupported,
+  recordCheckFiniteness, parseFinitenessStatusWords, resolveFinitenessAbsThreshold, FINITENESS_STATUS_BYTES,
 } from '../kernel-selector.js';
 import { getNative } from '../native.js';
 
 // A window of a device buffer starting `offset` bytes in (no ownership: never released).
 function bufferWindow(buffer, offset, size) {
   return { ptr: buffer.ptr + BigInt(offset), size, capacity: size, label: buffer.label };
+}
+
+// An activation left the f16 range (or the configured bound) during a decode step
+// (reference: src/inference/pipelines/text/generator-steps.js:164-169).
+export class FinitenessError extends Error {
+  constructor(message) {
+    super(message);
+    this.name = 'FinitenessError';
+  }
 }
 
 function upload(bytes, label) {
@@ -24,6 +34,9 @@ function upload(bytes, label) {
 
 export class HipTextDecoder {
   // config: {layers, hidden, inter, heads, kvHeads, headDim, vocab, eps, maxSeq}
+  //   finitenessGuard (default false): check every layer's output against finitenessAbsThreshold
+  //   (one more launch per layer) and read the status words back beside the token, as the
+  //   reference does for f16 activations (layer.js:1237-1252, generator-steps.js:786-798, :837-843)
   // weights: {layers: [{wqkv, wo, wgate, wup, wdown (Uint8Array Q4_K), inputNorm, postAttnNorm,
   //           qNorm, kNorm (Float32Array)}], embed (Uint16Array f16 bits), finalNorm, cos, sin}
   constructor(config, weights) {
@@ -53,7 +66,11 @@ export class HipTextDecoder {
     this.fuseQkvAttention = config.fuseQkvAttention !== false &&
       decodeAttentionFromQKVSupported(c.heads, c.kvHeads, c.headDim, c.headDim, false);
     this.ids = acquireBuffer(16, undefined, 'token_ids');
-    this.tokenOut = acquireBuffer(16, undefined, 'sampled_token');
+    // [token, status, layer, step, pad]: the staging layout of the reference's guarded readback
+    this.tokenOut = acquireBuffer(4 + FINITENESS_STATUS_BYTES, undefined, 'sampled_token');
+    this.finitenessGuard = config.finitenessGuard === true;
+    this.finitenessAbsThreshold = resolveFinitenessAbsThreshold(config.finitenessAbsThreshold);
+    this.finitenessStatus = bufferWindow(this.tokenOut, 4, FINITENESS_STATUS_BYTES);
     this.logits = null;
   }
 
@@ -196,6 +213,9 @@ export class HipTextDecoder {
         { batchSize: 1, activation: 'silu' }));
       x = temp(await recordMatmul(recorder, act, l.wdown, 1, c.hidden, c.inter,
         { outputDtype: 'f32', role: 'down_proj', layerIdx: li, residualTensor: x2 }));
+      if (this.finitenessGuard) {
+        recordCheckFiniteness(recorder, x, c.hidden, this.finitenessStatus, li, pos, this.finitenessAbsThreshold);
+      }
     }
     if (options.sampling) {
       await this.recordHead(recorder, temps, x, options.sampling);
@@ -214,11 +234,18 @@ export class HipTextDecoder {
     const recorder = options.recorder || createCommandRecorder('decode');
     const temps = [];
     uploadData(this.ids, new Uint32Array([token]));
+    if (this.finitenessGuard) getNative().fillZero(this.tokenOut.ptr, 4, FINITENESS_STATUS_BYTES);
     await this.recordDecodeStep(recorder, temps, pos, options);
     for (const b of temps) recorder.trackTemporaryBuffer(b);
     recorder.submit();
-    const bytes = await readBufferSlice(this.tokenOut, 0, 4);   // the only device->host crossing
-    return new Uint32Array(bytes)[0];
+    // the only device->host crossing: the token, with the guard's status words beside it
+    const bytes = await readBufferSlice(this.tokenOut, 0, this.finitenessGuard ? 4 + FINITENESS_STATUS_BYTES : 4);
+    const words = new Uint32Array(bytes);
+    if (this.finitenessGuard) {
+      const status = parseFinitenessStatusWords(words, 1);
+      if (status.triggered) throw new FinitenessError(`F16 bounds exceeded during generation${status.metadata}`);
+    }
+    return words[0];
   }
 
   // Captures the decode step into a HIP graph, the counterpart of the reference's
@@ -227,6 +254,8 @@ export class HipTextDecoder {
   // uses stay allocated for the graph's life.
   async captureDecodeStep(token, pos) {
     if (!this.fuseQkvAttention) throw new Error('[captureDecodeStep] serves the fused-attention step');
+    // the guard's step number is a launch argument: a replayed graph would report the capture's
+    if (this.finitenessGuard) throw new Error('[captureDecodeStep] does not serve a decoder with the finiteness guard on');
     const first = await this.decodeStep(token, pos);
     getNative().graphBegin();
     let graph = null;

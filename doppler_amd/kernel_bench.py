@@ -1,6 +1,6 @@
 """Per-kernel measurements of the HIP path on the benchmark configurations.
 
-    python -m doppler_amd.kernel_bench [--only gemv,gemm,attn,prefill_attn,lmhead] [--json out.jsonl]
+    python -m doppler_amd.kernel_bench [--only gemv,gemm,attn,prefill_attn,lmhead,dense] [--json out.jsonl]
 
 Every case is timed with events around back-to-back launches on the library's stream.  Weights
 (and KV caches) rotate through enough copies that their total exceeds the 256 MB Infinity Cache
@@ -235,9 +235,46 @@ def sample_cases(L, T, rows, reps):
              achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
 
 
+def dense_cases(L, T, rows, reps):
+    """Dense f32 matmul + RMSNorm over the output row (one activation row), f16 activations into the
+    Q4_K matmul, and the finiteness check of one hidden row."""
+    for N, K in ((1152, 6912), (4096, 8192)):
+        copies = n_copies(N * K * 4, 16)
+        Ws = [torch.randn(N * K, device="cuda") * K ** -0.5 for _ in range(copies)]
+        x = torch.randn(K, device="cuda")
+        nw, res, out = torch.randn(N, device="cuda"), torch.randn(N, device="cuda"), torch.zeros(N, device="cuda")
+        algo = N * K * 4 + K * 4 + 3 * N * 4
+        for tb in (1, 0):
+            us = T.us(lambda i: capi.check(L.dh_matmul_rmsnorm_f32(x.data_ptr(), Ws[i % copies].data_ptr(), tb,
+                                                                   nw.data_ptr(), capi.F32, 1e-6, 1, res.data_ptr(),
+                                                                   out.data_ptr(), N, K)), max(8, reps // 4))
+            emit(rows, config=4, kernel="dense matmul+rmsnorm f32", shape="N=%d K=%d %s" % (N, K, "[N,K]" if tb else "[K,N]"),
+                 mode="rotating", us=round(us, 2), achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
+        del Ws
+    M, N, K = 4, 6144, 1536
+    nbytes = synth.q4k_nbytes(N, K)
+    copies = n_copies(nbytes)
+    Ws = q4k_copies(nbytes, copies)
+    a16 = torch.randn(M * K, device="cuda").half()
+    a32 = a16.float()
+    c = torch.zeros(M * N, dtype=torch.float16, device="cuda")
+    algo = nbytes + M * K * 2 + M * N * 2
+    for name, a, dt in (("q4k matmul f16 activations", a16, capi.F16), ("q4k matmul f32 activations", a32, capi.F32)):
+        us = T.us(lambda i: capi.check(L.dh_q4k_matmul(a.data_ptr(), dt, Ws[i % copies].data_ptr(), c.data_ptr(), capi.F16,
+                                                       M, N, K, 1.0, None)), reps)
+        emit(rows, config=1, kernel=name, shape="M=%d N=%d K=%d" % (M, N, K), mode="rotating", us=round(us, 2),
+             achieved=round((algo + (M * K * 2 if dt == capi.F32 else 0)) / us / 1e3, 1), unit="GB/s",
+             algorithmic_bytes=algo + (M * K * 2 if dt == capi.F32 else 0))
+    h = torch.randn(4096, device="cuda")
+    status = torch.zeros(4, dtype=torch.int32, device="cuda")
+    us = T.us(lambda i: capi.check(L.dh_check_finiteness(h.data_ptr(), capi.F32, 4096, status.data_ptr(), 0, i, 65500.0)), reps)
+    emit(rows, config=4, kernel="check_finiteness f32", shape="hidden=4096", mode="warm", us=round(us, 2),
+         achieved=round(4096 * 4 / us / 1e3, 1), unit="GB/s", algorithmic_bytes=4096 * 4)
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="gemv,gemm,attn,prefill_attn,lmhead")
+    ap.add_argument("--only", default="gemv,gemm,attn,prefill_attn,lmhead,dense")
     ap.add_argument("--reps", type=int, default=96)
     ap.add_argument("--json", default=None, help="also write one JSON object per case to this file")
     args = ap.parse_args(argv)
@@ -258,6 +295,8 @@ def main(argv=None):
     if "lmhead" in which:
         lmhead_cases(L, T, rows, args.reps)
         sample_cases(L, T, rows, args.reps)
+    if "dense" in which:
+        dense_cases(L, T, rows, args.reps)
     if args.json:
         with open(args.json, "w") as f:
             for r in rows:

@@ -155,10 +155,14 @@ def runMatmul(A, B, M, N, K, alpha=1.0, outputBuffer=None, transposeB=True, outp
     bdtype = B.dtype if isinstance(B, (Tensor, WeightBuffer)) else None
     if not bdtype:
         raise DopplerHipError("[%s] B dtype is required for matmul dispatch%s." % (op, " (role=%s)" % role if role else ""))
-    if A.dtype != "f32":
-        raise DopplerHipError("[%s] f32 activations required, got %s" % (op, A.dtype))
-    if _nbytes(A) < M * K * 4:
-        raise DopplerHipError("[%s] A buffer too small: %d < %d (M=%d, K=%d, aDtype=f32)" % (op, _nbytes(A), M * K * 4, M, K))
+    if A.dtype not in ("f32", "f16"):
+        raise DopplerHipError("[%s] f32 or f16 activations required, got %s" % (op, A.dtype))
+    a_elem = 2 if A.dtype == "f16" else 4
+    if _nbytes(A) < M * K * a_elem:
+        raise DopplerHipError("[%s] A buffer too small: %d < %d (M=%d, K=%d, aDtype=%s)"
+                              % (op, _nbytes(A), M * K * a_elem, M, K, A.dtype))
+    if A.dtype == "f16" and (bdtype != "q4k" or (normWeight is not None and useFusedRmsnormWideTile)):
+        raise DopplerHipError("[%s] f16 activations are served for q4k weights without the fused RMSNorm only" % op)
     L = _lib()
     if bdtype == "q4k":
         need = N * ((K + QK_K - 1) // QK_K) * Q4K_BLOCK_BYTES
@@ -176,8 +180,8 @@ def runMatmul(A, B, M, N, K, alpha=1.0, outputBuffer=None, transposeB=True, outp
                                                1 if rmsNormOffset else 0, _ptr(B), out.data_ptr(), cdt,
                                                M, N, K, alpha, _ptr(residualTensor)))
         else:
-            capi.check(L.dh_q4k_matmul(_ptr(A), capi.F32, _ptr(B), out.data_ptr(), cdt, M, N, K, alpha,
-                                       _ptr(residualTensor)))
+            capi.check(L.dh_q4k_matmul(_ptr(A), capi.F16 if A.dtype == "f16" else capi.F32, _ptr(B),
+                                       out.data_ptr(), cdt, M, N, K, alpha, _ptr(residualTensor)))
         return Tensor(out, outputDtype, (M, N), "matmul_output")
     if bdtype == "f16":
         if transposeB not in (True, "auto"):
@@ -191,6 +195,146 @@ def runMatmul(A, B, M, N, K, alpha=1.0, outputBuffer=None, transposeB=True, outp
         capi.check(L.dh_f16w_matmul(_ptr(A), _ptr(B), out.data_ptr(), M, N, K, alpha))
         return Tensor(out, "f32", (M, N), "matmul_output")
     raise DopplerHipError("[%s] weight dtype %r is not supported by the HIP path" % (op, bdtype))
+
+
+# Limits of the fused dense matmul + RMSNorm (src/config/schema/kernel-thresholds.schema.js:87-88).
+FUSED_MATMUL_MAX_MEDIUM_N = 4096
+FUSED_MATMUL_MAX_MEDIUM_K = 8192
+_WORKGROUP_SIZE_DEFAULT = 256
+
+
+def selectMatmulRMSNormFusedVariant(N, dtype):
+    """src/gpu/kernels/fused_matmul_rmsnorm.js:30-37 with the rule table of
+    src/rules/kernels/fused-matmul-rmsnorm.rules.json.  The name is informational here: one pair
+    of kernels serves every N."""
+    if not dtype:
+        raise DopplerHipError("[MatmulRMSNormFused] dtype is required for variant selection.")
+    small = N <= _WORKGROUP_SIZE_DEFAULT
+    f16 = dtype == "f16"
+    return ("small" if small else "medium") + ("_f16" if f16 else "")
+
+
+def shouldUseFusedMatmulRMSNorm(M, N, K=None):
+    """src/gpu/kernels/fused_matmul_rmsnorm.js:295-312."""
+    if M != 1 or N > FUSED_MATMUL_MAX_MEDIUM_N:
+        return False
+    if isinstance(K, (int, float, np.integer)) and not isinstance(K, bool) and K > FUSED_MATMUL_MAX_MEDIUM_K:
+        return False
+    return True
+
+
+def runMatmulRMSNormFused(input, weight, normWeight, options=None, **kw):
+    """src/gpu/kernels/fused_matmul_rmsnorm.js:50 runMatmulRMSNormFused(input, weight, normWeight,
+    {N, K, eps, residual, outputBuffer, transposeB, rmsNormWeightOffset, label}): one f32
+    activation row through a dense f32 weight ([N, K] with transposeB, else [K, N]), RMSNorm over
+    the N outputs, residual added after the norm."""
+    o = dict(options or {})
+    o.update(kw)
+    if o.get("transposeB") is None:
+        raise DopplerHipError("[MatmulRMSNormFused] transposeB is required.")
+    if o.get("rmsNormWeightOffset") is None:
+        raise DopplerHipError("[MatmulRMSNormFused] rmsNormWeightOffset is required.")
+    if o.get("eps") is None:
+        raise DopplerHipError("[MatmulRMSNormFused] eps is required.")
+    N, K = o.get("N"), o.get("K")
+    for v in (N, K):
+        if not isinstance(v, (int, np.integer)) or v <= 0:
+            raise DopplerHipError("[MatmulRMSNormFused] N and K must be positive integers: N=%s, K=%s" % (N, K))
+    if N > FUSED_MATMUL_MAX_MEDIUM_N:
+        raise DopplerHipError("[MatmulRMSNormFused] N=%d exceeds maxMediumN=%d; kernel only supports "
+                              "single-workgroup RMSNorm." % (N, FUSED_MATMUL_MAX_MEDIUM_N))
+    if not getattr(input, "dtype", None):
+        raise DopplerHipError("[MatmulRMSNormFused] input dtype is required.")
+    selectMatmulRMSNormFusedVariant(N, input.dtype)
+    if input.dtype != "f32":
+        raise DopplerHipError("[MatmulRMSNormFused] f32 activations required, got %s" % input.dtype)
+    wdtype = weight.dtype if isinstance(weight, (Tensor, WeightBuffer)) else "f32"
+    if wdtype != "f32":
+        raise DopplerHipError("[MatmulRMSNormFused] dense f32 weights required, got %s" % wdtype)
+    if _nbytes(input) < K * 4 or _nbytes(weight) < N * K * 4:
+        raise DopplerHipError("[MatmulRMSNormFused] input or weight buffer too small for N=%d, K=%d" % (N, K))
+    # the reference tells an f16 norm weight from an f32 one by the buffer's size (:14-28)
+    nw_bytes = _nbytes(normWeight)
+    if nw_bytes >= N * 4:
+        nw = capi.F32
+    elif nw_bytes >= N * 2:
+        nw = capi.F16
+    else:
+        raise DopplerHipError("[MatmulRMSNormFused] norm weight size (%d bytes) does not match hiddenSize=%d "
+                              "(expected %d or %d bytes)." % (nw_bytes, N, N * 2, N * 4))
+    residual = o.get("residual")
+    if residual is not None and _nbytes(residual) < N * 4:
+        raise DopplerHipError("[MatmulRMSNormFused] residual buffer smaller than N=%d floats" % N)
+    out = _out(o.get("outputBuffer"), N * 4)
+    capi.check(_lib().dh_matmul_rmsnorm_f32(_ptr(input), _ptr(weight), 1 if o["transposeB"] else 0, _ptr(normWeight),
+                                            nw, float(o["eps"]), 1 if o["rmsNormWeightOffset"] else 0,
+                                            _ptr(residual), out.data_ptr(), int(N), int(K)))
+    return Tensor(out, "f32", (1, N), "matmul_rmsnorm_fused_output")
+
+
+def recordMatmulRMSNormFused(recorder, input, weight, normWeight, options=None, **kw):
+    """src/gpu/kernels/fused_matmul_rmsnorm.js:173 recordMatmulRMSNormFused.  `recorder` is accepted
+    for signature parity: every op already enqueues in order on one stream."""
+    return runMatmulRMSNormFused(input, weight, normWeight, options, **kw)
+
+
+# ------------------------------------------------------------------ finiteness guard
+
+DEFAULT_FINITENESS_ABS_THRESHOLD = 65500
+FINITENESS_STATUS_BYTES = 16
+
+
+def resolveFinitenessAbsThreshold(value):
+    """src/gpu/kernels/check-finiteness.js:7-12."""
+    if isinstance(value, (int, float, np.integer, np.floating)) and not isinstance(value, bool) \
+            and math.isfinite(value) and value > 0:
+        return value
+    return DEFAULT_FINITENESS_ABS_THRESHOLD
+
+
+def shouldTriggerFinitenessValue(value, absThreshold=DEFAULT_FINITENESS_ABS_THRESHOLD):
+    """src/gpu/kernels/check-finiteness.js:14-19."""
+    if not math.isfinite(value):
+        return True
+    return abs(value) > resolveFinitenessAbsThreshold(absThreshold)
+
+
+def parseFinitenessStatusWords(words, offset=0):
+    """src/inference/pipelines/text/finiteness-guard-status.js:1-21."""
+    status = int(words[offset]) if offset < len(words) else 0
+    if status <= 0:
+        return {"triggered": False, "layer": 0, "step": 0, "metadata": ""}
+    layer = int(words[offset + 1]) if offset + 1 < len(words) else 0
+    step = int(words[offset + 2]) if offset + 2 < len(words) else 0
+    return {"triggered": True, "layer": layer, "step": step, "metadata": " (layer %d, step %d)" % (layer, step)}
+
+
+def createFinitenessStatusBuffer():
+    """Four zeroed u32 words: [status, layer, step, pad], the layout the reference copies beside
+    the sampled token (src/inference/pipelines/text/generator-steps.js:786-798)."""
+    buf = acquireBuffer(FINITENESS_STATUS_BYTES)
+    buf.zero_()
+    return buf
+
+
+def recordCheckFiniteness(target, inputBuffer, size, statusBuffer, layerIdx=0, step=0,
+                          absThreshold=DEFAULT_FINITENESS_ABS_THRESHOLD, inputDtype=None):
+    """src/gpu/kernels/check-finiteness.js:98 recordCheckFiniteness(target, inputBuffer, size,
+    statusBuffer, layerIdx, step, absThreshold).  The reference's shader reads f16; here the
+    element type is the tensor's (or `inputDtype` for a bare buffer, default f16 as there)."""
+    dtype = inputDtype or getattr(inputBuffer, "dtype", None)
+    if not isinstance(dtype, str):
+        dtype = "f16"
+    if dtype not in ("f16", "f32"):
+        raise DopplerHipError("[check_finiteness] input dtype must be f16 or f32, got %s" % dtype)
+    elem = 2 if dtype == "f16" else 4
+    if _nbytes(inputBuffer) < size * elem:
+        raise DopplerHipError("[check_finiteness] input buffer smaller than size=%d" % size)
+    if _nbytes(statusBuffer) < FINITENESS_STATUS_BYTES:
+        raise DopplerHipError("[check_finiteness] status buffer must hold 4 u32 words")
+    capi.check(_lib().dh_check_finiteness(_ptr(inputBuffer), capi.F16 if dtype == "f16" else capi.F32, int(size),
+                                          _ptr(statusBuffer), int(layerIdx), int(step),
+                                          float(resolveFinitenessAbsThreshold(absThreshold))))
 
 
 def runDequantQ4K(W, numBlocks, outputBuffer=None):

@@ -95,8 +95,11 @@ int dh_q4k_dequant(const void* d_W, int64_t num_blocks, float* d_out);
 /* C[M,N] = alpha * A[M,K] . dequant(W)[N,K]^T (+ residual[M,N]).
  * Replaces runMatmul/recordMatmul for Q4_K weights, src/gpu/kernels/matmul.js:659-666
  * (kernels fused_matmul_q4.wgsl:122-258, fused_matmul_q4_batched.wgsl:123-194,
- * fused_matmul_q4_prefill_tiled_f16.wgsl:119-261).  A is f32 (a_dtype DH_F32); C is f32 or
- * f16 (c_dtype).  K need not be a multiple of 256: the padded tail of each row's last
+ * fused_matmul_q4_prefill_tiled_f16.wgsl:119-261; f16 activations: fused_matmul_q4_f16a.wgsl,
+ * fused_matmul_q4_batched_f16a.wgsl, selected at matmul-selection.js:24-27).  A is f32 or f16
+ * (a_dtype); f16 rows are widened exactly into a 64 MB f32 staging area of the library, in
+ * passes when they do not fit, and the product accumulates in f32 either way.  C is f32 or
+ * f16 (c_dtype); the residual is f32.  K need not be a multiple of 256: the padded tail of each row's last
  * block is ignored.  d_residual (may be NULL) is added after alpha, as the reference's
  * `residualTensor` option does.  M = 1..8 takes the HBM-bound GEMV path, larger M the
  * MFMA GEMM path (from 16 rows on a weight tensor must be smaller than 2 GB, as the kernel
@@ -323,6 +326,28 @@ int dh_sample_topk(const float* d_logits, int vocab, double temperature, int top
 /* f32 <-> f16 casts.  Replaces castF32ToF16/castF16ToF32, src/gpu/kernels/cast.js:98-116. */
 int dh_cast_f32_to_f16(const float* d_in, void* d_out, int64_t n);
 int dh_cast_f16_to_f32(const void* d_in, float* d_out, int64_t n);
+
+/* out[n] = y[n] / sqrt(mean(y^2 over N) + eps) * (w[n] | 1 + w[n]) (+ residual[n]) with
+ * y = x[1,K] . W, W dense f32 laid out [N,K] (transpose_b != 0) or [K,N].  Replaces
+ * runMatmulRMSNormFused/recordMatmulRMSNormFused, src/gpu/kernels/fused_matmul_rmsnorm.js:50-170
+ * and :173-296 (fused_matmul_rmsnorm.wgsl:166-213, :215-272): one activation row, N <= 4096
+ * (the reference's maxMediumN; larger N fails with its message), norm weight f32 or f16, the
+ * residual added after the norm.  Uses the library's split-K workspace: two or three launches
+ * on the library's stream, the product over the whole chip in K slices, the sum of the slices
+ * when there are many, and the row's norm in one workgroup. */
+int dh_matmul_rmsnorm_f32(const float* d_x, const float* d_W, int transpose_b,
+                          const void* d_norm_weight, int norm_weight_dtype, float eps,
+                          int weight_offset, const float* d_residual, float* d_out, int N, int K);
+
+/* Overflow guard for activations: the first element of d_input (f32 or f16) that is NaN,
+ * infinite or larger in magnitude than abs_threshold (<= 0 or not finite: 65500) turns
+ * d_status[0] from 0 to 1, and the launch that does so writes layer to d_status[1] and step to
+ * d_status[2]; a status that is already 1 is left alone.  d_status is 4 u32 words the caller
+ * zeroes before a step and reads back beside the token.  Replaces recordCheckFiniteness,
+ * src/gpu/kernels/check-finiteness.js:98-150 (shader :25-62); read back as the reference does at
+ * src/inference/pipelines/text/generator-steps.js:786-798. */
+int dh_check_finiteness(const void* d_input, int dtype, int64_t size, uint32_t* d_status,
+                        uint32_t layer, uint32_t step, float abs_threshold);
 
 #ifdef __cplusplus
 }

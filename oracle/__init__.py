@@ -369,6 +369,62 @@ def seeded_random(seed):
     return float(lib().dor_seeded_random(float(seed)))
 
 
+# --------------------------------------------------------------------------- dense matmul + RMSNorm
+
+def matmul_rmsnorm_fused(x, W, norm_weight, N, K, eps, transpose_b=True, weight_offset=False, residual=None):
+    """src/gpu/kernels/fused_matmul_rmsnorm.wgsl:215-272 (gemv_rmsnorm_medium; :166-213 is the same
+    arithmetic for N <= 256): y[n] = sum_k x[k] * W(n, k) with W stored [N, K] (transpose_b) or
+    [K, N]; out[n] = y[n] / sqrt(sum(y^2) / N + eps) * (w[n] | 1 + w[n]) + residual[n].  Sums run
+    in float64 and each stage is rounded to f32 where the shader stores one."""
+    x = _c(x, np.float32).reshape(K).astype(np.float64)
+    W = _c(W, np.float32).reshape((N, K) if transpose_b else (K, N)).astype(np.float64)
+    y = ((W @ x) if transpose_b else (x @ W)).astype(np.float32).astype(np.float64)
+    inv_rms = 1.0 / np.sqrt(np.sum(y * y) / N + float(eps))
+    w = _c(norm_weight, np.float32).reshape(N).astype(np.float64)
+    if weight_offset:
+        w = 1.0 + w
+    out = y * inv_rms * w
+    if residual is not None:
+        out = out.astype(np.float32).astype(np.float64) + _c(residual, np.float32).reshape(N)
+    return out.astype(np.float32)
+
+
+# --------------------------------------------------------------------------- finiteness guard
+
+def finiteness_should_trigger(value, abs_threshold=65500):
+    """src/gpu/kernels/check-finiteness.js:7-19: a threshold that is not a positive finite number
+    falls back to 65500; NaN and +-inf always trigger."""
+    thr = abs_threshold if (abs_threshold is not None and np.isfinite(abs_threshold) and abs_threshold > 0) else 65500
+    v = float(value)
+    return (not np.isfinite(v)) or abs(v) > thr
+
+
+def check_finiteness(values, status, layer=0, step=0, abs_threshold=65500):
+    """src/gpu/kernels/check-finiteness.js:25-62: `status` is 4 u32 words, updated in place; the
+    first triggering call turns word 0 from 0 to 1 and records its layer and step in words 1
+    and 2, later calls leave a set status alone.  The f32 compare is the shader's: the value
+    (f16 widened, or f32) against the threshold rounded to f32."""
+    v = np.asarray(values)
+    assert v.dtype in (np.float16, np.float32)
+    v = v.astype(np.float32).ravel()
+    thr = np.float32(abs_threshold if (np.isfinite(abs_threshold) and abs_threshold > 0) else 65500)
+    bits = v.view(np.uint32)
+    bad = ((bits & 0x7F800000) == 0x7F800000) | (np.abs(v) > thr)
+    if bad.any() and status[0] == 0:
+        status[0], status[1], status[2] = 1, layer, step
+    return status
+
+
+def finiteness_parse_status(words, offset=0):
+    """src/inference/pipelines/text/finiteness-guard-status.js:1-21."""
+    words = list(words)
+    get = lambda i: int(words[i]) if i < len(words) else 0
+    if get(offset) <= 0:
+        return {"triggered": False, "layer": 0, "step": 0, "metadata": ""}
+    layer, step = get(offset + 1), get(offset + 2)
+    return {"triggered": True, "layer": layer, "step": step, "metadata": " (layer %d, step %d)" % (layer, step)}
+
+
 # --------------------------------------------------------------------------- decode step
 
 class DecoderOracle:

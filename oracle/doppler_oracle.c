@@ -33,6 +33,11 @@
  *   attention             torch scaled_dot_product_attention (f64, repeated KV heads);
  *                         kvLen==1 => O==V; uniform scores => mean of V
  *   argmax                brute force incl. ties -> lowest index, pad excluded
+ *   (numpy, oracle/__init__.py)
+ *   matmul + rmsnorm      torch float64 matmul and rms_norm; unit weight and identity matrix
+ *                         give x / rms(x); both weight layouts agree on W and W^T
+ *   finiteness guard      the reference's own vectors (finiteness-overflow-gate.test.js,
+ *                         finiteness-guard-status.test.js); first trigger wins
  *
  * Build: see oracle/Makefile (gcc -O2 -fopenmp -shared).
  */

@@ -47,7 +47,7 @@ async function main() {
       await save(out, t.buffer, c.blocks * 256 * 4);
     } else if (c.op === 'matmul') {
       const W = dh.createWeightBuffer(dev(c.W), c.wdtype, 'row', [c.N, c.K], c.name);
-      const A = tensor(c.A, 'f32', [c.M, c.K]);
+      const A = tensor(c.A, c.aDtype || 'f32', [c.M, c.K]);
       const opts = { outputDtype: c.outputDtype, alpha: c.alpha, role: 'test' };
       if (c.residual) opts.residualTensor = tensor(c.residual, 'f32', [c.M, c.N]);
       if (c.normWeight) {
@@ -203,6 +203,12 @@ async function main() {
           tok = await dec.decodeStep(inp, pos, { recorder: rec });
           results.profile = await rec.resolveProfileTimings();
           results.profileOps = rec.opCount;
+        } else if (c.expectFinitenessAt === pos) {
+          // the guard's bound is set below this model's activations: the step must throw and name layer and step
+          let message = 'did not throw';
+          try { await dec.decodeStep(inp, pos); } catch (e) { message = `${e.name}: ${e.message}`; }
+          results.errors.push({ label: `${c.name}-guard`, ok: message === `FinitenessError: F16 bounds exceeded during generation (layer 0, step ${pos})`, message });
+          break;
         } else {
           tok = await dec.decodeStep(inp, pos);
         }
@@ -230,6 +236,26 @@ async function main() {
         tokens.push(tok);
       }
       fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
+    } else if (c.op === 'matmul_rmsnorm_fused') {
+      const opts = { N: c.N, K: c.K, eps: c.eps, transposeB: c.transposeB, rmsNormWeightOffset: c.weightOffset,
+        residual: c.residual ? tensor(c.residual, 'f32', [1, c.N]) : null, label: 'test' };
+      const x = tensor(c.x, 'f32', [1, c.K]);
+      const W = dh.createWeightBuffer(dev(c.W), 'f32', 'row', c.transposeB ? [c.N, c.K] : [c.K, c.N], c.name);
+      const nw = dev(c.normWeight);
+      if (!dh.shouldUseFusedMatmulRMSNorm(1, c.N, c.K)) throw new Error('shouldUseFusedMatmulRMSNorm said no');
+      const rec = c.record ? dh.createCommandRecorder('t') : null;
+      const t = rec ? await dh.recordMatmulRMSNormFused(rec, x, W, nw, opts) : await dh.runMatmulRMSNormFused(x, W, nw, opts);
+      if (rec) await rec.submitAndWait();
+      await save(out, t.buffer, c.N * 4);
+    } else if (c.op === 'check_finiteness') {
+      // one status buffer across the listed checks, in order: [input file, dtype, size, layer, step, threshold]
+      const status = dh.createFinitenessStatusBuffer();
+      const words = [];
+      for (const k of c.checks) {
+        dh.recordCheckFiniteness(null, tensor(k.input, k.dtype, [k.size]), k.size, status, k.layer, k.step, k.threshold === null ? undefined : k.threshold);
+        words.push(...new Uint32Array(await dh.readBuffer(status, 16)));
+      }
+      fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(words).buffer));
     } else {
       throw new Error(`unknown case op ${c.op}`);
     }
@@ -256,6 +282,21 @@ async function main() {
       shards: [{ filename: 'shard_00000.bin', size: 1024 }], tensors: { w: { offset: 0, size: 4, shape: [1], dtype: 'F32' } } })));
     await expectThrow(results, 'rdrr-size', 'should hold 144 bytes', async () => parseManifest(JSON.stringify({
       shards: [{ filename: 'shard_00000.bin', size: 1024 }], tensors: { w: { shard: 0, offset: 0, size: 100, shape: [1, 256], dtype: 'Q4_K_M' } } })));
+    await expectThrow(results, 'fused-mr-tb', 'transposeB is required', () => dh.runMatmulRMSNormFused(A, A, A, { N: 4, K: 8, eps: 1e-6, rmsNormWeightOffset: false }));
+    await expectThrow(results, 'fused-mr-n', 'exceeds maxMediumN=4096', () => dh.runMatmulRMSNormFused(A, A, A, { N: 4097, K: 8, eps: 1e-6, transposeB: true, rmsNormWeightOffset: false }));
+    await expectThrow(results, 'fused-mr-nw', 'does not match hiddenSize=1024', () => dh.runMatmulRMSNormFused(A, A, A, { N: 1024, K: 8, eps: 1e-6, transposeB: true, rmsNormWeightOffset: false }));
+    await expectThrow(results, 'f16a-norm', 'f16 activations are served', () => dh.runMatmul(dh.createTensor(A.buffer, 'f16', [1, 256]), W, 1, 8, 256, { outputDtype: 'f32', normWeight: A, rmsNormEps: 1e-6, useFusedRmsnormWideTile: true }));
+    await expectThrow(results, 'finite-status', 'status buffer must hold', () => dh.recordCheckFiniteness(null, A, 4, dh.acquireBuffer(8)));
+    if (dh.selectMatmulRMSNormFusedVariant(256, 'f32') !== 'small' || dh.selectMatmulRMSNormFusedVariant(1152, 'f16') !== 'medium_f16' ||
+        dh.shouldUseFusedMatmulRMSNorm(2, 8, 8) || dh.shouldUseFusedMatmulRMSNorm(1, 8, 8193) || !dh.shouldUseFusedMatmulRMSNorm(1, 4096, 8192) ||
+        dh.resolveFinitenessAbsThreshold(-1) !== 65500 || dh.resolveFinitenessAbsThreshold(50000) !== 50000 ||
+        dh.shouldTriggerFinitenessValue(100) || !dh.shouldTriggerFinitenessValue(65501, 65500) || !dh.shouldTriggerFinitenessValue(NaN, 65500) ||
+        dh.parseFinitenessStatusWords(new Uint32Array([42, 1, 3, 15, 0]), 1).metadata !== ' (layer 3, step 15)' ||
+        dh.parseFinitenessStatusWords(new Uint32Array([0, 7, 9]), 0).triggered) {
+      results.errors.push({ label: 'host-helpers', ok: false, message: 'a selection or finiteness helper disagrees with the reference tests' });
+    } else {
+      results.errors.push({ label: 'host-helpers', ok: true, message: '' });
+    }
     await expectThrow(results, 'ffn', 'matching gate/up dtypes', () => dh.runFusedFFN(A, W, dh.createWeightBuffer(W.buffer, 'f16', 'row', [8, 256]), 256, 8, {}));
   }
 

@@ -46,3 +46,38 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".js", ".mjs", ".hip", ".h", ".c")):
                 src = open(os.path.join(dirpath, f), errors="replace").read()
                 assert "import oracle" not in src and "from oracle" not in src and "doppler_oracle" not in src, f
+
+
+def test_finiteness_host_helpers_follow_the_reference_tests():
+    from doppler_amd import ops
+    # tests/inference/finiteness-overflow-gate.test.js
+    assert ops.resolveFinitenessAbsThreshold(None) == ops.DEFAULT_FINITENESS_ABS_THRESHOLD == 65500
+    assert ops.resolveFinitenessAbsThreshold(50000) == 50000
+    assert ops.resolveFinitenessAbsThreshold(-1) == 65500
+    assert ops.shouldTriggerFinitenessValue(100) is False
+    assert ops.shouldTriggerFinitenessValue(65501, 65500) is True
+    assert ops.shouldTriggerFinitenessValue(-70000, 65500) is True
+    for v in (float("inf"), float("-inf"), float("nan")):
+        assert ops.shouldTriggerFinitenessValue(v, 65500) is True
+    # tests/inference/finiteness-guard-status.test.js
+    assert ops.parseFinitenessStatusWords([0, 7, 9], 0) == {"triggered": False, "layer": 0, "step": 0, "metadata": ""}
+    assert ops.parseFinitenessStatusWords([1, 8, 12], 0) == {"triggered": True, "layer": 8, "step": 12,
+                                                             "metadata": " (layer 8, step 12)"}
+    assert ops.parseFinitenessStatusWords([42, 1, 3, 15, 0], 1)["metadata"] == " (layer 3, step 15)"
+
+
+def test_fused_matmul_rmsnorm_selection_follows_the_reference_rules():
+    from doppler_amd import ops
+    # src/rules/kernels/fused-matmul-rmsnorm.rules.json; small means N <= 256
+    assert ops.selectMatmulRMSNormFusedVariant(256, "f32") == "small"
+    assert ops.selectMatmulRMSNormFusedVariant(256, "f16") == "small_f16"
+    assert ops.selectMatmulRMSNormFusedVariant(257, "f32") == "medium"
+    assert ops.selectMatmulRMSNormFusedVariant(1152, "f16") == "medium_f16"
+    with pytest.raises(capi.DopplerHipError, match="dtype is required"):
+        ops.selectMatmulRMSNormFusedVariant(8, None)
+    # src/gpu/kernels/fused_matmul_rmsnorm.js:295-312
+    assert ops.shouldUseFusedMatmulRMSNorm(1, 4096, 8192) is True
+    assert ops.shouldUseFusedMatmulRMSNorm(2, 1152, 6912) is False
+    assert ops.shouldUseFusedMatmulRMSNorm(1, 4097, 1024) is False
+    assert ops.shouldUseFusedMatmulRMSNorm(1, 1152, 8193) is False
+    assert ops.shouldUseFusedMatmulRMSNorm(1, 1152) is True

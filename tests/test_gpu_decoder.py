@@ -304,3 +304,57 @@ def test_graph_replayed_steps_give_the_oracle_tokens(cfg):
         assert g == ctok, (pos, g, ctok)
         tok = g
     gpu.release_graph()
+
+
+def test_finiteness_guard_reads_status_beside_the_token():
+    """Guard on: the same tokens while nothing crosses the bound (single steps, sampled steps and the
+    batched ring); with the bound set inside the model's activation range the step raises and names
+    the first layer whose output crossed it, as the reference's guarded readback does
+    (src/inference/pipelines/text/generator-steps.js:786-798, :837-843).  The random-weight model's
+    residual stream is far outside the f16 range (1e6 and more), so the cases that must not trip
+    raise the bound and the default bound of 65500 trips at layer 0."""
+    cfg = dict(layers=3, hidden=256, inter=512, heads=4, kv_heads=2, head_dim=64, vocab=300, eps=1e-6, qk_norm=1,
+               max_seq=32, theta=1e6)
+    layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=61, max_seq=32)
+    plain = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32)
+    guarded = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32, finiteness_guard=True,
+                                 finiteness_abs_threshold=1e30)
+    prompt = [5, 17, 250, 3]
+    want = plain.generate(prompt, 12)
+    assert guarded.generate(prompt, 12) == want
+    samp = dict(temperature=0.8, topK=16, seed=9)
+    assert decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32, finiteness_guard=True,
+                              finiteness_abs_threshold=1e30).generate(prompt, 8, sampling=samp) == \
+        decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32).generate(prompt, 8, sampling=samp)
+    b_plain = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32)
+    b_guard = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32, finiteness_guard=True,
+                                 finiteness_abs_threshold=1e30)
+    t0 = b_plain.prefill(prompt)
+    assert b_guard.prefill(prompt) == t0
+    assert b_guard.decode_batch(t0, len(prompt), 9) == b_plain.decode_batch(t0, len(prompt), 9)
+    with pytest.raises(ValueError, match="finiteness guard"):
+        guarded.capture_step(20)
+    # the residual stream after each layer, from the unguarded decoder's buffers: pick a bound between
+    # layer 0's and layer 2's peak so that the layer the guard names is known
+    probe = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32)
+    probe.prefill(prompt)
+    peaks = []
+    for n_layers in (1, 2, 3):
+        sub = decoder.HipDecoder(dict(cfg, layers=n_layers), layers[:n_layers], embed, final_norm, cos, sin, 32)
+        sub.prefill(prompt)
+        sub.step(t0, len(prompt))
+        peaks.append(float(np.abs(sub.x.cpu().numpy()).max()))
+    first_over = next(i for i, p in enumerate(peaks) if p == max(peaks))
+    bound = (max(peaks) + max([p for p in peaks[:first_over]] + [0.0])) / 2
+    trip = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32, finiteness_guard=True,
+                              finiteness_abs_threshold=bound)
+    trip.prefill(prompt)
+    with pytest.raises(decoder.FinitenessError, match=r"F16 bounds exceeded during generation \(layer %d, step %d\)"
+                       % (first_over, len(prompt))):
+        trip.step(t0, len(prompt))
+    with pytest.raises(decoder.FinitenessError, match=r"during batch generation \(layer %d, step %d\)" % (first_over, len(prompt))):
+        trip.decode_batch(t0, len(prompt), 4)
+    default = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32, finiteness_guard=True)
+    default.prefill(prompt)
+    with pytest.raises(decoder.FinitenessError, match=r"\(layer 0, step %d\)" % len(prompt)):
+        default.step(t0, len(prompt))

@@ -86,6 +86,46 @@ def _matmul_case(M, N, K, seed, alpha=1.0, outputDtype="f32", residual=False):
     return rel_l2(got, want)
 
 
+@pytest.mark.parametrize("M,N,K,outputDtype,residual", [
+    (4, 6144, 1536, "f16", False),      # the shape of the reference's f16-activation parity test
+    (1, 1024, 4096, "f16", False), (1, 4096, 4096, "f32", True), (8, 512, 1152, "f32", False),
+    (12, 96, 300, "f16", True), (33, 257, 2048, "f32", True)])
+def test_matmul_f16_activations(M, N, K, outputDtype, residual):
+    """f16 activations (tests/kernels/fused-matmul-q4-widetile-f16a-parity.test.js runs M=4, K=1536,
+    N=6144): the product of the exactly widened rows, accumulated in f32."""
+    W, wb = q4k_weight(N, K, 1150 + M)
+    A16 = synth.normal_f32((M, K), 1151 + M).astype(np.float16)
+    a = ops.tensorFromNumpy(A16.view(np.uint16))
+    assert a.dtype == "f16"
+    res = synth.normal_f32((M, N), 1152 + M) if residual else None
+    out = ops.runMatmul(a, wb, M, N, K, outputDtype=outputDtype, role="test",
+                        residualTensor=ops.tensorFromNumpy(res) if residual else None)
+    got = ops.readTensor(out)
+    if outputDtype == "f16":
+        got = got.view(np.float16).astype(np.float32)
+    want = oracle.q4k_matmul(A16.astype(np.float32), W, M, N, K)
+    if residual:
+        want = want + res
+    assert rel_l2(got, want) <= matmul_bar(M) + (5e-4 if outputDtype == "f16" else 0)
+    # same rows handed over as f32 take the same kernels: identical bits
+    same = ops.readTensor(ops.runMatmul(ops.tensorFromNumpy(A16.astype(np.float32)), wb, M, N, K, outputDtype=outputDtype,
+                                        role="test", residualTensor=ops.tensorFromNumpy(res) if residual else None))
+    assert same.tobytes() == ops.readTensor(out).tobytes()
+
+
+def test_matmul_f16_activations_errors():
+    W, wb = q4k_weight(8, 256, 1160)
+    a = ops.tensorFromNumpy(np.zeros((1, 256), np.float16).view(np.uint16))
+    with pytest.raises(DopplerHipError, match="A buffer too small"):
+        ops.runMatmul(a, wb, 2, 8, 256, outputDtype="f32")
+    nw = ops.tensorFromNumpy(np.ones(256, np.float32))
+    with pytest.raises(DopplerHipError, match="f16 activations"):
+        ops.runMatmul(a, wb, 1, 8, 256, outputDtype="f32", normWeight=nw, rmsNormEps=1e-6, useFusedRmsnormWideTile=True)
+    with pytest.raises(DopplerHipError, match="activations must be f32 or f16|a_dtype"):
+        capi.check(capi.init(0).dh_q4k_matmul(a.buffer.data_ptr(), 7, wb.buffer.data_ptr(), a.buffer.data_ptr(), capi.F32,
+                                              1, 8, 256, 1.0, None))
+
+
 def test_matmul_cfg0_gemv():
     assert _matmul_case(1, synth.CFG0["N"], synth.CFG0["K"], seed=1100) <= REL_L2_F32
 
@@ -928,3 +968,101 @@ def test_attention_prefill_options_and_errors():
     with pytest.raises(DopplerHipError, match="contiguous cache"):
         ops.runAttention(qt, kt, vt, None, H, D, seqLen=T, kvLen=kv_len, numKVHeads=Hkv, startPos=start, kvLayout="ring",
                          slidingWindow=64)
+
+
+# ----------------------------------------------------------------------------- dense matmul + RMSNorm
+
+@pytest.mark.parametrize("N,K,transposeB,offset,residual,w16", [
+    (1152, 6912, True, True, True, False),      # Gemma-3 1B down projection + post-FFN norm
+    (1152, 6912, False, True, True, False),
+    (4096, 8192, True, False, False, False),    # the largest shape the reference routes here
+    (4096, 8192, False, False, True, True),
+    (256, 1000, True, False, False, True), (7, 13, False, True, True, False), (1, 5, True, False, False, False),
+    (1001, 301, False, False, True, True), (1001, 301, True, True, False, False)])
+def test_matmul_rmsnorm_fused(N, K, transposeB, offset, residual, w16):
+    g = synth.rng(7000 + N + K)
+    x = g.standard_normal(K).astype(np.float32)
+    W = (g.standard_normal((N, K)) * K ** -0.5).astype(np.float32)
+    w = g.standard_normal(N).astype(np.float32)
+    if w16:
+        w = w.astype(np.float16).astype(np.float32)
+    r = g.standard_normal(N).astype(np.float32) if residual else None
+    stored = W if transposeB else np.ascontiguousarray(W.T)
+    nw = ops.tensorFromNumpy(w.astype(np.float16).view(np.uint16)) if w16 else ops.tensorFromNumpy(w)
+    assert ops.shouldUseFusedMatmulRMSNorm(1, N, K)
+    out = ops.runMatmulRMSNormFused(ops.tensorFromNumpy(x), ops.tensorFromNumpy(stored), nw,
+                                    {"N": N, "K": K, "eps": 1e-6, "transposeB": transposeB, "rmsNormWeightOffset": offset,
+                                     "residual": ops.tensorFromNumpy(r) if residual else None})
+    assert out.shape == (1, N) and out.dtype == "f32"
+    want = oracle.matmul_rmsnorm_fused(x, stored, w, N, K, 1e-6, transpose_b=transposeB, weight_offset=offset, residual=r)
+    assert rel_l2(ops.readTensor(out), want) <= 1e-5
+    # equals the unfused pair of ops of this library to rounding
+    if transposeB and not w16:
+        a = ops.readTensor(out)
+        again = ops.readTensor(ops.recordMatmulRMSNormFused(None, ops.tensorFromNumpy(x), ops.tensorFromNumpy(stored), nw,
+                                                            N=N, K=K, eps=1e-6, transposeB=True, rmsNormWeightOffset=offset,
+                                                            residual=ops.tensorFromNumpy(r) if residual else None))
+        assert a.tobytes() == again.tobytes()       # run to run deterministic
+
+
+def test_matmul_rmsnorm_fused_errors_and_selection():
+    x = ops.tensorFromNumpy(np.zeros(8, np.float32))
+    W = ops.tensorFromNumpy(np.zeros((4, 8), np.float32))
+    nw = ops.tensorFromNumpy(np.ones(4, np.float32))
+    with pytest.raises(DopplerHipError, match="transposeB is required"):
+        ops.runMatmulRMSNormFused(x, W, nw, {"N": 4, "K": 8, "eps": 1e-6, "rmsNormWeightOffset": False})
+    with pytest.raises(DopplerHipError, match="rmsNormWeightOffset is required"):
+        ops.runMatmulRMSNormFused(x, W, nw, {"N": 4, "K": 8, "eps": 1e-6, "transposeB": True})
+    with pytest.raises(DopplerHipError, match="eps is required"):
+        ops.runMatmulRMSNormFused(x, W, nw, {"N": 4, "K": 8, "transposeB": True, "rmsNormWeightOffset": False})
+    with pytest.raises(DopplerHipError, match="exceeds maxMediumN=4096"):
+        ops.runMatmulRMSNormFused(x, W, nw, {"N": 4097, "K": 8, "eps": 1e-6, "transposeB": True, "rmsNormWeightOffset": False})
+    with pytest.raises(DopplerHipError, match="does not match hiddenSize=4"):
+        ops.runMatmulRMSNormFused(x, W, ops.tensorFromNumpy(np.ones(1, np.float32)),
+                                  {"N": 4, "K": 8, "eps": 1e-6, "transposeB": True, "rmsNormWeightOffset": False})
+    with pytest.raises(DopplerHipError, match="exceeds maxMediumN"):
+        capi.check(capi.init(0).dh_matmul_rmsnorm_f32(x.buffer.data_ptr(), W.buffer.data_ptr(), 1, nw.buffer.data_ptr(),
+                                                      capi.F32, 1e-6, 0, None, x.buffer.data_ptr(), 5000, 8))
+
+
+# ----------------------------------------------------------------------------- finiteness guard
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_check_finiteness_status_word(dtype):
+    npdt = np.float16 if dtype == "f16" else np.float32
+    n = 200_003
+    clean = (synth.normal_f32((n,), 7100) * 100).astype(npdt)
+    clean[5] = 65500 if dtype == "f32" else 65472      # at the threshold is not beyond it
+    up = lambda a: ops.tensorFromNumpy(a.view(np.uint16) if dtype == "f16" else a)
+    status = ops.createFinitenessStatusBuffer()
+    want = np.zeros(4, np.uint32)
+    ops.recordCheckFiniteness(None, up(clean), n, status, 3, 9)
+    oracle.check_finiteness(clean, want, 3, 9)
+    assert ops.readBuffer(status, 16, np.uint32).tolist() == want.tolist() == [0, 0, 0, 0]
+    # one bad element anywhere, of every kind, in the last position too
+    bads = [np.inf, -np.inf, np.nan, 65504.0, -65504.0] + ([1e30, 65500.01] if dtype == "f32" else [])
+    for i, bad in enumerate(bads):
+        dirty = clean.copy()
+        dirty[n - 1 if i % 2 else (i * 7919) % n] = bad
+        st = ops.createFinitenessStatusBuffer()
+        ops.recordCheckFiniteness(None, up(dirty), n, st, 10 + i, 20 + i)
+        want = oracle.check_finiteness(dirty, np.zeros(4, np.uint32), 10 + i, 20 + i)
+        assert want[0] == 1
+        assert ops.readBuffer(st, 16, np.uint32).tolist() == want.tolist(), bad
+        # a set status keeps its first layer and step
+        ops.recordCheckFiniteness(None, up(dirty), n, st, 99, 98)
+        assert ops.readBuffer(st, 16, np.uint32).tolist() == want.tolist()
+        assert ops.parseFinitenessStatusWords(ops.readBuffer(st, 16, np.uint32)) == \
+            oracle.finiteness_parse_status(want)
+    # the element past `size` is not looked at; a custom threshold; a bad threshold falls back to 65500
+    dirty = clean.copy()
+    dirty[1000] = np.inf
+    st = ops.createFinitenessStatusBuffer()
+    ops.recordCheckFiniteness(None, up(dirty), 1000, st, 1, 1)
+    assert ops.readBuffer(st, 16, np.uint32).tolist() == [0, 0, 0, 0]
+    ops.recordCheckFiniteness(None, up(clean), n, st, 4, 5, absThreshold=50.0)
+    assert ops.readBuffer(st, 16, np.uint32).tolist() == oracle.check_finiteness(clean, np.zeros(4, np.uint32), 4, 5, 50.0).tolist()
+    st = ops.createFinitenessStatusBuffer()
+    ops.recordCheckFiniteness(None, up(clean), n, st, 4, 5, absThreshold=-1)
+    assert ops.readBuffer(st, 16, np.uint32).tolist() == [0, 0, 0, 0]
+    ops.recordCheckFiniteness(None, up(clean), 0, st, 4, 5)

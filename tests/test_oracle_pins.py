@@ -585,3 +585,76 @@ def test_decode_step_wiring_matches_op_by_op():
         assert np.array_equal(logits, want)
         assert got_tok == int(np.argmax(want))
         tok = got_tok
+
+
+# ----------------------------------------------------------------------------- dense matmul + RMSNorm
+
+def test_matmul_rmsnorm_fused_matches_torch_f64_and_closed_forms():
+    g = np.random.default_rng(31)
+    for N, K, tb, off, res in [(7, 13, True, False, False), (256, 96, False, True, True),
+                               (1152, 300, True, True, True), (300, 1152, False, False, False)]:
+        x = g.standard_normal(K).astype(np.float32)
+        W = (g.standard_normal((N, K)) * 0.1).astype(np.float32)
+        w = g.standard_normal(N).astype(np.float32)
+        r = g.standard_normal(N).astype(np.float32) if res else None
+        stored = W if tb else np.ascontiguousarray(W.T)
+        got = oracle.matmul_rmsnorm_fused(x, stored, w, N, K, 1e-5, transpose_b=tb, weight_offset=off, residual=r)
+        y = torch.from_numpy(W).double() @ torch.from_numpy(x).double()
+        wt = torch.from_numpy(w).double() + (1.0 if off else 0.0)
+        want = torch.nn.functional.rms_norm(y, (N,), wt, 1e-5)
+        if res:
+            want = want + torch.from_numpy(r).double()
+        assert np.allclose(got, want.numpy(), rtol=2e-6, atol=2e-6), (N, K, tb, off, res)
+    # identity matrix, unit weight, eps 0: x / rms(x), whose squares average to one; a dropped
+    # 1/N or a norm over K instead of N fails here
+    N = 64
+    x = g.standard_normal(N).astype(np.float32)
+    out = oracle.matmul_rmsnorm_fused(x, np.eye(N, dtype=np.float32), np.ones(N, np.float32), N, N, 0.0)
+    assert np.allclose(out, x / np.sqrt(np.mean(x.astype(np.float64) ** 2)), rtol=1e-6)
+    assert abs(np.mean(out.astype(np.float64) ** 2) - 1.0) < 1e-6
+    # the residual comes after the norm: it shifts the output by exactly itself
+    r = g.standard_normal(N).astype(np.float32)
+    shifted = oracle.matmul_rmsnorm_fused(x, np.eye(N, dtype=np.float32), np.ones(N, np.float32), N, N, 0.0, residual=r)
+    assert np.allclose(shifted - out, r, atol=1e-6)
+    # a non-square one-hot matrix tells [N, K] from [K, N]
+    W = np.zeros((3, 5), np.float32)
+    W[2, 4] = 2.0
+    x = np.arange(1, 6, dtype=np.float32)
+    a = oracle.matmul_rmsnorm_fused(x, W, np.ones(3, np.float32), 3, 5, 0.0, transpose_b=True)
+    b = oracle.matmul_rmsnorm_fused(x, np.ascontiguousarray(W.T), np.ones(3, np.float32), 3, 5, 0.0, transpose_b=False)
+    assert np.allclose(a, [0, 0, math.sqrt(3.0)]) and np.allclose(b, a)
+
+
+# ----------------------------------------------------------------------------- finiteness guard
+
+def test_finiteness_guard_matches_the_reference_tests_vectors():
+    # tests/inference/finiteness-overflow-gate.test.js
+    assert oracle.finiteness_should_trigger(100) is False
+    assert oracle.finiteness_should_trigger(65501, 65500) is True
+    assert oracle.finiteness_should_trigger(-70000, 65500) is True
+    for v in (float("inf"), float("-inf"), float("nan")):
+        assert oracle.finiteness_should_trigger(v, 65500) is True
+    assert oracle.finiteness_should_trigger(60000, -1) is False      # bad threshold -> 65500
+    assert oracle.finiteness_should_trigger(60000, 50000) is True
+    # tests/inference/finiteness-guard-status.test.js
+    s = oracle.finiteness_parse_status(np.array([0, 7, 9], np.uint32), 0)
+    assert s == {"triggered": False, "layer": 0, "step": 0, "metadata": ""}
+    s = oracle.finiteness_parse_status(np.array([1, 8, 12], np.uint32), 0)
+    assert s == {"triggered": True, "layer": 8, "step": 12, "metadata": " (layer 8, step 12)"}
+    s = oracle.finiteness_parse_status(np.array([42, 1, 3, 15, 0], np.uint32), 1)
+    assert s == {"triggered": True, "layer": 3, "step": 15, "metadata": " (layer 3, step 15)"}
+    # the status word: clean input leaves it alone, the first trigger wins, later ones do not overwrite
+    st = np.zeros(4, np.uint32)
+    oracle.check_finiteness(np.array([1.0, -65500.0, 65500.0], np.float32), st, 3, 4)
+    assert st.tolist() == [0, 0, 0, 0]
+    oracle.check_finiteness(np.array([1.0, 65504.0], np.float16), st, 5, 6)
+    assert st.tolist() == [1, 5, 6, 0]
+    oracle.check_finiteness(np.array([np.nan], np.float32), st, 7, 8)
+    assert st.tolist() == [1, 5, 6, 0]
+    for bad in (np.inf, -np.inf, np.nan, 1e5, -1e5):
+        st = np.zeros(4, np.uint32)
+        oracle.check_finiteness(np.array([0.0, bad], np.float32), st, 1, 2)
+        assert st.tolist() == [1, 1, 2, 0], bad
+    st = np.zeros(4, np.uint32)
+    oracle.check_finiteness(np.array([70000.0], np.float32), st, 1, 2, abs_threshold=1e6)
+    assert st.tolist() == [0, 0, 0, 0]
