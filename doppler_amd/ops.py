@@ -3,7 +3,8 @@
 Names, argument meaning and error behaviour follow the reference's JavaScript wrappers
 (src/gpu/kernels/index.js): `runMatmul`, `runAttention`, `runRMSNorm`, `runRoPE`,
 `runKVCacheWriteF32ToF16`, `runSplitQKVRMSNormRoPEQK`, `runSiLU`, `runSiLURowSplit`, `runGeLU`,
-`runResidualAdd`, `runBiasAdd`, `runScale`, `runSplitQKV`, `runRoPEQK`, `runGather`, `runFusedFFN`, `runArgmax`, `recordLmHeadArgmaxF16`, plus the
+`runResidualAdd`, `runBiasAdd`, `runScale`, `runSplitQKV`, `runRoPEQK`, `runGather`, `runFusedFFN`, `runArgmax`,
+`recordLmHeadArgmaxF16`, `runMatmulRMSNormFused`, `recordCheckFiniteness`, plus the
 handle helpers `createTensor` / `createWeightBuffer` and the pool calls `acquireBuffer` /
 `uploadData` / `readBuffer`.  Options are keyword arguments with the reference's camelCase
 names.  Every op goes through the C ABI of libdopplerhip.so; torch only provides device
