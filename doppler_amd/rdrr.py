@@ -312,10 +312,11 @@ def load_model_arrays(art):
     return cfg, layers, embed, final_norm
 
 
-def load_decoder(directory, max_seq, **decoder_kwargs):
-    """Open an RDRR directory and return a ready HipDecoder (weights resident in HBM)."""
+def load_decoder(directory, max_seq, verify_hashes=True, **decoder_kwargs):
+    """Open an RDRR directory and return a ready HipDecoder (weights resident in HBM).
+    `verify_hashes` as in Artifact."""
     from . import decoder
-    art = Artifact(directory)
+    art = Artifact(directory, verify_hashes=verify_hashes)
     try:
         cfg, layers, embed, final_norm = load_model_arrays(art)
         cos, sin = synth.rope_tables(cfg["head_dim"], max_seq, cfg["theta"])
