@@ -86,6 +86,7 @@ SIGNATURES = {
     "dh_cast_f32_to_f16": (_I, [_P, _P, _I64]),
     "dh_cast_f16_to_f32": (_I, [_P, _P, _I64]),
     "dh_matmul_rmsnorm_f32": (_I, [_P, _P, _I, _P, _I, _F, _I, _P, _P, _I, _I]),
+    "dh_matmul_rmsnorm_f16": (_I, [_P, _P, _I, _P, _I, _F, _I, _P, _P, _I, _I]),
     "dh_check_finiteness": (_I, [_P, _I, _I64, _P, ctypes.c_uint32, ctypes.c_uint32, _F]),
 }
 

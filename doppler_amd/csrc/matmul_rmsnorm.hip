@@ -15,41 +15,81 @@ namespace {
 constexpr int kFinishThreads = 1024;
 constexpr int kMaxN = 4096;   // the reference's maxMediumN (src/config/schema/kernel-thresholds.schema.js:87)
 
+// Element types of activations, weights, residual and output: f32, or f16 widened on load and
+// rounded once on the final store (all sums run in f32 either way).
+template <typename T> struct Vec16;   // a 16-byte piece
+template <> struct Vec16<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  }
+};
+template <> struct Vec16<__half> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void load(const __half* p, float (&v)[8]) {
+    const uint4 t = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[2 * i] = __half2float(__ushort_as_half((unsigned short)(w[i] & 0xffffu)));
+      v[2 * i + 1] = __half2float(__ushort_as_half((unsigned short)(w[i] >> 16)));
+    }
+  }
+};
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(__half v) { return __half2float(v); }
+// four consecutive elements
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) { Vec16<float>::load(p, v); }
+__device__ __forceinline__ void load4(const __half* p, float (&v)[4]) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  v[0] = __half2float(__ushort_as_half((unsigned short)(t.x & 0xffffu)));
+  v[1] = __half2float(__ushort_as_half((unsigned short)(t.x >> 16)));
+  v[2] = __half2float(__ushort_as_half((unsigned short)(t.y & 0xffffu)));
+  v[3] = __half2float(__ushort_as_half((unsigned short)(t.y >> 16)));
+}
+
 // W is [N, K]: a wave per output row and K slice, lanes stride over the slice in 16-byte pieces,
 // four loads in flight per lane.  parts[slice][n] receives the wave's sum.
-__global__ __launch_bounds__(256) void gemv_rows_kernel(const float* __restrict__ x, const float* __restrict__ W,
+template <typename T>
+__global__ __launch_bounds__(256) void gemv_rows_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                         float* __restrict__ parts, int N, int K, int k_per_slice,
                                                         int vec) {
+  constexpr int V = Vec16<T>::N;
   const int lane = threadIdx.x & 63;
   const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (n >= N) return;
   const int k0 = blockIdx.y * k_per_slice;
   const int k1 = min(K, k0 + k_per_slice);
-  const float* row = W + (int64_t)n * K;
+  const T* row = W + (int64_t)n * K;
   float acc = 0.f;
   if (vec) {
-    // k_per_slice is a multiple of 4 here, so is K
-    const float4* row4 = reinterpret_cast<const float4*>(row);
-    const float4* x4 = reinterpret_cast<const float4*>(x);
-    const int q1 = k1 >> 2;
-    int k = (k0 >> 2) + lane;
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    for (; k + 192 < q1; k += 256) {
-      const float4 w0 = row4[k], w1 = row4[k + 64], w2 = row4[k + 128], w3 = row4[k + 192];
-      const float4 v0 = x4[k], v1 = x4[k + 64], v2 = x4[k + 128], v3 = x4[k + 192];
-      a0 += w0.x * v0.x + w0.y * v0.y + w0.z * v0.z + w0.w * v0.w;
-      a1 += w1.x * v1.x + w1.y * v1.y + w1.z * v1.z + w1.w * v1.w;
-      a2 += w2.x * v2.x + w2.y * v2.y + w2.z * v2.z + w2.w * v2.w;
-      a3 += w3.x * v3.x + w3.y * v3.y + w3.z * v3.z + w3.w * v3.w;
+    // k_per_slice and K are multiples of V here; pieces q0 .. q1 - 1 of the row
+    const int q1 = k1 / V;
+    int q = k0 / V + lane;
+    float a[4] = {0.f, 0.f, 0.f, 0.f};
+    for (; q + 192 < q1; q += 256) {
+      float w[4][V], v[4][V];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        Vec16<T>::load(row + (int64_t)(q + 64 * u) * V, w[u]);
+        Vec16<T>::load(x + (int64_t)(q + 64 * u) * V, v[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int e = 0; e < V; e++) a[u] = fmaf(w[u][e], v[u][e], a[u]);
     }
-    for (; k < q1; k += 64) {
-      const float4 w = row4[k];
-      const float4 v = x4[k];
-      a0 += w.x * v.x + w.y * v.y + w.z * v.z + w.w * v.w;
+    for (; q < q1; q += 64) {
+      float w[V], v[V];
+      Vec16<T>::load(row + (int64_t)q * V, w);
+      Vec16<T>::load(x + (int64_t)q * V, v);
+#pragma unroll
+      for (int e = 0; e < V; e++) a[0] = fmaf(w[e], v[e], a[0]);
     }
-    acc = (a0 + a1) + (a2 + a3);
+    acc = (a[0] + a[1]) + (a[2] + a[3]);
   } else {
-    for (int k = k0 + lane; k < k1; k += 64) acc += row[k] * x[k];
+    for (int k = k0 + lane; k < k1; k += 64) acc = fmaf(to_f32(row[k]), to_f32(x[k]), acc);
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
@@ -60,8 +100,8 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(const float* __restrict_
 // wave w takes rows w, w + 16, ... of the slice, four rows in flight, and the waves meet in LDS in
 // wave order.  parts[slice][n] receives the sum.
 constexpr int kColsWaves = 16;
-__global__ __launch_bounds__(kColsWaves * 64) void gemv_cols_kernel(const float* __restrict__ x,
-                                                                    const float* __restrict__ W,
+template <typename T>
+__global__ __launch_bounds__(kColsWaves * 64) void gemv_cols_kernel(const T* __restrict__ x, const T* __restrict__ W,
                                                                     float* __restrict__ parts, int N, int K,
                                                                     int k_per_slice, int vec) {
   __shared__ float red[kColsWaves][64][4];
@@ -73,34 +113,36 @@ __global__ __launch_bounds__(kColsWaves * 64) void gemv_cols_kernel(const float*
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
   if (vec) {
     if (n0 < N) {
-      const float* col = W + n0;
+      const T* col = W + n0;
       int k = k0 + wave;
       for (; k + 3 * kColsWaves < k1; k += 4 * kColsWaves) {
-        float4 w[4];
+        float w[4][4];
         float v[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-          w[u] = *reinterpret_cast<const float4*>(col + (int64_t)(k + u * kColsWaves) * N);
-          v[u] = x[k + u * kColsWaves];
+          load4(col + (int64_t)(k + u * kColsWaves) * N, w[u]);
+          v[u] = to_f32(x[k + u * kColsWaves]);
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-          acc[0] += w[u].x * v[u]; acc[1] += w[u].y * v[u]; acc[2] += w[u].z * v[u]; acc[3] += w[u].w * v[u];
-        }
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) acc[j] = fmaf(w[u][j], v[u], acc[j]);
       }
       for (; k < k1; k += kColsWaves) {
-        const float4 w = *reinterpret_cast<const float4*>(col + (int64_t)k * N);
-        const float v = x[k];
-        acc[0] += w.x * v; acc[1] += w.y * v; acc[2] += w.z * v; acc[3] += w.w * v;
+        float w[4];
+        load4(col + (int64_t)k * N, w);
+        const float v = to_f32(x[k]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] = fmaf(w[j], v, acc[j]);
       }
     }
   } else {
     for (int k = k0 + wave; k < k1; k += kColsWaves) {
-      const float v = x[k];
-      const float* row = W + (int64_t)k * N;
+      const float v = to_f32(x[k]);
+      const T* row = W + (int64_t)k * N;
 #pragma unroll
       for (int j = 0; j < 4; j++)
-        if (n0 + j < N) acc[j] += row[n0 + j] * v;
+        if (n0 + j < N) acc[j] = fmaf(to_f32(row[n0 + j]), v, acc[j]);
     }
   }
 #pragma unroll
@@ -133,11 +175,12 @@ __global__ __launch_bounds__(256) void slices_sum_kernel(const float* __restrict
 }
 
 // One workgroup: y[n] = sum over slices (in slice order), mean of squares, scale, weight, residual.
+template <typename T>
 __global__ __launch_bounds__(kFinishThreads) void rmsnorm_finish_kernel(const float* __restrict__ parts, int slices,
                                                                         const void* __restrict__ norm_weight,
                                                                         int weight_f16, int weight_offset,
-                                                                        const float* __restrict__ residual,
-                                                                        float* __restrict__ out, int N, float eps) {
+                                                                        const T* __restrict__ residual,
+                                                                        T* __restrict__ out, int N, float eps) {
   __shared__ float red[kFinishThreads / 64];
   float y[kMaxN / kFinishThreads];
   float ssq = 0.f;
@@ -166,18 +209,16 @@ __global__ __launch_bounds__(kFinishThreads) void rmsnorm_finish_kernel(const fl
                          : static_cast<const float*>(norm_weight)[n];
     if (weight_offset) w += 1.0f;
     float r = y[c] * inv_rms * w;
-    if (residual) r += residual[n];
-    out[n] = r;
+    if (residual) r += to_f32(residual[n]);
+    out[n] = static_cast<T>(r);
   }
 }
 
-}  // namespace
-
-extern "C" int dh_matmul_rmsnorm_f32(const float* d_x, const float* d_W, int transpose_b, const void* d_norm_weight,
-                                     int norm_weight_dtype, float eps, int weight_offset, const float* d_residual,
-                                     float* d_out, int N, int K) {
-  const char* op = "dh_matmul_rmsnorm_f32";
+template <typename T>
+int matmul_rmsnorm_impl(const char* op, const T* d_x, const T* d_W, int transpose_b, const void* d_norm_weight,
+                        int norm_weight_dtype, float eps, int weight_offset, const T* d_residual, T* d_out, int N, int K) {
   DH_REQUIRE_INIT(op);
+  constexpr int V = Vec16<T>::N;
   if (N <= 0 || K <= 0) return dh::fail(1, "[%s] Dimensions must be positive: N=%d, K=%d", op, N, K);
   if (N > kMaxN)
     return dh::fail(1, "[%s] N=%d exceeds maxMediumN=%d; the RMSNorm over the output row is one workgroup", op, N, kMaxN);
@@ -188,14 +229,14 @@ extern "C" int dh_matmul_rmsnorm_f32(const float* d_x, const float* d_W, int tra
   float* parts = dh::splitk_workspace(&ws_bytes);
   int slices = 1;
   if (transpose_b) {
-    const int vec = (K % 4 == 0) && ((reinterpret_cast<uintptr_t>(d_W) | reinterpret_cast<uintptr_t>(d_x)) % 16 == 0);
-    // about 16 waves per compute unit, at least 1024 elements of a row per wave
-    slices = std::max(1, std::min<int>((int)(K / 1024), (int)dh::ceil_div(16 * dh::num_cus(), N)));
-    const int k_per_slice = (int)dh::ceil_div(dh::ceil_div(K, slices), 4) * 4;
+    const int vec = (K % V == 0) && ((reinterpret_cast<uintptr_t>(d_W) | reinterpret_cast<uintptr_t>(d_x)) % 16 == 0);
+    // about 16 waves per compute unit, at least 256 16-byte pieces of a row per wave
+    slices = std::max(1, std::min<int>((int)(K / (256 * V)), (int)dh::ceil_div(16 * dh::num_cus(), N)));
+    const int k_per_slice = (int)dh::ceil_div(dh::ceil_div(K, slices), V) * V;
     slices = (int)dh::ceil_div(K, k_per_slice);
     if ((size_t)(slices + 1) * N * sizeof(float) > ws_bytes)
       return dh::fail(2, "[%s] internal: %d slices of %d floats do not fit the workspace", op, slices, N);
-    hipLaunchKernelGGL(gemv_rows_kernel, dim3((unsigned)dh::ceil_div(N, 4), slices), dim3(256), 0, dh::stream(), d_x,
+    hipLaunchKernelGGL(gemv_rows_kernel<T>, dim3((unsigned)dh::ceil_div(N, 4), slices), dim3(256), 0, dh::stream(), d_x,
                        d_W, parts, N, K, k_per_slice, vec);
   } else {
     const int col_blocks = (int)dh::ceil_div(N, 256);
@@ -205,8 +246,8 @@ extern "C" int dh_matmul_rmsnorm_f32(const float* d_x, const float* d_W, int tra
     slices = (int)dh::ceil_div(K, k_per_slice);
     if ((size_t)(slices + 1) * N * sizeof(float) > ws_bytes)
       return dh::fail(2, "[%s] internal: %d slices of %d floats do not fit the workspace", op, slices, N);
-    const int vec = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(d_W) % 16 == 0);
-    hipLaunchKernelGGL(gemv_cols_kernel, dim3(col_blocks, slices), dim3(kColsWaves * 64), 0, dh::stream(), d_x, d_W,
+    const int vec = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(d_W) % (4 * sizeof(T)) == 0);
+    hipLaunchKernelGGL(gemv_cols_kernel<T>, dim3(col_blocks, slices), dim3(kColsWaves * 64), 0, dh::stream(), d_x, d_W,
                        parts, N, K, k_per_slice, vec);
   }
   DH_CHECK_LAUNCH(op);
@@ -218,8 +259,25 @@ extern "C" int dh_matmul_rmsnorm_f32(const float* d_x, const float* d_W, int tra
     parts = y;
     slices = 1;
   }
-  hipLaunchKernelGGL(rmsnorm_finish_kernel, dim3(1), dim3(kFinishThreads), 0, dh::stream(), parts, slices,
+  hipLaunchKernelGGL(rmsnorm_finish_kernel<T>, dim3(1), dim3(kFinishThreads), 0, dh::stream(), parts, slices,
                      d_norm_weight, norm_weight_dtype == DH_F16, weight_offset, d_residual, d_out, N, eps);
   DH_CHECK_LAUNCH(op);
   return 0;
+}
+
+}  // namespace
+
+extern "C" int dh_matmul_rmsnorm_f32(const float* d_x, const float* d_W, int transpose_b, const void* d_norm_weight,
+                                     int norm_weight_dtype, float eps, int weight_offset, const float* d_residual,
+                                     float* d_out, int N, int K) {
+  return matmul_rmsnorm_impl<float>("dh_matmul_rmsnorm_f32", d_x, d_W, transpose_b, d_norm_weight, norm_weight_dtype, eps,
+                                    weight_offset, d_residual, d_out, N, K);
+}
+
+extern "C" int dh_matmul_rmsnorm_f16(const void* d_x, const void* d_W, int transpose_b, const void* d_norm_weight,
+                                     int norm_weight_dtype, float eps, int weight_offset, const void* d_residual,
+                                     void* d_out, int N, int K) {
+  return matmul_rmsnorm_impl<__half>("dh_matmul_rmsnorm_f16", static_cast<const __half*>(d_x),
+                                     static_cast<const __half*>(d_W), transpose_b, d_norm_weight, norm_weight_dtype, eps,
+                                     weight_offset, static_cast<const __half*>(d_residual), static_cast<__half*>(d_out), N, K);
 }

@@ -297,6 +297,10 @@ FN(js_matmul_rmsnorm_f32) {
   return ret_rc(env, dh_matmul_rmsnorm_f32((const float*)x, (const float*)W, tb, nw, nwdt, eps, off, (const float*)res,
                                            (float*)out, N, K));
 }
+FN(js_matmul_rmsnorm_f16) {
+  ARGS(11); P(0, x); P(1, W); I(2, tb); P(3, nw); I(4, nwdt); F(5, eps); I(6, off); P(7, res); P(8, out); I(9, N); I(10, K);
+  return ret_rc(env, dh_matmul_rmsnorm_f16(x, W, tb, nw, nwdt, eps, off, res, out, N, K));
+}
 FN(js_check_finiteness) {
   ARGS(7); P(0, in); I(1, dt); L(2, n); P(3, st); I(4, layer); I(5, step); F(6, thr);
   return ret_rc(env, dh_check_finiteness(in, dt, n, (uint32_t*)st, (uint32_t)layer, (uint32_t)step, thr));
@@ -324,7 +328,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"argmaxWorkspaceBytes", js_argmax_workspace_bytes}, {"argmax", js_argmax},
       {"sampleTopkWorkspaceBytes", js_sample_topk_workspace_bytes}, {"sampleTopk", js_sample_topk},
       {"castF32ToF16", js_cast_f32_to_f16}, {"castF16ToF32", js_cast_f16_to_f32},
-      {"matmulRmsnormF32", js_matmul_rmsnorm_f32}, {"checkFiniteness", js_check_finiteness},
+      {"matmulRmsnormF32", js_matmul_rmsnorm_f32}, {"matmulRmsnormF16", js_matmul_rmsnorm_f16}, {"checkFiniteness", js_check_finiteness},
   };
   for (size_t i = 0; i < sizeof(table) / sizeof(table[0]); i++) {
     napi_value fn;

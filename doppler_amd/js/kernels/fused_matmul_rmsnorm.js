@@ -1,7 +1,7 @@
 // runMatmulRMSNormFused / recordMatmulRMSNormFused / shouldUseFusedMatmulRMSNorm /
 // selectMatmulRMSNormFusedVariant: reference src/gpu/kernels/fused_matmul_rmsnorm.js:30-312.
-// One f32 activation row through a dense f32 weight, RMSNorm over the N outputs, the residual
-// added after the norm.
+// One activation row through a dense weight, RMSNorm over the N outputs, the residual added after
+// the norm; all f32, or all f16 with f32 sums (the reference's *_f16 variants).
 import { getNative, DTYPE } from '../native.js';
 import { createTensor } from '../tensor.js';
 import { acquireBuffer, releaseBuffer } from '../buffer-pool.js';
@@ -63,24 +63,31 @@ async function matmulRMSNormFused(recorder, input, weight, normWeight, options) 
     throw new Error('[MatmulRMSNormFused] input dtype is required.');
   }
   selectMatmulRMSNormFusedVariant(N, input.dtype);
-  if (input.dtype !== 'f32') {
-    throw new Error(`[MatmulRMSNormFused] the HIP path takes f32 activations, got ${input.dtype}.`);
+  const dtype = input.dtype;
+  if (dtype !== 'f32' && dtype !== 'f16') {
+    throw new Error(`[MatmulRMSNormFused] the HIP path takes f32 or f16 activations, got ${dtype}.`);
   }
-  const weightDtype = getWeightDtype(weight) || weight.dtype || 'f32';
-  if (weightDtype !== 'f32') {
-    throw new Error(`[MatmulRMSNormFused] the HIP path takes dense f32 weights, got ${weightDtype}.`);
+  const elem = dtype === 'f16' ? 2 : 4;
+  // the f16 variants take f16 weights, residual and output as well (fused_matmul_rmsnorm_f16.wgsl:41-45)
+  const weightDtype = getWeightDtype(weight) || weight.dtype || dtype;
+  if (weightDtype !== dtype) {
+    throw new Error(`[MatmulRMSNormFused] the HIP path takes dense ${dtype} weights for ${dtype} activations, got ${weightDtype}.`);
   }
-  if (input.buffer.size < K * 4 || weightBuffer.size < N * K * 4) {
+  if (input.buffer.size < K * elem || weightBuffer.size < N * K * elem) {
     throw new Error(`[MatmulRMSNormFused] input or weight buffer too small for N=${N}, K=${K}.`);
   }
   const residualBuffer = residual ? (residual.buffer || residual) : null;
-  if (residualBuffer && residualBuffer.size < N * 4) {
-    throw new Error(`[MatmulRMSNormFused] residual buffer smaller than N=${N} floats.`);
+  if (residualBuffer && residualBuffer.size < N * elem) {
+    throw new Error(`[MatmulRMSNormFused] residual buffer smaller than N=${N} elements.`);
   }
-  const output = outputBuffer || acquireBuffer(N * 4, undefined, 'matmul_rmsnorm_fused_output');
+  if (residual && residual.dtype && residual.dtype !== dtype) {
+    throw new Error(`[MatmulRMSNormFused] residual dtype must match the input's (${dtype}).`);
+  }
+  const output = outputBuffer || acquireBuffer(N * elem, undefined, 'matmul_rmsnorm_fused_output');
   const owned = outputBuffer ? null : output;
   try {
-    getNative().matmulRmsnormF32(input.buffer.ptr, weightBuffer.ptr, transposeB ? 1 : 0, normWeightBuffer.ptr,
+    const native = getNative();
+    (dtype === 'f16' ? native.matmulRmsnormF16 : native.matmulRmsnormF32)(input.buffer.ptr, weightBuffer.ptr, transposeB ? 1 : 0, normWeightBuffer.ptr,
       DTYPE[normWeightDtype], eps, rmsNormWeightOffset ? 1 : 0, residualBuffer ? residualBuffer.ptr : ptrOf(null),
       output.ptr, N, K);
   } catch (error) {

@@ -251,6 +251,16 @@ def dense_cases(L, T, rows, reps):
             emit(rows, config=4, kernel="dense matmul+rmsnorm f32", shape="N=%d K=%d %s" % (N, K, "[N,K]" if tb else "[K,N]"),
                  mode="rotating", us=round(us, 2), achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
         del Ws
+        Wh = [(torch.randn(N * K, device="cuda") * K ** -0.5).half() for _ in range(2 * copies)]
+        xh, resh, outh = x.half(), res.half(), torch.zeros(N, dtype=torch.float16, device="cuda")
+        algo = N * K * 2 + K * 2 + N * 4 + 2 * N * 2
+        for tb in (1, 0):
+            us = T.us(lambda i: capi.check(L.dh_matmul_rmsnorm_f16(xh.data_ptr(), Wh[i % (2 * copies)].data_ptr(), tb,
+                                                                   nw.data_ptr(), capi.F32, 1e-6, 1, resh.data_ptr(),
+                                                                   outh.data_ptr(), N, K)), max(8, reps // 4))
+            emit(rows, config=4, kernel="dense matmul+rmsnorm f16", shape="N=%d K=%d %s" % (N, K, "[N,K]" if tb else "[K,N]"),
+                 mode="rotating", us=round(us, 2), achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
+        del Wh
     M, N, K = 4, 6144, 1536
     nbytes = synth.q4k_nbytes(N, K)
     copies = n_copies(nbytes)

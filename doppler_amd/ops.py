@@ -226,9 +226,10 @@ def shouldUseFusedMatmulRMSNorm(M, N, K=None):
 
 def runMatmulRMSNormFused(input, weight, normWeight, options=None, **kw):
     """src/gpu/kernels/fused_matmul_rmsnorm.js:50 runMatmulRMSNormFused(input, weight, normWeight,
-    {N, K, eps, residual, outputBuffer, transposeB, rmsNormWeightOffset, label}): one f32
-    activation row through a dense f32 weight ([N, K] with transposeB, else [K, N]), RMSNorm over
-    the N outputs, residual added after the norm."""
+    {N, K, eps, residual, outputBuffer, transposeB, rmsNormWeightOffset, label}): one activation
+    row through a dense weight ([N, K] with transposeB, else [K, N]), RMSNorm over the N outputs,
+    residual added after the norm; all f32, or all f16 with f32 sums (the output dtype is the
+    input's, as in the reference)."""
     o = dict(options or {})
     o.update(kw)
     if o.get("transposeB") is None:
@@ -247,12 +248,16 @@ def runMatmulRMSNormFused(input, weight, normWeight, options=None, **kw):
     if not getattr(input, "dtype", None):
         raise DopplerHipError("[MatmulRMSNormFused] input dtype is required.")
     selectMatmulRMSNormFusedVariant(N, input.dtype)
-    if input.dtype != "f32":
-        raise DopplerHipError("[MatmulRMSNormFused] f32 activations required, got %s" % input.dtype)
-    wdtype = weight.dtype if isinstance(weight, (Tensor, WeightBuffer)) else "f32"
-    if wdtype != "f32":
-        raise DopplerHipError("[MatmulRMSNormFused] dense f32 weights required, got %s" % wdtype)
-    if _nbytes(input) < K * 4 or _nbytes(weight) < N * K * 4:
+    dtype = input.dtype
+    if dtype not in ("f32", "f16"):
+        raise DopplerHipError("[MatmulRMSNormFused] f32 or f16 activations required, got %s" % dtype)
+    elem = 2 if dtype == "f16" else 4
+    # the f16 variants take f16 weights, residual and output as well (fused_matmul_rmsnorm_f16.wgsl:41-45)
+    wdtype = weight.dtype if isinstance(weight, (Tensor, WeightBuffer)) else dtype
+    if wdtype != dtype:
+        raise DopplerHipError("[MatmulRMSNormFused] dense %s weights required for %s activations, got %s"
+                              % (dtype, dtype, wdtype))
+    if _nbytes(input) < K * elem or _nbytes(weight) < N * K * elem:
         raise DopplerHipError("[MatmulRMSNormFused] input or weight buffer too small for N=%d, K=%d" % (N, K))
     # the reference tells an f16 norm weight from an f32 one by the buffer's size (:14-28)
     nw_bytes = _nbytes(normWeight)
@@ -264,13 +269,15 @@ def runMatmulRMSNormFused(input, weight, normWeight, options=None, **kw):
         raise DopplerHipError("[MatmulRMSNormFused] norm weight size (%d bytes) does not match hiddenSize=%d "
                               "(expected %d or %d bytes)." % (nw_bytes, N, N * 2, N * 4))
     residual = o.get("residual")
-    if residual is not None and _nbytes(residual) < N * 4:
-        raise DopplerHipError("[MatmulRMSNormFused] residual buffer smaller than N=%d floats" % N)
-    out = _out(o.get("outputBuffer"), N * 4)
-    capi.check(_lib().dh_matmul_rmsnorm_f32(_ptr(input), _ptr(weight), 1 if o["transposeB"] else 0, _ptr(normWeight),
-                                            nw, float(o["eps"]), 1 if o["rmsNormWeightOffset"] else 0,
-                                            _ptr(residual), out.data_ptr(), int(N), int(K)))
-    return Tensor(out, "f32", (1, N), "matmul_rmsnorm_fused_output")
+    if residual is not None and _nbytes(residual) < N * elem:
+        raise DopplerHipError("[MatmulRMSNormFused] residual buffer smaller than N=%d elements" % N)
+    if residual is not None and getattr(residual, "dtype", dtype) != dtype:
+        raise DopplerHipError("[MatmulRMSNormFused] residual dtype must match the input's (%s)" % dtype)
+    out = _out(o.get("outputBuffer"), N * elem)
+    fn = _lib().dh_matmul_rmsnorm_f16 if dtype == "f16" else _lib().dh_matmul_rmsnorm_f32
+    capi.check(fn(_ptr(input), _ptr(weight), 1 if o["transposeB"] else 0, _ptr(normWeight), nw, float(o["eps"]),
+                  1 if o["rmsNormWeightOffset"] else 0, _ptr(residual), out.data_ptr(), int(N), int(K)))
+    return Tensor(out, dtype, (1, N), "matmul_rmsnorm_fused_output")
 
 
 def recordMatmulRMSNormFused(recorder, input, weight, normWeight, options=None, **kw):

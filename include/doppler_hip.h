@@ -338,6 +338,12 @@ int dh_cast_f16_to_f32(const void* d_in, float* d_out, int64_t n);
 int dh_matmul_rmsnorm_f32(const float* d_x, const float* d_W, int transpose_b,
                           const void* d_norm_weight, int norm_weight_dtype, float eps,
                           int weight_offset, const float* d_residual, float* d_out, int N, int K);
+/* The same with f16 activations, weights, residual and output (the reference's small_f16 /
+ * medium_f16 variants, fused_matmul_rmsnorm_f16.wgsl): every sum runs in f32 and the result is
+ * rounded to f16 once, on the final store. */
+int dh_matmul_rmsnorm_f16(const void* d_x, const void* d_W, int transpose_b,
+                          const void* d_norm_weight, int norm_weight_dtype, float eps,
+                          int weight_offset, const void* d_residual, void* d_out, int N, int K);
 
 /* Overflow guard for activations: the first element of d_input (f32 or f16) that is NaN,
  * infinite or larger in magnitude than abs_threshold (<= 0 or not finite: 65500) turns

@@ -237,16 +237,17 @@ async function main() {
       }
       fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
     } else if (c.op === 'matmul_rmsnorm_fused') {
+      const dt = c.dtype || 'f32';
       const opts = { N: c.N, K: c.K, eps: c.eps, transposeB: c.transposeB, rmsNormWeightOffset: c.weightOffset,
-        residual: c.residual ? tensor(c.residual, 'f32', [1, c.N]) : null, label: 'test' };
-      const x = tensor(c.x, 'f32', [1, c.K]);
-      const W = dh.createWeightBuffer(dev(c.W), 'f32', 'row', c.transposeB ? [c.N, c.K] : [c.K, c.N], c.name);
+        residual: c.residual ? tensor(c.residual, dt, [1, c.N]) : null, label: 'test' };
+      const x = tensor(c.x, dt, [1, c.K]);
+      const W = dh.createWeightBuffer(dev(c.W), dt, 'row', c.transposeB ? [c.N, c.K] : [c.K, c.N], c.name);
       const nw = dev(c.normWeight);
       if (!dh.shouldUseFusedMatmulRMSNorm(1, c.N, c.K)) throw new Error('shouldUseFusedMatmulRMSNorm said no');
       const rec = c.record ? dh.createCommandRecorder('t') : null;
       const t = rec ? await dh.recordMatmulRMSNormFused(rec, x, W, nw, opts) : await dh.runMatmulRMSNormFused(x, W, nw, opts);
       if (rec) await rec.submitAndWait();
-      await save(out, t.buffer, c.N * 4);
+      await save(out, t.buffer, c.N * (dt === 'f16' ? 2 : 4));
     } else if (c.op === 'check_finiteness') {
       // one status buffer across the listed checks, in order: [input file, dtype, size, layer, step, threshold]
       const status = dh.createFinitenessStatusBuffer();

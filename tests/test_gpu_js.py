@@ -120,6 +120,19 @@ def test_js_host_path_parity(tmp_path):
                                             weight_offset=off, residual=fr)
         checks.append(lambda nm=nm, fwant=fwant: rel_l2(get(nm + ".out.bin", np.float32), fwant) <= 1e-5)
 
+    # the all-f16 variant of the same op
+    g = synth.rng(9175)
+    hx = g.standard_normal(520).astype(np.float16)
+    hW = (g.standard_normal((1032, 520)) * 520 ** -0.5).astype(np.float16)
+    hw = g.standard_normal(1032).astype(np.float32)
+    hr = g.standard_normal(1032).astype(np.float16)
+    cases.append(dict(name="mr_h", op="matmul_rmsnorm_fused", dtype="f16", x=put("mr_h.x", hx.view(np.uint16)),
+                      W=put("mr_h.W", hW.view(np.uint16)), normWeight=put("mr_h.nw", hw), residual=put("mr_h.r", hr.view(np.uint16)),
+                      N=1032, K=520, eps=1e-6, transposeB=True, weightOffset=False, record=False))
+    hwant = oracle.matmul_rmsnorm_fused(hx.astype(np.float32), hW.astype(np.float32), hw, 1032, 520, 1e-6,
+                                        residual=hr.astype(np.float32))
+    checks.append(lambda: rel_l2(get("mr_h.out.bin", np.float16).astype(np.float32), hwant) <= 5e-4)
+
     # finiteness guard: clean f32, then an f16 overflow that sets the status, then a later NaN that must not overwrite it
     fin_clean = synth.normal_f32(5000, 9180, 100.0)
     fin_over = synth.normal_f32(5000, 9181).astype(np.float16)

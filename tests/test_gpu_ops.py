@@ -1005,6 +1005,37 @@ def test_matmul_rmsnorm_fused(N, K, transposeB, offset, residual, w16):
         assert a.tobytes() == again.tobytes()       # run to run deterministic
 
 
+@pytest.mark.parametrize("N,K,transposeB,offset,residual,w16", [
+    (1152, 6912, True, True, True, True), (1152, 6912, False, False, True, False),
+    (4096, 8192, True, False, False, False), (4096, 8192, False, True, True, True),
+    (250, 1000, True, False, True, False), (7, 13, False, True, False, True), (1001, 301, True, True, True, True),
+    (1004, 304, False, False, False, False)])
+def test_matmul_rmsnorm_fused_f16(N, K, transposeB, offset, residual, w16):
+    """The all-f16 variants (fused_matmul_rmsnorm_f16.wgsl): f16 activations, weights, residual and
+    output, sums in f32.  Checked against the f64 evaluation of the same f16 inputs; the bar is the
+    rounding of the f16 result (relative 2^-11 per element, and the reference's medium variant
+    rounds the product to f16 once more before it normalises)."""
+    g = synth.rng(7200 + N + K)
+    x = g.standard_normal(K).astype(np.float16)
+    W = (g.standard_normal((N, K)) * K ** -0.5).astype(np.float16)
+    w = g.standard_normal(N).astype(np.float16 if w16 else np.float32)
+    r = g.standard_normal(N).astype(np.float16) if residual else None
+    stored = W if transposeB else np.ascontiguousarray(W.T)
+    up16 = lambda a: ops.tensorFromNumpy(a.view(np.uint16))
+    assert ops.selectMatmulRMSNormFusedVariant(N, "f16") == ("small_f16" if N <= 256 else "medium_f16")
+    out = ops.runMatmulRMSNormFused(up16(x), ops.createWeightBuffer(up16(stored).buffer, "f16", "row", stored.shape), 
+                                    up16(w) if w16 else ops.tensorFromNumpy(w),
+                                    {"N": N, "K": K, "eps": 1e-6, "transposeB": transposeB, "rmsNormWeightOffset": offset,
+                                     "residual": up16(r) if residual else None})
+    assert out.shape == (1, N) and out.dtype == "f16"
+    got = ops.readTensor(out).view(np.float16).astype(np.float32)
+    want = oracle.matmul_rmsnorm_fused(x.astype(np.float32), stored.astype(np.float32), w.astype(np.float32), N, K, 1e-6,
+                                       transpose_b=transposeB, weight_offset=offset,
+                                       residual=r.astype(np.float32) if residual else None)
+    assert rel_l2(got, want) <= 5e-4
+    assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.maximum(np.abs(want), 2.0 ** -14) + 1e-6)
+
+
 def test_matmul_rmsnorm_fused_errors_and_selection():
     x = ops.tensorFromNumpy(np.zeros(8, np.float32))
     W = ops.tensorFromNumpy(np.zeros((4, 8), np.float32))
@@ -1019,6 +1050,9 @@ def test_matmul_rmsnorm_fused_errors_and_selection():
         ops.runMatmulRMSNormFused(x, W, nw, {"N": 4097, "K": 8, "eps": 1e-6, "transposeB": True, "rmsNormWeightOffset": False})
     with pytest.raises(DopplerHipError, match="does not match hiddenSize=4"):
         ops.runMatmulRMSNormFused(x, W, ops.tensorFromNumpy(np.ones(1, np.float32)),
+                                  {"N": 4, "K": 8, "eps": 1e-6, "transposeB": True, "rmsNormWeightOffset": False})
+    with pytest.raises(DopplerHipError, match="dense f16 weights required for f16 activations"):
+        ops.runMatmulRMSNormFused(ops.tensorFromNumpy(np.zeros(8, np.uint16)), W, nw,
                                   {"N": 4, "K": 8, "eps": 1e-6, "transposeB": True, "rmsNormWeightOffset": False})
     with pytest.raises(DopplerHipError, match="exceeds maxMediumN"):
         capi.check(capi.init(0).dh_matmul_rmsnorm_f32(x.buffer.data_ptr(), W.buffer.data_ptr(), 1, nw.buffer.data_ptr(),
