@@ -518,19 +518,55 @@ __global__ __launch_bounds__(256 * MG) void q4k_gemm_kernel(const GemmArgs a) {
     }
 }
 
-// C = alpha * (sum of the split-K pieces, in split order) + residual.
+// C = alpha * (sum of the split-K pieces, in split order) + residual.  Four consecutive outputs per
+// thread when the row length allows 16-byte accesses, every piece's load in flight before the sums.
+constexpr int kMaxSplit = 8;
+template <bool VEC>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs a) {
   const int64_t total = (int64_t)a.M * a.N;
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  constexpr int W = VEC ? 4 : 1;
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * W;
   if (i >= total) return;
-  float s = 0.f;
-  for (int z = 0; z < a.ksplit; z++) s += a.partial[(int64_t)z * total + i];
-  float v = s * a.alpha;
-  if (a.residual) v += a.residual[i];
-  if (a.c_f16)
-    reinterpret_cast<__half*>(a.C)[i] = __float2half(v);
-  else
-    reinterpret_cast<float*>(a.C)[i] = v;
+  float p[kMaxSplit][W];
+#pragma unroll
+  for (int z = 0; z < kMaxSplit; z++) {
+    if (z < a.ksplit) {
+      if constexpr (VEC) {
+        const float4 t = *reinterpret_cast<const float4*>(a.partial + (int64_t)z * total + i);
+        p[z][0] = t.x; p[z][1] = t.y; p[z][2] = t.z; p[z][3] = t.w;
+      } else {
+        p[z][0] = a.partial[(int64_t)z * total + i];
+      }
+    }
+  }
+  float r[W];
+#pragma unroll
+  for (int e = 0; e < W; e++) r[e] = 0.f;
+  if (a.residual) {
+    if constexpr (VEC) {
+      const float4 t = *reinterpret_cast<const float4*>(a.residual + i);
+      r[0] = t.x; r[1] = t.y; r[2] = t.z; r[3] = t.w;
+    } else {
+      r[0] = a.residual[i];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < W; e++) {
+    float s = 0.f;
+#pragma unroll
+    for (int z = 0; z < kMaxSplit; z++)
+      if (z < a.ksplit) s += p[z][e];
+    r[e] = s * a.alpha + r[e];
+  }
+  if (a.c_f16) {
+    __half* c = reinterpret_cast<__half*>(a.C) + i;
+#pragma unroll
+    for (int e = 0; e < W; e++) c[e] = __float2half(r[e]);
+  } else if constexpr (VEC) {
+    *reinterpret_cast<float4*>(reinterpret_cast<float*>(a.C) + i) = make_float4(r[0], r[1], r[2], r[3]);
+  } else {
+    reinterpret_cast<float*>(a.C)[i] = r[0];
+  }
 }
 
 template <bool DUAL, int T, int MG>
@@ -549,7 +585,12 @@ int launch_gemm_cfg(const GemmArgs& a, const char* op) {
   DH_CHECK_LAUNCH(op);
   if (a.ksplit > 1) {
     const int64_t total = (int64_t)a.M * a.N;
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)dh::ceil_div(total, 256)), dim3(256), 0, dh::stream(), a);
+    if (a.ksplit > kMaxSplit) return dh::fail(2, "[%s] internal: K cut into %d pieces, the reduction takes %d", op, a.ksplit, kMaxSplit);
+    const bool vec = total % 4 == 0 && (reinterpret_cast<uintptr_t>(a.C) | reinterpret_cast<uintptr_t>(a.residual)) % 16 == 0;
+    if (vec)
+      hipLaunchKernelGGL(splitk_reduce_kernel<true>, dim3((unsigned)dh::ceil_div(total / 4, 256)), dim3(256), 0, dh::stream(), a);
+    else
+      hipLaunchKernelGGL(splitk_reduce_kernel<false>, dim3((unsigned)dh::ceil_div(total, 256)), dim3(256), 0, dh::stream(), a);
     DH_CHECK_LAUNCH(op);
   }
   return 0;
