@@ -71,6 +71,17 @@ struct GraphAttnCall {
   void* ws;
   hipGraphNode_t split_node, merge_node;
 };
+// A dh_check_finiteness call recorded during a capture: its step number follows the position.
+struct GraphFiniteCall {
+  const void* input;
+  int dtype;
+  int64_t size;
+  uint32_t* status;
+  uint32_t layer, step;    // step at capture time
+  float abs_threshold;
+  unsigned grid;
+  hipGraphNode_t node;
+};
 struct Graph {
   hipGraph_t graph = nullptr;
   hipGraphExec_t exec = nullptr;
@@ -78,6 +89,8 @@ struct Graph {
   int captured_position = 0;
   GraphAttnCall* attn = nullptr;
   int n_attn = 0, cap_attn = 0;
+  GraphFiniteCall* fin = nullptr;
+  int n_fin = 0, cap_fin = 0;
 };
 // The graph being captured on the op stream, or null.
 Graph* capturing_graph();
@@ -86,6 +99,11 @@ void graph_note_attention(const GraphAttnCall& call);
 // attention.hip: finds the kernel nodes of the recorded calls in the captured graph / patches them for `position`.
 int attn_graph_bind(Graph* g);
 int attn_graph_set_position(Graph* g, int position);
+// elementwise.hip: the same for the finiteness checks of a captured step (their step number is a
+// launch argument: a replay at position p reports captured step + p - captured position).
+void graph_note_finiteness(const GraphFiniteCall& call);
+int finite_graph_bind(Graph* g);
+int finite_graph_set_position(Graph* g, int position);
 
 // Looks up, once per device, the address of the fixed device array that dh_attn_decode_static uses
 // for its split partials (attention.hip).  Called by dh_init with the device current.

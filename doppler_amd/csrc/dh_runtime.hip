@@ -48,6 +48,19 @@ void graph_note_attention(const GraphAttnCall& call) {
   }
   g->attn[g->n_attn++] = call;
 }
+void graph_note_finiteness(const GraphFiniteCall& call) {
+  Graph* g = g_capturing;
+  if (!g) return;
+  if (g->n_fin == g->cap_fin) {
+    const int cap = g->cap_fin ? 2 * g->cap_fin : 64;
+    GraphFiniteCall* grown = new GraphFiniteCall[cap];
+    for (int i = 0; i < g->n_fin; i++) grown[i] = g->fin[i];
+    delete[] g->fin;
+    g->fin = grown;
+    g->cap_fin = cap;
+  }
+  g->fin[g->n_fin++] = call;
+}
 float* splitk_workspace(size_t* bytes) {
   *bytes = g_splitk_ws ? kSplitKWsBytes : 0;
   return g_splitk_ws;
@@ -271,6 +284,7 @@ static void graph_free(dh::Graph* g) {
   if (g->exec) (void)hipGraphExecDestroy(g->exec);
   if (g->graph) (void)hipGraphDestroy(g->graph);
   delete[] g->attn;
+  delete[] g->fin;
   delete g;
 }
 
@@ -296,6 +310,10 @@ int dh_graph_end(int position, void** graph_out) {
     graph_free(g);
     return rc;
   }
+  if (int rc = dh::finite_graph_bind(g)) {
+    graph_free(g);
+    return rc;
+  }
   *graph_out = g;
   return 0;
 }
@@ -308,6 +326,7 @@ int dh_graph_launch(void* graph, int position) {
   if (position < 0) return dh::fail(1, "[dh_graph_launch] position must be non-negative");
   if (position != g->position) {
     if (int rc = dh::attn_graph_set_position(g, position)) return rc;
+    if (int rc = dh::finite_graph_set_position(g, position)) return rc;
     g->position = position;
   }
   DH_CHECK_HIP("dh_graph_launch", hipGraphLaunch(g->exec, g_stream));
@@ -321,6 +340,7 @@ int dh_graph_prepare(void* graph, int position) {
   if (position < 0) return dh::fail(1, "[dh_graph_prepare] position must be non-negative");
   if (position != g->position) {
     if (int rc = dh::attn_graph_set_position(g, position)) return rc;
+    if (int rc = dh::finite_graph_set_position(g, position)) return rc;
     g->position = position;
   }
   return 0;

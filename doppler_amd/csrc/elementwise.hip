@@ -425,6 +425,73 @@ unsigned grid_for(int64_t n) { return (unsigned)dh::ceil_div(n, 256); }
 
 }  // namespace
 
+namespace dh {
+
+static void* finiteness_kernel_for(int dtype) {
+  return dtype == DH_F16 ? reinterpret_cast<void*>(check_finiteness_kernel<__half>)
+                         : reinterpret_cast<void*>(check_finiteness_kernel<float>);
+}
+
+// Finds the kernel node of every recorded check: same kernel, input, status word, layer and step.
+int finite_graph_bind(Graph* g) {
+  if (g->n_fin == 0) return 0;
+  size_t n = 0;
+  DH_CHECK_HIP("dh_graph_end", hipGraphGetNodes(g->graph, nullptr, &n));
+  hipGraphNode_t* nodes = new hipGraphNode_t[n ? n : 1];
+  hipError_t e = hipGraphGetNodes(g->graph, nodes, &n);
+  if (e != hipSuccess) {
+    delete[] nodes;
+    return fail(2, "[dh_graph_end] hipGraphGetNodes failed: %s", hipGetErrorString(e));
+  }
+  int found = 0;
+  for (size_t i = 0; i < n; i++) {
+    hipGraphNodeType type;
+    if (hipGraphNodeGetType(nodes[i], &type) != hipSuccess || type != hipGraphNodeTypeKernel) continue;
+    hipKernelNodeParams kp{};
+    if (hipGraphKernelNodeGetParams(nodes[i], &kp) != hipSuccess || !kp.kernelParams) continue;
+    for (int c = 0; c < g->n_fin; c++) {
+      GraphFiniteCall& f = g->fin[c];
+      if (f.node || kp.func != finiteness_kernel_for(f.dtype)) continue;
+      const void* in = *static_cast<const void* const*>(kp.kernelParams[0]);
+      const uint32_t* status = *static_cast<uint32_t* const*>(kp.kernelParams[2]);
+      const uint32_t layer = *static_cast<const uint32_t*>(kp.kernelParams[3]);
+      const uint32_t step = *static_cast<const uint32_t*>(kp.kernelParams[4]);
+      if (in == f.input && status == f.status && layer == f.layer && step == f.step) {
+        f.node = nodes[i];
+        found++;
+        break;
+      }
+    }
+  }
+  delete[] nodes;
+  if (found != g->n_fin)
+    return fail(2, "[dh_graph_end] found the kernel nodes of %d of %d finiteness checks in the captured graph", found, g->n_fin);
+  return 0;
+}
+
+int finite_graph_set_position(Graph* g, int position) {
+  const int delta = position - g->captured_position;
+  for (int i = 0; i < g->n_fin; i++) {
+    const GraphFiniteCall& f = g->fin[i];
+    const void* in = f.input;
+    int64_t size = f.size;
+    uint32_t* status = f.status;
+    uint32_t layer = f.layer, step = (uint32_t)((int64_t)f.step + delta);
+    float thr = f.abs_threshold;
+    void* args[] = {&in, &size, &status, &layer, &step, &thr};
+    hipKernelNodeParams kp{};
+    kp.func = finiteness_kernel_for(f.dtype);
+    kp.gridDim = dim3(f.grid);
+    kp.blockDim = dim3(256);
+    kp.sharedMemBytes = 0;
+    kp.kernelParams = args;
+    DH_CHECK_HIP("dh_graph_launch", hipGraphExecKernelNodeSetParams(g->exec, f.node, &kp));
+  }
+  return 0;
+}
+
+}  // namespace dh
+
 extern "C" {
 
 int dh_rmsnorm(const float* d_x, const void* d_weight, int weight_dtype, float* d_out, int batch,
@@ -756,6 +823,7 @@ int dh_check_finiteness(const void* d_input, int dtype, int64_t size, uint32_t* 
     hipLaunchKernelGGL(check_finiteness_kernel<float>, dim3(grid), dim3(256), 0, dh::stream(),
                        static_cast<const float*>(d_input), size, d_status, layer, step, abs_threshold);
   DH_CHECK_LAUNCH(op);
+  dh::graph_note_finiteness(dh::GraphFiniteCall{d_input, dtype, size, d_status, layer, step, abs_threshold, grid, nullptr});
   return 0;
 }
 

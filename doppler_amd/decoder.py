@@ -229,14 +229,16 @@ class HipDecoder:
         normally first so that every kernel's one-time set-up is done outside the capture."""
         if not self.fuse_qkv_attention:
             raise ValueError("capture_step serves the step with the fused attention kernel")
-        if self.finiteness_guard:
-            # the guard's step number is a launch argument: a replayed graph would report the capture's
-            raise ValueError("capture_step does not serve a decoder with the finiteness guard on")
-        self.enqueue_step(pos, want_logits)
+        # with the guard on the captured step also clears the status words and leaves its token next
+        # to them (the library moves the checks' step number with the position at every replay)
+        out_index = self.TOKEN_RING - 1 if self.finiteness_guard else 0
+        self.enqueue_step(pos, want_logits, out_index=out_index)
         capi.check(self.L.dh_sync())
         capi.check(self.L.dh_graph_begin())
         try:
-            self.enqueue_step(pos, want_logits)
+            if self.finiteness_guard:
+                self._reset_finiteness()
+            self.enqueue_step(pos, want_logits, out_index=out_index)
         finally:
             g = ctypes.c_void_p()
             rc = self.L.dh_graph_end(pos, ctypes.byref(g))
@@ -246,7 +248,7 @@ class HipDecoder:
 
     def step_graph(self, token, pos):
         """One decode step by replaying the captured graph at position `pos`: one graph launch
-        and the 4-byte token readback."""
+        and the 4-byte token readback (20 bytes with the finiteness guard on)."""
         if not 0 <= pos < self.max_seq:
             raise ValueError("decode position %d is outside the KV cache (max_seq=%d)" % (pos, self.max_seq))
         if getattr(self, "_graph", None) is None:
@@ -256,7 +258,12 @@ class HipDecoder:
         if pos + 1 < self.max_seq:
             # the next position's node parameters are set while the GPU runs this one
             capi.check(self.L.dh_graph_prepare(self._graph, pos + 1))
-        return self.read_token()
+        if not self.finiteness_guard:
+            return self.read_token()
+        words = np.empty(5, np.uint32)
+        capi.check(self.L.dh_download(words.ctypes.data, self.token.data_ptr(), 4 * (self.TOKEN_RING - 1), 20))
+        self._raise_if_triggered(words, 1, "generation")
+        return int(words[0])
 
     def release_graph(self):
         if getattr(self, "_graph", None) is not None:

@@ -254,13 +254,14 @@ export class HipTextDecoder {
   // uses stay allocated for the graph's life.
   async captureDecodeStep(token, pos) {
     if (!this.fuseQkvAttention) throw new Error('[captureDecodeStep] serves the fused-attention step');
-    // the guard's step number is a launch argument: a replayed graph would report the capture's
-    if (this.finitenessGuard) throw new Error('[captureDecodeStep] does not serve a decoder with the finiteness guard on');
     const first = await this.decodeStep(token, pos);
     getNative().graphBegin();
     let graph = null;
     const temps = [];
     try {
+      // with the guard on the captured step also clears the status words (the library moves the
+      // checks' step number with the position at every replay)
+      if (this.finitenessGuard) getNative().fillZero(this.tokenOut.ptr, 4, FINITENESS_STATUS_BYTES);
       await this.recordDecodeStep(createCommandRecorder('decode_capture'), temps, pos, {});
     } finally {
       graph = getNative().graphEnd(pos);
@@ -281,8 +282,13 @@ export class HipTextDecoder {
     getNative().graphLaunch(this.graph, pos);
     // the next position's node parameters are set while the GPU runs this one
     if (pos + 1 < c.maxSeq) getNative().graphPrepare(this.graph, pos + 1);
-    const bytes = await readBufferSlice(this.tokenOut, 0, 4);
-    return new Uint32Array(bytes)[0];
+    const bytes = await readBufferSlice(this.tokenOut, 0, this.finitenessGuard ? 4 + FINITENESS_STATUS_BYTES : 4);
+    const words = new Uint32Array(bytes);
+    if (this.finitenessGuard) {
+      const status = parseFinitenessStatusWords(words, 1);
+      if (status.triggered) throw new FinitenessError(`F16 bounds exceeded during generation${status.metadata}`);
+    }
+    return words[0];
   }
 
   releaseGraph() {

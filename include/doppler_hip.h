@@ -351,7 +351,9 @@ int dh_matmul_rmsnorm_f16(const void* d_x, const void* d_W, int transpose_b,
  * d_status[2]; a status that is already 1 is left alone.  d_status is 4 u32 words the caller
  * zeroes before a step and reads back beside the token.  Replaces recordCheckFiniteness,
  * src/gpu/kernels/check-finiteness.js:98-150 (shader :25-62); read back as the reference does at
- * src/inference/pipelines/text/generator-steps.js:786-798. */
+ * src/inference/pipelines/text/generator-steps.js:786-798.  Recorded into a captured step
+ * (dh_graph_begin .. dh_graph_end) its step number follows the replay position:
+ * step + position - position of the capture. */
 int dh_check_finiteness(const void* d_input, int dtype, int64_t size, uint32_t* d_status,
                         uint32_t layer, uint32_t step, float abs_threshold);
 

@@ -332,8 +332,18 @@ def test_finiteness_guard_reads_status_beside_the_token():
     t0 = b_plain.prefill(prompt)
     assert b_guard.prefill(prompt) == t0
     assert b_guard.decode_batch(t0, len(prompt), 9) == b_plain.decode_batch(t0, len(prompt), 9)
-    with pytest.raises(ValueError, match="finiteness guard"):
-        guarded.capture_step(20)
+    # under a captured graph: same tokens as the unguarded replay
+    gp = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32)
+    gg = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32, finiteness_guard=True,
+                            finiteness_abs_threshold=1e30)
+    tok_p = gp.prefill(prompt)
+    assert gg.prefill(prompt) == tok_p
+    tok_g = tok_p
+    for i in range(7):
+        tok_p = gp.step_graph(tok_p, len(prompt) + i)
+        tok_g = gg.step_graph(tok_g, len(prompt) + i)
+        assert tok_g == tok_p, i
+    assert [tok_p] == want[7:8]
     # the residual stream after each layer, from the unguarded decoder's buffers: pick a bound between
     # layer 0's and layer 2's peak so that the layer the guard names is known
     probe = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32)
@@ -354,6 +364,13 @@ def test_finiteness_guard_reads_status_beside_the_token():
         trip.step(t0, len(prompt))
     with pytest.raises(decoder.FinitenessError, match=r"during batch generation \(layer %d, step %d\)" % (first_over, len(prompt))):
         trip.decode_batch(t0, len(prompt), 4)
+    # replayed steps report their own step number: the check's step argument follows the position
+    gt = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32, finiteness_guard=True,
+                            finiteness_abs_threshold=bound)
+    gt.prefill(prompt)
+    for i in range(3):
+        with pytest.raises(decoder.FinitenessError, match=r"\(layer \d+, step %d\)" % (len(prompt) + i)):
+            gt.step_graph(t0, len(prompt) + i)
     default = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, 32, finiteness_guard=True)
     default.prefill(prompt)
     with pytest.raises(decoder.FinitenessError, match=r"\(layer 0, step %d\)" % len(prompt)):

@@ -322,8 +322,10 @@ def test_js_host_path_parity(tmp_path):
     # bound of 65500 the first step throws and names layer 0
     cases.append(dict(cases[-3], name="decoder_guarded",
                       config=dict(cases[-3]["config"], finitenessGuard=True, finitenessAbsThreshold=1e30)))
-    cases.append(dict(cases[-4], name="decoder_guard_trips", expectFinitenessAt=0,
-                      config=dict(cases[-4]["config"], finitenessGuard=True)))
+    cases.append(dict(cases[-4], name="decoder_guarded_graph", graphFrom=2,
+                      config=dict(cases[-4]["config"], finitenessGuard=True, finitenessAbsThreshold=1e30)))
+    cases.append(dict(cases[-5], name="decoder_guard_trips", expectFinitenessAt=0,
+                      config=dict(cases[-5]["config"], finitenessGuard=True)))
     ol = []
     for l in layers:
         dd = dict(l)
@@ -339,6 +341,7 @@ def test_js_host_path_parity(tmp_path):
     checks.append(lambda: [int(t) for t in get("decoder_separate_qkv_kernel.out.bin", np.uint32)] == want_tokens)
     checks.append(lambda: [int(t) for t in get("decoder_graph_replay.out.bin", np.uint32)] == want_tokens)
     checks.append(lambda: [int(t) for t in get("decoder_guarded.out.bin", np.uint32)] == want_tokens)
+    checks.append(lambda: [int(t) for t in get("decoder_guarded_graph.out.bin", np.uint32)] == want_tokens)
     checks.append(lambda: get("decoder_guard_trips.out.bin", np.uint32).size == 0)
 
     # ---- top-k temperature sampling through the JS op (seeded draw as in the reference)
