@@ -24,6 +24,24 @@ _I64 = ctypes.c_int64
 _F = ctypes.c_float
 _SZ = ctypes.c_size_t
 
+class ChainPhase(ctypes.Structure):
+    """struct dh_chain_phase: one product of dh_q4k_gemv_chain."""
+    _fields_ = [("d_W", _P), ("d_W2", _P), ("d_C", _P), ("d_residual", _P), ("d_norm_weight", _P),
+                ("N", _I), ("K", _I), ("activation", _I), ("norm_weight_offset", _I),
+                ("alpha", _F), ("swiglu_limit", _F), ("norm_eps", _F)]
+
+
+def chain_phases(phases):
+    """list of dicts (W, W2, C, residual, norm_weight: device addresses or None; N, K; activation,
+    norm_weight_offset, alpha, swiglu_limit, norm_eps) -> ctypes array of dh_chain_phase."""
+    arr = (ChainPhase * len(phases))()
+    for i, ph in enumerate(phases):
+        arr[i] = ChainPhase(ph["W"], ph.get("W2"), ph["C"], ph.get("residual"), ph.get("norm_weight"), ph["N"], ph["K"],
+                            ph.get("activation", 0), ph.get("norm_weight_offset", 0), ph.get("alpha", 1.0),
+                            ph.get("swiglu_limit", 0.0), ph.get("norm_eps", 0.0))
+    return arr
+
+
 # name -> (restype, argtypes); every symbol include/doppler_hip.h declares
 SIGNATURES = {
     "dh_init": (_I, [_I]),
@@ -52,6 +70,8 @@ SIGNATURES = {
     "dh_q4k_matmul_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
     "dh_q4k_ffn_gate_up": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
     "dh_q4k_ffn_gate_up_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
+    "dh_q4k_gemv_chain": (_I, [_P, ctypes.POINTER(ChainPhase), _I]),
+    "dh_q4k_gemv_chain_limited": (_I, [_P, ctypes.POINTER(ChainPhase), _I, _I, _I]),
     "dh_f16w_matmul": (_I, [_P, _P, _P, _I, _I, _I, _F]),
     "dh_lmhead_argmax_workspace_bytes": (_SZ, [_I]),
     "dh_lmhead_argmax_f16": (_I, [_P, _P, _I, _I, _I64, _F, _P, _P, _I, _P]),

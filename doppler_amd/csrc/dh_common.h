@@ -36,6 +36,24 @@ float* widened_activations(size_t* bytes);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// ---- kernel status word ---------------------------------------------------------------------
+// Kernels that wait on other waves or workgroups bound every such wait; a wave whose wait runs
+// into its limit stores a code here and leaves.  The word lives in pinned host memory that the
+// device can write, so the host can look at it for free after every stream synchronisation
+// (dh_sync, dh_download, dh_upload, dh_free), which then fail with the decoded message.
+#define DH_KSTATUS_COLUMN_WAIT 1u     // GEMV: a column's activation operands never arrived
+#define DH_KSTATUS_SLOT_WAIT 2u       // GEMV: a tile slot was never released
+#define DH_KSTATUS_EXCHANGE_WAIT 3u   // chained GEMV: another workgroup's outputs never arrived
+uint32_t* kernel_status_word();
+// Reads and clears the word (call only after the stream has been synchronised); non-zero -> fail().
+int check_kernel_status(const char* op);
+// chained GEMV (q4k_gemv_chain.hip): called when a launch has reported a failed wait, so that the
+// next launch starts from a clean exchange area.
+void gemv_chain_reset();
+// chained GEMV: exchange area and launch counter (allocated by dh_init, freed with the runtime).
+int gemv_chain_init(int device);
+void gemv_chain_release();
+
 // Matrix-core GEMM for prefill-sized batches (q4k_gemm.hip).  `serves`: M >= 16, K a multiple
 // of 4, A 16-byte aligned.
 bool q4k_gemm_serves(int M, int K, const void* A);
@@ -121,6 +139,13 @@ int q4k_gemv_rows(const char* op, const float* A, const uint8_t* W, const uint8_
                   const float* residual, int M, int N, int K, float alpha, int activation, float clamp_max,
                   const float* norm_weight, float norm_eps, int norm_weight_offset);
 
+}  // namespace dh
+
+namespace dh {
+// kind in the top 4 bits (never zero), phase of a chained launch below it, workgroup in the low 24.
+__host__ __device__ inline uint32_t kstatus_code(uint32_t kind, uint32_t phase, uint32_t block) {
+  return (kind << 28) | ((phase & 0xFu) << 24) | (block & 0xFFFFFFu);
+}
 }  // namespace dh
 
 #ifdef __HIPCC__

@@ -21,6 +21,7 @@ void* g_packed_a = nullptr;          // packed f16 activations of the prefill GE
 constexpr size_t kPackedABytes = (size_t)64 << 20;
 float* g_widened_a = nullptr;        // f16 activations of dh_q4k_matmul widened to f32
 constexpr size_t kWidenedABytes = (size_t)64 << 20;
+uint32_t* g_kstatus = nullptr;       // kernel status word: pinned host memory, device-writable
 }  // namespace
 
 namespace dh {
@@ -75,6 +76,21 @@ float* widened_activations(size_t* bytes) {
   *bytes = g_widened_a ? kWidenedABytes : 0;
   return g_widened_a;
 }
+uint32_t* kernel_status_word() { return g_kstatus; }
+int check_kernel_status(const char* op) {
+  if (!g_kstatus) return 0;
+  const uint32_t code = *static_cast<volatile uint32_t*>(g_kstatus);
+  if (code == 0u) return 0;
+  *static_cast<volatile uint32_t*>(g_kstatus) = 0u;
+  gemv_chain_reset();
+  const uint32_t kind = code >> 28, phase = (code >> 24) & 0xFu, block = code & 0xFFFFFFu;
+  const char* what = kind == DH_KSTATUS_COLUMN_WAIT ? "a column's activation operands did not arrive (Q4_K GEMV)"
+                     : kind == DH_KSTATUS_SLOT_WAIT ? "a tile slot was not released (Q4_K GEMV)"
+                     : kind == DH_KSTATUS_EXCHANGE_WAIT ? "the previous product's outputs did not arrive from the other workgroups (chained Q4_K GEMV)"
+                                                        : "unknown wait";
+  return fail(3, "[%s] a kernel launched earlier gave up a bounded wait: %s; phase %u, workgroup %u; its outputs are "
+              "undefined", op, what, phase, block);
+}
 }  // namespace dh
 
 extern "C" {
@@ -93,12 +109,15 @@ static int release_all(const char* op) {
   if (g_row_scale) note(hipFree(g_row_scale));
   if (g_packed_a) note(hipFree(g_packed_a));
   if (g_widened_a) note(hipFree(g_widened_a));
+  if (g_kstatus) note(hipHostFree(g_kstatus));
+  dh::gemv_chain_release();
   g_own_stream = nullptr;
   g_stream = nullptr;
   g_splitk_ws = nullptr;
   g_row_scale = nullptr;
   g_packed_a = nullptr;
   g_widened_a = nullptr;
+  g_kstatus = nullptr;
   g_num_cus = 0;
   g_ready = false;
   g_device = -1;
@@ -124,7 +143,10 @@ static int init_locked(int device_ordinal) {
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_row_scale), (size_t)kRowScaleRows * 2 * sizeof(float)));
   DH_CHECK_HIP("dh_init", hipMalloc(&g_packed_a, kPackedABytes));
   DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_widened_a), kWidenedABytes));
+  DH_CHECK_HIP("dh_init", hipHostMalloc(reinterpret_cast<void**>(&g_kstatus), 64, hipHostMallocMapped));
+  *g_kstatus = 0u;
   if (int rc = dh::attn_static_scratch_init(device_ordinal)) return rc;
+  if (int rc = dh::gemv_chain_init(device_ordinal)) return rc;
   g_device = device_ordinal;
   g_ready = true;
   return 0;
@@ -178,7 +200,7 @@ int dh_free(void* d_ptr) {
   if (!d_ptr) return 0;
   DH_CHECK_HIP("dh_free", hipStreamSynchronize(g_stream));
   DH_CHECK_HIP("dh_free", hipFree(d_ptr));
-  return 0;
+  return dh::check_kernel_status("dh_free");
 }
 
 int dh_upload(void* d_dst, size_t dst_offset, const void* host_src, size_t bytes) {
@@ -191,7 +213,7 @@ int dh_upload(void* d_dst, size_t dst_offset, const void* host_src, size_t bytes
   DH_CHECK_HIP("dh_upload", hipMemcpyAsync(static_cast<char*>(d_dst) + dst_offset, host_src, bytes,
                                            hipMemcpyHostToDevice, g_stream));
   DH_CHECK_HIP("dh_upload", hipStreamSynchronize(g_stream));
-  return 0;
+  return dh::check_kernel_status("dh_upload");
 }
 
 int dh_download(void* host_dst, const void* d_src, size_t src_offset, size_t bytes) {
@@ -202,7 +224,7 @@ int dh_download(void* host_dst, const void* d_src, size_t src_offset, size_t byt
   DH_CHECK_HIP("dh_download", hipMemcpyAsync(host_dst, static_cast<const char*>(d_src) + src_offset,
                                              bytes, hipMemcpyDeviceToHost, g_stream));
   DH_CHECK_HIP("dh_download", hipStreamSynchronize(g_stream));
-  return 0;
+  return dh::check_kernel_status("dh_download");
 }
 
 int dh_copy(void* d_dst, size_t dst_offset, const void* d_src, size_t src_offset, size_t bytes) {
@@ -358,7 +380,7 @@ int dh_sync(void) {
   DH_REQUIRE_INIT("dh_sync");
   if (g_capturing) return dh::fail(1, "[dh_sync] not possible while a graph is being captured (it waits for the stream)");
   DH_CHECK_HIP("dh_sync", hipStreamSynchronize(g_stream));
-  return 0;
+  return dh::check_kernel_status("dh_sync");
 }
 
 }  // extern "C"

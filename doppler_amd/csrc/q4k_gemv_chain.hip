@@ -1,0 +1,806 @@
+// Chained Q4_K decode GEMVs: up to four dependent products of ONE activation row in a single launch,
+//
+//     x_0 given,   x_{p+1} = f_p( W_p . g_p(x_p) )            (p = 0 .. n-1)
+//
+// with g_p an optional RMSNorm of the input and f_p either  alpha * (.) + residual  or the gated pair
+// act(Wg . x) * (Wu . x) * alpha.  This is the dependent run of products between two attentions of a
+// decoder layer (o-projection, gate/up, down-projection, the next layer's q/k/v projection), which as
+// four launches costs four times the dispatch-to-first-byte floor of a launch with the HBM idle.
+//
+// One persistent workgroup of 16 waves per compute unit.  Every workgroup owns fixed row tiles of
+// every matrix; a work unit is one tile x one 256-weight super-block column (<= 16 rows x 144 bytes),
+// and the units of all phases form ONE sequence per workgroup that its waves draw from a counter in
+// LDS.  A wave keeps two units in flight (global_load_lds into its private two-stage ring), so the
+// weight stream runs on across a phase boundary: while the outputs of phase p travel between the
+// workgroups, the first 32 units per compute unit of phase p + 1 are already on their way into LDS.
+//
+// Exchange.  The wave that finishes a tile writes its outputs to C and, for every phase but the last,
+// publishes them as (value, sequence number) pairs with 8-byte device-scope stores (an 8-byte store
+// is single-copy atomic, so a reader that sees the number sees the value).  The consumers, every
+// workgroup for the whole vector, read the pairs with device-scope loads and retry until every number
+// is the one of this launch and phase.  No counters, no fences, no grid barrier; two buffers in
+// turn, so that a phase's outputs are never overwritten before every workgroup has consumed them
+// (a workgroup publishes phase p + 1 only after it has consumed phase p, and phase p + 2 can only be
+// published after every workgroup has published phase p + 1).  Every wait is bounded: a wave whose
+// wait runs into the limit stores a code in the library's status word and leaves, the other waves of
+// the workgroup follow, the other workgroups run into their own limits, and the host finds the code at
+// its next synchronisation.  The sequence numbers come from a launch counter in device memory that
+// the launch itself advances, so a captured graph can replay the launch.
+//
+// The arithmetic of a unit (int8 matrix cores over activations quantised per 32-element sub-block)
+// is that of q4k_gemv_i8.hip; the two share q4k_i8_device.h.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+
+#include "dh_common.h"
+#include "q4k_device.h"
+#include "q4k_i8_device.h"
+
+namespace {
+
+using dh::kBlockBytes;
+using dh::kQK;
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+
+constexpr int kWaves = 16;
+constexpr int kTileRows = 16;
+constexpr int kStage = kTileRows * kBlockBytes;   // 2304 bytes per ring stage
+constexpr int kUnitLoads = 3;                     // load instructions of a full unit: ceil(16 rows * 9 pieces / 64 lanes)
+constexpr int kDepth = 2;                         // ring stages per wave
+constexpr int kMaxPhases = DH_CHAIN_MAX_PHASES;
+constexpr int kSlots = 8;                         // tiles whose partial sums may be in LDS at once (a power of two)
+constexpr int kSlotShift = 3;
+constexpr int kZeroBytes = 144;                   // what a lane without an operand reads
+constexpr size_t kMaxLds = 160 * 1024;
+constexpr int kMaxChainN = 32768;                 // longest exchanged vector
+constexpr int kDefaultSpinLimit = 1 << 17;        // polls of one bounded wait
+constexpr int kColsPerPass = 3;                   // columns whose loads a wave has in flight at once in the prologue
+// counters in LDS: [0] next unit, [1 + s] units delivered to slot s, [1 + kSlots + s] tiles completed
+// in slot s, [1 + 2 kSlots] a wave has given up, [2 + 2 kSlots + p] tiles of phase p this workgroup has
+// finished, then the column flags of the two record areas
+constexpr int kCtrAbort = 1 + 2 * kSlots;
+constexpr int kCtrDone = 2 + 2 * kSlots;
+constexpr int kCtrFlags = kCtrDone + kMaxPhases;
+// a tile's partial sums are read four columns at a time: the last read may reach past the counters
+constexpr int kLdsPad = 1024;
+
+#define DH_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+// s_waitcnt with only the vector-memory counter set (6 bits, split 4 + 2 in the encoding).
+#define DH_WAIT_VM(k) __builtin_amdgcn_s_waitcnt(((k) & 0xF) | (((k) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+
+// Waits until at most n of this wave's vector-memory operations are outstanding (loads complete in
+// issue order).  Counts without a case wait for everything, which is always safe.
+__device__ __forceinline__ void wait_vm_at_most(int n) {
+  switch (n) {
+    case 1: DH_WAIT_VM(1); break;
+    case 2: DH_WAIT_VM(2); break;
+    case 3: DH_WAIT_VM(3); break;
+    case 4: DH_WAIT_VM(4); break;
+    case 5: DH_WAIT_VM(5); break;
+    case 6: DH_WAIT_VM(6); break;
+    default: DH_WAIT_VM(0); break;
+  }
+}
+
+struct Phase {
+  const uint8_t* W;            // Q4_K rows [N][nb]
+  const uint8_t* W2;           // second matrix of a gated pair, or null
+  float* C;                    // [N]
+  const float* residual;       // [N] or null
+  const float* norm_weight;    // [K] or null: RMSNorm of the phase's input
+  int N, K, nb, nmat;
+  int rows;                    // weight rows per tile (<= 16)
+  int nlw;                     // load instructions per unit: ceil(9 * rows / 64)
+  int upt;                     // units per tile: nb * nmat
+  int upt_mul;                 // ceil(2^24 / upt): u / upt == (u * upt_mul) >> 24 for the unit counts met here
+  int tiles_base, tiles_rem;   // tiles per workgroup: floor and remainder of tiles / grid
+  int activation, norm_weight_offset;
+  int wait_stores;             // a later phase reads this phase's C as its residual
+  float alpha, clamp_max, norm_eps;
+};
+
+struct ChainArgs {
+  Phase ph[kMaxPhases];
+  const float* x0;             // [K of phase 0]
+  v2u* ll;                     // [2][kMaxChainN] (value, sequence number)
+  uint32_t* epoch;             // launch counter (device memory)
+  uint32_t* status;            // the library's kernel status word
+  int nph;
+  int grid;                    // workgroups the tiles are dealt to (the launch may hold fewer: diagnostic)
+  int spin_limit;
+  int xq_bytes[2];             // bytes of the two record areas (phases 0, 2 / 1, 3)
+  int nb_max[2];               // columns of the two areas
+  int red_stride;              // floats per tile slot: 16 * the largest units-per-tile
+};
+
+__device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
+  uint32_t v;
+  asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(addr) : "memory");
+  return v;
+}
+
+#define DH_SEL4(p_, a0_, a1_, a2_, a3_) ((p_) == 0 ? (a0_) : (p_) == 1 ? (a1_) : (p_) == 2 ? (a2_) : (a3_))
+
+__global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const ChainArgs a) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int bid = blockIdx.x;
+
+  // ---- LDS: ring [16 waves][2][2304], record areas 0 and 1, zeros [144], partial sums
+  // [kSlots][red_stride], counters
+  unsigned char* ring = lds;
+  unsigned char* xq0 = ring + (size_t)kWaves * kDepth * kStage;
+  unsigned char* xq1 = xq0 + a.xq_bytes[0];
+  unsigned char* zeros = xq1 + a.xq_bytes[1];
+  float* red = reinterpret_cast<float*>(zeros + kZeroBytes);
+  unsigned* ctr = reinterpret_cast<unsigned*>(red + (size_t)kSlots * a.red_stride);
+  const int nflags = a.nb_max[0] + a.nb_max[1];
+  for (int i = tid; i < kCtrFlags + nflags; i += 64 * kWaves) ctr[i] = 0u;
+  if (tid >= 64 && tid < 64 + kZeroBytes / 4) reinterpret_cast<uint32_t*>(zeros)[tid - 64] = 0u;
+
+  const uint32_t seq_base = *a.epoch * 8u;       // phase p's outputs carry seq_base + p + 1
+  const int nph = a.nph;
+
+  // ---- this workgroup's unit and tile ranges: phase p holds units [ub_p, ub_{p+1}) and tile ordinals
+  // [tb_p, tb_{p+1}); its tiles are bid, bid + grid, ..
+  int ubv[kMaxPhases + 1], tbv[kMaxPhases + 1];
+  ubv[0] = 0;
+  tbv[0] = 0;
+#pragma unroll
+  for (int p = 0; p < kMaxPhases; p++) {
+    const int ntl = p < nph ? a.ph[p].tiles_base + (bid < a.ph[p].tiles_rem ? 1 : 0) : 0;
+    ubv[p + 1] = ubv[p] + ntl * (p < nph ? a.ph[p].upt : 0);
+    tbv[p + 1] = tbv[p] + ntl;
+  }
+  const int ub1 = ubv[1], ub2 = ubv[2], ub3 = ubv[3], total = ubv[4];
+  const int tb1 = tbv[1], tb2 = tbv[2], tb3 = tbv[3];
+  auto phase_of = [&](const int u) { return (u >= ub1 ? 1 : 0) + (u >= ub2 ? 1 : 0) + (u >= ub3 ? 1 : 0); };
+
+  unsigned char* my_ring = ring + (size_t)wave * kDepth * kStage;
+  const uint32_t ctr_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(ctr);
+  const uint32_t abort_addr = ctr_abs + 4 * kCtrAbort;
+  const uint32_t red_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(red);
+  const uint32_t xq_abs0 = (uint32_t)(uintptr_t)DH_LDS_PTR(xq0), xq_abs1 = (uint32_t)(uintptr_t)DH_LDS_PTR(xq1);
+
+  // A bounded wait ran into its limit: the wave lets its loads land, leaves the code where the host
+  // finds it, tells the other waves of the workgroup and ends.
+  auto give_up = [&](const uint32_t kind, const int phase) {
+    DH_WAIT_VM(0);
+    if (lane == 0) {
+      __hip_atomic_store(a.status, dh::kstatus_code(kind, (uint32_t)phase, (uint32_t)bid), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_SYSTEM);
+      ctr[kCtrAbort] = 1u;
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_endpgm();          // the wave ends here (no barrier follows)
+  };
+
+  // ---- issue side: the phase whose units are being requested
+  int ip = -1, i_rows = 0, i_N = 0, i_nb = 1, i_upt = 1, i_upt_mul = 0, i_ub = 0, i_nlw = 0;
+  const uint8_t* iW = nullptr;
+  const uint8_t* iW2 = nullptr;
+  int64_t i_row_bytes = 0;
+  uint32_t goff[kUnitLoads];       // piece t * 64 + lane of a unit: row p / 9, 16-byte piece p % 9 of that row's super-block
+#pragma unroll
+  for (int t = 0; t < kUnitLoads; t++) goff[t] = 0xFFFFFFFFu;
+  auto issue_setup = [&](const int p) {
+    ip = p;
+    const Phase& P = a.ph[p];
+    iW = P.W; iW2 = P.W2; i_rows = P.rows; i_N = P.N; i_nb = P.nb; i_upt = P.upt; i_upt_mul = P.upt_mul; i_nlw = P.nlw;
+    i_ub = DH_SEL4(p, 0, ub1, ub2, ub3);
+    i_row_bytes = (int64_t)P.nb * kBlockBytes;
+#pragma unroll
+    for (int t = 0; t < kUnitLoads; t++) {
+      const int q = t * 64 + lane, r = q / 9;
+      goff[t] = q < 9 * i_rows ? (uint32_t)(r * i_row_bytes + (q - r * 9) * 16) : 0xFFFFFFFFu;
+    }
+  };
+  // Puts the loads of unit u in flight into ring stage `stage`; returns the number of load instructions.
+  auto issue = [&](const int u, const int stage) -> int {
+    const int p = phase_of(u);
+    if (p != ip) issue_setup(p);
+    const int local = u - i_ub;
+    const int tl = (int)(((unsigned)local * (unsigned)i_upt_mul) >> 24);
+    const int r = local - tl * i_upt;
+    const int mat = r >= i_nb ? 1 : 0;
+    const int col = r - mat * i_nb;
+    const int tile = bid + tl * a.grid;
+    const uint8_t* base = (mat ? iW2 : iW) + (int64_t)tile * i_rows * i_row_bytes + (int64_t)col * kBlockBytes;
+    unsigned char* st = my_ring + stage * kStage;
+    const int rows_left = i_N - tile * i_rows;
+    if (rows_left >= i_rows) {
+#pragma unroll
+      for (int t = 0; t < kUnitLoads; t++) {
+        if (goff[t] != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + goff[t], DH_LDS_PTR(st + t * 1024), 16, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < kUnitLoads; t++) {
+        const int q = t * 64 + lane, rr = q / 9;
+        const int64_t o = (int64_t)min(rr, rows_left - 1) * i_row_bytes + (q - rr * 9) * 16;
+        if (goff[t] != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + o, DH_LDS_PTR(st + t * 1024), 16, 0, 0);
+      }
+    }
+    return i_nlw;
+  };
+
+  // ---- the prologue of phase p: this wave's share of the phase's activations, columns
+  // (wave - bid) mod 16, + 16, .. (rotated by workgroup so that the workgroups do not all ask for the
+  // same lines at the same moment), kColsPerPass of them per pass.  Lane t holds elements 4t .. 4t+3 of
+  // a column.  Phase 0 reads x0, written before the launch; later phases read the pairs the other
+  // workgroups publish and retry until every sequence number is the expected one.
+  struct Cols {
+    v4f xr[kColsPerPass], wr[kColsPerPass];
+  };
+  const int c_first = (wave - bid) & (kWaves - 1);
+  auto load_norm = [&](const Phase& P, const int c0, Cols& R) {
+    if (P.norm_weight == nullptr) return;
+#pragma unroll
+    for (int i = 0; i < kColsPerPass; i++) {
+      const int c = c0 + kWaves * i;
+      if (c < P.nb) {
+        const float* q = P.norm_weight + c * kQK + 4 * lane;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(R.wr[i]) : "v"(q) : "memory");
+      }
+    }
+  };
+  auto load_x0 = [&](const Phase& P, const int c0, Cols& R) {
+#pragma unroll
+    for (int i = 0; i < kColsPerPass; i++) {
+      const int c = c0 + kWaves * i;
+      if (c < P.nb) {
+        const float* q = a.x0 + c * kQK + 4 * lane;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(R.xr[i]) : "v"(q) : "memory");
+      }
+    }
+  };
+  // Quantises the columns of a pass (their values have landed) and raises their flags.
+  auto finish_pass = [&](const int p, const Phase& P, const int c0, Cols& R) {
+    const bool norm = P.norm_weight != nullptr;
+    unsigned char* xq = (p & 1) ? xq1 : xq0;
+    unsigned* flags = ctr + kCtrFlags + ((p & 1) ? a.nb_max[0] : 0);
+#pragma unroll
+    for (int i = 0; i < kColsPerPass; i++) {
+      const int c = c0 + kWaves * i;
+      if (c < P.nb) {
+        asm volatile("" : "+v"(R.xr[i]));
+        if (norm) asm volatile("" : "+v"(R.wr[i]));
+        float v[4], ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          v[e] = R.xr[i][e];
+          if (norm) {
+            ss = fmaf(v[e], v[e], ss);
+            v[e] *= P.norm_weight_offset ? 1.0f + R.wr[i][e] : R.wr[i][e];
+          }
+        }
+        unsigned char* rec = xq + (size_t)c * kRec;
+        i8_quantise_store(v, rec, lane);
+        if (norm) ss = dh::wave_sum_uniform(ss);
+        // LDS executes a wave's operations in order: whoever sees the flag sees the record
+        if (lane == 0) {
+          reinterpret_cast<float*>(rec)[kRecSsq / 4] = ss;
+          flags[c] = (unsigned)p + 1u;
+        }
+      }
+    }
+  };
+  // Phases after the first.
+  auto prologue = [&](const int p) {
+    const Phase& P = a.ph[p];
+    const int nb = P.nb;
+    const v2u* src = a.ll + (size_t)((p - 1) & 1) * kMaxChainN;
+    const uint32_t want = seq_base + (uint32_t)p;
+    // Not before this workgroup has finished its own tiles of the previous phase: the workgroups run
+    // the same work at the same pace, so until then the others have not finished theirs either, and
+    // polls that cannot succeed yet would only compete with the weight stream for the memory system.
+    {
+      const unsigned mine = (unsigned)(DH_SEL4(p, 0, tb1, tb2 - tb1, tb3 - tb2));
+      const uint32_t done_addr = ctr_abs + 4 * (kCtrDone + p - 1);
+      int spins = 0;
+#ifndef DH_CHAIN_EXP_NOWAIT
+      while (__builtin_amdgcn_readfirstlane(lds_read_u32(done_addr)) < mine) {
+        if (++spins > a.spin_limit * 8 || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u)
+          give_up(DH_KSTATUS_SLOT_WAIT, p);
+        __builtin_amdgcn_s_sleep(4);
+      }
+#endif
+    }
+#pragma unroll 1
+    for (int c0 = c_first; c0 < nb; c0 += kWaves * kColsPerPass) {
+      Cols R;
+      v4u la[kColsPerPass], lb[kColsPerPass];
+      load_norm(P, c0, R);
+      int spins = 0;
+      for (;;) {
+#pragma unroll
+        for (int i = 0; i < kColsPerPass; i++) {
+          const int c = c0 + kWaves * i;
+          if (c < nb) {
+            const v2u* q = src + c * kQK + 4 * lane;
+            asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1"
+                         : "=&v"(la[i]), "=&v"(lb[i]) : "v"(q) : "memory");
+          }
+        }
+        DH_WAIT_VM(0);
+        bool ok = true;
+#pragma unroll
+        for (int i = 0; i < kColsPerPass; i++) {
+          const int c = c0 + kWaves * i;
+          if (c < nb) {
+            asm volatile("" : "+v"(la[i]), "+v"(lb[i]));
+            ok = ok && la[i].y == want && la[i].w == want && lb[i].y == want && lb[i].w == want;
+          }
+        }
+#ifdef DH_CHAIN_EXP_NOWAIT
+        break;
+#endif
+        if (__builtin_amdgcn_ballot_w64(!ok) == 0ull) break;
+        if (++spins > a.spin_limit || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) {
+          give_up(DH_KSTATUS_EXCHANGE_WAIT, p);
+        }
+        __builtin_amdgcn_s_sleep(8);
+      }
+#pragma unroll
+      for (int i = 0; i < kColsPerPass; i++)
+        R.xr[i] = v4f{__uint_as_float(la[i].x), __uint_as_float(la[i].z), __uint_as_float(lb[i].x), __uint_as_float(lb[i].z)};
+      finish_pass(p, P, c0, R);
+    }
+  };
+
+  // the first pass of phase 0: its loads go out before the barrier and before any weights, so that
+  // they are at the head of the compute unit's memory queue
+  Cols first;
+  load_norm(a.ph[0], c_first, first);
+  load_x0(a.ph[0], c_first, first);
+
+  // counters, flags and the zero area are in place
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  if (total == 0) return;
+
+  // Draws the next unit of the workgroup (wave-uniform result).
+  auto draw = [&]() -> int {
+    unsigned v = 0;
+    if (lane == 0)
+      asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(ctr_abs), "v"(1u) : "memory");
+    return (int)__builtin_amdgcn_readfirstlane(v);
+  };
+
+  // ---- the first two units' loads go out before anything else is waited for
+  int u_st0 = 0x7fffffff, u_st1 = 0x7fffffff;     // units in the two ring stages (>= total: none)
+  int nl_st0 = 0, nl_st1 = 0;                      // their load instruction counts
+  u_st0 = draw();
+  if (u_st0 < total) {
+    nl_st0 = issue(u_st0, 0);
+    u_st1 = draw();
+    if (u_st1 < total) nl_st1 = issue(u_st1, 1);
+  }
+  // phase 0's activations: only they are waited for (the units were requested behind them)
+  wait_vm_at_most(nl_st0 + nl_st1);
+  finish_pass(0, a.ph[0], c_first, first);
+#pragma unroll 1
+  for (int c0 = c_first + kWaves * kColsPerPass; c0 < a.ph[0].nb; c0 += kWaves * kColsPerPass) {
+    load_norm(a.ph[0], c0, first);
+    load_x0(a.ph[0], c0, first);
+    DH_WAIT_VM(0);
+    finish_pass(0, a.ph[0], c0, first);
+  }
+
+  // operand addressing (see q4k_gemv_i8.hip): MFMA pair cc covers sub-blocks 4cc .. 4cc+3; lane
+  // (i = lane & 15, kg) supplies operand row i = 4g + digit: 16 digit bytes where its row's sub-block is
+  // the one its k-slots hold, zeros elsewhere and in the fourth row of every group
+  const int j = lane & 15, kg = lane >> 4;
+  uint32_t a_mul[2], a_off[2];                  // operand address = record * a_mul + a_off (+ 128 cc)
+  {
+    const int g = j >> 2, dg = j & 3;
+    const uint32_t zero_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(zeros);
+    const uint32_t data_off = 256 * min(dg, 2) + 32 * g + 16 * (kg & 1);
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const bool has = dg < 3 && (g >> 1) == (kg >> 1) && (g & 1) == h;
+      a_mul[h] = has ? 1u : 0u;
+      a_off[h] = has ? data_off : zero_abs;
+    }
+  }
+  const uint32_t lane_hdr = (uint32_t)(uintptr_t)DH_LDS_PTR(my_ring) + (uint32_t)j * kBlockBytes;
+  const uint32_t lane_q = lane_hdr + 16 + 32 * (kg >> 1) + 16 * (kg & 1);
+  const uint32_t sh_lo = 8 * kg;           // bit offset of this lane's byte in the header words
+
+  // ---- process side: the phase whose units are being multiplied
+  int pp = -1, p_nb = 1, p_upt = 1, p_upt_mul = 0, p_ub = 0, p_tb = 0, p_dual = 0;
+  uint32_t p_xq = 0, p_flags = 0;
+  int my_phase = 0;                        // prologues this wave has done: phases 0 .. my_phase
+  int rms_phase = -1;                      // phase inv_rms belongs to
+  float inv_rms = 1.f;
+
+  int cstage = 0;
+#pragma unroll 1
+  for (;;) {
+    const int cur = cstage ? u_st1 : u_st0;
+    if (cur >= total) break;              // draws only grow: nothing behind this one either
+    const int p = phase_of(cur);
+    if (p != pp) {
+      pp = p;
+      const Phase& P = a.ph[p];
+      p_nb = P.nb; p_upt = P.upt; p_upt_mul = P.upt_mul; p_dual = P.nmat - 1;
+      p_ub = DH_SEL4(p, 0, ub1, ub2, ub3);
+      p_tb = DH_SEL4(p, 0, tb1, tb2, tb3);
+      p_xq = (p & 1) ? xq_abs1 : xq_abs0;
+      p_flags = ctr_abs + 4 * (kCtrFlags + ((p & 1) ? a.nb_max[0] : 0));
+    }
+    // this wave's share of the activations of every phase up to the unit's
+    while (my_phase < p) prologue(++my_phase);
+
+    const int local = cur - p_ub;
+    const int tl = (int)(((unsigned)local * (unsigned)p_upt_mul) >> 24);
+    const int rr = local - tl * p_upt;
+    const int mat = (p_dual && rr >= p_nb) ? 1 : 0;
+    const int col = rr - mat * p_nb;
+    const int tord = p_tb + tl;                       // tile ordinal of the workgroup, over all phases
+    const int slot = tord & (kSlots - 1);
+    // draw the unit that will go into this stage once it has been read (the answer is collected with
+    // the reads below)
+    unsigned nxt = 0;
+    if (lane == 0) asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=&v"(nxt) : "v"(ctr_abs), "v"(1u) : "memory");
+    // the other stage's loads were issued after this one's
+    wait_vm_at_most(cstage ? nl_st0 : nl_st1);
+    const uint32_t hp = lane_hdr + cstage * kStage, qp = lane_q + cstage * kStage;
+    const uint32_t rec = p_xq + (uint32_t)col * kRec;
+    const uint32_t gen_addr = ctr_abs + 4 * (1 + kSlots + slot);
+    const uint32_t flag_addr = p_flags + 4 * col;
+    v4u h, q0, q1;
+    v4i ax[2][2];
+    v2f sx, xinv;
+    uint32_t gen, flag;
+    asm volatile(
+        "ds_read_b32 %4, %8\n\t"
+        "ds_read_b128 %0, %5\n\t"
+        "ds_read_b128 %1, %6\n\t"
+        "ds_read_b128 %2, %6 offset:64\n\t"
+        "ds_read_b32 %3, %7"
+        : "=&v"(h), "=&v"(q0), "=&v"(q1), "=&v"(gen), "=&v"(flag)
+        : "v"(hp), "v"(qp), "v"(gen_addr), "v"(flag_addr)
+        : "memory");
+    // the column's operands, read at once on the expectation that its flag is up; re-read below if it was not
+#define DH_READ_OPERANDS()                                                                        \
+    do {                                                                                          \
+      const uint32_t pa = rec * a_mul[0] + a_off[0], pb = rec * a_mul[1] + a_off[1], ps = rec + kRecSums + 4 * kg; \
+      asm volatile(                                                                               \
+          "ds_read_b128 %0, %6\n\t"                                                               \
+          "ds_read_b128 %1, %7\n\t"                                                               \
+          "ds_read_b128 %2, %6 offset:128\n\t"                                                    \
+          "ds_read_b128 %3, %7 offset:128\n\t"                                                    \
+          "ds_read2_b32 %4, %8 offset1:4\n\t"                                                     \
+          "ds_read2_b32 %5, %8 offset0:8 offset1:12"                                              \
+          : "=&v"(ax[0][0]), "=&v"(ax[0][1]), "=&v"(ax[1][0]), "=&v"(ax[1][1]), "=&v"(sx), "=&v"(xinv) \
+          : "v"(pa), "v"(pb), "v"(ps)                                                             \
+          : "memory");                                                                            \
+    } while (0)
+#define DH_TIE_OPERANDS() asm volatile("" : "+v"(ax[0][0]), "+v"(ax[0][1]), "+v"(ax[1][0]), "+v"(ax[1][1]), "+v"(sx), "+v"(xinv))
+    DH_READ_OPERANDS();
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(h), "+v"(q0), "+v"(q1), "+v"(gen), "+v"(flag), "+v"(nxt) :: "memory");
+    DH_TIE_OPERANDS();
+    const uint32_t flag_want = (uint32_t)p + 1u;
+    if (__builtin_amdgcn_readfirstlane(flag) != flag_want) {
+      int spins = 0;
+      do {
+        __builtin_amdgcn_s_sleep(2);
+        flag = lds_read_u32(flag_addr);
+        if (++spins > a.spin_limit * 8 || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) break;
+      } while (__builtin_amdgcn_readfirstlane(flag) != flag_want);
+      if (__builtin_amdgcn_readfirstlane(flag) != flag_want) {
+        give_up(DH_KSTATUS_COLUMN_WAIT, p);
+      }
+      DH_READ_OPERANDS();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      DH_TIE_OPERANDS();
+    }
+#undef DH_READ_OPERANDS
+#undef DH_TIE_OPERANDS
+    // the stage is free again: put the loads of the unit drawn above in flight
+    {
+      const int u = (int)__builtin_amdgcn_readfirstlane(nxt);
+      const int nl = u < total ? issue(u, cstage) : 0;
+      if (cstage) { u_st1 = u; nl_st1 = nl; } else { u_st0 = u; nl_st0 = nl; }
+    }
+    cstage ^= 1;
+
+    // 6-bit scales and mins of sub-blocks kg and 4 + kg of this lane's weight row
+    const int sc_a = (int)((h.y >> sh_lo) & 63u);
+    const int sc_b = (int)(((h.w >> sh_lo) & 15u) | (((h.y >> (sh_lo + 6)) & 3u) << 4));
+    const float mn_a = (float)((h.z >> sh_lo) & 63u);
+    const float mn_b = (float)(((h.w >> (sh_lo + 4)) & 15u) | (((h.z >> (sh_lo + 6)) & 3u) << 4));
+    const float d = f16lo(h.x), dmin = f16hi(h.x);
+    v4i blo[2], bhi[2];
+#pragma unroll
+    for (int cc = 0; cc < 2; cc++) {
+      const v4u q = cc ? q1 : q0;
+      blo[cc] = v4i{(int)(q.x & 0x0F0F0F0Fu), (int)(q.y & 0x0F0F0F0Fu), (int)(q.z & 0x0F0F0F0Fu),
+                    (int)(q.w & 0x0F0F0F0Fu)};
+      bhi[cc] = v4i{(int)((q.x >> 4) & 0x0F0F0F0Fu), (int)((q.y >> 4) & 0x0F0F0F0Fu),
+                    (int)((q.z >> 4) & 0x0F0F0F0Fu), (int)((q.w >> 4) & 0x0F0F0F0Fu)};
+    }
+    // wait (never, in practice) until the tile that used this slot kSlots tiles ago is written out
+    {
+      const unsigned want = (unsigned)tord >> kSlotShift;
+      int spins = 0;
+      while (__builtin_amdgcn_readfirstlane(gen) != want) {
+        __builtin_amdgcn_s_sleep(1);
+        gen = lds_read_u32(gen_addr);
+        if (++spins > a.spin_limit * 8 || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) break;
+      }
+      if (__builtin_amdgcn_readfirstlane(gen) != want) {
+        give_up(DH_KSTATUS_SLOT_WAIT, p);
+      }
+    }
+    v4i dd[2];
+#pragma unroll
+    for (int cc = 0; cc < 2; cc++) {
+      v4i t = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[cc][0], blo[cc], v4i{0, 0, 0, 0}, 0, 0, 0);
+      dd[cc] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[cc][1], bhi[cc], t, 0, 0, 0);
+    }
+    // the four lane groups hold different sub-blocks of the same 16 rows
+    const float sres = sum_lane_groups(i8_unit_term(dd[0], dd[1], sc_a, sc_b, mn_a, mn_b, d, dmin, sx, xinv));
+    if (lane < 16) red[(size_t)slot * a.red_stride + (mat * p_nb + col) * 16 + lane] = sres;
+
+    // ---- deliver.  LDS executes a wave's operations in order, so the partial sums above are in
+    // place before the count below is; the wave that delivers a tile's last unit finishes it.
+    unsigned arrived = 0;
+    if (lane == 0)
+      asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                   : "=&v"(arrived) : "v"(ctr_abs + 4 * (1 + slot)), "v"(1u) : "memory");
+    arrived = __builtin_amdgcn_readfirstlane(arrived);
+    if ((int)arrived == p_upt - 1) {
+      const Phase& P = a.ph[p];
+      const int nb = p_nb;
+      const int tile = bid + tl * a.grid;
+      const int64_t row = (int64_t)tile * P.rows + j;
+      const uint32_t slot_abs = red_abs + (uint32_t)slot * a.red_stride * 4;
+      // lane (j, kg) adds columns kg, kg + 4, .. (four reads in flight at a time); the four groups then
+      // meet.  The order is fixed, so the result does not depend on who arrives last.
+      float sg = 0.f, su = 0.f;
+      for (int c = kg; c < nb; c += 16) {
+        float r[2][4];
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) {
+          if (mt == 0 || p_dual) {
+            const uint32_t q = slot_abs + ((mt * nb + c) * 16 + j) * 4;
+            asm volatile(
+                "ds_read_b32 %0, %4\n\t"
+                "ds_read_b32 %1, %4 offset:256\n\t"
+                "ds_read_b32 %2, %4 offset:512\n\t"
+                "ds_read_b32 %3, %4 offset:768"
+                : "=&v"(r[mt][0]), "=&v"(r[mt][1]), "=&v"(r[mt][2]), "=&v"(r[mt][3])
+                : "v"(q)
+                : "memory");
+          } else {
+            r[mt][0] = r[mt][1] = r[mt][2] = r[mt][3] = 0.f;
+          }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]) :: "memory");
+        asm volatile("" : "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]));
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const bool ok = c + 4 * i < nb;       // columns past the last read whatever follows: dropped
+          sg += ok ? r[0][i] : 0.f;
+          su += ok ? r[1][i] : 0.f;
+        }
+      }
+      sg = sum_lane_groups(sg);
+      su = sum_lane_groups(su);
+      if (P.norm_weight != nullptr) {
+        if (rms_phase != p) {
+          // every column has been consumed by now, so every column's sum of squares is in place
+          float tot = 0.f;
+          for (int c = 0; c < nb; c++) tot += __uint_as_float(lds_read_u32(p_xq + (uint32_t)c * kRec + kRecSsq));
+          inv_rms = 1.0f / sqrtf(tot / (float)P.K + P.norm_eps);
+          rms_phase = p;
+        }
+        sg *= inv_rms;
+        su *= inv_rms;
+      }
+      const bool last_phase = p == nph - 1;
+      if (kg == 0 && j < P.rows && row < P.N) {
+        float v;
+        if (p_dual) {
+          const float act = P.activation == DH_ACT_SILU ? act_silu(sg) : act_gelu(sg);
+          v = act * su * P.alpha;
+          if (P.activation == DH_ACT_SILU && P.clamp_max > 0.f) v = fminf(fmaxf(v, -P.clamp_max), P.clamp_max);
+        } else {
+          v = sg * P.alpha;
+          // device-scope load: an earlier phase of this launch may have written the residual
+          if (P.residual) v += __hip_atomic_load(const_cast<float*>(P.residual) + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __hip_atomic_store(P.C + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (!last_phase) {
+          v2u pr;
+          pr.x = __float_as_uint(v);
+          pr.y = seq_base + (uint32_t)p + 1u;
+          v2u* dst = a.ll + (size_t)(p & 1) * kMaxChainN + row;
+          asm volatile("global_store_dwordx2 %0, %1, off sc1" :: "v"(dst), "v"(pr) : "memory");
+        }
+      }
+      // a later phase reads these outputs as its residual: they are in memory before this wave goes on
+      if (P.wait_stores) DH_WAIT_VM(0);
+      // slot free for the tile kSlots further on (after the reads above: same wave, in order)
+      if (lane == 0) {
+        ctr[1 + slot] = 0u;
+        ctr[1 + kSlots + slot] = ((unsigned)tord >> kSlotShift) + 1u;
+        unsigned was;
+        asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(was) : "v"(ctr_abs + 4 * (kCtrDone + p)), "v"(1u) : "memory");
+      }
+      // the launch counter moves on once: the workgroup that owns the last phase's first tile does it
+      if (last_phase && bid == 0 && tl == 0 && lane == 0) *a.epoch = (seq_base >> 3) + 1u;
+    }
+  }
+  // a wave that drew no unit of the later phases still owes the other waves its columns of them
+  while (my_phase < nph - 1) prologue(++my_phase);
+}
+
+// ---- host side ----------------------------------------------------------------------------------
+v2u* g_ll = nullptr;          // exchange pairs, 2 x kMaxChainN
+uint32_t* g_epoch = nullptr;  // launch counter
+bool g_coresident = false;
+
+struct Plan {
+  ChainArgs a;
+  size_t lds;
+};
+
+int make_plan(const char* op, const float* d_x0, const dh_chain_phase* ph, int n, Plan* out) {
+  if (n < 1 || n > kMaxPhases) return dh::fail(1, "[%s] a chain holds 1..%d products, got %d", op, kMaxPhases, n);
+  if (!d_x0 || !ph) return dh::fail(1, "[%s] null pointer", op);
+  if (reinterpret_cast<uintptr_t>(d_x0) & 15) return dh::fail(1, "[%s] x0 must be 16-byte aligned", op);
+  ChainArgs& a = out->a;
+  memset(&a, 0, sizeof(a));
+  const int ncu = dh::num_cus();
+  a.grid = ncu;
+  a.nph = n;
+  a.x0 = d_x0;
+  a.ll = g_ll;
+  a.epoch = g_epoch;
+  a.status = dh::kernel_status_word();
+  a.spin_limit = kDefaultSpinLimit;
+  int max_upt = 0, min_upt = 1 << 30;
+  for (int p = 0; p < n; p++) {
+    const dh_chain_phase& s = ph[p];
+    Phase& P = a.ph[p];
+    if (s.N <= 0 || s.K <= 0) return dh::fail(1, "[%s] product %d: dimensions must be positive: N=%d, K=%d", op, p, s.N, s.K);
+    if (s.K % kQK) return dh::fail(1, "[%s] product %d: K=%d must be a multiple of 256 in a chain", op, p, s.K);
+    if (p > 0 && s.K != ph[p - 1].N)
+      return dh::fail(1, "[%s] product %d takes K=%d inputs but product %d makes N=%d outputs", op, p, s.K, p - 1, ph[p - 1].N);
+    if (s.N > kMaxChainN || s.K > kMaxChainN) return dh::fail(1, "[%s] product %d: N and K are limited to %d in a chain", op, p, kMaxChainN);
+    if (!s.d_W || !s.d_C) return dh::fail(1, "[%s] product %d: null pointer", op, p);
+    if ((reinterpret_cast<uintptr_t>(s.d_W) | reinterpret_cast<uintptr_t>(s.d_W2)) & 15)
+      return dh::fail(1, "[%s] product %d: weight pointers must be 16-byte aligned", op, p);
+    if (s.d_norm_weight && (reinterpret_cast<uintptr_t>(s.d_norm_weight) & 15))
+      return dh::fail(1, "[%s] product %d: the norm weights must be 16-byte aligned", op, p);
+    if (s.d_W2 && s.activation != DH_ACT_SILU && s.activation != DH_ACT_GELU)
+      return dh::fail(1, "[%s] product %d: unknown activation %d", op, p, s.activation);
+    if (s.d_W2 && s.d_residual) return dh::fail(1, "[%s] product %d: a gated pair takes no residual", op, p);
+    P.W = static_cast<const uint8_t*>(s.d_W);
+    P.W2 = static_cast<const uint8_t*>(s.d_W2);
+    P.C = s.d_C;
+    P.residual = s.d_residual;
+    P.norm_weight = s.d_norm_weight;
+    P.N = s.N; P.K = s.K; P.nb = s.K / kQK; P.nmat = s.d_W2 ? 2 : 1;
+    P.activation = s.activation; P.norm_weight_offset = s.norm_weight_offset;
+    P.alpha = s.alpha; P.clamp_max = s.swiglu_limit; P.norm_eps = s.norm_eps;
+    // rows per tile: the largest count <= 16 that gives every workgroup the same number of tiles
+    const int per_cu = (int)dh::ceil_div(s.N, (int64_t)ncu * kTileRows);
+    P.rows = std::max(1, std::min(kTileRows, (int)dh::ceil_div(s.N, (int64_t)ncu * per_cu)));
+    P.nlw = (9 * P.rows + 63) / 64;
+    const int64_t ntiles = dh::ceil_div(s.N, P.rows);
+    P.upt = P.nb * P.nmat;
+    P.upt_mul = (int)(((1u << 24) + (unsigned)P.upt - 1) / (unsigned)P.upt);
+    P.tiles_base = (int)(ntiles / ncu);
+    P.tiles_rem = (int)(ntiles % ncu);
+    const int64_t units = (int64_t)(P.tiles_base + (P.tiles_rem ? 1 : 0)) * P.upt;
+    // the division by multiplication is exact while units * (upt_mul * upt - 2^24) < 2^24
+    if (units * ((int64_t)P.upt_mul * P.upt - (1 << 24)) >= (1 << 24) || units >= (1 << 20))
+      return dh::fail(1, "[%s] product %d: N=%d, K=%d is too large for a chain", op, p, s.N, s.K);
+    max_upt = std::max(max_upt, P.upt);
+    min_upt = std::min(min_upt, P.upt);
+    a.nb_max[p & 1] = std::max(a.nb_max[p & 1], P.nb);
+    // outputs that a later product reads back as its residual must have reached memory by then
+    for (int q = p + 1; q < n; q++)
+      if (ph[q].d_residual == s.d_C) P.wait_stores = 1;
+    // a product may not overwrite what an earlier or later one of the launch still reads elsewhere
+    if (s.d_C == d_x0) return dh::fail(1, "[%s] product %d writes over the chain's input", op, p);
+  }
+  // the units in flight (16 waves x 3 draws) must not span more tiles than there are slots
+  if ((kWaves * (kDepth + 1) + min_upt - 1) / min_upt + 2 > kSlots)
+    return dh::fail(1, "[%s] K=%d is too short for a chain (at least 2048)", op, min_upt * kQK);
+  a.xq_bytes[0] = a.nb_max[0] * kRec;
+  a.xq_bytes[1] = a.nb_max[1] * kRec;
+  a.red_stride = 16 * max_upt;
+  out->lds = (size_t)kWaves * kDepth * kStage + a.xq_bytes[0] + a.xq_bytes[1] + kZeroBytes +
+             sizeof(float) * kSlots * a.red_stride + sizeof(unsigned) * (kCtrFlags + a.nb_max[0] + a.nb_max[1]) + kLdsPad;
+  if (out->lds > kMaxLds)
+    return dh::fail(1, "[%s] the chain's activations do not fit the LDS (%zu of %zu bytes)", op, out->lds, kMaxLds);
+  return 0;
+}
+
+int launch(const char* op, Plan& plan, int workgroups) {
+  auto kern = q4k_gemv_chain_kernel;
+  static bool attr_set = false;
+  if (!attr_set) {
+    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)kMaxLds));
+    // the workgroups wait for each other: every one of them must be resident at once
+    int per_cu = 0;
+    DH_CHECK_HIP(op, hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kern), 64 * kWaves,
+                                                                  kMaxLds));
+    g_coresident = per_cu >= 1;
+    attr_set = true;
+  }
+  if (!g_coresident) return dh::fail(1, "[%s] the device cannot hold one workgroup of the chain per compute unit", op);
+  hipLaunchKernelGGL(kern, dim3(workgroups), dim3(64 * kWaves), plan.lds, dh::stream(), plan.a);
+  DH_CHECK_LAUNCH(op);
+  return 0;
+}
+
+}  // namespace
+
+namespace dh {
+
+int gemv_chain_init(int) {
+  DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_ll), (size_t)2 * kMaxChainN * sizeof(v2u)));
+  DH_CHECK_HIP("dh_init", hipMalloc(reinterpret_cast<void**>(&g_epoch), 256));
+  DH_CHECK_HIP("dh_init", hipMemset(g_ll, 0, (size_t)2 * kMaxChainN * sizeof(v2u)));
+  const uint32_t one = 1u;
+  DH_CHECK_HIP("dh_init", hipMemcpy(g_epoch, &one, 4, hipMemcpyHostToDevice));
+  return 0;
+}
+
+void gemv_chain_release() {
+  if (g_ll) (void)hipFree(g_ll);
+  if (g_epoch) (void)hipFree(g_epoch);
+  g_ll = nullptr;
+  g_epoch = nullptr;
+}
+
+// After a launch that gave up: sequence numbers of the abandoned launch may be anywhere in the
+// exchange area and the counter has not moved on; start over (the stream is idle when this runs).
+void gemv_chain_reset() {
+  if (!g_ll) return;
+  (void)hipMemset(g_ll, 0, (size_t)2 * kMaxChainN * sizeof(v2u));
+  uint32_t e = 0;
+  if (hipMemcpy(&e, g_epoch, 4, hipMemcpyDeviceToHost) != hipSuccess) e = 0;
+  e += 2u;
+  (void)hipMemcpy(g_epoch, &e, 4, hipMemcpyHostToDevice);
+}
+
+}  // namespace dh
+
+extern "C" {
+
+int dh_q4k_gemv_chain(const float* d_x0, const dh_chain_phase* phases, int n_phases) {
+  const char* op = "dh_q4k_gemv_chain";
+  DH_REQUIRE_INIT(op);
+  Plan plan;
+  if (int rc = make_plan(op, d_x0, phases, n_phases, &plan)) return rc;
+  return launch(op, plan, plan.a.grid);
+}
+
+int dh_q4k_gemv_chain_limited(const float* d_x0, const dh_chain_phase* phases, int n_phases, int workgroups,
+                              int spin_limit) {
+  const char* op = "dh_q4k_gemv_chain_limited";
+  DH_REQUIRE_INIT(op);
+  Plan plan;
+  if (int rc = make_plan(op, d_x0, phases, n_phases, &plan)) return rc;
+  if (workgroups < 1 || workgroups > plan.a.grid)
+    return dh::fail(1, "[%s] workgroups must be 1..%d", op, plan.a.grid);
+  if (spin_limit < 1 || spin_limit > kDefaultSpinLimit) return dh::fail(1, "[%s] spin_limit must be 1..%d", op, kDefaultSpinLimit);
+  plan.a.spin_limit = spin_limit;
+  return launch(op, plan, workgroups);
+}
+
+}  // extern "C"

@@ -32,6 +32,7 @@
 
 #include "dh_common.h"
 #include "q4k_device.h"
+#include "q4k_i8_device.h"
 
 namespace {
 
@@ -49,9 +50,9 @@ constexpr int kStage = kTileRows * kBlockBytes;   // 2304 bytes per ring stage
 constexpr int kUnitLoads = 3;                     // load instructions of a full unit: ceil(16 rows * 9 pieces / 64 lanes)
 constexpr int kMaxDepth = 3;
 constexpr int kMaxSlots = 32;                     // tiles whose partial sums may be in LDS at once
-constexpr int kRec = 832;                         // bytes per (column, activation row): 3 digit planes, 8 sums, 2^-E
 constexpr int kZeroBytes = 144;                   // what a lane without an operand reads
 constexpr size_t kMaxLds = 160 * 1024;
+constexpr int kSpinLimit = 1 << 18;               // polls of a wait inside the workgroup before the wave gives up
 
 #define DH_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 // s_waitcnt with only the vector-memory counter set (6 bits, split 4 + 2 in the encoding).
@@ -88,39 +89,8 @@ struct I8Args {
   int nslots, slot_shift;   // tile slots for partial sums: a power of two, and its log2
   int c_f16, activation, norm_weight_offset;
   float alpha, clamp_max, norm_eps;
+  uint32_t* status;      // the library's kernel status word (host memory the device can write)
 };
-
-// Largest value across the wave, wave-uniform (DPP inside the 16-lane rows, then scalar).
-__device__ __forceinline__ float wave_max_uniform(float v) {
-  auto shr = [](float x, auto ctrl) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(x), __float_as_int(x), decltype(ctrl)::value, 0xF, 0xF, false));
-  };
-  v = fmaxf(v, shr(v, std::integral_constant<int, 0x111>{}));
-  v = fmaxf(v, shr(v, std::integral_constant<int, 0x112>{}));
-  v = fmaxf(v, shr(v, std::integral_constant<int, 0x114>{}));
-  v = fmaxf(v, shr(v, std::integral_constant<int, 0x118>{}));
-  const int b = __float_as_int(v);
-  return fmaxf(fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 15)), __int_as_float(__builtin_amdgcn_readlane(b, 31))),
-               fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 47)), __int_as_float(__builtin_amdgcn_readlane(b, 63))));
-}
-
-// Sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48, left in all of them.
-__device__ __forceinline__ float sum_lane_groups(float v) {
-  const uint32_t u = __float_as_uint(v);
-  auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
-  const uint32_t w = __float_as_uint(v);
-  auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
-  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
-}
-
-// Sum over aligned groups of 8 lanes, left in all of them.
-__device__ __forceinline__ int sum8_i32(int v) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);    // quad_perm [1,0,3,2]
-  v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);    // quad_perm [2,3,0,1]
-  v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, false);   // row_half_mirror
-  return v;
-}
 
 // One LDS word read by hand (the compiler puts a wait for every weight load in flight in front of
 // its own LDS reads, because those loads write LDS too).
@@ -133,11 +103,11 @@ __device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
 // Layout of the dynamic LDS block, in this order:
 //   ring   [16 waves][depth][2304]
 //   xq     [nb][MT][kRec]: per column and activation row, digit plane p at 256 p (byte e = digit p
-//          of element e), the 8 sub-block sums at 768, 2^-E at 800, the column's sum of squares at 804
+//          of element e), the 8 sub-block sums at 768, their factors 2^-E at 800, the column's sum of squares at 832
 //   zeros  [144]
 //   red    [nslots][upt][MT][16] partial sums of a tile's units
 //   ctr    [0] next unit to draw, [1 + s] units delivered to slot s, [1 + nslots + s] tiles completed
-//          in slot s, [1 + 2 nslots + c] column c's operands are in place
+//          in slot s, [1 + 2 nslots + c] column c's operands are in place, [1 + 2 nslots + nb] a wave has given up
 template <int MT, bool DUAL, bool VEC>
 __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Args a) {
   constexpr int NMAT = DUAL ? 2 : 1;
@@ -147,7 +117,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // Every kernel argument is fetched in one batch here (left alone the compiler fetches some of
   // them only where they are first used: a second, dependent trip to memory).
-  asm volatile("" :: "s"(a.A), "s"(a.W), "s"(a.W2), "s"(a.C), "s"(a.residual), "s"(a.norm_weight));
+  asm volatile("" :: "s"(a.A), "s"(a.W), "s"(a.W2), "s"(a.C), "s"(a.residual), "s"(a.norm_weight), "s"(a.status));
   asm volatile("" :: "s"(a.M), "s"(a.N), "s"(a.K), "s"(a.nb), "s"(a.depth), "s"(a.rows), "s"(a.nlw), "s"(a.upt), "s"(a.upt_mul),
                "s"(a.grid), "s"(a.tiles_base), "s"(a.tiles_rem), "s"(a.nslots), "s"(a.slot_shift), "s"(a.c_f16), "s"(a.activation),
                "s"(a.norm_weight_offset));
@@ -161,7 +131,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
   unsigned* ctr = reinterpret_cast<unsigned*>(red + (size_t)nslots * upt * MT * 16);
 
   // counters, flags, zero area: set before the barrier, which costs only the skew of the wave launches
-  for (int i = tid; i < 1 + 2 * nslots + nb; i += 64 * kWaves) ctr[i] = 0u;
+  for (int i = tid; i < 2 + 2 * nslots + nb; i += 64 * kWaves) ctr[i] = 0u;
   if (tid >= 64 && tid < 64 + kZeroBytes / 4) reinterpret_cast<uint32_t*>(zeros)[tid - 64] = 0u;
 
   const int64_t row_bytes = (int64_t)nb * kBlockBytes;
@@ -264,6 +234,18 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
 
   // Draws the next unit of the workgroup (wave-uniform result).
   const uint32_t ctr_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(ctr);
+  const uint32_t abort_addr = ctr_abs + 4 * (1 + 2 * nslots + nb);
+  // A wait inside the workgroup ran into its limit: the wave lets its loads land, leaves the code in the
+  // library's status word (the host finds it at its next synchronisation), tells the other waves and ends.
+  auto give_up = [&](const uint32_t kind) {
+    DH_WAIT_VM(0);
+    if (lane == 0) {
+      __hip_atomic_store(a.status, dh::kstatus_code(kind, 0u, blockIdx.x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      ctr[1 + 2 * nslots + nb] = 1u;
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_endpgm();          // the wave ends here (no barrier follows in this kernel)
+  };
   auto draw = [&]() -> int {
     unsigned v = 0;
     if (lane == 0)
@@ -304,39 +286,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
                 v[e] *= a.norm_weight_offset ? 1.0f + wr[i][e] : wr[i][e];
               }
             }
-            const float mx = wave_max_uniform(fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
-            int ex = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;     // mx < 2^(ex+1)
-            ex = max(-100, min(100, ex));
-            if (mx == 0.f) ex = 0;
-            const float sf = __uint_as_float((uint32_t)(127 + 19 - ex) << 23);   // |x| * sf < 2^20
-            const float xinv = __uint_as_float((uint32_t)(127 - 19 + ex) << 23);
-            // X = round(x * sf) sits in the low mantissa bits of x * sf + 1.5 * 2^23 (two's complement)
-            uint32_t b[4], d2[4], d1[4], d0[4];
-            uint32_t xs = 0u;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              b[e] = __float_as_uint(fmaf(v[e], sf, 12582912.0f));
-              xs += b[e];
-              d2[e] = (uint32_t)__builtin_amdgcn_sbfe((int)b[e], 0, 7);              // signed low 7 bits
-              d1[e] = (uint32_t)__builtin_amdgcn_sbfe((int)(b[e] + 64u), 7, 7);
-              d0[e] = (b[e] + 8256u) >> 14;                                          // byte 0 = top digit
-            }
-            const uint32_t lo01 = 0x0c0c0400u, hi23 = 0x04000c0cu;   // byte 0 of (src1, src0) -> bytes 0,1 / 2,3
-            const uint32_t pk0 = __builtin_amdgcn_perm(d0[1], d0[0], lo01) | __builtin_amdgcn_perm(d0[3], d0[2], hi23);
-            const uint32_t pk1 = __builtin_amdgcn_perm(d1[1], d1[0], lo01) | __builtin_amdgcn_perm(d1[3], d1[2], hi23);
-            const uint32_t pk2 = __builtin_amdgcn_perm(d2[1], d2[0], lo01) | __builtin_amdgcn_perm(d2[3], d2[2], hi23);
-            // sum of the quantised activations of each sub-block (8 lanes x 4 elements)
-            const float sxf = (float)sum8_i32((int)(xs - 4u * 0x4B400000u)) * xinv;
             unsigned char* rec = xq + (size_t)(col * MT + m) * kRec;
-            reinterpret_cast<uint32_t*>(rec)[lane] = pk0;
-            reinterpret_cast<uint32_t*>(rec)[64 + lane] = pk1;
-            reinterpret_cast<uint32_t*>(rec)[128 + lane] = pk2;
-            if ((lane & 7) == 0) reinterpret_cast<float*>(rec)[192 + (lane >> 3)] = sxf;
+            i8_quantise_store(v, rec, lane);
             if (norm) ss = dh::wave_sum_uniform(ss);
-            if (lane == 0) {
-              reinterpret_cast<float*>(rec)[200] = xinv;
-              reinterpret_cast<float*>(rec)[201] = ss;
-            }
+            if (lane == 0) reinterpret_cast<float*>(rec)[kRecSsq / 4] = ss;
           }
           // LDS executes a wave's operations in order: whoever sees the flag sees the record
           if (lane == 0) ctr[1 + 2 * nslots + col] = 1u;
@@ -413,8 +366,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     constexpr int MP = MT < 2 ? MT : 2;
     v4u h, q0, q1;
     v4i ax[MP][2][2];
-    v2f sx[MP];
-    float xinv[MP];
+    v2f sx[MP], xinv[MP];     // activation sums and factors of sub-blocks kg and 4 + kg
     uint32_t gen, flag;
     asm volatile(
         "ds_read_b32 %4, %8\n\t"
@@ -430,16 +382,16 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
 #define DH_READ_OPERANDS(m0_)                                                                     \
     _Pragma("unroll") for (int m = 0; m < MP; m++) {                                              \
       const uint32_t rm = rec + ((m0_) + m) * kRec;                                               \
-      const uint32_t pa = rm * a_mul[0] + a_off[0], pb = rm * a_mul[1] + a_off[1], ps = rm + 768 + 4 * kg; \
+      const uint32_t pa = rm * a_mul[0] + a_off[0], pb = rm * a_mul[1] + a_off[1], ps = rm + kRecSums + 4 * kg; \
       asm volatile(                                                                               \
           "ds_read_b128 %0, %6\n\t"                                                               \
           "ds_read_b128 %1, %7\n\t"                                                               \
           "ds_read_b128 %2, %6 offset:128\n\t"                                                    \
           "ds_read_b128 %3, %7 offset:128\n\t"                                                    \
           "ds_read2_b32 %4, %8 offset1:4\n\t"                                                     \
-          "ds_read_b32 %5, %9 offset:800"                                                         \
+          "ds_read2_b32 %5, %8 offset0:8 offset1:12"                                              \
           : "=&v"(ax[m][0][0]), "=&v"(ax[m][0][1]), "=&v"(ax[m][1][0]), "=&v"(ax[m][1][1]), "=&v"(sx[m]), "=&v"(xinv[m]) \
-          : "v"(pa), "v"(pb), "v"(ps), "v"(rm)                                                    \
+          : "v"(pa), "v"(pb), "v"(ps)                                                             \
           : "memory");                                                                            \
     }
 #define DH_TIE_OPERANDS()                                                                         \
@@ -450,10 +402,16 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(h), "+v"(q0), "+v"(q1), "+v"(gen), "+v"(flag), "+v"(nxt) :: "memory");
     DH_TIE_OPERANDS();
     if (__builtin_amdgcn_readfirstlane(flag) == 0u) {
+      // bounded: a wave that is not served within the limit reports it and leaves; so do the others
+      int spins = 0;
       do {
         __builtin_amdgcn_s_sleep(2);
         flag = lds_read_u32(flag_addr);
+        if (++spins > kSpinLimit || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) break;
       } while (__builtin_amdgcn_readfirstlane(flag) == 0u);
+      if (__builtin_amdgcn_readfirstlane(flag) == 0u) {
+        give_up(DH_KSTATUS_COLUMN_WAIT);
+      }
       DH_READ_OPERANDS(0)
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       DH_TIE_OPERANDS();
@@ -486,9 +444,14 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     // wait (never, in practice) until the tile that used this slot nslots tiles ago is written out
     {
       const unsigned want = (unsigned)tl >> a.slot_shift;
-      while (gen != want) {
+      int spins = 0;
+      while (__builtin_amdgcn_readfirstlane(gen) != want) {
         __builtin_amdgcn_s_sleep(1);
         gen = lds_read_u32(gen_addr);
+        if (++spins > kSpinLimit || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) break;
+      }
+      if (__builtin_amdgcn_readfirstlane(gen) != want) {
+        give_up(DH_KSTATUS_SLOT_WAIT);
       }
     }
 #pragma unroll
@@ -506,14 +469,8 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
           v4i t = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[m][cc][0], blo[cc], v4i{0, 0, 0, 0}, 0, 0, 0);
           dd[cc] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[m][cc][1], bhi[cc], t, 0, 0, 0);
         }
-        // |digit sum| <= 32*15*64 and the scale is 6 bits: 24-bit multiplies are exact
-        const int p0 = __mul24(sc_a, dd[0][0]) + __mul24(sc_b, dd[1][0]);
-        const int p1 = __mul24(sc_a, dd[0][1]) + __mul24(sc_b, dd[1][1]);
-        const int p2 = __mul24(sc_a, dd[0][2]) + __mul24(sc_b, dd[1][2]);
-        const float t = fmaf((float)p0, 16384.f, fmaf((float)p1, 128.f, (float)p2));
-        const float mins = fmaf(mn_a, sx[m][0], mn_b * sx[m][1]);
         // the four lane groups hold different sub-blocks of the same 16 rows
-        const float sres = sum_lane_groups(fmaf(d * xinv[m], t, -dmin * mins));
+        const float sres = sum_lane_groups(i8_unit_term(dd[0], dd[1], sc_a, sc_b, mn_a, mn_b, d, dmin, sx[m], xinv[m]));
         if (lane < 16) red[(((size_t)slot * upt + (mat * nb + col)) * MT + m0 + m) * 16 + lane] = sres;
       }
     }
@@ -564,7 +521,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
           if (!have_rms) {
             // every column has been consumed by now, so every column's sum of squares is in place
             float tot = 0.f;
-            for (int c = 0; c < nb; c++) tot += __uint_as_float(lds_read_u32(xq_abs + (uint32_t)(c * MT + m) * kRec + 804));
+            for (int c = 0; c < nb; c++) tot += __uint_as_float(lds_read_u32(xq_abs + (uint32_t)(c * MT + m) * kRec + kRecSsq));
             inv_rms[m] = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
           }
           sg *= inv_rms[m];
@@ -644,7 +601,7 @@ int launch_i8_vec(I8Args a, const char* op) {
   while ((1 << a.slot_shift) < nslots) a.slot_shift++;
   auto lds_for = [&](int dep) {
     return (size_t)kWaves * dep * kStage + (size_t)a.nb * MT * kRec + kZeroBytes +
-           sizeof(float) * nslots * a.upt * MT * 16 + sizeof(unsigned) * (1 + 2 * nslots + a.nb);
+           sizeof(float) * nslots * a.upt * MT * 16 + sizeof(unsigned) * (2 + 2 * nslots + a.nb);
   };
   while (depth > 1 && lds_for(depth) > cap) depth--;
   if (lds_for(depth) > cap) return -1;
@@ -669,7 +626,7 @@ size_t i8_lds_bytes(int mt, int nb, int nmat) {
   int nslots = 2;
   while (nslots < need) nslots *= 2;
   return (size_t)kWaves * kStage + (size_t)nb * mt * kRec + kZeroBytes + sizeof(float) * nslots * upt * mt * 16 +
-         sizeof(unsigned) * (1 + 2 * nslots + nb);
+         sizeof(unsigned) * (2 + 2 * nslots + nb);
 }
 
 template <bool DUAL>
@@ -716,6 +673,7 @@ int q4k_gemv_i8(const char* op, const float* A, const uint8_t* W, const uint8_t*
   a.M = M; a.N = N; a.K = K; a.nb = (K + kQK - 1) / kQK;
   a.alpha = alpha; a.c_f16 = c_f16; a.activation = activation; a.clamp_max = clamp_max;
   a.norm_weight = norm_weight; a.norm_eps = norm_eps; a.norm_weight_offset = norm_weight_offset;
+  a.status = dh::kernel_status_word();
   return W2 ? dispatch_i8<true>(a, op) : dispatch_i8<false>(a, op);
 }
 

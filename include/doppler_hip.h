@@ -136,6 +136,48 @@ int dh_q4k_ffn_gate_up_rmsnorm(const float* d_x, const float* d_norm_weight, flo
                                float* d_out, int M, int hidden, int inter, int activation,
                                float alpha, float swiglu_limit);
 
+/* ---- chained decode products ----
+ * Up to DH_CHAIN_MAX_PHASES dependent Q4_K products of ONE activation row in a single launch:
+ *     x_0 = d_x0,   x_{p+1} = f_p( W_p . g_p(x_p) ),   C_p = x_{p+1}
+ * g_p: RMSNorm of the product's input when d_norm_weight is set (as in dh_q4k_matmul_rmsnorm);
+ * f_p: alpha * (.) + residual (as dh_q4k_matmul), or with d_W2 the gated pair
+ * act(W . x) * (W2 . x) * alpha (as dh_q4k_ffn_gate_up).  The reference records these products one
+ * after the other into the step's command encoder (src/inference/pipelines/text/layer.js:682
+ * processLayerGPU -> attention/interpreter.js:1148 o_proj, ffn/dense.js:727 gate/up and down, then
+ * the next layer's attention/projections.js:641 q/k/v) and submits once per token
+ * (generator-steps.js:814); here the run between two attentions is one persistent launch in which
+ * the weight stream of a product starts while the previous product's outputs still travel between
+ * the workgroups.  Results equal those of the separate calls (same kernels' arithmetic).
+ * Limits: K of every product a multiple of 256 and at least 2048, N and K at most 32768,
+ * K_p = N_{p-1}, f32 vectors, 16-byte aligned pointers; a product's d_residual may be an earlier
+ * product's d_C (or d_x0's producer's output), d_C must not be d_x0.  Launches are ordered on the
+ * op stream and share one exchange area of the library: one chain at a time per device.
+ * Every wait inside the launch is bounded: if one gives up (it cannot while the launch has the
+ * device's compute units to itself) all waves exit, the outputs are undefined, and the next call
+ * that waits for the stream (dh_sync, dh_download, dh_upload, dh_free) fails with the reason. */
+#define DH_CHAIN_MAX_PHASES 4
+typedef struct dh_chain_phase {
+  const void* d_W;             /* Q4_K [N,K] */
+  const void* d_W2;            /* second matrix of a gated pair (the "up" rows), or NULL */
+  float* d_C;                  /* [N] f32 */
+  const float* d_residual;     /* [N] f32 or NULL (not with d_W2) */
+  const float* d_norm_weight;  /* [K] f32 or NULL */
+  int N, K;
+  int activation;              /* DH_ACT_*, used with d_W2 */
+  int norm_weight_offset;      /* 1: weights are 1 + w */
+  float alpha;
+  float swiglu_limit;          /* clamp of the gated pair's output (DH_ACT_SILU only); 0 = off */
+  float norm_eps;
+} dh_chain_phase;
+int dh_q4k_gemv_chain(const float* d_x0, const dh_chain_phase* phases, int n_phases);
+/* Diagnostic form: launches only the first `workgroups` workgroups of the chain and bounds every
+ * wait at `spin_limit` polls.  With fewer workgroups than compute units the missing ones' outputs
+ * never arrive, so the waits give up, every wave exits, and the next synchronising call reports
+ * it: the way to exercise the failure path without hanging anything.  No counterpart in the
+ * reference. */
+int dh_q4k_gemv_chain_limited(const float* d_x0, const dh_chain_phase* phases, int n_phases,
+                              int workgroups, int spin_limit);
+
 /* ---- dense f16-weight GEMV (LM head) ----
  * C[M,N] = alpha * A[M,K] . f32(W[N,K])^T, W row-major f16.  Replaces the f16-weight branch
  * of runMatmul (matmul_gemv_subgroup.wgsl) used by recordLogitsGPU,
