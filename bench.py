@@ -27,8 +27,8 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per fused gate/up launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs, scaled
 # by the same counters' readings for a cast kernel of known traffic (x2.000 and x1.000):
-# 55,718 KiB fetched + 48 KiB written.
-GATE_UP_TRAFFIC_BYTES = 57104000
+# 55,683 KiB fetched + 48 KiB written.
+GATE_UP_TRAFFIC_BYTES = 57069000
 
 
 def log(*a):
@@ -288,7 +288,7 @@ def main():
         "metric": "decode tokens/sec at 9B-class Q4_K, 1 GPU (Q4_K GEMV HBM GB/s in roofline)",
         "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32 (Q4_K weights, f16 KV/LM head)", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32 activations and sums; Q4_K products on the int8 matrix cores with activations as 21-bit block fixed point (one exponent per 32-element sub-block, exact int32 sums); f16 KV cache and LM head", "data": "synthetic",
         "config": {"workload": "BASELINE configs[4]: 36-layer 9B-class Q4_K decoder, hidden 4096, FFN 12288, "
                                "32/8 heads x128, vocab 151936, KV prefilled to %d, greedy, batch 1" % prefill,
                    "layers": cfg["layers"], "context": prefill, "algorithmic_bytes_per_step": step_bytes,

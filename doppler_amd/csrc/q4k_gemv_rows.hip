@@ -285,7 +285,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
     }
     mx = row_lanes_max(mx);
     int ex = (int)((__float_as_uint(mx) >> 23) & 0xFF) - 127;      // mx < 2^(ex+1)
-    ex = max(-100, min(100, ex));
+    // The factors 2^(14 - ex) and 2^(10 + ex) must both be normal numbers.  Rows whose largest magnitude
+    // is 2^118 or more (or infinite) overflow the f16 operands and come out non-finite; a NaN
+    // activation is no maximum (v_max3 skips it) and travels through the matrix core as NaN.
+    ex = max(-112, min(117, ex));
     if (mx == 0.f) ex = 0;
     // |x| sf < 2^15; rows past M become zero operands
     const float sf = row_ok ? __uint_as_float((uint32_t)(127 + 14 - ex) << 23) : 0.f;

@@ -55,6 +55,21 @@ def q4k_pack_block_fields(d_bits, dmin_bits, sc, mn, q):
     return out
 
 
+def q4k_centred(W, shift=0):
+    """A copy of Q4_K tensor W with zero-mean weights of the same spread: every sub-block's min is set
+    to its scale and dmin to 7.5 d, so that w = d sc (q - 7.5); d is scaled by 2^-shift on the way.
+    (The benchmark's own distribution, mins and dmin drawn independently, gives every weight the same
+    large positive mean: a decoder stack of such matrices collapses onto the all-ones direction and
+    its logits hardly depend on the token or on the KV cache.)"""
+    w = np.ascontiguousarray(W).reshape(-1, Q4K_BLOCK_BYTES).copy()
+    d = (w[:, 0:2].copy().view(np.float16).astype(np.float32) * np.float32(2.0 ** -shift)).astype(np.float16)
+    w[:, 0:2] = d.view(np.uint8)
+    w[:, 2:4] = (d.astype(np.float32) * np.float32(7.5)).astype(np.float16).view(np.uint8)
+    w[:, 8:12] = w[:, 4:8]                                                  # mins 0..3 and the high bits of mins 4..7
+    w[:, 12:16] = (w[:, 12:16] & 0x0F) | ((w[:, 12:16] & 0x0F) << 4)        # low bits of mins 4..7
+    return w.reshape(-1)
+
+
 def normal_f32(shape, seed, scale=1.0):
     return (rng(seed).standard_normal(shape, dtype=np.float32) * np.float32(scale)).astype(np.float32)
 

@@ -219,6 +219,9 @@ def test_9b_class_greedy_64_steps_identical_tokens():
         gv = v0[p_ * ks:(p_ + 1) * ks].view(np.float16).astype(np.float64)
         assert rel_l2(gk, ek) <= 1e-3, p_          # f16 rounding of the row: ~3e-4
         assert rel_l2(gv, ev) <= 1e-3, p_
+    # rows of a middle and the last layer at the first three positions against an oracle that starts from nothing
+    _first_rows_against_a_fresh_oracle(cfg, layers, embed, final_norm, cos, sin, gpu, ids, 3, max_seq,
+                                       (cfg["layers"] // 2, cfg["layers"] - 1))
     cpu = oracle.DecoderOracle(cfg, ol, embed, final_norm, cos, sin)
     forced = synth.rng(41).integers(0, cfg["vocab"], steps)
     gpu_tokens, cpu_tokens, worst, margins = [], [], 0.0, []
@@ -244,6 +247,111 @@ def test_9b_class_greedy_64_steps_identical_tokens():
     assert worst <= 1e-3
     assert len(set(gpu_tokens)) > 1
     # the rows the 64 steps appended, every layer: both sides computed them from the same prefix
+    for i in range(cfg["layers"]):
+        k, v = gpu.read_kv(i, max_seq)
+        for got, name in ((k, "cache_k"), (v, "cache_v")):
+            g_rows = got[prefill * ks:].view(np.float16).astype(np.float64)
+            e_rows = ol[i][name].reshape(-1)[prefill * ks:max_seq * ks].view(np.float16).astype(np.float64)
+            assert rel_l2(g_rows, e_rows) <= 1e-3, (i, name)
+
+
+def _first_rows_against_a_fresh_oracle(cfg, layers, embed, final_norm, cos, sin, gpu, ids, n, max_seq, check_layers):
+    """The KV rows of positions 0..n-1 in the given layers against an oracle that starts from an
+    empty cache (everything those rows depend on is the first n tokens)."""
+    fresh = oracle_layers(layers, max_seq, cfg["kv_heads"], cfg["head_dim"])
+    cpu = oracle.DecoderOracle(cfg, fresh, embed, final_norm, cos, sin)
+    for pos in range(n):
+        cpu.step(int(ids[pos]), pos)
+    ks = cfg["kv_heads"] * cfg["head_dim"]
+    for li in check_layers:
+        k, v = gpu.read_kv(li, n)
+        for got, name in ((k, "cache_k"), (v, "cache_v")):
+            want = fresh[li][name].reshape(-1)[:n * ks].view(np.float16).astype(np.float64)
+            assert rel_l2(got.view(np.float16).astype(np.float64), want) <= 1e-3, (li, name)
+
+
+@pytest.mark.timeout(1500)
+def test_9b_class_centred_weights_sensitive_logits_and_greedy_tokens():
+    """Config 4's architecture with zero-mean weights (synth.q4k_centred, d scaled by 2^-6 so that the
+    residual stream stays O(1)): a stack whose logits DO depend on the token, the rotary row and
+    single cache rows, which the test first shows on the oracle and then uses: 32 steps, tokens
+    identical, logits within 1e-3, appended KV rows compared in every layer.  The first three
+    positions go through decode steps and their KV rows in the first, a middle and the last layer
+    are compared with an oracle that starts from nothing; the other 2045 prompt positions go
+    through the batched prefill path (GEMM + prefill attention) at full size."""
+    c = dict(synth.CFG4)
+    prefill, steps = c.pop("prefill"), 32
+    c.pop("steps")
+    max_seq = prefill + steps
+    cfg = dict(c, max_seq=max_seq)
+    layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=4, max_seq=max_seq)
+    for l in layers:
+        for n in ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown"):
+            l[n] = synth.q4k_centred(l[n], 6)
+    gpu = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, max_seq)
+    ids = synth.rng(40).integers(0, cfg["vocab"], prefill)
+    for pos in range(3):
+        gpu.step(int(ids[pos]), pos)
+    mid = cfg["layers"] // 2
+    _first_rows_against_a_fresh_oracle(cfg, layers, embed, final_norm, cos, sin, gpu, ids, 3, max_seq,
+                                       (0, mid, cfg["layers"] - 1))
+    tok = gpu.prefill(ids[3:], start_pos=3)
+    ol = oracle_layers(layers, max_seq, cfg["kv_heads"], cfg["head_dim"])
+    for i, l in enumerate(ol):
+        k, v = gpu.read_kv(i, prefill)
+        l["cache_k"].reshape(-1)[:k.size] = k
+        l["cache_v"].reshape(-1)[:v.size] = v
+    cpu = oracle.DecoderOracle(cfg, ol, embed, final_norm, cos, sin)
+
+    # ---- the oracle's logits move with what the step consumes
+    _, base = cpu.step(1234, prefill, want_logits=True)
+    _, other = cpu.step(4321, prefill, want_logits=True)
+    assert rel_l2(other, base) > 0.1                                    # another input token
+    row = ol[mid]["cache_k"][prefill // 2].copy()
+    ol[mid]["cache_k"][prefill // 2] ^= 0x8000                         # one negated key row in one layer
+    _, moved = cpu.step(1234, prefill, want_logits=True)
+    ol[mid]["cache_k"][prefill // 2] = row
+    one_row = rel_l2(moved, base)
+    for l in ol:                                                        # one position's rows in every layer
+        l["cache_k"][prefill // 2] ^= 0x8000
+        l["cache_v"][prefill // 2] ^= 0x8000
+    _, moved = cpu.step(1234, prefill, want_logits=True)
+    for l in ol:
+        l["cache_k"][prefill // 2] ^= 0x8000
+        l["cache_v"][prefill // 2] ^= 0x8000
+    one_position = rel_l2(moved, base)
+    shifted = oracle.DecoderOracle(cfg, ol, embed, final_norm, np.ascontiguousarray(np.roll(cos, -1, axis=0)),
+                                   np.ascontiguousarray(np.roll(sin, -1, axis=0)))
+    _, moved = shifted.step(1234, prefill, want_logits=True)
+    rotary = rel_l2(moved, base)
+    print("logits move by: one key row %.2e, one position's rows in every layer %.2e, rotary row off by one %.2e"
+          % (one_row, one_position, rotary), flush=True)
+    assert one_row > 1e-4 and one_position > 1e-2 and rotary > 0.1
+    # the same step on the GPU: far inside the smallest of those movements
+    g = gpu.step(1234, prefill, want_logits=True)
+    agree = rel_l2(gpu.read_logits(), base)
+    assert agree <= 1e-3 and agree < one_row / 4, (agree, one_row)
+
+    # ---- 32 greedy steps
+    gpu_tokens, cpu_tokens, worst, margins = [], [], 0.0, []
+    inp = tok
+    for s in range(steps):
+        pos = prefill + s
+        g = gpu.step(inp, pos, want_logits=True)
+        ctok, want = cpu.step(inp, pos, want_logits=True)
+        err = rel_l2(gpu.read_logits(), want)
+        worst = max(worst, err)
+        top2 = np.partition(np.asarray(want, np.float64), -2)[-2:]
+        margins.append(float(top2[1] - top2[0]))
+        print("step %2d pos %d input %6d -> gpu %6d cpu %6d  logits relL2 %.2e  top-2 margin %.4f" %
+              (s, pos, inp, g, ctok, err, margins[-1]), flush=True)
+        gpu_tokens.append(g)
+        cpu_tokens.append(ctok)
+        inp = g
+    assert gpu_tokens == cpu_tokens
+    assert worst <= 1e-3
+    assert len(set(gpu_tokens)) > steps // 2
+    ks = cfg["kv_heads"] * cfg["head_dim"]
     for i in range(cfg["layers"]):
         k, v = gpu.read_kv(i, max_seq)
         for got, name in ((k, "cache_k"), (v, "cache_v")):

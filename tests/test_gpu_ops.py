@@ -233,6 +233,27 @@ def test_fused_ffn_prefill_cfg2(M, activation):
     assert rel_l2(ops.readTensor(out), want) <= REL_L2_F16_MFMA
 
 
+def test_prefill_ffn_chain_cfg2():
+    """Config 2 as ONE chain: X[512,1152] -> fused gate/up with the GELU gate -> down projection, the
+    intermediate H staying on the device in f32, against the oracle's chain
+    (tests/kernels/reference/fused-ffn-q4k.js:42-73 then the row-major product)."""
+    M, hidden, inter = 512, synth.CFG2["hidden"], synth.CFG2["inter"]
+    Wg, wg = q4k_weight(inter, hidden, seed=2420)
+    Wu, wu = q4k_weight(inter, hidden, seed=2421)
+    Wd, wd = q4k_weight(hidden, inter, seed=2422)
+    X = synth.normal_f32((M, hidden), seed=2423, scale=0.05)
+    H = ops.runFusedFFN(ops.tensorFromNumpy(X), wg, wu, hidden, inter, batchSize=M, activation="gelu")
+    Y = ops.runMatmul(H, wd, M, hidden, inter, outputDtype="f32", role="ffn_down")
+    want_h = oracle.q4k_ffn_gate_up(X, Wg, Wu, M, hidden, inter, alpha=1.0, activation="gelu")
+    want_y = oracle.q4k_matmul(want_h.reshape(M, inter), Wd, M, hidden, inter)
+    assert rel_l2(ops.readTensor(H), want_h) <= REL_L2_F16_MFMA
+    assert rel_l2(ops.readTensor(Y), want_y) <= REL_L2_F16_MFMA
+    # row by row as well: no row may hide behind the others
+    got = ops.readTensor(Y).reshape(M, hidden)
+    want = want_y.reshape(M, hidden)
+    assert max(rel_l2(got[m], want[m]) for m in range(M)) <= 2 * REL_L2_F16_MFMA
+
+
 def test_matmul_alpha_residual_f16_output():
     assert _matmul_case(2, 512, 1024, seed=1500, alpha=0.125, residual=True) <= REL_L2_F32
     assert _matmul_case(4, 512, 1024, seed=1510, alpha=2.0 ** -8, outputDtype="f16") <= 1e-3
