@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libdopplerhip.so")
 F32, F16 = 0, 1
 ACT_SILU, ACT_GELU = 0, 1
 KV_CONTIGUOUS, KV_RING = 0, 1
+PLAN_GEMV_I8, PLAN_GEMV_ROWS, PLAN_GEMV_RING, PLAN_GEMM, PLAN_GEMV_LDS = 1, 2, 3, 4, 5
 
 
 class DopplerHipError(RuntimeError):
@@ -63,11 +64,13 @@ SIGNATURES = {
     "dh_graph_begin": (_I, []),
     "dh_graph_end": (_I, [_I, ctypes.POINTER(_P)]),
     "dh_graph_launch": (_I, [_P, _I]),
+    "dh_graph_set_max_position": (_I, [_P, _I]),
     "dh_graph_prepare": (_I, [_P, _I]),
     "dh_graph_destroy": (_I, [_P]),
     "dh_q4k_dequant": (_I, [_P, _I64, _P]),
     "dh_q4k_matmul": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
     "dh_q4k_matmul_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
+    "dh_q4k_matmul_plan": (_I, [_I, _I, _I, _I, _I, _I]),
     "dh_q4k_ffn_gate_up": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
     "dh_q4k_ffn_gate_up_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
     "dh_q4k_gemv_chain": (_I, [_P, ctypes.POINTER(ChainPhase), _I]),
@@ -83,6 +86,9 @@ SIGNATURES = {
     "dh_attn_decode_qkv_supported": (_I, [_I, _I, _I, _I, _I]),
     "dh_attn_decode_qkv": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _F, _I, _I,
                                 _I, _P]),
+    "dh_attn_decode_kvlen": (_I, [_P, _P, _P, _P, _I, _I, _I, _P, _I, _F, _I, _I, _F, _I, _I, _I, _P]),
+    "dh_attn_decode_qkv_kvlen": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _F, _I, _I, _F, _F, _I,
+                                      _I, _I, _P]),
     "dh_rmsnorm": (_I, [_P, _P, _I, _P, _I, _I, _F, _I, _P, _P, _P, _F]),
     "dh_rmsnorm_sandwich_pair": (_I, [_P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _F, _I]),
     "dh_residual_rmsnorm_pair": (_I, [_P, _P, _P, _I, _P, _P, _I, _I, _F, _I, _F]),

@@ -27,6 +27,54 @@ namespace {
 constexpr int kTileKeys = 64;
 constexpr int kMaxG = 8;       // query heads per kv head
 
+// What the kernels need to redo the host's key-range arithmetic from a key count in device memory.
+struct DynKeys {
+  const uint32_t* kv_len_ptr;   // null: everything comes in as launch arguments
+  int max_kv_len;               // the count is clamped to this (caches, tables and workspace are sized for it)
+  int causal, start_pos;        // start_pos < 0: the query sits at the last key, kv_start + kv_len - 1
+  int sliding_window, kv_start, qkv;
+  int one_per_cu;               // workgroups per kv head that fill the device once
+};
+struct KeyRange {
+  int kbeg, kend, nsplit, start_pos;
+};
+
+// Splits of the key range per kv head.  Fewer, longer workgroups beat more splits once every CU
+// has one: a workgroup's next chunk costs well under 1 us, every extra split costs the merge
+// kernel and the dispatch more (measured, 32/8 heads, four workgroups per CU against one:
+// 3000 keys 12.9 vs 10.4 us, 6000 keys 17.1 vs 12.6, 16384 keys 24.4 vs 20.4, 32768 keys 37.1 vs
+// 33.4).  One workgroup per CU, two once that would mean more than 16 chunks each.
+__host__ __device__ inline int splits_for(int one_per_cu, int nkeys) {
+  const int tiles = nkeys > 0 ? (nkeys + 63) / 64 : 1;
+  const int wgs = tiles <= 16 * one_per_cu ? one_per_cu : 2 * one_per_cu;
+  if (tiles <= wgs) return tiles;
+  // every workgroup the same number of chunks (the slowest one sets the time), in as few splits
+  // as that allows (the merge kernel pays per split)
+  const int chunks_each = (tiles + wgs - 1) / wgs;
+  return (tiles + chunks_each - 1) / chunks_each;
+}
+// The largest split count any key count up to max_keys can ask for: the grid of a launch whose key
+// count is only known on the device.
+__host__ __device__ inline int max_splits_upto(int one_per_cu, int max_keys) {
+  const int tiles = max_keys > 0 ? (max_keys + 63) / 64 : 1;
+  if (tiles <= one_per_cu) return tiles;
+  return tiles <= 16 * one_per_cu ? one_per_cu : 2 * one_per_cu;
+}
+// Visible key range [kbeg, kend) relative to kv_start, split count (0: no key is visible) and the
+// query's position for a key count read on the device.
+__device__ inline KeyRange dyn_key_range(const DynKeys& d) {
+  int kv_len = (int)*d.kv_len_ptr;
+  kv_len = kv_len < 0 ? 0 : (kv_len > d.max_kv_len ? d.max_kv_len : kv_len);
+  KeyRange r;
+  r.start_pos = d.start_pos < 0 ? d.kv_start + kv_len - 1 : d.start_pos;
+  r.kbeg = 0;
+  r.kend = kv_len;
+  if (!d.qkv && d.causal) r.kend = min(r.kend, r.start_pos - d.kv_start + 1);
+  if (d.sliding_window > 0 && r.start_pos >= d.sliding_window) r.kbeg = max(0, r.start_pos - d.sliding_window + 1 - d.kv_start);
+  r.nsplit = r.kend > r.kbeg ? splits_for(d.one_per_cu, r.kend - r.kbeg) : 0;
+  return r;
+}
+
 struct AttnArgs {
   const float* Q;       // [H][D]
   const __half* K;      // [rows][Hkv][D]
@@ -49,6 +97,12 @@ struct AttnArgs {
   int rotary_half, interleaved, w_offset, use_norm;
   float eps;
   int c_new, j_new;     // chunk, and key within the chunk, of the appended position
+  // ---- key count on the device (dh_attn_decode_kvlen, dh_attn_decode_qkv_kvlen): kbeg, kend, nsplit,
+  // direct and, for the stacked-projection form, cos_row, sin_row, new_row, c_new, j_new above are
+  // derived in the kernel from the word behind kv_len_ptr; the grid holds the splits of max_kv_len
+  DynKeys dyn;
+  const float* cos_base;
+  const float* sin_base;
 };
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -112,7 +166,22 @@ __device__ __forceinline__ float row_group_sum(float v) {
 // visible one, so the lanes that would read its row, or a clamped copy of it, from the not yet
 // written cache are patched from registers.
 template <int D, int GT, bool QKV>
-__global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a_in) {
+  AttnArgs a = a_in;
+  if (a.dyn.kv_len_ptr != nullptr) {
+    // the key count lives on the device: redo the host's arithmetic for it; surplus workgroups leave
+    const KeyRange r = dyn_key_range(a.dyn);
+    if ((int)blockIdx.y >= r.nsplit) return;
+    a.kbeg = r.kbeg; a.kend = r.kend; a.nsplit = r.nsplit; a.direct = 0;
+    if (QKV) {
+      a.cos_row = a.cos_base + (int64_t)r.start_pos * a.rotary_half;
+      a.sin_row = a.sin_base + (int64_t)r.start_pos * a.rotary_half;
+      const int row = a.ring_window > 0 ? r.start_pos % a.ring_window : r.start_pos;
+      a.new_row = (int64_t)row * a.Hkv * D;
+      a.c_new = (r.kend - r.kbeg - 1) / kTileKeys;
+      a.j_new = (r.kend - r.kbeg - 1) % kTileKeys;
+    }
+  }
   constexpr int STEPS = D / 32;          // MFMAs per 16 keys
   constexpr int DW = D / 4;              // output dims per wave
   constexpr int LPK = DW / 4;            // lanes per key in P.V (4 dims each)
@@ -438,11 +507,18 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
 // (Preloading 64 made short contexts slower, 8.9 vs 8.1 us at 512 keys.)
 template <int D>
 __global__ __launch_bounds__(D) void attn_decode_merge_kernel(const float* __restrict__ ws,
-                                                              float* __restrict__ O, int nsplit) {
+                                                              float* __restrict__ O, int nsplit, const DynKeys dyn) {
   constexpr int CH = 32;
   __shared__ float f_s[1024];
   __shared__ float red[4];
   const int h = blockIdx.x, d = threadIdx.x;
+  if (dyn.kv_len_ptr != nullptr) {
+    nsplit = dyn_key_range(dyn).nsplit;
+    if (nsplit == 0) {            // no visible key: the output is zero, as the host path writes it
+      O[(int64_t)h * D + d] = 0.f;
+      return;
+    }
+  }
   const float* base = ws + (int64_t)h * nsplit * (D + 2);
   float ov[CH];
 #pragma unroll
@@ -490,26 +566,18 @@ __global__ void zero_f32_kernel(float* p, int n) {
 
 int max_splits_for(int kv_len) { return std::max(1, (kv_len + kTileKeys - 1) / kTileKeys); }
 
-// Splits of the key range per kv head.  Fewer, longer workgroups beat more splits once every CU
-// has one: a workgroup's next chunk costs well under 1 us, every extra split costs the merge
-// kernel and the dispatch more (measured, 32/8 heads, four workgroups per CU against one:
-// 3000 keys 12.9 vs 10.4 us, 6000 keys 17.1 vs 12.6, 16384 keys 24.4 vs 20.4, 32768 keys 37.1 vs
-// 33.4).  One workgroup per CU, two once that would mean more than 16 chunks each.
+int one_per_cu_for(int Hkv) { return std::max(1, dh::num_cus() / std::max(1, Hkv)); }
+
 int choose_splits(int Hkv, int nkeys) {
   const int tiles = std::max(1, (nkeys + kTileKeys - 1) / kTileKeys);
-  static const double env_per_cu = getenv("DH_ATTN_WG_PER_CU") ? atof(getenv("DH_ATTN_WG_PER_CU")) : 0.0;
-  const int one_per_cu = std::max(1, dh::num_cus() / std::max(1, Hkv));
+  static const double env_per_cu = dh::tuning_double("DH_ATTN_WG_PER_CU", 0.0);
+  const int one_per_cu = one_per_cu_for(Hkv);
   if (env_per_cu > 0.0) return std::min(tiles, std::max(1, (int)(one_per_cu * env_per_cu)));
-  const int wgs = tiles <= 16 * one_per_cu ? one_per_cu : 2 * one_per_cu;
-  if (tiles <= wgs) return tiles;
-  // every workgroup the same number of chunks (the slowest one sets the time), in as few splits
-  // as that allows (the merge kernel pays per split)
-  const int chunks_each = (tiles + wgs - 1) / wgs;
-  return (tiles + chunks_each - 1) / chunks_each;
+  return splits_for(one_per_cu, nkeys);
 }
 
 typedef void (*SplitKernel)(const AttnArgs);
-typedef void (*MergeKernel)(const float*, float*, int);
+typedef void (*MergeKernel)(const float*, float*, int, const DynKeys);
 
 template <int D, bool QKV>
 SplitKernel split_kernel_for(int G) {
@@ -528,7 +596,7 @@ int launch(const AttnArgs& a, int D, bool qkv, const char* op) {
   hipLaunchKernelGGL(split_kernel_for(D, qkv, a.G), dim3(a.Hkv, a.nsplit), dim3(256), 0, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   if (!a.direct) {
-    hipLaunchKernelGGL(merge_kernel_for(D), dim3(a.H), dim3(D), 0, dh::stream(), a.ws, a.O, a.nsplit);
+    hipLaunchKernelGGL(merge_kernel_for(D), dim3(a.H), dim3(D), 0, dh::stream(), a.ws, a.O, a.nsplit, a.dyn);
     DH_CHECK_LAUNCH(op);
   }
   return 0;
@@ -667,6 +735,11 @@ int attn_graph_set_position(Graph* g, int position) {
     AttnArgs a;
     if (build_args(c, delta, true, a))
       return fail(1, "[dh_graph_launch] position %d leaves attention call %d without a visible key", position, i);
+    // the split partials of the new position must fit where the captured call put them
+    const size_t ws_need = (size_t)c.H * a.nsplit * (c.D + 2) * sizeof(float);
+    if (c.ws_capacity && ws_need > c.ws_capacity)
+      return fail(1, "[dh_graph_launch] position %d needs %zu bytes of split partials in attention call %d, the library's "
+                  "scratch holds %zu", position, ws_need, i, c.ws_capacity);
     AttnArgs* ap = &a;
     void* split_args[] = {ap};
     hipKernelNodeParams sp{};
@@ -679,7 +752,8 @@ int attn_graph_set_position(Graph* g, int position) {
     const float* ws = a.ws;
     float* O = a.O;
     int nsplit = a.nsplit;
-    void* merge_args[] = {&ws, &O, &nsplit};
+    DynKeys dyn = a.dyn;
+    void* merge_args[] = {&ws, &O, &nsplit, &dyn};
     hipKernelNodeParams mp{};
     mp.func = reinterpret_cast<void*>(merge_kernel_for(c.D));
     mp.gridDim = dim3(a.H);
@@ -735,7 +809,7 @@ static int attn_decode_impl(const char* op, const float* d_Q, const void* d_K, c
   c.qkv = 0; c.q = d_Q; c.K = const_cast<void*>(d_K); c.V = const_cast<void*>(d_V); c.O = d_O;
   c.H = H; c.Hkv = Hkv; c.D = D; c.kv_len = kv_len; c.start_pos = start_pos; c.causal = causal;
   c.scale = scale; c.softcap = softcap; c.sliding_window = sliding_window; c.kv_start = kv_start;
-  c.kv_layout = kv_layout; c.ws = d_workspace;
+  c.kv_layout = kv_layout; c.ws = d_workspace; c.ws_capacity = ws_capacity;
   const bool capturing = dh::capturing_graph() != nullptr;
   AttnArgs a;
   if (build_args(c, 0, capturing, a)) {
@@ -825,6 +899,87 @@ int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float*
   if (!a.direct && !d_workspace) return dh::fail(1, "[%s] workspace is required", op);
   dh::graph_note_attention(c);
   return launch(a, D, true, op);
+}
+
+// ---- key count on the device -------------------------------------------------------------------
+// Shared body of dh_attn_decode_kvlen and dh_attn_decode_qkv_kvlen: the launch arguments are built
+// for max_kv_len keys (that fixes pointers, shapes and the grid), the kernels replace everything
+// that depends on the key count by what the device word says.
+static int attn_decode_kvlen_impl(const char* op, dh::GraphAttnCall c, const uint32_t* d_kv_len, int max_kv_len,
+                                  int start_pos) {
+  if (!d_kv_len) return dh::fail(1, "[%s] the key-count pointer is null", op);
+  if (reinterpret_cast<uintptr_t>(d_kv_len) & 3) return dh::fail(1, "[%s] the key-count pointer must be 4-byte aligned", op);
+  if (max_kv_len < 1) return dh::fail(1, "[%s] max_kv_len must be at least 1", op);
+  if (!c.ws) return dh::fail(1, "[%s] workspace is required", op);
+  c.kv_len = max_kv_len;
+  c.start_pos = start_pos < 0 ? c.kv_start + max_kv_len - 1 : start_pos;
+  AttnArgs a;
+  if (build_args(c, 0, true, a)) return dh::fail(1, "[%s] no key is visible even at max_kv_len=%d", op, max_kv_len);
+  const int one_per_cu = one_per_cu_for(c.Hkv);
+  a.dyn = DynKeys{d_kv_len, max_kv_len, c.causal, start_pos, c.sliding_window, c.kv_start, c.qkv, one_per_cu};
+  a.cos_base = c.cos;
+  a.sin_base = c.sin;
+  a.nsplit = max_splits_upto(one_per_cu, max_kv_len);      // the grid; the kernels use the device word's split count
+  a.direct = 0;
+  // nothing is recorded for graph replays: a captured launch follows the device word by itself
+  return launch(a, c.D, c.qkv != 0, op);
+}
+
+int dh_attn_decode_kvlen(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H, int Hkv, int D,
+                         const uint32_t* d_kv_len, int max_kv_len, float scale, int causal, int start_pos,
+                         float softcap, int sliding_window, int kv_start, int kv_layout, void* d_workspace) {
+  const char* op = "dh_attn_decode_kvlen";
+  DH_REQUIRE_INIT(op);
+  if (H <= 0 || Hkv <= 0 || D <= 0) return dh::fail(1, "[%s] numHeads/numKVHeads/headDim must be positive", op);
+  if (H % Hkv) return dh::fail(1, "[%s] numHeads=%d must be a multiple of numKVHeads=%d", op, H, Hkv);
+  const int G = H / Hkv;
+  if (G > kMaxG) return dh::fail(1, "[%s] %d query heads per kv head not supported (max %d)", op, G, kMaxG);
+  if (D != 64 && D != 128) return dh::fail(1, "[%s] headDim %d not supported (64, 128)", op, D);
+  if (sliding_window < 0 || kv_start < 0) return dh::fail(1, "[%s] slidingWindow and kvStart must be non-negative", op);
+  if (kv_layout != DH_KV_CONTIGUOUS && kv_layout != DH_KV_RING)
+    return dh::fail(1, "[%s] kvLayout %d not supported (contiguous, ring)", op, kv_layout);
+  if (kv_layout == DH_KV_RING && sliding_window <= 0) return dh::fail(1, "[%s] ring layout needs slidingWindow > 0", op);
+  if (!d_Q || !d_O || !d_K || !d_V) return dh::fail(1, "[%s] null pointer", op);
+  if ((reinterpret_cast<uintptr_t>(d_K) | reinterpret_cast<uintptr_t>(d_V)) & 15)
+    return dh::fail(1, "[%s] K/V pointers must be 16-byte aligned", op);
+  dh::GraphAttnCall c{};
+  c.qkv = 0; c.q = d_Q; c.K = const_cast<void*>(d_K); c.V = const_cast<void*>(d_V); c.O = d_O;
+  c.H = H; c.Hkv = Hkv; c.D = D; c.causal = causal;
+  c.scale = scale; c.softcap = softcap; c.sliding_window = sliding_window; c.kv_start = kv_start;
+  c.kv_layout = kv_layout; c.ws = d_workspace;
+  return attn_decode_kvlen_impl(op, c, d_kv_len, max_kv_len, start_pos);
+}
+
+int dh_attn_decode_qkv_kvlen(const float* d_qkv, const float* d_q_weight, const float* d_k_weight, const float* d_cos,
+                             const float* d_sin, void* d_cache_k, void* d_cache_v, float* d_O, int H, int Hkv, int D,
+                             const uint32_t* d_kv_len, int max_kv_len, int rotary_dim, int interleaved, float eps,
+                             int weight_offset, int use_norm, float scale, float softcap, int sliding_window,
+                             int kv_start, int kv_layout, void* d_workspace) {
+  const char* op = "dh_attn_decode_qkv_kvlen";
+  DH_REQUIRE_INIT(op);
+  if (H <= 0 || Hkv <= 0 || D <= 0) return dh::fail(1, "[%s] numHeads/numKVHeads/headDim must be positive", op);
+  if (H % Hkv) return dh::fail(1, "[%s] numHeads=%d must be a multiple of numKVHeads=%d", op, H, Hkv);
+  if (!dh_attn_decode_qkv_supported(H, Hkv, D, rotary_dim, interleaved))
+    return dh::fail(1, "[%s] shape not served (heads %d/%d, headDim %d, rotaryDim %d, interleaved %d): use "
+                       "dh_qkv_norm_rope_kvwrite + dh_attn_decode_kvlen", op, H, Hkv, D, rotary_dim, interleaved);
+  if (sliding_window < 0 || kv_start < 0) return dh::fail(1, "[%s] slidingWindow and kvStart must be non-negative", op);
+  if (kv_layout != DH_KV_CONTIGUOUS && kv_layout != DH_KV_RING)
+    return dh::fail(1, "[%s] kvLayout %d not supported (contiguous, ring)", op, kv_layout);
+  if (kv_layout == DH_KV_RING && sliding_window <= 0) return dh::fail(1, "[%s] ring layout needs slidingWindow > 0", op);
+  if (!d_qkv || !d_cos || !d_sin || !d_cache_k || !d_cache_v || !d_O) return dh::fail(1, "[%s] null pointer", op);
+  if (use_norm && (!d_q_weight || !d_k_weight)) return dh::fail(1, "[%s] q/k norm weights are required", op);
+  if ((reinterpret_cast<uintptr_t>(d_cache_k) | reinterpret_cast<uintptr_t>(d_cache_v) |
+       reinterpret_cast<uintptr_t>(d_qkv) | reinterpret_cast<uintptr_t>(d_q_weight) |
+       reinterpret_cast<uintptr_t>(d_k_weight)) & 15)
+    return dh::fail(1, "[%s] qkv, the norm weights and the caches must be 16-byte aligned", op);
+  dh::GraphAttnCall c{};
+  c.qkv = 1; c.q = d_qkv; c.qw = d_q_weight; c.kw = d_k_weight; c.cos = d_cos; c.sin = d_sin;
+  c.K = d_cache_k; c.V = d_cache_v; c.O = d_O;
+  c.H = H; c.Hkv = Hkv; c.D = D; c.causal = 1;
+  c.rotary_dim = rotary_dim; c.interleaved = interleaved; c.weight_offset = weight_offset; c.use_norm = use_norm;
+  c.eps = eps; c.scale = scale; c.softcap = softcap; c.sliding_window = sliding_window; c.kv_start = kv_start;
+  c.kv_layout = kv_layout; c.ws = d_workspace;
+  return attn_decode_kvlen_impl(op, c, d_kv_len, max_kv_len, -1);
 }
 
 }  // extern "C"

@@ -289,7 +289,7 @@ extern "C" int dh_attn_prefill(const float* d_Q, const void* d_K, const void* d_
   a.causal = causal ? 1 : 0; a.window = sliding_window; a.scale = scale; a.softcap = softcap;
   // Two 16-query groups per wave (128 queries per workgroup) halve the LDS traffic per product;
   // short prompts keep 64-query tiles so that the grid still covers the compute units.
-  static const int env_qt = getenv("DH_ATTN_PREFILL_QT") ? atoi(getenv("DH_ATTN_PREFILL_QT")) : 0;
+  static const int env_qt = dh::tuning_int("DH_ATTN_PREFILL_QT", 0);
   const int qt = env_qt ? env_qt : ((int64_t)dh::ceil_div(T, 128) * H >= 2 * dh::num_cus() ? 2 : 1);
   const dim3 grid((unsigned)dh::ceil_div(T, 64 * qt), (unsigned)H);
   if (D == 64) {

@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <type_traits>
 
 #include "../../include/doppler_hip.h"
@@ -35,6 +36,34 @@ int gemm_row_scale_capacity();
 float* widened_activations(size_t* bytes);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Tile shapes, ring depths and kernel families have ONE setting in the library as it is built.  A
+// build with -DDH_TUNING_ENV (measurements only, never the shipped library) reads overrides of the
+// same names from the environment.
+inline const char* tuning_env(const char* name) {
+#ifdef DH_TUNING_ENV
+  return getenv(name);
+#else
+  (void)name;
+  return nullptr;
+#endif
+}
+inline int tuning_int(const char* name, int dflt) {
+  const char* e = tuning_env(name);
+  return e ? atoi(e) : dflt;
+}
+inline double tuning_double(const char* name, double dflt) {
+  const char* e = tuning_env(name);
+  return e ? atof(e) : dflt;
+}
+
+// ---- planning (dh_q4k_matmul_plan) ------------------------------------------------------------
+// While a plan is being made on this thread the dispatchers run as usual on the shape alone: ready()
+// holds, num_cus() is the planned device's count, and every launch site reports its kernel family
+// through plan_note() instead of launching (true = planning, return without touching the device).
+bool plan_note(int family);
+void plan_begin(int num_cus);
+int plan_end();
 
 // ---- kernel status word ---------------------------------------------------------------------
 // Kernels that wait on other waves or workgroups bound every such wait; a wave whose wait runs
@@ -87,6 +116,7 @@ struct GraphAttnCall {
   float eps, scale, softcap;
   int sliding_window, kv_start, kv_layout;
   void* ws;
+  size_t ws_capacity;      // bytes behind ws when the library knows them (its own scratch), else 0
   hipGraphNode_t split_node, merge_node;
 };
 // A dh_check_finiteness call recorded during a capture: its step number follows the position.
@@ -105,6 +135,7 @@ struct Graph {
   hipGraphExec_t exec = nullptr;
   int position = 0;                       // position the node parameters currently stand at
   int captured_position = 0;
+  int max_position = -1;                  // largest position the step's buffers cover, when the caller declared it
   GraphAttnCall* attn = nullptr;
   int n_attn = 0, cap_attn = 0;
   GraphFiniteCall* fin = nullptr;

@@ -22,6 +22,8 @@ constexpr size_t kPackedABytes = (size_t)64 << 20;
 float* g_widened_a = nullptr;        // f16 activations of dh_q4k_matmul widened to f32
 constexpr size_t kWidenedABytes = (size_t)64 << 20;
 uint32_t* g_kstatus = nullptr;       // kernel status word: pinned host memory, device-writable
+thread_local int t_plan_cus = 0;      // > 0: a plan is being made on this thread for a device of that many compute units
+thread_local int t_plan_family = 0;
 }  // namespace
 
 namespace dh {
@@ -33,8 +35,21 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 hipStream_t stream() { return g_stream; }
-bool ready() { return g_ready; }
-int num_cus() { return g_num_cus; }
+bool ready() { return g_ready || t_plan_cus > 0; }
+int num_cus() { return t_plan_cus > 0 ? t_plan_cus : g_num_cus; }
+void plan_begin(int cus) {
+  t_plan_cus = cus;
+  t_plan_family = 0;
+}
+int plan_end() {
+  t_plan_cus = 0;
+  return t_plan_family;
+}
+bool plan_note(int family) {
+  if (t_plan_cus <= 0) return false;
+  if (t_plan_family == 0) t_plan_family = family;
+  return true;
+}
 Graph* capturing_graph() { return g_capturing; }
 void graph_note_attention(const GraphAttnCall& call) {
   Graph* g = g_capturing;
@@ -104,6 +119,16 @@ static int release_all(const char* op) {
   auto note = [&](hipError_t e) {
     if (first == hipSuccess) first = e;
   };
+  if (g_capturing) {
+    // a capture left open: end it so the stream can be destroyed, and drop what it recorded
+    hipGraph_t abandoned = nullptr;
+    if (g_stream) (void)hipStreamEndCapture(g_stream, &abandoned);
+    if (abandoned) (void)hipGraphDestroy(abandoned);
+    delete[] g_capturing->attn;
+    delete[] g_capturing->fin;
+    delete g_capturing;
+    g_capturing = nullptr;
+  }
   if (g_own_stream) note(hipStreamDestroy(g_own_stream));
   if (g_splitk_ws) note(hipFree(g_splitk_ws));
   if (g_row_scale) note(hipFree(g_row_scale));
@@ -179,6 +204,7 @@ int dh_shutdown(void) {
 
 int dh_set_stream(void* hip_stream) {
   DH_REQUIRE_INIT("dh_set_stream");
+  if (g_capturing) return dh::fail(1, "[dh_set_stream] not possible while a graph is being captured (the capture belongs to the current stream)");
   g_stream = hip_stream ? static_cast<hipStream_t>(hip_stream) : g_own_stream;
   return 0;
 }
@@ -189,6 +215,7 @@ int dh_malloc(size_t bytes, void** d_out) {
   DH_REQUIRE_INIT("dh_malloc");
   if (!d_out) return dh::fail(1, "[dh_malloc] output pointer is null");
   *d_out = nullptr;
+  if (g_capturing) return dh::fail(1, "[dh_malloc] not possible while a graph is being captured (allocate the step's buffers before dh_graph_begin)");
   if (bytes == 0) return dh::fail(1, "[dh_malloc] size must be positive");
   DH_CHECK_HIP("dh_malloc", hipMalloc(d_out, bytes));
   return 0;
@@ -340,12 +367,25 @@ int dh_graph_end(int position, void** graph_out) {
   return 0;
 }
 
+int dh_graph_set_max_position(void* graph, int max_position) {
+  DH_REQUIRE_INIT("dh_graph_set_max_position");
+  dh::Graph* g = static_cast<dh::Graph*>(graph);
+  if (!g || !g->exec) return dh::fail(1, "[dh_graph_set_max_position] null graph");
+  if (max_position < g->captured_position)
+    return dh::fail(1, "[dh_graph_set_max_position] %d is below the captured position %d", max_position, g->captured_position);
+  g->max_position = max_position;
+  return 0;
+}
+
 int dh_graph_launch(void* graph, int position) {
   DH_REQUIRE_INIT("dh_graph_launch");
   dh::Graph* g = static_cast<dh::Graph*>(graph);
   if (!g || !g->exec) return dh::fail(1, "[dh_graph_launch] null graph");
   if (g_capturing) return dh::fail(1, "[dh_graph_launch] a capture is in progress");
   if (position < 0) return dh::fail(1, "[dh_graph_launch] position must be non-negative");
+  if (g->max_position >= 0 && position > g->max_position)
+    return dh::fail(1, "[dh_graph_launch] position %d is beyond the largest one the step's buffers were declared for (%d)",
+                    position, g->max_position);
   if (position != g->position) {
     if (int rc = dh::attn_graph_set_position(g, position)) return rc;
     if (int rc = dh::finite_graph_set_position(g, position)) return rc;
@@ -359,7 +399,11 @@ int dh_graph_prepare(void* graph, int position) {
   DH_REQUIRE_INIT("dh_graph_prepare");
   dh::Graph* g = static_cast<dh::Graph*>(graph);
   if (!g || !g->exec) return dh::fail(1, "[dh_graph_prepare] null graph");
+  if (g_capturing) return dh::fail(1, "[dh_graph_prepare] a capture is in progress");
   if (position < 0) return dh::fail(1, "[dh_graph_prepare] position must be non-negative");
+  if (g->max_position >= 0 && position > g->max_position)
+    return dh::fail(1, "[dh_graph_prepare] position %d is beyond the largest one the step's buffers were declared for (%d)",
+                    position, g->max_position);
   if (position != g->position) {
     if (int rc = dh::attn_graph_set_position(g, position)) return rc;
     if (int rc = dh::finite_graph_set_position(g, position)) return rc;

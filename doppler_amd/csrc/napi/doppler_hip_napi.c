@@ -93,6 +93,7 @@ FN(js_graph_end) {
   return ret_ptr(env, g);
 }
 FN(js_graph_launch) { ARGS(2); P(0, g); I(1, position); return ret_rc(env, dh_graph_launch(g, position)); }
+FN(js_graph_set_max_position) { ARGS(2); P(0, g); I(1, position); return ret_rc(env, dh_graph_set_max_position(g, position)); }
 FN(js_graph_prepare) { ARGS(2); P(0, g); I(1, position); return ret_rc(env, dh_graph_prepare(g, position)); }
 FN(js_graph_destroy) { ARGS(1); P(0, g); return ret_rc(env, dh_graph_destroy(g)); }
 
@@ -209,6 +210,20 @@ FN(js_attn_decode_qkv) {
                                         (const float*)s, ck, cv, (float*)O, H, Hkv, D, start, rd, inter, eps, woff,
                                         useNorm, scale, cap, win, kvStart, layout, ws));
 }
+FN(js_attn_decode_kvlen) {
+  ARGS(17); P(0, Q); P(1, K); P(2, V); P(3, O); I(4, H); I(5, Hkv); I(6, D); P(7, kvLenPtr); I(8, maxKvLen); F(9, scale);
+  I(10, causal); I(11, startPos); F(12, cap); I(13, win); I(14, kvStart); I(15, layout); P(16, ws);
+  return ret_rc(env, dh_attn_decode_kvlen((const float*)Q, K, V, (float*)O, H, Hkv, D, (const uint32_t*)kvLenPtr, maxKvLen,
+                                          scale, causal, startPos, cap, win, kvStart, layout, ws));
+}
+FN(js_attn_decode_qkv_kvlen) {
+  ARGS(24); P(0, qkv); P(1, qw); P(2, kw); P(3, c); P(4, s); P(5, ck); P(6, cv); P(7, O); I(8, H); I(9, Hkv); I(10, D);
+  P(11, kvLenPtr); I(12, maxKvLen); I(13, rd); I(14, inter); F(15, eps); I(16, woff); I(17, useNorm); F(18, scale);
+  F(19, cap); I(20, win); I(21, kvStart); I(22, layout); P(23, ws);
+  return ret_rc(env, dh_attn_decode_qkv_kvlen((const float*)qkv, (const float*)qw, (const float*)kw, (const float*)c,
+                                              (const float*)s, ck, cv, (float*)O, H, Hkv, D, (const uint32_t*)kvLenPtr,
+                                              maxKvLen, rd, inter, eps, woff, useNorm, scale, cap, win, kvStart, layout, ws));
+}
 FN(js_attn_prefill) {
   ARGS(14); P(0, Q); P(1, K); P(2, V); P(3, O); I(4, T); I(5, H); I(6, Hkv); I(7, D); I(8, kvLen); F(9, scale);
   I(10, causal); I(11, startPos); F(12, cap); I(13, win);
@@ -308,7 +323,7 @@ FN(js_check_finiteness) {
 
 static napi_value module_init(napi_env env, napi_value exports) {
   static const struct { const char* name; napi_callback fn; } table[] = {
-      {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end}, {"graphLaunch", js_graph_launch}, {"graphPrepare", js_graph_prepare},
+      {"graphBegin", js_graph_begin}, {"graphEnd", js_graph_end}, {"graphLaunch", js_graph_launch}, {"graphSetMaxPosition", js_graph_set_max_position}, {"graphPrepare", js_graph_prepare},
       {"graphDestroy", js_graph_destroy},
       {"init", js_init}, {"shutdown", js_shutdown}, {"sync", js_sync}, {"malloc", js_malloc}, {"free", js_free},
       {"upload", js_upload}, {"download", js_download}, {"copy", js_copy}, {"fillZero", js_fill_zero},
@@ -320,6 +335,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"attnDecodeWorkspaceBytes", js_attn_decode_workspace_bytes}, {"attnDecode", js_attn_decode},
       {"attnDecodeStatic", js_attn_decode_static}, {"attnDecodeStaticMaxBytes", js_attn_decode_static_max_bytes},
       {"attnDecodeQkvSupported", js_attn_decode_qkv_supported}, {"attnDecodeQkv", js_attn_decode_qkv},
+      {"attnDecodeKvLen", js_attn_decode_kvlen}, {"attnDecodeQkvKvLen", js_attn_decode_qkv_kvlen},
       {"attnPrefill", js_attn_prefill},
       {"rmsnorm", js_rmsnorm}, {"rmsnormQK", js_rmsnorm_qk}, {"rmsnormSandwichPair", js_rmsnorm_sandwich_pair},
       {"residualRmsnormPair", js_residual_rmsnorm_pair}, {"rope", js_rope}, {"ropeQK", js_rope_qk}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},

@@ -54,10 +54,7 @@ typedef __attribute__((ext_vector_type(2))) _Float16 half2_t;
 typedef __attribute__((ext_vector_type(16))) float float16_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
-int env_ksplit() {
-  const char* e = getenv("DH_GEMM_KSPLIT");
-  return e ? atoi(e) : 0;
-}
+int env_ksplit() { return dh::tuning_int("DH_GEMM_KSPLIT", 0); }
 
 constexpr int BK = 64;
 constexpr int LDS_ROW = BK + 8;                    // halves per LDS row (144 bytes)
@@ -602,16 +599,19 @@ template <bool DUAL>
 int launch_gemm(GemmArgs a, const char* op) {
   // rows beyond the capacity of the packed-activation scratch go in further passes
   a.kpad = (a.K + BK - 1) / BK * BK;
+  if (a.norm_weight && a.K > 16384)
+    return dh::fail(1, "[%s] the RMSNorm prologue serves K <= 16384 at M >= 16 (K=%d)", op, a.K);
+  // the kernel addresses a weight row as a 32-bit byte offset into a buffer descriptor
+  if ((int64_t)a.N * a.nb * kBlockBytes >= ((int64_t)1 << 31))
+    return dh::fail(1, "[%s] a weight tensor of %d x %d (2 GB or more) is beyond the prefill GEMM; split it by rows", op,
+                    a.N, a.K);
+  if (dh::plan_note(DH_PLAN_GEMM)) return 0;
   size_t pk_bytes = 0;
   _Float16* packed = reinterpret_cast<_Float16*>(dh::gemm_packed_a(&pk_bytes));
   float2* scales = reinterpret_cast<float2*>(dh::gemm_row_scale());
   if (!packed || !scales) return dh::fail(2, "[%s] the library's scratch buffers are missing (dh_init)", op);
   const int cap = (int)std::min<size_t>((size_t)dh::gemm_row_scale_capacity(), pk_bytes / ((size_t)a.kpad * 2));
   if (cap < 16) return dh::fail(1, "[%s] K=%d is too long for the prefill GEMM's activation scratch", op, a.K);
-  // the kernel addresses a weight row as a 32-bit byte offset into a buffer descriptor
-  if ((int64_t)a.N * a.nb * kBlockBytes >= ((int64_t)1 << 31))
-    return dh::fail(1, "[%s] a weight tensor of %d x %d (2 GB or more) is beyond the prefill GEMM; split it by rows", op,
-                    a.N, a.K);
   if (a.M > cap) {
     const size_t c_elem = a.c_f16 ? 2 : 4;
     for (int m0 = 0; m0 < a.M; m0 += cap) {
@@ -660,7 +660,7 @@ int launch_gemm(GemmArgs a, const char* op) {
   // waits; the pieces meet in the library's scratch buffer.
   if (!DUAL) {
     static const int env_split = env_ksplit();
-    static const int env_big = getenv("DH_GEMM_BIGSPLIT") ? atoi(getenv("DH_GEMM_BIGSPLIT")) : 1;
+    static const int env_big = dh::tuning_int("DH_GEMM_BIGSPLIT", 1);
     // 128 x 128 tiles with K cut into pieces when that fills the compute units: their matrix-core
     // share is higher than that of 64 x 64 tiles
     if (env_big) {

@@ -299,10 +299,7 @@ __device__ __forceinline__ void mfma_block(const WBlock& w, const _Float16* __re
   for (int k = 0; k < NO; k++) acc[k] += d * blk[k] - dmin * blk_min[k];
 }
 
-int env_int(const char* name, int dflt) {
-  const char* e = getenv(name);
-  return e ? atoi(e) : dflt;
-}
+int env_int(const char* name, int dflt) { return dh::tuning_int(name, dflt); }
 
 constexpr int kMaxDepth = 4;
 constexpr int kRedSlots = 4;       // tiles a fast wave may run ahead of the slowest one
@@ -739,13 +736,6 @@ int launch_ring_cfg(RingArgs a, const char* op, bool may_shorten_tiles) {
   constexpr int NO = MfmaShape<MT>::NI / 2, NMAT = DUAL ? 2 : 1;
   const size_t fixed = XBYTES + sizeof(float) * RingShape<MT>::RS * WAVES * NMAT * NO * RingShape<MT>::LW + 512;
   auto kern = q4k_gemv_ring_kernel<MT, DUAL, XBYTES, WAVES>;
-  static bool attr_set = false;   // once per instantiation: the call costs microseconds
-  if (!attr_set) {
-    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)(kRingMaxLds - fixed)));
-    attr_set = true;
-  }
   static const int env_rows = env_int("DH_GEMV_ROWS", 0), env_depth = env_int("DH_GEMV_DEPTH", 0);
   // rows per tile: the smallest count that covers N with a whole number of tiles per compute unit
   const int ncu = dh::num_cus();
@@ -765,6 +755,14 @@ int launch_ring_cfg(RingArgs a, const char* op, bool may_shorten_tiles) {
   a.depth = depth;
   const int64_t ntiles = dh::ceil_div(a.N, rows);
   const int grid = (int)std::min<int64_t>(ntiles, ncu);
+  if (dh::plan_note(DH_PLAN_GEMV_RING)) return 0;
+  static bool attr_set = false;   // once per instantiation: the call costs microseconds
+  if (!attr_set) {
+    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)(kRingMaxLds - fixed)));
+    attr_set = true;
+  }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), dyn, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   return 0;
@@ -847,6 +845,7 @@ template <int MT, bool DUAL>
 int launch_lds(const GemvArgs& a, const char* op) {
   const size_t lds = lds_bytes(MT, a.nb, DUAL);
   auto kern = q4k_gemv_lds_kernel<MT, DUAL>;
+  if (dh::plan_note(DH_PLAN_GEMV_LDS)) return 0;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
     DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -958,7 +957,7 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
   if ((path == 0 || normed) && M < 16) {
     // below the GEMM's batch size: passes of up to 8 rows, each one sweep over the weights
     int rc = 0;
-    for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
+    for (int m0 = 0; m0 < M && rc == 0; m0 += 8) {
       rc = dh::q4k_gemv_rows(op, a.A + (int64_t)m0 * K, a.W, nullptr, static_cast<char*>(d_C) + (int64_t)m0 * N * (a.c_f16 ? 2 : 4),
                              a.c_f16, a.residual ? a.residual + (int64_t)m0 * N : nullptr, std::min(8, M - m0), N, K, alpha, 0,
                              0.f, normed ? d_norm_weight : nullptr, eps, weight_offset);
@@ -969,7 +968,7 @@ static int q4k_matmul_impl(const char* op, const void* d_A, int a_dtype, const f
   if ((path == 0 || normed) && M < 16) {
     // below the GEMM's batch size: passes of up to 8 rows through the streaming GEMV
     int rc = 0;
-    for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
+    for (int m0 = 0; m0 < M && rc == 0; m0 += 8) {
       RingArgs g{};
       g.A = a.A + (int64_t)m0 * K; g.W = a.W; g.W2 = nullptr;
       g.C = static_cast<char*>(d_C) + (int64_t)m0 * N * (a.c_f16 ? 2 : 4);
@@ -1078,7 +1077,7 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
   }
   if ((path == 0 || normed) && M < 16) {
     int rc = 0;
-    for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
+    for (int m0 = 0; m0 < M && rc == 0; m0 += 8) {
       rc = dh::q4k_gemv_rows(op, d_x + (int64_t)m0 * hidden, a.W, a.W2, d_out + (int64_t)m0 * inter, 0, nullptr,
                              std::min(8, M - m0), inter, hidden, alpha, activation, swiglu_limit,
                              normed ? d_norm_weight : nullptr, eps, weight_offset);
@@ -1088,7 +1087,7 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
   }
   if ((path == 0 || normed) && M < 16) {
     int rc = 0;
-    for (int m0 = 0; m0 < M && rc >= 0; m0 += 8) {
+    for (int m0 = 0; m0 < M && rc == 0; m0 += 8) {
       RingArgs g{};
       g.A = d_x + (int64_t)m0 * hidden; g.W = a.W; g.W2 = a.W2; g.C = d_out + (int64_t)m0 * inter; g.residual = nullptr;
       g.M = std::min(8, M - m0); g.N = inter; g.K = hidden; g.nb = a.nb; g.alpha = alpha; g.c_f16 = 0;
@@ -1117,6 +1116,23 @@ static int q4k_ffn_impl(const char* op, const float* d_x, const float* d_norm_we
     if (rc) return rc;
   }
   return 0;
+}
+
+int dh_q4k_matmul_plan(int M, int N, int K, int normed, int dual, int num_cus) {
+  const char* op = "dh_q4k_matmul_plan";
+  if (num_cus <= 0) num_cus = dh::ready() ? dh::num_cus() : 256;
+  dh::plan_begin(num_cus);
+  // the dispatchers look at shapes, alignment and null-ness only: stand-in addresses, never touched
+  const float* x = reinterpret_cast<const float*>(uintptr_t{1} << 20);
+  const void* w = reinterpret_cast<const void*>(uintptr_t{2} << 20);
+  float* c = reinterpret_cast<float*>(uintptr_t{3} << 20);
+  int rc;
+  if (dual)
+    rc = q4k_ffn_impl(op, x, normed ? x : nullptr, 1e-6f, 0, normed != 0, w, w, c, M, K, N, DH_ACT_SILU, 1.0f, 0.0f);
+  else
+    rc = q4k_matmul_impl(op, x, DH_F32, normed ? x : nullptr, 1e-6f, 0, normed != 0, w, c, DH_F32, M, N, K, 1.0f, nullptr);
+  const int family = dh::plan_end();
+  return rc == 0 ? family : 0;
 }
 
 int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup, float* d_out, int M,

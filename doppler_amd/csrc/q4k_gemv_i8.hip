@@ -555,22 +555,13 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
 #undef DH_DECODE
 }
 
-int env_int(const char* name, int dflt) {
-  const char* e = getenv(name);
-  return e ? atoi(e) : dflt;
-}
+int env_int(const char* name, int dflt) { return dh::tuning_int(name, dflt); }
 
 template <int MT, bool DUAL, bool VEC>
 int launch_i8_vec(I8Args a, const char* op) {
   constexpr int NMAT = DUAL ? 2 : 1;
   size_t cap = kMaxLds;
   auto kern = q4k_gemv_i8_kernel<MT, DUAL, VEC>;
-  static bool attr_set = false;   // once per instantiation: the call costs microseconds
-  if (!attr_set) {
-    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)cap));
-    attr_set = true;
-  }
   static const int env_depth = env_int("DH_GEMV_DEPTH", 0);
   const int ncu = dh::num_cus();
   // rows per tile: the largest count <= 16 that gives every workgroup the same number of tiles
@@ -606,6 +597,13 @@ int launch_i8_vec(I8Args a, const char* op) {
   while (depth > 1 && lds_for(depth) > cap) depth--;
   if (lds_for(depth) > cap) return -1;
   a.depth = depth;
+  if (dh::plan_note(DH_PLAN_GEMV_I8)) return 0;
+  static bool attr_set = false;   // once per instantiation: the call costs microseconds
+  if (!attr_set) {
+    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)cap));
+    attr_set = true;
+  }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kWaves), lds_for(depth), dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   return 0;

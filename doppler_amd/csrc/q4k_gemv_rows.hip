@@ -532,21 +532,12 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
   }
 }
 
-int env_int(const char* name, int dflt) {
-  const char* e = getenv(name);
-  return e ? atoi(e) : dflt;
-}
+int env_int(const char* name, int dflt) { return dh::tuning_int(name, dflt); }
 
 template <bool DUAL, bool VEC>
 int launch_rows(RowsArgs a, const char* op) {
   constexpr int NMAT = DUAL ? 2 : 1;
   auto kern = q4k_gemv_rows_kernel<DUAL, VEC>;
-  static bool attr_set = false;   // once per instantiation: the call costs microseconds
-  if (!attr_set) {
-    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsCap));
-    attr_set = true;
-  }
   const int ncu = dh::num_cus();
   // rows per tile: the largest count <= 16 that gives every workgroup the same number of tiles
   const int per_cu = (int)dh::ceil_div(a.N, (int64_t)ncu * kTileRows);
@@ -571,6 +562,13 @@ int launch_rows(RowsArgs a, const char* op) {
   while (depth > 1 && lds_for(depth) > kLdsCap) depth--;
   if (lds_for(depth) > kLdsCap) return -1;
   a.depth = depth;
+  if (dh::plan_note(DH_PLAN_GEMV_ROWS)) return 0;
+  static bool attr_set = false;   // once per instantiation: the call costs microseconds
+  if (!attr_set) {
+    DH_CHECK_HIP(op, hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsCap));
+    attr_set = true;
+  }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kWaves), lds_for(depth), dh::stream(), a);
   DH_CHECK_LAUNCH(op);
   return 0;

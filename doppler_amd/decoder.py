@@ -103,6 +103,7 @@ class HipDecoder:
                                  device="cuda")
         self.scale = 1.0 / math.sqrt(D)
         self._host_token = np.zeros(1, np.uint32)
+        self._host_ids = np.zeros(2, np.uint32)
         torch.cuda.synchronize()
 
     def weight_bytes_per_token(self, ctx):
@@ -115,10 +116,13 @@ class HipDecoder:
             q4 += synth.q4k_nbytes(n, k)
         return c["layers"] * q4 + c["vocab"] * c["hidden"] * 2 + c["layers"] * 2 * self.ks * 2 * ctx
 
-    def enqueue_step(self, pos, want_logits=False, from_device_token=False, in_index=0, out_index=0):
+    def enqueue_step(self, pos, want_logits=False, from_device_token=False, in_index=0, out_index=0,
+                     device_kv_len=False):
         """Enqueue one decode step for the token id in self.ids[0] (or, when from_device_token,
         the argmax an earlier step left in self.token[in_index]) at position `pos`; the new
-        token goes to self.token[out_index].  No host synchronisation."""
+        token goes to self.token[out_index].  No host synchronisation.  device_kv_len: the
+        attention kernels take the key count (position + 1) from self.ids[1] instead of `pos`, so
+        that the enqueued step, captured into a graph, serves every later position as it is."""
         L, c = self.L, self.cfg
         ck = capi.check
         H, Hkv, D, Hd, I = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"], c["inter"]
@@ -141,7 +145,7 @@ class HipDecoder:
                                 c["eps"], 0, None, None, None, 1.0))
                 ck(L.dh_q4k_matmul(self.normed.data_ptr(), capi.F32, d["wqkv"].data_ptr(), self.qkv.data_ptr(),
                                    capi.F32, 1, self.qs + 2 * self.ks, Hd, 1.0, None))
-            self._enqueue_attention(d, pos)
+            self._enqueue_attention(d, pos, device_kv_len)
             ck(L.dh_q4k_matmul(self.attn.data_ptr(), capi.F32, d["wo"].data_ptr(), x2.data_ptr(), capi.F32, 1, Hd,
                                self.qs, 1.0, x.data_ptr()))
             if self.fuse_norm:
@@ -164,12 +168,21 @@ class HipDecoder:
                                   self.lm_ws.data_ptr(), self.token.data_ptr(), self._out_index,
                                   self.logits.data_ptr() if want_logits else None))
 
-    def _enqueue_attention(self, d, pos):
+    def _enqueue_attention(self, d, pos, device_kv_len=False):
         """self.qkv (raw stacked projection of the step's token) -> self.attn, appending the
         token's key/value to the layer's cache."""
         L, c, ck = self.L, self.cfg, capi.check
         H, Hkv, D = c["heads"], c["kv_heads"], c["head_dim"]
         use_norm = int(c.get("qk_norm", 1))
+        if device_kv_len:
+            if not self.fuse_qkv_attention:
+                raise ValueError("the device-side key count serves the fused attention kernel")
+            ck(L.dh_attn_decode_qkv_kvlen(self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
+                                          self.cos.data_ptr(), self.sin.data_ptr(), d["cache_k"].data_ptr(),
+                                          d["cache_v"].data_ptr(), self.attn.data_ptr(), H, Hkv, D,
+                                          self.ids.data_ptr() + 4, self.max_seq, D, 0, c["eps"], 0, use_norm, self.scale,
+                                          0.0, 0, 0, capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
+            return
         if self.fuse_qkv_attention:
             ck(L.dh_attn_decode_qkv(self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(),
                                     self.cos.data_ptr(), self.sin.data_ptr(), d["cache_k"].data_ptr(),
@@ -184,9 +197,11 @@ class HipDecoder:
                             self.attn.data_ptr(), H, Hkv, D, pos + 1, self.scale, 1, pos, 0.0, 0, 0,
                             capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
 
-    def set_token(self, token):
-        self._host_token[0] = token
-        capi.check(self.L.dh_upload(self.ids.data_ptr(), 0, self._host_token.ctypes.data, 4))
+    def set_token(self, token, kv_len=None):
+        """Token id of the step (and, for a captured step, its key count beside it: one upload)."""
+        self._host_ids[0] = token
+        self._host_ids[1] = 0 if kv_len is None else kv_len
+        capi.check(self.L.dh_upload(self.ids.data_ptr(), 0, self._host_ids.ctypes.data, 4 if kv_len is None else 8))
 
     def read_token(self):
         capi.check(self.L.dh_download(self._host_token.ctypes.data, self.token.data_ptr(), 0, 4))
@@ -222,11 +237,14 @@ class HipDecoder:
         self._raise_if_triggered(words, 1, "generation")
         return int(words[0])
 
-    def capture_step(self, pos, want_logits=False):
+    def capture_step(self, pos, want_logits=False, device_kv_len=True):
         """Captures one decode step (enqueued for position `pos`) into a HIP graph, the
         counterpart of the reference's one-submit-per-step recorder
         (src/inference/pipelines/text/generator-steps.js:605,814).  The step is run once
-        normally first so that every kernel's one-time set-up is done outside the capture."""
+        normally first so that every kernel's one-time set-up is done outside the capture.
+        device_kv_len: the captured attention launches read the key count from the word beside the
+        token id (the reference's kvLenBuffer), so a replay patches nothing; False keeps the
+        position in the launch arguments, which the library then moves before every replay."""
         if not self.fuse_qkv_attention:
             raise ValueError("capture_step serves the step with the fused attention kernel")
         # with the guard on the captured step also clears the status words and leaves its token next
@@ -234,15 +252,20 @@ class HipDecoder:
         out_index = self.TOKEN_RING - 1 if self.finiteness_guard else 0
         self.enqueue_step(pos, want_logits, out_index=out_index)
         capi.check(self.L.dh_sync())
+        self._graph_device_kv_len = bool(device_kv_len)
         capi.check(self.L.dh_graph_begin())
+        g = ctypes.c_void_p()
         try:
             if self.finiteness_guard:
                 self._reset_finiteness()
-            self.enqueue_step(pos, want_logits, out_index=out_index)
-        finally:
-            g = ctypes.c_void_p()
-            rc = self.L.dh_graph_end(pos, ctypes.byref(g))
-        capi.check(rc)
+            self.enqueue_step(pos, want_logits, out_index=out_index, device_kv_len=device_kv_len)
+        except BaseException:
+            # the capture must be closed either way; a graph that came out of it is not kept
+            if self.L.dh_graph_end(pos, ctypes.byref(g)) == 0 and g.value:
+                self.L.dh_graph_destroy(g)
+            raise
+        capi.check(self.L.dh_graph_end(pos, ctypes.byref(g)))
+        capi.check(self.L.dh_graph_set_max_position(g, self.max_seq - 1))
         self._graph = g
         return g
 
@@ -253,9 +276,9 @@ class HipDecoder:
             raise ValueError("decode position %d is outside the KV cache (max_seq=%d)" % (pos, self.max_seq))
         if getattr(self, "_graph", None) is None:
             self.capture_step(pos)
-        self.set_token(token)
+        self.set_token(token, pos + 1)
         capi.check(self.L.dh_graph_launch(self._graph, pos))
-        if pos + 1 < self.max_seq:
+        if pos + 1 < self.max_seq and not self._graph_device_kv_len:
             # the next position's node parameters are set while the GPU runs this one
             capi.check(self.L.dh_graph_prepare(self._graph, pos + 1))
         if not self.finiteness_guard:

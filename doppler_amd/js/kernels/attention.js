@@ -18,6 +18,7 @@ async function executeAttention(recorder, Q, K, V, mask, numHeads, headDim, opti
     slidingWindow = 0,
     kvStart = 0,
     kvLayout = 'contiguous',
+    kvLenBuffer = null,
   } = options;
   if (!(seqLen >= 1)) {
     throw new Error(`[Attention] seqLen must be positive, got ${seqLen}.`);
@@ -37,6 +38,12 @@ async function executeAttention(recorder, Q, K, V, mask, numHeads, headDim, opti
     throw new Error(`[Attention] KV buffers are smaller than kvLen=${kvLen} rows (${kvBytes} bytes).`);
   }
   const native = getNative();
+  if (kvLenBuffer && seqLen > 1) {
+    throw new Error(`[Attention] kvLenBuffer is served for decode (seqLen 1) only, got seqLen=${seqLen}.`);
+  }
+  if (kvLenBuffer && !(kvLenBuffer.size >= 4)) {
+    throw new Error('[Attention] kvLenBuffer must hold one u32.');
+  }
   if (seqLen > 1) {
     if (kvLayout !== 'contiguous' || kvStart !== 0) {
       throw new Error(`[Attention] prefill (seqLen=${seqLen}) needs a contiguous cache with kvStart=0.`);
@@ -58,8 +65,16 @@ async function executeAttention(recorder, Q, K, V, mask, numHeads, headDim, opti
   const workspace = acquireBuffer(native.attnDecodeWorkspaceBytes(numHeads, headDim, Math.max(kvLen, 1)), undefined,
     'attention_splitk_workspace');
   try {
-    native.attnDecode(Q.buffer.ptr, K.buffer.ptr, V.buffer.ptr, output.ptr, numHeads, numKVHeads, headDim, kvLen,
-      scale, causal ? 1 : 0, startPos, attnSoftcap, slidingWindow, kvStart, KV_LAYOUT[kvLayout], workspace.ptr);
+    if (kvLenBuffer) {
+      // the key count is read on the device (reference: kv_len_source == 1); kvLen bounds it, and
+      // startPos < 0 places the query at the last key (a decode step replayed for the next token)
+      native.attnDecodeKvLen(Q.buffer.ptr, K.buffer.ptr, V.buffer.ptr, output.ptr, numHeads, numKVHeads, headDim,
+        kvLenBuffer.ptr, Math.max(kvLen, 1), scale, causal ? 1 : 0, startPos, attnSoftcap, slidingWindow, kvStart,
+        KV_LAYOUT[kvLayout], workspace.ptr);
+    } else {
+      native.attnDecode(Q.buffer.ptr, K.buffer.ptr, V.buffer.ptr, output.ptr, numHeads, numKVHeads, headDim, kvLen,
+        scale, causal ? 1 : 0, startPos, attnSoftcap, slidingWindow, kvStart, KV_LAYOUT[kvLayout], workspace.ptr);
+    }
   } catch (error) {
     if (owned) releaseBuffer(owned);
     releaseBuffer(workspace);

@@ -194,7 +194,9 @@ export class HipTextDecoder {
       let attn;
       if (this.fuseQkvAttention) {
         attn = temp(await recordDecodeAttentionFromQKV(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps,
-          l.cacheK, l.cacheV, { numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim, startPos: pos, layerIdx: li }));
+          l.cacheK, l.cacheV, { numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim, startPos: pos, layerIdx: li,
+            // a captured step reads the key count from the word behind the token id, so a replay needs no patching
+            kvLenBuffer: options.deviceKvLen ? bufferWindow(this.ids, 4, 4) : null, maxKvLen: c.maxSeq }));
       } else {
         const split = await recordSplitQKVRMSNormRoPEQK(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps, {
           numTokens: 1, numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim,
@@ -254,7 +256,9 @@ export class HipTextDecoder {
   // uses stay allocated for the graph's life.
   async captureDecodeStep(token, pos) {
     if (!this.fuseQkvAttention) throw new Error('[captureDecodeStep] serves the fused-attention step');
+    const c = this.config;
     const first = await this.decodeStep(token, pos);
+    uploadData(this.ids, new Uint32Array([token, pos + 1]));
     getNative().graphBegin();
     let graph = null;
     const temps = [];
@@ -262,10 +266,11 @@ export class HipTextDecoder {
       // with the guard on the captured step also clears the status words (the library moves the
       // checks' step number with the position at every replay)
       if (this.finitenessGuard) getNative().fillZero(this.tokenOut.ptr, 4, FINITENESS_STATUS_BYTES);
-      await this.recordDecodeStep(createCommandRecorder('decode_capture'), temps, pos, {});
+      await this.recordDecodeStep(createCommandRecorder('decode_capture'), temps, pos, { deviceKvLen: true });
     } finally {
       graph = getNative().graphEnd(pos);
     }
+    getNative().graphSetMaxPosition(graph, c.maxSeq - 1);
     this.graph = graph;
     this.graphBuffers = temps;
     return first;
@@ -278,10 +283,9 @@ export class HipTextDecoder {
       throw new Error(`[decodeStepGraph] position ${pos} is outside the KV cache (maxSeq=${c.maxSeq})`);
     }
     if (!this.graph) return this.captureDecodeStep(token, pos);
-    uploadData(this.ids, new Uint32Array([token]));
+    // token id and key count travel together; the attention kernels of the captured step read the count
+    uploadData(this.ids, new Uint32Array([token, pos + 1]));
     getNative().graphLaunch(this.graph, pos);
-    // the next position's node parameters are set while the GPU runs this one
-    if (pos + 1 < c.maxSeq) getNative().graphPrepare(this.graph, pos + 1);
     const bytes = await readBufferSlice(this.tokenOut, 0, this.finitenessGuard ? 4 + FINITENESS_STATUS_BYTES : 4);
     const words = new Uint32Array(bytes);
     if (this.finitenessGuard) {

@@ -404,9 +404,11 @@ def attentionWorkspaceBytes(numHeads, headDim, kvLen):
 
 def runAttention(Q, K, V, mask, numHeads, headDim, seqLen=1, kvLen=None, numKVHeads=None, scale=None,
                  causal=True, startPos=0, outputBuffer=None, attnSoftcap=0, slidingWindow=0, kvStart=0,
-                 kvLayout="contiguous", workspace=None, **_ignored):
+                 kvLayout="contiguous", workspace=None, kvLenBuffer=None, **_ignored):
     """src/gpu/kernels/attention.js:2007 runAttention over an f16 KV cache: decode (seqLen == 1,
-    split-K kernel) or prefill (seqLen > 1, matrix-core flash kernel)."""
+    split-K kernel) or prefill (seqLen > 1, matrix-core flash kernel).  kvLenBuffer (decode only): a
+    device u32 holding the key count, read by the kernels (attention.js:1071,1224-1232); kvLen then
+    bounds it, and startPos < 0 places the query at the last key."""
     kvLen = seqLen if kvLen is None else kvLen
     numKVHeads = numHeads if numKVHeads is None else numKVHeads
     scale = 1.0 / math.sqrt(headDim) if scale is None else scale
@@ -419,6 +421,10 @@ def runAttention(Q, K, V, mask, numHeads, headDim, seqLen=1, kvLen=None, numKVHe
     layouts = {"contiguous": capi.KV_CONTIGUOUS, "ring": capi.KV_RING}
     if kvLayout not in layouts:
         raise DopplerHipError("[Attention] kvLayout %r is not supported by the HIP path" % (kvLayout,))
+    if kvLenBuffer is not None and seqLen > 1:
+        raise DopplerHipError("[Attention] kvLenBuffer is served for decode (seqLen 1) only, got seqLen=%d" % seqLen)
+    if kvLenBuffer is not None and _nbytes(kvLenBuffer) < 4:
+        raise DopplerHipError("[Attention] kvLenBuffer must hold one u32")
     if seqLen > 1:
         if kvLayout != "contiguous" or kvStart != 0:
             raise DopplerHipError("[Attention] prefill (seqLen=%d) needs a contiguous cache with kvStart=0" % seqLen)
@@ -437,9 +443,14 @@ def runAttention(Q, K, V, mask, numHeads, headDim, seqLen=1, kvLen=None, numKVHe
     L = _lib()
     if workspace is None:
         workspace = acquireBuffer(attentionWorkspaceBytes(numHeads, headDim, max(kvLen, 1)))
-    capi.check(L.dh_attn_decode(_ptr(Q), _ptr(K), _ptr(V), out.data_ptr(), numHeads, numKVHeads, headDim, kvLen,
-                                scale, int(bool(causal)), startPos, float(attnSoftcap), slidingWindow, kvStart,
-                                layouts[kvLayout], _ptr(workspace)))
+    if kvLenBuffer is not None:
+        capi.check(L.dh_attn_decode_kvlen(_ptr(Q), _ptr(K), _ptr(V), out.data_ptr(), numHeads, numKVHeads, headDim,
+                                          _ptr(kvLenBuffer), max(kvLen, 1), scale, int(bool(causal)), startPos,
+                                          float(attnSoftcap), slidingWindow, kvStart, layouts[kvLayout], _ptr(workspace)))
+    else:
+        capi.check(L.dh_attn_decode(_ptr(Q), _ptr(K), _ptr(V), out.data_ptr(), numHeads, numKVHeads, headDim, kvLen,
+                                    scale, int(bool(causal)), startPos, float(attnSoftcap), slidingWindow, kvStart,
+                                    layouts[kvLayout], _ptr(workspace)))
     return Tensor(out, "f32", (seqLen, numHeads, headDim), "attention_output")
 
 

@@ -173,17 +173,23 @@ class Artifact:
                                 (index, os.path.getsize(path), info["size"]))
             f = open(path, "rb")
             m = (f, mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_READ))
-            if self.verify_hashes and info["hash"]:
-                algorithm = self.manifest.get("hashAlgorithm")
-                if algorithm != "sha256":
-                    raise RdrrError("Shard %d carries a %r hash, which this loader cannot check "
-                                    "(pass verify_hashes=False to load it unchecked)" % (index, algorithm))
-                h = hashlib.sha256()
-                for at in range(0, info["size"], 64 << 20):
-                    h.update(m[1][at:at + (64 << 20)])
-                if h.hexdigest() != info["hash"].lower():
-                    raise RdrrError("Shard %d fails its sha256 check (manifest %s, file %s)" %
-                                    (index, info["hash"], h.hexdigest()))
+            try:
+                if self.verify_hashes and info["hash"]:
+                    algorithm = self.manifest.get("hashAlgorithm")
+                    if algorithm != "sha256":
+                        raise RdrrError("Shard %d carries a %r hash, which this loader cannot check "
+                                        "(pass verify_hashes=False to load it unchecked)" % (index, algorithm))
+                    h = hashlib.sha256()
+                    for at in range(0, info["size"], 64 << 20):
+                        h.update(m[1][at:at + (64 << 20)])
+                    if h.hexdigest() != info["hash"].lower():
+                        raise RdrrError("Shard %d fails its sha256 check (manifest %s, file %s)" %
+                                        (index, info["hash"], h.hexdigest()))
+            except BaseException:
+                # a shard that is refused is not kept open
+                m[1].close()
+                f.close()
+                raise
             self._maps[index] = m
         return m[1]
 

@@ -80,6 +80,15 @@ int dh_event_destroy(void* ev);
 int dh_graph_begin(void);
 int dh_graph_end(int position, void** graph_out);
 int dh_graph_launch(void* graph, int position);
+/* A replay at a later position appends further cache rows, reads further rotary rows and may cut the
+ * keys into more splits than the captured call did: the caches, the rotary tables and every
+ * d_workspace of the captured step must cover the LARGEST position the graph will be launched at
+ * (workspaces sized with dh_attn_decode_workspace_bytes for that position's key count).
+ * dh_graph_set_max_position declares that position; launches and preparations beyond it then fail
+ * with a message instead of writing past those buffers.  (Attention calls that take their key count
+ * from device memory, dh_attn_decode_kvlen / dh_attn_decode_qkv_kvlen, carry their own bound and need
+ * no patching at all.) */
+int dh_graph_set_max_position(void* graph, int max_position);
 /* Moves the step to `position` without launching it: a later dh_graph_launch at that position
  * then has nothing left to patch.  Launches already enqueued keep the position they were launched
  * at, so a host can prepare position p + 1 while the GPU still runs position p. */
@@ -101,8 +110,8 @@ int dh_q4k_dequant(const void* d_W, int64_t num_blocks, float* d_out);
  * passes when they do not fit, and the product accumulates in f32 either way.  C is f32 or
  * f16 (c_dtype); the residual is f32.  K need not be a multiple of 256: the padded tail of each row's last
  * block is ignored.  d_residual (may be NULL) is added after alpha, as the reference's
- * `residualTensor` option does.  M = 1..8 takes the HBM-bound GEMV path, larger M the
- * MFMA GEMM path (from 16 rows on a weight tensor must be smaller than 2 GB, as the kernel
+ * `residualTensor` option does.  M = 1..15 takes an HBM-bound GEMV path, M >= 16 the
+ * MFMA GEMM path (dh_q4k_matmul_plan tells which kernel family; from 16 rows on a weight tensor must be smaller than 2 GB, as the kernel
  * addresses it through one buffer descriptor; a larger one fails with a message). */
 int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int c_dtype,
                   int M, int N, int K, float alpha, const void* d_residual);
@@ -118,6 +127,19 @@ int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int 
 int dh_q4k_matmul_rmsnorm(const float* d_A, const float* d_norm_weight, float eps,
                           int weight_offset, const void* d_W, void* d_C, int c_dtype, int M,
                           int N, int K, float alpha, const void* d_residual);
+
+/* Which kernel family dh_q4k_matmul / dh_q4k_matmul_rmsnorm (dual = 0) or dh_q4k_ffn_gate_up[_rmsnorm]
+ * (dual = 1; N = intermediate size, K = hidden size) takes for f32 activations of this shape, without
+ * launching anything: the dispatch of src/gpu/kernels/matmul-selection.js:427-667
+ * selectMatmulVariantAndFlags made visible.  Needs no device: num_cus is the compute-unit count to
+ * plan for (<= 0: the initialised device's, or 256).  Returns a DH_PLAN_* family, or 0 with a message
+ * in dh_last_error() when no kernel serves the shape. */
+#define DH_PLAN_GEMV_I8 1    /* M <= 2: int8 matrix cores, activations as block fixed point */
+#define DH_PLAN_GEMV_ROWS 2  /* M = 3..15: f16 matrix cores, one sweep over the weights per 8 rows */
+#define DH_PLAN_GEMV_RING 3  /* few work units per workgroup: a tile's columns spread over the waves */
+#define DH_PLAN_GEMM 4       /* M >= 16: f16 matrix-core GEMM */
+#define DH_PLAN_GEMV_LDS 5   /* f32 vector GEMV, activations staged in LDS: last resort */
+int dh_q4k_matmul_plan(int M, int N, int K, int normed, int dual, int num_cus);
 
 /* out[M,inter] = clamp(act(x.Wgate^T) * (x.Wup^T) * alpha).
  * Replaces runFusedFFN/recordFusedFFN, src/gpu/kernels/fused_ffn.js:501,605
@@ -242,6 +264,30 @@ int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float*
                        int interleaved, float eps, int weight_offset, int use_norm, float scale,
                        float softcap, int sliding_window, int kv_start, int kv_layout,
                        void* d_workspace);
+
+/* ---- decode attention with the key count in device memory ----
+ * The reference's `kvLenBuffer` option of runAttention (src/gpu/kernels/attention.js:1071,1224-1232;
+ * attention_decode_online_f16kv.wgsl:27,39,55-58 get_kv_len with kv_len_source == 1): the number of
+ * cached keys is read by the kernels from a u32 in device memory, so a recorded decode step can be
+ * replayed for the next token without touching its launch arguments.  d_kv_len points at that
+ * word; max_kv_len bounds it (larger values are clamped): the caches, the rotary tables and
+ * d_workspace (dh_attn_decode_workspace_bytes(H, D, max_kv_len), always required) must cover it,
+ * and the launch holds the key splits of max_kv_len, of which the surplus exits at once.
+ * dh_attn_decode_kvlen: start_pos >= 0 is the query's position as in dh_attn_decode; start_pos < 0
+ * places the query at the last key, kv_start + kv_len - 1 (what a decode step means).  A key count of
+ * zero gives a zero output.
+ * dh_attn_decode_qkv_kvlen: dh_attn_decode_qkv for the token at position kv_start + kv_len - 1 (its
+ * rotary row, its appended cache row); the key count must be at least 1. */
+int dh_attn_decode_kvlen(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H, int Hkv,
+                         int D, const uint32_t* d_kv_len, int max_kv_len, float scale, int causal,
+                         int start_pos, float softcap, int sliding_window, int kv_start, int kv_layout,
+                         void* d_workspace);
+int dh_attn_decode_qkv_kvlen(const float* d_qkv, const float* d_q_weight, const float* d_k_weight,
+                             const float* d_cos, const float* d_sin, void* d_cache_k, void* d_cache_v,
+                             float* d_O, int H, int Hkv, int D, const uint32_t* d_kv_len,
+                             int max_kv_len, int rotary_dim, int interleaved, float eps,
+                             int weight_offset, int use_norm, float scale, float softcap,
+                             int sliding_window, int kv_start, int kv_layout, void* d_workspace);
 
 /* ---- normalisation / rotary / KV ---- */
 

@@ -147,6 +147,23 @@ async function main() {
         tensor(c.V, 'f16', [c.kvLen, c.kvHeads, c.headDim]), null, c.heads, c.headDim,
         { seqLen: 1, kvLen: c.kvLen, numKVHeads: c.kvHeads, causal: true, startPos: c.kvLen - 1 });
       await save(out, t.buffer, c.heads * c.headDim * 4);
+    } else if (c.op === 'attention_kvlen_buffer') {
+      // the key count comes from a device u32 (kvLenBuffer); kvLen only bounds it
+      const lenBuf = dh.acquireBuffer(4);
+      dh.uploadData(lenBuf, new Uint32Array([c.count]));
+      const t = await dh.runAttention(tensor(c.Q, 'f32', [c.heads, c.headDim]), tensor(c.K, 'f16', [c.kvLen, c.kvHeads, c.headDim]),
+        tensor(c.V, 'f16', [c.kvLen, c.kvHeads, c.headDim]), null, c.heads, c.headDim,
+        { seqLen: 1, kvLen: c.kvLen, numKVHeads: c.kvHeads, causal: true, startPos: -1, kvLenBuffer: lenBuf });
+      await save(out, t.buffer, c.heads * c.headDim * 4);
+      let refused = false;
+      try {
+        await dh.runAttention(tensor(c.Q, 'f32', [c.heads, c.headDim]), tensor(c.K, 'f16', [c.kvLen, c.kvHeads, c.headDim]),
+          tensor(c.V, 'f16', [c.kvLen, c.kvHeads, c.headDim]), null, c.heads, c.headDim,
+          { seqLen: 2, kvLen: c.kvLen, numKVHeads: c.kvHeads, kvLenBuffer: lenBuf });
+      } catch (error) {
+        refused = /kvLenBuffer/.test(error.message);
+      }
+      if (!refused) throw new Error('prefill with kvLenBuffer should be refused by name');
     } else if (c.op === 'attention_from_qkv') {
       // cache pre-filled with history rows; the op appends the row of startPos itself
       const keys = tensor(c.K, 'f16', [c.maxSeq, c.kvHeads, c.headDim]);

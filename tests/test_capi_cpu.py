@@ -81,3 +81,42 @@ def test_fused_matmul_rmsnorm_selection_follows_the_reference_rules():
     assert ops.shouldUseFusedMatmulRMSNorm(1, 4097, 1024) is False
     assert ops.shouldUseFusedMatmulRMSNorm(1, 1152, 8193) is False
     assert ops.shouldUseFusedMatmulRMSNorm(1, 1152) is True
+
+
+def test_matmul_plan_pins_the_kernel_family_of_every_benchmark_shape():
+    """dh_q4k_matmul_plan needs no device: the family each BASELINE shape (and the shapes on either
+    side of every dispatch boundary) is served by, so that a regression onto a slower family shows
+    up here and not only as a number in a benchmark."""
+    L = capi.load()
+    I8, ROWS, RING, GEMM, LDS = (capi.PLAN_GEMV_I8, capi.PLAN_GEMV_ROWS, capi.PLAN_GEMV_RING, capi.PLAN_GEMM,
+                                 capi.PLAN_GEMV_LDS)
+
+    def plan(M, N, K, normed=0, dual=0, cus=256):
+        return L.dh_q4k_matmul_plan(M, N, K, normed, dual, cus)
+
+    # config 0: one 640 -> 2048 product
+    assert plan(1, 2048, 640) == I8
+    # config 1: the linear layers of a hidden-1024 block at M = 1, 2, 4, 8
+    for N, K in ((2048, 1024), (1024, 1024), (1024, 2048), (3072, 1024)):
+        assert [plan(M, N, K) for M in (1, 2, 4, 8)] == [I8, I8, RING, RING], (N, K)
+    assert [plan(M, 3072, 1024, 1, 1) for M in (1, 2, 4, 8)] == [I8, I8, RING, RING]
+    assert [plan(M, 1024, 3072) for M in (1, 2, 4, 8)] == [I8, I8, ROWS, ROWS]
+    # config 2: prefill FFN at M = 512
+    assert plan(512, 6912, 1152, 0, 1) == GEMM and plan(512, 1152, 6912) == GEMM
+    # config 4: the decoder's products (normed q/k/v, o, normed gate/up pair, down), M across every boundary
+    for N, K, normed, dual in ((6144, 4096, 1, 0), (4096, 4096, 0, 0), (12288, 4096, 1, 1), (4096, 12288, 0, 0)):
+        got = [plan(M, N, K, normed, dual) for M in (1, 2, 3, 8, 9, 15, 16, 2048)]
+        assert got == [I8, I8, ROWS, ROWS, ROWS, ROWS, GEMM, GEMM], (N, K, got)
+    # rows longer than the int8 kernel's LDS holds with the RMSNorm prologue go to the few-row kernel
+    assert [plan(M, 4096, 32768, 1, 0) for M in (1, 2, 3)] == [ROWS, ROWS, ROWS]
+    assert plan(1, 4096, 28160, 1, 0) == I8 and plan(1, 4096, 28416, 1, 0) == ROWS
+    # K off the vector path, tiny shapes
+    assert plan(1, 512, 1023) == I8 and plan(4, 512, 1023) == RING and plan(16, 512, 1023) == GEMM
+    assert plan(1, 8, 256) == RING and plan(5, 8, 256) == RING      # one column per tile: too many tile slots for the int8 kernel
+    # a device with a quarter of the compute units: more tiles per workgroup; the few-row kernel's
+    # per-tile accumulators then no longer fit the LDS for the gate/up pair
+    assert plan(1, 12288, 4096, 1, 1, cus=64) == I8 and plan(8, 12288, 4096, 1, 1, cus=64) == RING
+    assert plan(8, 4096, 4096, 0, 0, cus=64) == ROWS
+    # what nothing serves fails with a message instead of a family
+    assert plan(16, 4096, 40000, 1, 0) == 0 and b"K <= 16384" in L.dh_last_error()
+    assert plan(0, 8, 256) == 0 and b"Dimensions must be positive" in L.dh_last_error()

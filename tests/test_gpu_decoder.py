@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import oracle
-from doppler_amd import decoder, synth
+from doppler_amd import capi, decoder, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -382,12 +382,14 @@ def test_decode_positions_outside_the_cache_are_refused():
     dict(layers=2, hidden=256, inter=512, heads=4, kv_heads=2, head_dim=64, vocab=300, eps=1e-6, qk_norm=1),
     dict(layers=3, hidden=1024, inter=3072, heads=16, kv_heads=8, head_dim=128, vocab=2000, eps=1e-6, qk_norm=1),
 ])
-def test_graph_replayed_steps_give_the_oracle_tokens(cfg):
-    """The decode step captured once into a HIP graph and replayed at every later position (its
-    attention nodes are moved to the position before each launch) against the CPU oracle: tokens
-    identical and logits within 1e-3 at every step, across positions where the number of key
-    splits changes (64-key chunk boundaries), with eager steps and synchronisations between
-    replays."""
+@pytest.mark.parametrize("device_kv_len", [True, False], ids=["key-count-on-device", "nodes-patched"])
+def test_graph_replayed_steps_give_the_oracle_tokens(cfg, device_kv_len):
+    """The decode step captured once into a HIP graph and replayed at every later position against
+    the CPU oracle: tokens identical and logits within 1e-3 at every step, across positions where
+    the number of key splits changes (64-key chunk boundaries), with eager steps and
+    synchronisations between replays.  Either the attention kernels read the key count from a
+    device word that travels with the token id (nothing is patched between replays), or the
+    library moves its attention nodes to the position before each launch."""
     max_seq = 200
     cfg = dict(cfg, max_seq=max_seq, theta=1e6)
     layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=61, max_seq=max_seq)
@@ -400,7 +402,7 @@ def test_graph_replayed_steps_give_the_oracle_tokens(cfg):
         inp = int(prompt[pos])
         tok = gpu.step(inp, pos)
         assert tok == cpu.step(inp, pos), pos
-    gpu.capture_step(60, want_logits=True)      # runs position 60 eagerly once, then captures it
+    gpu.capture_step(60, want_logits=True, device_kv_len=device_kv_len)      # runs position 60 eagerly once, then captures it
     for pos in range(60, 180):
         inp = int(prompt[pos]) if pos < len(prompt) else tok
         if pos % 7 == 3:                        # an eager step between replays
@@ -411,6 +413,11 @@ def test_graph_replayed_steps_give_the_oracle_tokens(cfg):
         assert rel_l2(gpu.read_logits(), want) <= 1e-3, pos
         assert g == ctok, (pos, g, ctok)
         tok = g
+    # positions beyond what the step's buffers were declared for are refused before anything is launched
+    with pytest.raises(ValueError):
+        gpu.step_graph(1, max_seq)
+    with pytest.raises(capi.DopplerHipError, match="beyond the largest"):
+        capi.check(gpu.L.dh_graph_launch(gpu._graph, max_seq))
     gpu.release_graph()
 
 

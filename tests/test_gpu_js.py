@@ -278,6 +278,11 @@ def test_js_host_path_parity(tmp_path):
                       kvHeads=8, headDim=128, kvLen=ctx))
     attn_want = oracle.attention_decode_f16kv(q, kb, vb, 16, 8, 128, ctx)
     checks.append(lambda: rel_l2(get("attn.out.bin", np.float32), attn_want) <= 1e-3)
+    # the same with the key count in a device buffer (kvLenBuffer): 300 of the 512 rows
+    cases.append(dict(name="attn_len", op="attention_kvlen_buffer", Q="attn.q", K="attn.k", V="attn.v", heads=16, kvHeads=8,
+                      headDim=128, kvLen=ctx, count=300))
+    attn_len_want = oracle.attention_decode_f16kv(q, kb, vb, 16, 8, 128, 300)
+    checks.append(lambda: rel_l2(get("attn_len.out.bin", np.float32), attn_len_want) <= 1e-3)
 
     # elementwise, gather, argmax
     a, b = synth.normal_f32(5000, 9900, 4.0), synth.normal_f32(5000, 9901)

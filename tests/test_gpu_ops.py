@@ -783,6 +783,49 @@ def test_attention_decode_cfg3(ctx):
     assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
 
 
+def test_attention_decode_key_count_on_the_device():
+    """runAttention's kvLenBuffer (src/gpu/kernels/attention.js:1071,1224-1232; kv_len_source == 1 in
+    attention_decode_online_f16kv.wgsl:55-58): the kernels read the key count from a device word.
+    Counts on both sides of every 64-key chunk boundary and of the point where the split count
+    changes, against the oracle; the same launch arguments serve every count."""
+    import torch
+    H, Hkv, D, cap = 32, 8, 128, 4400
+    q, kb, vb = _attn_inputs(H, Hkv, D, cap, seed=5050)
+    qt, kt, vt = ops.tensorFromNumpy(q), ops.tensorFromNumpy(kb), ops.tensorFromNumpy(vb)
+    word = torch.zeros(4, dtype=torch.int32, device="cuda")
+    for n in (1, 2, 63, 64, 65, 128, 129, 2047, 2048, 2049, 2112, 2113, 4095, 4097, cap):
+        word[0] = n
+        torch.cuda.synchronize()
+        got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, seqLen=1, kvLen=cap, numKVHeads=Hkv, causal=True,
+                                              startPos=-1, kvLenBuffer=word))
+        want = oracle.attention_decode_f16kv(q, kb, vb, H, Hkv, D, n)
+        assert rel_l2(got, want) <= REL_L2_F32, n
+        # identical to the launch that gets the count as an argument
+        same = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, seqLen=1, kvLen=n, numKVHeads=Hkv, causal=True,
+                                               startPos=n - 1))
+        assert rel_l2(got, same) <= 1e-6, n
+    # a fixed query position below the key count: the causal mask hides the keys behind it
+    word[0] = 3000
+    torch.cuda.synchronize()
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, kvLen=cap, numKVHeads=Hkv, startPos=700, kvLenBuffer=word))
+    assert rel_l2(got, oracle.attention_decode_f16kv(q, kb, vb, H, Hkv, D, 3000, start_pos=700)) <= REL_L2_F32
+    # sliding window follows the position
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, kvLen=cap, numKVHeads=Hkv, startPos=-1, slidingWindow=200,
+                                          kvLenBuffer=word))
+    assert rel_l2(got, oracle.attention_decode_f16kv(q, kb, vb, H, Hkv, D, 3000, sliding_window=200)) <= REL_L2_F32
+    # no key: zeros; a count beyond the bound is clamped to it
+    word[0] = 0
+    torch.cuda.synchronize()
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, kvLen=cap, numKVHeads=Hkv, startPos=-1, kvLenBuffer=word))
+    assert not got.any()
+    word[0] = cap + 100000
+    torch.cuda.synchronize()
+    got = ops.readTensor(ops.runAttention(qt, kt, vt, None, H, D, kvLen=cap, numKVHeads=Hkv, startPos=-1, kvLenBuffer=word))
+    assert rel_l2(got, oracle.attention_decode_f16kv(q, kb, vb, H, Hkv, D, cap)) <= REL_L2_F32
+    with pytest.raises(DopplerHipError, match="decode"):
+        ops.runAttention(qt, kt, vt, None, H, D, seqLen=2, kvLen=cap, numKVHeads=Hkv, kvLenBuffer=word)
+
+
 @pytest.mark.parametrize("H,Hkv,D", [(32, 8, 128), (8, 8, 128), (8, 1, 64), (6, 2, 64)])
 def test_attention_decode_head_geometries(H, Hkv, D):
     ctx = 777
