@@ -71,6 +71,7 @@ SIGNATURES = {
     "dh_q4k_matmul": (_I, [_P, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
     "dh_q4k_matmul_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _I, _I, _I, _I, _F, _P]),
     "dh_q4k_matmul_plan": (_I, [_I, _I, _I, _I, _I, _I]),
+    "dh_q4k_gemv_layout": (_I, [_I, _I, _I, _I, _I, _I, ctypes.POINTER(ctypes.c_int64)]),
     "dh_q4k_ffn_gate_up": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
     "dh_q4k_ffn_gate_up_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
     "dh_q4k_gemv_chain": (_I, [_P, ctypes.POINTER(ChainPhase), _I]),

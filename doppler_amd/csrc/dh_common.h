@@ -62,8 +62,11 @@ inline double tuning_double(const char* name, double dflt) {
 // holds, num_cus() is the planned device's count, and every launch site reports its kernel family
 // through plan_note() instead of launching (true = planning, return without touching the device).
 bool plan_note(int family);
+// What the noted launch would have been: entry i of the plan's layout record (see dh_q4k_gemv_layout).
+void plan_layout(int i, int64_t value);
 void plan_begin(int num_cus);
 int plan_end();
+const int64_t* plan_layout_record();
 
 // ---- kernel status word ---------------------------------------------------------------------
 // Kernels that wait on other waves or workgroups bound every such wait; a wave whose wait runs

@@ -24,6 +24,7 @@ constexpr size_t kWidenedABytes = (size_t)64 << 20;
 uint32_t* g_kstatus = nullptr;       // kernel status word: pinned host memory, device-writable
 thread_local int t_plan_cus = 0;      // > 0: a plan is being made on this thread for a device of that many compute units
 thread_local int t_plan_family = 0;
+thread_local int64_t t_plan_layout[16] = {};
 }  // namespace
 
 namespace dh {
@@ -40,7 +41,13 @@ int num_cus() { return t_plan_cus > 0 ? t_plan_cus : g_num_cus; }
 void plan_begin(int cus) {
   t_plan_cus = cus;
   t_plan_family = 0;
+  for (auto& v : t_plan_layout) v = 0;
 }
+void plan_layout(int i, int64_t value) {
+  // the first launch of a call describes it (further passes repeat it)
+  if (t_plan_cus > 0 && t_plan_family == 0 && i >= 0 && i < 16) t_plan_layout[i] = value;
+}
+const int64_t* plan_layout_record() { return t_plan_layout; }
 int plan_end() {
   t_plan_cus = 0;
   return t_plan_family;

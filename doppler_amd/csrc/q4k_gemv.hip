@@ -1135,6 +1135,14 @@ int dh_q4k_matmul_plan(int M, int N, int K, int normed, int dual, int num_cus) {
   return rc == 0 ? family : 0;
 }
 
+int dh_q4k_gemv_layout(int M, int N, int K, int normed, int dual, int num_cus, int64_t* out12) {
+  if (!out12) return 0;
+  const int family = dh_q4k_matmul_plan(M, N, K, normed, dual, num_cus);
+  const int64_t* rec = dh::plan_layout_record();
+  for (int i = 0; i < 12; i++) out12[i] = rec[i];
+  return family;
+}
+
 int dh_q4k_ffn_gate_up(const float* d_x, const void* d_Wgate, const void* d_Wup, float* d_out, int M,
                        int hidden, int inter, int activation, float alpha, float swiglu_limit) {
   return q4k_ffn_impl("dh_q4k_ffn_gate_up", d_x, nullptr, 0.f, 0, false, d_Wgate, d_Wup, d_out, M, hidden,

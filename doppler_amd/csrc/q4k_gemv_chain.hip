@@ -704,7 +704,8 @@ int make_plan(const char* op, const float* d_x0, const dh_chain_phase* ph, int n
     P.tiles_rem = (int)(ntiles % ncu);
     const int64_t units = (int64_t)(P.tiles_base + (P.tiles_rem ? 1 : 0)) * P.upt;
     // the division by multiplication is exact while units * (upt_mul * upt - 2^24) < 2^24
-    if (units * ((int64_t)P.upt_mul * P.upt - (1 << 24)) >= (1 << 24) || units >= (1 << 20))
+    if (units * ((int64_t)P.upt_mul * P.upt - (1 << 24)) >= (1 << 24) || units >= (1 << 20) ||
+        units * (int64_t)P.upt_mul >= ((int64_t)1 << 32))
       return dh::fail(1, "[%s] product %d: N=%d, K=%d is too large for a chain", op, p, s.N, s.K);
     max_upt = std::max(max_upt, P.upt);
     min_upt = std::min(min_upt, P.upt);

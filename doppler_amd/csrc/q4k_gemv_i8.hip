@@ -52,6 +52,9 @@ constexpr int kMaxDepth = 3;
 constexpr int kMaxSlots = 32;                     // tiles whose partial sums may be in LDS at once
 constexpr int kZeroBytes = 144;                   // what a lane without an operand reads
 constexpr size_t kMaxLds = 160 * 1024;
+// a finished tile's partial sums are read four columns at a time: the last read of the last slot reaches
+// up to twelve columns (of 64 bytes per activation row) past it, into the counters and this padding
+constexpr int kReadAhead = 12 * 64;
 constexpr int kSpinLimit = 1 << 18;               // polls of a wait inside the workgroup before the wave gives up
 
 #define DH_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
@@ -578,8 +581,11 @@ int launch_i8_vec(I8Args a, const char* op) {
   a.tiles_base = (int)(ntiles / grid);
   a.tiles_rem = (int)(ntiles % grid);
   const int64_t units = (int64_t)(a.tiles_base + (a.tiles_rem ? 1 : 0)) * a.upt;     // per workgroup, at most
-  // the division by multiplication is exact while units * (upt_mul * upt - 2^24) < 2^24
-  if (units * ((int64_t)a.upt_mul * a.upt - (1 << 24)) >= (1 << 24) || units >= (1 << 20)) return -1;
+  // the division by multiplication is exact while units * (upt_mul * upt - 2^24) < 2^24, and the
+  // kernel forms the product in 32 bits
+  if (units * ((int64_t)a.upt_mul * a.upt - (1 << 24)) >= (1 << 24) || units >= (1 << 20) ||
+      units * (int64_t)a.upt_mul >= ((int64_t)1 << 32))
+    return -1;
   int depth = 1;
   if (env_depth > 0) depth = std::min(kMaxDepth, env_depth);
   // tile slots: the units in flight (16 waves x (depth + 1) draws) span at most this many tiles
@@ -592,11 +598,16 @@ int launch_i8_vec(I8Args a, const char* op) {
   while ((1 << a.slot_shift) < nslots) a.slot_shift++;
   auto lds_for = [&](int dep) {
     return (size_t)kWaves * dep * kStage + (size_t)a.nb * MT * kRec + kZeroBytes +
-           sizeof(float) * nslots * a.upt * MT * 16 + sizeof(unsigned) * (2 + 2 * nslots + a.nb);
+           sizeof(float) * nslots * a.upt * MT * 16 + sizeof(unsigned) * (2 + 2 * nslots + a.nb) + kReadAhead * MT;
   };
   while (depth > 1 && lds_for(depth) > cap) depth--;
   if (lds_for(depth) > cap) return -1;
   a.depth = depth;
+  {
+    const int64_t rec[12] = {a.rows, a.nlw, grid, a.tiles_base, a.tiles_rem, depth, (int64_t)lds_for(depth), a.upt, a.upt_mul,
+                             nslots, 0, MT};
+    for (int i = 0; i < 12; i++) dh::plan_layout(i, rec[i]);
+  }
   if (dh::plan_note(DH_PLAN_GEMV_I8)) return 0;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {
@@ -624,7 +635,7 @@ size_t i8_lds_bytes(int mt, int nb, int nmat) {
   int nslots = 2;
   while (nslots < need) nslots *= 2;
   return (size_t)kWaves * kStage + (size_t)nb * mt * kRec + kZeroBytes + sizeof(float) * nslots * upt * mt * 16 +
-         sizeof(unsigned) * (2 + 2 * nslots + nb);
+         sizeof(unsigned) * (2 + 2 * nslots + nb) + kReadAhead * mt;
 }
 
 template <bool DUAL>

@@ -562,6 +562,11 @@ int launch_rows(RowsArgs a, const char* op) {
   while (depth > 1 && lds_for(depth) > kLdsCap) depth--;
   if (lds_for(depth) > kLdsCap) return -1;
   a.depth = depth;
+  {
+    const int64_t rec[12] = {a.rows, a.nlw, grid, a.tiles_base, a.tiles_rem, depth, (int64_t)lds_for(depth), 0, 0, 0, a.acc_max,
+                             a.M};
+    for (int i = 0; i < 12; i++) dh::plan_layout(i, rec[i]);
+  }
   if (dh::plan_note(DH_PLAN_GEMV_ROWS)) return 0;
   static bool attr_set = false;   // once per instantiation: the call costs microseconds
   if (!attr_set) {

@@ -140,6 +140,13 @@ int dh_q4k_matmul_rmsnorm(const float* d_A, const float* d_norm_weight, float ep
 #define DH_PLAN_GEMM 4       /* M >= 16: f16 matrix-core GEMM */
 #define DH_PLAN_GEMV_LDS 5   /* f32 vector GEMV, activations staged in LDS: last resort */
 int dh_q4k_matmul_plan(int M, int N, int K, int normed, int dual, int num_cus);
+/* dh_q4k_matmul_plan plus, for the two streaming GEMV families, the launch the call would make (its
+ * first pass): out12 = { weight rows per tile, load instructions per work unit, workgroups, tiles per
+ * workgroup (floor), workgroups with one tile more, ring stages per wave, bytes of dynamic LDS,
+ * int8 kernel: work units per tile, its reciprocal multiplier, tile slots; few-row kernel:
+ * accumulators per wave; activation rows per pass }.  For tests that check the kernels' address
+ * arithmetic on the host; other families leave the record zero.  No counterpart in the reference. */
+int dh_q4k_gemv_layout(int M, int N, int K, int normed, int dual, int num_cus, int64_t* out12);
 
 /* out[M,inter] = clamp(act(x.Wgate^T) * (x.Wup^T) * alpha).
  * Replaces runFusedFFN/recordFusedFFN, src/gpu/kernels/fused_ffn.js:501,605
