@@ -226,6 +226,33 @@ def main():
     dec.release_graph()
     log("[bench] graph replay: %.1f tok/s" % graph_tok_s)
 
+    # ---- side measurements (A/B, same positions rewritten): the captured step with its attention
+    #      nodes moved by the host before every replay instead of reading the key count on the device,
+    #      and the eager step with the four products between two attentions chained into one launch
+    def timed_steps(fn, first_tok, n=24):
+        t = first_tok
+        for i in range(4):
+            t = fn(t, pos_g + i)
+        capi_sync()
+        t0_ = time.perf_counter()
+        for i in range(n):
+            t = fn(t, pos_g + 4 + i)
+        capi_sync()
+        return n / (time.perf_counter() - t0_)
+    dec.capture_step(pos_g, device_kv_len=False)
+    graph_patched_tok_s = timed_steps(dec.step_graph, tok)
+    dec.release_graph()
+    log("[bench] graph replay with host-patched attention nodes: %.1f tok/s" % graph_patched_tok_s)
+    chained_tok_s = None
+    try:
+        dec.chain_gemvs = True
+        chained_tok_s = timed_steps(dec.step, tok)
+        log("[bench] eager steps with chained GEMVs (one launch for o, gate/up, down, next qkv): %.1f tok/s" % chained_tok_s)
+    except Exception as e:      # a side measurement, never a reason to lose the result
+        log("[bench] chained-GEMV measurement failed: %r" % (e,))
+    finally:
+        dec.chain_gemvs = False
+
     # ---- roofline of the dominant kernel
     Hd, I = cfg["hidden"], cfg["inter"]
     launch_bytes = 2 * synth.q4k_nbytes(I, Hd) + 2 * Hd * 4 + I * 4      # weights, x + norm weight, output
@@ -295,6 +322,8 @@ def main():
                    "hbm_frac_whole_step": round(step_bytes * tok_s / 1e9 / HBM_PEAK_GBPS, 4),
                    "batched_decode_16_per_submit_tokens_per_s": round(batched_tok_s, 2),
                    "graph_replay_tokens_per_s": round(graph_tok_s, 2),
+                   "graph_replay_host_patched_tokens_per_s": round(graph_patched_tok_s, 2),
+                   "chained_gemv_tokens_per_s": round(chained_tok_s, 2) if chained_tok_s else None,
                    "js_host": js_host,
                    "prefill_tokens_per_s": round(prefill / prefill_s, 1)},
         "roofline": roofline,

@@ -145,7 +145,11 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
   for (int i = tid; i < kCtrFlags + nflags; i += 64 * kWaves) ctr[i] = 0u;
   if (tid >= 64 && tid < 64 + kZeroBytes / 4) reinterpret_cast<uint32_t*>(zeros)[tid - 64] = 0u;
 
-  const uint32_t seq_base = *a.epoch * 8u;       // phase p's outputs carry seq_base + p + 1
+  // the launch counter: requested first, so that it arrives with (ahead of) phase 0's activations and
+  // costs no round trip of its own; phase p's outputs carry seq_base + p + 1
+  uint32_t epoch_v;
+  asm volatile("global_load_dword %0, %1, off" : "=&v"(epoch_v) : "v"(a.epoch) : "memory");
+  uint32_t seq_base = 0;
   const int nph = a.nph;
 
   // ---- this workgroup's unit and tile ranges: phase p holds units [ub_p, ub_{p+1}) and tile ordinals
@@ -384,6 +388,8 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
   }
   // phase 0's activations: only they are waited for (the units were requested behind them)
   wait_vm_at_most(nl_st0 + nl_st1);
+  asm volatile("" : "+v"(epoch_v));
+  seq_base = __builtin_amdgcn_readfirstlane(epoch_v) * 8u;
   finish_pass(0, a.ph[0], c_first, first);
 #pragma unroll 1
   for (int c0 = c_first + kWaves * kColsPerPass; c0 < a.ph[0].nb; c0 += kWaves * kColsPerPass) {
@@ -413,235 +419,228 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
   const uint32_t lane_q = lane_hdr + 16 + 32 * (kg >> 1) + 16 * (kg & 1);
   const uint32_t sh_lo = 8 * kg;           // bit offset of this lane's byte in the header words
 
-  // ---- process side: the phase whose units are being multiplied
-  int pp = -1, p_nb = 1, p_upt = 1, p_upt_mul = 0, p_ub = 0, p_tb = 0, p_dual = 0;
-  uint32_t p_xq = 0, p_flags = 0;
-  int my_phase = 0;                        // prologues this wave has done: phases 0 .. my_phase
-  int rms_phase = -1;                      // phase inv_rms belongs to
+  // ---- process side: phase by phase; inside a phase the unit loop runs on the phase's own scalars.
+  // A wave enters phase p when the unit at the head of its ring is not of an earlier phase any more;
+  // on the way in it prepares its share of the phase's activations (phase 0: done above), which the
+  // other waves count on whether or not this wave draws a unit of the phase.
   float inv_rms = 1.f;
-
+  bool have_rms = false;
   int cstage = 0;
 #pragma unroll 1
-  for (;;) {
-    const int cur = cstage ? u_st1 : u_st0;
-    if (cur >= total) break;              // draws only grow: nothing behind this one either
-    const int p = phase_of(cur);
-    if (p != pp) {
-      pp = p;
-      const Phase& P = a.ph[p];
-      p_nb = P.nb; p_upt = P.upt; p_upt_mul = P.upt_mul; p_dual = P.nmat - 1;
-      p_ub = DH_SEL4(p, 0, ub1, ub2, ub3);
-      p_tb = DH_SEL4(p, 0, tb1, tb2, tb3);
-      p_xq = (p & 1) ? xq_abs1 : xq_abs0;
-      p_flags = ctr_abs + 4 * (kCtrFlags + ((p & 1) ? a.nb_max[0] : 0));
-    }
-    // this wave's share of the activations of every phase up to the unit's
-    while (my_phase < p) prologue(++my_phase);
-
-    const int local = cur - p_ub;
-    const int tl = (int)(((unsigned)local * (unsigned)p_upt_mul) >> 24);
-    const int rr = local - tl * p_upt;
-    const int mat = (p_dual && rr >= p_nb) ? 1 : 0;
-    const int col = rr - mat * p_nb;
-    const int tord = p_tb + tl;                       // tile ordinal of the workgroup, over all phases
-    const int slot = tord & (kSlots - 1);
-    // draw the unit that will go into this stage once it has been read (the answer is collected with
-    // the reads below)
-    unsigned nxt = 0;
-    if (lane == 0) asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=&v"(nxt) : "v"(ctr_abs), "v"(1u) : "memory");
-    // the other stage's loads were issued after this one's
-    wait_vm_at_most(cstage ? nl_st0 : nl_st1);
-    const uint32_t hp = lane_hdr + cstage * kStage, qp = lane_q + cstage * kStage;
-    const uint32_t rec = p_xq + (uint32_t)col * kRec;
-    const uint32_t gen_addr = ctr_abs + 4 * (1 + kSlots + slot);
-    const uint32_t flag_addr = p_flags + 4 * col;
-    v4u h, q0, q1;
-    v4i ax[2][2];
-    v2f sx, xinv;
-    uint32_t gen, flag;
-    asm volatile(
-        "ds_read_b32 %4, %8\n\t"
-        "ds_read_b128 %0, %5\n\t"
-        "ds_read_b128 %1, %6\n\t"
-        "ds_read_b128 %2, %6 offset:64\n\t"
-        "ds_read_b32 %3, %7"
-        : "=&v"(h), "=&v"(q0), "=&v"(q1), "=&v"(gen), "=&v"(flag)
-        : "v"(hp), "v"(qp), "v"(gen_addr), "v"(flag_addr)
-        : "memory");
-    // the column's operands, read at once on the expectation that its flag is up; re-read below if it was not
-#define DH_READ_OPERANDS()                                                                        \
-    do {                                                                                          \
-      const uint32_t pa = rec * a_mul[0] + a_off[0], pb = rec * a_mul[1] + a_off[1], ps = rec + kRecSums + 4 * kg; \
-      asm volatile(                                                                               \
-          "ds_read_b128 %0, %6\n\t"                                                               \
-          "ds_read_b128 %1, %7\n\t"                                                               \
-          "ds_read_b128 %2, %6 offset:128\n\t"                                                    \
-          "ds_read_b128 %3, %7 offset:128\n\t"                                                    \
-          "ds_read2_b32 %4, %8 offset1:4\n\t"                                                     \
-          "ds_read2_b32 %5, %8 offset0:8 offset1:12"                                              \
-          : "=&v"(ax[0][0]), "=&v"(ax[0][1]), "=&v"(ax[1][0]), "=&v"(ax[1][1]), "=&v"(sx), "=&v"(xinv) \
-          : "v"(pa), "v"(pb), "v"(ps)                                                             \
-          : "memory");                                                                            \
-    } while (0)
-#define DH_TIE_OPERANDS() asm volatile("" : "+v"(ax[0][0]), "+v"(ax[0][1]), "+v"(ax[1][0]), "+v"(ax[1][1]), "+v"(sx), "+v"(xinv))
-    DH_READ_OPERANDS();
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(h), "+v"(q0), "+v"(q1), "+v"(gen), "+v"(flag), "+v"(nxt) :: "memory");
-    DH_TIE_OPERANDS();
+  for (int p = 0; p < nph; p++) {
+    if (p > 0) prologue(p);
+    const Phase& P = a.ph[p];
+    const int p_nb = P.nb, p_upt = P.upt, p_upt_mul = P.upt_mul, p_dual = P.nmat - 1;
+    const int p_ub = DH_SEL4(p, 0, ub1, ub2, ub3), p_ue = DH_SEL4(p, ub1, ub2, ub3, total);
+    const int p_tb = DH_SEL4(p, 0, tb1, tb2, tb3);
+    const uint32_t p_xq = (p & 1) ? xq_abs1 : xq_abs0;
+    const uint32_t p_flags = ctr_abs + 4 * (kCtrFlags + ((p & 1) ? a.nb_max[0] : 0));
     const uint32_t flag_want = (uint32_t)p + 1u;
-    if (__builtin_amdgcn_readfirstlane(flag) != flag_want) {
-      int spins = 0;
-      do {
-        __builtin_amdgcn_s_sleep(2);
-        flag = lds_read_u32(flag_addr);
-        if (++spins > a.spin_limit * 8 || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) break;
-      } while (__builtin_amdgcn_readfirstlane(flag) != flag_want);
-      if (__builtin_amdgcn_readfirstlane(flag) != flag_want) {
-        give_up(DH_KSTATUS_COLUMN_WAIT, p);
-      }
+    const bool last_phase = p == nph - 1;
+    have_rms = false;
+
+    // The units of this phase, from the head of the ring (stage cstage; the two stages alternate).
+#pragma unroll 1
+    for (;;) {
+      const int ST = cstage;
+      const int cur = ST ? u_st1 : u_st0;
+      if (cur >= p_ue) break;             // a later phase's unit (or none): draws only grow
+      const int local = cur - p_ub;
+      const int tl = (int)(((unsigned)local * (unsigned)p_upt_mul) >> 24);
+      const int rr = local - tl * p_upt;
+      const int mat = (p_dual && rr >= p_nb) ? 1 : 0;
+      const int col = rr - mat * p_nb;
+      const int tord = p_tb + tl;                       // tile ordinal of the workgroup, over all phases
+      const int slot = tord & (kSlots - 1);
+      // draw the unit that will go into this stage once it has been read (the answer is collected with
+      // the reads below)
+      unsigned nxt = 0;
+      if (lane == 0) asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=&v"(nxt) : "v"(ctr_abs), "v"(1u) : "memory");
+      // the other stage's loads were issued after this one's
+      wait_vm_at_most(ST ? nl_st0 : nl_st1);
+      const uint32_t hp = lane_hdr + ST * kStage, qp = lane_q + ST * kStage;
+      const uint32_t rec = p_xq + (uint32_t)col * kRec;
+      const uint32_t gen_addr = ctr_abs + 4 * (1 + kSlots + slot);
+      const uint32_t flag_addr = p_flags + 4 * col;
+      v4u h, q0, q1;
+      v4i ax[2][2];
+      v2f sx, xinv;
+      uint32_t gen, flag;
+      asm volatile(
+          "ds_read_b32 %4, %8\n\t"
+          "ds_read_b128 %0, %5\n\t"
+          "ds_read_b128 %1, %6\n\t"
+          "ds_read_b128 %2, %6 offset:64\n\t"
+          "ds_read_b32 %3, %7"
+          : "=&v"(h), "=&v"(q0), "=&v"(q1), "=&v"(gen), "=&v"(flag)
+          : "v"(hp), "v"(qp), "v"(gen_addr), "v"(flag_addr)
+          : "memory");
+      // the column's operands, read at once on the expectation that its flag is up; re-read below if it was not
+#define DH_READ_OPERANDS()                                                                        \
+      do {                                                                                        \
+        const uint32_t pa = rec * a_mul[0] + a_off[0], pb = rec * a_mul[1] + a_off[1], ps = rec + kRecSums + 4 * kg; \
+        asm volatile(                                                                             \
+            "ds_read_b128 %0, %6\n\t"                                                             \
+            "ds_read_b128 %1, %7\n\t"                                                             \
+            "ds_read_b128 %2, %6 offset:128\n\t"                                                  \
+            "ds_read_b128 %3, %7 offset:128\n\t"                                                  \
+            "ds_read2_b32 %4, %8 offset1:4\n\t"                                                   \
+            "ds_read2_b32 %5, %8 offset0:8 offset1:12"                                            \
+            : "=&v"(ax[0][0]), "=&v"(ax[0][1]), "=&v"(ax[1][0]), "=&v"(ax[1][1]), "=&v"(sx), "=&v"(xinv) \
+            : "v"(pa), "v"(pb), "v"(ps)                                                           \
+            : "memory");                                                                          \
+      } while (0)
+#define DH_TIE_OPERANDS() asm volatile("" : "+v"(ax[0][0]), "+v"(ax[0][1]), "+v"(ax[1][0]), "+v"(ax[1][1]), "+v"(sx), "+v"(xinv))
       DH_READ_OPERANDS();
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(h), "+v"(q0), "+v"(q1), "+v"(gen), "+v"(flag), "+v"(nxt) :: "memory");
       DH_TIE_OPERANDS();
-    }
+      if (__builtin_amdgcn_readfirstlane(flag) != flag_want) {
+        int spins = 0;
+        do {
+          __builtin_amdgcn_s_sleep(2);
+          flag = lds_read_u32(flag_addr);
+          if (++spins > a.spin_limit * 8 || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) break;
+        } while (__builtin_amdgcn_readfirstlane(flag) != flag_want);
+        if (__builtin_amdgcn_readfirstlane(flag) != flag_want) give_up(DH_KSTATUS_COLUMN_WAIT, p);
+        DH_READ_OPERANDS();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        DH_TIE_OPERANDS();
+      }
 #undef DH_READ_OPERANDS
 #undef DH_TIE_OPERANDS
-    // the stage is free again: put the loads of the unit drawn above in flight
-    {
-      const int u = (int)__builtin_amdgcn_readfirstlane(nxt);
-      const int nl = u < total ? issue(u, cstage) : 0;
-      if (cstage) { u_st1 = u; nl_st1 = nl; } else { u_st0 = u; nl_st0 = nl; }
-    }
-    cstage ^= 1;
-
-    // 6-bit scales and mins of sub-blocks kg and 4 + kg of this lane's weight row
-    const int sc_a = (int)((h.y >> sh_lo) & 63u);
-    const int sc_b = (int)(((h.w >> sh_lo) & 15u) | (((h.y >> (sh_lo + 6)) & 3u) << 4));
-    const float mn_a = (float)((h.z >> sh_lo) & 63u);
-    const float mn_b = (float)(((h.w >> (sh_lo + 4)) & 15u) | (((h.z >> (sh_lo + 6)) & 3u) << 4));
-    const float d = f16lo(h.x), dmin = f16hi(h.x);
-    v4i blo[2], bhi[2];
-#pragma unroll
-    for (int cc = 0; cc < 2; cc++) {
-      const v4u q = cc ? q1 : q0;
-      blo[cc] = v4i{(int)(q.x & 0x0F0F0F0Fu), (int)(q.y & 0x0F0F0F0Fu), (int)(q.z & 0x0F0F0F0Fu),
-                    (int)(q.w & 0x0F0F0F0Fu)};
-      bhi[cc] = v4i{(int)((q.x >> 4) & 0x0F0F0F0Fu), (int)((q.y >> 4) & 0x0F0F0F0Fu),
-                    (int)((q.z >> 4) & 0x0F0F0F0Fu), (int)((q.w >> 4) & 0x0F0F0F0Fu)};
-    }
-    // wait (never, in practice) until the tile that used this slot kSlots tiles ago is written out
-    {
-      const unsigned want = (unsigned)tord >> kSlotShift;
-      int spins = 0;
-      while (__builtin_amdgcn_readfirstlane(gen) != want) {
-        __builtin_amdgcn_s_sleep(1);
-        gen = lds_read_u32(gen_addr);
-        if (++spins > a.spin_limit * 8 || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) break;
+      // the stage is free again: put the loads of the unit drawn above in flight
+      {
+        const int u = (int)__builtin_amdgcn_readfirstlane(nxt);
+        const int nl = u < total ? issue(u, ST) : 0;
+        if (ST) { u_st1 = u; nl_st1 = nl; } else { u_st0 = u; nl_st0 = nl; }
       }
-      if (__builtin_amdgcn_readfirstlane(gen) != want) {
-        give_up(DH_KSTATUS_SLOT_WAIT, p);
-      }
-    }
-    v4i dd[2];
-#pragma unroll
-    for (int cc = 0; cc < 2; cc++) {
-      v4i t = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[cc][0], blo[cc], v4i{0, 0, 0, 0}, 0, 0, 0);
-      dd[cc] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[cc][1], bhi[cc], t, 0, 0, 0);
-    }
-    // the four lane groups hold different sub-blocks of the same 16 rows
-    const float sres = sum_lane_groups(i8_unit_term(dd[0], dd[1], sc_a, sc_b, mn_a, mn_b, d, dmin, sx, xinv));
-    if (lane < 16) red[(size_t)slot * a.red_stride + (mat * p_nb + col) * 16 + lane] = sres;
+      cstage ^= 1;
 
-    // ---- deliver.  LDS executes a wave's operations in order, so the partial sums above are in
-    // place before the count below is; the wave that delivers a tile's last unit finishes it.
-    unsigned arrived = 0;
-    if (lane == 0)
-      asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
-                   : "=&v"(arrived) : "v"(ctr_abs + 4 * (1 + slot)), "v"(1u) : "memory");
-    arrived = __builtin_amdgcn_readfirstlane(arrived);
-    if ((int)arrived == p_upt - 1) {
-      const Phase& P = a.ph[p];
-      const int nb = p_nb;
-      const int tile = bid + tl * a.grid;
-      const int64_t row = (int64_t)tile * P.rows + j;
-      const uint32_t slot_abs = red_abs + (uint32_t)slot * a.red_stride * 4;
-      // lane (j, kg) adds columns kg, kg + 4, .. (four reads in flight at a time); the four groups then
-      // meet.  The order is fixed, so the result does not depend on who arrives last.
-      float sg = 0.f, su = 0.f;
-      for (int c = kg; c < nb; c += 16) {
-        float r[2][4];
+      // 6-bit scales and mins of sub-blocks kg and 4 + kg of this lane's weight row
+      const int sc_a = (int)((h.y >> sh_lo) & 63u);
+      const int sc_b = (int)(((h.w >> sh_lo) & 15u) | (((h.y >> (sh_lo + 6)) & 3u) << 4));
+      const float mn_a = (float)((h.z >> sh_lo) & 63u);
+      const float mn_b = (float)(((h.w >> (sh_lo + 4)) & 15u) | (((h.z >> (sh_lo + 6)) & 3u) << 4));
+      const float d = f16lo(h.x), dmin = f16hi(h.x);
+      v4i blo[2], bhi[2];
 #pragma unroll
-        for (int mt = 0; mt < 2; mt++) {
-          if (mt == 0 || p_dual) {
-            const uint32_t q = slot_abs + ((mt * nb + c) * 16 + j) * 4;
-            asm volatile(
-                "ds_read_b32 %0, %4\n\t"
-                "ds_read_b32 %1, %4 offset:256\n\t"
-                "ds_read_b32 %2, %4 offset:512\n\t"
-                "ds_read_b32 %3, %4 offset:768"
-                : "=&v"(r[mt][0]), "=&v"(r[mt][1]), "=&v"(r[mt][2]), "=&v"(r[mt][3])
-                : "v"(q)
-                : "memory");
-          } else {
-            r[mt][0] = r[mt][1] = r[mt][2] = r[mt][3] = 0.f;
+      for (int cc = 0; cc < 2; cc++) {
+        const v4u q = cc ? q1 : q0;
+        blo[cc] = v4i{(int)(q.x & 0x0F0F0F0Fu), (int)(q.y & 0x0F0F0F0Fu), (int)(q.z & 0x0F0F0F0Fu),
+                      (int)(q.w & 0x0F0F0F0Fu)};
+        bhi[cc] = v4i{(int)((q.x >> 4) & 0x0F0F0F0Fu), (int)((q.y >> 4) & 0x0F0F0F0Fu),
+                      (int)((q.z >> 4) & 0x0F0F0F0Fu), (int)((q.w >> 4) & 0x0F0F0F0Fu)};
+      }
+      // wait (never, in practice) until the tile that used this slot kSlots tiles ago is written out
+      {
+        const unsigned want = (unsigned)tord >> kSlotShift;
+        int spins = 0;
+        while (__builtin_amdgcn_readfirstlane(gen) != want) {
+          __builtin_amdgcn_s_sleep(1);
+          gen = lds_read_u32(gen_addr);
+          if (++spins > a.spin_limit * 8 || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) break;
+        }
+        if (__builtin_amdgcn_readfirstlane(gen) != want) give_up(DH_KSTATUS_SLOT_WAIT, p);
+      }
+      v4i dd[2];
+#pragma unroll
+      for (int cc = 0; cc < 2; cc++) {
+        v4i t = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[cc][0], blo[cc], v4i{0, 0, 0, 0}, 0, 0, 0);
+        dd[cc] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ax[cc][1], bhi[cc], t, 0, 0, 0);
+      }
+      // the four lane groups hold different sub-blocks of the same 16 rows
+      const float sres = sum_lane_groups(i8_unit_term(dd[0], dd[1], sc_a, sc_b, mn_a, mn_b, d, dmin, sx, xinv));
+      if (lane < 16) red[(size_t)slot * a.red_stride + (mat * p_nb + col) * 16 + lane] = sres;
+
+      // ---- deliver.  LDS executes a wave's operations in order, so the partial sums above are in
+      // place before the count below is; the wave that delivers a tile's last unit finishes it.
+      unsigned arrived = 0;
+      if (lane == 0)
+        asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(arrived) : "v"(ctr_abs + 4 * (1 + slot)), "v"(1u) : "memory");
+      arrived = __builtin_amdgcn_readfirstlane(arrived);
+      if ((int)arrived == p_upt - 1) {
+        const int nb = p_nb;
+        const int tile = bid + tl * a.grid;
+        const int64_t row = (int64_t)tile * P.rows + j;
+        const uint32_t slot_abs = red_abs + (uint32_t)slot * a.red_stride * 4;
+        // lane (j, kg) adds columns kg, kg + 4, .. (four reads in flight at a time); the four groups then
+        // meet.  The order is fixed, so the result does not depend on who arrives last.
+        float sg = 0.f, su = 0.f;
+        for (int c = kg; c < nb; c += 16) {
+          float r[2][4];
+#pragma unroll
+          for (int mt = 0; mt < 2; mt++) {
+            if (mt == 0 || p_dual) {
+              const uint32_t q = slot_abs + ((mt * nb + c) * 16 + j) * 4;
+              asm volatile(
+                  "ds_read_b32 %0, %4\n\t"
+                  "ds_read_b32 %1, %4 offset:256\n\t"
+                  "ds_read_b32 %2, %4 offset:512\n\t"
+                  "ds_read_b32 %3, %4 offset:768"
+                  : "=&v"(r[mt][0]), "=&v"(r[mt][1]), "=&v"(r[mt][2]), "=&v"(r[mt][3])
+                  : "v"(q)
+                  : "memory");
+            } else {
+              r[mt][0] = r[mt][1] = r[mt][2] = r[mt][3] = 0.f;
+            }
+          }
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]) :: "memory");
+          asm volatile("" : "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]));
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const bool ok = c + 4 * i < nb;       // columns past the last read whatever follows: dropped
+            sg += ok ? r[0][i] : 0.f;
+            su += ok ? r[1][i] : 0.f;
           }
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]) :: "memory");
-        asm volatile("" : "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]));
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const bool ok = c + 4 * i < nb;       // columns past the last read whatever follows: dropped
-          sg += ok ? r[0][i] : 0.f;
-          su += ok ? r[1][i] : 0.f;
+        sg = sum_lane_groups(sg);
+        su = sum_lane_groups(su);
+        if (P.norm_weight != nullptr) {
+          if (!have_rms) {
+            // every column has been consumed by now, so every column's sum of squares is in place
+            float tot = 0.f;
+            for (int c = 0; c < nb; c++) tot += __uint_as_float(lds_read_u32(p_xq + (uint32_t)c * kRec + kRecSsq));
+            inv_rms = 1.0f / sqrtf(tot / (float)P.K + P.norm_eps);
+            have_rms = true;
+          }
+          sg *= inv_rms;
+          su *= inv_rms;
         }
-      }
-      sg = sum_lane_groups(sg);
-      su = sum_lane_groups(su);
-      if (P.norm_weight != nullptr) {
-        if (rms_phase != p) {
-          // every column has been consumed by now, so every column's sum of squares is in place
-          float tot = 0.f;
-          for (int c = 0; c < nb; c++) tot += __uint_as_float(lds_read_u32(p_xq + (uint32_t)c * kRec + kRecSsq));
-          inv_rms = 1.0f / sqrtf(tot / (float)P.K + P.norm_eps);
-          rms_phase = p;
+        if (kg == 0 && j < P.rows && row < P.N) {
+          float v;
+          if (p_dual) {
+            const float act = P.activation == DH_ACT_SILU ? act_silu(sg) : act_gelu(sg);
+            v = act * su * P.alpha;
+            if (P.activation == DH_ACT_SILU && P.clamp_max > 0.f) v = fminf(fmaxf(v, -P.clamp_max), P.clamp_max);
+          } else {
+            v = sg * P.alpha;
+            // device-scope load: an earlier phase of this launch may have written the residual
+            if (P.residual) v += __hip_atomic_load(const_cast<float*>(P.residual) + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          __hip_atomic_store(P.C + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (!last_phase) {
+            v2u pr;
+            pr.x = __float_as_uint(v);
+            pr.y = seq_base + (uint32_t)p + 1u;
+            v2u* dst = a.ll + (size_t)(p & 1) * kMaxChainN + row;
+            asm volatile("global_store_dwordx2 %0, %1, off sc1" :: "v"(dst), "v"(pr) : "memory");
+          }
         }
-        sg *= inv_rms;
-        su *= inv_rms;
-      }
-      const bool last_phase = p == nph - 1;
-      if (kg == 0 && j < P.rows && row < P.N) {
-        float v;
-        if (p_dual) {
-          const float act = P.activation == DH_ACT_SILU ? act_silu(sg) : act_gelu(sg);
-          v = act * su * P.alpha;
-          if (P.activation == DH_ACT_SILU && P.clamp_max > 0.f) v = fminf(fmaxf(v, -P.clamp_max), P.clamp_max);
-        } else {
-          v = sg * P.alpha;
-          // device-scope load: an earlier phase of this launch may have written the residual
-          if (P.residual) v += __hip_atomic_load(const_cast<float*>(P.residual) + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // a later phase reads these outputs as its residual: they are in memory before this wave goes on
+        if (P.wait_stores) DH_WAIT_VM(0);
+        // slot free for the tile kSlots further on (after the reads above: same wave, in order)
+        if (lane == 0) {
+          ctr[1 + slot] = 0u;
+          ctr[1 + kSlots + slot] = ((unsigned)tord >> kSlotShift) + 1u;
+          unsigned was;
+          asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(was) : "v"(ctr_abs + 4 * (kCtrDone + p)), "v"(1u) : "memory");
         }
-        __hip_atomic_store(P.C + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (!last_phase) {
-          v2u pr;
-          pr.x = __float_as_uint(v);
-          pr.y = seq_base + (uint32_t)p + 1u;
-          v2u* dst = a.ll + (size_t)(p & 1) * kMaxChainN + row;
-          asm volatile("global_store_dwordx2 %0, %1, off sc1" :: "v"(dst), "v"(pr) : "memory");
-        }
+        // the launch counter moves on once: the workgroup that owns the last phase's first tile does it
+        if (last_phase && bid == 0 && tl == 0 && lane == 0) *a.epoch = (seq_base >> 3) + 1u;
       }
-      // a later phase reads these outputs as its residual: they are in memory before this wave goes on
-      if (P.wait_stores) DH_WAIT_VM(0);
-      // slot free for the tile kSlots further on (after the reads above: same wave, in order)
-      if (lane == 0) {
-        ctr[1 + slot] = 0u;
-        ctr[1 + kSlots + slot] = ((unsigned)tord >> kSlotShift) + 1u;
-        unsigned was;
-        asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(was) : "v"(ctr_abs + 4 * (kCtrDone + p)), "v"(1u) : "memory");
-      }
-      // the launch counter moves on once: the workgroup that owns the last phase's first tile does it
-      if (last_phase && bid == 0 && tl == 0 && lane == 0) *a.epoch = (seq_base >> 3) + 1u;
     }
   }
-  // a wave that drew no unit of the later phases still owes the other waves its columns of them
-  while (my_phase < nph - 1) prologue(++my_phase);
 }
 
 // ---- host side ----------------------------------------------------------------------------------

@@ -48,7 +48,8 @@ constexpr int kWaves = 16;
 constexpr int kTileRows = 16;
 constexpr int kStage = kTileRows * kBlockBytes;   // 2304 bytes per ring stage
 constexpr int kUnitLoads = 3;                     // load instructions of a full unit: ceil(16 rows * 9 pieces / 64 lanes)
-constexpr int kMaxDepth = 3;
+constexpr int kMaxDepth = 1;                      // ring stages per wave (2..5 measured slower: the queue already keeps 16 units in flight)
+constexpr int kSlotDepth = 3;                     // what the tile-slot count is sized for
 constexpr int kMaxSlots = 32;                     // tiles whose partial sums may be in LDS at once
 constexpr int kZeroBytes = 144;                   // what a lane without an operand reads
 constexpr size_t kMaxLds = 160 * 1024;
@@ -126,7 +127,8 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
                "s"(a.norm_weight_offset));
   asm volatile("" :: "s"(a.alpha), "s"(a.clamp_max), "s"(a.norm_eps));
 
-  const int D = a.depth, nb = a.nb, upt = a.upt, nslots = a.nslots;
+  constexpr int D = kMaxDepth;
+  const int nb = a.nb, upt = a.upt, nslots = a.nslots;
   unsigned char* ring = lds;
   unsigned char* xq = ring + (size_t)kWaves * D * kStage;
   unsigned char* zeros = xq + (size_t)nb * MT * kRec;
@@ -359,7 +361,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     // with the reads below)
     unsigned nxt = 0;
     if (lane == 0) asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=&v"(nxt) : "v"(ctr_abs), "v"(1u) : "memory");
-    wait_vm_at_most((inflight - 1) * a.nlw);
+    if constexpr (D == 1) DH_WAIT_VM(0); else wait_vm_at_most((inflight - 1) * a.nlw);
     const uint32_t hp = lane_hdr + cstage * kStage, qp = lane_q + cstage * kStage;
     const uint32_t rec = xq_abs + (uint32_t)(col * MT) * kRec;
     const uint32_t gen_addr = ctr_abs + 4 * (1 + nslots + slot);
@@ -589,7 +591,7 @@ int launch_i8_vec(I8Args a, const char* op) {
   int depth = 1;
   if (env_depth > 0) depth = std::min(kMaxDepth, env_depth);
   // tile slots: the units in flight (16 waves x (depth + 1) draws) span at most this many tiles
-  const int need = (kWaves * (kMaxDepth + 1) + a.upt - 1) / a.upt + 2;
+  const int need = (kWaves * (kSlotDepth + 1) + a.upt - 1) / a.upt + 2;
   int nslots = 2;
   while (nslots < need) nslots *= 2;
   if (nslots > kMaxSlots) return -1;
@@ -631,7 +633,7 @@ int launch_i8(const I8Args& a, const char* op) {
 // Bytes of LDS a launch with MT activation rows needs at ring depth 1 (what launch_i8_vec computes).
 size_t i8_lds_bytes(int mt, int nb, int nmat) {
   const int upt = nb * nmat;
-  const int need = (kWaves * (kMaxDepth + 1) + upt - 1) / upt + 2;
+  const int need = (kWaves * (kSlotDepth + 1) + upt - 1) / upt + 2;
   int nslots = 2;
   while (nslots < need) nslots *= 2;
   return (size_t)kWaves * kStage + (size_t)nb * mt * kRec + kZeroBytes + sizeof(float) * nslots * upt * mt * 16 +

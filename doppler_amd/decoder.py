@@ -43,7 +43,7 @@ class HipDecoder:
     TOKEN_RING = 64      # tokens one decode_batch submit can produce
 
     def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True,
-                 fuse_qkv_attention=True, finiteness_guard=False, finiteness_abs_threshold=None):
+                 fuse_qkv_attention=True, finiteness_guard=False, finiteness_abs_threshold=None, chain_gemvs=False):
         """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
         layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
         input_norm, post_attn_norm, q_norm, k_norm: f32); embed_bits: uint16 [vocab, hidden].
@@ -52,6 +52,15 @@ class HipDecoder:
         activations are f16 (src/inference/pipelines/text/layer.js:1237-1252,
         generator-steps.js:786-798, :837-843); off by default, the activations here are f32."""
         self.cfg = dict(cfg)
+        # chain_gemvs: the four products between two attentions (o, gate/up, down, next q/k/v) as one
+        # dh_q4k_gemv_chain launch.  Same bits as the separate launches; measured slower on the 9B-class
+        # shapes (the exchange between the products costs what the launches cost), so off by default.
+        self.chain_gemvs = bool(chain_gemvs)
+        if self.chain_gemvs:
+            dims = (cfg["hidden"], cfg["inter"], cfg["heads"] * cfg["head_dim"])
+            if any(k % 256 or k < 2048 or k > 32768 for k in dims) or not fuse_norm or finiteness_guard:
+                raise ValueError("chain_gemvs serves hidden, FFN and attention widths that are multiples of 256 in "
+                                 "2048..32768, with the norms fused and the finiteness guard off (got %s)" % (dims,))
         self.finiteness_guard = bool(finiteness_guard)
         self.finiteness_abs_threshold = float(finiteness_abs_threshold) if finiteness_abs_threshold else 65500.0
         # RMSNorm runs inside the q/k/v and gate/up GEMVs (their prologue) unless told otherwise
@@ -135,6 +144,20 @@ class HipDecoder:
                            in_index if from_device_token else 0))
         self._out_index = out_index
         x, x2 = self.x, self.x2
+        if self.chain_gemvs and self.fuse_norm and not self.finiteness_guard:
+            self._enqueue_layers_chained(pos, device_kv_len)
+        else:
+            self._enqueue_layers(pos, device_kv_len)
+        ck(L.dh_rmsnorm(x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"],
+                        0, None, None, None, 1.0))
+        ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
+                                  self.lm_ws.data_ptr(), self.token.data_ptr(), self._out_index,
+                                  self.logits.data_ptr() if want_logits else None))
+
+    def _enqueue_layers(self, pos, device_kv_len):
+        L, c, ck = self.L, self.cfg, capi.check
+        Hd, I = c["hidden"], c["inter"]
+        x, x2 = self.x, self.x2
         for li, d in enumerate(self.layers):
             if self.fuse_norm:
                 ck(L.dh_q4k_matmul_rmsnorm(x.data_ptr(), d["input_norm"].data_ptr(), c["eps"], 0,
@@ -162,11 +185,35 @@ class HipDecoder:
             if self.finiteness_guard:
                 ck(L.dh_check_finiteness(x.data_ptr(), capi.F32, Hd, self.token.data_ptr() + 4 * self.TOKEN_RING, li,
                                          pos, self.finiteness_abs_threshold))
-        ck(L.dh_rmsnorm(x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"],
-                        0, None, None, None, 1.0))
-        ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
-                                  self.lm_ws.data_ptr(), self.token.data_ptr(), self._out_index,
-                                  self.logits.data_ptr() if want_logits else None))
+
+    def _chain_phases(self, li):
+        """o-projection, gate/up, down-projection of layer li and the q/k/v projection of layer li + 1 as
+        the products of one dh_q4k_gemv_chain launch (built once per layer and kept)."""
+        if not hasattr(self, "_chains"):
+            self._chains = {}
+        if li not in self._chains:
+            c, d = self.cfg, self.layers[li]
+            Hd, I = c["hidden"], c["inter"]
+            ph = [dict(W=d["wo"].data_ptr(), C=self.x2.data_ptr(), residual=self.x.data_ptr(), N=Hd, K=self.qs),
+                  dict(W=d["wgate"].data_ptr(), W2=d["wup"].data_ptr(), C=self.act.data_ptr(),
+                       norm_weight=d["post_attn_norm"].data_ptr(), N=I, K=Hd, activation=capi.ACT_SILU, norm_eps=c["eps"]),
+                  dict(W=d["wdown"].data_ptr(), C=self.x.data_ptr(), residual=self.x2.data_ptr(), N=Hd, K=I)]
+            if li + 1 < len(self.layers):
+                n = self.layers[li + 1]
+                ph.append(dict(W=n["wqkv"].data_ptr(), C=self.qkv.data_ptr(), norm_weight=n["input_norm"].data_ptr(),
+                               N=self.qs + 2 * self.ks, K=Hd, norm_eps=c["eps"]))
+            self._chains[li] = (capi.chain_phases(ph), len(ph))
+        return self._chains[li]
+
+    def _enqueue_layers_chained(self, pos, device_kv_len):
+        L, c, ck = self.L, self.cfg, capi.check
+        d0 = self.layers[0]
+        ck(L.dh_q4k_matmul_rmsnorm(self.x.data_ptr(), d0["input_norm"].data_ptr(), c["eps"], 0, d0["wqkv"].data_ptr(),
+                                   self.qkv.data_ptr(), capi.F32, 1, self.qs + 2 * self.ks, c["hidden"], 1.0, None))
+        for li, d in enumerate(self.layers):
+            self._enqueue_attention(d, pos, device_kv_len)
+            arr, n = self._chain_phases(li)
+            ck(L.dh_q4k_gemv_chain(self.attn.data_ptr(), arr, n))
 
     def _enqueue_attention(self, d, pos, device_kv_len=False):
         """self.qkv (raw stacked projection of the step's token) -> self.attn, appending the

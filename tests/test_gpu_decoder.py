@@ -360,6 +360,39 @@ def test_9b_class_centred_weights_sensitive_logits_and_greedy_tokens():
             assert rel_l2(g_rows, e_rows) <= 1e-3, (i, name)
 
 
+def test_chained_gemv_decoder_matches_the_oracle_and_the_separate_launches():
+    """chain_gemvs: o-projection, gate/up, down-projection and the next layer's q/k/v projection as one
+    launch per layer (dh_q4k_gemv_chain).  Tokens of the CPU oracle, logits within 1e-3, and the very
+    bits of the decoder that launches the products one by one; also replayed from a captured graph."""
+    cfg = dict(layers=3, hidden=2048, inter=4096, heads=16, kv_heads=4, head_dim=128, vocab=1000, eps=1e-6, qk_norm=1,
+               max_seq=48, theta=1e6)
+    layers, embed, final_norm, cos, sin = decoder.random_model(cfg, seed=81, max_seq=cfg["max_seq"])
+    for l in layers:
+        for n in ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown"):
+            l[n] = synth.q4k_centred(l[n], 5)           # a stack whose logits depend on what it is fed
+    chained = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, cfg["max_seq"], chain_gemvs=True)
+    plain = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, cfg["max_seq"])
+    ol = oracle_layers(layers, cfg["max_seq"], cfg["kv_heads"], cfg["head_dim"])
+    cpu = oracle.DecoderOracle(cfg, ol, embed, final_norm, cos, sin)
+    prompt = synth.rng(82).integers(0, cfg["vocab"], 10)
+    tok = None
+    for pos in range(30):
+        inp = int(prompt[pos]) if pos < len(prompt) else tok
+        g = chained.step_graph(inp, pos) if pos >= 20 else chained.step(inp, pos, want_logits=True)
+        p = plain.step(inp, pos, want_logits=True)
+        ctok, want = cpu.step(inp, pos, want_logits=True)
+        if pos < 20:
+            assert chained.read_logits().tobytes() == plain.read_logits().tobytes(), pos
+            assert rel_l2(chained.read_logits(), want) <= 1e-3, pos
+        assert g == p == ctok, (pos, g, p, ctok)
+        tok = g
+    chained.release_graph()
+    with pytest.raises(ValueError, match="chain"):
+        small = dict(cfg, hidden=512, inter=1024, heads=4, kv_heads=2)
+        sl, se, sf, sc, ss = decoder.random_model(small, seed=83, max_seq=cfg["max_seq"])
+        decoder.HipDecoder(small, sl, se, sf, sc, ss, cfg["max_seq"], chain_gemvs=True)
+
+
 def test_decode_positions_outside_the_cache_are_refused():
     """The ops take no cache capacity, so the host must refuse a position past the caches before
     anything is enqueued (no GPU work happens for the refused calls)."""
