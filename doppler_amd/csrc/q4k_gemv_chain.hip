@@ -8,11 +8,14 @@
 // four launches costs four times the dispatch-to-first-byte floor of a launch with the HBM idle.
 //
 // One persistent workgroup of 16 waves per compute unit.  Every workgroup owns fixed row tiles of
-// every matrix; a work unit is one tile x one 256-weight super-block column (<= 16 rows x 144 bytes),
-// and the units of all phases form ONE sequence per workgroup that its waves draw from a counter in
-// LDS.  A wave keeps two units in flight (global_load_lds into its private two-stage ring), so the
-// weight stream runs on across a phase boundary: while the outputs of phase p travel between the
-// workgroups, the first 32 units per compute unit of phase p + 1 are already on their way into LDS.
+// every matrix; a work unit is one tile x one 256-weight super-block column (<= 16 rows x 144 bytes).
+// Inside a phase the waves draw the workgroup's units from a counter in LDS, one unit in flight per
+// wave (global_load_lds into its private ring; a second one in flight was measured slower: the
+// stream is bandwidth-bound with sixteen, and a longer first burst only delays the first results).
+// A wave that finds no unit left in phase p moves on alone: it requests its first unit of phase p + 1
+// (unit `wave`, no draw) BEFORE it waits at the exchange, so while the outputs of phase p travel
+// between the workgroups the first sixteen units per compute unit of phase p + 1 are on their way
+// into LDS.
 //
 // Exchange.  The wave that finishes a tile writes its outputs to C and, for every phase but the last,
 // publishes them as (value, sequence number) pairs with 8-byte device-scope stores (an 8-byte store
@@ -50,9 +53,8 @@ typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 
 constexpr int kWaves = 16;
 constexpr int kTileRows = 16;
-constexpr int kStage = kTileRows * kBlockBytes;   // 2304 bytes per ring stage
+constexpr int kStage = kTileRows * kBlockBytes;   // 2304 bytes: a wave's ring holds one unit
 constexpr int kUnitLoads = 3;                     // load instructions of a full unit: ceil(16 rows * 9 pieces / 64 lanes)
-constexpr int kDepth = 2;                         // ring stages per wave
 constexpr int kMaxPhases = DH_CHAIN_MAX_PHASES;
 constexpr int kSlots = 8;                         // tiles whose partial sums may be in LDS at once (a power of two)
 constexpr int kSlotShift = 3;
@@ -61,11 +63,14 @@ constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kMaxChainN = 32768;                 // longest exchanged vector
 constexpr int kDefaultSpinLimit = 1 << 17;        // polls of one bounded wait
 constexpr int kColsPerPass = 3;                   // columns whose loads a wave has in flight at once in the prologue
-// counters in LDS: [0] next unit, [1 + s] units delivered to slot s, [1 + kSlots + s] tiles completed
-// in slot s, [1 + 2 kSlots] a wave has given up, [2 + 2 kSlots + p] tiles of phase p this workgroup has
-// finished, then the column flags of the two record areas
-constexpr int kCtrAbort = 1 + 2 * kSlots;
-constexpr int kCtrDone = 2 + 2 * kSlots;
+// counters in LDS: [p] next unit of phase p to draw, [kCtrArrived + s] units delivered to slot s,
+// [kCtrGen + s] tiles completed in slot s, [kCtrAbort] a wave has given up, [kCtrDone + p] tiles of
+// phase p this workgroup has finished, then the column flags of the two record areas
+constexpr int kCtrNext = 0;
+constexpr int kCtrArrived = kMaxPhases;
+constexpr int kCtrGen = kCtrArrived + kSlots;
+constexpr int kCtrAbort = kCtrGen + kSlots;
+constexpr int kCtrDone = kCtrAbort + 1;
 constexpr int kCtrFlags = kCtrDone + kMaxPhases;
 // a tile's partial sums are read four columns at a time: the last read may reach past the counters
 constexpr int kLdsPad = 1024;
@@ -74,16 +79,13 @@ constexpr int kLdsPad = 1024;
 // s_waitcnt with only the vector-memory counter set (6 bits, split 4 + 2 in the encoding).
 #define DH_WAIT_VM(k) __builtin_amdgcn_s_waitcnt(((k) & 0xF) | (((k) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
 
-// Waits until at most n of this wave's vector-memory operations are outstanding (loads complete in
-// issue order).  Counts without a case wait for everything, which is always safe.
+// Waits until at most n (0..3) of this wave's vector-memory operations are outstanding (they
+// complete in issue order).
 __device__ __forceinline__ void wait_vm_at_most(int n) {
   switch (n) {
     case 1: DH_WAIT_VM(1); break;
     case 2: DH_WAIT_VM(2); break;
     case 3: DH_WAIT_VM(3); break;
-    case 4: DH_WAIT_VM(4); break;
-    case 5: DH_WAIT_VM(5); break;
-    case 6: DH_WAIT_VM(6); break;
     default: DH_WAIT_VM(0); break;
   }
 }
@@ -125,24 +127,29 @@ __device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
   return v;
 }
 
-#define DH_SEL4(p_, a0_, a1_, a2_, a3_) ((p_) == 0 ? (a0_) : (p_) == 1 ? (a1_) : (p_) == 2 ? (a2_) : (a3_))
-
 __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const ChainArgs a) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bid = blockIdx.x;
+  // what every phase uses is fetched in one batch here (left alone the compiler fetches an argument
+  // where it is first used: a dependent trip to memory each time)
+  asm volatile("" :: "s"(a.x0), "s"(a.ll), "s"(a.epoch), "s"(a.status));
+  asm volatile("" :: "s"(a.nph), "s"(a.grid), "s"(a.spin_limit), "s"(a.xq_bytes[0]), "s"(a.xq_bytes[1]), "s"(a.nb_max[0]),
+               "s"(a.nb_max[1]), "s"(a.red_stride));
+  asm volatile("" :: "s"(a.ph[0].norm_weight), "s"(a.ph[0].nb));
 
-  // ---- LDS: ring [16 waves][2][2304], record areas 0 and 1, zeros [144], partial sums
+  // ---- LDS: ring [16 waves][2304], record areas 0 and 1, zeros [144], partial sums
   // [kSlots][red_stride], counters
   unsigned char* ring = lds;
-  unsigned char* xq0 = ring + (size_t)kWaves * kDepth * kStage;
+  unsigned char* xq0 = ring + (size_t)kWaves * kStage;
   unsigned char* xq1 = xq0 + a.xq_bytes[0];
   unsigned char* zeros = xq1 + a.xq_bytes[1];
   float* red = reinterpret_cast<float*>(zeros + kZeroBytes);
   unsigned* ctr = reinterpret_cast<unsigned*>(red + (size_t)kSlots * a.red_stride);
   const int nflags = a.nb_max[0] + a.nb_max[1];
-  for (int i = tid; i < kCtrFlags + nflags; i += 64 * kWaves) ctr[i] = 0u;
+  // (every wave takes unit `wave` of a phase without drawing: the unit counters start behind those)
+  for (int i = tid; i < kCtrFlags + nflags; i += 64 * kWaves) ctr[i] = i < kMaxPhases ? (unsigned)kWaves : 0u;
   if (tid >= 64 && tid < 64 + kZeroBytes / 4) reinterpret_cast<uint32_t*>(zeros)[tid - 64] = 0u;
 
   // the launch counter: requested first, so that it arrives with (ahead of) phase 0's activations and
@@ -152,22 +159,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
   uint32_t seq_base = 0;
   const int nph = a.nph;
 
-  // ---- this workgroup's unit and tile ranges: phase p holds units [ub_p, ub_{p+1}) and tile ordinals
-  // [tb_p, tb_{p+1}); its tiles are bid, bid + grid, ..
-  int ubv[kMaxPhases + 1], tbv[kMaxPhases + 1];
-  ubv[0] = 0;
-  tbv[0] = 0;
-#pragma unroll
-  for (int p = 0; p < kMaxPhases; p++) {
-    const int ntl = p < nph ? a.ph[p].tiles_base + (bid < a.ph[p].tiles_rem ? 1 : 0) : 0;
-    ubv[p + 1] = ubv[p] + ntl * (p < nph ? a.ph[p].upt : 0);
-    tbv[p + 1] = tbv[p] + ntl;
-  }
-  const int ub1 = ubv[1], ub2 = ubv[2], ub3 = ubv[3], total = ubv[4];
-  const int tb1 = tbv[1], tb2 = tbv[2], tb3 = tbv[3];
-  auto phase_of = [&](const int u) { return (u >= ub1 ? 1 : 0) + (u >= ub2 ? 1 : 0) + (u >= ub3 ? 1 : 0); };
-
-  unsigned char* my_ring = ring + (size_t)wave * kDepth * kStage;
+  unsigned char* my_ring = ring + (size_t)wave * kStage;
   const uint32_t ctr_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(ctr);
   const uint32_t abort_addr = ctr_abs + 4 * kCtrAbort;
   const uint32_t red_abs = (uint32_t)(uintptr_t)DH_LDS_PTR(red);
@@ -186,94 +178,44 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
     __builtin_amdgcn_endpgm();          // the wave ends here (no barrier follows)
   };
 
-  // ---- issue side: the phase whose units are being requested
-  int ip = -1, i_rows = 0, i_N = 0, i_nb = 1, i_upt = 1, i_upt_mul = 0, i_ub = 0, i_nlw = 0;
-  const uint8_t* iW = nullptr;
-  const uint8_t* iW2 = nullptr;
-  int64_t i_row_bytes = 0;
-  uint32_t goff[kUnitLoads];       // piece t * 64 + lane of a unit: row p / 9, 16-byte piece p % 9 of that row's super-block
-#pragma unroll
-  for (int t = 0; t < kUnitLoads; t++) goff[t] = 0xFFFFFFFFu;
-  auto issue_setup = [&](const int p) {
-    ip = p;
-    const Phase& P = a.ph[p];
-    iW = P.W; iW2 = P.W2; i_rows = P.rows; i_N = P.N; i_nb = P.nb; i_upt = P.upt; i_upt_mul = P.upt_mul; i_nlw = P.nlw;
-    i_ub = DH_SEL4(p, 0, ub1, ub2, ub3);
-    i_row_bytes = (int64_t)P.nb * kBlockBytes;
-#pragma unroll
-    for (int t = 0; t < kUnitLoads; t++) {
-      const int q = t * 64 + lane, r = q / 9;
-      goff[t] = q < 9 * i_rows ? (uint32_t)(r * i_row_bytes + (q - r * 9) * 16) : 0xFFFFFFFFu;
-    }
-  };
-  // Puts the loads of unit u in flight into ring stage `stage`; returns the number of load instructions.
-  auto issue = [&](const int u, const int stage) -> int {
-    const int p = phase_of(u);
-    if (p != ip) issue_setup(p);
-    const int local = u - i_ub;
-    const int tl = (int)(((unsigned)local * (unsigned)i_upt_mul) >> 24);
-    const int r = local - tl * i_upt;
-    const int mat = r >= i_nb ? 1 : 0;
-    const int col = r - mat * i_nb;
-    const int tile = bid + tl * a.grid;
-    const uint8_t* base = (mat ? iW2 : iW) + (int64_t)tile * i_rows * i_row_bytes + (int64_t)col * kBlockBytes;
-    unsigned char* st = my_ring + stage * kStage;
-    const int rows_left = i_N - tile * i_rows;
-    if (rows_left >= i_rows) {
-#pragma unroll
-      for (int t = 0; t < kUnitLoads; t++) {
-        if (goff[t] != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + goff[t], DH_LDS_PTR(st + t * 1024), 16, 0, 0);
-      }
-    } else {
-#pragma unroll
-      for (int t = 0; t < kUnitLoads; t++) {
-        const int q = t * 64 + lane, rr = q / 9;
-        const int64_t o = (int64_t)min(rr, rows_left - 1) * i_row_bytes + (q - rr * 9) * 16;
-        if (goff[t] != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + o, DH_LDS_PTR(st + t * 1024), 16, 0, 0);
-      }
-    }
-    return i_nlw;
-  };
-
-  // ---- the prologue of phase p: this wave's share of the phase's activations, columns
-  // (wave - bid) mod 16, + 16, .. (rotated by workgroup so that the workgroups do not all ask for the
-  // same lines at the same moment), kColsPerPass of them per pass.  Lane t holds elements 4t .. 4t+3 of
-  // a column.  Phase 0 reads x0, written before the launch; later phases read the pairs the other
-  // workgroups publish and retry until every sequence number is the expected one.
+  // ---- a phase's activations: this wave's share is columns (wave - bid) mod 16, + 16, .. (rotated by
+  // workgroup so that the workgroups do not all ask for the same lines at the same moment),
+  // kColsPerPass of them per pass.  Lane t holds elements 4t .. 4t+3 of a column.  Phase 0 reads x0,
+  // written before the launch; later phases read the pairs the other workgroups publish and retry
+  // until every sequence number is the expected one.
   struct Cols {
     v4f xr[kColsPerPass], wr[kColsPerPass];
   };
   const int c_first = (wave - bid) & (kWaves - 1);
-  auto load_norm = [&](const Phase& P, const int c0, Cols& R) {
-    if (P.norm_weight == nullptr) return;
+  auto load_norm = [&](const float* nw, const int nb, const int c0, Cols& R) {
+    if (nw == nullptr) return;
 #pragma unroll
     for (int i = 0; i < kColsPerPass; i++) {
       const int c = c0 + kWaves * i;
-      if (c < P.nb) {
-        const float* q = P.norm_weight + c * kQK + 4 * lane;
+      if (c < nb) {
+        const float* q = nw + c * kQK + 4 * lane;
         asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(R.wr[i]) : "v"(q) : "memory");
       }
     }
   };
-  auto load_x0 = [&](const Phase& P, const int c0, Cols& R) {
+  auto load_x0 = [&](const int nb, const int c0, Cols& R) {
 #pragma unroll
     for (int i = 0; i < kColsPerPass; i++) {
       const int c = c0 + kWaves * i;
-      if (c < P.nb) {
+      if (c < nb) {
         const float* q = a.x0 + c * kQK + 4 * lane;
         asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(R.xr[i]) : "v"(q) : "memory");
       }
     }
   };
   // Quantises the columns of a pass (their values have landed) and raises their flags.
-  auto finish_pass = [&](const int p, const Phase& P, const int c0, Cols& R) {
-    const bool norm = P.norm_weight != nullptr;
+  auto finish_pass = [&](const int p, const bool norm, const int nwo, const int nb, const int c0, Cols& R) {
     unsigned char* xq = (p & 1) ? xq1 : xq0;
     unsigned* flags = ctr + kCtrFlags + ((p & 1) ? a.nb_max[0] : 0);
 #pragma unroll
     for (int i = 0; i < kColsPerPass; i++) {
       const int c = c0 + kWaves * i;
-      if (c < P.nb) {
+      if (c < nb) {
         asm volatile("" : "+v"(R.xr[i]));
         if (norm) asm volatile("" : "+v"(R.wr[i]));
         float v[4], ss = 0.f;
@@ -282,7 +224,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
           v[e] = R.xr[i][e];
           if (norm) {
             ss = fmaf(v[e], v[e], ss);
-            v[e] *= P.norm_weight_offset ? 1.0f + R.wr[i][e] : R.wr[i][e];
+            v[e] *= nwo ? 1.0f + R.wr[i][e] : R.wr[i][e];
           }
         }
         unsigned char* rec = xq + (size_t)c * kRec;
@@ -296,108 +238,15 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
       }
     }
   };
-  // Phases after the first.
-  auto prologue = [&](const int p) {
-    const Phase& P = a.ph[p];
-    const int nb = P.nb;
-    const v2u* src = a.ll + (size_t)((p - 1) & 1) * kMaxChainN;
-    const uint32_t want = seq_base + (uint32_t)p;
-    // Not before this workgroup has finished its own tiles of the previous phase: the workgroups run
-    // the same work at the same pace, so until then the others have not finished theirs either, and
-    // polls that cannot succeed yet would only compete with the weight stream for the memory system.
-    {
-      const unsigned mine = (unsigned)(DH_SEL4(p, 0, tb1, tb2 - tb1, tb3 - tb2));
-      const uint32_t done_addr = ctr_abs + 4 * (kCtrDone + p - 1);
-      int spins = 0;
-#ifndef DH_CHAIN_EXP_NOWAIT
-      while (__builtin_amdgcn_readfirstlane(lds_read_u32(done_addr)) < mine) {
-        if (++spins > a.spin_limit * 8 || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u)
-          give_up(DH_KSTATUS_SLOT_WAIT, p);
-        __builtin_amdgcn_s_sleep(4);
-      }
-#endif
-    }
-#pragma unroll 1
-    for (int c0 = c_first; c0 < nb; c0 += kWaves * kColsPerPass) {
-      Cols R;
-      v4u la[kColsPerPass], lb[kColsPerPass];
-      load_norm(P, c0, R);
-      int spins = 0;
-      for (;;) {
-#pragma unroll
-        for (int i = 0; i < kColsPerPass; i++) {
-          const int c = c0 + kWaves * i;
-          if (c < nb) {
-            const v2u* q = src + c * kQK + 4 * lane;
-            asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1"
-                         : "=&v"(la[i]), "=&v"(lb[i]) : "v"(q) : "memory");
-          }
-        }
-        DH_WAIT_VM(0);
-        bool ok = true;
-#pragma unroll
-        for (int i = 0; i < kColsPerPass; i++) {
-          const int c = c0 + kWaves * i;
-          if (c < nb) {
-            asm volatile("" : "+v"(la[i]), "+v"(lb[i]));
-            ok = ok && la[i].y == want && la[i].w == want && lb[i].y == want && lb[i].w == want;
-          }
-        }
-#ifdef DH_CHAIN_EXP_NOWAIT
-        break;
-#endif
-        if (__builtin_amdgcn_ballot_w64(!ok) == 0ull) break;
-        if (++spins > a.spin_limit || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) {
-          give_up(DH_KSTATUS_EXCHANGE_WAIT, p);
-        }
-        __builtin_amdgcn_s_sleep(8);
-      }
-#pragma unroll
-      for (int i = 0; i < kColsPerPass; i++)
-        R.xr[i] = v4f{__uint_as_float(la[i].x), __uint_as_float(la[i].z), __uint_as_float(lb[i].x), __uint_as_float(lb[i].z)};
-      finish_pass(p, P, c0, R);
-    }
-  };
 
   // the first pass of phase 0: its loads go out before the barrier and before any weights, so that
   // they are at the head of the compute unit's memory queue
   Cols first;
-  load_norm(a.ph[0], c_first, first);
-  load_x0(a.ph[0], c_first, first);
+  load_norm(a.ph[0].norm_weight, a.ph[0].nb, c_first, first);
+  load_x0(a.ph[0].nb, c_first, first);
 
   // counters, flags and the zero area are in place
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  if (total == 0) return;
-
-  // Draws the next unit of the workgroup (wave-uniform result).
-  auto draw = [&]() -> int {
-    unsigned v = 0;
-    if (lane == 0)
-      asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(v) : "v"(ctr_abs), "v"(1u) : "memory");
-    return (int)__builtin_amdgcn_readfirstlane(v);
-  };
-
-  // ---- the first two units' loads go out before anything else is waited for
-  int u_st0 = 0x7fffffff, u_st1 = 0x7fffffff;     // units in the two ring stages (>= total: none)
-  int nl_st0 = 0, nl_st1 = 0;                      // their load instruction counts
-  u_st0 = draw();
-  if (u_st0 < total) {
-    nl_st0 = issue(u_st0, 0);
-    u_st1 = draw();
-    if (u_st1 < total) nl_st1 = issue(u_st1, 1);
-  }
-  // phase 0's activations: only they are waited for (the units were requested behind them)
-  wait_vm_at_most(nl_st0 + nl_st1);
-  asm volatile("" : "+v"(epoch_v));
-  seq_base = __builtin_amdgcn_readfirstlane(epoch_v) * 8u;
-  finish_pass(0, a.ph[0], c_first, first);
-#pragma unroll 1
-  for (int c0 = c_first + kWaves * kColsPerPass; c0 < a.ph[0].nb; c0 += kWaves * kColsPerPass) {
-    load_norm(a.ph[0], c0, first);
-    load_x0(a.ph[0], c0, first);
-    DH_WAIT_VM(0);
-    finish_pass(0, a.ph[0], c0, first);
-  }
 
   // operand addressing (see q4k_gemv_i8.hip): MFMA pair cc covers sub-blocks 4cc .. 4cc+3; lane
   // (i = lane & 15, kg) supplies operand row i = 4g + digit: 16 digit bytes where its row's sub-block is
@@ -415,53 +264,181 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
       a_off[h] = has ? data_off : zero_abs;
     }
   }
-  const uint32_t lane_hdr = (uint32_t)(uintptr_t)DH_LDS_PTR(my_ring) + (uint32_t)j * kBlockBytes;
-  const uint32_t lane_q = lane_hdr + 16 + 32 * (kg >> 1) + 16 * (kg & 1);
+  const uint32_t hp = (uint32_t)(uintptr_t)DH_LDS_PTR(my_ring) + (uint32_t)j * kBlockBytes;   // this lane's row header in the ring
+  const uint32_t qp = hp + 16 + 32 * (kg >> 1) + 16 * (kg & 1);                               // its 16 nibble bytes of chunk kg >> 1
   const uint32_t sh_lo = 8 * kg;           // bit offset of this lane's byte in the header words
 
-  // ---- process side: phase by phase; inside a phase the unit loop runs on the phase's own scalars.
-  // A wave enters phase p when the unit at the head of its ring is not of an earlier phase any more;
-  // on the way in it prepares its share of the phase's activations (phase 0: done above), which the
-  // other waves count on whether or not this wave draws a unit of the phase.
-  float inv_rms = 1.f;
-  bool have_rms = false;
-  int cstage = 0;
+  // What putting a unit's loads in flight needs of its phase.
+  struct Stream {
+    const uint8_t* W;
+    const uint8_t* W2;
+    int64_t row_bytes;
+    int N, nb, dual, rows, upt, upt_mul;
+    uint32_t goff[kUnitLoads];     // piece t * 64 + lane of a unit: row q / 9, 16-byte piece q % 9 of that row's super-block
+  };
+  auto stream_of = [&](const Phase& Q) {
+    Stream S;
+    S.W = Q.W; S.W2 = Q.W2; S.N = Q.N; S.nb = Q.nb; S.dual = Q.nmat - 1; S.rows = Q.rows; S.upt = Q.upt; S.upt_mul = Q.upt_mul;
+    S.row_bytes = (int64_t)Q.nb * kBlockBytes;
+#pragma unroll
+    for (int t = 0; t < kUnitLoads; t++) {
+      const int q = t * 64 + lane, r = q / 9;
+      S.goff[t] = q < 9 * S.rows ? (uint32_t)(r * S.row_bytes + (q - r * 9) * 16) : 0xFFFFFFFFu;
+    }
+    return S;
+  };
+  // Unit u of a workgroup's phase = (tile ordinal tl, matrix, column): u = (tl * nmat + mat) * nb + col.
+#define DH_DECODE(S_, u_, tl_, mat_, col_)                                   \
+  const int tl_ = (int)(((unsigned)(u_) * (unsigned)(S_).upt_mul) >> 24);    \
+  const int r__##tl_ = (u_) - tl_ * (S_).upt;                                \
+  const int mat_ = ((S_).dual && r__##tl_ >= (S_).nb) ? 1 : 0;               \
+  const int col_ = r__##tl_ - mat_ * (S_).nb;
+  // Puts the loads of unit u in flight into the wave's ring.
+  auto issue = [&](const Stream& S, const int u) {
+    DH_DECODE(S, u, itl, imat, icol)
+    const int tile = bid + itl * a.grid;
+    const uint8_t* base = (imat ? S.W2 : S.W) + (int64_t)tile * S.rows * S.row_bytes + (int64_t)icol * kBlockBytes;
+    const int rows_left = S.N - tile * S.rows;
+    if (rows_left >= S.rows) {
+#pragma unroll
+      for (int t = 0; t < kUnitLoads; t++) {
+        if (S.goff[t] != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + S.goff[t], DH_LDS_PTR(my_ring + t * 1024), 16, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < kUnitLoads; t++) {
+        const int q = t * 64 + lane, rr = q / 9;
+        const int64_t o = (int64_t)min(rr, rows_left - 1) * S.row_bytes + (q - rr * 9) * 16;
+        if (S.goff[t] != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + o, DH_LDS_PTR(my_ring + t * 1024), 16, 0, 0);
+      }
+    }
+  };
+
+  // ---- phase 0's activations come from x0: the wave's first unit (unit `wave`, no draw) is requested
+  // behind their loads, and only they are waited for
+  int cur;                                  // the unit in the ring (>= its phase's total: none)
+  {
+    const Phase& Q = a.ph[0];
+    const Stream S = stream_of(Q);
+    const int total = (Q.tiles_base + (bid < Q.tiles_rem ? 1 : 0)) * Q.upt;
+    const int nb = Q.nb, nwo = Q.norm_weight_offset;
+    const float* const nw = Q.norm_weight;
+    cur = wave < total ? wave : 0x7fffffff;
+    if (cur < total) issue(S, cur);
+    wait_vm_at_most(cur < total ? Q.nlw : 0);
+    asm volatile("" : "+v"(epoch_v));
+    seq_base = __builtin_amdgcn_readfirstlane(epoch_v) * 8u;
+    finish_pass(0, nw != nullptr, nwo, nb, c_first, first);
+#pragma unroll 1
+    for (int c0 = c_first + kWaves * kColsPerPass; c0 < nb; c0 += kWaves * kColsPerPass) {
+      Cols R;
+      load_norm(nw, nb, c0, R);
+      load_x0(nb, c0, R);
+      DH_WAIT_VM(0);
+      finish_pass(0, nw != nullptr, nwo, nb, c0, R);
+    }
+  }
+
+  // ---- phase by phase.  A wave enters phase p when phase p - 1 has no unit left for it to draw.
+  // On the way in it requests its first unit of the phase (the weights do not depend on the
+  // exchange, and its ring is free), then prepares its share of the phase's activations, which the
+  // other waves count on whether or not this wave gets a unit of the phase.
+  int tb = 0;                               // tile ordinal (over all phases) of the phase's first tile in this workgroup
+  int prev_ntl = 0;                         // tiles of this workgroup in the previous phase
 #pragma unroll 1
   for (int p = 0; p < nph; p++) {
-    if (p > 0) prologue(p);
-    const Phase& P = a.ph[p];
-    const int p_nb = P.nb, p_upt = P.upt, p_upt_mul = P.upt_mul, p_dual = P.nmat - 1;
-    const int p_ub = DH_SEL4(p, 0, ub1, ub2, ub3), p_ue = DH_SEL4(p, ub1, ub2, ub3, total);
-    const int p_tb = DH_SEL4(p, 0, tb1, tb2, tb3);
-    const uint32_t p_xq = (p & 1) ? xq_abs1 : xq_abs0;
-    const uint32_t p_flags = ctr_abs + 4 * (kCtrFlags + ((p & 1) ? a.nb_max[0] : 0));
+    const Phase& Q = a.ph[p];
+    const Stream S = stream_of(Q);
+    // what the unit loop itself reads is fetched together; what only a tile's end needs is fetched there
+    asm volatile("" :: "s"(S.W), "s"(S.W2), "s"(S.N), "s"(S.nb), "s"(S.dual), "s"(S.rows), "s"(S.upt), "s"(S.upt_mul));
+    const int nb = S.nb, upt = S.upt;
+    const float* const nw = Q.norm_weight;
+    const bool norm = nw != nullptr;
+    const int ntl = Q.tiles_base + (bid < Q.tiles_rem ? 1 : 0);
+    const int total = ntl * upt;                       // units of this workgroup in this phase
+    const uint32_t xq_abs = (p & 1) ? xq_abs1 : xq_abs0;
+    const uint32_t flags_abs = ctr_abs + 4 * (kCtrFlags + ((p & 1) ? a.nb_max[0] : 0));
+    const uint32_t next_abs = ctr_abs + 4 * (kCtrNext + p);
     const uint32_t flag_want = (uint32_t)p + 1u;
     const bool last_phase = p == nph - 1;
-    have_rms = false;
 
-    // The units of this phase, from the head of the ring (stage cstage; the two stages alternate).
+    if (p > 0) {
+      // ---- the wave's first unit of the phase: unit `wave`, no draw
+      cur = wave < total ? wave : 0x7fffffff;
+      if (cur < total) issue(S, cur);
+
+      // ---- the phase's activations
+      const int nwo = Q.norm_weight_offset;
+      const v2u* src = a.ll + (size_t)((p - 1) & 1) * kMaxChainN;
+      const uint32_t want = seq_base + (uint32_t)p;
+      // Not before this workgroup has finished its own tiles of the previous phase: the workgroups run
+      // the same work at the same pace, so until then the others have not finished theirs either, and
+      // polls that cannot succeed yet would only compete with the weight stream for the memory system.
+      {
+        const uint32_t done_addr = ctr_abs + 4 * (kCtrDone + p - 1);
+        int spins = 0;
+        while (__builtin_amdgcn_readfirstlane(lds_read_u32(done_addr)) < (unsigned)prev_ntl) {
+          if (++spins > a.spin_limit * 8 || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u)
+            give_up(DH_KSTATUS_SLOT_WAIT, p);
+          __builtin_amdgcn_s_sleep(4);
+        }
+      }
+#pragma unroll 1
+      for (int c0 = c_first; c0 < nb; c0 += kWaves * kColsPerPass) {
+        Cols R;
+        v4u la[kColsPerPass], lb[kColsPerPass];
+        load_norm(nw, nb, c0, R);
+        int spins = 0;
+        for (;;) {
+#pragma unroll
+          for (int i = 0; i < kColsPerPass; i++) {
+            const int c = c0 + kWaves * i;
+            if (c < nb) {
+              const v2u* q = src + c * kQK + 4 * lane;
+              asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1"
+                           : "=&v"(la[i]), "=&v"(lb[i]) : "v"(q) : "memory");
+            }
+          }
+          DH_WAIT_VM(0);
+          bool ok = true;
+#pragma unroll
+          for (int i = 0; i < kColsPerPass; i++) {
+            const int c = c0 + kWaves * i;
+            if (c < nb) {
+              asm volatile("" : "+v"(la[i]), "+v"(lb[i]));
+              ok = ok && la[i].y == want && la[i].w == want && lb[i].y == want && lb[i].w == want;
+            }
+          }
+          if (__builtin_amdgcn_ballot_w64(!ok) == 0ull) break;
+          if (++spins > a.spin_limit || __builtin_amdgcn_readfirstlane(lds_read_u32(abort_addr)) != 0u) {
+            give_up(DH_KSTATUS_EXCHANGE_WAIT, p);
+          }
+          __builtin_amdgcn_s_sleep(8);
+        }
+#pragma unroll
+        for (int i = 0; i < kColsPerPass; i++)
+          R.xr[i] = v4f{__uint_as_float(la[i].x), __uint_as_float(la[i].z), __uint_as_float(lb[i].x), __uint_as_float(lb[i].z)};
+        finish_pass(p, norm, nwo, nb, c0, R);
+      }
+    }
+
+    // ---- the phase's units
+    float inv_rms = 1.f;
+    bool have_rms = false;
 #pragma unroll 1
     for (;;) {
-      const int ST = cstage;
-      const int cur = ST ? u_st1 : u_st0;
-      if (cur >= p_ue) break;             // a later phase's unit (or none): draws only grow
-      const int local = cur - p_ub;
-      const int tl = (int)(((unsigned)local * (unsigned)p_upt_mul) >> 24);
-      const int rr = local - tl * p_upt;
-      const int mat = (p_dual && rr >= p_nb) ? 1 : 0;
-      const int col = rr - mat * p_nb;
-      const int tord = p_tb + tl;                       // tile ordinal of the workgroup, over all phases
+      if (cur >= total) break;              // draws only grow: nothing behind this one either
+      DH_DECODE(S, cur, tl, mat, col)
+      const int tord = tb + tl;                         // tile ordinal of the workgroup, over all phases
       const int slot = tord & (kSlots - 1);
-      // draw the unit that will go into this stage once it has been read (the answer is collected with
-      // the reads below)
+      // draw the unit that will go into the ring once this one has been read (the answer is collected
+      // with the reads below)
       unsigned nxt = 0;
-      if (lane == 0) asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=&v"(nxt) : "v"(ctr_abs), "v"(1u) : "memory");
-      // the other stage's loads were issued after this one's
-      wait_vm_at_most(ST ? nl_st0 : nl_st1);
-      const uint32_t hp = lane_hdr + ST * kStage, qp = lane_q + ST * kStage;
-      const uint32_t rec = p_xq + (uint32_t)col * kRec;
-      const uint32_t gen_addr = ctr_abs + 4 * (1 + kSlots + slot);
-      const uint32_t flag_addr = p_flags + 4 * col;
+      if (lane == 0) asm volatile("ds_add_rtn_u32 %0, %1, %2" : "=&v"(nxt) : "v"(next_abs), "v"(1u) : "memory");
+      DH_WAIT_VM(0);
+      const uint32_t rec = xq_abs + (uint32_t)col * kRec;
+      const uint32_t gen_addr = ctr_abs + 4 * (kCtrGen + slot);
+      const uint32_t flag_addr = flags_abs + 4 * col;
       v4u h, q0, q1;
       v4i ax[2][2];
       v2f sx, xinv;
@@ -508,13 +485,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
       }
 #undef DH_READ_OPERANDS
 #undef DH_TIE_OPERANDS
-      // the stage is free again: put the loads of the unit drawn above in flight
-      {
-        const int u = (int)__builtin_amdgcn_readfirstlane(nxt);
-        const int nl = u < total ? issue(u, ST) : 0;
-        if (ST) { u_st1 = u; nl_st1 = nl; } else { u_st0 = u; nl_st0 = nl; }
-      }
-      cstage ^= 1;
+      // the ring is free again: put the loads of the unit drawn above in flight
+      cur = (int)__builtin_amdgcn_readfirstlane(nxt);
+      if (cur < total) issue(S, cur);
 
       // 6-bit scales and mins of sub-blocks kg and 4 + kg of this lane's weight row
       const int sc_a = (int)((h.y >> sh_lo) & 63u);
@@ -550,19 +523,19 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
       }
       // the four lane groups hold different sub-blocks of the same 16 rows
       const float sres = sum_lane_groups(i8_unit_term(dd[0], dd[1], sc_a, sc_b, mn_a, mn_b, d, dmin, sx, xinv));
-      if (lane < 16) red[(size_t)slot * a.red_stride + (mat * p_nb + col) * 16 + lane] = sres;
+      if (lane < 16) red[(size_t)slot * a.red_stride + (mat * nb + col) * 16 + lane] = sres;
 
       // ---- deliver.  LDS executes a wave's operations in order, so the partial sums above are in
       // place before the count below is; the wave that delivers a tile's last unit finishes it.
       unsigned arrived = 0;
       if (lane == 0)
         asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)"
-                     : "=&v"(arrived) : "v"(ctr_abs + 4 * (1 + slot)), "v"(1u) : "memory");
+                     : "=&v"(arrived) : "v"(ctr_abs + 4 * (kCtrArrived + slot)), "v"(1u) : "memory");
       arrived = __builtin_amdgcn_readfirstlane(arrived);
-      if ((int)arrived == p_upt - 1) {
-        const int nb = p_nb;
+      if ((int)arrived == upt - 1) {
         const int tile = bid + tl * a.grid;
-        const int64_t row = (int64_t)tile * P.rows + j;
+        const int rows = S.rows, N = S.N, dual = S.dual;
+        const int64_t row = (int64_t)tile * rows + j;
         const uint32_t slot_abs = red_abs + (uint32_t)slot * a.red_stride * 4;
         // lane (j, kg) adds columns kg, kg + 4, .. (four reads in flight at a time); the four groups then
         // meet.  The order is fixed, so the result does not depend on who arrives last.
@@ -571,7 +544,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
           float r[2][4];
 #pragma unroll
           for (int mt = 0; mt < 2; mt++) {
-            if (mt == 0 || p_dual) {
+            if (mt == 0 || S.dual) {
               const uint32_t q = slot_abs + ((mt * nb + c) * 16 + j) * 4;
               asm volatile(
                   "ds_read_b32 %0, %4\n\t"
@@ -596,29 +569,32 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
         }
         sg = sum_lane_groups(sg);
         su = sum_lane_groups(su);
-        if (P.norm_weight != nullptr) {
+        if (norm) {
           if (!have_rms) {
             // every column has been consumed by now, so every column's sum of squares is in place
             float tot = 0.f;
-            for (int c = 0; c < nb; c++) tot += __uint_as_float(lds_read_u32(p_xq + (uint32_t)c * kRec + kRecSsq));
-            inv_rms = 1.0f / sqrtf(tot / (float)P.K + P.norm_eps);
+            for (int c = 0; c < nb; c++) tot += __uint_as_float(lds_read_u32(xq_abs + (uint32_t)c * kRec + kRecSsq));
+            inv_rms = 1.0f / sqrtf(tot / (float)Q.K + Q.norm_eps);
             have_rms = true;
           }
           sg *= inv_rms;
           su *= inv_rms;
         }
-        if (kg == 0 && j < P.rows && row < P.N) {
+        if (kg == 0 && j < rows && row < N) {
           float v;
-          if (p_dual) {
-            const float act = P.activation == DH_ACT_SILU ? act_silu(sg) : act_gelu(sg);
-            v = act * su * P.alpha;
-            if (P.activation == DH_ACT_SILU && P.clamp_max > 0.f) v = fminf(fmaxf(v, -P.clamp_max), P.clamp_max);
+          if (dual) {
+            const int activation = Q.activation;
+            const float clamp_max = Q.clamp_max;
+            const float act = activation == DH_ACT_SILU ? act_silu(sg) : act_gelu(sg);
+            v = act * su * Q.alpha;
+            if (activation == DH_ACT_SILU && clamp_max > 0.f) v = fminf(fmaxf(v, -clamp_max), clamp_max);
           } else {
-            v = sg * P.alpha;
+            v = sg * Q.alpha;
+            const float* const residual = Q.residual;
             // device-scope load: an earlier phase of this launch may have written the residual
-            if (P.residual) v += __hip_atomic_load(const_cast<float*>(P.residual) + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (residual) v += __hip_atomic_load(const_cast<float*>(residual) + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
-          __hip_atomic_store(P.C + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(Q.C + row, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           if (!last_phase) {
             v2u pr;
             pr.x = __float_as_uint(v);
@@ -628,11 +604,11 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
           }
         }
         // a later phase reads these outputs as its residual: they are in memory before this wave goes on
-        if (P.wait_stores) DH_WAIT_VM(0);
+        if (Q.wait_stores) DH_WAIT_VM(0);
         // slot free for the tile kSlots further on (after the reads above: same wave, in order)
         if (lane == 0) {
-          ctr[1 + slot] = 0u;
-          ctr[1 + kSlots + slot] = ((unsigned)tord >> kSlotShift) + 1u;
+          ctr[kCtrArrived + slot] = 0u;
+          ctr[kCtrGen + slot] = ((unsigned)tord >> kSlotShift) + 1u;
           unsigned was;
           asm volatile("ds_add_rtn_u32 %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=&v"(was) : "v"(ctr_abs + 4 * (kCtrDone + p)), "v"(1u) : "memory");
         }
@@ -640,7 +616,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
         if (last_phase && bid == 0 && tl == 0 && lane == 0) *a.epoch = (seq_base >> 3) + 1u;
       }
     }
+    prev_ntl = ntl;
+    tb += ntl;
   }
+#undef DH_DECODE
 }
 
 // ---- host side ----------------------------------------------------------------------------------
@@ -715,13 +694,13 @@ int make_plan(const char* op, const float* d_x0, const dh_chain_phase* ph, int n
     // a product may not overwrite what an earlier or later one of the launch still reads elsewhere
     if (s.d_C == d_x0) return dh::fail(1, "[%s] product %d writes over the chain's input", op, p);
   }
-  // the units in flight (16 waves x 3 draws) must not span more tiles than there are slots
-  if ((kWaves * (kDepth + 1) + min_upt - 1) / min_upt + 2 > kSlots)
-    return dh::fail(1, "[%s] K=%d is too short for a chain (at least 2048)", op, min_upt * kQK);
+  // the units in flight (16 waves x 2 draws) must not span more tiles than there are slots
+  if ((kWaves * 2 + min_upt - 1) / min_upt + 2 > kSlots)
+    return dh::fail(1, "[%s] K=%d is too short for a chain (at least 1536)", op, min_upt * kQK);
   a.xq_bytes[0] = a.nb_max[0] * kRec;
   a.xq_bytes[1] = a.nb_max[1] * kRec;
   a.red_stride = 16 * max_upt;
-  out->lds = (size_t)kWaves * kDepth * kStage + a.xq_bytes[0] + a.xq_bytes[1] + kZeroBytes +
+  out->lds = (size_t)kWaves * kStage + a.xq_bytes[0] + a.xq_bytes[1] + kZeroBytes +
              sizeof(float) * kSlots * a.red_stride + sizeof(unsigned) * (kCtrFlags + a.nb_max[0] + a.nb_max[1]) + kLdsPad;
   if (out->lds > kMaxLds)
     return dh::fail(1, "[%s] the chain's activations do not fit the LDS (%zu of %zu bytes)", op, out->lds, kMaxLds);
