@@ -63,19 +63,26 @@ __device__ __forceinline__ void i8_quantise_store(const float (&v)[4], unsigned 
   const uint32_t mb = max8_u32(max(max(ab[0], ab[1]), max(ab[2], ab[3])));
   const int ef = (int)(mb >> 23);
   const bool special = ef == 255;
-  const bool has_nan = mb > 0x7F800000u;
   const int ex = max(ef - 127, -107);                      // the sub-block's largest magnitude is below 2^(ex+1)
-  const float sf = special ? 1.0f : __uint_as_float((uint32_t)(127 + 19 - ex) << 23);     // |x| * sf < 2^20
-  const float xinv = special ? __uint_as_float(has_nan ? 0x7FC00000u : 0x7F800000u)
-                             : __uint_as_float((uint32_t)(127 - 19 + ex) << 23);
+  float sf = __uint_as_float((uint32_t)(127 + 19 - ex) << 23);       // |x| * sf < 2^20
+  float xinv = __uint_as_float((uint32_t)(127 - 19 + ex) << 23);
+  float q[4] = {v[0], v[1], v[2], v[3]};
+  // non-finite values are rare: their handling stays off the common path (one wave-uniform branch)
+  if (__builtin_amdgcn_ballot_w64(special) != 0ull) {
+    if (special) {
+      const bool has_nan = mb > 0x7F800000u;
+      sf = 1.0f;
+      xinv = __uint_as_float(has_nan ? 0x7FC00000u : 0x7F800000u);
+#pragma unroll
+      for (int e = 0; e < 4; e++) q[e] = (ab[e] == 0x7F800000u && !has_nan) ? copysignf(1.0f, v[e]) : 0.0f;
+    }
+  }
   // X = round(x * sf) sits in the low mantissa bits of x * sf + 1.5 * 2^23 (two's complement)
   uint32_t b[4], d2[4], d1[4], d0[4];
   uint32_t xs = 0u;
 #pragma unroll
   for (int e = 0; e < 4; e++) {
-    float q = v[e];
-    if (special) q = (ab[e] == 0x7F800000u && !has_nan) ? copysignf(1.0f, v[e]) : 0.0f;
-    b[e] = __float_as_uint(fmaf(q, sf, 12582912.0f));
+    b[e] = __float_as_uint(fmaf(q[e], sf, 12582912.0f));
     xs += b[e];
     d2[e] = (uint32_t)__builtin_amdgcn_sbfe((int)b[e], 0, 7);              // signed low 7 bits
     d1[e] = (uint32_t)__builtin_amdgcn_sbfe((int)(b[e] + 64u), 7, 7);
