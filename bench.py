@@ -227,8 +227,7 @@ def main():
     log("[bench] graph replay: %.1f tok/s" % graph_tok_s)
 
     # ---- side measurements (A/B, same positions rewritten): the captured step with its attention
-    #      nodes moved by the host before every replay instead of reading the key count on the device,
-    #      and the eager step with the four products between two attentions chained into one launch
+    #      nodes moved by the host before every replay instead of reading the key count on the device
     def timed_steps(fn, first_tok, n=24):
         t = first_tok
         for i in range(4):
@@ -243,15 +242,17 @@ def main():
     graph_patched_tok_s = timed_steps(dec.step_graph, tok)
     dec.release_graph()
     log("[bench] graph replay with host-patched attention nodes: %.1f tok/s" % graph_patched_tok_s)
-    chained_tok_s = None
-    try:
-        dec.chain_gemvs = True
-        chained_tok_s = timed_steps(dec.step, tok)
-        log("[bench] eager steps with chained GEMVs (one launch for o, gate/up, down, next qkv): %.1f tok/s" % chained_tok_s)
-    except Exception as e:      # a side measurement, never a reason to lose the result
-        log("[bench] chained-GEMV measurement failed: %r" % (e,))
-    finally:
-        dec.chain_gemvs = False
+    # ... and the eager step with every product its own launch (six per layer)
+    unchained_tok_s = None
+    if dec.chain_gemvs:
+        try:
+            dec.set_chain_gemvs(False)
+            unchained_tok_s = timed_steps(dec.step, tok)
+            log("[bench] eager steps with one launch per product (no chained GEMVs): %.1f tok/s" % unchained_tok_s)
+        except Exception as e:      # a side measurement, never a reason to lose the result
+            log("[bench] unchained measurement failed: %r" % (e,))
+        finally:
+            dec.set_chain_gemvs(True)
 
     # ---- roofline of the dominant kernel
     Hd, I = cfg["hidden"], cfg["inter"]
@@ -323,7 +324,8 @@ def main():
                    "batched_decode_16_per_submit_tokens_per_s": round(batched_tok_s, 2),
                    "graph_replay_tokens_per_s": round(graph_tok_s, 2),
                    "graph_replay_host_patched_tokens_per_s": round(graph_patched_tok_s, 2),
-                   "chained_gemv_tokens_per_s": round(chained_tok_s, 2) if chained_tok_s else None,
+                   "launches_per_layer": 2 if dec.chain_merges_attention else (3 if dec.chain_gemvs else 6),
+                   "unchained_tokens_per_s": round(unchained_tok_s, 2) if unchained_tok_s else None,
                    "js_host": js_host,
                    "prefill_tokens_per_s": round(prefill / prefill_s, 1)},
         "roofline": roofline,

@@ -32,6 +32,12 @@ class ChainPhase(ctypes.Structure):
                 ("alpha", _F), ("swiglu_limit", _F), ("norm_eps", _F)]
 
 
+class ChainAttnSource(ctypes.Structure):
+    """struct dh_chain_attn_source: the attention partial results a chain's first product merges."""
+    _fields_ = [("d_workspace", _P), ("H", _I), ("Hkv", _I), ("D", _I), ("nsplit", _I), ("d_kv_len", _P),
+                ("max_kv_len", _I), ("sliding_window", _I), ("kv_start", _I)]
+
+
 def chain_phases(phases):
     """list of dicts (W, W2, C, residual, norm_weight: device addresses or None; N, K; activation,
     norm_weight_offset, alpha, swiglu_limit, norm_eps) -> ctypes array of dh_chain_phase."""
@@ -76,6 +82,8 @@ SIGNATURES = {
     "dh_q4k_ffn_gate_up_rmsnorm": (_I, [_P, _P, _F, _I, _P, _P, _P, _I, _I, _I, _I, _F, _F]),
     "dh_q4k_gemv_chain": (_I, [_P, ctypes.POINTER(ChainPhase), _I]),
     "dh_q4k_gemv_chain_limited": (_I, [_P, ctypes.POINTER(ChainPhase), _I, _I, _I]),
+    "dh_q4k_gemv_chain_attn_supported": (_I, [_I, _I, _I, _I]),
+    "dh_q4k_gemv_chain_attn": (_I, [ctypes.POINTER(ChainAttnSource), ctypes.POINTER(ChainPhase), _I]),
     "dh_f16w_matmul": (_I, [_P, _P, _P, _I, _I, _I, _F]),
     "dh_lmhead_argmax_workspace_bytes": (_SZ, [_I]),
     "dh_lmhead_argmax_f16": (_I, [_P, _P, _I, _I, _I64, _F, _P, _P, _I, _P]),
@@ -90,6 +98,10 @@ SIGNATURES = {
     "dh_attn_decode_kvlen": (_I, [_P, _P, _P, _P, _I, _I, _I, _P, _I, _F, _I, _I, _F, _I, _I, _I, _P]),
     "dh_attn_decode_qkv_kvlen": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _F, _I, _I, _F, _F, _I,
                                       _I, _I, _P]),
+    "dh_attn_decode_qkv_partials": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _F, _I, _I,
+                                         _I, _P, ctypes.POINTER(_I)]),
+    "dh_attn_decode_qkv_kvlen_partials": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _F, _I, _I, _F, _F,
+                                               _I, _I, _I, _P]),
     "dh_rmsnorm": (_I, [_P, _P, _I, _P, _I, _I, _F, _I, _P, _P, _P, _F]),
     "dh_rmsnorm_sandwich_pair": (_I, [_P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _F, _I]),
     "dh_residual_rmsnorm_pair": (_I, [_P, _P, _P, _I, _P, _P, _I, _I, _F, _I, _F]),

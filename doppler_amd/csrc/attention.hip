@@ -20,60 +20,19 @@
 #include <type_traits>
 #include <cfloat>
 
+#include "attention_keys.h"
 #include "dh_common.h"
 
 namespace {
 
-constexpr int kTileKeys = 64;
+constexpr int kTileKeys = dh::kAttnTileKeys;
 constexpr int kMaxG = 8;       // query heads per kv head
 
-// What the kernels need to redo the host's key-range arithmetic from a key count in device memory.
-struct DynKeys {
-  const uint32_t* kv_len_ptr;   // null: everything comes in as launch arguments
-  int max_kv_len;               // the count is clamped to this (caches, tables and workspace are sized for it)
-  int causal, start_pos;        // start_pos < 0: the query sits at the last key, kv_start + kv_len - 1
-  int sliding_window, kv_start, qkv;
-  int one_per_cu;               // workgroups per kv head that fill the device once
-};
-struct KeyRange {
-  int kbeg, kend, nsplit, start_pos;
-};
-
-// Splits of the key range per kv head.  Fewer, longer workgroups beat more splits once every CU
-// has one: a workgroup's next chunk costs well under 1 us, every extra split costs the merge
-// kernel and the dispatch more (measured, 32/8 heads, four workgroups per CU against one:
-// 3000 keys 12.9 vs 10.4 us, 6000 keys 17.1 vs 12.6, 16384 keys 24.4 vs 20.4, 32768 keys 37.1 vs
-// 33.4).  One workgroup per CU, two once that would mean more than 16 chunks each.
-__host__ __device__ inline int splits_for(int one_per_cu, int nkeys) {
-  const int tiles = nkeys > 0 ? (nkeys + 63) / 64 : 1;
-  const int wgs = tiles <= 16 * one_per_cu ? one_per_cu : 2 * one_per_cu;
-  if (tiles <= wgs) return tiles;
-  // every workgroup the same number of chunks (the slowest one sets the time), in as few splits
-  // as that allows (the merge kernel pays per split)
-  const int chunks_each = (tiles + wgs - 1) / wgs;
-  return (tiles + chunks_each - 1) / chunks_each;
-}
-// The largest split count any key count up to max_keys can ask for: the grid of a launch whose key
-// count is only known on the device.
-__host__ __device__ inline int max_splits_upto(int one_per_cu, int max_keys) {
-  const int tiles = max_keys > 0 ? (max_keys + 63) / 64 : 1;
-  if (tiles <= one_per_cu) return tiles;
-  return tiles <= 16 * one_per_cu ? one_per_cu : 2 * one_per_cu;
-}
-// Visible key range [kbeg, kend) relative to kv_start, split count (0: no key is visible) and the
-// query's position for a key count read on the device.
-__device__ inline KeyRange dyn_key_range(const DynKeys& d) {
-  int kv_len = (int)*d.kv_len_ptr;
-  kv_len = kv_len < 0 ? 0 : (kv_len > d.max_kv_len ? d.max_kv_len : kv_len);
-  KeyRange r;
-  r.start_pos = d.start_pos < 0 ? d.kv_start + kv_len - 1 : d.start_pos;
-  r.kbeg = 0;
-  r.kend = kv_len;
-  if (!d.qkv && d.causal) r.kend = min(r.kend, r.start_pos - d.kv_start + 1);
-  if (d.sliding_window > 0 && r.start_pos >= d.sliding_window) r.kbeg = max(0, r.start_pos - d.sliding_window + 1 - d.kv_start);
-  r.nsplit = r.kend > r.kbeg ? splits_for(d.one_per_cu, r.kend - r.kbeg) : 0;
-  return r;
-}
+using dh::DynKeys;
+using dh::KeyRange;
+using dh::splits_for;
+using dh::max_splits_upto;
+using dh::dyn_key_range;
 
 struct AttnArgs {
   const float* Q;       // [H][D]
@@ -566,7 +525,7 @@ __global__ void zero_f32_kernel(float* p, int n) {
 
 int max_splits_for(int kv_len) { return std::max(1, (kv_len + kTileKeys - 1) / kTileKeys); }
 
-int one_per_cu_for(int Hkv) { return std::max(1, dh::num_cus() / std::max(1, Hkv)); }
+int one_per_cu_for(int Hkv) { return dh::attn_one_per_cu(dh::num_cus(), Hkv); }
 
 int choose_splits(int Hkv, int nkeys) {
   const int tiles = std::max(1, (nkeys + kTileKeys - 1) / kTileKeys);
@@ -592,10 +551,10 @@ SplitKernel split_kernel_for(int D, bool qkv, int G) {
 }
 MergeKernel merge_kernel_for(int D) { return D == 64 ? attn_decode_merge_kernel<64> : attn_decode_merge_kernel<128>; }
 
-int launch(const AttnArgs& a, int D, bool qkv, const char* op) {
+int launch(const AttnArgs& a, int D, bool qkv, const char* op, bool merge = true) {
   hipLaunchKernelGGL(split_kernel_for(D, qkv, a.G), dim3(a.Hkv, a.nsplit), dim3(256), 0, dh::stream(), a);
   DH_CHECK_LAUNCH(op);
-  if (!a.direct) {
+  if (!a.direct && merge) {
     hipLaunchKernelGGL(merge_kernel_for(D), dim3(a.H), dim3(D), 0, dh::stream(), a.ws, a.O, a.nsplit, a.dyn);
     DH_CHECK_LAUNCH(op);
   }
@@ -862,13 +821,15 @@ int dh_attn_decode_qkv_supported(int H, int Hkv, int D, int rotary_dim, int inte
   return (rotary_dim & (rotary_dim - 1)) == 0 && rotary_dim / 2 >= D / 32;
 }
 
-int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float* d_k_weight, const float* d_cos,
-                       const float* d_sin, void* d_cache_k, void* d_cache_v, float* d_O, int H, int Hkv, int D,
-                       int start_pos, int rotary_dim, int interleaved, float eps, int weight_offset, int use_norm,
-                       float scale, float softcap, int sliding_window, int kv_start, int kv_layout,
-                       void* d_workspace) {
-  const char* op = "dh_attn_decode_qkv";
+// Shared body of dh_attn_decode_qkv and dh_attn_decode_qkv_partials (out_nsplit != null: the splits'
+// partial results stay in the workspace, no merge launch, *out_nsplit receives their number).
+static int attn_decode_qkv_impl(const char* op, const float* d_qkv, const float* d_q_weight, const float* d_k_weight,
+                                const float* d_cos, const float* d_sin, void* d_cache_k, void* d_cache_v, float* d_O, int H,
+                                int Hkv, int D, int start_pos, int rotary_dim, int interleaved, float eps, int weight_offset,
+                                int use_norm, float scale, float softcap, int sliding_window, int kv_start, int kv_layout,
+                                void* d_workspace, int* out_nsplit) {
   DH_REQUIRE_INIT(op);
+  const bool partials = out_nsplit != nullptr;
   if (H <= 0 || Hkv <= 0 || D <= 0) return dh::fail(1, "[%s] numHeads/numKVHeads/headDim must be positive", op);
   if (H % Hkv) return dh::fail(1, "[%s] numHeads=%d must be a multiple of numKVHeads=%d", op, H, Hkv);
   if (!dh_attn_decode_qkv_supported(H, Hkv, D, rotary_dim, interleaved))
@@ -880,7 +841,7 @@ int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float*
     return dh::fail(1, "[%s] kvLayout %d not supported (contiguous, ring)", op, kv_layout);
   if (kv_layout == DH_KV_RING && sliding_window <= 0)
     return dh::fail(1, "[%s] ring layout needs slidingWindow > 0", op);
-  if (!d_qkv || !d_cos || !d_sin || !d_cache_k || !d_cache_v || !d_O) return dh::fail(1, "[%s] null pointer", op);
+  if (!d_qkv || !d_cos || !d_sin || !d_cache_k || !d_cache_v || (!d_O && !partials)) return dh::fail(1, "[%s] null pointer", op);
   if (use_norm && (!d_q_weight || !d_k_weight)) return dh::fail(1, "[%s] q/k norm weights are required", op);
   if ((reinterpret_cast<uintptr_t>(d_cache_k) | reinterpret_cast<uintptr_t>(d_cache_v) |
        reinterpret_cast<uintptr_t>(d_qkv) | reinterpret_cast<uintptr_t>(d_q_weight) |
@@ -894,11 +855,41 @@ int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float*
   c.eps = eps; c.scale = scale; c.softcap = softcap; c.sliding_window = sliding_window; c.kv_start = kv_start;
   c.kv_layout = kv_layout; c.ws = d_workspace;
   const bool capturing = dh::capturing_graph() != nullptr;
+  // (a consumer of the partial results is given the split count of THIS position: a replay at another
+  // position would need both patched, so the captured form is the one with the key count on the device)
+  if (partials && capturing)
+    return dh::fail(1, "[%s] not while a graph is being captured: use dh_attn_decode_qkv_kvlen_partials there", op);
   AttnArgs a;
-  if (build_args(c, 0, capturing, a)) return dh::fail(2, "[%s] internal: no visible key", op);
+  if (build_args(c, 0, capturing || partials, a)) return dh::fail(2, "[%s] internal: no visible key", op);
   if (!a.direct && !d_workspace) return dh::fail(1, "[%s] workspace is required", op);
+  if (partials) {
+    *out_nsplit = a.nsplit;
+    return launch(a, D, true, op, false);
+  }
   dh::graph_note_attention(c);
   return launch(a, D, true, op);
+}
+
+int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float* d_k_weight, const float* d_cos,
+                       const float* d_sin, void* d_cache_k, void* d_cache_v, float* d_O, int H, int Hkv, int D,
+                       int start_pos, int rotary_dim, int interleaved, float eps, int weight_offset, int use_norm,
+                       float scale, float softcap, int sliding_window, int kv_start, int kv_layout,
+                       void* d_workspace) {
+  return attn_decode_qkv_impl("dh_attn_decode_qkv", d_qkv, d_q_weight, d_k_weight, d_cos, d_sin, d_cache_k, d_cache_v, d_O, H,
+                              Hkv, D, start_pos, rotary_dim, interleaved, eps, weight_offset, use_norm, scale, softcap,
+                              sliding_window, kv_start, kv_layout, d_workspace, nullptr);
+}
+
+int dh_attn_decode_qkv_partials(const float* d_qkv, const float* d_q_weight, const float* d_k_weight, const float* d_cos,
+                                const float* d_sin, void* d_cache_k, void* d_cache_v, int H, int Hkv, int D, int start_pos,
+                                int rotary_dim, int interleaved, float eps, int weight_offset, int use_norm, float scale,
+                                float softcap, int sliding_window, int kv_start, int kv_layout, void* d_workspace,
+                                int* out_nsplit) {
+  const char* op = "dh_attn_decode_qkv_partials";
+  if (!out_nsplit) return dh::fail(1, "[%s] out_nsplit is null", op);
+  return attn_decode_qkv_impl(op, d_qkv, d_q_weight, d_k_weight, d_cos, d_sin, d_cache_k, d_cache_v, nullptr, H, Hkv, D,
+                              start_pos, rotary_dim, interleaved, eps, weight_offset, use_norm, scale, softcap,
+                              sliding_window, kv_start, kv_layout, d_workspace, out_nsplit);
 }
 
 // ---- key count on the device -------------------------------------------------------------------
@@ -906,7 +897,7 @@ int dh_attn_decode_qkv(const float* d_qkv, const float* d_q_weight, const float*
 // for max_kv_len keys (that fixes pointers, shapes and the grid), the kernels replace everything
 // that depends on the key count by what the device word says.
 static int attn_decode_kvlen_impl(const char* op, dh::GraphAttnCall c, const uint32_t* d_kv_len, int max_kv_len,
-                                  int start_pos) {
+                                  int start_pos, bool merge = true) {
   if (!d_kv_len) return dh::fail(1, "[%s] the key-count pointer is null", op);
   if (reinterpret_cast<uintptr_t>(d_kv_len) & 3) return dh::fail(1, "[%s] the key-count pointer must be 4-byte aligned", op);
   if (max_kv_len < 1) return dh::fail(1, "[%s] max_kv_len must be at least 1", op);
@@ -922,7 +913,7 @@ static int attn_decode_kvlen_impl(const char* op, dh::GraphAttnCall c, const uin
   a.nsplit = max_splits_upto(one_per_cu, max_kv_len);      // the grid; the kernels use the device word's split count
   a.direct = 0;
   // nothing is recorded for graph replays: a captured launch follows the device word by itself
-  return launch(a, c.D, c.qkv != 0, op);
+  return launch(a, c.D, c.qkv != 0, op, merge);
 }
 
 int dh_attn_decode_kvlen(const float* d_Q, const void* d_K, const void* d_V, float* d_O, int H, int Hkv, int D,
@@ -950,12 +941,12 @@ int dh_attn_decode_kvlen(const float* d_Q, const void* d_K, const void* d_V, flo
   return attn_decode_kvlen_impl(op, c, d_kv_len, max_kv_len, start_pos);
 }
 
-int dh_attn_decode_qkv_kvlen(const float* d_qkv, const float* d_q_weight, const float* d_k_weight, const float* d_cos,
-                             const float* d_sin, void* d_cache_k, void* d_cache_v, float* d_O, int H, int Hkv, int D,
-                             const uint32_t* d_kv_len, int max_kv_len, int rotary_dim, int interleaved, float eps,
-                             int weight_offset, int use_norm, float scale, float softcap, int sliding_window,
-                             int kv_start, int kv_layout, void* d_workspace) {
-  const char* op = "dh_attn_decode_qkv_kvlen";
+static int attn_decode_qkv_kvlen_impl(const char* op, bool partials, const float* d_qkv, const float* d_q_weight,
+                                      const float* d_k_weight, const float* d_cos, const float* d_sin, void* d_cache_k,
+                                      void* d_cache_v, float* d_O, int H, int Hkv, int D, const uint32_t* d_kv_len,
+                                      int max_kv_len, int rotary_dim, int interleaved, float eps, int weight_offset,
+                                      int use_norm, float scale, float softcap, int sliding_window, int kv_start,
+                                      int kv_layout, void* d_workspace) {
   DH_REQUIRE_INIT(op);
   if (H <= 0 || Hkv <= 0 || D <= 0) return dh::fail(1, "[%s] numHeads/numKVHeads/headDim must be positive", op);
   if (H % Hkv) return dh::fail(1, "[%s] numHeads=%d must be a multiple of numKVHeads=%d", op, H, Hkv);
@@ -966,7 +957,7 @@ int dh_attn_decode_qkv_kvlen(const float* d_qkv, const float* d_q_weight, const 
   if (kv_layout != DH_KV_CONTIGUOUS && kv_layout != DH_KV_RING)
     return dh::fail(1, "[%s] kvLayout %d not supported (contiguous, ring)", op, kv_layout);
   if (kv_layout == DH_KV_RING && sliding_window <= 0) return dh::fail(1, "[%s] ring layout needs slidingWindow > 0", op);
-  if (!d_qkv || !d_cos || !d_sin || !d_cache_k || !d_cache_v || !d_O) return dh::fail(1, "[%s] null pointer", op);
+  if (!d_qkv || !d_cos || !d_sin || !d_cache_k || !d_cache_v || (!d_O && !partials)) return dh::fail(1, "[%s] null pointer", op);
   if (use_norm && (!d_q_weight || !d_k_weight)) return dh::fail(1, "[%s] q/k norm weights are required", op);
   if ((reinterpret_cast<uintptr_t>(d_cache_k) | reinterpret_cast<uintptr_t>(d_cache_v) |
        reinterpret_cast<uintptr_t>(d_qkv) | reinterpret_cast<uintptr_t>(d_q_weight) |
@@ -979,7 +970,28 @@ int dh_attn_decode_qkv_kvlen(const float* d_qkv, const float* d_q_weight, const 
   c.rotary_dim = rotary_dim; c.interleaved = interleaved; c.weight_offset = weight_offset; c.use_norm = use_norm;
   c.eps = eps; c.scale = scale; c.softcap = softcap; c.sliding_window = sliding_window; c.kv_start = kv_start;
   c.kv_layout = kv_layout; c.ws = d_workspace;
-  return attn_decode_kvlen_impl(op, c, d_kv_len, max_kv_len, -1);
+  return attn_decode_kvlen_impl(op, c, d_kv_len, max_kv_len, -1, !partials);
+}
+
+int dh_attn_decode_qkv_kvlen(const float* d_qkv, const float* d_q_weight, const float* d_k_weight, const float* d_cos,
+                             const float* d_sin, void* d_cache_k, void* d_cache_v, float* d_O, int H, int Hkv, int D,
+                             const uint32_t* d_kv_len, int max_kv_len, int rotary_dim, int interleaved, float eps,
+                             int weight_offset, int use_norm, float scale, float softcap, int sliding_window,
+                             int kv_start, int kv_layout, void* d_workspace) {
+  return attn_decode_qkv_kvlen_impl("dh_attn_decode_qkv_kvlen", false, d_qkv, d_q_weight, d_k_weight, d_cos, d_sin, d_cache_k,
+                                    d_cache_v, d_O, H, Hkv, D, d_kv_len, max_kv_len, rotary_dim, interleaved, eps,
+                                    weight_offset, use_norm, scale, softcap, sliding_window, kv_start, kv_layout, d_workspace);
+}
+
+int dh_attn_decode_qkv_kvlen_partials(const float* d_qkv, const float* d_q_weight, const float* d_k_weight,
+                                      const float* d_cos, const float* d_sin, void* d_cache_k, void* d_cache_v, int H,
+                                      int Hkv, int D, const uint32_t* d_kv_len, int max_kv_len, int rotary_dim,
+                                      int interleaved, float eps, int weight_offset, int use_norm, float scale,
+                                      float softcap, int sliding_window, int kv_start, int kv_layout, void* d_workspace) {
+  return attn_decode_qkv_kvlen_impl("dh_attn_decode_qkv_kvlen_partials", true, d_qkv, d_q_weight, d_k_weight, d_cos, d_sin,
+                                    d_cache_k, d_cache_v, nullptr, H, Hkv, D, d_kv_len, max_kv_len, rotary_dim, interleaved,
+                                    eps, weight_offset, use_norm, scale, softcap, sliding_window, kv_start, kv_layout,
+                                    d_workspace);
 }
 
 }  // extern "C"

@@ -33,9 +33,11 @@
 // The arithmetic of a unit (int8 matrix cores over activations quantised per 32-element sub-block)
 // is that of q4k_gemv_i8.hip; the two share q4k_i8_device.h.
 #include <algorithm>
+#include <cfloat>
 #include <cstdlib>
 #include <cstring>
 
+#include "attention_keys.h"
 #include "dh_common.h"
 #include "q4k_device.h"
 #include "q4k_i8_device.h"
@@ -119,7 +121,24 @@ struct ChainArgs {
   int xq_bytes[2];             // bytes of the two record areas (phases 0, 2 / 1, 3)
   int nb_max[2];               // columns of the two areas
   int red_stride;              // floats per tile slot: 16 * the largest units-per-tile
+  // phase 0's input as the split-K partial results of a decode attention (null: x0): [H][nsplit][D + 2]
+  // (o..., m, l) per query head and split; the split count is attn_nsplit, or follows the key count
+  // on the device as the attention kernels' own does
+  const float* attn_ws;
+  int attn_H, attn_D, attn_nsplit;
+  dh::DynKeys attn_dyn;
 };
+
+__device__ __forceinline__ float wave_max64(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum64(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
 
 __device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
   uint32_t v;
@@ -241,12 +260,96 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
 
   // the first pass of phase 0: its loads go out before the barrier and before any weights, so that
   // they are at the head of the compute unit's memory queue
+  const bool from_attn = a.attn_ws != nullptr;
   Cols first;
-  load_norm(a.ph[0].norm_weight, a.ph[0].nb, c_first, first);
-  load_x0(a.ph[0].nb, c_first, first);
+  // Phase 0's input from a decode attention's split-K partial results: the first wave of workgroup h
+  // merges query head h (out[d] = sum_s e^{m_s - M} o_s[d] / sum_s e^{m_s - M} l_s, the arithmetic and
+  // summation order of the attention's own merge kernel) and publishes it as phase "-1" of the
+  // exchange; every workgroup then takes phase 0's input from there as it takes a later phase's.
+  // Everything the merge reads (of the first 32 splits) is requested here, before the barrier: one
+  // trip to memory.  Lane s holds (m, l) of split s, lane t the output dims 2t, 2t + 1.
+  constexpr int kMergePre = 32;
+  const bool merger = from_attn && wave == 0 && bid < a.attn_H;
+  int m_nsplit = 0;
+  const float* m_base = nullptr;
+  v2f m_ml = {-FLT_MAX, 0.f};
+  v2f m_ov[kMergePre];
+  if (merger) {
+    m_nsplit = a.attn_nsplit;
+    if (a.attn_dyn.kv_len_ptr != nullptr) m_nsplit = dh::dyn_key_range(a.attn_dyn).nsplit;
+    m_nsplit = __builtin_amdgcn_readfirstlane(m_nsplit);
+    m_base = a.attn_ws + (int64_t)bid * m_nsplit * (a.attn_D + 2);
+    if (lane < m_nsplit) {
+      const float* q = m_base + (int64_t)lane * (a.attn_D + 2) + a.attn_D;
+      asm volatile("global_load_dwordx2 %0, %1, off" : "=&v"(m_ml) : "v"(q) : "memory");
+    }
+    if (2 * lane < a.attn_D && m_nsplit > 0) {
+#pragma unroll
+      for (int i = 0; i < kMergePre; i++) {
+        const float* q = m_base + (int64_t)min(i, m_nsplit - 1) * (a.attn_D + 2) + 2 * lane;
+        asm volatile("global_load_dwordx2 %0, %1, off" : "=&v"(m_ov[i]) : "v"(q) : "memory");
+      }
+    }
+  }
+  if (!from_attn) {
+    load_norm(a.ph[0].norm_weight, a.ph[0].nb, c_first, first);
+    load_x0(a.ph[0].nb, c_first, first);
+  }
 
   // counters, flags and the zero area are in place
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+  if (from_attn) {
+    DH_WAIT_VM(0);
+    asm volatile("" : "+v"(epoch_v));
+    seq_base = __builtin_amdgcn_readfirstlane(epoch_v) * 8u;
+    if (merger) {
+      const int AD = a.attn_D;
+      asm volatile("" : "+v"(m_ml));
+      const bool has = lane < m_nsplit;
+      const float m0 = has ? m_ml[0] : -FLT_MAX, l0 = has ? m_ml[1] : 0.f;
+      const float M = wave_max64(m0);
+      const float f = has ? __expf(m0 - M) : 0.f;
+      const float den = wave_sum64(has ? f * l0 : 0.f);
+      const bool dims = 2 * lane < AD;
+      float n0 = 0.f, n1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < kMergePre; i++) {
+        asm volatile("" : "+v"(m_ov[i]));
+        if (i < m_nsplit) {
+          const float fs = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), i));
+          n0 = fmaf(fs, m_ov[i][0], n0);
+          n1 = fmaf(fs, m_ov[i][1], n1);
+        }
+      }
+#pragma unroll 1
+      for (int s0 = kMergePre; s0 < m_nsplit; s0 += 16) {
+        float2 ov[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          const int sidx = min(s0 + i, m_nsplit - 1);
+          ov[i] = dims ? *reinterpret_cast<const float2*>(m_base + (int64_t)sidx * (AD + 2) + 2 * lane) : make_float2(0.f, 0.f);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+          if (s0 + i < m_nsplit) {
+            const float fs = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), s0 + i));
+            n0 = fmaf(fs, ov[i].x, n0);
+            n1 = fmaf(fs, ov[i].y, n1);
+          }
+        }
+      }
+      if (dims) {
+        v2u p0, p1;
+        p0.x = __float_as_uint(den > 0.f ? n0 / den : 0.f);
+        p1.x = __float_as_uint(den > 0.f ? n1 / den : 0.f);
+        p0.y = p1.y = seq_base;
+        v2u* dst = a.ll + (size_t)kMaxChainN + (size_t)bid * AD + 2 * lane;
+        asm volatile("global_store_dwordx2 %0, %1, off sc1\n\tglobal_store_dwordx2 %0, %2, off offset:8 sc1"
+                     :: "v"(dst), "v"(p0), "v"(p1) : "memory");
+      }
+    }
+  }
 
   // operand addressing (see q4k_gemv_i8.hip): MFMA pair cc covers sub-blocks 4cc .. 4cc+3; lane
   // (i = lane & 15, kg) supplies operand row i = 4g + digit: 16 digit bytes where its row's sub-block is
@@ -316,8 +419,8 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
 
   // ---- phase 0's activations come from x0: the wave's first unit (unit `wave`, no draw) is requested
   // behind their loads, and only they are waited for
-  int cur;                                  // the unit in the ring (>= its phase's total: none)
-  {
+  int cur = 0x7fffffff;                     // the unit in the ring (>= its phase's total: none)
+  if (!from_attn) {
     const Phase& Q = a.ph[0];
     const Stream S = stream_of(Q);
     const int total = (Q.tiles_base + (bid < Q.tiles_rem ? 1 : 0)) * Q.upt;
@@ -362,7 +465,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
     const uint32_t flag_want = (uint32_t)p + 1u;
     const bool last_phase = p == nph - 1;
 
-    if (p > 0) {
+    if (p > 0 || from_attn) {
       // ---- the wave's first unit of the phase: unit `wave`, no draw
       cur = wave < total ? wave : 0x7fffffff;
       if (cur < total) issue(S, cur);
@@ -374,7 +477,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
       // Not before this workgroup has finished its own tiles of the previous phase: the workgroups run
       // the same work at the same pace, so until then the others have not finished theirs either, and
       // polls that cannot succeed yet would only compete with the weight stream for the memory system.
-      {
+      if (p > 0) {
         const uint32_t done_addr = ctr_abs + 4 * (kCtrDone + p - 1);
         int spins = 0;
         while (__builtin_amdgcn_readfirstlane(lds_read_u32(done_addr)) < (unsigned)prev_ntl) {
@@ -632,9 +735,9 @@ struct Plan {
   size_t lds;
 };
 
-int make_plan(const char* op, const float* d_x0, const dh_chain_phase* ph, int n, Plan* out) {
+int make_plan(const char* op, const float* d_x0, const dh_chain_attn_source* src, const dh_chain_phase* ph, int n, Plan* out) {
   if (n < 1 || n > kMaxPhases) return dh::fail(1, "[%s] a chain holds 1..%d products, got %d", op, kMaxPhases, n);
-  if (!d_x0 || !ph) return dh::fail(1, "[%s] null pointer", op);
+  if ((!d_x0 && !src) || !ph) return dh::fail(1, "[%s] null pointer", op);
   if (reinterpret_cast<uintptr_t>(d_x0) & 15) return dh::fail(1, "[%s] x0 must be 16-byte aligned", op);
   ChainArgs& a = out->a;
   memset(&a, 0, sizeof(a));
@@ -692,11 +795,40 @@ int make_plan(const char* op, const float* d_x0, const dh_chain_phase* ph, int n
     for (int q = p + 1; q < n; q++)
       if (ph[q].d_residual == s.d_C) P.wait_stores = 1;
     // a product may not overwrite what an earlier or later one of the launch still reads elsewhere
-    if (s.d_C == d_x0) return dh::fail(1, "[%s] product %d writes over the chain's input", op, p);
+    if (d_x0 && s.d_C == d_x0) return dh::fail(1, "[%s] product %d writes over the chain's input", op, p);
   }
   // the units in flight (16 waves x 2 draws) must not span more tiles than there are slots
   if ((kWaves * 2 + min_upt - 1) / min_upt + 2 > kSlots)
     return dh::fail(1, "[%s] K=%d is too short for a chain (at least 1536)", op, min_upt * kQK);
+  if (src) {
+    // the first product's input is the merge of a decode attention's split-K partial results
+    const int ncus = dh::num_cus();
+    if (!src->d_workspace) return dh::fail(1, "[%s] the attention workspace is null", op);
+    if (reinterpret_cast<uintptr_t>(src->d_workspace) & 7) return dh::fail(1, "[%s] the attention workspace must be 8-byte aligned", op);
+    if (src->H <= 0 || src->Hkv <= 0 || src->H % src->Hkv) return dh::fail(1, "[%s] attention heads %d/%d", op, src->H, src->Hkv);
+    if (src->D != 64 && src->D != 128) return dh::fail(1, "[%s] headDim %d not supported (64, 128)", op, src->D);
+    if (src->H * src->D != ph[0].K)
+      return dh::fail(1, "[%s] the attention makes %d x %d values but product 0 takes K=%d", op, src->H, src->D, ph[0].K);
+    if (src->H > ncus) return dh::fail(1, "[%s] %d query heads need as many workgroups (%d)", op, src->H, ncus);
+    const int one_per_cu = dh::attn_one_per_cu(ncus, src->Hkv);
+    int max_splits;
+    if (src->d_kv_len) {
+      if (reinterpret_cast<uintptr_t>(src->d_kv_len) & 3) return dh::fail(1, "[%s] the key-count pointer must be 4-byte aligned", op);
+      if (src->max_kv_len < 1 || src->sliding_window < 0 || src->kv_start < 0)
+        return dh::fail(1, "[%s] need max_kv_len >= 1, slidingWindow >= 0, kvStart >= 0", op);
+      max_splits = dh::max_splits_upto(one_per_cu, src->max_kv_len);
+      // the arithmetic of dh_attn_decode_qkv_kvlen_partials: causal, the query at the last key
+      a.attn_dyn = dh::DynKeys{src->d_kv_len, src->max_kv_len, 1, -1, src->sliding_window, src->kv_start, 1, one_per_cu};
+    } else {
+      if (src->nsplit < 1) return dh::fail(1, "[%s] nsplit must be at least 1", op);
+      max_splits = src->nsplit;
+    }
+    if (max_splits > 64) return dh::fail(1, "[%s] up to 64 splits are merged in the chain (this call may have %d)", op, max_splits);
+    a.attn_ws = static_cast<const float*>(src->d_workspace);
+    a.attn_H = src->H;
+    a.attn_D = src->D;
+    a.attn_nsplit = src->nsplit;
+  }
   a.xq_bytes[0] = a.nb_max[0] * kRec;
   a.xq_bytes[1] = a.nb_max[1] * kRec;
   a.red_stride = 16 * max_upt;
@@ -765,7 +897,23 @@ int dh_q4k_gemv_chain(const float* d_x0, const dh_chain_phase* phases, int n_pha
   const char* op = "dh_q4k_gemv_chain";
   DH_REQUIRE_INIT(op);
   Plan plan;
-  if (int rc = make_plan(op, d_x0, phases, n_phases, &plan)) return rc;
+  if (!d_x0) return dh::fail(1, "[%s] null pointer", op);
+  if (int rc = make_plan(op, d_x0, nullptr, phases, n_phases, &plan)) return rc;
+  return launch(op, plan, plan.a.grid);
+}
+
+int dh_q4k_gemv_chain_attn_supported(int H, int Hkv, int D, int max_kv_len) {
+  if (!dh::ready() || H <= 0 || Hkv <= 0 || H % Hkv || (D != 64 && D != 128) || max_kv_len < 1) return 0;
+  const int ncus = dh::num_cus();
+  return H <= ncus && dh::max_splits_upto(dh::attn_one_per_cu(ncus, Hkv), max_kv_len) <= 64 ? 1 : 0;
+}
+
+int dh_q4k_gemv_chain_attn(const dh_chain_attn_source* source, const dh_chain_phase* phases, int n_phases) {
+  const char* op = "dh_q4k_gemv_chain_attn";
+  DH_REQUIRE_INIT(op);
+  if (!source) return dh::fail(1, "[%s] null pointer", op);
+  Plan plan;
+  if (int rc = make_plan(op, nullptr, source, phases, n_phases, &plan)) return rc;
   return launch(op, plan, plan.a.grid);
 }
 
@@ -774,7 +922,8 @@ int dh_q4k_gemv_chain_limited(const float* d_x0, const dh_chain_phase* phases, i
   const char* op = "dh_q4k_gemv_chain_limited";
   DH_REQUIRE_INIT(op);
   Plan plan;
-  if (int rc = make_plan(op, d_x0, phases, n_phases, &plan)) return rc;
+  if (!d_x0) return dh::fail(1, "[%s] null pointer", op);
+  if (int rc = make_plan(op, d_x0, nullptr, phases, n_phases, &plan)) return rc;
   if (workgroups < 1 || workgroups > plan.a.grid)
     return dh::fail(1, "[%s] workgroups must be 1..%d", op, plan.a.grid);
   if (spin_limit < 1 || spin_limit > kDefaultSpinLimit) return dh::fail(1, "[%s] spin_limit must be 1..%d", op, kDefaultSpinLimit);

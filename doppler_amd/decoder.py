@@ -43,24 +43,19 @@ class HipDecoder:
     TOKEN_RING = 64      # tokens one decode_batch submit can produce
 
     def __init__(self, cfg, layers, embed_bits, final_norm, cos, sin, max_seq, fuse_norm=True,
-                 fuse_qkv_attention=True, finiteness_guard=False, finiteness_abs_threshold=None, chain_gemvs=False):
+                 fuse_qkv_attention=True, finiteness_guard=False, finiteness_abs_threshold=None, chain_gemvs=None,
+                 chain_merge_attention=True):
         """cfg: dict(layers, hidden, inter, heads, kv_heads, head_dim, vocab, eps, qk_norm);
         layers: list of dicts of numpy arrays (wq, wk, wv, wo, wgate, wup, wdown: Q4_K bytes;
         input_norm, post_attn_norm, q_norm, k_norm: f32); embed_bits: uint16 [vocab, hidden].
         finiteness_guard: check every layer's output against the overflow bound (one more launch
         per layer) and read the 4-word status back beside the token, as the reference does when
         activations are f16 (src/inference/pipelines/text/layer.js:1237-1252,
-        generator-steps.js:786-798, :837-843); off by default, the activations here are f32."""
+        generator-steps.js:786-798, :837-843); off by default, the activations here are f32.
+        chain_gemvs: see set_chain_gemvs; None (default) turns it on where it is served."""
         self.cfg = dict(cfg)
-        # chain_gemvs: the four products between two attentions (o, gate/up, down, next q/k/v) as one
-        # dh_q4k_gemv_chain launch.  Same bits as the separate launches; measured slower on the 9B-class
-        # shapes (the exchange between the products costs what the launches cost), so off by default.
-        self.chain_gemvs = bool(chain_gemvs)
-        if self.chain_gemvs:
-            dims = (cfg["hidden"], cfg["inter"], cfg["heads"] * cfg["head_dim"])
-            if any(k % 256 or k < 2048 or k > 32768 for k in dims) or not fuse_norm or finiteness_guard:
-                raise ValueError("chain_gemvs serves hidden, FFN and attention widths that are multiples of 256 in "
-                                 "2048..32768, with the norms fused and the finiteness guard off (got %s)" % (dims,))
+        self.chain_gemvs = False
+        self.chain_merges_attention = False
         self.finiteness_guard = bool(finiteness_guard)
         self.finiteness_abs_threshold = float(finiteness_abs_threshold) if finiteness_abs_threshold else 65500.0
         # RMSNorm runs inside the q/k/v and gate/up GEMVs (their prologue) unless told otherwise
@@ -73,6 +68,9 @@ class HipDecoder:
             c["heads"], c["kv_heads"], c["head_dim"], c["head_dim"], 0))
         self.max_seq = max_seq
         H, Hkv, D, Hd, I = c["heads"], c["kv_heads"], c["head_dim"], c["hidden"], c["inter"]
+        if chain_gemvs is None:
+            chain_gemvs = self.chain_gemvs_served()
+        self.set_chain_gemvs(chain_gemvs, chain_merge_attention)
         self.qs, self.ks = H * D, Hkv * D
         self.layers = []
         for l in layers:
@@ -114,6 +112,30 @@ class HipDecoder:
         self._host_token = np.zeros(1, np.uint32)
         self._host_ids = np.zeros(2, np.uint32)
         torch.cuda.synchronize()
+
+    def chain_gemvs_served(self):
+        """Whether set_chain_gemvs(True) accepts this model: hidden, FFN and attention widths that are
+        multiples of 256 in 2048..32768, norms fused, finiteness guard off."""
+        c = self.cfg
+        dims = (c["hidden"], c["inter"], c["heads"] * c["head_dim"])
+        return bool(all(k % 256 == 0 and 2048 <= k <= 32768 for k in dims) and self.fuse_norm and not self.finiteness_guard)
+
+    def set_chain_gemvs(self, on, merge_attention=True):
+        """on: the four products between two attentions (o, gate/up, down, next q/k/v) go out as one
+        dh_q4k_gemv_chain launch (same bits as the separate launches).  merge_attention: the chain's first
+        product also merges the attention's key splits itself, from the partial results the attention
+        leaves in its workspace (dh_q4k_gemv_chain_attn: two launches per layer instead of six), where
+        the fused attention serves the head geometry and its splits fit."""
+        c = self.cfg
+        if on and not self.chain_gemvs_served():
+            raise ValueError("chain_gemvs serves hidden, FFN and attention widths that are multiples of 256 in "
+                             "2048..32768, with the norms fused and the finiteness guard off (got %s)"
+                             % ((c["hidden"], c["inter"], c["heads"] * c["head_dim"]),))
+        self.chain_gemvs = bool(on)
+        self.chain_merges_attention = bool(on and merge_attention and self.fuse_qkv_attention and
+                                           self.L.dh_q4k_gemv_chain_attn_supported(c["heads"], c["kv_heads"], c["head_dim"],
+                                                                                   self.max_seq))
+        self._chains = {}
 
     def weight_bytes_per_token(self, ctx):
         """Algorithmic HBM bytes one decode step must read: all Q4_K weights, the f16 LM head
@@ -189,8 +211,6 @@ class HipDecoder:
     def _chain_phases(self, li):
         """o-projection, gate/up, down-projection of layer li and the q/k/v projection of layer li + 1 as
         the products of one dh_q4k_gemv_chain launch (built once per layer and kept)."""
-        if not hasattr(self, "_chains"):
-            self._chains = {}
         if li not in self._chains:
             c, d = self.cfg, self.layers[li]
             Hd, I = c["hidden"], c["inter"]
@@ -207,13 +227,37 @@ class HipDecoder:
 
     def _enqueue_layers_chained(self, pos, device_kv_len):
         L, c, ck = self.L, self.cfg, capi.check
+        H, Hkv, D = c["heads"], c["kv_heads"], c["head_dim"]
+        use_norm = int(c.get("qk_norm", 1))
         d0 = self.layers[0]
         ck(L.dh_q4k_matmul_rmsnorm(self.x.data_ptr(), d0["input_norm"].data_ptr(), c["eps"], 0, d0["wqkv"].data_ptr(),
                                    self.qkv.data_ptr(), capi.F32, 1, self.qs + 2 * self.ks, c["hidden"], 1.0, None))
         for li, d in enumerate(self.layers):
-            self._enqueue_attention(d, pos, device_kv_len)
             arr, n = self._chain_phases(li)
-            ck(L.dh_q4k_gemv_chain(self.attn.data_ptr(), arr, n))
+            # (a captured step with the position in the launch arguments keeps the attention's own merge:
+            # the library moves that launch with the position, a split count handed to the chain it could not)
+            if not self.chain_merges_attention or (getattr(self, "_capturing", False) and not device_kv_len):
+                self._enqueue_attention(d, pos, device_kv_len)
+                ck(L.dh_q4k_gemv_chain(self.attn.data_ptr(), arr, n))
+                continue
+            # the key splits' partial results stay in the workspace; the chain's first waves merge them
+            src = capi.ChainAttnSource(self.attn_ws.data_ptr(), H, Hkv, D, 0, None, 0, 0, 0)
+            if device_kv_len:
+                ck(L.dh_attn_decode_qkv_kvlen_partials(
+                    self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(), self.cos.data_ptr(),
+                    self.sin.data_ptr(), d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), H, Hkv, D,
+                    self.ids.data_ptr() + 4, self.max_seq, D, 0, c["eps"], 0, use_norm, self.scale, 0.0, 0, 0,
+                    capi.KV_CONTIGUOUS, self.attn_ws.data_ptr()))
+                src.d_kv_len = self.ids.data_ptr() + 4
+                src.max_kv_len = self.max_seq
+            else:
+                nsplit = ctypes.c_int(0)
+                ck(L.dh_attn_decode_qkv_partials(
+                    self.qkv.data_ptr(), d["q_norm"].data_ptr(), d["k_norm"].data_ptr(), self.cos.data_ptr(),
+                    self.sin.data_ptr(), d["cache_k"].data_ptr(), d["cache_v"].data_ptr(), H, Hkv, D, pos, D, 0, c["eps"],
+                    0, use_norm, self.scale, 0.0, 0, 0, capi.KV_CONTIGUOUS, self.attn_ws.data_ptr(), ctypes.byref(nsplit)))
+                src.nsplit = nsplit.value
+            ck(L.dh_q4k_gemv_chain_attn(ctypes.byref(src), arr, n))
 
     def _enqueue_attention(self, d, pos, device_kv_len=False):
         """self.qkv (raw stacked projection of the step's token) -> self.attn, appending the
@@ -302,6 +346,7 @@ class HipDecoder:
         self._graph_device_kv_len = bool(device_kv_len)
         capi.check(self.L.dh_graph_begin())
         g = ctypes.c_void_p()
+        self._capturing = True
         try:
             if self.finiteness_guard:
                 self._reset_finiteness()
@@ -311,6 +356,8 @@ class HipDecoder:
             if self.L.dh_graph_end(pos, ctypes.byref(g)) == 0 and g.value:
                 self.L.dh_graph_destroy(g)
             raise
+        finally:
+            self._capturing = False
         capi.check(self.L.dh_graph_end(pos, ctypes.byref(g)))
         capi.check(self.L.dh_graph_set_max_position(g, self.max_seq - 1))
         self._graph = g

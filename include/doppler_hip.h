@@ -206,6 +206,24 @@ int dh_q4k_gemv_chain(const float* d_x0, const dh_chain_phase* phases, int n_pha
  * reference. */
 int dh_q4k_gemv_chain_limited(const float* d_x0, const dh_chain_phase* phases, int n_phases,
                               int workgroups, int spin_limit);
+/* dh_q4k_gemv_chain whose first product reads the attention output of the step: the merge of the
+ * split-K partial results that dh_attn_decode_qkv_partials / dh_attn_decode_qkv_kvlen_partials left
+ * in their workspace (the arithmetic of the attention's own merge, same bits), done inside the
+ * launch by one wave per query head and handed to every workgroup through the chain's exchange.
+ * H * D must be the first product's K; at most 64 key splits.  d_kv_len NULL: nsplit is the count
+ * dh_attn_decode_qkv_partials returned; else the key count is read on the device and max_kv_len,
+ * sliding_window and kv_start are those given to dh_attn_decode_qkv_kvlen_partials. */
+typedef struct dh_chain_attn_source {
+  const void* d_workspace;
+  int H, Hkv, D;
+  int nsplit;
+  const uint32_t* d_kv_len;
+  int max_kv_len, sliding_window, kv_start;
+} dh_chain_attn_source;
+int dh_q4k_gemv_chain_attn(const dh_chain_attn_source* source, const dh_chain_phase* phases, int n_phases);
+/* 1 when dh_q4k_gemv_chain_attn serves this head geometry for key counts up to max_kv_len on the
+ * current device (after dh_init), else 0. */
+int dh_q4k_gemv_chain_attn_supported(int H, int Hkv, int D, int max_kv_len);
 
 /* ---- dense f16-weight GEMV (LM head) ----
  * C[M,N] = alpha * A[M,K] . f32(W[N,K])^T, W row-major f16.  Replaces the f16-weight branch
@@ -295,6 +313,26 @@ int dh_attn_decode_qkv_kvlen(const float* d_qkv, const float* d_q_weight, const 
                              int max_kv_len, int rotary_dim, int interleaved, float eps,
                              int weight_offset, int use_norm, float scale, float softcap,
                              int sliding_window, int kv_start, int kv_layout, void* d_workspace);
+/* dh_attn_decode_qkv / dh_attn_decode_qkv_kvlen without the merge of the key splits: the splits'
+ * partial results stay in the workspace, [H][nsplit][D + 2] floats (unnormalised output, running
+ * maximum, running sum per query head and split), for a consumer that merges them itself
+ * (dh_q4k_gemv_chain_attn: the reference's single attention dispatch,
+ * src/gpu/kernels/attention_decode_online_f16kv.wgsl:84-243, followed by its o-projection,
+ * src/inference/pipelines/text/attention/interpreter.js:1121-1160, with the launch between them removed).
+ * dh_attn_decode_qkv_partials hands back the split count of this position (not while a graph is
+ * being captured); with the key count on the device the consumer derives it from the same word. */
+int dh_attn_decode_qkv_partials(const float* d_qkv, const float* d_q_weight, const float* d_k_weight,
+                                const float* d_cos, const float* d_sin, void* d_cache_k, void* d_cache_v,
+                                int H, int Hkv, int D, int start_pos, int rotary_dim, int interleaved,
+                                float eps, int weight_offset, int use_norm, float scale, float softcap,
+                                int sliding_window, int kv_start, int kv_layout, void* d_workspace,
+                                int* out_nsplit);
+int dh_attn_decode_qkv_kvlen_partials(const float* d_qkv, const float* d_q_weight, const float* d_k_weight,
+                                      const float* d_cos, const float* d_sin, void* d_cache_k,
+                                      void* d_cache_v, int H, int Hkv, int D, const uint32_t* d_kv_len,
+                                      int max_kv_len, int rotary_dim, int interleaved, float eps,
+                                      int weight_offset, int use_norm, float scale, float softcap,
+                                      int sliding_window, int kv_start, int kv_layout, void* d_workspace);
 
 /* ---- normalisation / rotary / KV ---- */
 

@@ -210,3 +210,107 @@ def test_chain_argument_errors():
     fails(short, 1, "too short for a chain")
     with pytest.raises(DopplerHipError, match="workgroups must be"):
         capi.check(L.dh_q4k_gemv_chain_limited(x0, capi.chain_phases(ph), 4, 0, 64))
+
+
+# ---- the chain's first product fed by the attention's split-K partial results ---------------------------------
+
+class AttnLayer(Layer):
+    """A layer whose o-projection input is the decode attention of a step: caches prefilled with seeded
+    rows, the step's raw q/k/v in one stacked vector."""
+
+    def __init__(self, H, Hkv, D, Hd, I, ctx_max, seed):
+        super().__init__(Hd, I, H * D, (H + 2 * Hkv) * D, seed)
+        self.H, self.Hkv, self.D, self.ctx_max = H, Hkv, D, ctx_max
+        rng = np.random.default_rng(seed)
+        self.cache_k = torch.from_numpy((rng.standard_normal((ctx_max, Hkv * D)) / np.sqrt(D)).astype(np.float16)).cuda()
+        self.cache_v = torch.from_numpy((rng.standard_normal((ctx_max, Hkv * D)) / np.sqrt(D)).astype(np.float16)).cuda()
+        self.qkv_in = torch.from_numpy(rng.standard_normal((H + 2 * Hkv) * D).astype(np.float32)).cuda()
+        self.qw = torch.from_numpy((1 + 0.02 * rng.standard_normal(D)).astype(np.float32)).cuda()
+        self.kw = torch.from_numpy((1 + 0.02 * rng.standard_normal(D)).astype(np.float32)).cuda()
+        inv = 1.0 / (1e6 ** (np.arange(0, D, 2, dtype=np.float64) / D))
+        ang = np.arange(ctx_max, dtype=np.float64)[:, None] * inv[None, :]
+        self.cos = torch.from_numpy(np.cos(ang).astype(np.float32)).cuda()
+        self.sin = torch.from_numpy(np.sin(ang).astype(np.float32)).cuda()
+        L = capi.init(0)
+        self.ws = torch.zeros(int(L.dh_attn_decode_workspace_bytes(H, D, ctx_max)), dtype=torch.uint8, device="cuda")
+        self.attn_out = f32(H * D)
+        self.kvlen = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    def attn_args(self):
+        return (self.qkv_in.data_ptr(), self.qw.data_ptr(), self.kw.data_ptr(), self.cos.data_ptr(), self.sin.data_ptr(),
+                self.cache_k.data_ptr(), self.cache_v.data_ptr())
+
+    def tail(self):
+        return (self.D, 0, EPS, 0, 1, 1.0 / np.sqrt(self.D), 0.0, 0, 0, capi.KV_CONTIGUOUS, self.ws.data_ptr())
+
+
+@pytest.mark.parametrize("pos", [0, 63, 700, 2047, 4100])
+def test_chain_merges_the_attention_partials_like_the_merge_kernel(pos):
+    """attention (merge kernel) -> chain against attention partials -> chain that merges them: same bits in
+    every product, with the split count given by the host and with the key count on the device."""
+    L = capi.init(0)
+    H, Hkv, D = 32, 8, 128
+    lay = AttnLayer(H, Hkv, D, 2048, 4096, 4608, seed=7400 + pos)
+    assert L.dh_q4k_gemv_chain_attn_supported(H, Hkv, D, lay.ctx_max) == 1
+    arr = capi.chain_phases(lay.phases())
+    # first a launch at another key count (it appends the step's key/value there, so it comes before the
+    # reference is taken): the launches below follow the device word back to this test's position
+    lay.kvlen.fill_(max(1, pos // 2))
+    torch.cuda.synchronize()
+    capi.check(L.dh_attn_decode_qkv_kvlen_partials(*lay.attn_args(), H, Hkv, D, lay.kvlen.data_ptr(), lay.ctx_max, *lay.tail()))
+    src = capi.ChainAttnSource(lay.ws.data_ptr(), H, Hkv, D, 0, lay.kvlen.data_ptr(), lay.ctx_max, 0, 0)
+    capi.check(L.dh_q4k_gemv_chain_attn(ctypes.byref(src), arr, 4))
+    capi.check(L.dh_sync())
+    assert all(np.isfinite(_read(v)).all() for v in lay.out.values())
+    # reference path: attention with its own merge, then the chain on the merged vector
+    capi.check(L.dh_attn_decode_qkv(*lay.attn_args(), lay.attn_out.data_ptr(), H, Hkv, D, pos, *lay.tail()))
+    want_out = {k: torch.zeros_like(v) for k, v in lay.out.items()}
+    ph = lay.phases(want_out)
+    ph[0]["residual"] = lay.d["x"].data_ptr()
+    capi.check(L.dh_q4k_gemv_chain(lay.attn_out.data_ptr(), capi.chain_phases(ph), 4))
+    capi.check(L.dh_sync())
+    want = {k: _read(v) for k, v in want_out.items()}
+    assert all(np.isfinite(v).all() for v in want.values())
+    # host-known split count
+    for t in lay.out.values():
+        t.fill_(float("nan"))
+    nsplit = ctypes.c_int(0)
+    capi.check(L.dh_attn_decode_qkv_partials(*lay.attn_args(), H, Hkv, D, pos, *lay.tail(), ctypes.byref(nsplit)))
+    assert 1 <= nsplit.value <= 64
+    src = capi.ChainAttnSource(lay.ws.data_ptr(), H, Hkv, D, nsplit.value, None, 0, 0, 0)
+    capi.check(L.dh_q4k_gemv_chain_attn(ctypes.byref(src), arr, 4))
+    capi.check(L.dh_sync())
+    for k, v in lay.out.items():
+        assert _read(v).tobytes() == want[k].tobytes(), ("host", k)
+    # key count on the device, twice in a row
+    for rep in range(2):
+        for t in lay.out.values():
+            t.fill_(float("nan"))
+        lay.kvlen.fill_(pos + 1)
+        torch.cuda.synchronize()
+        capi.check(L.dh_attn_decode_qkv_kvlen_partials(*lay.attn_args(), H, Hkv, D, lay.kvlen.data_ptr(), lay.ctx_max,
+                                                       *lay.tail()))
+        src = capi.ChainAttnSource(lay.ws.data_ptr(), H, Hkv, D, 0, lay.kvlen.data_ptr(), lay.ctx_max, 0, 0)
+        capi.check(L.dh_q4k_gemv_chain_attn(ctypes.byref(src), arr, 4))
+        capi.check(L.dh_sync())
+        for k, v in lay.out.items():
+            assert _read(v).tobytes() == want[k].tobytes(), ("device", rep, k)
+
+
+def test_chain_attn_argument_errors():
+    L = capi.init(0)
+    lay = AttnLayer(32, 8, 128, 2048, 4096, 1024, seed=7500)
+    arr = capi.chain_phases(lay.phases())
+
+    def fails(src, match, n=4):
+        with pytest.raises(DopplerHipError, match=match):
+            capi.check(L.dh_q4k_gemv_chain_attn(ctypes.byref(src), arr, n))
+
+    ws = lay.ws.data_ptr()
+    fails(capi.ChainAttnSource(None, 32, 8, 128, 4, None, 0, 0, 0), "workspace is null")
+    fails(capi.ChainAttnSource(ws, 16, 8, 128, 4, None, 0, 0, 0), "product 0 takes K=4096")
+    fails(capi.ChainAttnSource(ws, 32, 8, 128, 0, None, 0, 0, 0), "nsplit must be at least 1")
+    fails(capi.ChainAttnSource(ws, 32, 8, 128, 65, None, 0, 0, 0), "up to 64 splits")
+    fails(capi.ChainAttnSource(ws, 32, 8, 128, 0, lay.kvlen.data_ptr(), 0, 0, 0), "max_kv_len >= 1")
+    assert L.dh_q4k_gemv_chain_attn_supported(32, 8, 96, 1024) == 0
+    assert L.dh_q4k_gemv_chain_attn_supported(32, 5, 128, 1024) == 0

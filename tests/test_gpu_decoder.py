@@ -371,7 +371,8 @@ def test_chained_gemv_decoder_matches_the_oracle_and_the_separate_launches():
         for n in ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown"):
             l[n] = synth.q4k_centred(l[n], 5)           # a stack whose logits depend on what it is fed
     chained = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, cfg["max_seq"], chain_gemvs=True)
-    plain = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, cfg["max_seq"])
+    plain = decoder.HipDecoder(cfg, layers, embed, final_norm, cos, sin, cfg["max_seq"], chain_gemvs=False)
+    assert not plain.chain_gemvs
     ol = oracle_layers(layers, cfg["max_seq"], cfg["kv_heads"], cfg["head_dim"])
     cpu = oracle.DecoderOracle(cfg, ol, embed, final_norm, cos, sin)
     prompt = synth.rng(82).integers(0, cfg["vocab"], 10)
@@ -387,6 +388,16 @@ def test_chained_gemv_decoder_matches_the_oracle_and_the_separate_launches():
         assert g == p == ctok, (pos, g, p, ctok)
         tok = g
     chained.release_graph()
+    # the same with the attention's own merge launch in front of the chain
+    assert chained.chain_merges_attention
+    chained.set_chain_gemvs(True, merge_attention=False)
+    assert not chained.chain_merges_attention
+    for pos in range(30, 34):
+        g = chained.step(tok, pos, want_logits=True)
+        p = plain.step(tok, pos, want_logits=True)
+        assert chained.read_logits().tobytes() == plain.read_logits().tobytes(), pos
+        assert g == p, pos
+        tok = g
     with pytest.raises(ValueError, match="chain"):
         small = dict(cfg, hidden=512, inter=1024, heads=4, kv_heads=2)
         sl, se, sf, sc, ss = decoder.random_model(small, seed=83, max_seq=cfg["max_seq"])
