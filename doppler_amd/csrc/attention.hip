@@ -39,7 +39,7 @@ struct AttnArgs {
   const __half* K;      // [rows][Hkv][D]
   const __half* V;
   float* O;             // [H][D]
-  float* ws;            // [H][nsplit][D + 2]  (o..., m, l)
+  float* ws;            // [H][nsplit of the launch][D + 2]  (o..., m, l)
   int H, Hkv, G, kbeg, kend, nsplit, tiles_per_split;
   int direct;           // one split and no merge launch behind it: the split kernel writes O itself
   float scale, softcap;
@@ -127,6 +127,10 @@ __device__ __forceinline__ float row_group_sum(float v) {
 template <int D, int GT, bool QKV>
 __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a_in) {
   AttnArgs a = a_in;
+  // splits per query head in the workspace: the launch's split count, which with the key count on the
+  // device is the largest any count can ask for, so that a reader finds a head's partial results
+  // without knowing the count
+  const int ws_stride = a.nsplit;
   if (a.dyn.kv_len_ptr != nullptr) {
     // the key count lives on the device: redo the host's arithmetic for it; surplus workgroups leave
     const KeyRange r = dyn_key_range(a.dyn);
@@ -443,12 +447,12 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
         for (int gg = 0; gg < GT; gg++) l = gg == g ? l_run[gg] : l;
         a.O[(int64_t)h * D + DW * wave + dim] = l > 0.f ? v / l : 0.f;
       } else {
-        a.ws[((int64_t)h * a.nsplit + split) * (D + 2) + DW * wave + dim] = v;
+        a.ws[((int64_t)h * ws_stride + split) * (D + 2) + DW * wave + dim] = v;
       }
     }
   }
   if (!a.direct && wave == 0 && lane < G) {
-    float* w = a.ws + ((int64_t)(kvh * G + lane) * a.nsplit + split) * (D + 2);
+    float* w = a.ws + ((int64_t)(kvh * G + lane) * ws_stride + split) * (D + 2);
     float mv = 0.f, lv = 0.f;
 #pragma unroll
     for (int g = 0; g < GT; g++) {     // pick this lane's head without dynamic register indexing
@@ -471,6 +475,7 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(const float* __res
   __shared__ float f_s[1024];
   __shared__ float red[4];
   const int h = blockIdx.x, d = threadIdx.x;
+  const int ws_stride = nsplit;      // splits per head in the workspace (see the split kernel)
   if (dyn.kv_len_ptr != nullptr) {
     nsplit = dyn_key_range(dyn).nsplit;
     if (nsplit == 0) {            // no visible key: the output is zero, as the host path writes it
@@ -478,7 +483,7 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(const float* __res
       return;
     }
   }
-  const float* base = ws + (int64_t)h * nsplit * (D + 2);
+  const float* base = ws + (int64_t)h * ws_stride * (D + 2);
   float ov[CH];
 #pragma unroll
   for (int i = 0; i < CH; i++) ov[i] = base[(int64_t)min(i, nsplit - 1) * (D + 2) + d];

@@ -121,11 +121,12 @@ struct ChainArgs {
   int xq_bytes[2];             // bytes of the two record areas (phases 0, 2 / 1, 3)
   int nb_max[2];               // columns of the two areas
   int red_stride;              // floats per tile slot: 16 * the largest units-per-tile
-  // phase 0's input as the split-K partial results of a decode attention (null: x0): [H][nsplit][D + 2]
+  // phase 0's input as the split-K partial results of a decode attention (null: x0): [H][attn_stride][D + 2]
   // (o..., m, l) per query head and split; the split count is attn_nsplit, or follows the key count
   // on the device as the attention kernels' own does
   const float* attn_ws;
   int attn_H, attn_D, attn_nsplit;
+  int attn_stride;             // splits per head in the workspace layout
   dh::DynKeys attn_dyn;
 };
 
@@ -275,21 +276,24 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
   v2f m_ml = {-FLT_MAX, 0.f};
   v2f m_ov[kMergePre];
   if (merger) {
-    m_nsplit = a.attn_nsplit;
-    if (a.attn_dyn.kv_len_ptr != nullptr) m_nsplit = dh::dyn_key_range(a.attn_dyn).nsplit;
-    m_nsplit = __builtin_amdgcn_readfirstlane(m_nsplit);
-    m_base = a.attn_ws + (int64_t)bid * m_nsplit * (a.attn_D + 2);
-    if (lane < m_nsplit) {
+    // the loads do not wait for the split count (with the key count on the device it is one more load):
+    // splits past it are read and ignored
+    m_base = a.attn_ws + (int64_t)bid * a.attn_stride * (a.attn_D + 2);
+    const int smax = a.attn_stride;
+    if (lane < smax) {
       const float* q = m_base + (int64_t)lane * (a.attn_D + 2) + a.attn_D;
       asm volatile("global_load_dwordx2 %0, %1, off" : "=&v"(m_ml) : "v"(q) : "memory");
     }
-    if (2 * lane < a.attn_D && m_nsplit > 0) {
+    if (2 * lane < a.attn_D) {
 #pragma unroll
       for (int i = 0; i < kMergePre; i++) {
-        const float* q = m_base + (int64_t)min(i, m_nsplit - 1) * (a.attn_D + 2) + 2 * lane;
+        const float* q = m_base + (int64_t)min(i, smax - 1) * (a.attn_D + 2) + 2 * lane;
         asm volatile("global_load_dwordx2 %0, %1, off" : "=&v"(m_ov[i]) : "v"(q) : "memory");
       }
     }
+    m_nsplit = a.attn_nsplit;
+    if (a.attn_dyn.kv_len_ptr != nullptr) m_nsplit = dh::dyn_key_range(a.attn_dyn).nsplit;
+    m_nsplit = __builtin_amdgcn_readfirstlane(m_nsplit);
   }
   if (!from_attn) {
     load_norm(a.ph[0].norm_weight, a.ph[0].nb, c_first, first);
@@ -828,6 +832,7 @@ int make_plan(const char* op, const float* d_x0, const dh_chain_attn_source* src
     a.attn_H = src->H;
     a.attn_D = src->D;
     a.attn_nsplit = src->nsplit;
+    a.attn_stride = max_splits;
   }
   a.xq_bytes[0] = a.nb_max[0] * kRec;
   a.xq_bytes[1] = a.nb_max[1] * kRec;

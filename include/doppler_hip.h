@@ -314,8 +314,9 @@ int dh_attn_decode_qkv_kvlen(const float* d_qkv, const float* d_q_weight, const 
                              int weight_offset, int use_norm, float scale, float softcap,
                              int sliding_window, int kv_start, int kv_layout, void* d_workspace);
 /* dh_attn_decode_qkv / dh_attn_decode_qkv_kvlen without the merge of the key splits: the splits'
- * partial results stay in the workspace, [H][nsplit][D + 2] floats (unnormalised output, running
- * maximum, running sum per query head and split), for a consumer that merges them itself
+ * partial results stay in the workspace, [H][S][D + 2] floats (unnormalised output, running
+ * maximum, running sum per query head and split; S = the split count, or with the key count on the
+ * device the largest count any key count up to max_kv_len can ask for), for a consumer that merges them itself
  * (dh_q4k_gemv_chain_attn: the reference's single attention dispatch,
  * src/gpu/kernels/attention_decode_online_f16kv.wgsl:84-243, followed by its o-projection,
  * src/inference/pipelines/text/attention/interpreter.js:1121-1160, with the launch between them removed).
