@@ -70,6 +70,42 @@ def gate_up_kernel_bandwidth(dec, reps):
     return total_ms / max(n, 1)
 
 
+def layer_chain_bandwidth(dec, reps):
+    """Average duration of the chained launch of a layer (o + residual, RMSNorm + gate/up + SiLU, down +
+    residual, next layer's RMSNorm + q/k/v: dh_q4k_gemv_chain), measured like the gate/up launch above,
+    cycling through the layers' weights; (ms per launch, algorithmic bytes per launch)."""
+    from doppler_amd import capi, synth
+    L, c = dec.L, dec.cfg
+    Hd, I = c["hidden"], c["inter"]
+    chains = [dec._chain_phases(li) for li in range(len(dec.layers) - 1)]      # the last layer's has three products
+    if not chains:
+        return None
+    qkv_n = dec.qs + 2 * dec.ks
+    nbytes = (synth.q4k_nbytes(Hd, dec.qs) + 2 * synth.q4k_nbytes(I, Hd) + synth.q4k_nbytes(Hd, I) + synth.q4k_nbytes(qkv_n, Hd)
+              + 4 * (dec.qs + 2 * Hd + Hd + Hd + I + I + Hd + Hd + Hd + Hd + qkv_n))   # inputs, residuals, norm weights, outputs
+    ev = [ctypes.c_void_p() for _ in range(2)]
+    for e in ev:
+        capi.check(L.dh_event_create(ctypes.byref(e)))
+
+    def sweep():
+        for arr, n in chains:
+            capi.check(L.dh_q4k_gemv_chain(dec.attn.data_ptr(), arr, n))
+    sweep()
+    capi.check(L.dh_sync())
+    total_ms, n = 0.0, 0
+    for r in range(reps):
+        capi.check(L.dh_event_record(ev[0]))
+        sweep()
+        capi.check(L.dh_event_record(ev[1]))
+        ms = ctypes.c_float()
+        capi.check(L.dh_event_elapsed_ms(ev[0], ev[1], ctypes.byref(ms)))
+        total_ms += ms.value
+        n += len(chains)
+    for e in ev:
+        capi.check(L.dh_event_destroy(e))
+    return total_ms / max(n, 1), nbytes
+
+
 def js_reference_timings():
     """Runs oracle/js/reference_port.mjs (one thread, as the reference's JS is) and returns its
     timings in milliseconds, or None when node is missing."""
@@ -259,12 +295,26 @@ def main():
     launch_bytes = 2 * synth.q4k_nbytes(I, Hd) + 2 * Hd * 4 + I * 4      # weights, x + norm weight, output
     avg_ms = gate_up_kernel_bandwidth(dec, reps=4)
     achieved = launch_bytes / (avg_ms * 1e-3) / 1e9
+    # the same product runs inside the decode step as the second phase of the layer's chained launch; that
+    # launch as a whole (four products, 108.5 MB) is measured beside it
+    chain_roof = None
+    if dec.chain_gemvs:
+        try:
+            m = layer_chain_bandwidth(dec, reps=4)
+            if m:
+                chain_roof = {"kernel": "chained layer launch: o + residual, RMSNorm + gate/up + SiLU, down + residual, RMSNorm + next q/k/v",
+                              "bytes_per_launch": int(m[1]), "avg_launch_us": round(m[0] * 1e3, 2),
+                              "achieved": round(m[1] / (m[0] * 1e-3) / 1e9, 1), "frac": round(m[1] / (m[0] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                log("[bench] chained layer launch: %.2f us, %.0f GB/s" % (chain_roof["avg_launch_us"], chain_roof["achieved"]))
+        except Exception as e:      # a side measurement
+            log("[bench] chained-launch measurement failed: %r" % (e,))
     roofline = {"bound": "hbm", "kernel": "q4k fused RMSNorm + gate/up GEMV + SiLU [2x12288x4096]", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                 "bytes_per_launch": launch_bytes, "avg_launch_us": round(avg_ms * 1e3, 2),
                 "traffic": GATE_UP_TRAFFIC_BYTES if (Hd, I) == (4096, 12288) else None,
                 "traffic_source": "stored figure from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs summarised under "
-                                  "profiles/ (not measured in this run)"}
+                                  "profiles/ (not measured in this run)",
+                "in_step": chain_roof}
 
     if args.copy_calibration:
         # a streaming kernel of known traffic: reads 64 MiB of f32, writes 32 MiB of f16

@@ -224,6 +224,55 @@ FN(js_attn_decode_qkv_kvlen) {
                                               (const float*)s, ck, cv, (float*)O, H, Hkv, D, (const uint32_t*)kvLenPtr,
                                               maxKvLen, rd, inter, eps, woff, useNorm, scale, cap, win, kvStart, layout, ws));
 }
+/* the splits left unmerged: returns the split count */
+FN(js_attn_decode_qkv_partials) {
+  ARGS(22); P(0, qkv); P(1, qw); P(2, kw); P(3, c); P(4, s); P(5, ck); P(6, cv); I(7, H); I(8, Hkv); I(9, D);
+  I(10, startPos); I(11, rd); I(12, inter); F(13, eps); I(14, woff); I(15, useNorm); F(16, scale); F(17, cap);
+  I(18, win); I(19, kvStart); I(20, layout); P(21, ws);
+  int nsplit = 0;
+  if (dh_attn_decode_qkv_partials((const float*)qkv, (const float*)qw, (const float*)kw, (const float*)c, (const float*)s, ck,
+                                  cv, H, Hkv, D, startPos, rd, inter, eps, woff, useNorm, scale, cap, win, kvStart, layout,
+                                  ws, &nsplit) != 0)
+    return fail(env, dh_last_error());
+  return ret_num(env, nsplit);
+}
+FN(js_attn_decode_qkv_kvlen_partials) {
+  ARGS(23); P(0, qkv); P(1, qw); P(2, kw); P(3, c); P(4, s); P(5, ck); P(6, cv); I(7, H); I(8, Hkv); I(9, D);
+  P(10, kvLenPtr); I(11, maxKvLen); I(12, rd); I(13, inter); F(14, eps); I(15, woff); I(16, useNorm); F(17, scale);
+  F(18, cap); I(19, win); I(20, kvStart); I(21, layout); P(22, ws);
+  return ret_rc(env, dh_attn_decode_qkv_kvlen_partials((const float*)qkv, (const float*)qw, (const float*)kw, (const float*)c,
+                                                       (const float*)s, ck, cv, H, Hkv, D, (const uint32_t*)kvLenPtr,
+                                                       maxKvLen, rd, inter, eps, woff, useNorm, scale, cap, win, kvStart,
+                                                       layout, ws));
+}
+/* ---- chained GEMVs: the structs travel as bytes laid out by the caller (sizes checked here) ---- */
+FN(js_chain_struct_sizes) {
+  (void)info;
+  napi_value arr, v;
+  napi_create_array_with_length(env, 2, &arr);
+  napi_create_uint32(env, (uint32_t)sizeof(dh_chain_phase), &v); napi_set_element(env, arr, 0, v);
+  napi_create_uint32(env, (uint32_t)sizeof(dh_chain_attn_source), &v); napi_set_element(env, arr, 1, v);
+  return arr;
+}
+FN(js_q4k_gemv_chain) {
+  ARGS(3); P(0, x0); I(2, n);
+  void* ph = NULL; size_t len = 0;
+  if (!arg_bytes(env, a[1], &ph, &len)) return NULL;
+  if (n < 0 || len < (size_t)n * sizeof(dh_chain_phase)) return fail(env, "[q4kGemvChain] the phase bytes are shorter than n_phases structs");
+  return ret_rc(env, dh_q4k_gemv_chain((const float*)x0, (const dh_chain_phase*)ph, n));
+}
+FN(js_q4k_gemv_chain_attn) {
+  ARGS(3); I(2, n);
+  void* src = NULL; void* ph = NULL; size_t slen = 0, len = 0;
+  if (!arg_bytes(env, a[0], &src, &slen) || !arg_bytes(env, a[1], &ph, &len)) return NULL;
+  if (slen < sizeof(dh_chain_attn_source)) return fail(env, "[q4kGemvChainAttn] the source bytes are shorter than the struct");
+  if (n < 0 || len < (size_t)n * sizeof(dh_chain_phase)) return fail(env, "[q4kGemvChainAttn] the phase bytes are shorter than n_phases structs");
+  return ret_rc(env, dh_q4k_gemv_chain_attn((const dh_chain_attn_source*)src, (const dh_chain_phase*)ph, n));
+}
+FN(js_q4k_gemv_chain_attn_supported) {
+  ARGS(4); I(0, H); I(1, Hkv); I(2, D); I(3, maxKvLen);
+  return ret_num(env, dh_q4k_gemv_chain_attn_supported(H, Hkv, D, maxKvLen));
+}
 FN(js_attn_prefill) {
   ARGS(14); P(0, Q); P(1, K); P(2, V); P(3, O); I(4, T); I(5, H); I(6, Hkv); I(7, D); I(8, kvLen); F(9, scale);
   I(10, causal); I(11, startPos); F(12, cap); I(13, win);
@@ -336,6 +385,9 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"attnDecodeStatic", js_attn_decode_static}, {"attnDecodeStaticMaxBytes", js_attn_decode_static_max_bytes},
       {"attnDecodeQkvSupported", js_attn_decode_qkv_supported}, {"attnDecodeQkv", js_attn_decode_qkv},
       {"attnDecodeKvLen", js_attn_decode_kvlen}, {"attnDecodeQkvKvLen", js_attn_decode_qkv_kvlen},
+      {"attnDecodeQkvPartials", js_attn_decode_qkv_partials}, {"attnDecodeQkvKvLenPartials", js_attn_decode_qkv_kvlen_partials},
+      {"chainStructSizes", js_chain_struct_sizes}, {"q4kGemvChain", js_q4k_gemv_chain}, {"q4kGemvChainAttn", js_q4k_gemv_chain_attn},
+      {"q4kGemvChainAttnSupported", js_q4k_gemv_chain_attn_supported},
       {"attnPrefill", js_attn_prefill},
       {"rmsnorm", js_rmsnorm}, {"rmsnormQK", js_rmsnorm_qk}, {"rmsnormSandwichPair", js_rmsnorm_sandwich_pair},
       {"residualRmsnormPair", js_residual_rmsnorm_pair}, {"rope", js_rope}, {"ropeQK", js_rope_qk}, {"qkvNormRopeKvwrite", js_qkv_norm_rope_kvwrite},

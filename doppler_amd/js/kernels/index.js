@@ -5,6 +5,10 @@ export { runMatmul, recordMatmul, runDequantQ4K } from './matmul.js';
 export { runFusedFFN, recordFusedFFN, runFusedNormedFFN, recordFusedNormedFFN } from './fused_ffn.js';
 export { runAttention, recordAttention } from './attention.js';
 export { runDecodeAttentionFromQKV, recordDecodeAttentionFromQKV, decodeAttentionFromQKVSupported } from './attention-from-qkv.js';
+export {
+  recordLayerChain, recordDecodeAttentionPartials, layerChainSupported, layerChainMergesAttention, packChainPhases,
+  packChainAttnSource,
+} from './gemv-chain.js';
 export { runRMSNorm, recordRMSNorm } from './rmsnorm.js';
 export { runRMSNormQK, recordRMSNormQK, canUseRMSNormQK } from './rmsnorm-qk.js';
 export {

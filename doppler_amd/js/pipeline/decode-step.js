@@ -8,6 +8,7 @@ import {
   createCommandRecorder, recordGather, recordRMSNorm, recordMatmul, recordSplitQKVRMSNormRoPEQK,
   recordAttention, recordFusedNormedFFN, recordFusedFFN, recordLmHeadArgmaxF16, recordGPUSample,
   recordDecodeAttentionFromQKV, decodeAttentionFromQKVSupported,
+  recordLayerChain, recordDecodeAttentionPartials, layerChainSupported, layerChainMergesAttention,
   recordCheckFiniteness, parseFinitenessStatusWords, resolveFinitenessAbsThreshold, FINITENESS_STATUS_BYTES,
 } from '../kernel-selector.js';
 import { getNative } from '../native.js';
@@ -65,6 +66,10 @@ export class HipTextDecoder {
     // geometry allows it (one launch fewer per layer)
     this.fuseQkvAttention = config.fuseQkvAttention !== false &&
       decodeAttentionFromQKVSupported(c.heads, c.kvHeads, c.headDim, c.headDim, false);
+    // ... and the products between two attentions go out as one chained launch that also merges the
+    // attention's key splits (two launches per layer), where the shapes are served and the guard is off
+    this.chainGemvs = config.chainGemvs !== false && this.fuseQkvAttention && config.finitenessGuard !== true &&
+      layerChainSupported(c.hidden, c.inter, this.qSize) && layerChainMergesAttention(c.heads, c.kvHeads, c.headDim, c.maxSeq);
     this.ids = acquireBuffer(16, undefined, 'token_ids');
     // [token, status, layer, step, pad]: the staging layout of the reference's guarded readback
     this.tokenOut = acquireBuffer(4 + FINITENESS_STATUS_BYTES, undefined, 'sampled_token');
@@ -185,7 +190,9 @@ export class HipTextDecoder {
     const temp = (t) => { temps.push(t.buffer); return t; };
     let x = temp(await recordGather(recorder, this.ids, this.embed, 1, c.hidden, c.vocab,
       { embeddingDtype: 'f16', outputDtype: 'f32' }));
-    for (let li = 0; li < this.layers.length; li++) {
+    if (this.chainGemvs) {
+      x = await this.recordChainedLayers(recorder, temps, x, pos, options);
+    } else for (let li = 0; li < this.layers.length; li++) {
       const l = this.layers[li];
       // input RMSNorm runs in the prologue of the stacked q/k/v projection
       const qkv = temp(await recordMatmul(recorder, x, l.wqkv, 1, this.qSize + 2 * this.kSize, c.hidden,
@@ -228,6 +235,44 @@ export class HipTextDecoder {
         logitsOutput: options.logitsOutput || null,
       });
     }
+  }
+
+  // The layers of a decode step at two launches each: the attention's split kernel, then one chained
+  // launch that merges the splits and runs o + residual, RMSNorm + gate/up + SiLU, down + residual and
+  // the next layer's RMSNorm + q/k/v.  Returns the last layer's output row.
+  async recordChainedLayers(recorder, temps, x, pos, options) {
+    const c = this.config;
+    const qkvSize = this.qSize + 2 * this.kSize;
+    const f32 = (n, label) => { const b = acquireBuffer(n * 4, undefined, label); temps.push(b); return b; };
+    const l0 = this.layers[0];
+    let qkv = await recordMatmul(recorder, x, l0.wqkv, 1, qkvSize, c.hidden,
+      { outputDtype: 'f32', role: 'qkv_proj', layerIdx: 0, normWeight: l0.inputNorm, rmsNormEps: c.eps, useFusedRmsnormWideTile: true });
+    temps.push(qkv.buffer);
+    let xb = x.buffer;
+    for (let li = 0; li < this.layers.length; li++) {
+      const l = this.layers[li];
+      const next = li + 1 < this.layers.length ? this.layers[li + 1] : null;
+      const attention = recordDecodeAttentionPartials(recorder, qkv, l.qNorm, l.kNorm, this.cos, this.sin, c.eps, l.cacheK, l.cacheV, {
+        numHeads: c.heads, numKVHeads: c.kvHeads, headDim: c.headDim, startPos: pos,
+        kvLenBuffer: options.deviceKvLen ? bufferWindow(this.ids, 4, 4) : null, maxKvLen: c.maxSeq,
+      });
+      temps.push(attention.workspace);
+      const x2 = f32(c.hidden, 'attn_output'), act = f32(c.inter, 'ffn_act'), xOut = f32(c.hidden, 'layer_output');
+      const phases = [
+        { weight: l.wo, output: x2, residual: xb, N: c.hidden, K: this.qSize },
+        { weight: l.wgate, weight2: l.wup, output: act, normWeight: l.postAttnNorm, N: c.inter, K: c.hidden, activation: 'silu', rmsNormEps: c.eps },
+        { weight: l.wdown, output: xOut, residual: x2, N: c.hidden, K: c.inter },
+      ];
+      let qkvNext = null;
+      if (next) {
+        qkvNext = f32(qkvSize, 'qkv');
+        phases.push({ weight: next.wqkv, output: qkvNext, normWeight: next.inputNorm, N: qkvSize, K: c.hidden, rmsNormEps: c.eps });
+      }
+      recordLayerChain(recorder, null, phases, attention);
+      xb = xOut;
+      if (next) qkv = createTensor(qkvNext, 'f32', [1, qkvSize], 'qkv');
+    }
+    return createTensor(xb, 'f32', [1, c.hidden], 'layer_output');
   }
 
   // Returns the greedy token for `token` at position `pos` (KV rows 0..pos-1 present).

@@ -207,6 +207,9 @@ async function main() {
         embed: load(c.embed), finalNorm: load(c.finalNorm), cos: load(c.cos), sin: load(c.sin),
       };
       const dec = new HipTextDecoder(cfg, weights);
+      if (c.expectChained !== undefined) {
+        results.errors.push({ label: `${c.name}-chained`, ok: dec.chainGemvs === c.expectChained, message: `chainGemvs=${dec.chainGemvs}` });
+      }
       const tokens = [];
       let tok = c.prompt[0];
       for (let pos = 0; pos < c.prompt.length + c.steps; pos++) {

@@ -349,6 +349,42 @@ def test_js_host_path_parity(tmp_path):
     checks.append(lambda: [int(t) for t in get("decoder_guarded_graph.out.bin", np.uint32)] == want_tokens)
     checks.append(lambda: get("decoder_guard_trips.out.bin", np.uint32).size == 0)
 
+    # ---- the chained layer launch from the JS decoder: a model wide enough for it (the small one above
+    #      keeps one launch per op), weights centred so that the logits depend on what the stack is fed;
+    #      eager and from the captured graph, and the same model with the chain switched off
+    ccfg = dict(layers=2, hidden=2048, inter=4096, heads=16, kv_heads=4, head_dim=128, vocab=700, eps=1e-6, qk_norm=1,
+                max_seq=24, theta=1e6)
+    clayers, cembed, cfinal, cmc, cms = decoder.random_model(ccfg, seed=91, max_seq=24)
+    for l in clayers:
+        for n in ("wq", "wk", "wv", "wo", "wgate", "wup", "wdown"):
+            l[n] = synth.q4k_centred(l[n], 5)
+    cjl = []
+    for i, l in enumerate(clayers):
+        cjl.append(dict(wqkv=put("C%d.qkv" % i, np.concatenate([l["wq"], l["wk"], l["wv"]])), wo=put("C%d.o" % i, l["wo"]),
+                        wgate=put("C%d.g" % i, l["wgate"]), wup=put("C%d.u" % i, l["wup"]), wdown=put("C%d.d" % i, l["wdown"]),
+                        inputNorm=put("C%d.in" % i, l["input_norm"]), postAttnNorm=put("C%d.pn" % i, l["post_attn_norm"]),
+                        qNorm=put("C%d.qn" % i, l["q_norm"]), kNorm=put("C%d.kn" % i, l["k_norm"])))
+    cprompt = [int(t) for t in synth.rng(92).integers(0, 700, 5)]
+    cases.append(dict(name="decoder_chained", op="decoder", layers=cjl, embed=put("c.embed", cembed), finalNorm=put("c.fn", cfinal),
+                      cos=put("c.cos", cmc), sin=put("c.sin", cms), prompt=cprompt, steps=9, graphFrom=7, expectChained=True,
+                      config=dict(layers=2, hidden=2048, inter=4096, heads=16, kvHeads=4, headDim=128, vocab=700, eps=1e-6, maxSeq=24)))
+    cases.append(dict(cases[-1], name="decoder_chain_off", expectChained=False,
+                      config=dict(cases[-1]["config"], chainGemvs=False)))
+    col = []
+    for l in clayers:
+        dd = dict(l)
+        dd["cache_k"] = np.zeros((24, 4, 128), np.uint16)
+        dd["cache_v"] = np.zeros((24, 4, 128), np.uint16)
+        col.append(dd)
+    ccpu = oracle.DecoderOracle(ccfg, col, cembed, cfinal, cmc, cms)
+    cwant, ctok = [], None
+    for pos in range(len(cprompt) + 9):
+        ctok = ccpu.step(cprompt[pos] if pos < len(cprompt) else ctok, pos)
+        cwant.append(ctok)
+    assert len(set(cwant)) > 2, cwant
+    checks.append(lambda: [int(t) for t in get("decoder_chained.out.bin", np.uint32)] == cwant)
+    checks.append(lambda: [int(t) for t in get("decoder_chain_off.out.bin", np.uint32)] == cwant)
+
     # ---- top-k temperature sampling through the JS op (seeded draw as in the reference)
     slog = (synth.rng(79).standard_normal(4000) * 3).astype(np.float32)
     cases.append(dict(name="sample", op="sample", logits=put("s.logits", slog), vocab=4000, temperature=0.9, topK=40, seed=42))
