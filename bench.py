@@ -220,16 +220,30 @@ def main():
     torch.cuda.synchronize()
     capi_sync = dec.L.dh_sync
     capi_sync()
+    # the timed region: K greedy steps through the generation loop (every token read back, one step late:
+    # HipDecoder.decode_greedy), then the same K positions again one blocking step at a time for comparison
+    dec.decode_greedy(tok, pos, 2)                # pinned staging memory and events are made here, outside the timing
+    capi_sync()
     t0 = time.perf_counter()
-    tokens = []
-    for _ in range(args.steps):
-        tok = dec.step(tok, pos)
-        tokens.append(tok)
-        pos += 1
+    tokens = dec.decode_greedy(tok, pos, args.steps)
     capi_sync()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     tok_s = args.steps / elapsed
+    t0 = time.perf_counter()
+    tokens_blocking = []
+    t_ = tok
+    for i in range(args.steps):
+        t_ = dec.step(t_, pos + i)
+        tokens_blocking.append(t_)
+    capi_sync()
+    blocking_tok_s = args.steps / (time.perf_counter() - t0)
+    if tokens_blocking != tokens:
+        log("[bench] FAILED: the generation loop and the blocking steps disagree: %r vs %r" % (tokens[:8], tokens_blocking[:8]))
+        sys.exit(1)
+    tok = tokens[-1]
+    pos += args.steps
+    log("[bench] the same %d steps, one blocking step at a time: %.1f tok/s" % (args.steps, blocking_tok_s))
     ctx_mid = prefill + args.warmup + args.steps // 2
     step_bytes = dec.weight_bytes_per_token(ctx_mid)
     log("[bench] %d steps in %.3f s -> %.1f tok/s (%.0f GB/s of algorithmic traffic)" %
@@ -374,6 +388,7 @@ def main():
                    "batched_decode_16_per_submit_tokens_per_s": round(batched_tok_s, 2),
                    "graph_replay_tokens_per_s": round(graph_tok_s, 2),
                    "graph_replay_host_patched_tokens_per_s": round(graph_patched_tok_s, 2),
+                   "blocking_step_tokens_per_s": round(blocking_tok_s, 2),
                    "launches_per_layer": 2 if dec.chain_merges_attention else (3 if dec.chain_gemvs else 6),
                    "unchained_tokens_per_s": round(unchained_tok_s, 2) if unchained_tok_s else None,
                    "js_host": js_host,

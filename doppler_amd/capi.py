@@ -63,6 +63,10 @@ SIGNATURES = {
     "dh_copy": (_I, [_P, _SZ, _P, _SZ, _SZ]),
     "dh_fill_zero": (_I, [_P, _SZ, _SZ]),
     "dh_sync": (_I, []),
+    "dh_host_alloc": (_I, [_SZ, ctypes.POINTER(_P)]),
+    "dh_host_free": (_I, [_P]),
+    "dh_download_async": (_I, [_P, _P, _SZ, _SZ]),
+    "dh_event_synchronize": (_I, [_P]),
     "dh_event_create": (_I, [ctypes.POINTER(_P)]),
     "dh_event_record": (_I, [_P]),
     "dh_event_elapsed_ms": (_I, [_P, _P, ctypes.POINTER(_F)]),

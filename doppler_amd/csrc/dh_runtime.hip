@@ -261,6 +261,39 @@ int dh_download(void* host_dst, const void* d_src, size_t src_offset, size_t byt
   return dh::check_kernel_status("dh_download");
 }
 
+// ---- readback that does not wait: pinned host memory, an enqueued copy, an event to wait for -----
+int dh_host_alloc(size_t bytes, void** out) {
+  DH_REQUIRE_INIT("dh_host_alloc");
+  if (!out || bytes == 0) return dh::fail(1, "[dh_host_alloc] need a size and a place for the pointer");
+  DH_CHECK_HIP("dh_host_alloc", hipHostMalloc(out, bytes, hipHostMallocDefault));
+  return 0;
+}
+
+int dh_host_free(void* p) {
+  DH_REQUIRE_INIT("dh_host_free");
+  if (!p) return 0;
+  DH_CHECK_HIP("dh_host_free", hipHostFree(p));
+  return 0;
+}
+
+int dh_download_async(void* host_dst, const void* d_src, size_t src_offset, size_t bytes) {
+  DH_REQUIRE_INIT("dh_download_async");
+  if (g_capturing) return dh::fail(1, "[dh_download_async] not possible while a graph is being captured");
+  if (bytes == 0) return 0;
+  if (!host_dst || !d_src) return dh::fail(1, "[dh_download_async] null pointer");
+  DH_CHECK_HIP("dh_download_async", hipMemcpyAsync(host_dst, static_cast<const char*>(d_src) + src_offset, bytes,
+                                                   hipMemcpyDeviceToHost, g_stream));
+  return 0;
+}
+
+int dh_event_synchronize(void* ev) {
+  DH_REQUIRE_INIT("dh_event_synchronize");
+  if (!ev) return dh::fail(1, "[dh_event_synchronize] null event");
+  DH_CHECK_HIP("dh_event_synchronize", hipEventSynchronize(static_cast<hipEvent_t>(ev)));
+  // everything enqueued before the event has run: a kernel among it may have given up a bounded wait
+  return dh::check_kernel_status("dh_event_synchronize");
+}
+
 int dh_copy(void* d_dst, size_t dst_offset, const void* d_src, size_t src_offset, size_t bytes) {
   DH_REQUIRE_INIT("dh_copy");
   if (bytes == 0) return 0;

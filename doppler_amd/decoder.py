@@ -328,6 +328,62 @@ class HipDecoder:
         self._raise_if_triggered(words, 1, "generation")
         return int(words[0])
 
+    def decode_greedy(self, token, pos, n):
+        """n greedy steps starting with `token` at position `pos`; returns the n new token ids.  Every
+        step's token is read back (4 bytes per step, as in step()), but one step late: step k + 1 takes its
+        input token from device memory and is enqueued before the host waits for token k, whose copy into
+        pinned memory was enqueued behind step k, so the GPU never waits for the host between steps (the
+        reference stages its token readbacks through a ring the same way, src/inference/decode-ring.js:141-177).
+        A caller with a stop condition checks the tokens as they come and drops the one step in flight."""
+        if n <= 0:
+            return []
+        if self.finiteness_guard:
+            out = []
+            for k in range(n):
+                token = self.step(token, pos + k)
+                out.append(token)
+            return out
+        L, ck, R, E = self.L, capi.check, self.TOKEN_RING, 4
+        if getattr(self, "_pinned", None) is None:
+            p = ctypes.c_void_p()
+            ck(L.dh_host_alloc(4 * R, ctypes.byref(p)))
+            self._pinned = p
+            self._pinned_tokens = (ctypes.c_uint32 * R).from_address(p.value)
+            self._read_events = []
+            for _ in range(E):
+                e = ctypes.c_void_p()
+                ck(L.dh_event_create(ctypes.byref(e)))
+                self._read_events.append(e)
+
+        def enqueue_read(k):
+            slot = k % R
+            ck(L.dh_download_async(self._pinned.value + 4 * slot, self.token.data_ptr(), 4 * slot, 4))
+            ck(L.dh_event_record(self._read_events[k % E]))
+
+        def wait_read(k):
+            ck(L.dh_event_synchronize(self._read_events[k % E]))
+            return int(self._pinned_tokens[k % R])
+
+        self.set_token(token)
+        self.enqueue_step(pos, out_index=0)
+        enqueue_read(0)
+        out = []
+        for k in range(1, n):
+            self.enqueue_step(pos + k, from_device_token=True, in_index=(k - 1) % R, out_index=k % R)
+            enqueue_read(k)
+            out.append(wait_read(k - 1))
+        out.append(wait_read(n - 1))
+        return out
+
+    def release_readback(self):
+        """Frees the pinned staging memory and the events decode_greedy() made."""
+        if getattr(self, "_pinned", None) is not None:
+            for e in self._read_events:
+                capi.check(self.L.dh_event_destroy(e))
+            self._pinned_tokens = None
+            capi.check(self.L.dh_host_free(self._pinned))
+            self._pinned = None
+
     def capture_step(self, pos, want_logits=False, device_kv_len=True):
         """Captures one decode step (enqueued for position `pos`) into a HIP graph, the
         counterpart of the reference's one-submit-per-step recorder

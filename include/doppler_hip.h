@@ -64,6 +64,14 @@ int dh_event_create(void** ev_out);
 int dh_event_record(void* ev);
 int dh_event_elapsed_ms(void* start, void* stop, float* ms_out);
 int dh_event_destroy(void* ev);
+/* Readback that does not wait for the stream (reference: the ring of token staging buffers that lets a
+ * step's token be mapped while later work is queued, src/inference/decode-ring.js:141-177): pinned host
+ * memory, a copy enqueued behind the ops so far, and a wait for an event recorded behind that copy.
+ * dh_event_synchronize also reports a kernel that gave up a bounded wait, like dh_sync. */
+int dh_host_alloc(size_t bytes, void** host_out);
+int dh_host_free(void* host_ptr);
+int dh_download_async(void* host_dst, const void* d_src, size_t src_offset, size_t bytes);
+int dh_event_synchronize(void* ev);
 
 /* ---- captured decode steps ----
  * The reference records a whole decode step into one command encoder and submits it once

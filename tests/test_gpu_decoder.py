@@ -398,6 +398,18 @@ def test_chained_gemv_decoder_matches_the_oracle_and_the_separate_launches():
         assert chained.read_logits().tobytes() == plain.read_logits().tobytes(), pos
         assert g == p, pos
         tok = g
+    # decode_greedy(): the same steps with every token read back one step late (the next step is enqueued first)
+    chained.set_chain_gemvs(True)
+    want = []
+    t = tok
+    for pos in range(34, 44):
+        t = plain.step(t, pos)
+        want.append(t)
+    assert chained.decode_greedy(tok, 34, 10) == want
+    assert plain.decode_greedy(tok, 34, 10) == want
+    assert chained.decode_greedy(tok, 34, 1) == want[:1] and chained.decode_greedy(tok, 34, 0) == []
+    chained.release_readback()
+    plain.release_readback()
     with pytest.raises(ValueError, match="chain"):
         small = dict(cfg, hidden=512, inter=1024, heads=4, kv_heads=2)
         sl, se, sf, sc, ss = decoder.random_model(small, seed=83, max_seq=cfg["max_seq"])
