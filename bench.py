@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per fused gate/up launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs, scaled
 # by the same counters' readings for a cast kernel of known traffic (x2.000 and x1.000):
 # 55,683 KiB fetched + 48 KiB written.
-GATE_UP_TRAFFIC_BYTES = 57069000
+GATE_UP_TRAFFIC_BYTES = 57088000
 
 
 def log(*a):

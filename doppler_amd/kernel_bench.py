@@ -1,6 +1,6 @@
 """Per-kernel measurements of the HIP path on the benchmark configurations.
 
-    python -m doppler_amd.kernel_bench [--only gemv,gemm,attn,prefill_attn,lmhead,dense] [--json out.jsonl]
+    python -m doppler_amd.kernel_bench [--only gemv,chain,gemm,attn,prefill_attn,lmhead,dense] [--json out.jsonl]
 
 Every case is timed with events around back-to-back launches on the library's stream.  Weights
 (and KV caches) rotate through enough copies that their total exceeds the 256 MB Infinity Cache
@@ -121,6 +121,46 @@ def gemv_cases(L, T, rows, reps):
         run(4, "o+residual (cfg4)", M, 4096, 4096, residual=True)
         run(4, "norm+gate/up+silu (cfg4)", M, 12288, 4096, dual=True, norm=True)
         run(4, "down+residual (cfg4)", M, 4096, 12288, residual=True)
+
+
+def chain_cases(L, T, rows, reps):
+    """The four dependent products of a cfg4 decoder layer as one launch (dh_q4k_gemv_chain) against the
+    same products as four launches; weights rotating through enough layers to stay out of the caches."""
+    Hd, I, QS, QKV = 4096, 12288, 4096, 6144
+    shapes = [(Hd, QS), (I, Hd), (I, Hd), (Hd, I), (QKV, Hd)]                 # o, gate, up, down, next qkv
+    per_layer = sum(synth.q4k_nbytes(n, k) for n, k in shapes)
+    algo = per_layer + 4 * (QS + 2 * Hd + Hd + Hd + I + I + Hd + Hd + Hd + Hd + QKV)
+    f32 = lambda n: torch.zeros(n, device="cuda")
+    attn, x, x2, act, x3, qkv = torch.randn(QS, device="cuda") * 0.01, torch.randn(Hd, device="cuda") * 0.01, f32(Hd), f32(I), f32(Hd), f32(QKV)
+    n1, n2 = torch.ones(Hd, device="cuda"), torch.ones(Hd, device="cuda")
+    for mode in ("rotating", "warm"):
+        layers = n_copies(per_layer, 16) if mode == "rotating" else 1
+        W = [[q4k_copies(synth.q4k_nbytes(n, k), 1)[0] for n, k in shapes] for _ in range(layers)]
+        chains = []
+        for wo, wg, wu, wd, wq in W:
+            chains.append(capi.chain_phases([
+                dict(W=wo.data_ptr(), C=x2.data_ptr(), residual=x.data_ptr(), N=Hd, K=QS),
+                dict(W=wg.data_ptr(), W2=wu.data_ptr(), C=act.data_ptr(), norm_weight=n1.data_ptr(), N=I, K=Hd,
+                     activation=capi.ACT_SILU, norm_eps=1e-6),
+                dict(W=wd.data_ptr(), C=x3.data_ptr(), residual=x2.data_ptr(), N=Hd, K=I),
+                dict(W=wq.data_ptr(), C=qkv.data_ptr(), norm_weight=n2.data_ptr(), N=QKV, K=Hd, norm_eps=1e-6)]))
+
+        def chained(i):
+            capi.check(L.dh_q4k_gemv_chain(attn.data_ptr(), chains[i % layers], 4))
+
+        def separate(i):
+            wo, wg, wu, wd, wq = W[i % layers]
+            capi.check(L.dh_q4k_matmul(attn.data_ptr(), 0, wo.data_ptr(), x2.data_ptr(), 0, 1, Hd, QS, 1.0, x.data_ptr()))
+            capi.check(L.dh_q4k_ffn_gate_up_rmsnorm(x2.data_ptr(), n1.data_ptr(), 1e-6, 0, wg.data_ptr(), wu.data_ptr(),
+                                                    act.data_ptr(), 1, Hd, I, capi.ACT_SILU, 1.0, 0.0))
+            capi.check(L.dh_q4k_matmul(act.data_ptr(), 0, wd.data_ptr(), x3.data_ptr(), 0, 1, Hd, I, 1.0, x2.data_ptr()))
+            capi.check(L.dh_q4k_matmul_rmsnorm(x3.data_ptr(), n2.data_ptr(), 1e-6, 0, wq.data_ptr(), qkv.data_ptr(), 0, 1, QKV,
+                                               Hd, 1.0, None))
+        for name, fn in (("q4k_gemv_chain o,gate/up,down,qkv (cfg4)", chained), ("the same as four launches (cfg4)", separate)):
+            us = T.us(fn, reps)
+            emit(rows, config=4, kernel=name, shape="one decoder layer, M=1", mode=mode, us=round(us, 3),
+                 achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
+        del W, chains
 
 
 def gemm_cases(L, T, rows, reps):
@@ -284,7 +324,7 @@ def dense_cases(L, T, rows, reps):
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", default="gemv,gemm,attn,prefill_attn,lmhead,dense")
+    ap.add_argument("--only", default="gemv,chain,gemm,attn,prefill_attn,lmhead,dense")
     ap.add_argument("--reps", type=int, default=96)
     ap.add_argument("--json", default=None, help="also write one JSON object per case to this file")
     args = ap.parse_args(argv)
@@ -296,6 +336,8 @@ def main(argv=None):
     which = set(args.only.split(","))
     if "gemv" in which:
         gemv_cases(L, T, rows, args.reps)
+    if "chain" in which:
+        chain_cases(L, T, rows, args.reps)
     if "gemm" in which:
         gemm_cases(L, T, rows, max(8, args.reps // 4))
     if "attn" in which:
