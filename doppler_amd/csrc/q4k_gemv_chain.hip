@@ -678,9 +678,12 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
         su = sum_lane_groups(su);
         if (norm) {
           if (!have_rms) {
-            // every column has been consumed by now, so every column's sum of squares is in place
-            float tot = 0.f;
-            for (int c = 0; c < nb; c++) tot += __uint_as_float(lds_read_u32(xq_abs + (uint32_t)c * kRec + kRecSsq));
+            // every column has been consumed by now, so every column's sum of squares is in place: lane l
+            // takes columns l, l + 64, .. (one LDS read each, all lanes at once), then the lanes meet in a
+            // fixed order (the single-product kernel's)
+            float part = 0.f;
+            for (int c = lane; c < nb; c += 64) part += __uint_as_float(lds_read_u32(xq_abs + (uint32_t)c * kRec + kRecSsq));
+            const float tot = dh::wave_sum_uniform(part);
             inv_rms = 1.0f / sqrtf(tot / (float)Q.K + Q.norm_eps);
             have_rms = true;
           }
