@@ -164,14 +164,16 @@ int attn_static_scratch_init(int device);
 // Decode GEMV on the int8 matrix cores (q4k_gemv_i8.hip): C = alpha * A . W^T + residual, or with W2
 // the gated pair act(A . W^T) * (A . W2^T) * alpha; norm_weight != null normalises A's rows first.
 // Returns -1 when the shape is not served (the caller then takes another kernel), 0 on success.
+// a_f16: A holds f16 rows (single matrix, no norm prologue, K a multiple of 4, rows 8-byte aligned;
+// -1 otherwise), widened exactly as they are loaded.
 int q4k_gemv_i8(const char* op, const float* A, const uint8_t* W, const uint8_t* W2, void* C, int c_f16,
                 const float* residual, int M, int N, int K, float alpha, int activation, float clamp_max,
-                const float* norm_weight, float norm_eps, int norm_weight_offset);
+                const float* norm_weight, float norm_eps, int norm_weight_offset, int a_f16 = 0);
 // The same product for up to 8 activation rows in one pass over the weights, on the f16 matrix cores
 // (q4k_gemv_rows.hip).  Same arguments and return values.
 int q4k_gemv_rows(const char* op, const float* A, const uint8_t* W, const uint8_t* W2, void* C, int c_f16,
                   const float* residual, int M, int N, int K, float alpha, int activation, float clamp_max,
-                  const float* norm_weight, float norm_eps, int norm_weight_offset);
+                  const float* norm_weight, float norm_eps, int norm_weight_offset, int a_f16 = 0);
 
 }  // namespace dh
 

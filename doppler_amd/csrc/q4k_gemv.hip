@@ -1014,6 +1014,30 @@ int dh_q4k_matmul(const void* d_A, int a_dtype, const void* d_W, void* d_C, int 
     if (!d_A || !d_W || !d_C) return dh::fail(1, "[%s] null pointer", op);
     if (c_dtype != DH_F32 && c_dtype != DH_F16)
       return dh::fail(1, "[%s] output dtype must be f32 or f16 (c_dtype=%d)", op, c_dtype);
+    if (M < 16 && gemv_path() == 0) {
+      // below the GEMM's batch size the GEMV kernels load the f16 rows themselves (K a multiple of 4 and
+      // 8-byte aligned rows; otherwise they decline and the rows are widened first)
+      if (reinterpret_cast<uintptr_t>(d_W) & 15)
+        return dh::fail(1, "[%s] weight pointer must be 16-byte aligned", op);
+      const uint16_t* A16 = static_cast<const uint16_t*>(d_A);
+      const float* res = static_cast<const float*>(d_residual);
+      const int c_f16 = c_dtype == DH_F16;
+      int rc = -1;
+      if (M <= 2)
+        rc = dh::q4k_gemv_i8(op, reinterpret_cast<const float*>(A16), static_cast<const uint8_t*>(d_W), nullptr, d_C, c_f16,
+                             res, M, N, K, alpha, 0, 0.f, nullptr, 0.f, 0, 1);
+      if (rc < 0) {
+        rc = 0;
+        for (int m0 = 0; m0 < M && rc == 0; m0 += 8) {
+          rc = dh::q4k_gemv_rows(op, reinterpret_cast<const float*>(A16 + (int64_t)m0 * K), static_cast<const uint8_t*>(d_W),
+                                 nullptr, static_cast<char*>(d_C) + (int64_t)m0 * N * (c_f16 ? 2 : 4), c_f16,
+                                 res ? res + (int64_t)m0 * N : nullptr, std::min(8, M - m0), N, K, alpha, 0, 0.f, nullptr, 0.f,
+                                 0, 1);
+          if (rc < 0 && m0 > 0) return dh::fail(2, "[%s] internal: GEMV pass %d did not launch after pass 0 did", op, m0 / 8);
+        }
+      }
+      if (rc >= 0) return rc;
+    }
     size_t bytes = 0;
     float* wide = dh::widened_activations(&bytes);
     int64_t rows_per_pass = (int64_t)(bytes / sizeof(float)) / K;

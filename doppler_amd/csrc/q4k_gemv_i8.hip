@@ -29,6 +29,7 @@
 // is one at the very start.
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 #include "dh_common.h"
 #include "q4k_device.h"
@@ -43,6 +44,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 
 constexpr int kWaves = 16;
 constexpr int kTileRows = 16;
@@ -76,13 +78,14 @@ __device__ __forceinline__ void wait_vm_at_most(int n) {
 }
 
 struct I8Args {
-  const float* A;        // [M][K]
+  const float* A;        // [M][K] f32, or f16 in the AF16 kernels (a_f16 set)
   const uint8_t* W;      // Q4_K rows
   const uint8_t* W2;     // second matrix (DUAL) or null
   void* C;               // [M][N] f32 or f16
   const float* residual; // [M][N] or null
   const float* norm_weight;   // RMSNorm prologue (null = off)
   int M, N, K, nb;
+  int a_f16;             // the activations are f16 (widened exactly as they are loaded)
   int depth;             // ring stages per wave
   int rows;              // weight rows per tile (<= 16), chosen so that the tiles divide evenly among the workgroups
   int nlw;               // load instructions per unit: ceil(9 * rows / 64)
@@ -112,7 +115,7 @@ __device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
 //   red    [nslots][upt][MT][16] partial sums of a tile's units
 //   ctr    [0] next unit to draw, [1 + s] units delivered to slot s, [1 + nslots + s] tiles completed
 //          in slot s, [1 + 2 nslots + c] column c's operands are in place, [1 + 2 nslots + nb] a wave has given up
-template <int MT, bool DUAL, bool VEC>
+template <int MT, bool DUAL, bool VEC, bool AF16 = false>
 __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Args a) {
   constexpr int NMAT = DUAL ? 2 : 1;
   extern __shared__ __align__(16) unsigned char lds[];
@@ -194,7 +197,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
   const int kg = lane >> 4;
   constexpr int SC = MT == 1 ? 3 : (MT == 2 ? 2 : 1);    // columns per pass (all loads of a pass in flight at once)
   const int my_cols = wave < nb ? (nb - wave + kWaves - 1) >> 4 : 0;
-  v4f xr[SC][MT], wr[SC];
+  // (f16 activations: the lane's four elements are two registers, widened after the wait)
+  using XRaw = std::conditional_t<AF16, v2u, v4f>;
+  XRaw xr[SC][MT];
+  v4f wr[SC];
 #define DH_LOAD_X(c0_)                                                                            \
   do {                                                                                            \
     _Pragma("unroll") for (int i = 0; i < SC; i++) {                                              \
@@ -203,8 +209,13 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
         if constexpr (VEC) {                                                                      \
           const int kc = k0 < a.K ? k0 : 0;                                                       \
           _Pragma("unroll") for (int m = 0; m < MT; m++) {                                        \
-            const float* p_ = a.A + (int64_t)min(m, a.M - 1) * a.K + kc;                          \
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(xr[i][m]) : "v"(p_) : "memory"); \
+            if constexpr (AF16) {                                                                 \
+              const uint16_t* p_ = reinterpret_cast<const uint16_t*>(a.A) + (int64_t)min(m, a.M - 1) * a.K + kc; \
+              asm volatile("global_load_dwordx2 %0, %1, off" : "=&v"(xr[i][m]) : "v"(p_) : "memory"); \
+            } else {                                                                              \
+              const float* p_ = a.A + (int64_t)min(m, a.M - 1) * a.K + kc;                        \
+              asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(xr[i][m]) : "v"(p_) : "memory"); \
+            }                                                                                     \
           }                                                                                       \
           if (norm) {                                                                             \
             const float* p_ = a.norm_weight + kc;                                                 \
@@ -213,8 +224,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
         } else {                                                                                  \
           _Pragma("unroll") for (int e = 0; e < 4; e++) {                                         \
             const int kc = min(k0 + e, a.K - 1);                                                  \
-            _Pragma("unroll") for (int m = 0; m < MT; m++)                                        \
-              xr[i][m][e] = a.A[(int64_t)min(m, a.M - 1) * a.K + kc];                             \
+            if constexpr (!AF16) {                                                                \
+              _Pragma("unroll") for (int m = 0; m < MT; m++)                                      \
+                xr[i][m][e] = a.A[(int64_t)min(m, a.M - 1) * a.K + kc];                           \
+            }                                                                                     \
             if (norm) wr[i][e] = a.norm_weight[kc];                                               \
           }                                                                                       \
         }                                                                                         \
@@ -285,7 +298,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
             float v[4], ss = 0.f;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-              v[e] = (m < a.M && col * kQK + 4 * lane + e < a.K) ? xr[i][m][e] : 0.f;
+              float raw;
+              if constexpr (AF16) raw = (e & 1) ? f16hi(xr[i][m][e >> 1]) : f16lo(xr[i][m][e >> 1]);
+              else raw = xr[i][m][e];
+              v[e] = (m < a.M && col * kQK + 4 * lane + e < a.K) ? raw : 0.f;
               if (norm) {
                 ss = fmaf(v[e], v[e], ss);
                 v[e] *= a.norm_weight_offset ? 1.0f + wr[i][e] : wr[i][e];
@@ -565,11 +581,11 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
 
 int env_int(const char* name, int dflt) { return dh::tuning_int(name, dflt); }
 
-template <int MT, bool DUAL, bool VEC>
+template <int MT, bool DUAL, bool VEC, bool AF16 = false>
 int launch_i8_vec(I8Args a, const char* op) {
   constexpr int NMAT = DUAL ? 2 : 1;
   size_t cap = kMaxLds;
-  auto kern = q4k_gemv_i8_kernel<MT, DUAL, VEC>;
+  auto kern = q4k_gemv_i8_kernel<MT, DUAL, VEC, AF16>;
   static const int env_depth = env_int("DH_GEMV_DEPTH", 0);
   const int ncu = dh::num_cus();
   // rows per tile: the largest count <= 16 that gives every workgroup the same number of tiles
@@ -628,6 +644,15 @@ int launch_i8_vec(I8Args a, const char* op) {
 // Fast path: K a multiple of 4 and 16-byte aligned rows (vector loads of the activations).
 template <int MT, bool DUAL>
 int launch_i8(const I8Args& a, const char* op) {
+  if (a.a_f16) {
+    // f16 rows: only the single-matrix product without a norm prologue, K a multiple of 4 and 8-byte
+    // aligned rows; anything else is left to the caller (which widens the rows first)
+    if constexpr (!DUAL) {
+      if ((a.K & 3) == 0 && (reinterpret_cast<uintptr_t>(a.A) & 7) == 0 && !a.norm_weight)
+        return launch_i8_vec<MT, false, true, true>(a, op);
+    }
+    return -1;
+  }
   const bool vec = (a.K & 3) == 0 && (reinterpret_cast<uintptr_t>(a.A) & 15) == 0 &&
                    (!a.norm_weight || (reinterpret_cast<uintptr_t>(a.norm_weight) & 15) == 0);
   return vec ? launch_i8_vec<MT, DUAL, true>(a, op) : launch_i8_vec<MT, DUAL, false>(a, op);
@@ -661,7 +686,8 @@ int dispatch_i8(const I8Args& a, const char* op) {
   for (int m0 = 0; m0 < a.M; m0 += mt) {
     I8Args b = a;
     b.M = std::min(mt, a.M - m0);
-    b.A = a.A + (int64_t)m0 * a.K;
+    b.A = a.a_f16 ? reinterpret_cast<const float*>(reinterpret_cast<const uint16_t*>(a.A) + (int64_t)m0 * a.K)
+                  : a.A + (int64_t)m0 * a.K;
     b.C = static_cast<char*>(a.C) + (int64_t)m0 * a.N * c_elem;
     b.residual = a.residual ? a.residual + (int64_t)m0 * a.N : nullptr;
     const int rc = launch_mt<DUAL>(mt, b, op);
@@ -676,7 +702,7 @@ namespace dh {
 
 int q4k_gemv_i8(const char* op, const float* A, const uint8_t* W, const uint8_t* W2, void* C, int c_f16,
                 const float* residual, int M, int N, int K, float alpha, int activation, float clamp_max,
-                const float* norm_weight, float norm_eps, int norm_weight_offset) {
+                const float* norm_weight, float norm_eps, int norm_weight_offset, int a_f16) {
   static const int off = env_int("DH_GEMV_I8_OFF", 0);
   // three and more activation rows stay with the f16 matrix-core kernel of q4k_gemv.hip: their
   // operands (832 bytes per row and column) crowd the LDS and the per-row epilogue outweighs the
@@ -685,6 +711,7 @@ int q4k_gemv_i8(const char* op, const float* A, const uint8_t* W, const uint8_t*
   I8Args a{};
   a.A = A; a.W = W; a.W2 = W2; a.C = C; a.residual = residual;
   a.M = M; a.N = N; a.K = K; a.nb = (K + kQK - 1) / kQK;
+  a.a_f16 = a_f16;
   a.alpha = alpha; a.c_f16 = c_f16; a.activation = activation; a.clamp_max = clamp_max;
   a.norm_weight = norm_weight; a.norm_eps = norm_eps; a.norm_weight_offset = norm_weight_offset;
   a.status = dh::kernel_status_word();

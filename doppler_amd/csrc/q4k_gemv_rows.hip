@@ -26,6 +26,7 @@
 // matrix); after one barrier at the end the sixteen waves' accumulators are added in wave order
 // (deterministic) and the outputs written.
 #include <algorithm>
+#include <type_traits>
 #include <cstdlib>
 
 #include "dh_common.h"
@@ -71,7 +72,7 @@ __device__ __forceinline__ void wait_vm_at_most(int n) {
 }
 
 struct RowsArgs {
-  const float* A;        // [M][K]
+  const float* A;        // [M][K] f32, or f16 in the AF16 kernels
   const uint8_t* W;      // Q4_K rows
   const uint8_t* W2;     // second matrix (DUAL) or null
   void* C;               // [M][N] f32 or f16
@@ -135,7 +136,7 @@ struct ColOps {
 //   wn    [16 waves][256] floats: RMSNorm weights of the column being converted (norm prologue only)
 //   ssq   [16 waves][kSsqFloats]: the wave's sum of squares of activation row r at r
 //   acc   [16 waves][acc_max][64 lanes][2]: lane (j, kg) keeps weight row j x activation rows 2 kg, 2 kg + 1
-template <bool DUAL, bool VEC>
+template <bool DUAL, bool VEC, bool AF16 = false>
 __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const RowsArgs a) {
   constexpr int NMAT = DUAL ? 2 : 1;
   extern __shared__ __align__(16) unsigned char lds[];
@@ -208,13 +209,19 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
   const int xk = 8 * kg + 4 * part;             // offset of the lane's 4 activations inside a sub-block
   const bool row_ok = xrow < a.M;
   const float* xbase = a.A + (int64_t)min(xrow, a.M - 1) * a.K;
-  const uint32_t xrow_off = 4u * (uint32_t)(min(xrow, a.M - 1) * a.K);     // M K stays far below 2^30 (M <= 8)
+  // (f16 rows: two bytes per element, the lane's four elements are two registers, widened where they are converted)
+  constexpr uint32_t XB = AF16 ? 2u : 4u;
+  using XRaw = std::conditional_t<AF16, v2u, v4f>;
+  const uint32_t xrow_off = XB * (uint32_t)(min(xrow, a.M - 1) * a.K);     // M K stays far below 2^30 (M <= 8)
   const uint32_t wn_lane = (uint32_t)(uintptr_t)DH_LDS_PTR(wn + wave * kQK) + 4 * xk;   // this lane's norm weights of sub-block 0
 #define DH_LOAD_X_ONE(xr_, col_, s_)                                                              \
   do {                                                                                            \
     const int k_ = (col_) * kQK + 32 * (s_) + xk;                                                 \
-    if constexpr (VEC) {                                                                          \
-      const uint32_t o_ = xrow_off + 4u * (uint32_t)min(k_, a.K - 4);                             \
+    if constexpr (AF16) {                                                                         \
+      const uint32_t o_ = xrow_off + XB * (uint32_t)min(k_, a.K - 4);                             \
+      asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"((xr_)[s_]) : "v"(o_), "s"(a.A) : "memory"); \
+    } else if constexpr (VEC) {                                                                   \
+      const uint32_t o_ = xrow_off + XB * (uint32_t)min(k_, a.K - 4);                             \
       asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"((xr_)[s_]) : "v"(o_), "s"(a.A) : "memory"); \
     } else {                                                                                      \
       _Pragma("unroll") for (int e = 0; e < 4; e++) (xr_)[s_][e] = xbase[min(k_ + e, a.K - 1)];   \
@@ -232,7 +239,16 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
   float ssq = 0.f;                              // this lane's share of the sum of squares of row xrow
   // Turns the raw activations xr of column col into operands.  count: the column's squares go into
   // this wave's sum (the wave that holds the column's first unit counts them).
-  auto convert = [&](v4f (&xr)[8], const int col, const bool count, ColOps& out) __attribute__((always_inline)) {
+  auto convert = [&](XRaw (&xraw)[8], const int col, const bool count, ColOps& out) __attribute__((always_inline)) {
+    v4f xwide[8];
+    if constexpr (AF16) {
+#pragma unroll
+      for (int s = 0; s < 8; s++)
+        xwide[s] = v4f{f16lo(xraw[s].x), f16hi(xraw[s].x), f16lo(xraw[s].y), f16hi(xraw[s].y)};
+    }
+    v4f (&xr)[8] = *[&]() {
+      if constexpr (AF16) return &xwide; else return &xraw;
+    }();
     const bool tail = col * kQK + kQK > a.K;          // the column reaches past K: those elements count as zero
     float mx = 0.f;
     if (norm) {
@@ -357,7 +373,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
   cur.xm = 0u;
   cur.xinv0 = cur.xinv1 = 0.f;
   if (nun > 0) {
-    v4f xr[8];
+    XRaw xr[8];
 #pragma unroll
     for (int s = 0; s < 8; s++) DH_LOAD_X_ONE(xr, colc, s);
     DH_LOAD_NORM_WEIGHTS(colc);
@@ -385,7 +401,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
   // multiplied and converted at the end.
   auto unit = [&](auto sw_tag, const int coln) __attribute__((always_inline)) {
     constexpr bool SW = decltype(sw_tag)::value;
-    v4f xr[8];
+    XRaw xr[8];
     wait_vm_at_most((issued - consumed - 1) * a.nlw);
     const uint32_t hp = lane_hdr + cstage * kStage, qp = lane_q + cstage * kStage;
     v4u h;
@@ -534,10 +550,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
 
 int env_int(const char* name, int dflt) { return dh::tuning_int(name, dflt); }
 
-template <bool DUAL, bool VEC>
+template <bool DUAL, bool VEC, bool AF16 = false>
 int launch_rows(RowsArgs a, const char* op) {
   constexpr int NMAT = DUAL ? 2 : 1;
-  auto kern = q4k_gemv_rows_kernel<DUAL, VEC>;
+  auto kern = q4k_gemv_rows_kernel<DUAL, VEC, AF16>;
   const int ncu = dh::num_cus();
   // rows per tile: the largest count <= 16 that gives every workgroup the same number of tiles
   const int per_cu = (int)dh::ceil_div(a.N, (int64_t)ncu * kTileRows);
@@ -585,7 +601,7 @@ namespace dh {
 
 int q4k_gemv_rows(const char* op, const float* A, const uint8_t* W, const uint8_t* W2, void* C, int c_f16,
                   const float* residual, int M, int N, int K, float alpha, int activation, float clamp_max,
-                  const float* norm_weight, float norm_eps, int norm_weight_offset) {
+                  const float* norm_weight, float norm_eps, int norm_weight_offset, int a_f16) {
   static const int off = env_int("DH_GEMV_ROWS_OFF", 0);
   if (off || M < 1 || M > 8) return -1;
   RowsArgs a{};
@@ -595,6 +611,11 @@ int q4k_gemv_rows(const char* op, const float* A, const uint8_t* W, const uint8_
   a.norm_weight = norm_weight; a.norm_eps = norm_eps; a.norm_weight_offset = norm_weight_offset;
   const bool vec = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0 &&
                    (!norm_weight || (reinterpret_cast<uintptr_t>(norm_weight) & 15) == 0);
+  if (a_f16) {
+    // f16 rows: the single-matrix product without a norm prologue, K a multiple of 4, 8-byte aligned rows
+    if (W2 || norm_weight || (K & 3) != 0 || (reinterpret_cast<uintptr_t>(A) & 7) != 0) return -1;
+    return launch_rows<false, true, true>(a, op);
+  }
   if (W2) return vec ? launch_rows<true, true>(a, op) : launch_rows<true, false>(a, op);
   return vec ? launch_rows<false, true>(a, op) : launch_rows<false, false>(a, op);
 }

@@ -114,8 +114,9 @@ int dh_q4k_dequant(const void* d_W, int64_t num_blocks, float* d_out);
  * (kernels fused_matmul_q4.wgsl:122-258, fused_matmul_q4_batched.wgsl:123-194,
  * fused_matmul_q4_prefill_tiled_f16.wgsl:119-261; f16 activations: fused_matmul_q4_f16a.wgsl,
  * fused_matmul_q4_batched_f16a.wgsl, selected at matmul-selection.js:24-27).  A is f32 or f16
- * (a_dtype); f16 rows are widened exactly into a 64 MB f32 staging area of the library, in
- * passes when they do not fit, and the product accumulates in f32 either way.  C is f32 or
+ * (a_dtype); up to 15 f16 rows are loaded as they are by the GEMV kernels and widened (exactly) in registers
+ * (K a multiple of 4, rows 8-byte aligned); otherwise they are widened into a 64 MB f32 staging area of the
+ * library first, in passes when they do not fit.  The product accumulates in f32 either way.  C is f32 or
  * f16 (c_dtype); the residual is f32.  K need not be a multiple of 256: the padded tail of each row's last
  * block is ignored.  d_residual (may be NULL) is added after alpha, as the reference's
  * `residualTensor` option does.  M = 1..15 takes an HBM-bound GEMV path, M >= 16 the

@@ -89,7 +89,11 @@ def _matmul_case(M, N, K, seed, alpha=1.0, outputDtype="f32", residual=False):
 @pytest.mark.parametrize("M,N,K,outputDtype,residual", [
     (4, 6144, 1536, "f16", False),      # the shape of the reference's f16-activation parity test
     (1, 1024, 4096, "f16", False), (1, 4096, 4096, "f32", True), (8, 512, 1152, "f32", False),
-    (12, 96, 300, "f16", True), (33, 257, 2048, "f32", True)])
+    (12, 96, 300, "f16", True), (33, 257, 2048, "f32", True),
+    # rows loaded as f16 by the decode kernels themselves: one and two rows (int8 kernel, K with a partial last
+    # column too), three to eight and two passes of them (rows kernel)
+    (2, 4096, 4096, "f16", True), (2, 1024, 1156, "f32", False), (1, 12288, 4096, "f32", False),
+    (5, 4096, 3204, "f32", True), (8, 4096, 4096, "f16", False), (13, 4096, 3072, "f32", True)])
 def test_matmul_f16_activations(M, N, K, outputDtype, residual):
     """f16 activations (tests/kernels/fused-matmul-q4-widetile-f16a-parity.test.js runs M=4, K=1536,
     N=6144): the product of the exactly widened rows, accumulated in f32."""
@@ -111,6 +115,24 @@ def test_matmul_f16_activations(M, N, K, outputDtype, residual):
     same = ops.readTensor(ops.runMatmul(ops.tensorFromNumpy(A16.astype(np.float32)), wb, M, N, K, outputDtype=outputDtype,
                                         role="test", residualTensor=ops.tensorFromNumpy(res) if residual else None))
     assert same.tobytes() == ops.readTensor(out).tobytes()
+
+
+@pytest.mark.parametrize("M", [1, 4])
+def test_matmul_f16_activations_at_an_odd_address(M):
+    """Rows that start 2 bytes past an 8-byte boundary cannot be loaded four elements at a time: the
+    library widens them first, and the product is the same."""
+    import torch
+    N, K = 4096, 4096
+    W, wb = q4k_weight(N, K, 1170 + M)
+    A16 = synth.normal_f32((M, K), 1171 + M).astype(np.float16)
+    buf = torch.zeros(M * K + 8, dtype=torch.float16, device="cuda")
+    buf[1:1 + M * K] = torch.from_numpy(A16.reshape(-1)).cuda()
+    out = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    capi.check(capi.init(0).dh_q4k_matmul(buf.data_ptr() + 2, capi.F16, wb.buffer.data_ptr(), out.data_ptr(), capi.F32,
+                                          M, N, K, 1.0, None))
+    capi.check(capi.init(0).dh_sync())
+    want = oracle.q4k_matmul(A16.astype(np.float32), W, M, N, K)
+    assert rel_l2(out.cpu().numpy().reshape(M, N), want) <= matmul_bar(M)
 
 
 def test_matmul_f16_activations_errors():
