@@ -125,8 +125,8 @@ def js_reference_timings():
 
 def js_host_decode(cfg, layers, embed, final_norm, prefill, warmup, steps):
     """Decode tokens/s of the JavaScript host on the same model: node subprocess over
-    doppler_amd/js/bench/decode_bench.mjs (loader -> prefill -> decodeStep loop, then the
-    captured-graph loop).  Returns its JSON, or None when node or the addon is missing."""
+    doppler_amd/js/bench/decode_bench.mjs (loader -> prefill -> decodeStep loop with a blocking readback per
+    step, the same positions through decodeGreedy's staged readback, then the captured-graph loop).  Returns its JSON, or None when node or the addon is missing."""
     import shutil
     import subprocess
     import tempfile
@@ -148,7 +148,8 @@ def js_host_decode(cfg, layers, embed, final_norm, prefill, warmup, steps):
             log("[bench] JS host failed: %s" % r.stderr[-2000:])
             return None
         res = json.loads(r.stdout.strip().splitlines()[-1])
-        for k in ("tokens_per_s", "ms_per_step", "graph_tokens_per_s", "graph_ms_per_step"):
+        for k in ("tokens_per_s", "ms_per_step", "graph_tokens_per_s", "graph_ms_per_step", "greedy_tokens_per_s",
+                  "greedy_ms_per_step"):
             if k in res:
                 res[k] = round(res[k], 3)
         return res

@@ -153,6 +153,27 @@ FN(js_event_elapsed_ms) {
   return ret_num(env, ms);
 }
 FN(js_event_destroy) { ARGS(1); P(0, e); return ret_rc(env, dh_event_destroy(e)); }
+FN(js_event_synchronize) { ARGS(1); P(0, e); return ret_rc(env, dh_event_synchronize(e)); }
+/* hostAlloc(bytes) -> {ptr: BigInt, view: ArrayBuffer over the pinned memory (valid until hostFree(ptr))} */
+FN(js_host_alloc) {
+  ARGS(1); L(0, bytes);
+  void* p = NULL;
+  if (dh_host_alloc((size_t)bytes, &p) != 0) return fail(env, dh_last_error());
+  napi_value obj, view;
+  if (napi_create_external_arraybuffer(env, p, (size_t)bytes, NULL, NULL, &view) != napi_ok || napi_create_object(env, &obj) != napi_ok) {
+    dh_host_free(p);
+    return fail(env, "doppler_hip: could not wrap the pinned memory");
+  }
+  napi_set_named_property(env, obj, "ptr", ret_ptr(env, p));
+  napi_set_named_property(env, obj, "view", view);
+  return obj;
+}
+FN(js_host_free) { ARGS(1); P(0, p); return ret_rc(env, dh_host_free(p)); }
+/* downloadAsync(hostPtr, hostOffset, src, srcOffset, bytes): enqueued behind the ops so far, returns at once */
+FN(js_download_async) {
+  ARGS(5); P(0, h); L(1, hoff); P(2, src); L(3, off); L(4, bytes);
+  return ret_rc(env, dh_download_async((char*)h + hoff, src, (size_t)off, (size_t)bytes));
+}
 
 /* ---- ops (argument order = the C ABI's) ---- */
 FN(js_q4k_dequant) { ARGS(3); P(0, w); L(1, nb); P(2, o); return ret_rc(env, dh_q4k_dequant(w, nb, (float*)o)); }
@@ -377,6 +398,8 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"init", js_init}, {"shutdown", js_shutdown}, {"sync", js_sync}, {"malloc", js_malloc}, {"free", js_free},
       {"upload", js_upload}, {"download", js_download}, {"copy", js_copy}, {"fillZero", js_fill_zero},
       {"eventCreate", js_event_create}, {"eventRecord", js_event_record}, {"eventElapsedMs", js_event_elapsed_ms},
+      {"eventSynchronize", js_event_synchronize}, {"hostAlloc", js_host_alloc}, {"hostFree", js_host_free},
+      {"downloadAsync", js_download_async},
       {"eventDestroy", js_event_destroy}, {"q4kDequant", js_q4k_dequant}, {"q4kMatmul", js_q4k_matmul},
       {"q4kFfnGateUp", js_q4k_ffn_gate_up}, {"f16wMatmul", js_f16w_matmul},
       {"q4kMatmulRmsnorm", js_q4k_matmul_rmsnorm}, {"q4kFfnGateUpRmsnorm", js_q4k_ffn_gate_up_rmsnorm},

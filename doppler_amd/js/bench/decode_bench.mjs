@@ -1,6 +1,6 @@
 // Decode throughput of the JavaScript host: RDRR artifact -> JS loader -> HIP buffers -> prefill
-// path -> timed decode loop through the op API (N-API addon -> C ABI), one 4-byte token readback
-// per step.  Prints one JSON line.
+// path -> timed decode loops through the op API (N-API addon -> C ABI): one blocking 4-byte token readback
+// per step, then the generation loop with staged readback, then (graph) the captured step.  Prints one JSON line.
 //   node doppler_amd/js/bench/decode_bench.mjs <artifact-dir> <prefill> <warmup> <steps> [graph]
 import { initDevice } from '../kernel-selector.js';
 import { HipTextDecoder } from '../pipeline/decode-step.js';
@@ -33,11 +33,19 @@ async function main() {
   let pos = prefill;
   for (let i = 0; i < warmup; i++) tok = await dec.decodeStep(tok, pos++);
   const eager = await timed(dec, (t, p) => dec.decodeStep(t, p), tok, pos);
+  // the same positions again through the generation loop with staged readback (step k + 1 is enqueued from
+  // the device-side token before the host waits for token k): the tokens must be the same
+  await dec.decodeGreedy(tok, pos, Math.min(4, steps));
+  const g0 = process.hrtime.bigint();
+  const greedy = await dec.decodeGreedy(tok, pos, steps);
+  const greedySeconds = Number(process.hrtime.bigint() - g0) / 1e9;
   pos += steps;
   const out = {
     host: 'javascript (node ' + process.version + ') -> N-API addon -> C ABI',
     tokens_per_s: steps / eager.seconds, ms_per_step: eager.seconds / steps * 1e3, load_ms: loadMs,
     tokens_head: eager.tokens.slice(0, 4),
+    greedy_tokens_per_s: steps / greedySeconds, greedy_ms_per_step: greedySeconds / steps * 1e3,
+    greedy_matches_blocking_steps: JSON.stringify(greedy) === JSON.stringify(eager.tokens),
   };
   if (mode === 'graph') {
     tok = await dec.captureDecodeStep(eager.tok, pos++);

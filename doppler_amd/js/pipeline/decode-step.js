@@ -33,6 +33,11 @@ function upload(bytes, label) {
   return buf;
 }
 
+// decodeGreedy: tokens in flight between the device and the host (ring slots), and the events that mark
+// their copies
+const TOKEN_RING = 64;
+const READ_EVENTS = 4;
+
 export class HipTextDecoder {
   // config: {layers, hidden, inter, heads, kvHeads, headDim, vocab, eps, maxSeq}
   //   finitenessGuard (default false): check every layer's output against finitenessAbsThreshold
@@ -77,21 +82,22 @@ export class HipTextDecoder {
     this.finitenessAbsThreshold = resolveFinitenessAbsThreshold(config.finitenessAbsThreshold);
     this.finitenessStatus = bufferWindow(this.tokenOut, 4, FINITENESS_STATUS_BYTES);
     this.logits = null;
+    this.readback = null;
   }
 
   // Final RMSNorm + LM head for one hidden row; greedy, or top-k temperature sampling when
   // `sampling` = {temperature, topK, randomSeed} is given (the logits then go through memory).
-  async recordHead(recorder, temps, hiddenRow, sampling) {
+  async recordHead(recorder, temps, hiddenRow, sampling, tokenOut = this.tokenOut, tokenIndex = 0) {
     const c = this.config;
     const normed = await recordRMSNorm(recorder, hiddenRow, this.finalNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden });
     temps.push(normed.buffer);
     if (sampling && !this.logits) this.logits = acquireBuffer(c.vocab * 4, undefined, 'logits');
     await recordLmHeadArgmaxF16(recorder, normed, this.embed, {
-      vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: this.tokenOut, outputIndex: 0,
+      vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: tokenOut, outputIndex: tokenIndex,
       logitsOutput: sampling ? this.logits : null,
     });
     if (sampling) {
-      await recordGPUSample(recorder, this.logits, c.vocab, Object.assign({ outputBuffer: this.tokenOut, outputIndex: 0 }, sampling));
+      await recordGPUSample(recorder, this.logits, c.vocab, Object.assign({ outputBuffer: tokenOut, outputIndex: tokenIndex }, sampling));
     }
   }
 
@@ -181,6 +187,8 @@ export class HipTextDecoder {
 
   // Records the ops of one decode step for the token id in this.ids at position `pos`; the new
   // token id goes to this.tokenOut.  Temporaries are pushed onto `temps`.
+  // options.idsBuffer: the input token id is read from this device word instead; options.tokenOutBuffer /
+  // tokenOutIndex: the new token goes to that word of that buffer instead.
   async recordDecodeStep(recorder, temps, pos, options = {}) {
     const c = this.config;
     if (!(pos >= 0 && pos < c.maxSeq)) {
@@ -188,7 +196,8 @@ export class HipTextDecoder {
       throw new Error(`[decodeStep] position ${pos} is outside the KV cache (maxSeq=${c.maxSeq})`);
     }
     const temp = (t) => { temps.push(t.buffer); return t; };
-    let x = temp(await recordGather(recorder, this.ids, this.embed, 1, c.hidden, c.vocab,
+    const tokenOut = options.tokenOutBuffer || this.tokenOut, tokenIndex = options.tokenOutIndex || 0;
+    let x = temp(await recordGather(recorder, options.idsBuffer || this.ids, this.embed, 1, c.hidden, c.vocab,
       { embeddingDtype: 'f16', outputDtype: 'f32' }));
     if (this.chainGemvs) {
       x = await this.recordChainedLayers(recorder, temps, x, pos, options);
@@ -227,11 +236,11 @@ export class HipTextDecoder {
       }
     }
     if (options.sampling) {
-      await this.recordHead(recorder, temps, x, options.sampling);
+      await this.recordHead(recorder, temps, x, options.sampling, tokenOut, tokenIndex);
     } else {
       const finalNormed = temp(await recordRMSNorm(recorder, x, this.finalNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden }));
       await recordLmHeadArgmaxF16(recorder, finalNormed, this.embed, {
-        vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: this.tokenOut, outputIndex: 0,
+        vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: tokenOut, outputIndex: tokenIndex,
         logitsOutput: options.logitsOutput || null,
       });
     }
@@ -295,6 +304,70 @@ export class HipTextDecoder {
     return words[0];
   }
 
+  // n greedy steps starting with `token` at position `pos`; returns the n new token ids.  Every step's
+  // token is read back (4 bytes per step, as in decodeStep), but one step late: step k + 1 takes its input
+  // token from device memory and is enqueued before the host waits for token k, whose copy into pinned
+  // memory was enqueued behind step k, so the GPU never waits for the host between steps (the reference
+  // stages its token readbacks through a ring the same way, src/inference/decode-ring.js:141-177).  A
+  // caller with a stop condition checks the tokens as they come and drops the one step in flight.
+  async decodeGreedy(token, pos, n) {
+    if (n <= 0) return [];
+    if (this.finitenessGuard) {
+      const guarded = [];
+      for (let k = 0; k < n; k++) {
+        token = await this.decodeStep(token, pos + k);
+        guarded.push(token);
+      }
+      return guarded;
+    }
+    const native = getNative();
+    if (!this.readback) {
+      const host = native.hostAlloc(4 * TOKEN_RING);
+      const events = [];
+      for (let i = 0; i < READ_EVENTS; i++) events.push(native.eventCreate());
+      this.readback = { host, tokens: new Uint32Array(host.view), events, ring: acquireBuffer(4 * TOKEN_RING, undefined, 'token_ring') };
+    }
+    const rb = this.readback;
+    const enqueueStep = async (k) => {
+      const recorder = createCommandRecorder('decode');
+      const temps = [];
+      const slot = k % TOKEN_RING;
+      const options = { tokenOutBuffer: rb.ring, tokenOutIndex: slot };
+      if (k > 0) options.idsBuffer = bufferWindow(rb.ring, 4 * ((k - 1) % TOKEN_RING), 4);
+      await this.recordDecodeStep(recorder, temps, pos + k, options);
+      for (const b of temps) recorder.trackTemporaryBuffer(b);
+      recorder.submit();
+      native.downloadAsync(rb.host.ptr, 4 * slot, rb.ring.ptr, 4 * slot, 4);
+      native.eventRecord(rb.events[k % READ_EVENTS]);
+    };
+    const waitToken = (k) => {
+      native.eventSynchronize(rb.events[k % READ_EVENTS]);
+      return rb.tokens[k % TOKEN_RING];
+    };
+    uploadData(this.ids, new Uint32Array([token]));
+    await enqueueStep(0);
+    const out = [];
+    for (let k = 1; k < n; k++) {
+      await enqueueStep(k);
+      out.push(waitToken(k - 1));
+    }
+    out.push(waitToken(n - 1));
+    return out;
+  }
+
+  // Frees the pinned staging memory, the device ring and the events decodeGreedy made.
+  releaseReadback() {
+    if (this.readback) {
+      const native = getNative();
+      native.sync();
+      for (const ev of this.readback.events) native.eventDestroy(ev);
+      this.readback.tokens = null;
+      native.hostFree(this.readback.host.ptr);
+      releaseBuffer(this.readback.ring);
+      this.readback = null;
+    }
+  }
+
   // Captures the decode step into a HIP graph, the counterpart of the reference's
   // one-submit-per-step recorder (generator-steps.js:605,814).  The step runs once normally first
   // (every kernel's one-time set-up then lies outside the capture); the buffers the captured step
@@ -351,6 +424,7 @@ export class HipTextDecoder {
 
   destroy() {
     this.releaseGraph();
+    this.releaseReadback();
     for (const l of this.layers) {
       for (const key of Object.keys(l)) releaseBuffer(l[key].buffer);
     }

@@ -214,6 +214,16 @@ async function main() {
       let tok = c.prompt[0];
       for (let pos = 0; pos < c.prompt.length + c.steps; pos++) {
         const inp = pos < c.prompt.length ? c.prompt[pos] : tok;
+        if (c.greedyFrom !== undefined && pos === c.greedyFrom) {
+          // the rest of the tokens from the generation loop with staged readback, twice (the second call
+          // reuses the pinned ring and overwrites the same KV rows with the same values)
+          const n = c.prompt.length + c.steps - pos;
+          const first = await dec.decodeGreedy(inp, pos, n);
+          const again = await dec.decodeGreedy(inp, pos, n);
+          results.errors.push({ label: `${c.name}-greedy-repeat`, ok: JSON.stringify(first) === JSON.stringify(again), message: JSON.stringify([first, again]) });
+          tokens.push(...first);
+          break;
+        }
         if (c.graphFrom !== undefined && pos >= c.graphFrom && pos % 5 !== 4) {
           // replay of the captured step (captured at the first such position), an eager step now and then
           tok = await dec.decodeStepGraph(inp, pos);
@@ -235,6 +245,7 @@ async function main() {
         tokens.push(tok);
       }
       dec.releaseGraph();
+      dec.releaseReadback();
       fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array(tokens).buffer));
     } else if (c.op === 'generate') {
       // RDRR artifact -> JS loader -> prefill path -> decode loop, greedy or sampled

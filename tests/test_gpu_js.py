@@ -370,6 +370,9 @@ def test_js_host_path_parity(tmp_path):
                       config=dict(layers=2, hidden=2048, inter=4096, heads=16, kvHeads=4, headDim=128, vocab=700, eps=1e-6, maxSeq=24)))
     cases.append(dict(cases[-1], name="decoder_chain_off", expectChained=False,
                       config=dict(cases[-1]["config"], chainGemvs=False)))
+    # the generation loop with staged token readback (decodeGreedy) from position 6 on, chained and not
+    for src, name in ((cases[-2], "decoder_chained_greedy"), (cases[-1], "decoder_chain_off_greedy")):
+        cases.append(dict({k: v for k, v in src.items() if k != "graphFrom"}, name=name, greedyFrom=6))
     col = []
     for l in clayers:
         dd = dict(l)
@@ -384,6 +387,8 @@ def test_js_host_path_parity(tmp_path):
     assert len(set(cwant)) > 2, cwant
     checks.append(lambda: [int(t) for t in get("decoder_chained.out.bin", np.uint32)] == cwant)
     checks.append(lambda: [int(t) for t in get("decoder_chain_off.out.bin", np.uint32)] == cwant)
+    checks.append(lambda: [int(t) for t in get("decoder_chained_greedy.out.bin", np.uint32)] == cwant)
+    checks.append(lambda: [int(t) for t in get("decoder_chain_off_greedy.out.bin", np.uint32)] == cwant)
 
     # ---- top-k temperature sampling through the JS op (seeded draw as in the reference)
     slog = (synth.rng(79).standard_normal(4000) * 3).astype(np.float32)
