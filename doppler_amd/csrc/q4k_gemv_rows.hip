@@ -203,7 +203,12 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
   // 256 col + 32 s + 8 kg + 4 part .. + 3 of its row.  The loads are hand-written instructions (scalar
   // base + 32-bit lane offset), so the compiler believes them complete at once: the raw registers
   // are declared where they are loaded and only straight-line code lies between the load and the
-  // wait, which leaves it no reason to move them earlier.
+  // wait, which leaves it no reason to move them earlier.  The s_nop in front of each load is not
+  // padding: a vector-memory instruction must not read a scalar register within five wait states of a
+  // vector instruction writing it (v_readlane restoring a spilled scalar, v_readfirstlane), the compiler
+  // keeps that distance only for instructions it emits itself, and a build under scalar-register
+  // pressure put such a restore of the activation pointer directly in front of one of these loads: the
+  // load then went to a wild address.
   const int kg = lane >> 4, j = lane & 15;
   const int xrow = j >> 1, part = j & 1;
   const int xk = 8 * kg + 4 * part;             // offset of the lane's 4 activations inside a sub-block
@@ -219,10 +224,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_rows_kernel(const Row
     const int k_ = (col_) * kQK + 32 * (s_) + xk;                                                 \
     if constexpr (AF16) {                                                                         \
       const uint32_t o_ = xrow_off + XB * (uint32_t)min(k_, a.K - 4);                             \
-      asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"((xr_)[s_]) : "v"(o_), "s"(a.A) : "memory"); \
+      asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %1, %2" : "=&v"((xr_)[s_]) : "v"(o_), "s"(a.A) : "memory"); \
     } else if constexpr (VEC) {                                                                   \
       const uint32_t o_ = xrow_off + XB * (uint32_t)min(k_, a.K - 4);                             \
-      asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"((xr_)[s_]) : "v"(o_), "s"(a.A) : "memory"); \
+      asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2" : "=&v"((xr_)[s_]) : "v"(o_), "s"(a.A) : "memory"); \
     } else {                                                                                      \
       _Pragma("unroll") for (int e = 0; e < 4; e++) (xr_)[s_][e] = xbase[min(k_ + e, a.K - 1)];   \
     }                                                                                             \
