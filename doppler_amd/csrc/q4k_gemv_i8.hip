@@ -195,7 +195,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
   // compute unit's memory queue.  (Fast path, K a multiple of 4 and 16-byte aligned rows: the loads
   // are hand-issued so that the first weight unit can follow them and only THEY are waited for.)
   const int kg = lane >> 4;
-  constexpr int SC = MT == 1 ? 3 : (MT == 2 ? 2 : 1);    // columns per pass (all loads of a pass in flight at once)
+  constexpr int SC = 3;    // columns per pass (all loads of a pass in flight at once)
   const int my_cols = wave < nb ? (nb - wave + kWaves - 1) >> 4 : 0;
   // (f16 activations: the lane's four elements are two registers, widened after the wait)
   using XRaw = std::conditional_t<AF16, v2u, v4f>;
@@ -508,13 +508,16 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
       const int tile = (int)blockIdx.x + tl * a.grid;
       const int64_t row = (int64_t)tile * a.rows + j;
       const uint32_t slot_abs = red_abs + (uint32_t)slot * upt * MT * 64;
-#pragma unroll 1
-      for (int m = 0; m < MT; m++) {
-        // lane (j, kg) adds columns kg, kg + 4, .. (four reads in flight at a time); the four
-        // groups then meet.  The order is fixed, so the result does not depend on who arrives last.
-        float sg = 0.f, su = 0.f;
-        for (int c = kg; c < nb; c += 16) {
-          float r[2][4];
+      // lane (j, kg) adds columns kg, kg + 4, .. of every activation row (four reads per row and matrix
+      // in flight at a time); the four groups then meet.  The order is fixed, so the result does not
+      // depend on who arrives last.
+      float sg[MT], su[MT];
+#pragma unroll
+      for (int m = 0; m < MT; m++) sg[m] = su[m] = 0.f;
+      for (int c = kg; c < nb; c += 16) {
+        float r[MT][2][4];
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
 #pragma unroll
           for (int mt = 0; mt < NMAT; mt++) {
             const uint32_t p = slot_abs + (((mt * nb + c) * MT + m) * 16 + j) * 4;
@@ -523,42 +526,52 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
                 "ds_read_b32 %1, %4 offset:%5\n\t"
                 "ds_read_b32 %2, %4 offset:%6\n\t"
                 "ds_read_b32 %3, %4 offset:%7"
-                : "=&v"(r[mt][0]), "=&v"(r[mt][1]), "=&v"(r[mt][2]), "=&v"(r[mt][3])
+                : "=&v"(r[m][mt][0]), "=&v"(r[m][mt][1]), "=&v"(r[m][mt][2]), "=&v"(r[m][mt][3])
                 : "v"(p), "n"(4 * MT * 64), "n"(8 * MT * 64), "n"(12 * MT * 64)
                 : "memory");
           }
-          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]) :: "memory");
-          if (DUAL) asm volatile("" : "+v"(r[NMAT - 1][0]), "+v"(r[NMAT - 1][1]), "+v"(r[NMAT - 1][2]), "+v"(r[NMAT - 1][3]));
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+          asm volatile("" : "+v"(r[m][0][0]), "+v"(r[m][0][1]), "+v"(r[m][0][2]), "+v"(r[m][0][3]));
+          if (DUAL) asm volatile("" : "+v"(r[m][NMAT - 1][0]), "+v"(r[m][NMAT - 1][1]), "+v"(r[m][NMAT - 1][2]), "+v"(r[m][NMAT - 1][3]));
 #pragma unroll
           for (int i = 0; i < 4; i++) {
             const bool ok = c + 4 * i < nb;       // columns past the last read whatever follows: dropped
-            sg += ok ? r[0][i] : 0.f;
-            if (DUAL) su += ok ? r[NMAT - 1][i] : 0.f;
+            sg[m] += ok ? r[m][0][i] : 0.f;
+            if (DUAL) su[m] += ok ? r[m][NMAT - 1][i] : 0.f;
           }
         }
-        sg = sum_lane_groups(sg);
-        if (DUAL) su = sum_lane_groups(su);
+      }
+      if (norm && !have_rms) {
+        // every column has been consumed by now, so every column's sum of squares is in place: lane l
+        // takes columns l, l + 64, .. (one LDS read each, all lanes at once), then the lanes meet in a
+        // fixed order
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+          float part = 0.f;
+          for (int c = lane; c < nb; c += 64) part += __uint_as_float(lds_read_u32(xq_abs + (uint32_t)(c * MT + m) * kRec + kRecSsq));
+          const float tot = dh::wave_sum_uniform(part);
+          inv_rms[m] = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < MT; m++) {
+        float g = sum_lane_groups(sg[m]), u = 0.f;
+        if (DUAL) u = sum_lane_groups(su[m]);
         if (norm) {
-          if (!have_rms) {
-            // every column has been consumed by now, so every column's sum of squares is in place: lane l
-            // takes columns l, l + 64, .. (one LDS read each, all lanes at once), then the lanes meet in a
-            // fixed order
-            float part = 0.f;
-            for (int c = lane; c < nb; c += 64) part += __uint_as_float(lds_read_u32(xq_abs + (uint32_t)(c * MT + m) * kRec + kRecSsq));
-            const float tot = dh::wave_sum_uniform(part);
-            inv_rms[m] = 1.0f / sqrtf(tot / (float)a.K + a.norm_eps);
-          }
-          sg *= inv_rms[m];
-          su *= inv_rms[m];
+          g *= inv_rms[m];
+          u *= inv_rms[m];
         }
         if (kg == 0 && j < a.rows && m < a.M && row < a.N) {
           float v;
           if (DUAL) {
-            const float act = a.activation == DH_ACT_SILU ? act_silu(sg) : act_gelu(sg);
-            v = act * su * a.alpha;
+            const float act = a.activation == DH_ACT_SILU ? act_silu(g) : act_gelu(g);
+            v = act * u * a.alpha;
             if (a.activation == DH_ACT_SILU && a.clamp_max > 0.f) v = fminf(fmaxf(v, -a.clamp_max), a.clamp_max);
           } else {
-            v = sg * a.alpha;
+            v = g * a.alpha;
             if (a.residual) v += a.residual[(int64_t)m * a.N + row];
           }
           if (a.c_f16)

@@ -231,6 +231,19 @@ def attn_cases(L, T, rows, reps):
                     algo = kv_bytes + (H + 2 * Hkv) * D * 4 + H * D * 4
                     emit(rows, config=cfg, kernel="attn_decode_qkv (cfg%d)" % cfg, shape="H=%d/%d D=128 ctx=%d" % (H, Hkv, ctx),
                          mode=mode, us=round(us, 3), achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
+                if cfg == 4:
+                    # what the decoder launches: the split kernel alone, its partial results left for the
+                    # chained launch that follows (which merges them: + ~1.5 us there, see the chain rows)
+                    nsplit = ctypes.c_int(0)
+                    for mode in ("rotating", "warm"):
+                        n = copies if mode == "rotating" else 1
+                        us = T.us(lambda i: capi.check(L.dh_attn_decode_qkv_partials(
+                            qkv.data_ptr(), w.data_ptr(), w.data_ptr(), cs.data_ptr(), cs.data_ptr(),
+                            K.data_ptr() + (i % n) * step, V.data_ptr() + (i % n) * step, H, Hkv, D, ctx - 1, D, 0,
+                            1e-6, 0, 1, 1.0 / D ** 0.5, 0.0, 0, 0, 0, ws.data_ptr(), ctypes.byref(nsplit))), reps)
+                        emit(rows, config=cfg, kernel="attn_decode_qkv partials only (cfg%d)" % cfg,
+                             shape="H=%d/%d D=128 ctx=%d" % (H, Hkv, ctx), mode=mode, us=round(us, 3),
+                             achieved=round(algo / us / 1e3, 1), unit="GB/s", algorithmic_bytes=algo)
             del K, V
 
 

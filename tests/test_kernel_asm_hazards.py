@@ -192,6 +192,20 @@ def test_destinations_of_hand_written_loads_are_left_alone_until_their_wait(asse
     assert hits == []
 
 
+@pytest.mark.parametrize("src", SOURCES)
+def test_no_scratch_memory_in_the_streaming_kernels(assembly, src):
+    """Scratch loads and stores are vector-memory operations: the compiler waits for them with vmcnt(0), i.e.
+    for the weight load in flight too, once per use (an array indexed by a loop counter did that at every
+    tile end of the two-row int8 kernel).  Only the scalar-load fallback of the few-row kernel (rows that
+    cannot be loaded four elements at a time) may spill."""
+    used = {}
+    for _, s, _, kernel in _instructions(assembly[src]):
+        if s.startswith("scratch_"):
+            used[kernel] = used.get(kernel, 0) + 1
+    allowed = ("q4k_gemv_rows_kernelILb0ELb0E", "q4k_gemv_rows_kernelILb1ELb0E")
+    assert {k: v for k, v in used.items() if not any(a in k for a in allowed)} == {}
+
+
 def test_the_scans_see_what_they_look_for(tmp_path):
     """The assembly of the build that faulted, reduced to the lines that matter, and a register reuse."""
     bad = tmp_path / "bad.s"
