@@ -5,16 +5,16 @@
 //
 // The inner sums  sum_k q_k x_k  are exact integer dot products: the activations of one
 // super-block column (256 values) are quantised ONCE per launch to 21-bit integers
-// X = round(x * 2^E) (E from the column's largest magnitude) and split into three signed
-// 7-bit digits X = x0 * 2^14 + x1 * 2^7 + x2, each a valid int8.  v_mfma_i32_16x16x64_i8 then
-// multiplies 16 weight rows x 64 weights by up to 16 "activation rows": the three digits of
-// four sub-blocks occupy 12 of them, so a pair of MFMAs leaves, in lane (weight row j, group g),
-// the three digit sums of sub-block g of weight row j.  The nibbles only need `& 0x0F0F0F0F` /
-// `>> 4 & 0x0F0F0F0F` to become int8 operands (3 vector ops per 8 weights), the 6-bit scales are
-// applied to the integer sums with 24-bit integer multiply-adds, and one int->float conversion per
-// digit and super-block brings in d, dmin and 2^-E.  The result carries every activation to 2^-21
-// of its column's maximum and is otherwise exact up to the final f32 roundings (observed 1e-6
-// relative L2 against an f64 evaluation).
+// X = round(x * 2^E) (E from the largest magnitude of each 32-element sub-block) and split into three
+// 7-bit digits X = x0 * 2^14 + x1 * 2^7 + x2 (x0 signed, x1 and x2 0..127), each a valid int8.
+// v_mfma_i32_16x16x64_i8 then multiplies 16 weight rows x 64 weights by up to 16 "activation rows":
+// the three digits of four sub-blocks occupy 12 of them, so a pair of MFMAs leaves, in lane (weight
+// row j, group g), the three digit sums of sub-block g of weight row j.  The nibbles only need
+// `& 0x0F0F0F0F` / `>> 4 & 0x0F0F0F0F` to become int8 operands (3 vector ops per 8 weights), the
+// three digit sums are put together as integers (that IS sum_k q_k X_k, exactly), and one int->float
+// conversion per sub-block brings in the scale, d, dmin and 2^-E.  The result carries every
+// activation to 2^-20 of its sub-block's maximum and is otherwise exact up to the final f32
+// roundings (observed 1e-6 relative L2 against an f64 evaluation).
 //
 // Work split: a workgroup of 16 waves owns 16-row tiles; a work unit is 16 weight rows x one
 // super-block column = 2304 bytes (144 contiguous per row).  Units are NOT bound to waves: every

@@ -5,7 +5,9 @@
 //
 // Activation format.  A super-block column (256 activations) is quantised per 32-element sub-block:
 // X = round(x * 2^E) with E chosen from the sub-block's largest magnitude so that |X| < 2^20, split
-// into three signed 7-bit digits X = x0 * 2^14 + x1 * 2^7 + x2.  Every finite f32 activation keeps
+// into three 7-bit digits X = x0 * 2^14 + x1 * 2^7 + x2: the top one signed (-64..63), the lower two
+// the plain bit fields 0..127 (three instructions per element, against five for balanced digits;
+// all are valid int8 operands and the digit sums stay far inside 24 bits).  Every finite f32 activation keeps
 // 20 bits below its sub-block's maximum (magnitudes below 2^-127 round to zero, as on flush-to-zero
 // hardware).  A sub-block that holds a NaN gets the factor NaN; one that holds an infinity (and no
 // NaN) gets the factor +Inf and the digits +-1 at the infinite elements, 0 elsewhere, so that the
@@ -78,20 +80,21 @@ __device__ __forceinline__ void i8_quantise_store(const float (&v)[4], unsigned 
     }
   }
   // X = round(x * sf) sits in the low mantissa bits of x * sf + 1.5 * 2^23 (two's complement)
-  uint32_t b[4], d2[4], d1[4], d0[4];
+  // (the bit pattern is 0x4B400000 + X: bits 0..6, 7..13 and 14..21 are the digits, the last one as a
+  // two's-complement byte)
+  uint32_t b[4], d1[4], d0[4];
   uint32_t xs = 0u;
 #pragma unroll
   for (int e = 0; e < 4; e++) {
     b[e] = __float_as_uint(fmaf(q[e], sf, 12582912.0f));
     xs += b[e];
-    d2[e] = (uint32_t)__builtin_amdgcn_sbfe((int)b[e], 0, 7);              // signed low 7 bits
-    d1[e] = (uint32_t)__builtin_amdgcn_sbfe((int)(b[e] + 64u), 7, 7);
-    d0[e] = (b[e] + 8256u) >> 14;                                          // byte 0 = top digit
+    d1[e] = b[e] >> 7;                                                     // byte 0: middle digit and one bit of the top one
+    d0[e] = b[e] >> 14;                                                    // byte 0 = top digit
   }
   const uint32_t lo01 = 0x0c0c0400u, hi23 = 0x04000c0cu;   // byte 0 of (src1, src0) -> bytes 0,1 / 2,3
   const uint32_t pk0 = __builtin_amdgcn_perm(d0[1], d0[0], lo01) | __builtin_amdgcn_perm(d0[3], d0[2], hi23);
-  const uint32_t pk1 = __builtin_amdgcn_perm(d1[1], d1[0], lo01) | __builtin_amdgcn_perm(d1[3], d1[2], hi23);
-  const uint32_t pk2 = __builtin_amdgcn_perm(d2[1], d2[0], lo01) | __builtin_amdgcn_perm(d2[3], d2[2], hi23);
+  const uint32_t pk1 = (__builtin_amdgcn_perm(d1[1], d1[0], lo01) | __builtin_amdgcn_perm(d1[3], d1[2], hi23)) & 0x7F7F7F7Fu;
+  const uint32_t pk2 = (__builtin_amdgcn_perm(b[1], b[0], lo01) | __builtin_amdgcn_perm(b[3], b[2], hi23)) & 0x7F7F7F7Fu;
   // sum of the quantised activations of the sub-block (8 lanes x 4 elements, |sum| < 2^25)
   const float sxf = (float)sum8_i32((int)(xs - 4u * 0x4B400000u));
   reinterpret_cast<uint32_t*>(rec)[lane] = pk0;
@@ -105,18 +108,20 @@ __device__ __forceinline__ void i8_quantise_store(const float (&v)[4], unsigned 
 
 // What lane (weight row j, group kg) of a unit contributes: sub-blocks kg (digit sums da, scale
 // sc_a, min mn_a, activation sum and factor sx[0] / xinv[0]) and 4 + kg (db, sc_b, mn_b, sx[1] /
-// xinv[1]) of its row's super-block.  |digit sum| <= 32 * 15 * 64 and the scales are 6 bits, so the
-// 24-bit multiplies are exact; each sub-block is finished in f32 before its factor is applied,
-// which keeps a non-finite factor from meeting the other sub-block's terms.
+// xinv[1]) of its row's super-block.  The three digit sums are put together as integers first:
+// da[0] * 2^14 + da[1] * 2^7 + da[2] IS sum_k q_k X_k, exactly (at most 32 * 15 * 2^20 in magnitude), so
+// the dot product of a sub-block meets one rounding when it becomes a float and one when it is scaled.
+// Each sub-block is finished in f32 before its factor is applied, which keeps a non-finite factor
+// from meeting the other sub-block's terms.
 typedef int i8dev_v4i __attribute__((ext_vector_type(4)));
 typedef float i8dev_v2f __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ float i8_unit_term(const i8dev_v4i da, const i8dev_v4i db, const int sc_a, const int sc_b,
                                               const float mn_a, const float mn_b, const float d, const float dmin,
                                               const i8dev_v2f sx, const i8dev_v2f xinv) {
-  const float ta = fmaf((float)__mul24(sc_a, da[0]), 16384.f, fmaf((float)__mul24(sc_a, da[1]), 128.f, (float)__mul24(sc_a, da[2])));
-  const float tb = fmaf((float)__mul24(sc_b, db[0]), 16384.f, fmaf((float)__mul24(sc_b, db[1]), 128.f, (float)__mul24(sc_b, db[2])));
-  const float ca = fmaf(d, ta, -(dmin * mn_a) * sx[0]);
-  const float cb = fmaf(d, tb, -(dmin * mn_b) * sx[1]);
+  const float ta = (float)((((da[0] << 7) + da[1]) << 7) + da[2]);
+  const float tb = (float)((((db[0] << 7) + db[1]) << 7) + db[2]);
+  const float ca = fmaf(d * (float)sc_a, ta, -(dmin * mn_a) * sx[0]);
+  const float cb = fmaf(d * (float)sc_b, tb, -(dmin * mn_b) * sx[1]);
   return fmaf(xinv[0], ca, xinv[1] * cb);
 }
 
