@@ -381,12 +381,21 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
     const uint8_t* W2;
     int64_t row_bytes;
     int N, nb, dual, rows, upt, upt_mul;
+    // byte offsets inside a weight matrix fit 32 bits (checked on the host): a unit's address is one
+    // 64-bit base plus 32-bit scalar arithmetic
+    uint32_t wg_off;               // this workgroup's first tile
+    uint32_t tile_stride;          // to its next tile
+    int rows_left0, rows_round;    // rows from the first tile's first row to the matrix's end; rows per round of tiles
     uint32_t goff[kUnitLoads];     // piece t * 64 + lane of a unit: row q / 9, 16-byte piece q % 9 of that row's super-block
   };
   auto stream_of = [&](const Phase& Q) {
     Stream S;
     S.W = Q.W; S.W2 = Q.W2; S.N = Q.N; S.nb = Q.nb; S.dual = Q.nmat - 1; S.rows = Q.rows; S.upt = Q.upt; S.upt_mul = Q.upt_mul;
     S.row_bytes = (int64_t)Q.nb * kBlockBytes;
+    S.wg_off = (uint32_t)bid * (uint32_t)Q.rows * (uint32_t)S.row_bytes;
+    S.tile_stride = (uint32_t)a.grid * (uint32_t)Q.rows * (uint32_t)S.row_bytes;
+    S.rows_left0 = Q.N - bid * Q.rows;
+    S.rows_round = a.grid * Q.rows;
 #pragma unroll
     for (int t = 0; t < kUnitLoads; t++) {
       const int q = t * 64 + lane, r = q / 9;
@@ -403,9 +412,9 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
   // Puts the loads of unit u in flight into the wave's ring.
   auto issue = [&](const Stream& S, const int u) {
     DH_DECODE(S, u, itl, imat, icol)
-    const int tile = bid + itl * a.grid;
-    const uint8_t* base = (imat ? S.W2 : S.W) + (int64_t)tile * S.rows * S.row_bytes + (int64_t)icol * kBlockBytes;
-    const int rows_left = S.N - tile * S.rows;
+    const uint32_t off = S.wg_off + (uint32_t)itl * S.tile_stride + (uint32_t)icol * kBlockBytes;
+    const uint8_t* base = (imat ? S.W2 : S.W) + off;
+    const int rows_left = S.rows_left0 - itl * S.rows_round;
     if (rows_left >= S.rows) {
 #pragma unroll
       for (int t = 0; t < kUnitLoads; t++) {
@@ -458,6 +467,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
     const Stream S = stream_of(Q);
     // what the unit loop itself reads is fetched together; what only a tile's end needs is fetched there
     asm volatile("" :: "s"(S.W), "s"(S.W2), "s"(S.N), "s"(S.nb), "s"(S.dual), "s"(S.rows), "s"(S.upt), "s"(S.upt_mul));
+    asm volatile("" :: "s"(S.wg_off), "s"(S.tile_stride), "s"(S.rows_left0), "s"(S.rows_round));
     const int nb = S.nb, upt = S.upt;
     const float* const nw = Q.norm_weight;
     const bool norm = nw != nullptr;

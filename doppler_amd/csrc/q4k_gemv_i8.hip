@@ -143,6 +143,12 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
   if (tid >= 64 && tid < 64 + kZeroBytes / 4) reinterpret_cast<uint32_t*>(zeros)[tid - 64] = 0u;
 
   const int64_t row_bytes = (int64_t)nb * kBlockBytes;
+  // byte offsets inside a weight matrix fit 32 bits (checked on the host): a unit's address is one
+  // 64-bit base plus 32-bit scalar arithmetic
+  const uint32_t wg_off = (uint32_t)blockIdx.x * (uint32_t)a.rows * (uint32_t)row_bytes;   // this workgroup's first tile
+  const uint32_t tile_stride = (uint32_t)a.grid * (uint32_t)a.rows * (uint32_t)row_bytes;   // to its next tile
+  const int rows_left0 = a.N - (int)blockIdx.x * a.rows;        // rows from the first tile's first row to the end
+  const int rows_round = a.grid * a.rows;
   // this workgroup's tiles: blockIdx.x, blockIdx.x + grid, ...
   const int ntl = a.tiles_base + ((int)blockIdx.x < a.tiles_rem ? 1 : 0);
   const int total = ntl * upt;                                  // units of this workgroup
@@ -168,11 +174,10 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
 #define DH_ISSUE(u_, stage_)                                                                      \
   do {                                                                                            \
     DH_DECODE(u_, itl_, imat_, icol_)                                                             \
-    const int tile_ = (int)blockIdx.x + itl_ * a.grid;                                    \
-    const uint8_t* base_ = ((DUAL && imat_) ? a.W2 : a.W) + (int64_t)tile_ * a.rows * row_bytes +   \
-                           (int64_t)icol_ * kBlockBytes;                                          \
+    const uint32_t off_ = wg_off + (uint32_t)itl_ * tile_stride + (uint32_t)icol_ * kBlockBytes;  \
+    const uint8_t* base_ = ((DUAL && imat_) ? a.W2 : a.W) + off_;                                 \
     unsigned char* st_ = my_ring + (stage_) * kStage;                                             \
-    const int rows_left_ = a.N - tile_ * a.rows;                                                  \
+    const int rows_left_ = rows_left0 - itl_ * rows_round;                                        \
     if (rows_left_ >= a.rows) {                                                                   \
       _Pragma("unroll") for (int t = 0; t < kUnitLoads; t++) {                                    \
         if (goff[t] != 0xFFFFFFFFu)                                                               \
@@ -620,6 +625,8 @@ int launch_i8_vec(I8Args a, const char* op) {
   if (units * ((int64_t)a.upt_mul * a.upt - (1 << 24)) >= (1 << 24) || units >= (1 << 20) ||
       units * (int64_t)a.upt_mul >= ((int64_t)1 << 32))
     return -1;
+  // the kernel forms byte offsets inside a matrix in 32 bits (the last tile's rows are clamped, never read past)
+  if (((int64_t)ntiles * a.rows + kTileRows) * a.nb * kBlockBytes >= ((int64_t)1 << 32)) return -1;
   int depth = 1;
   if (env_depth > 0) depth = std::min(kMaxDepth, env_depth);
   // tile slots: the units in flight (16 waves x (depth + 1) draws) span at most this many tiles
