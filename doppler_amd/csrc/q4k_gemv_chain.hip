@@ -418,7 +418,11 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
     if (rows_left >= S.rows) {
 #pragma unroll
       for (int t = 0; t < kUnitLoads; t++) {
-        if (S.goff[t] != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + S.goff[t], DH_LDS_PTR(my_ring + t * 1024), 16, 0, 0);
+        // (the offset is made opaque here so that its widening to 64 bits is not hoisted out of the unit
+        // loop: only then does the load take the form scalar base + 32-bit lane offset, with no vector add)
+        uint32_t g = S.goff[t];
+        asm volatile("" : "+v"(g));
+        if (g != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + g, DH_LDS_PTR(my_ring + t * 1024), 16, 0, 0);
       }
     } else {
 #pragma unroll
