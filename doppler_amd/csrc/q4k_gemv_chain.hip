@@ -55,7 +55,9 @@ typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 
 constexpr int kWaves = 16;
 constexpr int kTileRows = 16;
-constexpr int kStage = kTileRows * kBlockBytes;   // 2304 bytes: a wave's ring holds one unit
+constexpr int kStage = 3 * 1024;                   // a wave's ring: one unit (16 rows x 144 bytes = 2304) as three
+                                                   // full 64-lane loads of 16 bytes: the third one's lanes past the unit
+                                                   // land in the stage's own tail, so no load needs a lane mask
 constexpr int kUnitLoads = 3;                     // load instructions of a full unit: ceil(16 rows * 9 pieces / 64 lanes)
 constexpr int kMaxPhases = DH_CHAIN_MAX_PHASES;
 constexpr int kSlots = 8;                         // tiles whose partial sums may be in LDS at once (a power of two)
@@ -159,7 +161,7 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
                "s"(a.nb_max[1]), "s"(a.red_stride));
   asm volatile("" :: "s"(a.ph[0].norm_weight), "s"(a.ph[0].nb));
 
-  // ---- LDS: ring [16 waves][2304], record areas 0 and 1, zeros [144], partial sums
+  // ---- LDS: ring [16 waves][3072], record areas 0 and 1, zeros [144], partial sums
   // [kSlots][red_stride], counters
   unsigned char* ring = lds;
   unsigned char* xq0 = ring + (size_t)kWaves * kStage;
@@ -399,7 +401,8 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
 #pragma unroll
     for (int t = 0; t < kUnitLoads; t++) {
       const int q = t * 64 + lane, r = q / 9;
-      S.goff[t] = q < 9 * S.rows ? (uint32_t)(r * S.row_bytes + (q - r * 9) * 16) : 0xFFFFFFFFu;
+      // (lanes past the tile's pieces fetch piece 0 again: their 16 bytes land behind the unit, unread)
+      S.goff[t] = q < 9 * S.rows ? (uint32_t)(r * S.row_bytes + (q - r * 9) * 16) : 0u;
     }
     return S;
   };
@@ -422,14 +425,14 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_chain_kernel(const Ch
         // loop: only then does the load take the form scalar base + 32-bit lane offset, with no vector add)
         uint32_t g = S.goff[t];
         asm volatile("" : "+v"(g));
-        if (g != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + g, DH_LDS_PTR(my_ring + t * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(base + g, DH_LDS_PTR(my_ring + t * 1024), 16, 0, 0);
       }
     } else {
 #pragma unroll
       for (int t = 0; t < kUnitLoads; t++) {
         const int q = t * 64 + lane, rr = q / 9;
         const int64_t o = (int64_t)min(rr, rows_left - 1) * S.row_bytes + (q - rr * 9) * 16;
-        if (S.goff[t] != 0xFFFFFFFFu) __builtin_amdgcn_global_load_lds(base + o, DH_LDS_PTR(my_ring + t * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(base + o, DH_LDS_PTR(my_ring + t * 1024), 16, 0, 0);
       }
     }
   };
