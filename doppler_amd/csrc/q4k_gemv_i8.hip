@@ -48,7 +48,9 @@ typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 
 constexpr int kWaves = 16;
 constexpr int kTileRows = 16;
-constexpr int kStage = kTileRows * kBlockBytes;   // 2304 bytes per ring stage
+constexpr int kStage = 3 * 1024;                   // a ring stage: one unit (16 rows x 144 bytes = 2304) as three full
+                                                   // 64-lane loads of 16 bytes: the third one's lanes past the unit land in
+                                                   // the stage's own tail, so no load needs a lane mask
 constexpr int kUnitLoads = 3;                     // load instructions of a full unit: ceil(16 rows * 9 pieces / 64 lanes)
 constexpr int kMaxDepth = 1;                      // ring stages per wave (2..5 measured slower: the queue already keeps 16 units in flight)
 constexpr int kSlotDepth = 3;                     // what the tile-slot count is sized for
@@ -108,7 +110,7 @@ __device__ __forceinline__ uint32_t lds_read_u32(uint32_t addr) {
 }
 
 // Layout of the dynamic LDS block, in this order:
-//   ring   [16 waves][depth][2304]
+//   ring   [16 waves][depth][3072]
 //   xq     [nb][MT][kRec]: per column and activation row, digit plane p at 256 p (byte e = digit p
 //          of element e), the 8 sub-block sums at 768, their factors 2^-E at 800, the column's sum of squares at 832
 //   zeros  [144]
@@ -160,7 +162,8 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
 #pragma unroll
   for (int t = 0; t < kUnitLoads; t++) {
     const int p = t * 64 + lane, r = p / 9;
-    goff[t] = p < 9 * a.rows ? (uint32_t)(r * row_bytes + (p - r * 9) * 16) : 0xFFFFFFFFu;
+    // (lanes past the tile's pieces fetch piece 0 again: their 16 bytes land behind the unit, unread)
+    goff[t] = p < 9 * a.rows ? (uint32_t)(r * row_bytes + (p - r * 9) * 16) : 0u;
   }
 
   // Unit u of the workgroup = (tile ordinal tl, matrix, column): u = (tl * NMAT + mat) * nb + col.
@@ -180,15 +183,17 @@ __global__ __launch_bounds__(64 * kWaves, 1) void q4k_gemv_i8_kernel(const I8Arg
     const int rows_left_ = rows_left0 - itl_ * rows_round;                                        \
     if (rows_left_ >= a.rows) {                                                                   \
       _Pragma("unroll") for (int t = 0; t < kUnitLoads; t++) {                                    \
-        if (goff[t] != 0xFFFFFFFFu)                                                               \
-          __builtin_amdgcn_global_load_lds(base_ + goff[t], DH_LDS_PTR(st_ + t * 1024), 16, 0, 0); \
+        /* the offset is made opaque here so that its widening to 64 bits is not hoisted out of the */ \
+        /* unit loop: only then does the load take the form scalar base + 32-bit lane offset        */ \
+        uint32_t g_ = goff[t];                                                                    \
+        asm volatile("" : "+v"(g_));                                                              \
+        __builtin_amdgcn_global_load_lds(base_ + g_, DH_LDS_PTR(st_ + t * 1024), 16, 0, 0);       \
       }                                                                                           \
     } else {                                                                                      \
       _Pragma("unroll") for (int t = 0; t < kUnitLoads; t++) {                                    \
         const int p_ = t * 64 + lane, r_ = p_ / 9;                                                \
         const int64_t o_ = (int64_t)min(r_, rows_left_ - 1) * row_bytes + (p_ - r_ * 9) * 16;     \
-        if (goff[t] != 0xFFFFFFFFu)                                                               \
-          __builtin_amdgcn_global_load_lds(base_ + o_, DH_LDS_PTR(st_ + t * 1024), 16, 0, 0);     \
+        __builtin_amdgcn_global_load_lds(base_ + o_, DH_LDS_PTR(st_ + t * 1024), 16, 0, 0);       \
       }                                                                                           \
     }                                                                                             \
   } while (0)

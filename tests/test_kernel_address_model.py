@@ -16,7 +16,8 @@ import pytest
 from doppler_amd import capi
 
 WAVES, TILE_ROWS, BLOCK, QK = 16, 16, 144, 256
-STAGE = TILE_ROWS * BLOCK            # bytes of a ring stage
+STAGE = TILE_ROWS * BLOCK            # bytes of a ring stage (few-row kernel)
+STAGE_I8 = 3 * 1024                  # int8 kernel: a stage takes three full 64-lane loads (a unit is the first 2304 bytes)
 REC, ZERO = 848, 144                 # int8 kernel: bytes of an activation record, of the zero area
 READ_AHEAD = 12 * 64                 # int8 kernel: the last partial-sum read reaches this far past its slot, per activation row
 I8, ROWS = capi.PLAN_GEMV_I8, capi.PLAN_GEMV_ROWS
@@ -61,14 +62,14 @@ def check_i8(M, N, K, normed, dual, ncu=NCU):
     while nslots < need:
         nslots *= 2
     assert MT == (2 if M == 2 and lay["mt"] == 2 else 1)
-    lds = WAVES * 1 * STAGE + nb * MT * REC + ZERO + 4 * nslots * upt * MT * 16 + 4 * (2 + 2 * nslots + nb) + READ_AHEAD * MT
+    lds = WAVES * 1 * STAGE_I8 + nb * MT * REC + ZERO + 4 * nslots * upt * MT * 16 + 4 * (2 + 2 * nslots + nb) + READ_AHEAD * MT
     assert (lay["rows"], lay["nlw"], lay["grid"], lay["tiles_base"], lay["tiles_rem"]) == \
         (rows, ceil_div(9 * rows, 64), grid, ntiles // grid, ntiles % grid)
     assert (lay["upt"], lay["upt_mul"], lay["nslots"], lay["depth"], lay["lds"]) == (upt, upt_mul, nslots, 1, lds)
     assert lds <= 160 * 1024
     row_bytes = nb * BLOCK
     # ---- LDS layout: ring, records, zeros, partial sums, counters (+ read-ahead padding)
-    o_xq = WAVES * 1 * STAGE
+    o_xq = WAVES * 1 * STAGE_I8
     o_zero = o_xq + nb * MT * REC
     o_red = o_zero + ZERO
     o_ctr = o_red + 4 * nslots * upt * MT * 16
@@ -77,13 +78,12 @@ def check_i8(M, N, K, normed, dual, ncu=NCU):
     lane = lanes()
     j, kg = lane & 15, lane >> 4
     # ring: what the load unit writes (piece t * 64 + lane of a unit, 16 bytes) and what the lanes read back
+    # (every lane of the three loads writes: the lanes past the unit's pieces land in the stage's tail)
     for t in range(3):
-        p = t * 64 + lane
-        valid = p < 9 * rows
-        assert np.all((t * 1024 + lane * 16 + 16)[valid] <= STAGE)
+        assert np.all(t * 1024 + lane * 16 + 16 <= STAGE_I8)
     hdr = j * BLOCK
     q = hdr + 16 + 32 * (kg >> 1) + 16 * (kg & 1)
-    assert np.all(hdr + 16 <= STAGE) and np.all(q + 64 + 16 <= STAGE)
+    assert np.all(hdr + 16 <= TILE_ROWS * BLOCK) and np.all(q + 64 + 16 <= TILE_ROWS * BLOCK)
     # records: digit operands (or the zero area), sub-block sums and factors, sum of squares
     g, dg = j >> 2, j & 3
     data_off = 256 * np.minimum(dg, 2) + 32 * g + 16 * (kg & 1)
@@ -111,16 +111,21 @@ def check_i8(M, N, K, normed, dual, ncu=NCU):
         rows_left = N - tile * rows
         assert np.all(rows_left >= 1)
         base = tile * rows * row_bytes + col * BLOCK
+        assert np.all(base + rows * row_bytes < (1 << 32))          # offsets inside a matrix are formed in 32 bits
         for t in range(3):
             p = t * 64 + lane
             valid = p < 9 * rows
             rr = p // 9
             piece = (p - rr * 9) * 16
             for b_, left in zip(base, rows_left):
-                rsel = rr if left >= rows else np.minimum(rr, left - 1)
-                off = b_ + rsel * row_bytes + piece
-                assert np.all((off + 16)[valid] <= N * row_bytes), (bid, t)
-                assert np.all(off[valid] >= 0)
+                if left >= rows:
+                    # full tile: lanes past the tile's pieces fetch piece 0 of row 0 again
+                    off = b_ + np.where(valid, rr * row_bytes + piece, 0)
+                else:
+                    # last, partial tile: every lane's row is clamped to the last one
+                    off = b_ + np.minimum(rr, left - 1) * row_bytes + piece
+                assert np.all(off + 16 <= N * row_bytes), (bid, t)
+                assert np.all(off >= 0)
         # partial sums: writes of a unit, and the finishing wave's four-columns-at-a-time reads
         slot = tl & (nslots - 1)
         for m in range(MT):
@@ -160,7 +165,7 @@ I8_SHAPES = [
     (2, 6144, 4096, 1, 0), (2, 4096, 4096, 0, 0), (2, 12288, 4096, 1, 1), (2, 4096, 12288, 0, 0),
     (1, 151936, 4096, 0, 0),                                        # many tiles per workgroup
     (1, 4097, 4096, 0, 0), (2, 300, 700, 0, 0), (1, 17, 1023, 0, 0), (1, 5000, 2560, 1, 1),   # ragged N, K off 4
-    (1, 4096, 28160, 1, 0), (2, 1024, 8192, 1, 0), (1, 64, 16384, 0, 0),   # the longest rows the kernel takes
+    (1, 4096, 25088, 1, 0), (2, 1024, 8192, 1, 0), (1, 64, 16384, 0, 0),   # the longest rows the kernel takes
     (1, 1_000_000, 4096, 0, 0),                                     # more than 200 tiles per workgroup
 ]
 
