@@ -76,6 +76,25 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 typedef __attribute__((ext_vector_type(8))) _Float16 half8_t;
+
+// Eight query values as one matrix-core operand: even operand rows take the f16 high parts of sc * q,
+// odd rows what the high parts left over, so that the two rows together carry q to ~22 bits.  Both
+// parts are rounded toward zero, two elements per instruction (the residual is exact in f32, so the
+// rounding mode of the high part does not matter).  sc = 0 gives a zero operand.
+__device__ __forceinline__ half8_t q_operand(const float (&qv)[8], const float sc, const bool odd) {
+  typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+  u32x4 w;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const float x0 = qv[2 * i] * sc, x1 = qv[2 * i + 1] * sc;
+    const uint32_t hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x0, x1));
+    const float h0 = __half2float(__ushort_as_half((unsigned short)(hi & 0xffffu)));
+    const float h1 = __half2float(__ushort_as_half((unsigned short)(hi >> 16)));
+    const uint32_t lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x0 - h0, x1 - h1));
+    w[i] = odd ? lo : hi;
+  }
+  return __builtin_bit_cast(half8_t, w);
+}
 typedef __attribute__((ext_vector_type(4))) float float4_t;
 
 
@@ -305,12 +324,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
       const float* qp = &q_rows[min(qrow >> 1, GT - 1)][32 * s + 8 * kg];
       const float4 q0 = reinterpret_cast<const float4*>(qp)[0], q1 = reinterpret_cast<const float4*>(qp)[1];
       const float qv[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-#pragma unroll
-      for (int i = 0; i < 8; i++) {
-        const float xs = live ? qv[i] * a.scale : 0.f;
-        const _Float16 h = (_Float16)xs;
-        qa[s][i] = (qrow & 1) ? (_Float16)(xs - (float)h) : h;
-      }
+      qa[s] = q_operand(qv, live ? a.scale : 0.f, (qrow & 1) != 0);
     }
     if (owner) {
 #pragma unroll
@@ -327,12 +341,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const AttnArgs a
         const float* qp = a.Q + (int64_t)(kvh * G + (qrow >> 1)) * D + 32 * s + 8 * kg;
         const float4 q0 = reinterpret_cast<const float4*>(qp)[0], q1 = reinterpret_cast<const float4*>(qp)[1];
         const float qv[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-          const float xs = qv[i] * a.scale;
-          const _Float16 h = (_Float16)xs;
-          qa[s][i] = (qrow & 1) ? (_Float16)(xs - (float)h) : h;
-        }
+        qa[s] = q_operand(qv, a.scale, (qrow & 1) != 0);
       }
     }
   }
