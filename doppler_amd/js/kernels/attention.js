@@ -1,5 +1,7 @@
 // runAttention / recordAttention over an f16 KV cache, decode (seqLen 1) and prefill (seqLen > 1):
-// reference src/gpu/kernels/attention.js:1047-1310,2007-2030.
+// reference src/gpu/kernels/attention.js:1047-1310,2007-2030.  An f16 Q (the reference's f16-activation
+// plan: variants *_f16 with outputDtype f16, src/config/kernels/registry.json) is widened into a temporary
+// (exact), the kernels run as for f32 and the output is narrowed to f16 once.
 import { getNative, KV_LAYOUT } from '../native.js';
 import { createTensor } from '../tensor.js';
 import { acquireBuffer, releaseBuffer } from '../buffer-pool.js';
@@ -29,8 +31,38 @@ async function executeAttention(recorder, Q, K, V, mask, numHeads, headDim, opti
   if (!(kvLayout in KV_LAYOUT)) {
     throw new Error(`[Attention] kvLayout "${kvLayout}" is not supported by the HIP path (contiguous, ring).`);
   }
-  if (Q.dtype !== 'f32' || K.dtype !== 'f16' || V.dtype !== 'f16') {
-    throw new Error(`[Attention] decode needs f32 Q and f16 K/V, got ${Q.dtype}/${K.dtype}/${V.dtype}.`);
+  if ((Q.dtype !== 'f32' && Q.dtype !== 'f16') || K.dtype !== 'f16' || V.dtype !== 'f16') {
+    throw new Error(`[Attention] the HIP path needs f32 or f16 Q and f16 K/V, got ${Q.dtype}/${K.dtype}/${V.dtype}.`);
+  }
+  if (Q.dtype === 'f16') {
+    // widened Q and an f32 output of our own; the caller's outputBuffer (if any) takes the f16 result
+    const n = seqLen * numHeads * headDim;
+    if (Q.buffer.size < n * 2) {
+      throw new Error(`[Attention] Q buffer is smaller than [${seqLen}, ${numHeads}, ${headDim}] f16.`);
+    }
+    if (outputBuffer && outputBuffer.size < n * 2) {
+      throw new Error(`[Attention] outputBuffer is smaller than [${seqLen}, ${numHeads}, ${headDim}] f16.`);
+    }
+    const wideQ = acquireBuffer(n * 4, undefined, 'attention_q_f32_temp');
+    let wideOut = null;
+    let out16 = null;
+    try {
+      getNative().castF16ToF32(Q.buffer.ptr, wideQ.ptr, n);
+      const r = await executeAttention(recorder, createTensor(wideQ, 'f32', [...Q.shape], 'attention_q_f32'), K, V, mask,
+        numHeads, headDim, { ...options, outputBuffer: null });
+      wideOut = r.buffer;
+      out16 = outputBuffer || acquireBuffer(n * 2, undefined, 'attention_output');
+      getNative().castF32ToF16(wideOut.ptr, out16.ptr, n);
+    } catch (error) {
+      releaseBuffer(wideQ);
+      if (wideOut) releaseBuffer(wideOut);
+      if (out16 && !outputBuffer) releaseBuffer(out16);
+      throw error;
+    }
+    for (const b of [wideQ, wideOut]) {
+      if (recorder) recorder.trackTemporaryBuffer(b); else releaseBuffer(b);
+    }
+    return createTensor(out16, 'f16', [seqLen, numHeads, headDim], 'attention_output');
   }
   const rows = kvLayout === 'ring' ? slidingWindow : kvStart + kvLen;
   const kvBytes = rows * numKVHeads * headDim * 2;

@@ -1,7 +1,11 @@
 // runRoPE / recordRoPE: reference src/gpu/kernels/rope.js:14-114.  In place; the returned
-// Tensor aliases the input buffer.
+// Tensor aliases the input buffer.  f16 activations take the reference's own route for a device
+// without an f16 rotary kernel (rope.js:44-63,89-107): widened into a temporary, rotated in f32,
+// narrowed back into the input buffer (one rounding, as a kernel that computes in f32 and stores
+// f16 would make).
 import { getNative } from '../native.js';
 import { createTensor } from '../tensor.js';
+import { acquireBuffer, releaseBuffer } from '../buffer-pool.js';
 import { bufferOf, noteDispatch } from './constants.js';
 
 async function rope(recorder, input, freqsCos, freqsSin, seqLen, options = {}) {
@@ -30,8 +34,8 @@ async function rope(recorder, input, freqsCos, freqsSin, seqLen, options = {}) {
       `RoPE pairSpanDim must be in [rotaryDim, headDim]; got ${pairSpanDim} for rotaryDim ${rotaryDim} and headDim ${headDim}`
     );
   }
-  if (input.dtype !== 'f32') {
-    throw new Error(`RoPE on the HIP path takes f32 activations, got ${input.dtype}`);
+  if (input.dtype !== 'f32' && input.dtype !== 'f16') {
+    throw new Error(`RoPE on the HIP path takes f32 or f16 activations, got ${input.dtype}`);
   }
   const cos = bufferOf(freqsCos);
   const sin = bufferOf(freqsSin);
@@ -39,8 +43,27 @@ async function rope(recorder, input, freqsCos, freqsSin, seqLen, options = {}) {
   if (cos.size < need || sin.size < need) {
     throw new Error(`RoPE frequency tables are smaller than ${need} bytes (startPos=${startPos}, seqLen=${seqLen})`);
   }
-  getNative().rope(input.buffer.ptr, cos.ptr, sin.ptr, seqLen, numHeads, headDim, rotaryDim, pairSpanDim,
-    interleaved ? 1 : 0, startPos);
+  const native = getNative();
+  if (input.dtype === 'f16') {
+    const n = seqLen * numHeads * headDim;
+    if (input.buffer.size < n * 2) {
+      throw new Error(`RoPE input buffer is smaller than [${seqLen}, ${numHeads}, ${headDim}] f16.`);
+    }
+    const wide = acquireBuffer(n * 4, undefined, 'rope_f32_temp');
+    try {
+      native.castF16ToF32(input.buffer.ptr, wide.ptr, n);
+      native.rope(wide.ptr, cos.ptr, sin.ptr, seqLen, numHeads, headDim, rotaryDim, pairSpanDim,
+        interleaved ? 1 : 0, startPos);
+      native.castF32ToF16(wide.ptr, input.buffer.ptr, n);
+    } catch (error) {
+      releaseBuffer(wide);
+      throw error;
+    }
+    if (recorder) recorder.trackTemporaryBuffer(wide); else releaseBuffer(wide);
+  } else {
+    native.rope(input.buffer.ptr, cos.ptr, sin.ptr, seqLen, numHeads, headDim, rotaryDim, pairSpanDim,
+      interleaved ? 1 : 0, startPos);
+  }
   noteDispatch(recorder, 'rope');
   return createTensor(input.buffer, input.dtype, [...input.shape], 'rope_output');
 }

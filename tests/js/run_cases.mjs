@@ -98,11 +98,12 @@ async function main() {
       await save(c.name + '.res.out.bin', n.residual.buffer, c.batch * c.hidden * 4);
       await save(c.name + '.next.out.bin', n.nextInput.buffer, c.batch * c.hidden * 4);
     } else if (c.op === 'rope') {
-      const x = tensor(c.x, 'f32', [c.seq, c.heads, c.headDim]);
+      const dt = c.dtype || 'f32';
+      const x = tensor(c.x, dt, [c.seq, c.heads, c.headDim]);
       const t = await dh.runRoPE(x, tensor(c.cos, 'f32', [1]), tensor(c.sin, 'f32', [1]), c.seq,
         { numHeads: c.heads, headDim: c.headDim, startPos: c.startPos, interleaved: c.interleaved });
-      if (t.buffer !== x.buffer) throw new Error('runRoPE must alias its input');
-      await save(out, t.buffer, c.seq * c.heads * c.headDim * 4);
+      if (t.buffer !== x.buffer || t.dtype !== dt) throw new Error('runRoPE must alias its input and keep its dtype');
+      await save(out, t.buffer, c.seq * c.heads * c.headDim * (dt === 'f16' ? 2 : 4));
     } else if (c.op === 'rope_qk') {
       const q = tensor(c.q, 'f32', [c.seq, c.heads, c.headDim]);
       const k = tensor(c.k, 'f32', [c.seq, c.kvHeads, c.headDim]);
@@ -143,10 +144,12 @@ async function main() {
       await save(out, ck, c.cacheElems * 2);
       await save(`${c.name}.v.bin`, cv, c.cacheElems * 2);
     } else if (c.op === 'attention') {
-      const t = await dh.runAttention(tensor(c.Q, 'f32', [c.heads, c.headDim]), tensor(c.K, 'f16', [c.kvLen, c.kvHeads, c.headDim]),
+      const dt = c.dtype || 'f32';
+      const t = await dh.runAttention(tensor(c.Q, dt, [c.heads, c.headDim]), tensor(c.K, 'f16', [c.kvLen, c.kvHeads, c.headDim]),
         tensor(c.V, 'f16', [c.kvLen, c.kvHeads, c.headDim]), null, c.heads, c.headDim,
         { seqLen: 1, kvLen: c.kvLen, numKVHeads: c.kvHeads, causal: true, startPos: c.kvLen - 1 });
-      await save(out, t.buffer, c.heads * c.headDim * 4);
+      if (t.dtype !== dt) throw new Error(`runAttention with ${dt} Q must return ${dt}, got ${t.dtype}`);
+      await save(out, t.buffer, c.heads * c.headDim * (dt === 'f16' ? 2 : 4));
     } else if (c.op === 'attention_kvlen_buffer') {
       // the key count comes from a device u32 (kvLenBuffer); kvLen only bounds it
       const lenBuf = dh.acquireBuffer(4);
@@ -186,8 +189,10 @@ async function main() {
       const t = await fn(tensor(c.up, 'f32', [c.n]), { size: c.n, gate: tensor(c.gate, 'f32', [c.n]) });
       await save(out, t.buffer, c.n * 4);
     } else if (c.op === 'gather') {
-      const t = await dh.runGather(dev(c.ids), dev(c.table), c.T, c.hidden, c.vocab, { embeddingDtype: 'f16', outputDtype: 'f32' });
-      await save(out, t.buffer, c.T * c.hidden * 4);
+      const dt = c.dtype || 'f32';
+      const t = await dh.runGather(dev(c.ids), dev(c.table), c.T, c.hidden, c.vocab, { embeddingDtype: 'f16', outputDtype: dt });
+      if (t.dtype !== dt) throw new Error(`runGather must return ${dt}, got ${t.dtype}`);
+      await save(out, t.buffer, c.T * c.hidden * (dt === 'f16' ? 2 : 4));
     } else if (c.op === 'argmax') {
       const tok = await dh.runArgmax(dev(c.logits), c.vocab, { padTokenId: c.padTokenId });
       fs.writeFileSync(path.join(dir, out), Buffer.from(new Uint32Array([tok]).buffer));

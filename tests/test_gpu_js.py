@@ -218,6 +218,14 @@ def test_js_host_path_parity(tmp_path):
                       heads=16, headDim=128, startPos=40, interleaved=False))
     rope_want = oracle.rope_apply(xr, cos, sin, 2, 16, 128, 40)
     checks.append(lambda: rel_l2(get("rope.out.bin", np.float32), rope_want) <= 1e-6)
+    # f16 activations (the reference's f16-activation plan, rope.js:44-63): the rotation of the f16 values,
+    # computed in f32 and rounded to f16 once
+    xr16 = xr.astype(np.float16)
+    cases.append(dict(cases[-1], name="rope_f16", x=put("rope.x16", xr16.view(np.uint16)), dtype="f16"))
+    rope16_want = oracle.rope_apply(xr16.astype(np.float32), cos, sin, 2, 16, 128, 40).astype(np.float16)
+    checks.append(lambda: np.max(np.abs(get("rope_f16.out.bin", np.float16).astype(np.float32)
+                                        - rope16_want.reshape(-1).astype(np.float32))
+                                 / np.maximum(np.abs(rope16_want.reshape(-1).astype(np.float32)), 1e-3)) <= 2 ** -10)
     bx, bb = synth.normal_f32((3, 1024), 9510, 2.0), synth.normal_f32((2, 1024), 9511)
     cases.append(dict(name="biasscale", op="bias_scale", x=put("bs.x", bx), bias=put("bs.b", bb), tokens=3, dim=1024, scale=0.125))
     checks.append(lambda: np.array_equal(get("biasscale.bias.out.bin", np.float32).reshape(3, 1024), bx + bb[1]))
@@ -278,6 +286,9 @@ def test_js_host_path_parity(tmp_path):
                       kvHeads=8, headDim=128, kvLen=ctx))
     attn_want = oracle.attention_decode_f16kv(q, kb, vb, 16, 8, 128, ctx)
     checks.append(lambda: rel_l2(get("attn.out.bin", np.float32), attn_want) <= 1e-3)
+    # f16 Q (q above is f16-representable), f16 output
+    cases.append(dict(cases[-1], name="attn_f16q", Q=put("attn.q16", q.astype(np.float16).view(np.uint16)), dtype="f16"))
+    checks.append(lambda: rel_l2(get("attn_f16q.out.bin", np.float16).astype(np.float32), attn_want) <= 1e-3)
     # the same with the key count in a device buffer (kvLenBuffer): 300 of the 512 rows
     cases.append(dict(name="attn_len", op="attention_kvlen_buffer", Q="attn.q", K="attn.k", V="attn.v", heads=16, kvHeads=8,
                       headDim=128, kvLen=ctx, count=300))
@@ -298,6 +309,10 @@ def test_js_host_path_parity(tmp_path):
     tab = synth.normal_f16_bits((300, 640), 9903, 0.02)
     cases.append(dict(name="gather", op="gather", ids=put("g.ids", ids), table=put("g.tab", tab), T=4, hidden=640, vocab=300))
     checks.append(lambda: np.array_equal(get("gather.out.bin", np.float32).reshape(4, 640), oracle.gather_f16(ids, tab, 640, 300)))
+    # f16 rows out: the stored bits of the gathered rows (zeros for the id past the table)
+    cases.append(dict(cases[-1], name="gather_f16", dtype="f16"))
+    checks.append(lambda: np.array_equal(get("gather_f16.out.bin", np.float16).reshape(4, 640).astype(np.float32),
+                                         oracle.gather_f16(ids, tab, 640, 300)))
     lg = synth.rng(9904).integers(-50, 50, 151936).astype(np.float32)
     pad = oracle.argmax(lg)
     cases.append(dict(name="argmax", op="argmax", logits=put("am.l", lg), vocab=151936, padTokenId=pad))
