@@ -68,6 +68,17 @@ struct F16GemvArgs {
   uint32_t* part_idx;
 };
 
+// 16 bytes of a weight row, marked non-temporal.  Every row is read once per call, by one wave, as whole
+// cache lines (a wave's load covers 1 KB of consecutive bytes): with the streaming hint the [151936 x 4096]
+// f16 head is read at 6.6 TB/s against 5.9 TB/s with ordinary loads.  (The same hint on loads whose cache
+// lines are shared between waves, the Q4_K units' 144-byte row pieces and the decode attention's K/V rows,
+// made those kernels slower.)
+__device__ __forceinline__ uint4 stream_load_16(const uint4* p) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(t[0], t[1], t[2], t[3]);
+}
+
 // M = 1, K <= 4096: every lane meets the same 64 activations in every row (its eight 16-byte
 // chunks sit at fixed k), so they live in registers for the whole kernel: no LDS at all.
 template <bool ARGMAX>
@@ -97,7 +108,7 @@ __global__ __launch_bounds__(256) void f16w_gemv_xreg_kernel(const F16GemvArgs a
 #pragma unroll
     for (int u = 0; u < 8; u++) {
       const int v = lane + 64 * u;
-      raw[u] = v < kvec ? wrow[v] : make_uint4(0, 0, 0, 0);
+      raw[u] = v < kvec ? stream_load_16(wrow + v) : make_uint4(0, 0, 0, 0);
     }
     float s0 = 0.f, s1 = 0.f;
 #pragma unroll
@@ -151,7 +162,7 @@ __global__ __launch_bounds__(256) void f16w_gemv_kernel(const F16GemvArgs a) {
 #pragma unroll
       for (int u = 0; u < 8; u++) {
         const int v = v0 + 64 * u;
-        raw[u] = v < kvec ? wrow[v] : make_uint4(0, 0, 0, 0);
+        raw[u] = v < kvec ? stream_load_16(wrow + v) : make_uint4(0, 0, 0, 0);
       }
 #pragma unroll
       for (int u = 0; u < 8; u++) {
