@@ -91,6 +91,7 @@ SIGNATURES = {
     "dh_f16w_matmul": (_I, [_P, _P, _P, _I, _I, _I, _F]),
     "dh_lmhead_argmax_workspace_bytes": (_SZ, [_I]),
     "dh_lmhead_argmax_f16": (_I, [_P, _P, _I, _I, _I64, _F, _P, _P, _I, _P]),
+    "dh_lmhead_argmax_f16_rmsnorm": (_I, [_P, _P, _F, _I, _P, _I, _I, _I64, _F, _P, _P, _I, _P]),
     "dh_attn_decode_workspace_bytes": (_SZ, [_I, _I, _I]),
     "dh_attn_prefill": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I, _F, _I]),
     "dh_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _F, _I, _I, _I, _P]),

@@ -66,6 +66,10 @@ struct F16GemvArgs {
   int64_t pad_id;
   float* part_val;
   uint32_t* part_idx;
+  // RMSNorm of the activation row in the prologue (register kernel only; null = off)
+  const float* norm_weight;
+  float norm_eps;
+  int norm_weight_offset;
 };
 
 // 16 bytes of a weight row, marked non-temporal.  Every row is read once per call, by one wave, as whole
@@ -98,6 +102,28 @@ __global__ __launch_bounds__(256) void f16w_gemv_xreg_kernel(const F16GemvArgs a
     }
     x[u][0] = xa.x; x[u][1] = xa.y; x[u][2] = xa.z; x[u][3] = xa.w;
     x[u][4] = xb.x; x[u][5] = xb.y; x[u][6] = xb.z; x[u][7] = xb.w;
+  }
+  if (a.norm_weight != nullptr) {
+    // the row's RMSNorm, redone by every wave on its registers (4096 values: a few hundred instructions,
+    // against a launch of its own in front of this kernel)
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) ss = fmaf(x[u][i], x[u][i], ss);
+    }
+    const float inv = 1.0f / sqrtf(dh::wave_sum_uniform(ss) / (float)a.K + a.norm_eps);
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int v = lane + 64 * u;
+      if (v < kvec) {
+        const float4 wa = *reinterpret_cast<const float4*>(a.norm_weight + v * 8);
+        const float4 wb = *reinterpret_cast<const float4*>(a.norm_weight + v * 8 + 4);
+        const float w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) x[u][i] = x[u][i] * inv * (a.norm_weight_offset ? 1.0f + w[i] : w[i]);
+      }
+    }
   }
   Cand best{-3.402823e+38f, 0xFFFFFFFFu};   // only lane 0 ever updates its candidate
   for (int r = 0; r < a.rows_per_wave; r++) {
@@ -303,27 +329,50 @@ size_t dh_lmhead_argmax_workspace_bytes(int vocab) {
   return (size_t)kMaxParts * 8;
 }
 
-int dh_lmhead_argmax_f16(const float* d_h, const void* d_E, int vocab, int hidden, int64_t pad_token_id,
-                         float logit_softcap, void* d_workspace, uint32_t* d_token_out, int output_index,
-                         float* d_logits_out) {
-  const char* op = "dh_lmhead_argmax_f16";
+static int lmhead_argmax_impl(const char* op, const float* d_h, const float* d_norm_weight, float eps, int weight_offset,
+                              const void* d_E, int vocab, int hidden, int64_t pad_token_id, float logit_softcap,
+                              void* d_workspace, uint32_t* d_token_out, int output_index, float* d_logits_out) {
   DH_REQUIRE_INIT(op);
   if (int rc = check_f16w_shape(op, 1, vocab, hidden)) return rc;
   if (!d_h || !d_E || !d_workspace || !d_token_out) return dh::fail(1, "[%s] null pointer", op);
   if (output_index < 0) return dh::fail(1, "[%s] outputIndex must be non-negative", op);
   if (reinterpret_cast<uintptr_t>(d_E) & 15) return dh::fail(1, "[%s] weight pointer must be 16-byte aligned", op);
+  if (d_norm_weight) {
+    // the norm runs on the row in registers: only the kernel that keeps it there serves it
+    if (hidden > 4096 || (reinterpret_cast<uintptr_t>(d_h) & 15) || (reinterpret_cast<uintptr_t>(d_norm_weight) & 15))
+      return dh::fail(1, "[%s] the RMSNorm prologue is served for hidden <= 4096 and 16-byte aligned rows (hidden=%d): "
+                         "run dh_rmsnorm in front of dh_lmhead_argmax_f16 instead", op, hidden);
+    if (!(eps >= 0.f)) return dh::fail(1, "[%s] eps must be non-negative", op);
+  }
   F16GemvArgs a{};
   a.A = d_h; a.W = static_cast<const __half*>(d_E); a.C = d_logits_out;
   a.N = vocab; a.K = hidden; a.alpha = 1.0f;
   a.softcap = logit_softcap; a.pad_id = pad_token_id;
   a.part_val = static_cast<float*>(d_workspace);
   a.part_idx = reinterpret_cast<uint32_t*>(static_cast<char*>(d_workspace) + (size_t)kMaxParts * 4);
+  a.norm_weight = d_norm_weight; a.norm_eps = eps; a.norm_weight_offset = weight_offset;
   int parts = 0;
   if (int rc = launch_gemv<1, true>(a, &parts, op)) return rc;
   hipLaunchKernelGGL(argmax_final_kernel, dim3(1), dim3(256), 0, dh::stream(), a.part_val, a.part_idx, parts,
                      d_token_out, output_index);
   DH_CHECK_LAUNCH(op);
   return 0;
+}
+
+int dh_lmhead_argmax_f16(const float* d_h, const void* d_E, int vocab, int hidden, int64_t pad_token_id,
+                         float logit_softcap, void* d_workspace, uint32_t* d_token_out, int output_index,
+                         float* d_logits_out) {
+  return lmhead_argmax_impl("dh_lmhead_argmax_f16", d_h, nullptr, 0.f, 0, d_E, vocab, hidden, pad_token_id, logit_softcap,
+                            d_workspace, d_token_out, output_index, d_logits_out);
+}
+
+int dh_lmhead_argmax_f16_rmsnorm(const float* d_h, const float* d_norm_weight, float eps, int weight_offset,
+                                 const void* d_E, int vocab, int hidden, int64_t pad_token_id, float logit_softcap,
+                                 void* d_workspace, uint32_t* d_token_out, int output_index, float* d_logits_out) {
+  const char* op = "dh_lmhead_argmax_f16_rmsnorm";
+  if (!d_norm_weight) return dh::fail(1, "[%s] null norm weight", op);
+  return lmhead_argmax_impl(op, d_h, d_norm_weight, eps, weight_offset, d_E, vocab, hidden, pad_token_id, logit_softcap,
+                            d_workspace, d_token_out, output_index, d_logits_out);
 }
 
 size_t dh_argmax_workspace_bytes(void) { return (size_t)kMaxParts * 8; }

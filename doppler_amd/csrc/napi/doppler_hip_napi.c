@@ -205,6 +205,12 @@ FN(js_lmhead_argmax_f16) {
   ARGS(10); P(0, h); P(1, E); I(2, vocab); I(3, hid); L(4, pad); F(5, cap); P(6, ws); P(7, tok); I(8, idx); P(9, logits);
   return ret_rc(env, dh_lmhead_argmax_f16((const float*)h, E, vocab, hid, pad, cap, ws, (uint32_t*)tok, idx, (float*)logits));
 }
+FN(js_lmhead_argmax_f16_rmsnorm) {
+  ARGS(13); P(0, h); P(1, nw); F(2, eps); I(3, off); P(4, E); I(5, vocab); I(6, hid); L(7, pad); F(8, cap); P(9, ws);
+  P(10, tok); I(11, idx); P(12, logits);
+  return ret_rc(env, dh_lmhead_argmax_f16_rmsnorm((const float*)h, (const float*)nw, eps, off, E, vocab, hid, pad, cap, ws,
+                                                  (uint32_t*)tok, idx, (float*)logits));
+}
 FN(js_attn_decode_workspace_bytes) { ARGS(3); I(0, H); I(1, D); I(2, kv); return ret_num(env, (double)dh_attn_decode_workspace_bytes(H, D, kv)); }
 FN(js_attn_decode) {
   ARGS(16); P(0, Q); P(1, K); P(2, V); P(3, O); I(4, H); I(5, Hkv); I(6, D); I(7, kvLen); F(8, scale); I(9, causal);
@@ -404,6 +410,7 @@ static napi_value module_init(napi_env env, napi_value exports) {
       {"q4kFfnGateUp", js_q4k_ffn_gate_up}, {"f16wMatmul", js_f16w_matmul},
       {"q4kMatmulRmsnorm", js_q4k_matmul_rmsnorm}, {"q4kFfnGateUpRmsnorm", js_q4k_ffn_gate_up_rmsnorm},
       {"lmheadArgmaxWorkspaceBytes", js_lmhead_argmax_workspace_bytes}, {"lmheadArgmaxF16", js_lmhead_argmax_f16},
+      {"lmheadArgmaxF16RMSNorm", js_lmhead_argmax_f16_rmsnorm},
       {"attnDecodeWorkspaceBytes", js_attn_decode_workspace_bytes}, {"attnDecode", js_attn_decode},
       {"attnDecodeStatic", js_attn_decode_static}, {"attnDecodeStaticMaxBytes", js_attn_decode_static_max_bytes},
       {"attnDecodeQkvSupported", js_attn_decode_qkv_supported}, {"attnDecodeQkv", js_attn_decode_qkv},

@@ -170,11 +170,23 @@ class HipDecoder:
             self._enqueue_layers_chained(pos, device_kv_len)
         else:
             self._enqueue_layers(pos, device_kv_len)
-        ck(L.dh_rmsnorm(x.data_ptr(), self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"],
+        self._enqueue_head(x.data_ptr(), self._out_index, self.logits.data_ptr() if want_logits else None)
+
+    def _enqueue_head(self, hidden_ptr, out_index, logits_ptr):
+        """Final RMSNorm + tied f16 LM head + argmax of one hidden row (recordLogitsGPU + recordLmHeadArgmaxF16,
+        src/inference/pipelines/text/logits/gpu.js:1122-1157): one launch with the norm inside the LM head kernel
+        where the hidden size allows it, else the norm as a launch of its own in front."""
+        L, c, ck = self.L, self.cfg, capi.check
+        Hd = c["hidden"]
+        if Hd <= 4096 and Hd % 8 == 0:
+            ck(L.dh_lmhead_argmax_f16_rmsnorm(hidden_ptr, self.final_norm.data_ptr(), c["eps"], 0, self.embed.data_ptr(),
+                                              c["vocab"], Hd, -1, 0.0, self.lm_ws.data_ptr(), self.token.data_ptr(),
+                                              out_index, logits_ptr))
+            return
+        ck(L.dh_rmsnorm(hidden_ptr, self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"],
                         0, None, None, None, 1.0))
         ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
-                                  self.lm_ws.data_ptr(), self.token.data_ptr(), self._out_index,
-                                  self.logits.data_ptr() if want_logits else None))
+                                  self.lm_ws.data_ptr(), self.token.data_ptr(), out_index, logits_ptr))
 
     def _enqueue_layers(self, pos, device_kv_len):
         L, c, ck = self.L, self.cfg, capi.check
@@ -535,11 +547,7 @@ class HipDecoder:
                                    1.0, x2.data_ptr()))
         # logits of the last prompt token only
         last = b["x"].data_ptr() + (T - 1) * Hd * 4
-        ck(L.dh_rmsnorm(last, self.final_norm.data_ptr(), capi.F32, self.normed.data_ptr(), 1, Hd, c["eps"], 0, None,
-                        None, None, 1.0))
-        ck(L.dh_lmhead_argmax_f16(self.normed.data_ptr(), self.embed.data_ptr(), c["vocab"], Hd, -1, 0.0,
-                                  self.lm_ws.data_ptr(), self.token.data_ptr(), 0,
-                                  self.logits.data_ptr() if (want_logits or sampling is not None) else None))
+        self._enqueue_head(last, 0, self.logits.data_ptr() if (want_logits or sampling is not None) else None)
         if sampling is not None:
             self._enqueue_sample(sampling)
         return self.read_token()

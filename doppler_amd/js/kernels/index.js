@@ -25,7 +25,7 @@ export { runSplitQKV, recordSplitQKV } from './split_qkv.js';
 export { runBiasAdd, recordBiasAdd, runScale, recordScale } from './bias-scale.js';
 export { runGather, recordGather } from './gather.js';
 export { runArgmax, recordArgmax, runGPUSample, recordGPUSample, seededRandom } from './sample.js';
-export { recordLmHeadArgmax, recordLmHeadArgmaxF16 } from './lm-head-argmax.js';
+export { recordLmHeadArgmax, recordLmHeadArgmaxF16, lmHeadArgmaxNormFusable } from './lm-head-argmax.js';
 export { castF32ToF16, castF16ToF32, recordCastF32ToF16, recordCastF16ToF32 } from './cast.js';
 export {
   runMatmulRMSNormFused, recordMatmulRMSNormFused, shouldUseFusedMatmulRMSNorm, selectMatmulRMSNormFusedVariant,

@@ -1,6 +1,9 @@
 // recordLmHeadArgmax / recordLmHeadArgmaxF16: reference src/gpu/kernels/lm-head-argmax.js:292-315.
 // Final-logit GEMV over the f16 (tied) embedding fused with greedy argmax; returns the
-// output buffer with the token id at `outputIndex`.
+// output buffer with the token id at `outputIndex`.  Beyond the reference's options: `normWeight` (f32
+// tensor [hiddenSize]) with `rmsNormEps` and `rmsNormWeightOffset` applies the final RMSNorm of
+// recordLogitsGPU (src/inference/pipelines/text/logits/gpu.js:1122-1157) to the row inside the same
+// kernel (hiddenSize <= 4096; use lmHeadArgmaxNormFusable to ask).
 import { getNative } from '../native.js';
 import { acquireBuffer, releaseBuffer } from '../buffer-pool.js';
 import { getBuffer, getWeightDtype } from '../weight-buffer.js';
@@ -17,6 +20,10 @@ function validateArgmaxOptions(options) {
     throw new Error(`[LmHeadArgmax] outputIndex must be a non-negative integer, got ${idx}.`);
   }
   return idx;
+}
+
+export function lmHeadArgmaxNormFusable(hiddenSize) {
+  return Number.isInteger(hiddenSize) && hiddenSize > 0 && hiddenSize <= 4096 && hiddenSize % 8 === 0;
 }
 
 export async function recordLmHeadArgmaxF16(recorder, inputTensor, lmHead, options = {}) {
@@ -43,10 +50,24 @@ export async function recordLmHeadArgmaxF16(recorder, inputTensor, lmHead, optio
   }
   const workspace = acquireBuffer(native.lmheadArgmaxWorkspaceBytes(options.vocabSize), undefined, 'lm_head_argmax_temp');
   const pad = options.padTokenId === null || options.padTokenId === undefined ? -1 : options.padTokenId;
+  const normWeight = options.normWeight || null;
   try {
-    native.lmheadArgmaxF16(inputTensor.buffer.ptr, weight.ptr, options.vocabSize, options.hiddenSize, pad,
-      options.logitSoftcap || 0, workspace.ptr, output.ptr, outputIndex,
-      options.logitsOutput ? options.logitsOutput.ptr : null);
+    if (normWeight) {
+      if (normWeight.dtype !== 'f32' || normWeight.buffer.size < options.hiddenSize * 4) {
+        throw new Error(`[LmHeadArgmax] normWeight must be an f32 tensor of ${options.hiddenSize} values.`);
+      }
+      if (!(options.rmsNormEps >= 0)) {
+        throw new Error('[LmHeadArgmax] rmsNormEps is required with normWeight.');
+      }
+      native.lmheadArgmaxF16RMSNorm(inputTensor.buffer.ptr, normWeight.buffer.ptr, options.rmsNormEps,
+        options.rmsNormWeightOffset ? 1 : 0, weight.ptr, options.vocabSize, options.hiddenSize, pad,
+        options.logitSoftcap || 0, workspace.ptr, output.ptr, outputIndex,
+        options.logitsOutput ? options.logitsOutput.ptr : null);
+    } else {
+      native.lmheadArgmaxF16(inputTensor.buffer.ptr, weight.ptr, options.vocabSize, options.hiddenSize, pad,
+        options.logitSoftcap || 0, workspace.ptr, output.ptr, outputIndex,
+        options.logitsOutput ? options.logitsOutput.ptr : null);
+    }
   } catch (error) {
     if (!options.outputBuffer) releaseBuffer(output);
     releaseBuffer(workspace);

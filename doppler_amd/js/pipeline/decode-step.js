@@ -6,7 +6,7 @@
 import {
   createTensor, createWeightBuffer, acquireBuffer, releaseBuffer, uploadData, readBufferSlice,
   createCommandRecorder, recordGather, recordRMSNorm, recordMatmul, recordSplitQKVRMSNormRoPEQK,
-  recordAttention, recordFusedNormedFFN, recordFusedFFN, recordLmHeadArgmaxF16, recordGPUSample,
+  recordAttention, recordFusedNormedFFN, recordFusedFFN, recordLmHeadArgmaxF16, lmHeadArgmaxNormFusable, recordGPUSample,
   recordDecodeAttentionFromQKV, decodeAttentionFromQKVSupported,
   recordLayerChain, recordDecodeAttentionPartials, layerChainSupported, layerChainMergesAttention,
   recordCheckFiniteness, parseFinitenessStatusWords, resolveFinitenessAbsThreshold, FINITENESS_STATUS_BYTES,
@@ -85,17 +85,26 @@ export class HipTextDecoder {
     this.readback = null;
   }
 
+  // Final RMSNorm + LM head + argmax of one hidden row: one launch with the norm inside the LM head kernel
+  // where the hidden size allows it, else the norm as a launch of its own in front.
+  async recordNormedLmHead(recorder, temps, hiddenRow, tokenOut, tokenIndex, logitsOutput) {
+    const c = this.config;
+    const opts = { vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: tokenOut, outputIndex: tokenIndex, logitsOutput };
+    if (lmHeadArgmaxNormFusable(c.hidden)) {
+      await recordLmHeadArgmaxF16(recorder, hiddenRow, this.embed, Object.assign({ normWeight: this.finalNorm, rmsNormEps: c.eps }, opts));
+      return;
+    }
+    const normed = await recordRMSNorm(recorder, hiddenRow, this.finalNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden });
+    temps.push(normed.buffer);
+    await recordLmHeadArgmaxF16(recorder, normed, this.embed, opts);
+  }
+
   // Final RMSNorm + LM head for one hidden row; greedy, or top-k temperature sampling when
   // `sampling` = {temperature, topK, randomSeed} is given (the logits then go through memory).
   async recordHead(recorder, temps, hiddenRow, sampling, tokenOut = this.tokenOut, tokenIndex = 0) {
     const c = this.config;
-    const normed = await recordRMSNorm(recorder, hiddenRow, this.finalNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden });
-    temps.push(normed.buffer);
     if (sampling && !this.logits) this.logits = acquireBuffer(c.vocab * 4, undefined, 'logits');
-    await recordLmHeadArgmaxF16(recorder, normed, this.embed, {
-      vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: tokenOut, outputIndex: tokenIndex,
-      logitsOutput: sampling ? this.logits : null,
-    });
+    await this.recordNormedLmHead(recorder, temps, hiddenRow, tokenOut, tokenIndex, sampling ? this.logits : null);
     if (sampling) {
       await recordGPUSample(recorder, this.logits, c.vocab, Object.assign({ outputBuffer: tokenOut, outputIndex: tokenIndex }, sampling));
     }
@@ -238,11 +247,7 @@ export class HipTextDecoder {
     if (options.sampling) {
       await this.recordHead(recorder, temps, x, options.sampling, tokenOut, tokenIndex);
     } else {
-      const finalNormed = temp(await recordRMSNorm(recorder, x, this.finalNorm, c.eps, { batchSize: 1, hiddenSize: c.hidden }));
-      await recordLmHeadArgmaxF16(recorder, finalNormed, this.embed, {
-        vocabSize: c.vocab, hiddenSize: c.hidden, outputBuffer: tokenOut, outputIndex: tokenIndex,
-        logitsOutput: options.logitsOutput || null,
-      });
+      await this.recordNormedLmHead(recorder, temps, x, tokenOut, tokenIndex, options.logitsOutput || null);
     }
   }
 

@@ -863,19 +863,38 @@ def runGPUSample(logits, vocabSize, temperature=1.0, topK=40, randomSeed=None, r
     return int(readBuffer(out, (outputIndex + 1) * 4, np.uint32)[outputIndex])
 
 
+def lmHeadArgmaxNormFusable(hiddenSize):
+    """Whether recordLmHeadArgmaxF16 takes `normWeight` for this hidden size (the row must fit the registers
+    of the LM head kernel)."""
+    return 0 < hiddenSize <= 4096 and hiddenSize % 8 == 0
+
+
 def recordLmHeadArgmaxF16(recorder, inputTensor, lmHead, vocabSize=None, hiddenSize=None, padTokenId=None,
-                          logitSoftcap=0.0, outputBuffer=None, outputIndex=0, logitsOutput=None):
+                          logitSoftcap=0.0, outputBuffer=None, outputIndex=0, logitsOutput=None, normWeight=None,
+                          rmsNormEps=None, rmsNormWeightOffset=False):
     """src/gpu/kernels/lm-head-argmax.js:304 recordLmHeadArgmaxF16: returns the output buffer
     (token at outputIndex).  `recorder` is accepted for signature parity and unused: every op
-    already enqueues in order on one stream."""
+    already enqueues in order on one stream.  Beyond the reference's options: `normWeight` (f32 tensor
+    [hiddenSize]) with `rmsNormEps` applies the final RMSNorm of recordLogitsGPU
+    (src/inference/pipelines/text/logits/gpu.js:1122-1157) to the row inside the same kernel."""
     if inputTensor.dtype != "f32":
         raise DopplerHipError('[LmHeadArgmax] input tensor must be f32, got "%s".' % inputTensor.dtype)
     L = _lib()
     ws = acquireBuffer(int(L.dh_lmhead_argmax_workspace_bytes(vocabSize)))
     out = _out(outputBuffer, max(4, (outputIndex + 1) * 4))
-    capi.check(L.dh_lmhead_argmax_f16(_ptr(inputTensor), _ptr(lmHead), vocabSize, hiddenSize,
-                                      -1 if padTokenId is None else padTokenId, logitSoftcap, ws.data_ptr(),
-                                      out.data_ptr(), outputIndex, _ptr(logitsOutput)))
+    pad = -1 if padTokenId is None else padTokenId
+    if normWeight is not None:
+        if rmsNormEps is None:
+            raise DopplerHipError("[LmHeadArgmax] rmsNormEps is required with normWeight.")
+        if getattr(normWeight, "dtype", "f32") != "f32" or _nbytes(normWeight) < hiddenSize * 4:
+            raise DopplerHipError("[LmHeadArgmax] normWeight must be an f32 tensor of %d values." % hiddenSize)
+        capi.check(L.dh_lmhead_argmax_f16_rmsnorm(_ptr(inputTensor), _ptr(normWeight), float(rmsNormEps),
+                                                  1 if rmsNormWeightOffset else 0, _ptr(lmHead), vocabSize, hiddenSize,
+                                                  pad, logitSoftcap, ws.data_ptr(), out.data_ptr(), outputIndex,
+                                                  _ptr(logitsOutput)))
+        return out
+    capi.check(L.dh_lmhead_argmax_f16(_ptr(inputTensor), _ptr(lmHead), vocabSize, hiddenSize, pad, logitSoftcap,
+                                      ws.data_ptr(), out.data_ptr(), outputIndex, _ptr(logitsOutput)))
     return out
 
 

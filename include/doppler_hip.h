@@ -249,6 +249,14 @@ size_t dh_lmhead_argmax_workspace_bytes(int vocab);
 int dh_lmhead_argmax_f16(const float* d_h, const void* d_E, int vocab, int hidden,
                          int64_t pad_token_id, float logit_softcap, void* d_workspace,
                          uint32_t* d_token_out, int output_index, float* d_logits_out);
+/* The same over RMSNorm(h) (weight f32 [hidden], w or 1 + w), the norm done on the row in the GEMV's
+ * registers: recordLogitsGPU's final norm + LM head (src/inference/pipelines/text/logits/gpu.js:1122-1157)
+ * fused with recordLmHeadArgmaxF16 into one call.  hidden <= 4096, h and the weight 16-byte aligned;
+ * other shapes fail with a message (run dh_rmsnorm in front of dh_lmhead_argmax_f16 there). */
+int dh_lmhead_argmax_f16_rmsnorm(const float* d_h, const float* d_norm_weight, float eps, int weight_offset,
+                                 const void* d_E, int vocab, int hidden, int64_t pad_token_id,
+                                 float logit_softcap, void* d_workspace, uint32_t* d_token_out,
+                                 int output_index, float* d_logits_out);
 
 /* ---- attention ----
  * Decode attention of one query token over an f16 KV cache.  Replaces

@@ -199,7 +199,13 @@ async function main() {
     } else if (c.op === 'lm_head') {
       const rec = dh.createCommandRecorder('lm');
       const E = dh.createWeightBuffer(dev(c.E), 'f16', 'row', [c.vocab, c.hidden]);
-      const buf = await dh.recordLmHeadArgmaxF16(rec, tensor(c.h, 'f32', [1, c.hidden]), E, { vocabSize: c.vocab, hiddenSize: c.hidden });
+      const opts = { vocabSize: c.vocab, hiddenSize: c.hidden };
+      if (c.normWeight) {
+        if (!dh.lmHeadArgmaxNormFusable(c.hidden)) throw new Error('lmHeadArgmaxNormFusable');
+        opts.normWeight = tensor(c.normWeight, 'f32', [c.hidden]);
+        opts.rmsNormEps = c.rmsNormEps;
+      }
+      const buf = await dh.recordLmHeadArgmaxF16(rec, tensor(c.h, 'f32', [1, c.hidden]), E, opts);
       await rec.submitAndWait();
       await save(out, buf, 4);
     } else if (c.op === 'decoder') {

@@ -165,6 +165,12 @@ def test_js_host_path_parity(tmp_path):
     checks.append(lambda: rel_l2(get("mm_f16w.out.bin", np.float32), logits) <= 1e-3)
     cases.append(dict(name="lm_head", op="lm_head", E="e.W", h="e.A", vocab=3000, hidden=512))
     checks.append(lambda: int(get("lm_head.out.bin", np.uint32)[0]) == oracle.argmax(logits[0]))
+    # the final RMSNorm inside the LM head kernel (normWeight option)
+    lnw = synth.normal_f32(512, 9202, 0.3)
+    cases.append(dict(name="lm_head_normed", op="lm_head", E="e.W", h="e.A", vocab=3000, hidden=512,
+                      normWeight=put("e.nw", lnw), rmsNormEps=1e-6))
+    want_normed = oracle.f16w_matmul(oracle.rmsnorm(h, lnw, 1e-6).reshape(1, 512), E, 1, 3000, 512)
+    checks.append(lambda: int(get("lm_head_normed.out.bin", np.uint32)[0]) == oracle.argmax(want_normed[0]))
 
     # fused FFN
     Wg, Wu = synth.q4k_tensor(1024, 768, 9300), synth.q4k_tensor(1024, 768, 9301)
@@ -455,11 +461,11 @@ def test_js_host_path_parity(tmp_path):
     for i, chk in enumerate(checks):
         assert chk(), "check %d failed" % i
     # the profiled step: every op of the step carries a label with a positive time (2 layers x 5 ops
-    # + gather + final norm + LM head)
+    # + gather + LM head with the final norm inside)
     prof = res["profile"]
-    assert res["profileOps"] == 13, res["profileOps"]
+    assert res["profileOps"] == 12, res["profileOps"]
     assert set(prof) == {"gather", "matmul:qkv_proj", "attention:from_qkv", "matmul:o_proj", "fused_normed_ffn",
-                         "matmul:down_proj", "rmsnorm", "lm_head_argmax"}, prof
+                         "matmul:down_proj", "lm_head_argmax"}, prof
     assert all(0.0 < ms < 50.0 for ms in prof.values()), prof
     bad = [e for e in res["errors"] if not e["ok"]]
     assert not bad and len(res["errors"]) >= 21, bad

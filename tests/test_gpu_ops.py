@@ -478,6 +478,21 @@ def test_f16_weight_matmul_and_lmhead_argmax():
     tok = ops.recordLmHeadArgmaxF16(None, ht, eb, vocabSize=vocab, hiddenSize=hidden, padTokenId=pad, outputIndex=3,
                                     outputBuffer=ops.acquireBuffer(16))
     assert int(ops.readBuffer(tok, 16, np.uint32)[3]) == oracle.argmax(want[0], pad_id=pad)
+    # the final RMSNorm inside the LM head kernel (w and 1 + w), against norm then product in the oracle
+    nw = synth.normal_f32(hidden, seed=3003, scale=0.3)
+    nwt = ops.tensorFromNumpy(nw)
+    for offset in (False, True):
+        hn = oracle.rmsnorm(h, nw, 1e-6, weight_offset=offset).reshape(1, hidden)
+        want_n = oracle.f16w_matmul(hn, E, 1, vocab, hidden)
+        tok = ops.recordLmHeadArgmaxF16(None, ht, eb, vocabSize=vocab, hiddenSize=hidden, logitsOutput=logits,
+                                        normWeight=nwt, rmsNormEps=1e-6, rmsNormWeightOffset=offset)
+        assert rel_l2(ops.readBuffer(logits, vocab * 4, np.float32), want_n) <= REL_L2_F32
+        assert int(ops.readBuffer(tok, 4, np.uint32)[0]) == oracle.argmax(want_n[0])
+    assert ops.lmHeadArgmaxNormFusable(4096) and not ops.lmHeadArgmaxNormFusable(5120)
+    big = ops.tensorFromNumpy(synth.normal_f32((1, 5120), seed=3004))
+    with pytest.raises(ops.DopplerHipError, match="hidden <= 4096"):
+        ops.recordLmHeadArgmaxF16(None, big, eb, vocabSize=1000, hiddenSize=5120, normWeight=ops.tensorFromNumpy(
+            np.ones(5120, np.float32)), rmsNormEps=1e-6)
     # batched dense rows
     A = synth.normal_f32((5, hidden), seed=3002)
     got = ops.readTensor(ops.runMatmul(ops.tensorFromNumpy(A), eb, 5, vocab, hidden, outputDtype="f32"))
