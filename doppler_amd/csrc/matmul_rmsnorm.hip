@@ -17,19 +17,33 @@ constexpr int kMaxN = 4096;   // the reference's maxMediumN (src/config/schema/k
 
 // Element types of activations, weights, residual and output: f32, or f16 widened on load and
 // rounded once on the final store (all sums run in f32 either way).
+// The weight matrix is read once per call, every wave whole cache lines of it: those loads carry the
+// non-temporal hint (STREAM), the activations' do not.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+template <bool STREAM>
+__device__ __forceinline__ u32x4_t load_16(const void* p) {
+  return STREAM ? __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p)) : *reinterpret_cast<const u32x4_t*>(p);
+}
+template <bool STREAM>
+__device__ __forceinline__ u32x2_t load_8(const void* p) {
+  return STREAM ? __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p)) : *reinterpret_cast<const u32x2_t*>(p);
+}
 template <typename T> struct Vec16;   // a 16-byte piece
 template <> struct Vec16<float> {
   static constexpr int N = 4;
+  template <bool STREAM = false>
   static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
-    const float4 t = *reinterpret_cast<const float4*>(p);
-    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    const u32x4_t t = load_16<STREAM>(p);
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[i] = __uint_as_float(t[i]);
   }
 };
 template <> struct Vec16<__half> {
   static constexpr int N = 8;
+  template <bool STREAM = false>
   static __device__ __forceinline__ void load(const __half* p, float (&v)[8]) {
-    const uint4 t = *reinterpret_cast<const uint4*>(p);
-    const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+    const u32x4_t w = load_16<STREAM>(p);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       v[2 * i] = __half2float(__ushort_as_half((unsigned short)(w[i] & 0xffffu)));
@@ -40,13 +54,15 @@ template <> struct Vec16<__half> {
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(__half v) { return __half2float(v); }
 // four consecutive elements
-__device__ __forceinline__ void load4(const float* p, float (&v)[4]) { Vec16<float>::load(p, v); }
+template <bool STREAM = false>
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) { Vec16<float>::load<STREAM>(p, v); }
+template <bool STREAM = false>
 __device__ __forceinline__ void load4(const __half* p, float (&v)[4]) {
-  const uint2 t = *reinterpret_cast<const uint2*>(p);
-  v[0] = __half2float(__ushort_as_half((unsigned short)(t.x & 0xffffu)));
-  v[1] = __half2float(__ushort_as_half((unsigned short)(t.x >> 16)));
-  v[2] = __half2float(__ushort_as_half((unsigned short)(t.y & 0xffffu)));
-  v[3] = __half2float(__ushort_as_half((unsigned short)(t.y >> 16)));
+  const u32x2_t t = load_8<STREAM>(p);
+  v[0] = __half2float(__ushort_as_half((unsigned short)(t[0] & 0xffffu)));
+  v[1] = __half2float(__ushort_as_half((unsigned short)(t[0] >> 16)));
+  v[2] = __half2float(__ushort_as_half((unsigned short)(t[1] & 0xffffu)));
+  v[3] = __half2float(__ushort_as_half((unsigned short)(t[1] >> 16)));
 }
 
 // W is [N, K]: a wave per output row and K slice, lanes stride over the slice in 16-byte pieces,
@@ -72,7 +88,7 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(const T* __restrict__ x,
       float w[4][V], v[4][V];
 #pragma unroll
       for (int u = 0; u < 4; u++) {
-        Vec16<T>::load(row + (int64_t)(q + 64 * u) * V, w[u]);
+        Vec16<T>::template load<true>(row + (int64_t)(q + 64 * u) * V, w[u]);
         Vec16<T>::load(x + (int64_t)(q + 64 * u) * V, v[u]);
       }
 #pragma unroll
@@ -82,7 +98,7 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(const T* __restrict__ x,
     }
     for (; q < q1; q += 64) {
       float w[V], v[V];
-      Vec16<T>::load(row + (int64_t)q * V, w);
+      Vec16<T>::template load<true>(row + (int64_t)q * V, w);
       Vec16<T>::load(x + (int64_t)q * V, v);
 #pragma unroll
       for (int e = 0; e < V; e++) a[0] = fmaf(w[e], v[e], a[0]);
@@ -120,7 +136,7 @@ __global__ __launch_bounds__(kColsWaves * 64) void gemv_cols_kernel(const T* __r
         float v[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-          load4(col + (int64_t)(k + u * kColsWaves) * N, w[u]);
+          load4<true>(col + (int64_t)(k + u * kColsWaves) * N, w[u]);
           v[u] = to_f32(x[k + u * kColsWaves]);
         }
 #pragma unroll
@@ -130,7 +146,7 @@ __global__ __launch_bounds__(kColsWaves * 64) void gemv_cols_kernel(const T* __r
       }
       for (; k < k1; k += kColsWaves) {
         float w[4];
-        load4(col + (int64_t)k * N, w);
+        load4<true>(col + (int64_t)k * N, w);
         const float v = to_f32(x[k]);
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[j] = fmaf(w[j], v, acc[j]);
