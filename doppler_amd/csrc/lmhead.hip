@@ -84,57 +84,88 @@ __device__ __forceinline__ uint4 stream_load_16(const uint4* p) {
 }
 
 // M = 1, K <= 4096: every lane meets the same 64 activations in every row (its eight 16-byte
-// chunks sit at fixed k), so they live in registers for the whole kernel: no LDS at all.
+// chunks sit at fixed k), so they live in registers for the whole kernel; LDS only hands the row to
+// the lanes once, at the start.
 template <bool ARGMAX>
 __global__ __launch_bounds__(256) void f16w_gemv_xreg_kernel(const F16GemvArgs a) {
   __shared__ float sv[4];
   __shared__ uint32_t si[4];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int kvec = a.K >> 3;
-  float x[8][8];
-#pragma unroll
-  for (int u = 0; u < 8; u++) {
-    const int v = lane + 64 * u;
-    float4 xa = make_float4(0.f, 0.f, 0.f, 0.f), xb = xa;
-    if (v < kvec) {
-      xa = *reinterpret_cast<const float4*>(a.A + v * 8);
-      xb = *reinterpret_cast<const float4*>(a.A + v * 8 + 4);
-    }
-    x[u][0] = xa.x; x[u][1] = xa.y; x[u][2] = xa.z; x[u][3] = xa.w;
-    x[u][4] = xb.x; x[u][5] = xb.y; x[u][6] = xb.z; x[u][7] = xb.w;
-  }
-  if (a.norm_weight != nullptr) {
-    // the row's RMSNorm, redone by every wave on its registers (4096 values: a few hundred instructions,
-    // against a launch of its own in front of this kernel)
-    float ss = 0.f;
-#pragma unroll
-    for (int u = 0; u < 8; u++) {
-#pragma unroll
-      for (int i = 0; i < 8; i++) ss = fmaf(x[u][i], x[u][i], ss);
-    }
-    const float inv = 1.0f / sqrtf(dh::wave_sum_uniform(ss) / (float)a.K + a.norm_eps);
+  // The activation row reaches the lanes through LDS: the workgroup loads it once (thread t takes the
+  // 16-byte pieces t, t + 256, ..), and with a norm weight normalises it on the way, the same arithmetic
+  // in the same order as the stand-alone RMSNorm launch (per-thread sums of squares over its pieces, wave
+  // sums, the four waves added in order; (x * inv_rms) * w), so the fused call gives the bits of norm
+  // launch + plain call.  Four waves loading the row each cost four times the traffic through the L2.
+  __shared__ __align__(16) float xs[4096];
+  __shared__ float red[4];
+  // the wave's first weight row is requested before any of that, so that it travels meanwhile
+  uint4 raw[8];
+  {
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    const uint4* wrow = reinterpret_cast<const uint4*>(a.W + min(row, (int64_t)a.N - 1) * a.K);
 #pragma unroll
     for (int u = 0; u < 8; u++) {
       const int v = lane + 64 * u;
-      if (v < kvec) {
-        const float4 wa = *reinterpret_cast<const float4*>(a.norm_weight + v * 8);
-        const float4 wb = *reinterpret_cast<const float4*>(a.norm_weight + v * 8 + 4);
-        const float w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+      raw[u] = v < kvec ? stream_load_16(wrow + v) : make_uint4(0, 0, 0, 0);
+    }
+  }
+  {
+    const int nvec = a.K >> 2;
+    float4 xv[4], wv[4];
 #pragma unroll
-        for (int i = 0; i < 8; i++) x[u][i] = x[u][i] * inv * (a.norm_weight_offset ? 1.0f + w[i] : w[i]);
+    for (int j = 0; j < 4; j++) {
+      const int iv = tid + 256 * j;
+      xv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+      wv[j] = make_float4(1.f, 1.f, 1.f, 1.f);
+      if (iv < nvec) {
+        xv[j] = reinterpret_cast<const float4*>(a.A)[iv];
+        if (a.norm_weight != nullptr) wv[j] = reinterpret_cast<const float4*>(a.norm_weight)[iv];
       }
     }
+    if (a.norm_weight != nullptr) {
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        ss = fmaf(xv[j].x, xv[j].x, ss); ss = fmaf(xv[j].y, xv[j].y, ss);
+        ss = fmaf(xv[j].z, xv[j].z, ss); ss = fmaf(xv[j].w, xv[j].w, ss);
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      if (lane == 0) red[wave] = ss;
+      __syncthreads();
+      const float total = red[0] + red[1] + red[2] + red[3];
+      const float inv = 1.0f / sqrtf(total / (float)a.K + a.norm_eps);
+      const bool off = a.norm_weight_offset != 0;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        xv[j].x = xv[j].x * inv * (off ? 1.0f + wv[j].x : wv[j].x); xv[j].y = xv[j].y * inv * (off ? 1.0f + wv[j].y : wv[j].y);
+        xv[j].z = xv[j].z * inv * (off ? 1.0f + wv[j].z : wv[j].z); xv[j].w = xv[j].w * inv * (off ? 1.0f + wv[j].w : wv[j].w);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) reinterpret_cast<float4*>(xs)[tid + 256 * j] = xv[j];
+    __syncthreads();
+  }
+  float x[8][8];
+#pragma unroll
+  for (int u = 0; u < 8; u++) {
+    const int v = lane + 64 * u;     // v < 512: inside xs (pieces past K hold zeros)
+    const float4 xa = reinterpret_cast<const float4*>(xs)[2 * v], xb = reinterpret_cast<const float4*>(xs)[2 * v + 1];
+    x[u][0] = xa.x; x[u][1] = xa.y; x[u][2] = xa.z; x[u][3] = xa.w;
+    x[u][4] = xb.x; x[u][5] = xb.y; x[u][6] = xb.z; x[u][7] = xb.w;
   }
   Cand best{-3.402823e+38f, 0xFFFFFFFFu};   // only lane 0 ever updates its candidate
   for (int r = 0; r < a.rows_per_wave; r++) {
     const int64_t row = ((int64_t)r * gridDim.x + blockIdx.x) * 4 + wave;
     if (row >= a.N) break;   // wave-uniform
     const uint4* wrow = reinterpret_cast<const uint4*>(a.W + row * a.K);
-    uint4 raw[8];
+    if (r > 0) {
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-      const int v = lane + 64 * u;
-      raw[u] = v < kvec ? stream_load_16(wrow + v) : make_uint4(0, 0, 0, 0);
+      for (int u = 0; u < 8; u++) {
+        const int v = lane + 64 * u;
+        raw[u] = v < kvec ? stream_load_16(wrow + v) : make_uint4(0, 0, 0, 0);
+      }
     }
     float s0 = 0.f, s1 = 0.f;
 #pragma unroll

@@ -486,8 +486,13 @@ def test_f16_weight_matmul_and_lmhead_argmax():
         want_n = oracle.f16w_matmul(hn, E, 1, vocab, hidden)
         tok = ops.recordLmHeadArgmaxF16(None, ht, eb, vocabSize=vocab, hiddenSize=hidden, logitsOutput=logits,
                                         normWeight=nwt, rmsNormEps=1e-6, rmsNormWeightOffset=offset)
-        assert rel_l2(ops.readBuffer(logits, vocab * 4, np.float32), want_n) <= REL_L2_F32
+        fused = ops.readBuffer(logits, vocab * 4, np.float32).copy()
+        assert rel_l2(fused, want_n) <= REL_L2_F32
         assert int(ops.readBuffer(tok, 4, np.uint32)[0]) == oracle.argmax(want_n[0])
+        # the same bits as the norm as a launch of its own in front of the plain call
+        normed = ops.runRMSNorm(ht, nwt, 1e-6, batchSize=1, hiddenSize=hidden, rmsNormWeightOffset=offset)
+        ops.recordLmHeadArgmaxF16(None, normed, eb, vocabSize=vocab, hiddenSize=hidden, logitsOutput=logits)
+        assert np.array_equal(ops.readBuffer(logits, vocab * 4, np.float32), fused)
     assert ops.lmHeadArgmaxNormFusable(4096) and not ops.lmHeadArgmaxNormFusable(5120)
     big = ops.tensorFromNumpy(synth.normal_f32((1, 5120), seed=3004))
     with pytest.raises(ops.DopplerHipError, match="hidden <= 4096"):
