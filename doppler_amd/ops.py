@@ -416,8 +416,23 @@ def runAttention(Q, K, V, mask, numHeads, headDim, seqLen=1, kvLen=None, numKVHe
         raise DopplerHipError("[Attention] seqLen must be positive, got %d" % seqLen)
     if mask is not None:
         raise DopplerHipError("[Attention] explicit masks are not supported on the HIP path")
-    if Q.dtype != "f32" or K.dtype != "f16" or V.dtype != "f16":
-        raise DopplerHipError("[Attention] the HIP path needs f32 Q and f16 K/V (got %s/%s/%s)" % (Q.dtype, K.dtype, V.dtype))
+    if Q.dtype not in ("f32", "f16") or K.dtype != "f16" or V.dtype != "f16":
+        raise DopplerHipError("[Attention] the HIP path needs f32 or f16 Q and f16 K/V (got %s/%s/%s)" % (Q.dtype, K.dtype, V.dtype))
+    if Q.dtype == "f16":
+        # the reference's f16-activation plan (variants *_f16, outputDtype f16): Q widened (exact), the f32-Q
+        # kernels, the output narrowed once
+        n = seqLen * numHeads * headDim
+        if _nbytes(Q) < n * 2:
+            raise DopplerHipError("[Attention] Q buffer smaller than [%d, %d, %d] f16" % (seqLen, numHeads, headDim))
+        wide = acquireBuffer(n * 4)
+        capi.check(_lib().dh_cast_f16_to_f32(_ptr(Q), _ptr(wide), n))
+        r = runAttention(Tensor(wide, "f32", Q.shape, "attention_q_f32"), K, V, mask, numHeads, headDim, seqLen=seqLen,
+                         kvLen=kvLen, numKVHeads=numKVHeads, scale=scale, causal=causal, startPos=startPos,
+                         attnSoftcap=attnSoftcap, slidingWindow=slidingWindow, kvStart=kvStart, kvLayout=kvLayout,
+                         workspace=workspace, kvLenBuffer=kvLenBuffer)
+        out = _out(outputBuffer, n * 2)
+        capi.check(_lib().dh_cast_f32_to_f16(_ptr(r), _ptr(out), n))
+        return Tensor(out, "f16", (seqLen, numHeads, headDim), "attention_output")
     layouts = {"contiguous": capi.KV_CONTIGUOUS, "ring": capi.KV_RING}
     if kvLayout not in layouts:
         raise DopplerHipError("[Attention] kvLayout %r is not supported by the HIP path" % (kvLayout,))
@@ -576,13 +591,25 @@ def runRoPE(input, freqsCos, freqsSin, seqLen, numHeads=1, headDim=64, rotaryDim
     """src/gpu/kernels/rope.js:108 runRoPE: in place, returns a Tensor aliasing the input."""
     rotaryDim = headDim if rotaryDim is None else rotaryDim
     pairSpanDim = rotaryDim if pairSpanDim is None else pairSpanDim
-    if input.dtype != "f32":
-        raise DopplerHipError("[RoPE] f32 input required, got %s" % input.dtype)
+    if input.dtype not in ("f32", "f16"):
+        raise DopplerHipError("[RoPE] f32 or f16 input required, got %s" % input.dtype)
     need = (startPos + seqLen) * (rotaryDim // 2) * 4
     if min(_nbytes(freqsCos), _nbytes(freqsSin)) < need:
         raise DopplerHipError("[RoPE] cos/sin tables smaller than %d bytes" % need)
-    capi.check(_lib().dh_rope(_ptr(input), _ptr(freqsCos), _ptr(freqsSin), seqLen, numHeads, headDim, rotaryDim,
-                              pairSpanDim, int(bool(interleaved)), startPos))
+    L = _lib()
+    target = input
+    if input.dtype == "f16":
+        # the reference's route for a device without the f16 kernel (rope.js:44-63,89-107): widen, rotate in
+        # f32, narrow back into the input buffer
+        n = seqLen * numHeads * headDim
+        if _nbytes(input) < n * 2:
+            raise DopplerHipError("[RoPE] input buffer smaller than [%d, %d, %d] f16" % (seqLen, numHeads, headDim))
+        target = acquireBuffer(n * 4)
+        capi.check(L.dh_cast_f16_to_f32(_ptr(input), _ptr(target), n))
+    capi.check(L.dh_rope(_ptr(target), _ptr(freqsCos), _ptr(freqsSin), seqLen, numHeads, headDim, rotaryDim,
+                         pairSpanDim, int(bool(interleaved)), startPos))
+    if input.dtype == "f16":
+        capi.check(L.dh_cast_f32_to_f16(_ptr(target), _ptr(input), seqLen * numHeads * headDim))
     return Tensor(input.buffer, input.dtype, input.shape, "rope_output")
 
 
@@ -775,17 +802,22 @@ def runScale(input, scale, count=None, outputBuffer=None, inplace=False, **_igno
 
 def runGather(indices, embeddings, numTokens, hiddenSize, vocabSize, outputBuffer=None, embeddingDtype=None,
               outputDtype=None, transpose=False, indexOffset=0, **_ignored):
-    """src/gpu/kernels/gather.js:370 runGather for f16 tables -> f32 rows."""
+    """src/gpu/kernels/gather.js:370 runGather for f16 tables -> f32 rows, or (outputDtype 'f16', the
+    reference's f16-activation plan) the stored bits of the rows."""
     if embeddingDtype is None:
         raise DopplerHipError("[Gather] embeddingDtype is required.")
     if outputDtype is None:
         raise DopplerHipError("[Gather] outputDtype is required.")
-    if embeddingDtype != "f16" or outputDtype != "f32" or transpose:
+    if embeddingDtype != "f16" or outputDtype not in ("f32", "f16") or transpose:
         raise DopplerHipError('[Gather] unsupported embeddingDtype="%s" / outputDtype="%s" on the HIP path.' % (embeddingDtype, outputDtype))
-    out = _out(outputBuffer, numTokens * padToQ4KBlock(hiddenSize) * 4)
-    capi.check(_lib().dh_gather_f16(_ptr(indices), _ptr(embeddings), out.data_ptr(), numTokens, hiddenSize, vocabSize,
+    narrow = outputDtype == "f16"
+    out = _out(outputBuffer, numTokens * padToQ4KBlock(hiddenSize) * (2 if narrow else 4))
+    wide = acquireBuffer(numTokens * hiddenSize * 4) if narrow else out
+    capi.check(_lib().dh_gather_f16(_ptr(indices), _ptr(embeddings), wide.data_ptr(), numTokens, hiddenSize, vocabSize,
                                     indexOffset))
-    return Tensor(out, "f32", (numTokens, hiddenSize), "gather_output")
+    if narrow:
+        capi.check(_lib().dh_cast_f32_to_f16(wide.data_ptr(), out.data_ptr(), numTokens * hiddenSize))   # exact
+    return Tensor(out, outputDtype, (numTokens, hiddenSize), "gather_output")
 
 
 def runSiLU(input, size=None, gate=None, outputBuffer=None, swigluLimit=None, **_ignored):

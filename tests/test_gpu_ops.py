@@ -561,6 +561,11 @@ def test_gather_f16_exact():
     assert np.array_equal(ops.readTensor(out).reshape(4, hidden), want)
     with pytest.raises(DopplerHipError, match="embeddingDtype is required"):
         ops.runGather(ops.tensorFromNumpy(ids).buffer, ops.tensorFromNumpy(E).buffer, 4, hidden, vocab)
+    # f16 rows out (the reference's f16-activation plan): the stored bits, zeros for ids past the table
+    out16 = ops.runGather(ops.tensorFromNumpy(ids).buffer, ops.tensorFromNumpy(E).buffer, 4, hidden, vocab,
+                          embeddingDtype="f16", outputDtype="f16", indexOffset=1)
+    assert out16.dtype == "f16"
+    assert np.array_equal(ops.readTensor(out16).view(np.float16).reshape(4, hidden).astype(np.float32), want)
 
 
 # ----------------------------------------------------------------------------- norm / rope / kv / elementwise
@@ -663,6 +668,14 @@ def test_rope_variants():
         assert rel_l2(got, oracle.rope_apply(x, c32, s32, S, H, D, start, rotary_dim=32, pair_span_dim=span)) <= 1e-6
     with pytest.raises(DopplerHipError, match="rotaryDim must be even"):
         ops.runRoPE(xt, ct, st, S, numHeads=H, headDim=D, rotaryDim=31)
+    # f16 activations (src/gpu/kernels/rope.js:44-63): rotated in f32, rounded to f16 once, in place
+    x16 = x.astype(np.float16)
+    t16 = ops.tensorFromNumpy(x16)
+    out16 = ops.runRoPE(t16, ct, st, S, numHeads=H, headDim=D, startPos=start)
+    assert out16.buffer is t16.buffer and out16.dtype == "f16"
+    want16 = oracle.rope_apply(x16.astype(np.float32), cos, sin, S, H, D, start).reshape(-1)
+    got16 = ops.readTensor(out16).view(np.float16).astype(np.float32)
+    assert np.max(np.abs(got16 - want16) / np.maximum(np.abs(want16), 1e-3)) <= 2 ** -10
 
 
 def test_rope_qk_one_launch_equals_two_single_buffer_calls():
@@ -823,6 +836,14 @@ def test_attention_decode_cfg3(ctx):
     assert out.shape == (1, H, D)
     want = oracle.attention_decode_f16kv(q, kb, vb, H, Hkv, D, ctx)
     assert rel_l2(ops.readTensor(out), want) <= REL_L2_F32
+    if ctx == 512:
+        # f16 Q in, f16 out (the reference's *_f16 variants): the f32 result of the f16-rounded query, rounded once
+        q16 = q.astype(np.float16)
+        out16 = ops.runAttention(ops.tensorFromNumpy(q16), ops.tensorFromNumpy(kb), ops.tensorFromNumpy(vb), None, H, D,
+                                 seqLen=1, kvLen=ctx, numKVHeads=Hkv, causal=True, startPos=ctx - 1)
+        assert out16.dtype == "f16" and out16.shape == (1, H, D)
+        want16 = oracle.attention_decode_f16kv(q16.astype(np.float32), kb, vb, H, Hkv, D, ctx)
+        assert rel_l2(ops.readTensor(out16).view(np.float16).astype(np.float32), want16) <= 1e-3
 
 
 def test_attention_decode_key_count_on_the_device():
